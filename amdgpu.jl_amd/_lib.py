@@ -1,0 +1,130 @@
+"""ctypes binding of librk.so -- the only route from the host mirror to the kernels.
+
+There is no fallback: if the shared library has not been built, importing this module raises
+(build it with ``python amdgpu.jl_amd/build.py`` or ``__graft_entry__.build()``).
+The prototypes below restate ``include/rk.h``; ``tests/test_abi_cpu.py`` checks that every symbol
+the header declares is exported.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "librk.so")
+
+RK_MAX_DIMS = 8
+RK_MAX_OPERANDS = 8
+RK_MAX_PROGRAM = 48
+
+# status codes
+RK_SUCCESS = 0
+RK_ERR_INVALID_ARGUMENT = 10001
+RK_ERR_UNSUPPORTED = 10002
+RK_ERR_WORKSPACE = 10003
+RK_ERR_DIMENSION = 10004
+RK_ERR_TOO_LARGE = 10005
+
+# rk_dtype
+RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64 = range(7)
+# rk_map
+RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
+# rk_op
+RK_OP_ADD, RK_OP_MUL, RK_OP_MAX, RK_OP_MIN = range(4)
+# rk_opkind
+RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE = range(3)
+# rk_bc_token
+(RK_BC_ADD, RK_BC_SUB, RK_BC_MUL, RK_BC_DIV, RK_BC_MAX, RK_BC_MIN, RK_BC_POW, RK_BC_FMA) = range(32, 40)
+(RK_BC_NEG, RK_BC_ABS, RK_BC_ABS2, RK_BC_SQRT, RK_BC_EXP, RK_BC_LOG, RK_BC_SIN, RK_BC_COS, RK_BC_TANH,
+ RK_BC_INV, RK_BC_IDENTITY) = range(64, 75)
+
+
+class RkOperand(C.Structure):
+    _fields_ = [
+        ("ptr", C.c_void_p),
+        ("dtype", C.c_int32),
+        ("ndim", C.c_int32),
+        ("shape", C.c_int64 * RK_MAX_DIMS),
+        ("scalar_f", C.c_double),
+        ("scalar_i", C.c_int64),
+    ]
+
+
+class RkProgram(C.Structure):
+    _fields_ = [
+        ("compute", C.c_int32),
+        ("n_operands", C.c_int32),
+        ("operands", RkOperand * RK_MAX_OPERANDS),
+        ("n_tokens", C.c_int32),
+        ("tokens", C.c_int32 * RK_MAX_PROGRAM),
+    ]
+
+
+_I64P = C.POINTER(C.c_int64)
+
+PROTOTYPES = {
+    "rk_version": (C.c_int32, []),
+    "rk_status_string": (C.c_char_p, [C.c_int32]),
+    "rk_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, _I64P, C.c_uint32]),
+    "rk_workspace_init": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_mapreduce": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
+                                 C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_findminmax": (C.c_int32, [C.c_int32, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
+                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_accumulate": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,
+                                  C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_broadcast": (C.c_int32, [C.POINTER(RkProgram), C.c_void_p, C.c_int, C.c_int, _I64P, C.c_void_p]),
+    "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
+                                     C.c_void_p]),
+    "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),
+}
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: the HIP kernels have not been built. "
+            "Run `python amdgpu.jl_amd/build.py` (needs hipcc). There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)      # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+class RKError(RuntimeError):
+    """Non-zero status from librk.so (the analogue of the reference's HIPError, src/hip/error.jl:143-147)."""
+
+    def __init__(self, status: int, where: str = ""):
+        self.status = int(status)
+        msg = lib.rk_status_string(self.status)
+        text = msg.decode() if msg else "?"
+        super().__init__(f"{where + ': ' if where else ''}rk status {self.status}: {text}")
+
+
+class DimensionMismatch(RKError, ValueError):
+    """Julia's DimensionMismatch."""
+
+
+class UnsupportedError(RKError, NotImplementedError):
+    """The request is legal Julia but outside the enumerated native op set."""
+
+
+def check(status: int, where: str = "") -> None:
+    if status == RK_SUCCESS:
+        return
+    if status == RK_ERR_DIMENSION:
+        raise DimensionMismatch(status, where)
+    if status == RK_ERR_UNSUPPORTED:
+        raise UnsupportedError(status, where)
+    raise RKError(status, where)
+
+
+def shape_array(shape):
+    n = len(shape)
+    arr = (C.c_int64 * max(n, 1))(*[int(s) for s in shape])
+    return arr

@@ -1,0 +1,56 @@
+"""Host mirror of ``Base.accumulate!/accumulate/cumsum/cumprod(::AnyROCArray)``
+(src/kernels/accumulate.jl:1-8): defaults and eltype rule on the host, one call through the C ABI.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import _lib as L
+from .array import ROCArray, stream_ptr, workspace
+from .mapreduce import _OP, _scalar_buffer
+
+
+def accumulate_eltype(op: str, dtype) -> np.dtype:
+    """``promote_op(op, T, typeof(init))`` with the reference's default ``init = zero(eltype(A))``
+    (accumulate.jl:1,4): the eltype is preserved (Int32 stays Int32 and wraps); Bool counts in Int64."""
+    dt = np.dtype(dtype)
+    return np.dtype(np.int64) if dt == np.bool_ else dt
+
+
+def accumulate_(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusive: bool = True) -> ROCArray:
+    """``accumulate!(op, B, A; dims, init)``; ``B`` may be ``A`` itself.  Returns ``B``."""
+    if op not in ("add", "mul", "max", "min"):
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"scan operator {op!r}")
+    if B.dims != A.dims:
+        raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"accumulate!: {B.dims} vs {A.dims}")
+    if dims is None:
+        if A.ndim != 1:
+            raise ValueError("accumulate without dims needs a vector (Base semantics)")
+        dims = 1
+    if dims < 1:
+        raise ValueError("dims must be >= 1")
+    if len(A) == 0:
+        return B
+    bytes_needed = L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, B.code, A.ndim, L.shape_array(A.dims),
+                                            (1 << (dims - 1)) if dims <= A.ndim else 0)
+    ws, ws_bytes = workspace(bytes_needed)
+    ibuf = _scalar_buffer(init, B.dtype)
+    st = L.lib.rk_accumulate(_OP[op], A.code, B.code, A.ptr, B.ptr, A.ndim, L.shape_array(A.dims), int(dims),
+                             1 if inclusive else 0, ibuf, ws, ws_bytes, stream_ptr())
+    L.check(st, "rk_accumulate")
+    return B
+
+
+def accumulate(op: str, A: ROCArray, dims=None, init=None, inclusive: bool = True) -> ROCArray:
+    """``accumulate(op, A; dims, init)`` -> new ROCArray of eltype ``accumulate_eltype``."""
+    B = ROCArray(dims=A.dims, dtype=accumulate_eltype(op, A.dtype))
+    return accumulate_(op, B, A, dims=dims, init=init, inclusive=inclusive)
+
+
+def cumsum(A: ROCArray, dims=None) -> ROCArray:
+    """``cumsum(::AnyROCArray; dims)`` (accumulate.jl:7).  Eltype-preserving: Int32 wraps."""
+    return accumulate("add", A, dims=dims)
+
+
+def cumprod(A: ROCArray, dims=None) -> ROCArray:
+    return accumulate("mul", A, dims=dims)

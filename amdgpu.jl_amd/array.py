@@ -1,0 +1,161 @@
+"""ROCArray: the boundary data type of the path (reference: src/array.jl:19-39).
+
+A dense COLUMN-MAJOR device array: a device buffer, Julia ``dims`` and a byte ``offset``; the device
+pointer handed to the kernels is ``buffer + offset`` exactly like
+``Base.unsafe_convert(Ptr{T}, ::ROCArray)`` (src/array.jl:353-354).  PyTorch supplies the device
+memory and the stream, nothing else: no torch kernel runs on the path.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import _lib as L
+
+_DTYPE_CODE = {
+    np.dtype(np.float32): L.RK_F32, np.dtype(np.float64): L.RK_F64,
+    np.dtype(np.int32): L.RK_I32, np.dtype(np.int64): L.RK_I64,
+    np.dtype(np.bool_): L.RK_U8, np.dtype(np.uint8): L.RK_U8,
+    np.dtype(np.uint32): L.RK_U32, np.dtype(np.uint64): L.RK_U64,
+}
+
+
+def dtype_code(dt) -> int:
+    try:
+        return _DTYPE_CODE[np.dtype(dt)]
+    except KeyError:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"eltype {np.dtype(dt)}") from None
+
+
+def device() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU visible: ROCArray needs a HIP device (there is no CPU path)")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def stream_ptr() -> int:
+    """The current (task-local, in the reference: src/tls.jl:71-86) stream as a hipStream_t."""
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+class ROCArray:
+    """Column-major device array with Julia's logical ``dims`` (1-based API at the op level)."""
+
+    __slots__ = ("buf", "dims", "dtype", "offset")
+
+    def __init__(self, data=None, *, dims=None, dtype=None, buf=None, offset=0):
+        if buf is not None:                      # wrap existing storage (views, reshape)
+            self.buf = buf
+            self.dims = tuple(int(d) for d in dims)
+            self.dtype = np.dtype(dtype)
+            self.offset = int(offset)
+            return
+        if data is None:                         # ROCArray{T}(undef, dims)
+            self.dims = tuple(int(d) for d in dims)
+            self.dtype = np.dtype(dtype)
+            self.offset = 0
+            nbytes = int(np.prod(self.dims, dtype=np.int64)) * self.dtype.itemsize
+            self.buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device())
+            return
+        host = np.asarray(data)
+        if dtype is not None:
+            host = host.astype(dtype)
+        self.dims = tuple(host.shape)
+        self.dtype = host.dtype
+        self.offset = 0
+        flat = np.ascontiguousarray(host.reshape(-1, order="F"))
+        raw = torch.from_numpy(flat.view(np.uint8).copy()) if flat.size else torch.empty(1, dtype=torch.uint8)
+        self.buf = raw.to(device(), non_blocking=False)
+
+    # -- Julia-like queries ---------------------------------------------------------------------
+    @property
+    def ndim(self) -> int:
+        return len(self.dims)
+
+    def size(self, d=None):
+        if d is None:
+            return self.dims
+        return self.dims[d - 1] if d <= len(self.dims) else 1
+
+    def __len__(self) -> int:
+        return int(np.prod(self.dims, dtype=np.int64))
+
+    length = __len__
+
+    @property
+    def ptr(self) -> int:
+        return int(self.buf.data_ptr()) + self.offset
+
+    @property
+    def code(self) -> int:
+        return dtype_code(self.dtype)
+
+    def __repr__(self):
+        return f"ROCArray{{{self.dtype}}}{self.dims}"
+
+    # -- host transfer (src/array.jl:215-249) ------------------------------------------------------
+    def to_host(self) -> np.ndarray:
+        """``Array(x)``: synchronises the stream and copies to the host (Julia-shaped NumPy array)."""
+        n = len(self)
+        nbytes = n * self.dtype.itemsize
+        torch.cuda.current_stream().synchronize()
+        raw = self.buf[self.offset:self.offset + nbytes].cpu().numpy()
+        return raw.view(self.dtype)[:n].reshape(self.dims, order="F").copy()
+
+    def item(self):
+        a = self.to_host()
+        return a.reshape(-1)[0]
+
+    # -- wrappers that keep the storage ----------------------------------------------------------
+    def reshape(self, *dims):
+        if len(dims) == 1 and isinstance(dims[0], (tuple, list)):
+            dims = tuple(dims[0])
+        if int(np.prod(dims, dtype=np.int64)) != len(self):
+            raise L.DimensionMismatch(L.RK_ERR_DIMENSION, "reshape")
+        return ROCArray(buf=self.buf, dims=dims, dtype=self.dtype, offset=self.offset)
+
+    def view_range(self, first: int, last: int):
+        """``view(x, first:last)`` of a vector (1-based, inclusive): contiguous, possibly unaligned."""
+        if self.ndim != 1 or not (1 <= first and last <= self.dims[0]):
+            raise IndexError("view_range needs a vector and an in-bounds range")
+        return ROCArray(buf=self.buf, dims=(max(last - first + 1, 0),), dtype=self.dtype,
+                        offset=self.offset + (first - 1) * self.dtype.itemsize)
+
+    def copy(self):
+        out = similar(self)
+        n = len(self) * self.dtype.itemsize
+        out.buf[:n].copy_(self.buf[self.offset:self.offset + n])
+        return out
+
+
+def similar(x: ROCArray, dtype=None, dims=None) -> ROCArray:
+    """``similar(x, T, dims)`` (src/broadcast.jl:26-30 for broadcast outputs)."""
+    return ROCArray(dims=x.dims if dims is None else dims, dtype=x.dtype if dtype is None else dtype)
+
+
+def zeros(dtype, *dims) -> ROCArray:
+    out = ROCArray(dims=dims, dtype=dtype)
+    out.buf.zero_()
+    return out
+
+
+def Array(x: ROCArray) -> np.ndarray:
+    return x.to_host()
+
+
+# ---- per-(device, stream) workspace: the analogue of the reference's per-task library state --------
+_workspaces: dict = {}
+
+
+def workspace(min_bytes: int = 0):
+    """(pointer, bytes) of the initialised workspace bound to the current device and stream."""
+    key = (torch.cuda.current_device(), stream_ptr())
+    need = max(int(min_bytes), 16 << 20)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        size = max(need, 2 * ws.numel() if ws is not None else 0)
+        ws = torch.empty(size, dtype=torch.uint8, device=device())
+        assert ws.data_ptr() % 256 == 0
+        L.check(L.lib.rk_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr()), "rk_workspace_init")
+        _workspaces[key] = ws
+    return ws.data_ptr(), ws.numel()

@@ -1,0 +1,174 @@
+// C ABI entry points of librk.so: argument validation (runs without a GPU), dispatch on the
+// element types, workspace management.  The kernels live in rk_*_impl.hpp / rk_*.hip.
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
+
+#include "rk_common.hpp"
+#include "rk_reduce_impl.hpp"
+#include "rk_scan_impl.hpp"
+
+namespace rk {
+
+const DeviceInfo& device_info() {
+    static DeviceInfo info[64];
+    static std::atomic<int> ready[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (!ready[dev].load(std::memory_order_acquire)) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        info[dev].cus = cus;      // benign race: every writer stores the same value
+        ready[dev].store(1, std::memory_order_release);
+    }
+    return info[dev];
+}
+
+static int env_int(const char* name, int dflt, int lo, int hi) {
+    const char* s = std::getenv(name);
+    if (!s || !*s) return dflt;
+    const long v = std::strtol(s, nullptr, 10);
+    if (v < lo || v > hi) return dflt;
+    return (int)v;
+}
+
+// Workgroups per compute unit the multi-workgroup reductions aim for (RK_REDUCE_BLOCKS_PER_CU).
+int tune_reduce_blocks_per_cu() {
+    static const int v = env_int("RK_REDUCE_BLOCKS_PER_CU", 8, 1, 64);
+    return v;
+}
+
+static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_U64; }
+
+static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {
+    if (ndim < 0 || ndim > RK_MAX_DIMS) return false;
+    if (ndim > 0 && shape == nullptr) return false;
+    int64_t n = 1;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] < 0) return false;
+        if (shape[d] != 0 && n > INT64_MAX / shape[d]) return false;
+        n *= shape[d];
+    }
+    *total = n;
+    return true;
+}
+
+}  // namespace rk
+
+using namespace rk;
+
+extern "C" {
+
+int32_t rk_version(void) { return RK_VERSION; }
+
+const char* rk_status_string(int32_t status) {
+    switch (status) {
+        case RK_SUCCESS: return "RK_SUCCESS";
+        case RK_ERR_INVALID_ARGUMENT: return "RK_ERR_INVALID_ARGUMENT: null pointer, bad enum value or rank out of range";
+        case RK_ERR_UNSUPPORTED: return "RK_ERR_UNSUPPORTED: combination outside the enumerated op / element-type set";
+        case RK_ERR_WORKSPACE: return "RK_ERR_WORKSPACE: workspace missing, not 256-byte aligned or too small";
+        case RK_ERR_DIMENSION: return "RK_ERR_DIMENSION: array extents do not agree";
+        case RK_ERR_TOO_LARGE: return "RK_ERR_TOO_LARGE: an extent exceeds what the kernels can index";
+        default: break;
+    }
+    if (status > 0 && status < 10000) return hipGetErrorString((hipError_t)status);
+    return "unknown rk status";
+}
+
+size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* shape, uint32_t dims_mask) {
+    size_t need = WS_DESC_OFFSET;
+    int64_t total = 0;
+    if (kind == RK_KIND_ACCUMULATE && valid_dtype(dt) && valid_shape(ndim, shape, &total) && total > 0) {
+        // descriptors of the look-back scan: one tagged word per 4 bytes of the value, per tile
+        const Shape3 s = collapse3(ndim, shape, dims_mask);
+        const size_t esz = dtype_size(dt) < 4 ? 4 : dtype_size(dt);
+        const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 4;
+        const int64_t tpl = (s.mid + tile - 1) / tile;
+        if (s.inner == 1 && tpl > 1) need += (size_t)(tpl * s.outer) * (esz / 4) * sizeof(uint64_t);
+    }
+    return (need + 255) & ~(size_t)255;
+}
+
+int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
+    if (ws == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (!is_aligned(ws, 256) || ws_bytes < WS_DESC_OFFSET) return RK_ERR_WORKSPACE;
+    // header + tickets to zero, descriptors to zero (tag 0 = never valid), then epoch = first
+    RK_HIP(hipMemsetAsync(ws, 0, WS_PARTIALS_OFFSET, (hipStream_t)stream));
+    if (ws_bytes > WS_DESC_OFFSET)
+        RK_HIP(hipMemsetAsync((char*)ws + WS_DESC_OFFSET, 0, ws_bytes - WS_DESC_OFFSET, (hipStream_t)stream));
+    const uint32_t first = WS_EPOCH_FIRST;
+    static_assert(WS_EPOCH_FIRST == 1, "the byte-wise memset below writes the value 1");
+    RK_HIP(hipMemsetAsync(ws, (int)first, 1, (hipStream_t)stream));   // little endian: epoch = 1
+    return RK_SUCCESS;
+}
+
+int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
+                     uint32_t reduce_mask, void* R, const void* init, void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)f < RK_MAP_IDENTITY || (int)f > RK_MAP_ABS) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91
+    if (A == nullptr || R == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    reduce_mask &= (1u << ndim) - 1u;       // dims beyond ndim reduce nothing
+    MapreduceArgs a{(int)f, (int)op, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream};
+    if (in == out) {
+        switch (in) {
+            case RK_F32: return mapreduce_f32(a);
+            case RK_F64: return mapreduce_f64(a);
+            case RK_I32: return mapreduce_i32(a);
+            case RK_I64: return mapreduce_i64(a);
+            default: return RK_ERR_UNSUPPORTED;
+        }
+    }
+    if (in == RK_I32 && out == RK_I64) return mapreduce_i32_i64(a);
+    if (in == RK_U8 && out == RK_I64) return mapreduce_u8_i64(a);
+    return RK_ERR_UNSUPPORTED;
+}
+
+int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, const int64_t* shape, uint32_t reduce_mask,
+                      void* vals, int64_t* cart_idx, void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_dtype(in)) return RK_ERR_INVALID_ARGUMENT;
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    if (A == nullptr || (vals == nullptr && cart_idx == nullptr)) return RK_ERR_INVALID_ARGUMENT;
+    reduce_mask &= (1u << ndim) - 1u;
+    FindArgs a{want_max ? 1 : 0, A, ndim, shape, reduce_mask, vals, cart_idx, ws, ws_bytes, (hipStream_t)stream};
+    switch (in) {
+        case RK_F32: return findminmax_f32(a);
+        case RK_F64: return findminmax_f64(a);
+        case RK_I32: return findminmax_i32(a);
+        case RK_I64: return findminmax_i64(a);
+        default: return RK_ERR_UNSUPPORTED;
+    }
+}
+
+int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, void* out_ptr, int ndim, const int64_t* shape,
+                      int dim, int32_t inclusive, const void* init, void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (dim < 1) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    if (in_ptr == nullptr || out_ptr == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (!inclusive && init == nullptr && (op == RK_OP_MAX || op == RK_OP_MIN)) return RK_ERR_INVALID_ARGUMENT;
+    ScanArgs a{(int)op, in_ptr, out_ptr, ndim, shape, dim, inclusive, init, ws, ws_bytes, (hipStream_t)stream};
+    if (in == out) {
+        switch (in) {
+            case RK_F32: return scan_f32(a);
+            case RK_F64: return scan_f64(a);
+            case RK_I32: return scan_i32(a);
+            case RK_I64: return scan_i64(a);
+            default: return RK_ERR_UNSUPPORTED;
+        }
+    }
+    if (in_ptr == out_ptr) return RK_ERR_INVALID_ARGUMENT;   // aliasing needs equal element sizes
+    if (in == RK_U8 && out == RK_I64) return scan_u8_i64(a);
+    if (in == RK_U8 && out == RK_I32) return scan_u8_i32(a);
+    return RK_ERR_UNSUPPORTED;
+}
+
+}  // extern "C"

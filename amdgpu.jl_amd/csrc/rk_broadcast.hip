@@ -1,0 +1,438 @@
+// Fused broadcast: dest .= f(args...) for a flattened Broadcasted tree.
+// Replaces copyto!(dest, ::Broadcasted{<:ROCArrayStyle}) (src/broadcast.jl:3-35), i.e. GPUArrays'
+// one-element-per-work-item broadcast kernel carried by src/ROCKernels.jl:107-129.
+//
+// One kernel skeleton, two index modes, pluggable evaluators:
+//   linear   every array operand has dest's shape: one flat index, 16-byte loads and stores
+//   rows     operands with extruded (size-1) dims: adjacent dims with compatible strides are merged on
+//            the host, lanes run along dim 0 (stride 1 or 0 per operand), a workgroup covers TY rows
+//            and decomposes the row number once per thread -- no div/mod per element
+//   evaluators: fused forms for the frequent trees (no interpretation at all) and a postfix
+//            interpreter for everything else (uniform control flow: every lane runs the same program;
+//            the value stack lives in LDS with the top of stack cached in registers).
+// Arithmetic is NOT contracted into FMAs: Julia evaluates a .* x .+ y as separate mul and add.
+#include <cmath>
+#include <cstring>
+
+#include "rk_common.hpp"
+
+#pragma clang fp contract(off)
+
+namespace rk {
+
+constexpr int BC_BLOCK = 256;
+constexpr int BC_MAX_DEPTH = 8;
+
+struct BcOperand {
+    const void* ptr;        // nullptr: scalar
+    int32_t     dtype;
+    int32_t     stride0;    // 0 or 1 (elements) along merged dim 0
+    int64_t     stride[RK_MAX_DIMS];   // element strides of merged dims 1.. (index d-1)
+    double      sf;
+    int64_t     si;
+};
+
+struct BcArgs {
+    int32_t   n_operands, n_tokens;
+    int32_t   tokens[RK_MAX_PROGRAM];
+    BcOperand op[RK_MAX_OPERANDS];
+    int32_t   ndim;                    // merged rank (>= 1)
+    int64_t   shape[RK_MAX_DIMS];      // merged dest shape
+    int64_t   total;
+    int64_t   nrows;                   // product of shape[1..]
+    int32_t   tx_log2;                 // rows mode: lanes along dim 0 = 1 << tx_log2
+    int64_t   nxb;                     // rows mode: workgroups along dim 0
+    void*     dest;
+    int32_t   dest_dtype;
+};
+
+// ---- typed loads / stores --------------------------------------------------------------------------
+template <typename CT, typename S, int VEC>
+__device__ __forceinline__ void load_as(const void* p, int64_t off, bool contiguous, CT (&v)[VEC]) {
+    const S* q = (const S*)p + off;
+    if (contiguous) {
+        if constexpr (VEC == 1) v[0] = (CT)q[0];
+        else {
+            typedef typename VecOf<S, VEC>::type V;
+            const V x = load_nt((const V*)q);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = (CT)x[j];
+        }
+    } else {
+        const CT x = (CT)q[0];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = x;
+    }
+}
+
+template <typename CT, int VEC>
+__device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT (&v)[VEC]) {
+    if (o.ptr == nullptr) {
+        const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64) ? (CT)o.sf : (CT)o.si;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = x;
+        return;
+    }
+    const bool contiguous = o.stride0 != 0;
+    switch (o.dtype) {
+        case RK_F32: load_as<CT, float, VEC>(o.ptr, off, contiguous, v); break;
+        case RK_F64: load_as<CT, double, VEC>(o.ptr, off, contiguous, v); break;
+        case RK_I32: load_as<CT, int32_t, VEC>(o.ptr, off, contiguous, v); break;
+        case RK_I64: load_as<CT, int64_t, VEC>(o.ptr, off, contiguous, v); break;
+        case RK_U32: load_as<CT, uint32_t, VEC>(o.ptr, off, contiguous, v); break;
+        case RK_U64: load_as<CT, uint64_t, VEC>(o.ptr, off, contiguous, v); break;
+        default:     load_as<CT, uint8_t, VEC>(o.ptr, off, contiguous, v); break;
+    }
+}
+
+template <typename CT, typename D, int VEC>
+__device__ __forceinline__ void store_as(void* p, int64_t off, const CT (&v)[VEC]) {
+    D* q = (D*)p + off;
+    if constexpr (VEC == 1) q[0] = (D)v[0];
+    else {
+        typedef typename VecOf<D, VEC>::type V;
+        V x;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[j] = (D)v[j];
+        store_nt((V*)q, x);
+    }
+}
+
+template <typename CT, int VEC>
+__device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, const CT (&v)[VEC]) {
+    switch (dtype) {
+        case RK_F32: store_as<CT, float, VEC>(p, off, v); break;
+        case RK_F64: store_as<CT, double, VEC>(p, off, v); break;
+        case RK_I32: store_as<CT, int32_t, VEC>(p, off, v); break;
+        case RK_I64: store_as<CT, int64_t, VEC>(p, off, v); break;
+        case RK_U32: store_as<CT, uint32_t, VEC>(p, off, v); break;
+        case RK_U64: store_as<CT, uint64_t, VEC>(p, off, v); break;
+        default:     store_as<CT, uint8_t, VEC>(p, off, v); break;
+    }
+}
+
+// ---- scalar math in the compute type ---------------------------------------------------------------
+template <typename CT> __device__ __forceinline__ CT bc_unary(int tok, CT a) {
+    switch (tok) {
+        case RK_BC_NEG: return -a;
+        case RK_BC_ABS: return a < CT(0) ? -a : (a == CT(0) ? CT(0) : a);
+        case RK_BC_ABS2: return a * a;
+        case RK_BC_SQRT: return sqrt(a);
+        case RK_BC_EXP: return exp(a);
+        case RK_BC_LOG: return log(a);
+        case RK_BC_SIN: return sin(a);
+        case RK_BC_COS: return cos(a);
+        case RK_BC_TANH: return tanh(a);
+        case RK_BC_INV: return CT(1) / a;
+        default: return a;   // RK_BC_IDENTITY
+    }
+}
+template <typename CT> __device__ __forceinline__ CT bc_binary(int tok, CT a, CT b) {
+    switch (tok) {
+        case RK_BC_ADD: return a + b;
+        case RK_BC_SUB: return a - b;
+        case RK_BC_MUL: return a * b;
+        case RK_BC_DIV: return a / b;
+        case RK_BC_MAX: return OpMax()(a, b);
+        case RK_BC_MIN: return OpMin()(a, b);
+        default: return pow(a, b);   // RK_BC_POW
+    }
+}
+
+// ---- evaluators ---------------------------------------------------------------------------------------
+// Postfix interpreter.  Stack slot s of thread t, component j lives at lds[(s * VEC + j) * BLOCK + t]
+// (conflict-free); the top of the stack stays in registers.
+struct EvalInterp {
+    static constexpr int NOPS = RK_MAX_OPERANDS;   // load what the program declares
+    static constexpr bool USES_LDS = true;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
+        const int t = threadIdx.x;
+        CT top[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) top[j] = CT(0);
+        int depth = 0;   // values on the stack, including `top`
+        for (int i = 0; i < a.n_tokens; ++i) {
+            const int tok = a.tokens[i];
+            if (tok < RK_MAX_OPERANDS) {
+                if (depth > 0) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) lds[((depth - 1) * VEC + j) * BC_BLOCK + t] = top[j];
+                }
+                ++depth;
+                // static register indices: select the operand with a uniform branch
+#pragma unroll
+                for (int k = 0; k < RK_MAX_OPERANDS; ++k)
+                    if (tok == k) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) top[j] = in[k][j];
+                    }
+            } else if (tok >= RK_BC_NEG) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) top[j] = bc_unary<CT>(tok, top[j]);
+            } else if (tok == RK_BC_FMA) {
+                CT x[VEC], y[VEC];
+                depth -= 2;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    y[j] = lds[((depth) * VEC + j) * BC_BLOCK + t];
+                    x[j] = lds[((depth - 1) * VEC + j) * BC_BLOCK + t];
+                    top[j] = x[j] * y[j] + top[j];
+                }
+            } else {
+                --depth;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const CT x = lds[((depth - 1) * VEC + j) * BC_BLOCK + t];
+                    top[j] = bc_binary<CT>(tok, x, top[j]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = top[j];
+    }
+};
+
+// z = a * x + y * exp(w)            tokens: 0 1 MUL 2 3 EXP MUL ADD
+struct EvalAxpbyExp {
+    static constexpr int NOPS = 4;
+    static constexpr bool USES_LDS = false;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = in[0][j] * in[1][j] + in[2][j] * exp(in[3][j]);
+    }
+};
+// C = A + r * c                     tokens: 0 1 2 MUL ADD
+struct EvalAddMul {
+    static constexpr int NOPS = 3;
+    static constexpr bool USES_LDS = false;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = in[0][j] + in[1][j] * in[2][j];
+    }
+};
+// dest = x (copy / fill / convert)  tokens: 0
+struct EvalCopy {
+    static constexpr int NOPS = 1;
+    static constexpr bool USES_LDS = false;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = in[0][j];
+    }
+};
+// dest = x op y                     tokens: 0 1 <binary>
+struct EvalBinary {
+    static constexpr int NOPS = 2;
+    static constexpr bool USES_LDS = false;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        const int tok = a.tokens[2];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = bc_binary<CT>(tok, in[0][j], in[1][j]);
+    }
+};
+
+// ---- kernels --------------------------------------------------------------------------------------------
+extern __shared__ __align__(16) unsigned char bc_lds_raw[];
+
+template <typename Eval, typename CT, int VEC, bool ROWS>
+__global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
+    CT* lds = (CT*)bc_lds_raw;
+    const int t = threadIdx.x;
+    int64_t dest_off;
+    int64_t off[RK_MAX_OPERANDS];
+    if constexpr (!ROWS) {
+        dest_off = ((int64_t)blockIdx.x * BC_BLOCK + t) * VEC;
+        if (dest_off >= a.total) return;     // total % VEC == 0 on the vector path
+#pragma unroll
+        for (int k = 0; k < Eval::NOPS; ++k) off[k] = dest_off * a.op[k].stride0;
+    } else {
+        const int64_t rb = (int64_t)blockIdx.x / a.nxb, xb = (int64_t)blockIdx.x - rb * a.nxb;
+        const int tx = t & ((1 << a.tx_log2) - 1), ty = t >> a.tx_log2;
+        const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
+        const int64_t row = rb * (BC_BLOCK >> a.tx_log2) + ty;
+        if (i0 >= a.shape[0] || row >= a.nrows) return;
+        dest_off = row * a.shape[0] + i0;
+#pragma unroll
+        for (int k = 0; k < Eval::NOPS; ++k) off[k] = i0 * a.op[k].stride0;
+        int64_t rem = row;
+        for (int d = 1; d < a.ndim; ++d) {
+            int64_t c;
+            if (d == a.ndim - 1) c = rem;
+            else { c = rem % a.shape[d]; rem /= a.shape[d]; }
+#pragma unroll
+            for (int k = 0; k < Eval::NOPS; ++k) off[k] += c * a.op[k].stride[d - 1];
+        }
+    }
+    CT in[RK_MAX_OPERANDS][VEC];
+#pragma unroll
+    for (int k = 0; k < Eval::NOPS; ++k)
+        if (k < a.n_operands) load_operand<CT, VEC>(a.op[k], off[k], in[k]);
+    CT out[VEC];
+    Eval::template run<CT, VEC>(a, in, out, lds);
+    store_dest<CT, VEC>(a.dest, a.dest_dtype, dest_off, out);
+}
+
+template <typename Eval, typename CT>
+static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
+    const int VECN = vec ? 4 : 1;
+    int64_t blocks;
+    if (!rows) blocks = (a.total / VECN + BC_BLOCK - 1) / BC_BLOCK;
+    else blocks = a.nxb * ((a.nrows + (BC_BLOCK >> a.tx_log2) - 1) / (BC_BLOCK >> a.tx_log2));
+    if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - 1) * VECN * BC_BLOCK * sizeof(CT) : 0;
+    if (vec) {
+        if (rows) bc_kernel<Eval, CT, 4, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        else      bc_kernel<Eval, CT, 4, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+    } else {
+        if (rows) bc_kernel<Eval, CT, 1, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        else      bc_kernel<Eval, CT, 1, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+    }
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+static bool tokens_are(const BcArgs& a, std::initializer_list<int> want) {
+    if ((size_t)a.n_tokens != want.size()) return false;
+    int i = 0;
+    for (int w : want) if (a.tokens[i++] != w) return false;
+    return true;
+}
+
+template <typename CT>
+static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
+    if (tokens_are(a, {0, 1, RK_BC_MUL, 2, 3, RK_BC_EXP, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAxpbyExp, CT>(a, vec, rows, stream);
+    if (tokens_are(a, {0, 1, 2, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAddMul, CT>(a, vec, rows, stream);
+    if (tokens_are(a, {0})) return bc_launch<EvalCopy, CT>(a, vec, rows, stream);
+    if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 && a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW)
+        return bc_launch<EvalBinary, CT>(a, vec, rows, stream);
+    return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
+}
+
+}  // namespace rk
+
+using namespace rk;
+
+extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
+                                void* stream) {
+    if (prog == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
+    if (prog->compute != RK_F32 && prog->compute != RK_F64) return RK_ERR_UNSUPPORTED;
+    if (prog->n_operands < 0 || prog->n_operands > RK_MAX_OPERANDS) return RK_ERR_INVALID_ARGUMENT;
+    if (prog->n_tokens < 1 || prog->n_tokens > RK_MAX_PROGRAM) return RK_ERR_INVALID_ARGUMENT;
+
+    // the program must be a well-formed postfix expression that leaves exactly one value
+    int depth = 0, max_depth = 0;
+    for (int i = 0; i < prog->n_tokens; ++i) {
+        const int tok = prog->tokens[i];
+        if (tok >= 0 && tok < RK_MAX_OPERANDS) {
+            if (tok >= prog->n_operands) return RK_ERR_INVALID_ARGUMENT;
+            ++depth;
+        } else if (tok >= RK_BC_ADD && tok <= RK_BC_POW) {
+            if (depth < 2) return RK_ERR_INVALID_ARGUMENT;
+            --depth;
+        } else if (tok == RK_BC_FMA) {
+            if (depth < 3) return RK_ERR_INVALID_ARGUMENT;
+            depth -= 2;
+        } else if (tok >= RK_BC_NEG && tok <= RK_BC_IDENTITY) {
+            if (depth < 1) return RK_ERR_INVALID_ARGUMENT;
+        } else return RK_ERR_INVALID_ARGUMENT;
+        if (depth > max_depth) max_depth = depth;
+    }
+    if (depth != 1) return RK_ERR_INVALID_ARGUMENT;
+    if (max_depth > BC_MAX_DEPTH) return RK_ERR_UNSUPPORTED;
+
+    int64_t total = 1;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] < 0) return RK_ERR_INVALID_ARGUMENT;
+        total *= shape[d];
+    }
+    // operand shapes against dest (Julia: DimensionMismatch), per-dim strides with 0 on extruded dims
+    int64_t stride[RK_MAX_OPERANDS][RK_MAX_DIMS];
+    for (int k = 0; k < prog->n_operands; ++k) {
+        const rk_operand& o = prog->operands[k];
+        if (o.dtype < RK_F32 || o.dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
+        if (o.ptr == nullptr) {
+            if (o.ndim != 0) return RK_ERR_INVALID_ARGUMENT;
+            for (int d = 0; d < ndim; ++d) stride[k][d] = 0;
+            continue;
+        }
+        if (o.ndim < 0 || o.ndim > ndim) return o.ndim > RK_MAX_DIMS || o.ndim < 0 ? RK_ERR_INVALID_ARGUMENT : RK_ERR_DIMENSION;
+        int64_t s = 1;
+        for (int d = 0; d < ndim; ++d) {
+            const int64_t n = d < o.ndim ? o.shape[d] : 1;
+            if (n != shape[d] && n != 1) return RK_ERR_DIMENSION;
+            stride[k][d] = (n == 1) ? 0 : s;
+            s *= n;
+        }
+    }
+    if (total == 0) return RK_SUCCESS;
+    if (dest == nullptr) return RK_ERR_INVALID_ARGUMENT;
+
+    // merge adjacent dims: (d, d+1) merge when every operand has stride[d+1] == stride[d] * shape[d]
+    // (extruded in both, or dense in both); size-1 dims vanish
+    BcArgs a;
+    std::memset(&a, 0, sizeof(a));
+    int64_t mshape[RK_MAX_DIMS];
+    int64_t mstride[RK_MAX_OPERANDS][RK_MAX_DIMS];
+    int m = 0;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] == 1) continue;
+        bool merge = m > 0;
+        if (merge)
+            for (int k = 0; k < prog->n_operands; ++k)
+                if (stride[k][d] != mstride[k][m - 1] * mshape[m - 1]) { merge = false; break; }
+        if (merge) mshape[m - 1] *= shape[d];
+        else {
+            mshape[m] = shape[d];
+            for (int k = 0; k < prog->n_operands; ++k) mstride[k][m] = stride[k][d];
+            ++m;
+        }
+    }
+    if (m == 0) { mshape[0] = 1; for (int k = 0; k < prog->n_operands; ++k) mstride[k][0] = 0; m = 1; }
+
+    a.n_operands = prog->n_operands;
+    a.n_tokens = prog->n_tokens;
+    for (int i = 0; i < prog->n_tokens; ++i) a.tokens[i] = prog->tokens[i];
+    a.ndim = m;
+    a.total = total;
+    a.nrows = 1;
+    for (int d = 0; d < m; ++d) { a.shape[d] = mshape[d]; if (d > 0) a.nrows *= mshape[d]; }
+    a.dest = dest;
+    a.dest_dtype = (int32_t)dest_dtype;
+    bool linear = true;     // every array operand dense over the merged shape
+    bool vec = (mshape[0] % 4 == 0) && is_aligned(dest, 4 * dtype_size(dest_dtype));
+    for (int k = 0; k < prog->n_operands; ++k) {
+        const rk_operand& o = prog->operands[k];
+        BcOperand& b = a.op[k];
+        b.ptr = o.ptr;
+        b.dtype = o.dtype;
+        b.sf = o.scalar_f;
+        b.si = o.scalar_i;
+        b.stride0 = (int32_t)mstride[k][0];
+        for (int d = 1; d < m; ++d) b.stride[d - 1] = mstride[k][d];
+        if (o.ptr != nullptr) {
+            if (m > 1 || mstride[k][0] != 1) linear = false;
+            if (mstride[k][0] == 1 && !is_aligned(o.ptr, 4 * dtype_size(o.dtype))) vec = false;
+        }
+    }
+    if (m > 1) linear = false;
+    if (m == 1) {
+        // one merged dim: operands are dense (stride 1) or fully extruded (stride 0, same as a scalar load)
+        linear = true;
+    }
+    if (!linear) {
+        // lanes along dim 0: TX = smallest power of two covering shape[0] / VEC, at most the workgroup
+        const int64_t n0v = (mshape[0] + (vec ? 4 : 1) - 1) / (vec ? 4 : 1);
+        int l2 = 0;
+        while ((1 << l2) < BC_BLOCK && (1ll << l2) < n0v) ++l2;
+        a.tx_log2 = l2;
+        a.nxb = (n0v + (1ll << l2) - 1) >> l2;
+    }
+    if (prog->compute == RK_F32) return bc_dispatch<float>(a, vec, !linear, (hipStream_t)stream);
+    return bc_dispatch<double>(a, vec, !linear, (hipStream_t)stream);
+}

@@ -1,0 +1,352 @@
+// Shared host + device helpers of librk.so (gfx950 / wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+#include "../../include/rk.h"
+
+// ---------------------------------------------------------------------------------------
+// host helpers
+// ---------------------------------------------------------------------------------------
+
+#define RK_HIP(expr)                                      \
+    do {                                                  \
+        hipError_t rk_e_ = (expr);                        \
+        if (rk_e_ != hipSuccess) return (int32_t)rk_e_;   \
+    } while (0)
+
+// Launch errors are per-thread state in HIP; read-and-clear right after the launch.
+#define RK_LAUNCH_CHECK()                                 \
+    do {                                                  \
+        hipError_t rk_e_ = hipGetLastError();             \
+        if (rk_e_ != hipSuccess) return (int32_t)rk_e_;   \
+    } while (0)
+
+namespace rk {
+
+constexpr int WAVE = 64;
+
+inline size_t dtype_size(int dt) {
+    switch (dt) {
+        case RK_F32: case RK_I32: case RK_U32: return 4;
+        case RK_F64: case RK_I64: case RK_U64: return 8;
+        case RK_U8: return 1;
+        default: return 0;
+    }
+}
+
+inline bool is_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// Device properties the launch heuristics need; queried once per device.
+struct DeviceInfo {
+    int cus;        // compute units (256 on MI355X)
+};
+const DeviceInfo& device_info();   // rk_api.hip
+
+// ---- workspace layout -------------------------------------------------------------------
+// [0, 256)                       WsHeader
+// [256, +64 KiB)                 completion tickets of the multi-workgroup reductions
+// [.., +WS_PARTIALS_BYTES)       partial results of the reductions
+// [WS_DESC_OFFSET, end)          tile descriptors of the look-back scan (tagged words; kept apart
+//                                from the partials so arbitrary partial bits never look like a tag)
+struct WsHeader {
+    uint32_t epoch;         // scan generation; descriptors of other generations are stale
+    uint32_t tile_counter;  // dynamic tile ids of the scan
+    uint32_t done_counter;  // tiles finished with their descriptors
+    uint32_t pad[61];
+};
+static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
+
+constexpr size_t WS_HEADER_BYTES = 256;
+constexpr size_t WS_TICKET_COUNT = 16384;
+constexpr size_t WS_TICKET_BYTES = WS_TICKET_COUNT * sizeof(uint32_t);
+constexpr size_t WS_PARTIALS_OFFSET = WS_HEADER_BYTES + WS_TICKET_BYTES;
+constexpr size_t WS_PARTIALS_BYTES = (size_t)8 << 20;
+constexpr size_t WS_DESC_OFFSET = WS_PARTIALS_OFFSET + WS_PARTIALS_BYTES;
+constexpr uint32_t WS_EPOCH_FIRST = 1;
+constexpr uint32_t WS_EPOCH_LAST = (1u << 30) - 2;   // after this the scan clears its descriptors
+
+struct Workspace {
+    WsHeader* hdr;
+    uint32_t* tickets;
+    char*     partials;
+    uint64_t* desc;
+    size_t    desc_bytes;
+};
+
+inline bool carve_workspace(void* ws, size_t bytes, size_t desc_needed, Workspace* out) {
+    if (ws == nullptr || !is_aligned(ws, 256)) return false;
+    if (bytes < WS_DESC_OFFSET + desc_needed) return false;
+    out->hdr = (WsHeader*)ws;
+    out->tickets = (uint32_t*)((char*)ws + WS_HEADER_BYTES);
+    out->partials = (char*)ws + WS_PARTIALS_OFFSET;
+    out->desc = (uint64_t*)((char*)ws + WS_DESC_OFFSET);
+    out->desc_bytes = (bytes - WS_DESC_OFFSET) & ~(size_t)7;
+    return true;
+}
+
+// ---- shape canonicalisation ---------------------------------------------------------------
+// A column-major array with a set of marked dims collapses to alternating groups; for a
+// single marked run this is (inner, mid, outer): inner = product of the unmarked dims in
+// front of the run (stride 1), mid = extent of the marked run (stride inner), outer = the
+// unmarked rest (stride inner * mid).
+struct Shape3 {
+    int64_t inner, mid, outer;
+    bool    single_run;   // false: the marked dims do not form one run after dropping size-1 dims
+    int64_t total;
+};
+
+inline Shape3 collapse3(int ndim, const int64_t* shape, uint32_t mask) {
+    Shape3 s{1, 1, 1, true, 1};
+    int state = 0;  // 0: before the run, 1: in the run, 2: after it
+    for (int d = 0; d < ndim; ++d) {
+        int64_t n = shape[d];
+        s.total *= n;
+        if (n == 1) continue;            // size-1 dims belong to whichever group is convenient
+        bool marked = (mask >> d) & 1u;
+        if (state == 0) {
+            if (marked) { state = 1; s.mid *= n; } else s.inner *= n;
+        } else if (state == 1) {
+            if (marked) s.mid *= n; else { state = 2; s.outer *= n; }
+        } else {
+            if (marked) s.single_run = false; else s.outer *= n;
+        }
+    }
+    return s;
+}
+
+}  // namespace rk
+
+// ---------------------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------------------
+#if defined(__HIPCC__)
+
+namespace rk {
+
+template <typename T, int N> struct VecOf { typedef T type __attribute__((ext_vector_type(N))); };
+template <typename T> struct VecOf<T, 1> { typedef T type; };
+
+// 16-byte vectors of each element type
+template <typename T> struct Vec16 {
+    static constexpr int N = 16 / sizeof(T);
+    typedef typename VecOf<T, N>::type type;
+};
+
+template <typename V> __device__ __forceinline__ V load_nt(const V* p) {
+    return __builtin_nontemporal_load(p);
+}
+template <typename V> __device__ __forceinline__ void store_nt(V* p, V v) {
+    __builtin_nontemporal_store(v, p);
+}
+
+// ---- cross-lane data movement on 32-bit words ---------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, bool BOUND = false>
+__device__ __forceinline__ uint32_t dpp_word(uint32_t old, uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)old, (int)v, CTRL, ROW_MASK, BANK_MASK, BOUND);
+}
+
+template <typename T> struct Words {
+    static constexpr int N = (sizeof(T) + 3) / 4;
+    uint32_t w[N];
+};
+template <typename T> __device__ __forceinline__ Words<T> to_words(const T& v) {
+    Words<T> r;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) r.w[i] = 0;
+    __builtin_memcpy(&r, &v, sizeof(T));
+    return r;
+}
+template <typename T> __device__ __forceinline__ T from_words(const Words<T>& w) {
+    T v;
+    __builtin_memcpy(&v, &w, sizeof(T));
+    return v;
+}
+
+// DPP move of a whole value; lanes whose source is invalid or masked receive `old`.
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, typename T>
+__device__ __forceinline__ T dpp_move(const T& old, const T& v) {
+    Words<T> o = to_words(old), s = to_words(v), r;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) r.w[i] = dpp_word<CTRL, ROW_MASK, BANK_MASK>(o.w[i], s.w[i]);
+    return from_words<T>(r);
+}
+
+template <int PATTERN, typename T> __device__ __forceinline__ T swizzle_move(const T& v) {
+    Words<T> s = to_words(v), r;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) r.w[i] = (uint32_t)__builtin_amdgcn_ds_swizzle((int)s.w[i], PATTERN);
+    return from_words<T>(r);
+}
+
+template <typename T> __device__ __forceinline__ T read_lane(const T& v, int lane) {
+    Words<T> s = to_words(v), r;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) r.w[i] = (uint32_t)__builtin_amdgcn_readlane((int)s.w[i], lane);
+    return from_words<T>(r);
+}
+
+// DPP control words (GFX9 encoding)
+constexpr int DPP_QUAD_XOR1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_MIRROR = 0x140;
+constexpr int DPP_ROW_SHR1 = 0x111, DPP_ROW_SHR2 = 0x112, DPP_ROW_SHR4 = 0x114, DPP_ROW_SHR8 = 0x118;
+constexpr int DPP_ROW_BCAST15 = 0x142, DPP_ROW_BCAST31 = 0x143;
+constexpr int DPP_WAVE_SHR1 = 0x138;
+constexpr int SWIZZLE_XOR16 = 0x401F;      // bit mode: and 0x1f, or 0, xor 0x10
+
+// Reduction over the 64 lanes of a wave; the result is wave-uniform.  `op` must be
+// commutative.  Four DPP butterflies inside each row of 16, one ds_swizzle across the two
+// rows of a half, two v_readlane for the halves.
+template <typename T, typename Op> __device__ __forceinline__ T wave_reduce(T v, Op op) {
+    v = op(v, dpp_move<DPP_QUAD_XOR1>(v, v));
+    v = op(v, dpp_move<DPP_QUAD_XOR2>(v, v));
+    v = op(v, dpp_move<DPP_ROW_HALF_MIRROR>(v, v));
+    v = op(v, dpp_move<DPP_ROW_MIRROR>(v, v));
+    v = op(v, swizzle_move<SWIZZLE_XOR16>(v));
+    return op(read_lane(v, 0), read_lane(v, 32));
+}
+
+// Inclusive scan over the 64 lanes of a wave (Kogge-Stone inside rows with row_shr, then
+// row_bcast15 / row_bcast31 carry the row totals).  `ident` is op's neutral element.
+template <typename T, typename Op> __device__ __forceinline__ T wave_scan_inclusive(T v, Op op, T ident) {
+    v = op(dpp_move<DPP_ROW_SHR1>(ident, v), v);
+    v = op(dpp_move<DPP_ROW_SHR2>(ident, v), v);
+    v = op(dpp_move<DPP_ROW_SHR4>(ident, v), v);
+    v = op(dpp_move<DPP_ROW_SHR8>(ident, v), v);
+    v = op(dpp_move<DPP_ROW_BCAST15, 0xa>(ident, v), v);
+    v = op(dpp_move<DPP_ROW_BCAST31, 0xc>(ident, v), v);
+    return v;
+}
+
+// Value of the previous lane (lane 0 receives `ident`): turns an inclusive wave scan into
+// an exclusive one without subtracting.
+template <typename T> __device__ __forceinline__ T wave_shift_right(T v, T ident) {
+    return dpp_move<DPP_WAVE_SHR1>(ident, v);
+}
+
+__device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
+
+// Reduction over a workgroup of NW waves.  Every thread returns the total.  `lds` must
+// hold NW values of T; safe to call repeatedly (leading barrier protects the buffer).
+template <int NW, typename T, typename Op>
+__device__ __forceinline__ T block_reduce(T v, Op op, T* lds) {
+    v = wave_reduce(v, op);
+    if constexpr (NW == 1) return v;
+    const int wave = threadIdx.x / WAVE;
+    __syncthreads();
+    if (lane_id() == 0) lds[wave] = v;
+    __syncthreads();
+    T r = lds[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) r = op(r, lds[i]);
+    return r;
+}
+
+// ---- element-wise maps f of mapreduce(f, op, A) ----------------------------------------------
+struct MapIdentity { template <typename T> __device__ __forceinline__ T operator()(T x) const { return x; } };
+struct MapAbs2     { template <typename T> __device__ __forceinline__ T operator()(T x) const { return x * x; } };
+struct MapAbs {
+    template <typename T> __device__ __forceinline__ T operator()(T x) const {
+        if constexpr (std::is_unsigned<T>::value) return x; else return x < T(0) ? T(0) - x : x;
+    }
+};
+
+// ---- reduction operators ------------------------------------------------------------------
+template <typename T> struct Limits;
+template <> struct Limits<float>    { static __host__ __device__ float lowest() { return -__builtin_inff(); } static __host__ __device__ float highest() { return __builtin_inff(); } };
+template <> struct Limits<double>   { static __host__ __device__ double lowest() { return -__builtin_inf(); } static __host__ __device__ double highest() { return __builtin_inf(); } };
+template <> struct Limits<int32_t>  { static __host__ __device__ int32_t lowest() { return INT32_MIN; } static __host__ __device__ int32_t highest() { return INT32_MAX; } };
+template <> struct Limits<int64_t>  { static __host__ __device__ int64_t lowest() { return INT64_MIN; } static __host__ __device__ int64_t highest() { return INT64_MAX; } };
+template <> struct Limits<uint32_t> { static __host__ __device__ uint32_t lowest() { return 0; } static __host__ __device__ uint32_t highest() { return UINT32_MAX; } };
+template <> struct Limits<uint64_t> { static __host__ __device__ uint64_t lowest() { return 0; } static __host__ __device__ uint64_t highest() { return UINT64_MAX; } };
+template <> struct Limits<uint8_t>  { static __host__ __device__ uint8_t lowest() { return 0; } static __host__ __device__ uint8_t highest() { return 255; } };
+
+// Integer arithmetic wraps like Julia's: do it on the unsigned counterpart.
+template <typename T> __host__ __device__ __forceinline__ T wrap_add(T a, T b) {
+    if constexpr (std::is_integral<T>::value) { typedef typename std::make_unsigned<T>::type U; return (T)((U)a + (U)b); }
+    else return a + b;
+}
+template <typename T> __host__ __device__ __forceinline__ T wrap_mul(T a, T b) {
+    if constexpr (std::is_integral<T>::value) { typedef typename std::make_unsigned<T>::type U; return (T)((U)a * (U)b); }
+    else return a * b;
+}
+
+struct OpAdd {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const { return wrap_add(a, b); }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return T(0); }
+};
+struct OpMul {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const { return wrap_mul(a, b); }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return T(1); }
+};
+// Base.max / Base.min: NaN propagates; max(-0.0, 0.0) == 0.0, min(-0.0, 0.0) == -0.0.
+struct OpMax {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const {
+        if constexpr (std::is_floating_point<T>::value) {
+            if (a != a) return a;
+            if (b != b) return b;
+            if (a == b) return __builtin_signbit(a) ? b : a;
+            return a > b ? a : b;
+        } else return a > b ? a : b;
+    }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return Limits<T>::lowest(); }
+};
+struct OpMin {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const {
+        if constexpr (std::is_floating_point<T>::value) {
+            if (a != a) return a;
+            if (b != b) return b;
+            if (a == b) return __builtin_signbit(a) ? a : b;
+            return a < b ? a : b;
+        } else return a < b ? a : b;
+    }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return Limits<T>::highest(); }
+};
+
+// ---- (value, index) pairs for findmax / findmin ---------------------------------------------
+template <typename T> struct ValIdx {
+    T       v;
+    int64_t i;     // 0-based column-major linear index into A; -1 = nothing yet
+};
+
+// Base.isless total order on values: -0.0 < 0.0 and NaN above everything.
+template <typename T> __host__ __device__ __forceinline__ bool total_less(T a, T b) {
+    if constexpr (std::is_floating_point<T>::value) {
+        const bool an = a != a, bn = b != b;
+        if (an || bn) return !an && bn;
+        if (a == b) return __builtin_signbit(a) && !__builtin_signbit(b);
+        return a < b;
+    } else return a < b;
+}
+
+// findmax: larger under isless wins, ties -> smaller index.  findmin (Base.isgreater):
+// NaN still wins, otherwise the smaller value, ties -> smaller index.  Commutative and
+// associative, so any reduction tree gives the sequential answer.
+template <bool WANT_MAX> struct OpArg {
+    template <typename T> __host__ __device__ __forceinline__ ValIdx<T> operator()(ValIdx<T> a, ValIdx<T> b) const {
+        if (a.i < 0) return b;
+        if (b.i < 0) return a;
+        bool a_better, b_better;
+        if constexpr (WANT_MAX) {
+            a_better = total_less(b.v, a.v);
+            b_better = total_less(a.v, b.v);
+        } else {
+            if constexpr (std::is_floating_point<T>::value) {
+                const bool an = a.v != a.v, bn = b.v != b.v;
+                if (an || bn) { a_better = an && !bn; b_better = bn && !an; }
+                else { a_better = total_less(a.v, b.v); b_better = total_less(b.v, a.v); }
+            } else { a_better = a.v < b.v; b_better = b.v < a.v; }
+        }
+        if (a_better) return a;
+        if (b_better) return b;
+        return a.i < b.i ? a : b;
+    }
+    template <typename P> static __host__ __device__ __forceinline__ P identity() { P p; p.v = 0; p.i = -1; return p; }
+};
+
+}  // namespace rk
+#endif  // __HIPCC__

@@ -1,0 +1,504 @@
+// Reduction kernels: mapreduce over all / some dimensions of a column-major array, and the
+// (value, index) reductions of findmax / findmin.  Replaces partial_mapreduce_device and
+// reduce_group of the reference (src/kernels/mapreduce.jl:43-82, :8-34) and the host driver
+// mapreducedim! (:86-173): one launch, no recursion, no temporary allocation.
+//
+// A reduction over one run of adjacent dimensions sees the array as (inner, mid, outer) with
+// `mid` reduced.  Output q = i + inner * o is the reduction of the "line"
+//     A[i + inner * (m + mid * o)],  m = 0 .. mid-1          (element stride `inner`).
+// Four kernels cover the shapes:
+//   reduce_split_kernel    few long lines (incl. the full reduction): `splits` workgroups per
+//                          line, 128-bit loads when the line is contiguous, partials + a
+//                          completion ticket, the last workgroup of a line combines them in a
+//                          fixed order (deterministic, single launch)
+//   reduce_wave_kernel     many medium lines: one wave per line, no LDS, no barrier
+//   reduce_thread_kernel   very many tiny lines: one lane per line
+//   reduce_strided_kernel  inner >= 64: lanes run along the contiguous `inner` axis (128-bit
+//                          loads), waves and workgroups split `mid`
+// plus reduce_generic_kernel for masks that are not one run (e.g. dims=(1,3)).
+#pragma once
+
+#include "rk_common.hpp"
+
+namespace rk {
+
+struct LineGeom {
+    int64_t inner;   // lines per outer slab == element stride along a line
+    int64_t mid;     // line length
+    int64_t nlines;  // inner * outer
+};
+
+__device__ __forceinline__ int64_t line_base(const LineGeom& g, int64_t q) {
+    if (g.inner == 1) return q * g.mid;
+    const int64_t o = q / g.inner, i = q - o * g.inner;
+    return i + o * g.inner * g.mid;
+}
+
+// ---- element transforms ---------------------------------------------------------------------
+// f is applied in the input type, then converted (Julia: add_sum(widen(f(x)))).
+template <typename In, typename Acc, typename Map> struct MapXform {
+    __device__ __forceinline__ Acc operator()(In x, int64_t) const { return (Acc)Map()(x); }
+};
+template <typename T> struct ArgXform {
+    __device__ __forceinline__ ValIdx<T> operator()(T x, int64_t idx) const { ValIdx<T> p; p.v = x; p.i = idx; return p; }
+};
+
+// ---- result sinks ---------------------------------------------------------------------------
+template <typename Acc, typename Op> struct ReduceSink {
+    Acc* R;
+    Acc  init;
+    int  has_init;
+    __device__ __forceinline__ void operator()(int64_t q, Acc t) const { R[q] = has_init ? Op()(init, t) : t; }
+};
+template <typename T> struct ArgSink {
+    T*       vals;
+    int64_t* cart;
+    int      ndim;
+    int64_t  shape[RK_MAX_DIMS];
+    __device__ __forceinline__ void operator()(int64_t q, ValIdx<T> t) const {
+        if (vals) vals[q] = t.v;
+        if (cart) {
+            int64_t rem = t.i;
+            for (int d = 0; d < ndim; ++d) {
+                const int64_t c = rem % shape[d];
+                rem /= shape[d];
+                cart[q * ndim + d] = c + 1;
+            }
+        }
+    }
+};
+
+// ---- accumulate one slice of one line with GROUP cooperating threads --------------------------
+// slice s of `splits`; `t` = thread index inside the group.  Contiguous lines are read as
+// 16-byte vectors after peeling the unaligned head.
+template <typename In, typename Acc, typename Xf, typename Op, bool VECTOR, int GROUP, int UNROLL>
+__device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t base, int64_t n, int64_t stride,
+                                               int s, int splits, int t, Xf xf, Op op) {
+    if constexpr (VECTOR) {
+        constexpr int VEC = 16 / sizeof(In);
+        typedef typename VecOf<In, VEC>::type V;
+        Acc acc[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = Op::template identity<Acc>();
+        const In* p = A + base;
+        int64_t head = (int64_t)(((16 - ((uintptr_t)p & 15)) & 15) / sizeof(In));
+        if (head > n) head = n;
+        const int64_t nvec = (n - head) / VEC;
+        const V* pv = (const V*)(p + head);
+        const int64_t tail = head + nvec * VEC;
+        if (s == 0) {   // fewer than VEC (<= 16 <= GROUP) scalars on either side
+            if (t < head) acc[0] = op(acc[0], xf(p[t], base + t));
+            if (tail + t < n) acc[0] = op(acc[0], xf(p[tail + t], base + tail + t));
+        }
+        constexpr int64_t CHUNK = (int64_t)GROUP * UNROLL;
+        const int64_t nchunks = nvec / CHUNK;
+        for (int64_t c = s; c < nchunks; c += splits) {
+            V v[UNROLL];
+            const int64_t i0 = c * CHUNK + t;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) v[u] = load_nt(pv + i0 + (int64_t)u * GROUP);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int64_t e0 = base + head + (i0 + (int64_t)u * GROUP) * VEC;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[u][j], e0 + j));
+            }
+        }
+        for (int64_t i = nchunks * CHUNK + (int64_t)s * GROUP + t; i < nvec; i += (int64_t)splits * GROUP) {
+            const V v = load_nt(pv + i);
+            const int64_t e0 = base + head + i * VEC;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[j], e0 + j));
+        }
+        Acc a = acc[0];
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) a = op(a, acc[j]);
+        return a;
+    } else {
+        Acc acc[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) acc[u] = Op::template identity<Acc>();
+        const int64_t step = (int64_t)splits * GROUP;
+        int64_t k = (int64_t)s * GROUP + t;
+        for (; k + (UNROLL - 1) * step < n; k += UNROLL * step) {
+            In v[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) v[u] = A[base + (k + u * step) * stride];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) acc[u] = op(acc[u], xf(v[u], base + (k + u * step) * stride));
+        }
+        for (; k < n; k += step) acc[0] = op(acc[0], xf(A[base + k * stride], base + k * stride));
+        Acc a = acc[0];
+#pragma unroll
+        for (int u = 1; u < UNROLL; ++u) a = op(a, acc[u]);
+        return a;
+    }
+}
+
+// ---- few long lines: grid (splits, nlines) ---------------------------------------------------
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void reduce_split_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
+                                                             Acc* partials, uint32_t* tickets) {
+    constexpr int NW = BLOCK / WAVE;
+    __shared__ Acc lds[NW];
+    __shared__ int is_last;
+    const int s = blockIdx.x, splits = gridDim.x, t = threadIdx.x;
+    const int64_t line = blockIdx.y;
+    const int64_t base = line_base(g, line);
+    Acc a = accumulate_line<In, Acc, Xf, Op, VECTOR, BLOCK, UNROLL>(A, base, g.mid, g.inner, s, splits, t, xf, op);
+    a = block_reduce<NW>(a, op, lds);
+    if (splits == 1) {
+        if (t == 0) sink(line, a);
+        return;
+    }
+    if (t == 0) {
+        partials[line * splits + s] = a;
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[line], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (old == (uint32_t)splits - 1u);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    Acc r = Op::template identity<Acc>();
+    for (int i = t; i < splits; i += BLOCK) r = op(r, partials[line * splits + i]);
+    r = block_reduce<NW>(r, op, lds);
+    if (t == 0) {
+        sink(line, r);
+        tickets[line] = 0;   // leave the workspace clean for the next call
+    }
+}
+
+// ---- many medium lines: one wave per line ------------------------------------------------------
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void reduce_wave_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink) {
+    const int64_t line = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (line >= g.nlines) return;
+    const int64_t base = line_base(g, line);
+    Acc a = accumulate_line<In, Acc, Xf, Op, VECTOR, WAVE, UNROLL>(A, base, g.mid, g.inner, 0, 1, lane_id(), xf, op);
+    a = wave_reduce(a, op);
+    if (lane_id() == 0) sink(line, a);
+}
+
+// ---- very many tiny lines: one lane per line -----------------------------------------------------
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink) {
+    const int64_t line = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (line >= g.nlines) return;
+    const int64_t base = line_base(g, line);
+    Acc a = Op::template identity<Acc>();
+    for (int64_t k = 0; k < g.mid; ++k) a = op(a, xf(A[base + k * g.inner], base + k * g.inner));
+    sink(line, a);
+}
+
+// ---- inner >= 64: lanes along `inner` -------------------------------------------------------------
+// grid (strips, msplits, outer); workgroup = 4 waves; a wave owns 64 * VEC adjacent columns of a
+// strip and every 4th row of the workgroup's slice of `mid`.
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int UNROLL>
+__global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
+                                                             Acc* partials, uint32_t* tickets) {
+    constexpr int VEC = VECTOR ? 16 / sizeof(In) : 1;
+    constexpr int COLS = WAVE * VEC;   // columns per strip
+    constexpr int NW = 4;
+    typedef typename VecOf<In, VEC>::type V;
+    __shared__ Acc lds[NW][COLS];
+    __shared__ int is_last;
+    const int strip = blockIdx.x, ms = blockIdx.y, msplits = gridDim.y;
+    const int64_t o = blockIdx.z;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int64_t col0 = (int64_t)strip * COLS + (int64_t)lane * VEC;
+    const bool live = col0 < g.inner;      // inner % VEC == 0 on the vector path
+    const int64_t slab = o * g.inner * g.mid;
+
+    Acc acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = Op::template identity<Acc>();
+    // rows of this workgroup: contiguous slice [m0, m1) of mid
+    const int64_t per = (g.mid + msplits - 1) / msplits;
+    const int64_t m0 = (int64_t)ms * per;
+    const int64_t m1 = (m0 + per < g.mid) ? m0 + per : g.mid;
+    if (live) {
+        int64_t m = m0 + wave;
+        for (; m + (UNROLL - 1) * NW < m1; m += UNROLL * NW) {
+            V v[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(A + slab + (m + u * NW) * g.inner + col0));
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int64_t e0 = slab + (m + u * NW) * g.inner + col0;
+                if constexpr (VEC == 1) acc[0] = op(acc[0], xf(v[u], e0));
+                else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[u][j], e0 + j));
+                }
+            }
+        }
+        for (; m < m1; m += NW) {
+            const V v = load_nt((const V*)(A + slab + m * g.inner + col0));
+            const int64_t e0 = slab + m * g.inner + col0;
+            if constexpr (VEC == 1) acc[0] = op(acc[0], xf(v, e0));
+            else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[j], e0 + j));
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = acc[j];
+    __syncthreads();
+    const int t = threadIdx.x;
+    const int64_t col = (int64_t)strip * COLS + t;
+    Acc r = Op::template identity<Acc>();
+    if (t < COLS) {
+        r = lds[0][t];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) r = op(r, lds[w][t]);
+    }
+    if (msplits == 1) {
+        if (t < COLS && col < g.inner) sink(col + o * g.inner, r);
+        return;
+    }
+    // partials[(o * strips + strip) * msplits + ms][COLS]
+    const int64_t tile = o * gridDim.x + strip;
+    if (t < COLS) partials[(tile * msplits + ms) * COLS + t] = r;
+    __syncthreads();   // all partial stores of this workgroup are issued before the release below
+    if (t == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (old == (uint32_t)msplits - 1u);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (t < COLS && col < g.inner) {
+        Acc f = Op::template identity<Acc>();
+        for (int i = 0; i < msplits; ++i) f = op(f, partials[(tile * msplits + i) * COLS + t]);
+        sink(col + o * g.inner, f);
+    }
+    if (t == 0) tickets[tile] = 0;
+}
+
+// ---- arbitrary masks: one wave per output ------------------------------------------------------------
+struct GenericGeom {
+    int     nkeep, nred;
+    int64_t keep_size[RK_MAX_DIMS], keep_stride[RK_MAX_DIMS];
+    int64_t red_size[RK_MAX_DIMS], red_stride[RK_MAX_DIMS];
+    int64_t nout, nred_total;
+};
+
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restrict__ A, GenericGeom g, Xf xf, Op op, Sink sink) {
+    const int64_t q = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
+    if (q >= g.nout) return;
+    int64_t base = 0, rem = q;
+    for (int d = 0; d < g.nkeep; ++d) {
+        base += (rem % g.keep_size[d]) * g.keep_stride[d];
+        rem /= g.keep_size[d];
+    }
+    Acc a = Op::template identity<Acc>();
+    for (int64_t k = lane_id(); k < g.nred_total; k += WAVE) {
+        int64_t off = base, r = k;
+        for (int d = 0; d < g.nred; ++d) {
+            off += (r % g.red_size[d]) * g.red_stride[d];
+            r /= g.red_size[d];
+        }
+        a = op(a, xf(A[off], off));
+    }
+    a = wave_reduce(a, op);
+    if (lane_id() == 0) sink(q, a);
+}
+
+// ---- host side: pick a kernel and launch -------------------------------------------------------------
+struct ReducePlan {
+    enum Kind { SPLIT, WAVE_LINES, THREAD_LINES, STRIDED, GENERIC } kind;
+    bool    vector;
+    int     splits;      // SPLIT: workgroups per line; STRIDED: slices of mid
+    int     strips;      // STRIDED
+    size_t  payload;     // bytes of partials
+};
+
+// Tunables (workgroups per compute unit the streaming kernels aim for).
+int tune_reduce_blocks_per_cu();   // rk_api.hip
+
+template <typename In, typename Acc>
+inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
+    ReducePlan p{};
+    const int cus = device_info().cus;
+    const int64_t target_blocks = (int64_t)cus * tune_reduce_blocks_per_cu();
+    constexpr int VEC = 16 / sizeof(In);
+    if (!single_run) { p.kind = ReducePlan::GENERIC; return p; }
+    const int64_t nlines = s.inner * s.outer;
+    if (s.inner >= 64) {
+        p.kind = ReducePlan::STRIDED;
+        p.vector = (s.inner % VEC == 0) && is_aligned(A, 16);
+        const int cols = WAVE * (p.vector ? VEC : 1);
+        const int64_t strips = (s.inner + cols - 1) / cols;
+        p.strips = (int)strips;
+        int64_t tiles = strips * s.outer;
+        int64_t ms = 1;
+        if (tiles < target_blocks && tiles <= (int64_t)WS_TICKET_COUNT) {
+            ms = (target_blocks + tiles - 1) / tiles;
+            const int64_t max_ms = (s.mid + 31) / 32;      // at least 32 rows per workgroup
+            if (ms > max_ms) ms = max_ms;
+            if (ms > 1024) ms = 1024;
+            const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / (tiles * cols);
+            if (ms > fit) ms = fit;
+            if (ms < 1) ms = 1;
+        }
+        p.splits = (int)ms;
+        p.payload = ms > 1 ? (size_t)(tiles * ms * cols) * sizeof(Acc) : 0;
+        return p;
+    }
+    if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
+    const bool contiguous = (s.inner == 1);
+    if (nlines >= target_blocks * 2) {
+        p.kind = ReducePlan::WAVE_LINES;
+        p.vector = contiguous && s.mid >= 2 * VEC;
+        return p;
+    }
+    p.kind = ReducePlan::SPLIT;
+    p.vector = contiguous && s.mid >= 2 * VEC;
+    // a workgroup pass covers 256 lanes * 16 B * 4 loads = 16 KiB; give each split >= 2 passes
+    const int64_t per_pass = 256 * (p.vector ? VEC : 1) * 4;
+    int64_t want = (target_blocks + nlines - 1) / nlines;
+    int64_t max_splits = (s.mid + 2 * per_pass - 1) / (2 * per_pass);
+    if (want > max_splits) want = max_splits;
+    if (want > 4096) want = 4096;
+    const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / nlines;
+    if (want > fit) want = fit;
+    if (want < 1 || nlines > (int64_t)WS_TICKET_COUNT) want = 1;
+    p.splits = (int)want;
+    p.payload = want > 1 ? (size_t)(nlines * want) * sizeof(Acc) : 0;
+    return p;
+}
+
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink>
+inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32_t mask, Xf xf, Op op, Sink sink,
+                             void* ws, size_t ws_bytes, hipStream_t stream) {
+    const Shape3 s = collapse3(ndim, shape, mask);
+    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run);
+    Workspace w{};
+    if (p.payload > WS_PARTIALS_BYTES) return RK_ERR_WORKSPACE;   // the planner never asks for more
+    if (p.payload > 0 && !carve_workspace(ws, ws_bytes, 0, &w)) return RK_ERR_WORKSPACE;
+    LineGeom g{s.inner, s.mid, s.inner * s.outer};
+    constexpr int UNROLL = sizeof(In) >= 4 ? 4 : 2;
+    switch (p.kind) {
+        case ReducePlan::SPLIT: {
+            if (g.nlines > 65535) return RK_ERR_TOO_LARGE;
+            dim3 grid(p.splits, (unsigned)g.nlines);
+            if (p.vector)
+                reduce_split_kernel<In, Acc, Xf, Op, Sink, true, 256, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+            else
+                reduce_split_kernel<In, Acc, Xf, Op, Sink, false, 256, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+            break;
+        }
+        case ReducePlan::WAVE_LINES: {
+            const int64_t blocks = (g.nlines + 3) / 4;
+            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            if (p.vector)
+                reduce_wave_kernel<In, Acc, Xf, Op, Sink, true, 256, UNROLL><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink);
+            else
+                reduce_wave_kernel<In, Acc, Xf, Op, Sink, false, 256, UNROLL><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink);
+            break;
+        }
+        case ReducePlan::THREAD_LINES: {
+            const int64_t blocks = (g.nlines + 255) / 256;
+            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            reduce_thread_kernel<In, Acc, Xf, Op, Sink, 256><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink);
+            break;
+        }
+        case ReducePlan::STRIDED: {
+            if (s.outer > 65535) return RK_ERR_TOO_LARGE;
+            dim3 grid(p.strips, p.splits, (unsigned)s.outer);
+            if (p.vector)
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+            else
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+            break;
+        }
+        case ReducePlan::GENERIC: {
+            GenericGeom gg{};
+            int64_t stride = 1;
+            gg.nout = 1; gg.nred_total = 1;
+            for (int d = 0; d < ndim; ++d) {
+                if (shape[d] != 1) {
+                    if ((mask >> d) & 1u) { gg.red_size[gg.nred] = shape[d]; gg.red_stride[gg.nred] = stride; ++gg.nred; gg.nred_total *= shape[d]; }
+                    else { gg.keep_size[gg.nkeep] = shape[d]; gg.keep_stride[gg.nkeep] = stride; ++gg.nkeep; gg.nout *= shape[d]; }
+                }
+                stride *= shape[d];
+            }
+            const int64_t blocks = (gg.nout + 3) / 4;
+            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            reduce_generic_kernel<In, Acc, Xf, Op, Sink, 256><<<(unsigned)blocks, 256, 0, stream>>>(A, gg, xf, op, sink);
+            break;
+        }
+    }
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+// ---- typed entry points instantiated once per (in, out) pair ---------------------------------------
+struct MapreduceArgs {
+    int f, op;
+    const void* A; int ndim; const int64_t* shape; uint32_t mask;
+    void* R; const void* init;
+    void* ws; size_t ws_bytes; hipStream_t stream;
+};
+struct FindArgs {
+    int want_max;
+    const void* A; int ndim; const int64_t* shape; uint32_t mask;
+    void* vals; int64_t* cart;
+    void* ws; size_t ws_bytes; hipStream_t stream;
+};
+
+template <typename In, typename Acc, typename Map, typename Op>
+inline int32_t mapreduce_one(const MapreduceArgs& a) {
+    ReduceSink<Acc, Op> sink{(Acc*)a.R, a.init ? *(const Acc*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
+    return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, MapXform<In, Acc, Map>(), Op(), sink,
+                                  a.ws, a.ws_bytes, a.stream);
+}
+
+template <typename In, typename Acc, typename Map>
+inline int32_t mapreduce_op(const MapreduceArgs& a) {
+    switch (a.op) {
+        case RK_OP_ADD: return mapreduce_one<In, Acc, Map, OpAdd>(a);
+        case RK_OP_MUL: return mapreduce_one<In, Acc, Map, OpMul>(a);
+        case RK_OP_MAX: return mapreduce_one<In, Acc, Map, OpMax>(a);
+        case RK_OP_MIN: return mapreduce_one<In, Acc, Map, OpMin>(a);
+        default: return RK_ERR_INVALID_ARGUMENT;
+    }
+}
+
+template <typename In, typename Acc>
+inline int32_t mapreduce_typed(const MapreduceArgs& a) {
+    switch (a.f) {
+        case RK_MAP_IDENTITY: return mapreduce_op<In, Acc, MapIdentity>(a);
+        case RK_MAP_ABS2:     return mapreduce_op<In, Acc, MapAbs2>(a);
+        case RK_MAP_ABS:      return mapreduce_op<In, Acc, MapAbs>(a);
+        default: return RK_ERR_INVALID_ARGUMENT;
+    }
+}
+
+template <typename T>
+inline int32_t findminmax_typed(const FindArgs& a) {
+    ArgSink<T> sink{};
+    sink.vals = (T*)a.vals;
+    sink.cart = a.cart;
+    sink.ndim = a.ndim;
+    for (int d = 0; d < a.ndim; ++d) sink.shape[d] = a.shape[d];
+    if (a.want_max)
+        return launch_reduce<T, ValIdx<T>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T>(), OpArg<true>(), sink, a.ws, a.ws_bytes, a.stream);
+    return launch_reduce<T, ValIdx<T>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T>(), OpArg<false>(), sink, a.ws, a.ws_bytes, a.stream);
+}
+
+// one translation unit per type pair (keeps compile times parallel)
+int32_t mapreduce_f32(const MapreduceArgs&);
+int32_t mapreduce_f64(const MapreduceArgs&);
+int32_t mapreduce_i32(const MapreduceArgs&);
+int32_t mapreduce_i64(const MapreduceArgs&);
+int32_t mapreduce_i32_i64(const MapreduceArgs&);
+int32_t mapreduce_u8_i64(const MapreduceArgs&);
+int32_t findminmax_f32(const FindArgs&);
+int32_t findminmax_f64(const FindArgs&);
+int32_t findminmax_i32(const FindArgs&);
+int32_t findminmax_i64(const FindArgs&);
+
+}  // namespace rk

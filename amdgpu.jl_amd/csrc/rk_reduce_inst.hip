@@ -1,0 +1,25 @@
+// Instantiates the reduction kernels for one element-type pair per object file
+// (compiled several times with -DRK_INST=<n> so the instantiations build in parallel).
+#include "rk_reduce_impl.hpp"
+
+namespace rk {
+#if RK_INST == 0
+int32_t mapreduce_f32(const MapreduceArgs& a) { return mapreduce_typed<float, float>(a); }
+int32_t findminmax_f32(const FindArgs& a) { return findminmax_typed<float>(a); }
+#elif RK_INST == 1
+int32_t mapreduce_f64(const MapreduceArgs& a) { return mapreduce_typed<double, double>(a); }
+int32_t findminmax_f64(const FindArgs& a) { return findminmax_typed<double>(a); }
+#elif RK_INST == 2
+int32_t mapreduce_i32(const MapreduceArgs& a) { return mapreduce_typed<int32_t, int32_t>(a); }
+int32_t findminmax_i32(const FindArgs& a) { return findminmax_typed<int32_t>(a); }
+#elif RK_INST == 3
+int32_t mapreduce_i64(const MapreduceArgs& a) { return mapreduce_typed<int64_t, int64_t>(a); }
+int32_t findminmax_i64(const FindArgs& a) { return findminmax_typed<int64_t>(a); }
+#elif RK_INST == 4
+int32_t mapreduce_i32_i64(const MapreduceArgs& a) { return mapreduce_typed<int32_t, int64_t>(a); }
+#elif RK_INST == 5
+int32_t mapreduce_u8_i64(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, int64_t>(a); }
+#else
+#error "RK_INST must be 0..5"
+#endif
+}  // namespace rk

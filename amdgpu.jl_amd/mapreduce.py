@@ -1,0 +1,171 @@
+"""Host mirror of the reduction front end: Base.mapreduce / sum / maximum / findmax on ROCArray and
+``GPUArrays.mapreducedim!`` (src/kernels/mapreduce.jl:86-173).
+
+Everything here is argument plumbing that the Julia front end does before the kernel runs --
+eltype and ``init`` selection (``Base.add_sum`` widens Int32 to Int64), the shape of ``R`` with
+singleton reduced dims (mapreduce.jl:95-107), the scalar fetch for ``dims=:`` -- followed by one call
+through the C ABI.  No arithmetic happens on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib as L
+from .array import ROCArray, dtype_code, stream_ptr, workspace
+
+# f of mapreduce(f, op, A): enumerated, like the C ABI
+identity, abs2, abs_ = "identity", "abs2", "abs"
+# op: "add_sum"/"mul_prod" are what sum/prod use (they widen small integers), "add"/"mul" keep the eltype
+add_sum, mul_prod, add, mul, max_, min_ = "add_sum", "mul_prod", "add", "mul", "max", "min"
+
+_MAP = {"identity": L.RK_MAP_IDENTITY, "abs2": L.RK_MAP_ABS2, "abs": L.RK_MAP_ABS}
+_OP = {"add_sum": L.RK_OP_ADD, "add": L.RK_OP_ADD, "mul_prod": L.RK_OP_MUL, "mul": L.RK_OP_MUL,
+       "max": L.RK_OP_MAX, "min": L.RK_OP_MIN}
+
+
+def reduce_eltype(op: str, dtype) -> np.dtype:
+    """``promote_op(op, T, T)`` as GPUArrays' ``_mapreduce`` infers it: add_sum / mul_prod widen
+    Int8..Int32 and Bool to Int64 (UInt8..UInt32 to UInt64); ``+``/``*``/``max``/``min`` keep T."""
+    dt = np.dtype(dtype)
+    if op in ("add_sum", "mul_prod"):
+        if dt == np.bool_ or dt.type in (np.int8, np.int16, np.int32):
+            return np.dtype(np.int64)
+        if dt.type in (np.uint8, np.uint16, np.uint32):
+            return np.dtype(np.uint64)
+        return dt
+    if op in ("add", "mul") and dt == np.bool_:
+        return np.dtype(np.int64)
+    if op not in _OP:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"reduction operator {op!r}")
+    return dt
+
+
+def _dims_mask(dims, ndim: int) -> int:
+    if dims is None:
+        return (1 << ndim) - 1
+    if isinstance(dims, (int, np.integer)):
+        dims = (int(dims),)
+    mask = 0
+    for d in dims:
+        if d < 1:
+            raise ValueError("dims must be >= 1")
+        if d <= ndim:
+            mask |= 1 << (d - 1)
+    return mask
+
+
+def _reduced_dims(dims_in, mask):
+    return tuple(1 if (mask >> d) & 1 else n for d, n in enumerate(dims_in))
+
+
+def _scalar_buffer(value, dtype: np.dtype):
+    """Host scalar of ``dtype`` as a ctypes buffer (the ABI reads it during the call)."""
+    if value is None:
+        return None
+    return C.create_string_buffer(np.array(value, dtype=dtype).tobytes(), dtype.itemsize)
+
+
+def mapreducedim_(f: str, op: str, R: ROCArray, A: ROCArray, init=None) -> ROCArray:
+    """``GPUArrays.mapreducedim!(f, op, R, A; init)``: reduces A into R over every dimension in which
+    R has extent 1 and A does not; returns the R object it was given (mapreduce.jl:93,172;
+    test/core/rocarray_base.jl:263-267).  With ``init=None`` the neutral element of ``op`` is used."""
+    if f not in _MAP:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"map {f!r}")
+    if op not in _OP:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"reduction operator {op!r}")
+    # Base.check_reducedims (mapreduce.jl:90)
+    rdims = R.dims + (1,) * (A.ndim - R.ndim)          # pad with singleton dims (mapreduce.jl:95-98)
+    if len(rdims) != A.ndim:
+        raise L.DimensionMismatch(L.RK_ERR_DIMENSION, "mapreducedim!: R has more dimensions than A")
+    mask = 0
+    for d, (r, a) in enumerate(zip(rdims, A.dims)):
+        if r == a:
+            continue
+        if r != 1:
+            raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"mapreducedim!: cannot reduce {A.dims} into {R.dims}")
+        mask |= 1 << d
+    if len(A) == 0:
+        return R                                        # mapreduce.jl:91
+    ws, ws_bytes = workspace()
+    ibuf = _scalar_buffer(init, R.dtype)
+    st = L.lib.rk_mapreduce(_MAP[f], _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask,
+                            R.ptr, ibuf, ws, ws_bytes, stream_ptr())
+    L.check(st, "rk_mapreduce")
+    return R
+
+
+def mapreduce(f: str, op: str, A: ROCArray, dims=None, init=None):
+    """``mapreduce(f, op, A; dims, init)``.  ``dims=None`` is Julia's ``:`` and returns a host scalar
+    (a blocking 4/8-byte read, like ``@allowscalar R[]`` in GPUArrays); otherwise a ROCArray whose
+    reduced dims have extent 1."""
+    mask = _dims_mask(dims, A.ndim)
+    out_dt = reduce_eltype(op, A.dtype)
+    if len(A) == 0:
+        if op in ("max", "min"):
+            raise ValueError("reducing over an empty collection is not allowed")
+        neutral = init if init is not None else (0 if _OP[op] == L.RK_OP_ADD else 1)
+        if dims is None:
+            return out_dt.type(neutral)
+        R = ROCArray(np.full(_reduced_dims(A.dims, mask), neutral, dtype=out_dt))
+        return R
+    rshape = (1,) * A.ndim if dims is None else _reduced_dims(A.dims, mask)
+    R = ROCArray(dims=rshape, dtype=out_dt)
+    mapreducedim_(f, op, R, A, init=init)
+    if dims is None:
+        return R.item()
+    return R
+
+
+def sum(A: ROCArray, dims=None, f: str = identity):          # noqa: A001 - mirrors Base.sum
+    return mapreduce(f, add_sum, A, dims=dims)
+
+
+def prod(A: ROCArray, dims=None):
+    return mapreduce(identity, mul_prod, A, dims=dims)
+
+
+def maximum(A: ROCArray, dims=None):
+    return mapreduce(identity, max_, A, dims=dims)
+
+
+def minimum(A: ROCArray, dims=None):
+    return mapreduce(identity, min_, A, dims=dims)
+
+
+def count(A: ROCArray, dims=None):
+    """``count(::ROCArray{Bool})`` == sum of the Bool array in Int64."""
+    if A.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "count needs a Bool array")
+    return mapreduce(identity, add_sum, A, dims=dims)
+
+
+def _findminmax(A: ROCArray, want_max: bool, dims):
+    if len(A) == 0:
+        raise ValueError("reducing over an empty collection is not allowed")
+    mask = _dims_mask(dims, A.ndim)
+    rshape = (1,) * A.ndim if dims is None else _reduced_dims(A.dims, mask)
+    vals = ROCArray(dims=rshape, dtype=A.dtype)
+    # Array{CartesianIndex{N}}: N Int64 per element; kept as an Int64 array with a leading dim N
+    idx = ROCArray(dims=(A.ndim,) + rshape, dtype=np.int64)
+    ws, ws_bytes = workspace()
+    st = L.lib.rk_findminmax(1 if want_max else 0, A.code, A.ptr, A.ndim, L.shape_array(A.dims), mask,
+                             vals.ptr, idx.ptr, ws, ws_bytes, stream_ptr())
+    L.check(st, "rk_findminmax")
+    if dims is None:
+        c = tuple(int(v) for v in idx.to_host().reshape(-1))
+        return vals.item(), (c[0] if A.ndim == 1 else c)
+    return vals, idx
+
+
+def findmax(A: ROCArray, dims=None):
+    """``findmax(A; dims)``: (values, indices).  With ``dims``: ``values`` is a ROCArray with reduced
+    dims of extent 1 and ``indices`` an Int64 ROCArray of dims ``(ndims(A), size(values)...)`` whose
+    column ``[:, I]`` is the CartesianIndex of the winner.  Without: host scalar and index tuple
+    (an Int for vectors)."""
+    return _findminmax(A, True, dims)
+
+
+def findmin(A: ROCArray, dims=None):
+    return _findminmax(A, False, dims)

@@ -1,0 +1,206 @@
+/*
+ * rk.h -- C ABI of librk.so: hand-written gfx950 (MI355X) kernels for the array-kernel
+ * layer behind AMDGPU.jl's ROCArray.
+ *
+ * Every entry point replaces one Julia method family of the reference (file:line given
+ * at each declaration, relative to the AMDGPU.jl tree).  The Julia signatures stay as
+ * they are; their bodies become a `ccall` of the functions below.
+ *
+ * Conventions (they mirror how the reference calls ROCm libraries,
+ * src/hip/libhip.jl:5599-5610 and src/hip/error.jl:143-147):
+ *   - plain pointers and sizes only; arrays are DENSE COLUMN-MAJOR device buffers
+ *     described by (pointer, ndim, shape[ndim]); the pointer is what
+ *     `Base.unsafe_convert(Ptr{T}, ::ROCArray)` yields (src/array.jl:353-354);
+ *   - every call is asynchronous on the given hipStream_t (passed as void*), does not
+ *     synchronise, does not allocate and does not retain caller pointers;
+ *   - the return value is 0 (RK_SUCCESS), a hipError_t (1..9999) reported by the HIP
+ *     runtime, or one of the RK_ERR_* codes (>= 10000); no exceptions, no errno, no abort;
+ *   - zero-length inputs return RK_SUCCESS without launching (src/kernels/mapreduce.jl:91);
+ *   - scalar arguments passed by pointer (`init`) are HOST pointers, read during the call.
+ *
+ * Workspace.  Reductions over many workgroups and the single-pass scan keep small
+ * bookkeeping state (completion tickets, an epoch, per-tile descriptors, partials) in a
+ * caller-owned device buffer.  Contract: allocate at least rk_workspace_bytes(...) bytes
+ * (256-byte aligned), call rk_workspace_init() ONCE on it, and from then on pass it to
+ * calls that are ordered on one stream at a time.  The kernels leave the bookkeeping
+ * clean for the next call, so no per-call memset is needed.  One workspace per stream
+ * corresponds to the reference's per-task library handles (src/cache.jl:102-137).
+ */
+#ifndef RK_H
+#define RK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define RK_API __attribute__((visibility("default")))
+#else
+#define RK_API
+#endif
+
+#define RK_VERSION 100          /* 0.1.0 */
+#define RK_MAX_DIMS 8
+#define RK_MAX_OPERANDS 8
+#define RK_MAX_PROGRAM 48
+
+/* ---- status codes -------------------------------------------------------------- */
+enum {
+    RK_SUCCESS = 0,
+    /* 1..9999: hipError_t values passed through unchanged */
+    RK_ERR_INVALID_ARGUMENT = 10001, /* null pointer, bad enum, ndim out of range, ...   */
+    RK_ERR_UNSUPPORTED      = 10002, /* legal request outside the enumerated op set      */
+    RK_ERR_WORKSPACE        = 10003, /* workspace missing, misaligned or too small       */
+    RK_ERR_DIMENSION        = 10004, /* shapes do not agree (Julia: DimensionMismatch)   */
+    RK_ERR_TOO_LARGE        = 10005  /* an extent exceeds what the kernels index         */
+};
+
+/* ---- element types (Julia eltype <-> code) -------------------------------------- */
+typedef enum {
+    RK_F32 = 0,  /* Float32 */
+    RK_F64 = 1,  /* Float64 */
+    RK_I32 = 2,  /* Int32   */
+    RK_I64 = 3,  /* Int64   */
+    RK_U8  = 4,  /* Bool / UInt8 (one byte per element) */
+    RK_U32 = 5,  /* UInt32  */
+    RK_U64 = 6   /* UInt64  */
+} rk_dtype;
+
+/* f of mapreduce(f, op, A) */
+typedef enum { RK_MAP_IDENTITY = 0, RK_MAP_ABS2 = 1, RK_MAP_ABS = 2 } rk_map;
+
+/* op of mapreduce / accumulate.  Base.add_sum / mul_prod are ADD / MUL with a wider
+ * output dtype chosen by the caller (Int32 -> Int64). */
+typedef enum { RK_OP_ADD = 0, RK_OP_MUL = 1, RK_OP_MAX = 2, RK_OP_MIN = 3 } rk_op;
+
+/* which entry point a workspace is sized for */
+typedef enum {
+    RK_KIND_MAPREDUCE = 0, RK_KIND_FINDMINMAX = 1, RK_KIND_ACCUMULATE = 2
+} rk_opkind;
+
+/* ---- library ------------------------------------------------------------------- */
+RK_API int32_t     rk_version(void);
+RK_API const char* rk_status_string(int32_t status);
+
+/* Bytes of workspace that a call of `kind` on an array of `ndim`/`shape` with element
+ * type `dt` needs (dims_mask: bit d-1 set = Julia dim d is reduced; for accumulate the
+ * single scanned dim).  Never fails: bad arguments return the generic minimum.
+ * A buffer of RK_WORKSPACE_DEFAULT bytes serves every call up to 2^31 elements. */
+#define RK_WORKSPACE_DEFAULT ((size_t)16 << 20)
+RK_API size_t  rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* shape,
+                           uint32_t dims_mask);
+
+/* Zero the bookkeeping area of a freshly allocated workspace (asynchronous on `stream`).
+ * Call once per allocation, before its first use. */
+RK_API int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream);
+
+/* ---- mapreduce ------------------------------------------------------------------
+ * Replaces GPUArrays.mapreducedim!(f, op, R, A; init)      src/kernels/mapreduce.jl:86-173
+ * and its device kernels partial_mapreduce_device / reduce_group        :43-82, :8-34.
+ *
+ * A: `ndim`-dimensional column-major array of `in` elements.  Bit d-1 of `reduce_mask`
+ * set = Julia dimension d is reduced; R has A's shape with every reduced dimension of
+ * size 1 (mapreduce.jl:95-107) and element type `out`.  R is OVERWRITTEN with
+ * op(init, reduction); `init` = host pointer to one `out` element, or NULL for op's
+ * neutral element (0, 1, typemin, typemax).  One launch, no recursion, no allocation.
+ * Supported (in -> out): same type; I32/U8 -> I64 and U32 -> U64 (add_sum widening);
+ * F32 -> F64.  MAX/MIN on floats follow Base.max/min (NaN propagates, -0.0 < 0.0). */
+RK_API int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
+                     const void* A, int ndim, const int64_t* shape, uint32_t reduce_mask,
+                     void* R, const void* init,
+                     void* ws, size_t ws_bytes, void* stream);
+
+/* ---- findmax / findmin -----------------------------------------------------------
+ * Replaces the (value, CartesianIndex) tuple reduction that GPUArrays' findminmax sends
+ * through mapreducedim!                                    src/kernels/mapreduce.jl:86
+ * (benchmarked in perf/array.jl:50-53).
+ *
+ * vals: A's shape with reduced dims of size 1, element type `in`.
+ * cart_idx: for each output element `ndim` consecutive Int64 = the 1-based CartesianIndex
+ * of the winner in A (memory layout of Array{CartesianIndex{ndim}}).  Ties -> smallest
+ * column-major index; the first NaN wins; +0.0 > -0.0 (Base.isless order).
+ * Either output pointer may be NULL to skip it. */
+RK_API int32_t rk_findminmax(int32_t want_max, rk_dtype in,
+                      const void* A, int ndim, const int64_t* shape, uint32_t reduce_mask,
+                      void* vals, int64_t* cart_idx,
+                      void* ws, size_t ws_bytes, void* stream);
+
+/* ---- accumulate / cumsum / cumprod -------------------------------------------------
+ * Replaces Base.accumulate!/accumulate/cumsum/cumprod(::AnyROCArray)
+ *                                                        src/kernels/accumulate.jl:1-8
+ * (forwarders into AcceleratedKernels.accumulate!).
+ *
+ * Scans along Julia dimension `dim` (1-based; dim > ndim copies, with init folded in).
+ * `out` may alias `in` when the dtypes agree.  inclusive != 0: out[k] = init op a[1] op ..
+ * op a[k]; inclusive == 0: out[k] = init op a[1] op .. op a[k-1].  `init` = host pointer to
+ * one `out` element or NULL for the neutral element.  Integer arithmetic wraps.
+ * Supported (in -> out): same type; U8 -> I64, U8 -> I32 (Bool counts). ADD and MUL;
+ * MAX/MIN for same-type scans. */
+RK_API int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out,
+                      const void* in_ptr, void* out_ptr,
+                      int ndim, const int64_t* shape, int dim, int32_t inclusive,
+                      const void* init,
+                      void* ws, size_t ws_bytes, void* stream);
+
+/* ---- fused broadcast ---------------------------------------------------------------
+ * Replaces copyto!(dest, ::Broadcasted{<:ROCArrayStyle})              src/broadcast.jl:3-35
+ * i.e. GPUArrays' broadcast kernel launched through the KernelAbstractions functor
+ *                                                              src/ROCKernels.jl:107-129.
+ *
+ * The Broadcasted tree is flattened to a postfix program over up to RK_MAX_OPERANDS
+ * operands.  An array operand has `ndim` <= dest's ndim and each extent either equal to
+ * dest's or 1 (extruded: stride 0, what Broadcast.preprocess/Extruded does); missing
+ * trailing dims count as 1.  A scalar operand is passed by value. */
+typedef enum {
+    /* tokens 0 .. RK_MAX_OPERANDS-1 push that operand */
+    RK_BC_ADD = 32, RK_BC_SUB, RK_BC_MUL, RK_BC_DIV, RK_BC_MAX, RK_BC_MIN, RK_BC_POW,
+    RK_BC_FMA,                 /* muladd(a, b, c): pops c, b, a                         */
+    RK_BC_NEG = 64, RK_BC_ABS, RK_BC_ABS2, RK_BC_SQRT, RK_BC_EXP, RK_BC_LOG, RK_BC_SIN,
+    RK_BC_COS, RK_BC_TANH, RK_BC_INV, RK_BC_IDENTITY
+} rk_bc_token;
+
+typedef struct {
+    const void* ptr;              /* device pointer; NULL for a scalar operand           */
+    int32_t     dtype;            /* rk_dtype of the array elements / of the scalar      */
+    int32_t     ndim;             /* 0 for scalars                                       */
+    int64_t     shape[RK_MAX_DIMS];
+    double      scalar_f;         /* scalar value when dtype is F32/F64                  */
+    int64_t     scalar_i;         /* scalar value when dtype is an integer type          */
+} rk_operand;
+
+typedef struct {
+    int32_t    compute;           /* rk_dtype every operand is converted to: F32 or F64 */
+    int32_t    n_operands;
+    rk_operand operands[RK_MAX_OPERANDS];
+    int32_t    n_tokens;
+    int32_t    tokens[RK_MAX_PROGRAM];
+} rk_program;
+
+RK_API int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype,
+                     int ndim, const int64_t* shape, void* stream);
+
+/* ---- volumerhs -----------------------------------------------------------------------
+ * Replaces `@roc groupsize=(5,5) gridsize=nelem volumerhs!(rhs, Q, vgeo, gravity, D, nelem)`
+ *                                                   perf/volumerhs.jl:42-176, :200-201.
+ * N = 4 (Nq = 5), 5 states, 14 metric fields, Float32, like the reference's benchmark:
+ * rhs, Q: (5,5,5,5,nelem); vgeo: (5,5,5,14,nelem); D: (5,5); all column-major.
+ * rhs is accumulated into (+=).  rhs must not alias Q or vgeo. */
+RK_API int32_t rk_volumerhs_f32(float* rhs, const float* Q, const float* vgeo, float gravity,
+                         const float* D, int64_t nelem, void* stream);
+
+/* ---- findall scatter (caller of the scan) -----------------------------------------------
+ * Replaces the scatter kernel `_ker!` of Base.findall(::AnyROCArray{Bool})
+ *                                                        src/kernels/indexing.jl:16-31.
+ * `indices` = inclusive Int64 cumsum of the flattened `bools` (rk_accumulate U8 -> I64).
+ * Writes, for every true element, its 1-based CartesianIndex (`ndim` Int64, or the linear
+ * index when ndim == 1) to ys[indices[i]-1]. */
+RK_API int32_t rk_findall_scatter(const uint8_t* bools, const int64_t* indices, int64_t* ys,
+                           int ndim, const int64_t* shape, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RK_H */

@@ -1,0 +1,131 @@
+"""GPU parity of fused broadcast against the oracle, through the C ABI.
+
+Float32 arithmetic is not contracted, so +,-,*,/ match a Float32 host evaluation bit for bit; results
+that involve exp/log/sin/... are compared with the mixed tolerance
+|got - ref| <= 1e-6 * (|a x| + |y e^w|) + 1e-5 * |ref| against Float64."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+def _axpby_check(rk, orc, a, x, y, w):
+    z = rk.ROCArray(dims=x.shape, dtype=np.float32)
+    L = rk.lazy
+    out = rk.materialize_(z, a * L(rk.ROCArray(x)) + L(rk.ROCArray(y)) * rk.broadcast.exp(L(rk.ROCArray(w))))
+    assert out is z
+    got = rk.Array(z).astype(np.float64)
+    ref = orc.broadcast_axpby_exp(a, x, y, w)
+    x64, y64, w64 = (v.astype(np.float64) for v in (x, y, w))
+    bound = 1e-6 * (np.abs(float(a) * x64) + np.abs(y64 * np.exp(w64))) + 1e-5 * np.abs(ref)
+    assert np.all(np.abs(got - ref) <= bound)
+
+
+@pytest.mark.parametrize("shape", [(1,), (5,), (64,), (1000,), (4096,), (33, 7), (32, 16, 8), (100, 100, 10), (3, 5, 7, 2)])
+def test_axpby_exp_shapes(rk, orc, shape):
+    rng = _rng(40)
+    x, y, w = (rng.standard_normal(shape, dtype=np.float32) for _ in range(3))
+    _axpby_check(rk, orc, np.float32(0.5), x, y, w)
+
+
+def test_config4a_full_size(rk, orc):
+    c = orc.config_inputs("bcast_axpby_exp")
+    _axpby_check(rk, orc, c["a"], c["x"], c["y"], c["w"])
+
+
+@pytest.mark.parametrize("m,n", [(4, 4), (5, 3), (64, 64), (100, 1000), (1000, 100), (1024, 37), (3, 100_000)])
+def test_rowcol(rk, orc, m, n):
+    rng = _rng(41)
+    u = lambda *s: (rng.random(s, dtype=np.float32) * 2 - 1).astype(np.float32)
+    A, r, c = u(m, n), u(1, n), u(m, 1)
+    C = rk.ROCArray(dims=(m, n), dtype=np.float32)
+    L = rk.lazy
+    rk.materialize_(C, L(rk.ROCArray(A)) + L(rk.ROCArray(r)) * L(rk.ROCArray(c)))
+    got = rk.Array(C)
+    assert np.array_equal(got, A + r * c)            # un-contracted Float32: bit-exact with a Float32 host evaluation
+    np.testing.assert_allclose(got, orc.broadcast_rowcol(A, r, c), rtol=1e-6, atol=1e-7)
+
+
+def test_config4b_full_size(rk, orc):
+    c = orc.config_inputs("bcast_rowcol")
+    L = rk.lazy
+    C = rk.materialize(L(rk.ROCArray(c["A"])) + L(rk.ROCArray(c["r"])) * L(rk.ROCArray(c["c"])))
+    assert np.array_equal(rk.Array(C), c["A"] + c["r"] * c["c"])
+
+
+def test_reference_broadcast_cases(rk, orc):
+    """test/core/rocarray_broadcast.jl:5-28, the cases inside the enumerated op set."""
+    L, B = rk.lazy, rk.broadcast
+    rng = _rng(42)
+    x = rng.random((3, 3))
+    d = rk.ROCArray(x.copy())
+    assert np.array_equal(rk.Array(rk.fill_(d, 1)), np.ones((3, 3)))                      # fill!(x, 1)
+    a, b = rng.random((2, 3)), rng.random((2, 3))
+    assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(a)) + L(rk.ROCArray(b)))), a + b)   # map(+, x, y)
+    np.testing.assert_allclose(rk.Array(rk.materialize(B.sin(L(rk.ROCArray(a))))), np.sin(a), rtol=1e-14)
+    np.testing.assert_allclose(rk.Array(rk.materialize(B.log(L(rk.ROCArray(a))) + 1)), np.log(a) + 1, rtol=1e-14)
+    assert np.array_equal(rk.Array(rk.materialize(2 * L(rk.ROCArray(a)))), 2 * a)          # 2x
+    np.testing.assert_allclose(rk.Array(rk.materialize(L(rk.ROCArray(a)) ** 3)), a ** 3, rtol=1e-13)
+    np.testing.assert_allclose(rk.Array(rk.materialize(L(rk.ROCArray(a)) ** np.pi)), a ** np.pi, rtol=1e-13)
+    # (2,3) .+ (1,3): row extrusion                                                         :19
+    r = rng.random((1, 3))
+    assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(a)) + L(rk.ROCArray(r)))), a + r)
+    # z .= x .+ y with y a vector extruded along dim 2                                      :20
+    y = rng.random(2)
+    z = rk.ROCArray(rng.random((2, 3)))
+    rk.materialize_(z, L(rk.ROCArray(a)) + L(rk.ROCArray(y)))
+    assert np.array_equal(rk.Array(z), a + y[:, None])
+    # Int + Float64 promotes to Float64                                                     :22
+    got = rk.materialize(L(rk.ROCArray(np.array([1, 2, 3]))) + L(rk.ROCArray(np.array([1.0, 2.0, 3.0]))))
+    assert got.dtype == np.float64 and np.array_equal(rk.Array(got), [2, 4, 6])
+    # Ref(1) scalar operand: log.(x .+ xs)                                                  :38
+    np.testing.assert_allclose(rk.Array(rk.materialize(B.log(1 + L(rk.ROCArray(x))))), np.log(1 + x), rtol=1e-14)
+    # benchmark broadcast: gpu_mat .= 0f0 (perf/array.jl:67)
+    g = rk.ROCArray(rng.random((512, 1000), dtype=np.float32))
+    rk.fill_(g, np.float32(0))
+    assert not rk.Array(g).any()
+
+
+def test_interpreter_general_expression(rk, orc):
+    L, B = rk.lazy, rk.broadcast
+    rng = _rng(43)
+    a, b, c = (rng.random((37, 11), dtype=np.float32) + np.float32(0.5) for _ in range(3))
+    col = rng.random((37, 1), dtype=np.float32)
+    da, db, dc, dcol = (rk.ROCArray(v) for v in (a, b, c, col))
+    expr = B.sqrt(L(da) * L(db) + L(dc)) / (L(dcol) + np.float32(2)) - B.max_(L(da), L(db)) * B.abs2(L(dc))
+    got = rk.Array(rk.materialize(expr))
+    post = [("arg", 0), ("arg", 1), "mul", ("arg", 2), "add", "sqrt", ("arg", 3), ("arg", 4), "add", "div",
+            ("arg", 0), ("arg", 1), "max", ("arg", 2), "abs2", "mul", "sub"]
+    ref = orc.broadcast_eval(post, [a, b, c, col, np.float32(2)])
+    assert got.dtype == np.float32
+    np.testing.assert_allclose(got, ref, rtol=2e-6, atol=1e-6)
+    # muladd and deep nesting on vector-aligned shapes
+    x = rng.random((64, 32), dtype=np.float32)
+    dx = rk.ROCArray(x)
+    e2 = B.muladd(L(dx), L(dx), B.exp(-(L(dx)))) + B.tanh(L(dx)) * B.cos(L(dx)) - B.inv(L(dx) + np.float32(1))
+    ref2 = x.astype(np.float64) ** 2 + np.exp(-x.astype(np.float64)) + np.tanh(x) * np.cos(x) - 1 / (x.astype(np.float64) + 1)
+    np.testing.assert_allclose(rk.Array(rk.materialize(e2)), ref2, rtol=1e-5, atol=1e-6)
+
+
+def test_dimension_mismatch(rk):
+    L = rk.lazy
+    a = rk.ROCArray(np.zeros((2, 3), dtype=np.float32))
+    b = rk.ROCArray(np.zeros((3, 3), dtype=np.float32))
+    with pytest.raises(rk.DimensionMismatch):
+        rk.materialize(L(a) + L(b))
+    with pytest.raises(rk.DimensionMismatch):
+        rk.materialize_(rk.ROCArray(np.zeros((2,), dtype=np.float32)), L(a) + 1.0)
+
+
+def test_unaligned_and_f64(rk, orc):
+    L = rk.lazy
+    x = _rng(44).random(10_001)
+    d = rk.ROCArray(x)
+    v = d.view_range(2, 10_001)
+    got = rk.materialize(L(v) * 3.0 + 1.0)
+    assert got.dtype == np.float64
+    assert np.array_equal(rk.Array(got), x[1:] * 3.0 + 1.0)

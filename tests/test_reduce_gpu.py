@@ -1,0 +1,227 @@
+"""GPU parity of mapreduce / sum / maximum / findmax against the oracle, through the C ABI.
+
+Tolerances (stated by the task): Float32 sums rtol 1e-5 against a Float64 host sum; integer results and
+findmax values + indices bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL_SUM = 1e-5
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 63, 64, 65, 255, 256, 257, 1000, 4095, 4096, 4097, 65536, 100_003, 1 << 20, (1 << 22) + 7])
+def test_sum_f32_sizes(rk, orc, n):
+    x = _rng(n).random(n, dtype=np.float32)
+    got = rk.sum(rk.ROCArray(x))
+    assert isinstance(got, np.float32)
+    np.testing.assert_allclose(got, orc.sum_(x), rtol=RTOL_SUM)
+
+
+@pytest.mark.parametrize("n", [1, 5, 64, 1000, 4097, 1 << 18, (1 << 21) + 3])
+def test_sum_i32_widens_and_is_exact(rk, orc, n):
+    x = _rng(n).integers(-1000, 1001, n, dtype=np.int32)
+    got = rk.sum(rk.ROCArray(x))
+    assert isinstance(got, np.int64)
+    assert got == orc.sum_(x)
+
+
+def test_sum_i32_needs_int64(rk):
+    # 2^22 * 1000 > 2^31: an Int32 accumulator would wrap
+    x = np.full(1 << 22, 1000, dtype=np.int32)
+    assert rk.sum(rk.ROCArray(x)) == (1 << 22) * 1000
+
+
+def test_config1_full_size(rk, orc):
+    x = orc.config_inputs("sum_f32")["x"]
+    np.testing.assert_allclose(rk.sum(rk.ROCArray(x)), np.sum(x, dtype=np.float64), rtol=RTOL_SUM)
+    xi = orc.config_inputs("sum_i32")["x"]
+    assert rk.sum(rk.ROCArray(xi)) == int(xi.astype(np.int64).sum())
+
+
+def test_reference_doctests(rk):
+    # docs/src/usage/arrays.md:85-89
+    assert rk.sum(rk.ROCArray(np.arange(1, 101, dtype=np.int64))) == 5050
+    assert rk.mapreduce(rk.abs2, rk.add, rk.ROCArray(np.arange(1, 5, dtype=np.int64))) == 30
+    # test/hip_rocarray/multi_gpu.jl:45
+    assert rk.sum(rk.ROCArray(np.ones(16, dtype=np.int64))) == 16
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("op", ["add", "mul", "max", "min"])
+def test_ops_and_dtypes_full(rk, orc, dtype, op):
+    rng = _rng(7)
+    n = 5000
+    if op == "mul":
+        x = (rng.random(n) * 0.02 + 0.99).astype(dtype) if np.dtype(dtype).kind == "f" else rng.integers(-3, 4, n).astype(dtype)
+    else:
+        x = (rng.standard_normal(n) * 100).astype(dtype)
+    got = rk.mapreduce(rk.identity, op, rk.ROCArray(x))
+    want = orc.mapreduce("identity", op, x)
+    assert got.dtype == want.dtype
+    if np.dtype(dtype).kind == "f" and op in ("add", "mul"):
+        np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-3 if op == "add" else 0)
+    else:
+        assert got == want
+
+
+@pytest.mark.parametrize("f", ["identity", "abs2", "abs"])
+def test_maps(rk, orc, f):
+    x = _rng(3).standard_normal(70_001).astype(np.float32)
+    np.testing.assert_allclose(rk.mapreduce(f, "add", rk.ROCArray(x)), orc.mapreduce(f, "add", x), rtol=RTOL_SUM, atol=1e-3)
+    xi = _rng(4).integers(-50, 50, 70_001, dtype=np.int32)
+    assert rk.mapreduce(f, "add_sum", rk.ROCArray(xi)) == orc.mapreduce(f, "add_sum", xi)
+
+
+def test_bool_count(rk, orc):
+    b = _rng(5).random(100_000) < 0.3
+    assert rk.sum(rk.ROCArray(b)) == int(b.sum())
+    assert rk.count(rk.ROCArray(b)) == int(b.sum())
+
+
+def test_unaligned_view(rk, orc):
+    x = _rng(6).random(100_000, dtype=np.float32)
+    d = rk.ROCArray(x)
+    for first, last in [(2, 100_000), (3, 99_999), (4, 77_777), (1, 5)]:
+        np.testing.assert_allclose(rk.sum(d.view_range(first, last)), orc.sum_(x[first - 1:last]), rtol=RTOL_SUM)
+
+
+def test_init_is_folded_in(rk, orc):
+    x = _rng(8).random(10_000, dtype=np.float32)
+    np.testing.assert_allclose(rk.mapreduce("identity", "add", rk.ROCArray(x), init=np.float32(100)), orc.sum_(x) + 100, rtol=RTOL_SUM)
+
+
+def test_empty(rk):
+    e = rk.ROCArray(np.zeros(0, dtype=np.float32))
+    assert rk.sum(e) == 0
+    with pytest.raises(ValueError):
+        rk.maximum(e)
+
+
+def test_maximum_nan_and_signed_zero(rk):
+    x = np.array([1, -0.0, 0.0, -5], dtype=np.float32)
+    assert rk.maximum(rk.ROCArray(np.array([-0.0, 0.0], dtype=np.float32))) == 0 and not np.signbit(rk.maximum(rk.ROCArray(np.array([-0.0, 0.0], dtype=np.float32))))
+    assert np.signbit(rk.minimum(rk.ROCArray(np.array([0.0, -0.0], dtype=np.float32))))
+    y = np.concatenate([_rng(0).random(5000, dtype=np.float32), [np.nan], _rng(1).random(5000, dtype=np.float32)]).astype(np.float32)
+    assert np.isnan(rk.maximum(rk.ROCArray(y))) and np.isnan(rk.minimum(rk.ROCArray(y)))
+    assert rk.maximum(rk.ROCArray(x)) == 1 and rk.minimum(rk.ROCArray(x)) == -5
+
+
+# ---- dimensional reductions ---------------------------------------------------------------------------
+SHAPES_DIMS = [
+    ((7,), 1), ((5, 3), 1), ((5, 3), 2), ((3, 4, 5), 1), ((3, 4, 5), 2), ((3, 4, 5), 3), ((1, 70, 50, 20), 3),
+    ((64, 64), 1), ((64, 64), 2), ((100, 1000), 1), ((100, 1000), 2), ((1000, 100), 1), ((1000, 100), 2),
+    ((512, 1000), 1), ((512, 1000), 2), ((3, 100_000), 1), ((3, 100_000), 2), ((100_000, 3), 1), ((100_000, 3), 2),
+    ((257, 129, 5), 2), ((8, 4096, 3), 2), ((2, 3, 4, 5, 6), 4), ((33, 65), (1, 2)), ((6, 7, 8), (1, 3)),
+    ((6, 7, 8), (2, 3)), ((6, 7, 8), (1, 2)), ((40, 50), 3),
+]
+
+
+@pytest.mark.parametrize("shape,dims", SHAPES_DIMS)
+def test_abs2_sum_dims(rk, orc, shape, dims):
+    A = _rng(11).standard_normal(shape).astype(np.float32)
+    got = rk.mapreduce(rk.abs2, rk.add, rk.ROCArray(A), dims=dims)
+    want = orc.mapreduce("abs2", "add", A, dims=dims)
+    assert got.dims == want.shape
+    np.testing.assert_allclose(rk.Array(got), want, rtol=RTOL_SUM)
+
+
+@pytest.mark.parametrize("shape,dims", SHAPES_DIMS)
+def test_sum_dims_i32_exact(rk, orc, shape, dims):
+    A = _rng(12).integers(-1000, 1001, shape).astype(np.int32)
+    got = rk.sum(rk.ROCArray(A), dims=dims)
+    want = orc.sum_(A, dims=dims)
+    assert got.dtype == np.int64 and got.dims == want.shape
+    assert np.array_equal(rk.Array(got), want)
+
+
+@pytest.mark.parametrize("shape,dims", SHAPES_DIMS)
+def test_maximum_dims_exact(rk, orc, shape, dims):
+    A = _rng(13).standard_normal(shape).astype(np.float32)
+    assert np.array_equal(rk.Array(rk.maximum(rk.ROCArray(A), dims=dims)), orc.maximum(A, dims=dims))
+    assert np.array_equal(rk.Array(rk.minimum(rk.ROCArray(A), dims=dims)), orc.minimum(A, dims=dims))
+
+
+def _check_findminmax(rk, orc, A, dims):
+    dA = rk.ROCArray(A)
+    for gpu, cpu in ((rk.findmax, orc.findmax), (rk.findmin, orc.findmin)):
+        gv, gi = gpu(dA, dims=dims)
+        ov, oi = cpu(A, dims=dims)
+        if dims is None:
+            assert (gv == ov or (np.isnan(gv) and np.isnan(ov))) and gi == oi
+            assert np.signbit(gv) == np.signbit(ov)
+        else:
+            assert np.array_equal(rk.Array(gv), ov, equal_nan=True)
+            assert np.array_equal(np.signbit(rk.Array(gv)), np.signbit(ov))
+            assert np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
+
+
+@pytest.mark.parametrize("shape,dims", SHAPES_DIMS + [((1000,), None), ((50, 60), None), ((1 << 20,), None)])
+def test_findminmax_dims(rk, orc, shape, dims):
+    rng = _rng(14)
+    # few distinct values -> many ties, so the first-index rule is exercised
+    A = rng.integers(-4, 5, shape).astype(np.float32)
+    _check_findminmax(rk, orc, A, dims)
+    _check_findminmax(rk, orc, rng.standard_normal(shape).astype(np.float32), dims)
+
+
+def test_findmax_nan_and_zero_rules(rk, orc):
+    A = np.array([[1, np.nan, -0.0, 3], [np.nan, 2, 0.0, 3], [5, np.nan, -0.0, -np.inf]], dtype=np.float32)
+    for dims in (1, 2, None):
+        _check_findminmax(rk, orc, A, dims)
+    big = _rng(15).standard_normal((300, 70)).astype(np.float32)
+    big[17, 3] = np.nan
+    big[200, 3] = np.nan
+    big[5, 9] = np.nan
+    for dims in (1, 2, None):
+        _check_findminmax(rk, orc, big, dims)
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.int32, np.int64])
+def test_findmax_other_dtypes(rk, orc, dtype):
+    A = _rng(16).integers(-100, 100, (65, 130)).astype(dtype)
+    for dims in (1, 2, None):
+        _check_findminmax(rk, orc, A, dims)
+
+
+def test_config2_full_size(rk, orc):
+    A = orc.config_inputs("dims_f32")["A"]
+    dA = rk.ROCArray(A)
+    A64 = A.astype(np.float64)
+    for d in (1, 2):
+        got = rk.Array(rk.mapreduce(rk.abs2, rk.add, dA, dims=d))
+        np.testing.assert_allclose(got, (A64 * A64).sum(axis=d - 1, keepdims=True), rtol=RTOL_SUM)
+    v, i = rk.findmax(dA, dims=1)
+    v, i = rk.Array(v), rk.Array(i)
+    assert np.array_equal(v, A.max(axis=0, keepdims=True))
+    assert np.array_equal(i[0, 0, :], A.argmax(axis=0) + 1)
+    assert np.array_equal(i[1, 0, :], np.arange(1, A.shape[1] + 1))
+
+
+def test_mapreducedim_returns_R_and_pads_dims(rk):
+    # test/core/rocarray_base.jl:263-267: R of size (3, 2) reduces A of size (3, 2, 10) over dim 3
+    A = _rng(17).random((3, 2, 10), dtype=np.float32)
+    R = rk.zeros(np.float32, 3, 2)
+    out = rk.mapreducedim_(rk.identity, rk.add, R, rk.ROCArray(A))
+    assert out is R
+    np.testing.assert_allclose(rk.Array(R), A.astype(np.float64).sum(axis=2), rtol=RTOL_SUM)
+    with pytest.raises(rk.DimensionMismatch):
+        rk.mapreducedim_(rk.identity, rk.add, rk.zeros(np.float32, 2, 2), rk.ROCArray(A))
+
+
+def test_repeated_calls_reuse_clean_workspace(rk, orc):
+    # the multi-workgroup kernels must leave their tickets clean
+    x = _rng(18).random(1 << 21, dtype=np.float32)
+    d = rk.ROCArray(x)
+    first = rk.sum(d)
+    for _ in range(5):
+        assert rk.sum(d) == first          # deterministic: same launch geometry, fixed combine order
+    A = _rng(19).standard_normal((2048, 512)).astype(np.float32)
+    dA = rk.ROCArray(A)
+    r0 = rk.Array(rk.sum(dA, dims=2))
+    for _ in range(3):
+        assert np.array_equal(rk.Array(rk.sum(dA, dims=2)), r0)

@@ -1,0 +1,157 @@
+"""GPU parity of accumulate / cumsum / cumprod / findall against the oracle, through the C ABI.
+
+Tolerances: integer scans bit-exact (wraparound); Float32 scans rtol 1e-4 against a Float64 host scan
+(atol covers prefixes that pass near zero)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+SIZES = [0, 1, 2, 3, 10, 63, 64, 65, 1000, 4095, 4096, 4097, 8192, 10_000, 16384, 16385, 100_003, (1 << 20) + 5]
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_accumulate_f64_sizes(rk, orc, n):
+    # test/core/rocarray_base.jl:194-201 (Float64, with and without init)
+    x = _rng(n).random(n)
+    d = rk.ROCArray(x)
+    np.testing.assert_allclose(rk.Array(rk.accumulate("add", d)), orc.accumulate("add", x), rtol=1e-12)
+    init = 0.37
+    np.testing.assert_allclose(rk.Array(rk.accumulate("add", d, init=init)), orc.accumulate("add", x, init=init), rtol=1e-12)
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_cumsum_i32_exact(rk, orc, n):
+    x = _rng(n + 1).integers(-1000, 1001, n, dtype=np.int32)
+    got = rk.cumsum(rk.ROCArray(x))
+    assert got.dtype == np.int32
+    assert np.array_equal(rk.Array(got), orc.cumsum(x))
+
+
+def test_cumsum_i32_wraps(rk, orc):
+    x = np.full(100_000, 2_000_000_000, dtype=np.int32)
+    want = np.cumsum(x.astype(np.int64)).astype(np.uint64).astype(np.uint32).view(np.int32)   # mod 2^32
+    assert np.array_equal(orc.cumsum(x), want)
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(x))), want)
+
+
+@pytest.mark.parametrize("n", [1, 100, 4096, 4097, 50_000, (1 << 19) + 1])
+def test_cumsum_f32(rk, orc, n):
+    x = _rng(n).random(n, dtype=np.float32)
+    want = orc.cumsum(x)
+    np.testing.assert_allclose(rk.Array(rk.cumsum(rk.ROCArray(x))), want, rtol=RTOL)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.int64])
+@pytest.mark.parametrize("op", ["add", "mul", "max", "min"])
+@pytest.mark.parametrize("inclusive", [True, False])
+def test_ops_dtypes_exclusive(rk, orc, dtype, op, inclusive):
+    rng = _rng(21)
+    n = 20_000
+    if op == "mul":
+        x = (rng.random(n) * 0.002 + 0.999).astype(dtype) if np.dtype(dtype).kind == "f" else rng.integers(-2, 3, n).astype(dtype)
+        init = 2
+    else:
+        x = (rng.standard_normal(n) * 50).astype(dtype)
+        init = 3
+    got = rk.Array(rk.accumulate(op, rk.ROCArray(x), init=init, inclusive=inclusive))
+    want = orc.accumulate(op, x, init=init, inclusive=inclusive)
+    if np.dtype(dtype).kind == "f" and op in ("add", "mul"):
+        np.testing.assert_allclose(got, want, rtol=RTOL if dtype == np.float32 else 1e-11, atol=2e-2 if (op == "add" and dtype == np.float32) else 1e-9)
+    else:
+        assert np.array_equal(got, want.astype(dtype))
+
+
+DIM_CASES = [
+    ((2,), 2), ((3, 4, 5), 2), ((1, 70, 50, 20), 3),            # test/core/rocarray_base.jl:204-213
+    ((3, 4, 5), 1), ((3, 4, 5), 3), ((64, 64), 1), ((64, 64), 2), ((100, 1000), 1), ((100, 1000), 2),
+    ((512, 1000), 1), ((512, 1000), 2), ((3, 100_000), 1), ((3, 100_000), 2), ((100_000, 3), 1), ((100_000, 3), 2),
+    ((4096, 33), 1), ((4100, 33), 1), ((9000, 7), 1), ((257, 129, 5), 2), ((256, 40, 3), 2), ((40, 50), 3),
+    ((1024, 300), 1), ((1000, 300), 1), ((300, 70), 1), ((20, 5000), 1),
+]
+
+
+@pytest.mark.parametrize("shape,dims", DIM_CASES)
+def test_accumulate_dims_i64_exact(rk, orc, shape, dims):
+    x = _rng(22).integers(-10**12, 10**12, shape, dtype=np.int64)
+    assert np.array_equal(rk.Array(rk.accumulate("add", rk.ROCArray(x), dims=dims)), orc.accumulate("add", x, dims=dims))
+
+
+@pytest.mark.parametrize("shape,dims", DIM_CASES)
+def test_cumsum_dims_f32(rk, orc, shape, dims):
+    x = _rng(23).random(shape, dtype=np.float32)
+    np.testing.assert_allclose(rk.Array(rk.cumsum(rk.ROCArray(x), dims=dims)), orc.cumsum(x, dims=dims), rtol=RTOL)
+
+
+@pytest.mark.parametrize("shape,dims", [((3, 4, 5), 2), ((4096, 9), 1), ((9000, 3), 1), ((130, 70), 2)])
+def test_exclusive_with_init_dims(rk, orc, shape, dims):
+    x = _rng(24).integers(-100, 100, shape, dtype=np.int32)
+    got = rk.Array(rk.accumulate("add", rk.ROCArray(x), dims=dims, init=7, inclusive=False))
+    assert np.array_equal(got, orc.accumulate("add", x, dims=dims, init=7, inclusive=False))
+
+
+def test_in_place(rk, orc):
+    # test/core/rocarray_base.jl:216-220
+    x = _rng(25).random(2)
+    d = rk.ROCArray(x)
+    out = rk.accumulate_("add", d, d)
+    assert out is d
+    np.testing.assert_allclose(rk.Array(d), np.cumsum(x))
+    y = _rng(26).integers(-1000, 1000, 1 << 18, dtype=np.int32)
+    dy = rk.ROCArray(y)
+    rk.accumulate_("add", dy, dy)
+    assert np.array_equal(rk.Array(dy), orc.cumsum(y))
+
+
+def test_cumprod_and_doctest(rk, orc):
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(np.array([1, 2, 3, 4])))), [1, 3, 6, 10])   # arrays.md:91-96
+    x = _rng(27).random(2)
+    np.testing.assert_allclose(rk.Array(rk.cumprod(rk.ROCArray(x))), np.cumprod(x))
+
+
+def test_unaligned_view_scan(rk, orc):
+    x = _rng(28).integers(-1000, 1000, 50_001, dtype=np.int32)
+    d = rk.ROCArray(x)
+    v = d.view_range(2, 50_001)
+    assert np.array_equal(rk.Array(rk.cumsum(v)), orc.cumsum(x[1:]))
+
+
+def test_repeated_scans_bump_generation(rk, orc):
+    # many look-back scans in a row through one workspace: stale descriptors must never be accepted
+    rng = _rng(29)
+    for it in range(12):
+        n = int(rng.integers(5000, 300_000))
+        x = rng.integers(-1000, 1001, n, dtype=np.int32)
+        assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(x))), orc.cumsum(x)), (it, n)
+
+
+def test_config3_full_size(rk, orc):
+    x = orc.config_inputs("cumsum_i32")["x"]                      # 2^27 Int32
+    got = rk.Array(rk.cumsum(rk.ROCArray(x)))
+    assert np.array_equal(got, np.cumsum(x, dtype=np.int32))
+    del got
+    B = orc.config_inputs("cumsum_f32_dims1")["B"]                # 4096 x 16384 Float32
+    got = rk.Array(rk.cumsum(rk.ROCArray(B), dims=1))
+    np.testing.assert_allclose(got, np.cumsum(B.astype(np.float64), axis=0), rtol=RTOL)
+
+
+def test_bool_scan_and_findall(rk, orc):
+    b = _rng(30).random(100_000) < 0.25
+    got = rk.cumsum(rk.ROCArray(b))
+    assert got.dtype == np.int64
+    assert np.array_equal(rk.Array(got), np.cumsum(b))
+    assert np.array_equal(rk.Array(rk.findall(rk.ROCArray(b))), orc.findall(b))
+    # test/hip_rocarray/indexing.jl:5-18 shapes
+    for shape in [(16,), (1, 16), (3, 1, 16), (33, 65)]:
+        m = _rng(31).random(shape) < 0.5
+        got = rk.Array(rk.findall(rk.ROCArray(m)))
+        want = orc.findall(m)
+        assert np.array_equal(got if m.ndim == 1 else got.T, want)
+    assert len(rk.findall(rk.ROCArray(np.zeros(100, dtype=bool)))) == 0
