@@ -10,6 +10,12 @@ from __future__ import annotations
 import ctypes as C
 import os
 
+# PyTorch supplies device memory and streams on this side of the ABI, and it ships its own HIP
+# runtime (libamdhip64.so.7).  It must be in the process BEFORE librk.so is opened so that the
+# loader binds librk.so to that same runtime instance; two runtimes in one process do not share
+# devices or streams.  (A Julia host binds librk.so to the runtime AMDGPU.jl already loaded.)
+import torch  # noqa: F401  (import order matters)
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "librk.so")
 
