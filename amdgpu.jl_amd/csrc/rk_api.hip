@@ -2,6 +2,7 @@
 // element types, workspace management.  The kernels live in rk_*_impl.hpp / rk_*.hip.
 #include <atomic>
 #include <cstdlib>
+#include <cstddef>
 #include <cstring>
 
 #include "rk_common.hpp"
@@ -35,6 +36,18 @@ static int env_int(const char* name, int dflt, int lo, int hi) {
 // Workgroups per compute unit the multi-workgroup reductions aim for (RK_REDUCE_BLOCKS_PER_CU).
 int tune_reduce_blocks_per_cu() {
     static const int v = env_int("RK_REDUCE_BLOCKS_PER_CU", 8, 1, 64);
+    return v;
+}
+
+// Look-back polling back-off of the scan, in units of 512 clocks (RK_SCAN_BACKOFF).
+int tune_scan_backoff() {
+    static const int v = env_int("RK_SCAN_BACKOFF", 1, 0, 64);
+    return v;
+}
+
+// Persistent workgroups per compute unit of the look-back scan (RK_SCAN_BLOCKS_PER_CU).
+int tune_scan_blocks_per_cu() {
+    static const int v = env_int("RK_SCAN_BLOCKS_PER_CU", 6, 1, 16);
     return v;
 }
 
@@ -82,9 +95,9 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
         // descriptors of the look-back scan: one tagged word per 4 bytes of the value, per tile
         const Shape3 s = collapse3(ndim, shape, dims_mask);
         const size_t esz = dtype_size(dt) < 4 ? 4 : dtype_size(dt);
-        const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 4;
-        const int64_t tpl = (s.mid + tile - 1) / tile;
-        if (s.inner == 1 && tpl > 1) need += (size_t)(tpl * s.outer) * (esz / 4) * sizeof(uint64_t);
+        const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 8;           // ScanTile<T>::TILE
+        const int64_t tpl = (s.mid + tile - 1) / tile, gpl = (tpl + WAVE - 1) / WAVE;
+        if (s.inner == 1 && tpl > 1) need += (size_t)((tpl + gpl) * s.outer) * (esz / 4) * sizeof(uint64_t);
     }
     return (need + 255) & ~(size_t)255;
 }
@@ -92,13 +105,13 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
 int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
     if (ws == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (!is_aligned(ws, 256) || ws_bytes < WS_DESC_OFFSET) return RK_ERR_WORKSPACE;
-    // header + tickets to zero, descriptors to zero (tag 0 = never valid), then epoch = first
+    // header + tickets to zero, descriptors to zero (tag 0 = never valid), then the scan epoch = 1:
+    // scan_counter = 1 << 32, i.e. byte 4 of the header (little endian)
     RK_HIP(hipMemsetAsync(ws, 0, WS_PARTIALS_OFFSET, (hipStream_t)stream));
     if (ws_bytes > WS_DESC_OFFSET)
         RK_HIP(hipMemsetAsync((char*)ws + WS_DESC_OFFSET, 0, ws_bytes - WS_DESC_OFFSET, (hipStream_t)stream));
-    const uint32_t first = WS_EPOCH_FIRST;
-    static_assert(WS_EPOCH_FIRST == 1, "the byte-wise memset below writes the value 1");
-    RK_HIP(hipMemsetAsync(ws, (int)first, 1, (hipStream_t)stream));   // little endian: epoch = 1
+    static_assert(WS_EPOCH_FIRST == 1 && offsetof(WsHeader, scan_counter) == 0, "the byte-wise memset below writes epoch 1");
+    RK_HIP(hipMemsetAsync((char*)ws + 4, 1, 1, (hipStream_t)stream));
     return RK_SUCCESS;
 }
 

@@ -52,10 +52,8 @@ const DeviceInfo& device_info();   // rk_api.hip
 // [WS_DESC_OFFSET, end)          tile descriptors of the look-back scan (tagged words; kept apart
 //                                from the partials so arbitrary partial bits never look like a tag)
 struct WsHeader {
-    uint32_t epoch;         // scan generation; descriptors of other generations are stale
-    uint32_t tile_counter;  // dynamic tile ids of the scan
-    uint32_t done_counter;  // tiles finished with their descriptors
-    uint32_t pad[61];
+    uint64_t scan_counter;  // look-back scan: epoch << 32 | tile acquisitions of the running call
+    uint32_t pad[62];
 };
 static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
 
@@ -66,7 +64,6 @@ constexpr size_t WS_PARTIALS_OFFSET = WS_HEADER_BYTES + WS_TICKET_BYTES;
 constexpr size_t WS_PARTIALS_BYTES = (size_t)8 << 20;
 constexpr size_t WS_DESC_OFFSET = WS_PARTIALS_OFFSET + WS_PARTIALS_BYTES;
 constexpr uint32_t WS_EPOCH_FIRST = 1;
-constexpr uint32_t WS_EPOCH_LAST = (1u << 30) - 2;   // after this the scan clears its descriptors
 
 struct Workspace {
     WsHeader* hdr;
@@ -230,6 +227,52 @@ template <typename T> __device__ __forceinline__ T wave_shift_right(T v, T ident
 
 __device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
 
+// ---- hand-off of small values between workgroups ---------------------------------------------
+// Values are written and read word by word with relaxed agent-scope atomics: such accesses are
+// performed at the device-coherent level and need no cache write-back or invalidate.  A full
+// release fence at agent scope writes back the whole L2 of the XCD; issued by thousands of
+// workgroups it costs more than the streaming kernel it sits in.  The writer orders
+// "value, then flag/ticket" with publish_barrier() (waits until its own stores have completed).
+template <typename T> __device__ __forceinline__ void store_agent(T* p, const T& v) {
+    static_assert(sizeof(T) % 4 == 0, "whole words only");
+    if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
+        uint64_t w[sizeof(T) / 8];
+        __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+        for (unsigned i = 0; i < sizeof(T) / 8; ++i)
+            __hip_atomic_store((uint64_t*)p + i, w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        uint32_t w[sizeof(T) / 4];
+        __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+        for (unsigned i = 0; i < sizeof(T) / 4; ++i)
+            __hip_atomic_store((uint32_t*)p + i, w[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+template <typename T> __device__ __forceinline__ T load_agent(const T* p) {
+    static_assert(sizeof(T) % 4 == 0, "whole words only");
+    T v;
+    if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
+        uint64_t w[sizeof(T) / 8];
+#pragma unroll
+        for (unsigned i = 0; i < sizeof(T) / 8; ++i)
+            w[i] = __hip_atomic_load((const uint64_t*)p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&v, w, sizeof(T));
+    } else {
+        uint32_t w[sizeof(T) / 4];
+#pragma unroll
+        for (unsigned i = 0; i < sizeof(T) / 4; ++i)
+            w[i] = __hip_atomic_load((const uint32_t*)p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_memcpy(&v, w, sizeof(T));
+    }
+    return v;
+}
+// All earlier stores of this thread have completed (s_waitcnt vmcnt(0)) before anything later issues.
+__device__ __forceinline__ void publish_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+}
+
 // Reduction over a workgroup of NW waves.  Every thread returns the total.  `lds` must
 // hold NW values of T; safe to call repeatedly (leading barrier protects the buffer).
 template <int NW, typename T, typename Op>
@@ -307,46 +350,71 @@ struct OpMin {
     template <typename T> static __host__ __device__ __forceinline__ T identity() { return Limits<T>::highest(); }
 };
 
-// ---- (value, index) pairs for findmax / findmin ---------------------------------------------
-template <typename T> struct ValIdx {
-    T       v;
+// ---- findmax / findmin: argmax over order-preserving integer keys ------------------------------
+// Base.isless is a total order on floats (-0.0 < 0.0, NaN above everything) and findmax keeps the
+// first maximum; findmin (Base.isgreater) keeps the first minimum but NaN still wins.  Each value
+// is mapped to a signed integer key that is monotone in that order, so the reduction itself is a
+// plain integer argmax with "smaller index wins ties" -- commutative and associative, hence any
+// reduction tree returns what the sequential scan returns.
+template <typename T> struct OrderKey;
+template <> struct OrderKey<float> {
+    typedef int32_t Key;
+    static __device__ __forceinline__ Key make(float v, bool want_max) {
+        const int32_t b = __builtin_bit_cast(int32_t, v);
+        const int32_t k = b ^ ((b >> 31) & 0x7fffffff);       // sign-magnitude -> two's complement
+        return (v != v) ? INT32_MAX : (want_max ? k : ~k);
+    }
+    static __device__ __forceinline__ float value(Key k, bool want_max) {
+        if (k == INT32_MAX) return __builtin_nanf("");
+        const int32_t kk = want_max ? k : ~k;
+        return __builtin_bit_cast(float, kk ^ ((kk >> 31) & 0x7fffffff));
+    }
+};
+template <> struct OrderKey<double> {
+    typedef int64_t Key;
+    static __device__ __forceinline__ Key make(double v, bool want_max) {
+        const int64_t b = __builtin_bit_cast(int64_t, v);
+        const int64_t k = b ^ ((b >> 63) & INT64_MAX);
+        return (v != v) ? INT64_MAX : (want_max ? k : ~k);
+    }
+    static __device__ __forceinline__ double value(Key k, bool want_max) {
+        if (k == INT64_MAX) return __builtin_nan("");
+        const int64_t kk = want_max ? k : ~k;
+        return __builtin_bit_cast(double, kk ^ ((kk >> 63) & INT64_MAX));
+    }
+};
+template <> struct OrderKey<int32_t> {
+    typedef int32_t Key;
+    static __device__ __forceinline__ Key make(int32_t v, bool want_max) { return want_max ? v : ~v; }
+    static __device__ __forceinline__ int32_t value(Key k, bool want_max) { return want_max ? k : ~k; }
+};
+template <> struct OrderKey<int64_t> {
+    typedef int64_t Key;
+    static __device__ __forceinline__ Key make(int64_t v, bool want_max) { return want_max ? v : ~v; }
+    static __device__ __forceinline__ int64_t value(Key k, bool want_max) { return want_max ? k : ~k; }
+};
+
+template <typename K> struct KeyIdx {
+    K       k;
     int64_t i;     // 0-based column-major linear index into A; -1 = nothing yet
 };
 
-// Base.isless total order on values: -0.0 < 0.0 and NaN above everything.
-template <typename T> __host__ __device__ __forceinline__ bool total_less(T a, T b) {
-    if constexpr (std::is_floating_point<T>::value) {
-        const bool an = a != a, bn = b != b;
-        if (an || bn) return !an && bn;
-        if (a == b) return __builtin_signbit(a) && !__builtin_signbit(b);
-        return a < b;
-    } else return a < b;
-}
-
-// findmax: larger under isless wins, ties -> smaller index.  findmin (Base.isgreater):
-// NaN still wins, otherwise the smaller value, ties -> smaller index.  Commutative and
-// associative, so any reduction tree gives the sequential answer.
-template <bool WANT_MAX> struct OpArg {
-    template <typename T> __host__ __device__ __forceinline__ ValIdx<T> operator()(ValIdx<T> a, ValIdx<T> b) const {
+struct OpArgKey {
+    template <typename K> __host__ __device__ __forceinline__ KeyIdx<K> operator()(KeyIdx<K> a, KeyIdx<K> b) const {
         if (a.i < 0) return b;
         if (b.i < 0) return a;
-        bool a_better, b_better;
-        if constexpr (WANT_MAX) {
-            a_better = total_less(b.v, a.v);
-            b_better = total_less(a.v, b.v);
-        } else {
-            if constexpr (std::is_floating_point<T>::value) {
-                const bool an = a.v != a.v, bn = b.v != b.v;
-                if (an || bn) { a_better = an && !bn; b_better = bn && !an; }
-                else { a_better = total_less(a.v, b.v); b_better = total_less(b.v, a.v); }
-            } else { a_better = a.v < b.v; b_better = b.v < a.v; }
-        }
-        if (a_better) return a;
-        if (b_better) return b;
+        if (a.k != b.k) return a.k > b.k ? a : b;
         return a.i < b.i ? a : b;
     }
-    template <typename P> static __host__ __device__ __forceinline__ P identity() { P p; p.v = 0; p.i = -1; return p; }
+    template <typename P> static __host__ __device__ __forceinline__ P identity() { P p; p.k = 0; p.i = -1; return p; }
 };
+
+// One step of a streaming accumulation: `x` comes later in index order than everything already in
+// `acc`.  Generic operators just combine; the argmax only replaces on a strictly larger key.
+template <typename Op, typename A> __device__ __forceinline__ A acc_step(Op op, const A& acc, const A& x) { return op(acc, x); }
+template <typename K> __device__ __forceinline__ KeyIdx<K> acc_step(OpArgKey, const KeyIdx<K>& acc, const KeyIdx<K>& x) {
+    return (acc.i < 0 || x.k > acc.k) ? x : acc;
+}
 
 }  // namespace rk
 #endif  // __HIPCC__

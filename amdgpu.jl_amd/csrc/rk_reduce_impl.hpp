@@ -40,7 +40,9 @@ template <typename In, typename Acc, typename Map> struct MapXform {
     __device__ __forceinline__ Acc operator()(In x, int64_t) const { return (Acc)Map()(x); }
 };
 template <typename T> struct ArgXform {
-    __device__ __forceinline__ ValIdx<T> operator()(T x, int64_t idx) const { ValIdx<T> p; p.v = x; p.i = idx; return p; }
+    bool want_max;
+    typedef KeyIdx<typename OrderKey<T>::Key> P;
+    __device__ __forceinline__ P operator()(T x, int64_t idx) const { P p; p.k = OrderKey<T>::make(x, want_max); p.i = idx; return p; }
 };
 
 // ---- result sinks ---------------------------------------------------------------------------
@@ -55,8 +57,9 @@ template <typename T> struct ArgSink {
     int64_t* cart;
     int      ndim;
     int64_t  shape[RK_MAX_DIMS];
-    __device__ __forceinline__ void operator()(int64_t q, ValIdx<T> t) const {
-        if (vals) vals[q] = t.v;
+    bool     want_max;
+    __device__ __forceinline__ void operator()(int64_t q, KeyIdx<typename OrderKey<T>::Key> t) const {
+        if (vals) vals[q] = OrderKey<T>::value(t.k, want_max);
         if (cart) {
             int64_t rem = t.i;
             for (int d = 0; d < ndim; ++d) {
@@ -86,9 +89,10 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
         const int64_t nvec = (n - head) / VEC;
         const V* pv = (const V*)(p + head);
         const int64_t tail = head + nvec * VEC;
+        Acc edge = Op::template identity<Acc>();   // kept apart: the vector body below must see increasing indices
         if (s == 0) {   // fewer than VEC (<= 16 <= GROUP) scalars on either side
-            if (t < head) acc[0] = op(acc[0], xf(p[t], base + t));
-            if (tail + t < n) acc[0] = op(acc[0], xf(p[tail + t], base + tail + t));
+            if (t < head) edge = op(edge, xf(p[t], base + t));
+            if (tail + t < n) edge = op(edge, xf(p[tail + t], base + tail + t));
         }
         constexpr int64_t CHUNK = (int64_t)GROUP * UNROLL;
         const int64_t nchunks = nvec / CHUNK;
@@ -101,18 +105,18 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
             for (int u = 0; u < UNROLL; ++u) {
                 const int64_t e0 = base + head + (i0 + (int64_t)u * GROUP) * VEC;
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[u][j], e0 + j));
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0 + j));
             }
         }
         for (int64_t i = nchunks * CHUNK + (int64_t)s * GROUP + t; i < nvec; i += (int64_t)splits * GROUP) {
             const V v = load_nt(pv + i);
             const int64_t e0 = base + head + i * VEC;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[j], e0 + j));
+            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0 + j));
         }
-        Acc a = acc[0];
+        Acc a = edge;
 #pragma unroll
-        for (int j = 1; j < VEC; ++j) a = op(a, acc[j]);
+        for (int j = 0; j < VEC; ++j) a = op(a, acc[j]);
         return a;
     } else {
         Acc acc[UNROLL];
@@ -125,9 +129,9 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) v[u] = A[base + (k + u * step) * stride];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) acc[u] = op(acc[u], xf(v[u], base + (k + u * step) * stride));
+            for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], base + (k + u * step) * stride));
         }
-        for (; k < n; k += step) acc[0] = op(acc[0], xf(A[base + k * stride], base + k * stride));
+        for (; k < n; k += step) acc[0] = acc_step(op, acc[0], xf(A[base + k * stride], base + k * stride));
         Acc a = acc[0];
 #pragma unroll
         for (int u = 1; u < UNROLL; ++u) a = op(a, acc[u]);
@@ -152,15 +156,15 @@ __global__ __launch_bounds__(BLOCK) void reduce_split_kernel(const In* __restric
         return;
     }
     if (t == 0) {
-        partials[line * splits + s] = a;
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[line], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        store_agent(&partials[line * splits + s], a);
+        publish_barrier();      // the partial is at the coherent level before the ticket moves
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[line], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (old == (uint32_t)splits - 1u);
     }
     __syncthreads();
     if (!is_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     Acc r = Op::template identity<Acc>();
-    for (int i = t; i < splits; i += BLOCK) r = op(r, partials[line * splits + i]);
+    for (int i = t; i < splits; i += BLOCK) r = op(r, load_agent(&partials[line * splits + i]));
     r = block_reduce<NW>(r, op, lds);
     if (t == 0) {
         sink(line, r);
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
     if (line >= g.nlines) return;
     const int64_t base = line_base(g, line);
     Acc a = Op::template identity<Acc>();
-    for (int64_t k = 0; k < g.mid; ++k) a = op(a, xf(A[base + k * g.inner], base + k * g.inner));
+    for (int64_t k = 0; k < g.mid; ++k) a = acc_step(op, a, xf(A[base + k * g.inner], base + k * g.inner));
     sink(line, a);
 }
 
@@ -225,20 +229,20 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const int64_t e0 = slab + (m + u * NW) * g.inner + col0;
-                if constexpr (VEC == 1) acc[0] = op(acc[0], xf(v[u], e0));
+                if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
                 else {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[u][j], e0 + j));
+                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0 + j));
                 }
             }
         }
         for (; m < m1; m += NW) {
             const V v = load_nt((const V*)(A + slab + m * g.inner + col0));
             const int64_t e0 = slab + m * g.inner + col0;
-            if constexpr (VEC == 1) acc[0] = op(acc[0], xf(v, e0));
+            if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v, e0));
             else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], xf(v[j], e0 + j));
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0 + j));
             }
         }
     }
@@ -259,18 +263,20 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     }
     // partials[(o * strips + strip) * msplits + ms][COLS]
     const int64_t tile = o * gridDim.x + strip;
-    if (t < COLS) partials[(tile * msplits + ms) * COLS + t] = r;
-    __syncthreads();   // all partial stores of this workgroup are issued before the release below
+    if (t < COLS) {
+        store_agent(&partials[(tile * msplits + ms) * COLS + t], r);
+        publish_barrier();
+    }
+    __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
     if (t == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (old == (uint32_t)msplits - 1u);
     }
     __syncthreads();
     if (!is_last) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (t < COLS && col < g.inner) {
         Acc f = Op::template identity<Acc>();
-        for (int i = 0; i < msplits; ++i) f = op(f, partials[(tile * msplits + i) * COLS + t]);
+        for (int i = 0; i < msplits; ++i) f = op(f, load_agent(&partials[(tile * msplits + i) * COLS + t]));
         sink(col + o * g.inner, f);
     }
     if (t == 0) tickets[tile] = 0;
@@ -484,9 +490,10 @@ inline int32_t findminmax_typed(const FindArgs& a) {
     sink.cart = a.cart;
     sink.ndim = a.ndim;
     for (int d = 0; d < a.ndim; ++d) sink.shape[d] = a.shape[d];
-    if (a.want_max)
-        return launch_reduce<T, ValIdx<T>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T>(), OpArg<true>(), sink, a.ws, a.ws_bytes, a.stream);
-    return launch_reduce<T, ValIdx<T>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T>(), OpArg<false>(), sink, a.ws, a.ws_bytes, a.stream);
+    sink.want_max = a.want_max != 0;
+    ArgXform<T> xf{a.want_max != 0};
+    return launch_reduce<T, KeyIdx<typename OrderKey<T>::Key>>((const T*)a.A, a.ndim, a.shape, a.mask, xf, OpArgKey(), sink, a.ws,
+                                                               a.ws_bytes, a.stream);
 }
 
 // one translation unit per type pair (keeps compile times parallel)

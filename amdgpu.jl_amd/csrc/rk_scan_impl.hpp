@@ -34,50 +34,84 @@ __device__ __forceinline__ void desc_publish(uint64_t* desc, int64_t stride, int
                            __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Exclusive prefix of `tile` inside its line; executed by one full wave, result wave-uniform.
-// `tl` = number of predecessors the tile has in its line.
+// Reads one descriptor value; returns its status (0 = not of this call / not yet written).
+template <typename T>
+__device__ __forceinline__ uint32_t desc_read(const uint64_t* desc, int64_t stride, int64_t idx, uint32_t tagA, uint32_t tagP,
+                                              Words<T>& val) {
+    uint32_t status = 0;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) {
+        const uint64_t d = __hip_atomic_load(&desc[i * stride + idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t tag = (uint32_t)(d >> 32);
+        val.w[i] = (uint32_t)d;
+        const uint32_t st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
+        status = (i == 0) ? st : (st == status ? st : 0u);
+    }
+    return status;
+}
+
+// Two-level decoupled look-back; executed by one full wave, returns the wave-uniform exclusive
+// prefix of `tile` inside its line.
+//
+// With one level, a tile can only finish once it sees an *inclusive* prefix within the 64
+// descriptors it polls at a time, so inclusive prefixes advance at most 64 tiles per poll round trip
+// (a device-coherent load: microseconds under load) -- far below the tile rate 8 TB/s needs.  Here
+// the tiles of a line form groups of 64.  A tile sums the plain aggregates of the predecessors inside
+// its group (they depend on nobody, so they appear as soon as those tiles have read their data), and
+// takes the rest from group descriptors: the last tile of a group publishes the group aggregate (GA)
+// as soon as its in-group sum is complete and the inclusive prefix at the group end (GP) when it has
+// its own prefix.  One poll of 64 group descriptors spans 4096 tiles, so the two polls (issued
+// together) normally resolve in one or two round trips whatever the distance to the nearest
+// inclusive prefix.
+//   tl   index of the tile in its line          gl   global index of the tile's group
+//   agg  aggregate of this tile (already published by the caller as the tile's descriptor)
 template <typename T, typename Op>
-__device__ __forceinline__ T desc_lookback(const uint64_t* desc, int64_t stride, int64_t tile, int64_t tl, uint32_t epoch,
-                                           Op op, T ident) {
+__device__ __forceinline__ T desc_lookback2(uint64_t* tile_desc, int64_t tstride, uint64_t* group_desc, int64_t gstride,
+                                            int64_t tile, int64_t tl, int64_t gl, uint32_t epoch, T agg, T init, Op op, T ident, int backoff) {
     const int lane = lane_id();
     const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
-    T prefix = ident;
-    int64_t first = tile - 1;   // nearest predecessor of the current window
-    int64_t remaining = tl;
-    while (true) {
-        const bool in_line = lane < remaining;
-        const int64_t p = first - lane;
-        uint32_t status;
-        Words<T> val;
-        int np;
-        while (true) {
-            if (in_line) {
-                status = 0;
-#pragma unroll
-                for (int i = 0; i < Words<T>::N; ++i) {
-                    const uint64_t d = __hip_atomic_load(&desc[i * stride + p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    const uint32_t tag = (uint32_t)(d >> 32);
-                    val.w[i] = (uint32_t)d;
-                    const uint32_t st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
-                    status = (i == 0) ? st : (st == status ? st : 0u);
-                }
-            } else {            // before the start of the line: terminates the search
-                status = DESC_P;
-                val = to_words(ident);
-            }
-            const uint64_t ballotP = __ballot(status == DESC_P);
-            const uint64_t ballotX = __ballot(status == 0u);
-            np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
-            const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
-            if ((ballotX & needed) == 0) break;
-            __builtin_amdgcn_s_sleep(1);
+    const int r = (int)(tl & (WAVE - 1));           // predecessors inside the group
+    const int64_t g = tl >> 6;                      // groups in front of this one in the line
+    const int64_t t0 = tile - r;
+    T local = ident, gacc = ident, gpre = init;
+    bool local_done = (r == 0), group_done = (g == 0), ga_published = false;
+    int64_t gfirst = gl - 1, grem = g;              // nearest group of the current window, groups left
+    while (!(local_done && group_done)) {
+        Words<T> tv = to_words(ident), gv = to_words(ident);
+        uint32_t tstat = DESC_A, gstat = DESC_P;    // lanes outside the range: terminators holding ident
+        if (!local_done && lane < r) tstat = desc_read<T>(tile_desc, tstride, t0 + lane, tagA, tagP, tv);
+        if (!group_done && lane < grem) gstat = desc_read<T>(group_desc, gstride, gfirst - lane, tagA, tagP, gv);
+        if (!local_done && __ballot(tstat == 0u) == 0ull) {
+            local = wave_reduce(from_words<T>(tv), op);
+            local_done = true;
         }
-        const T x = (np < 0 || lane <= np) ? from_words<T>(val) : ident;
-        prefix = op(wave_reduce(x, op), prefix);
-        if (np >= 0) break;
-        first -= WAVE;
-        remaining -= WAVE;
+        if (local_done && r == WAVE - 1 && !ga_published && !group_done) {
+            if (lane == 0) desc_publish(group_desc, gstride, gl, op(local, agg), tagA);
+            ga_published = true;
+        }
+        if (!group_done) {
+            const uint64_t ballotP = __ballot(gstat == DESC_P);
+            const uint64_t ballotX = __ballot(gstat == 0u);
+            const int np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
+            const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
+            if ((ballotX & needed) == 0ull) {
+                const T x = (np < 0 || lane <= np) ? from_words<T>(gv) : ident;
+                gacc = op(wave_reduce(x, op), gacc);
+                if (np >= 0) {
+                    group_done = true;
+                    // a real GP already contains init; running off the line start does not
+                    gpre = (np >= grem) ? op(init, gacc) : gacc;
+                } else {
+                    gfirst -= WAVE;
+                    grem -= WAVE;
+                }
+            }
+        }
+        if (!(local_done && group_done))
+            for (int b = 0; b < backoff; ++b) __builtin_amdgcn_s_sleep(8);
     }
+    const T prefix = op(gpre, local);
+    if (r == WAVE - 1 && lane == 0) desc_publish(group_desc, gstride, gl, op(prefix, agg), tagP);
     return prefix;
 }
 
@@ -85,54 +119,30 @@ struct ScanGeom {
     int64_t inner, mid, outer;
 };
 
-// ---- contiguous lines, tiles with look-back ------------------------------------------------------
-template <typename In, typename T, typename Op, bool VECTOR, bool LOOKBACK, int BLOCK, int K>
-__global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
-                                                              int64_t tiles_per_line, int64_t ntiles, T init, int inclusive,
-                                                              Op op, WsHeader* hdr, uint64_t* desc, int64_t desc_stride,
-                                                              int64_t desc_capacity) {
+// ---- one tile of a contiguous line, scanned in registers ---------------------------------------------
+// 256 threads x K loads of 16 output bytes.  Wave w owns the w-th quarter of the tile; its k-th load
+// covers 64 * VEC consecutive elements (one fully coalesced 1 KiB request for 4-byte inputs).  Per load:
+// scan inside the lane, DPP scan across the wave, carry to the next load; wave totals meet in LDS.
+template <typename T, typename Op, int K> struct TileRegs {
+    static constexpr int VEC = 16 / sizeof(T);
+    T v[K][VEC];     // inclusive scan inside each lane's vector
+    T excl[K];       // exclusive prefix of that vector inside the wave's quarter
+};
+
+template <typename In, typename T, typename Op, bool VECTOR, int K>
+__device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e0, int valid, Op op, TileRegs<T, Op, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int NW = BLOCK / WAVE;
-    constexpr int WAVE_ELEMS = WAVE * VEC * K;
-    constexpr int TILE = NW * WAVE_ELEMS;
-    typedef typename VecOf<T, VEC>::type VT;
+    constexpr int TILE = 4 * WAVE * VEC * K;
     typedef typename VecOf<In, VEC>::type VI;
-    __shared__ T lds_wave[NW];
-    __shared__ T lds_prefix;
-    __shared__ uint32_t lds_tile, lds_epoch;
-
     const T ident = Op::template identity<T>();
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
-    int64_t tile;
-    uint32_t epoch = 0;
-    if constexpr (LOOKBACK) {
-        // tile ids in start order: every predecessor of a tile is already running or finished
-        if (tid == 0) {
-            lds_tile = __hip_atomic_fetch_add(&hdr->tile_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            lds_epoch = __hip_atomic_load(&hdr->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();
-        tile = lds_tile;
-        epoch = lds_epoch;
-    } else {
-        tile = blockIdx.x;
-    }
-    const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
-    const int64_t e0 = line * line_len + tl * TILE;
-    const int64_t left = line_len - tl * TILE;
-    const int valid = left < TILE ? (int)left : TILE;
-    const int woff = wave * WAVE_ELEMS + lane * VEC;
-
-    T v[K][VEC];
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int woff = wave * (WAVE * VEC * K) + lane * VEC;
     if (VECTOR && valid == TILE) {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const VI x = load_nt((const VI*)(in + e0 + woff + k * WAVE * VEC));
-            if constexpr (VEC == 1) v[k][0] = (T)x;
-            else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) v[k][j] = (T)x[j];
-            }
+            for (int j = 0; j < VEC; ++j) r.v[k][j] = (T)x[j];
         }
     } else {
 #pragma unroll
@@ -140,98 +150,156 @@ __global__ __launch_bounds__(BLOCK) void scan_lookback_kernel(const In* __restri
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const int idx = woff + k * WAVE * VEC + j;
-                v[k][j] = idx < valid ? (T)in[e0 + idx] : ident;
+                r.v[k][j] = idx < valid ? (T)in[e0 + idx] : ident;
             }
     }
-
-    // scan inside the thread, then across the wave, carrying the running total from load k to k+1
-    T excl[K];
     T carry = ident;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
-        for (int j = 1; j < VEC; ++j) v[k][j] = op(v[k][j - 1], v[k][j]);
-        const T inc = wave_scan_inclusive(v[k][VEC - 1], op, ident);
-        excl[k] = op(carry, wave_shift_right(inc, ident));
+        for (int j = 1; j < VEC; ++j) r.v[k][j] = op(r.v[k][j - 1], r.v[k][j]);
+        const T inc = wave_scan_inclusive(r.v[k][VEC - 1], op, ident);
+        r.excl[k] = op(carry, wave_shift_right(inc, ident));
         carry = op(carry, read_lane(inc, WAVE - 1));
     }
-    if (lane == 0) lds_wave[wave] = carry;
-    __syncthreads();
-    T wave_prefix = ident, tile_agg = ident;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-        const T x = lds_wave[w];
-        if (w < wave) wave_prefix = op(wave_prefix, x);
-        tile_agg = op(tile_agg, x);
-    }
+    return carry;    // total of this wave's quarter
+}
 
-    T tile_prefix = init;
-    if constexpr (LOOKBACK) {
-        if (wave == 0) {
-            if (tl == 0) {
-                if (lane == 0) desc_publish(desc, desc_stride, tile, op(init, tile_agg), (epoch << 2) | DESC_P);
-            } else {
-                if (lane == 0) desc_publish(desc, desc_stride, tile, tile_agg, (epoch << 2) | DESC_A);
-                // the chain of aggregates always ends at an inclusive prefix (tile 0 of the line
-                // publishes one directly), which already contains init
-                tile_prefix = desc_lookback(desc, desc_stride, tile, tl, epoch, op, ident);
-                if (lane == 0) desc_publish(desc, desc_stride, tile, op(tile_prefix, tile_agg), (epoch << 2) | DESC_P);
-            }
-            if (lane == 0) lds_prefix = tile_prefix;
-        }
-        __syncthreads();
-        tile_prefix = lds_prefix;
-    }
-    const T base = op(tile_prefix, wave_prefix);
-
+template <typename T, typename Op, bool VECTOR, int K>
+__device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int valid, int inclusive, T base, Op op,
+                                           const TileRegs<T, Op, K>& r) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int TILE = 4 * WAVE * VEC * K;
+    typedef typename VecOf<T, VEC>::type VT;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int woff = wave * (WAVE * VEC * K) + lane * VEC;
     if (VECTOR && valid == TILE) {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const T off = op(base, excl[k]);
+            const T off = op(base, r.excl[k]);
             VT o;
-            if constexpr (VEC == 1) o = inclusive ? op(off, v[k][0]) : off;
-            else {
-                if (inclusive) {
+            if (inclusive) {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) o[j] = op(off, v[k][j]);
-                } else {
-                    o[0] = off;
+                for (int j = 0; j < VEC; ++j) o[j] = op(off, r.v[k][j]);
+            } else {
+                o[0] = off;
 #pragma unroll
-                    for (int j = 1; j < VEC; ++j) o[j] = op(off, v[k][j - 1]);
-                }
+                for (int j = 1; j < VEC; ++j) o[j] = op(off, r.v[k][j - 1]);
             }
             store_nt((VT*)(out + e0 + woff + k * WAVE * VEC), o);
         }
     } else {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const T off = op(base, excl[k]);
+            const T off = op(base, r.excl[k]);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const int idx = woff + k * WAVE * VEC + j;
-                if (idx < valid) out[e0 + idx] = inclusive ? op(off, v[k][j]) : (j == 0 ? off : op(off, v[k][j - 1]));
-            }
-        }
-    }
-
-    if constexpr (LOOKBACK) {
-        // Only wave 0 touches the descriptors; once it has published, this tile is done with them.
-        if (wave == 0) {
-            uint32_t old = 0;
-            if (lane == 0) old = __hip_atomic_fetch_add(&hdr->done_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            old = (uint32_t)__builtin_amdgcn_readfirstlane((int)old);
-            if (old == (uint32_t)ntiles - 1u) {
-                // last tile of the call: leave counters clean, move to the next generation
-                if (epoch >= WS_EPOCH_LAST) {
-                    for (int64_t i = lane; i < desc_capacity; i += WAVE) desc[i] = 0;
-                    if (lane == 0) hdr->epoch = WS_EPOCH_FIRST;
-                } else if (lane == 0) hdr->epoch = epoch + 1;
-                if (lane == 0) { hdr->tile_counter = 0; hdr->done_counter = 0; }
+                if (idx < valid) out[e0 + idx] = inclusive ? op(off, r.v[k][j]) : (j == 0 ? off : op(off, r.v[k][j - 1]));
             }
         }
     }
 }
 
+// ---- contiguous lines that fit one tile: one workgroup per line, no communication ------------------------
+template <typename In, typename T, typename Op, bool VECTOR, int K>
+__global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len, T init,
+                                                         int inclusive, Op op) {
+    constexpr int NW = 4;
+    __shared__ T lds_wave[NW];
+    const T ident = Op::template identity<T>();
+    const int wave = threadIdx.x / WAVE;
+    const int64_t e0 = (int64_t)blockIdx.x * line_len;
+    TileRegs<T, Op, K> r;
+    const T wtot = tile_load_scan<In, T, Op, VECTOR, K>(in, e0, (int)line_len, op, r);
+    if (lane_id() == 0) lds_wave[wave] = wtot;
+    __syncthreads();
+    T wave_prefix = ident;
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+        if (w < wave) wave_prefix = op(wave_prefix, lds_wave[w]);
+    tile_store<T, Op, VECTOR, K>(out, e0, (int)line_len, inclusive, op(init, wave_prefix), op, r);
+}
+
+// ---- long contiguous lines: persistent workgroups, single pass, two-level decoupled look-back --------------
+// `counter` packs (epoch << 32 | acquisitions).  A workgroup takes its tiles from it in acquisition order
+// (every predecessor of a tile is therefore already owned by a running workgroup: the look-back cannot wait
+// on work that has not started) and fetches the NEXT id while it works on the current tile, which hides the
+// latency of the device-wide atomic.  Every workgroup makes exactly one acquisition beyond the last tile, so
+// the acquisition number ntiles + gridDim.x - 1 is the last access of the call: its owner advances the epoch
+// and resets the count for the next call, and clears a rotating slice of the descriptor slots this call did
+// not use, so that no slot can keep a tag for more than SWEEP calls (tags are 30-bit epochs).
+constexpr int SCAN_SWEEP = 1024;
+
+template <typename In, typename T, typename Op, bool VECTOR, int K>
+__global__ __launch_bounds__(256) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+                                                         int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
+                                                         unsigned long long* counter, uint64_t* desc, int64_t ngroups_per_line,
+                                                         int64_t ngroups, int64_t desc_capacity, int backoff) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int NW = 4;
+    constexpr int TILE = NW * WAVE * VEC * K;
+    __shared__ T lds_wave[NW];
+    __shared__ T lds_prefix;
+    __shared__ unsigned long long lds_id;
+
+    const T ident = Op::template identity<T>();
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    uint64_t* tile_desc = desc;                                        // [words][ntiles]
+    uint64_t* group_desc = desc + (int64_t)Words<T>::N * ntiles;       // [words][ngroups]
+
+    unsigned long long pending = 0;
+    if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    unsigned long long cur = lds_id;
+    while ((int64_t)(cur & 0xffffffffull) < ntiles) {
+        const int64_t tile = (int64_t)(cur & 0xffffffffull);
+        const uint32_t epoch = (uint32_t)(cur >> 32);
+        if (tid == 0) pending = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+        const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
+        const int64_t e0 = line * line_len + tl * TILE;
+        const int64_t left = line_len - tl * TILE;
+        const int valid = left < TILE ? (int)left : TILE;
+        TileRegs<T, Op, K> r;
+        const T wtot = tile_load_scan<In, T, Op, VECTOR, K>(in, e0, valid, op, r);
+        if (lane == 0) lds_wave[wave] = wtot;
+        __syncthreads();
+        T wave_prefix = ident, tile_agg = ident;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const T x = lds_wave[w];
+            if (w < wave) wave_prefix = op(wave_prefix, x);
+            tile_agg = op(tile_agg, x);
+        }
+        if (wave == 0) {
+            T tile_prefix = init;
+            if (lane == 0) desc_publish(tile_desc, ntiles, tile, tile_agg, (epoch << 2) | DESC_A);
+            if (tl > 0)
+                tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tl, line * ngroups_per_line + (tl >> 6),
+                                             epoch, tile_agg, init, op, ident, backoff);
+            if (lane == 0) lds_prefix = tile_prefix;
+        }
+        __syncthreads();
+        tile_store<T, Op, VECTOR, K>(out, e0, valid, inclusive, op(lds_prefix, wave_prefix), op, r);
+        if (tid == 0) lds_id = pending;
+        __syncthreads();
+        cur = lds_id;
+    }
+    // `cur` is this workgroup's one acquisition past the end
+    if (wave == 0 && (int64_t)(cur & 0xffffffffull) == ntiles + (int64_t)gridDim.x - 1) {
+        uint32_t epoch = (uint32_t)(cur >> 32);
+        const int64_t used = (int64_t)Words<T>::N * (ntiles + ngroups);
+        const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
+        int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
+        if (lo < used) lo = used;
+        if (hi > desc_capacity) hi = desc_capacity;
+        for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
+        epoch = (epoch + 1u) & 0x3fffffffu;
+        if (epoch == 0u) epoch = 1u;          // tag 0 marks a cleared slot
+        if (lane == 0) *counter = (unsigned long long)epoch << 32;
+    }
+}
 
 // ---- contiguous lines shorter than a tile: one wave per line -------------------------------------
 template <typename In, typename T, typename Op, bool VECTOR, int BLOCK>
@@ -374,11 +442,13 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
 }
 
 // ---- host side ---------------------------------------------------------------------------------------
-template <typename T> struct ScanTile {            // geometry of scan_lookback_kernel<..., 256, 4>
-    static constexpr int K = 4;
+template <typename T, int K> struct ScanTile {     // geometry of the tile kernels: 256 threads x K x 16 bytes of output
     static constexpr int VEC = 16 / sizeof(T);
-    static constexpr int TILE = 4 * WAVE * VEC * K;  // 4096 elements of 4 bytes, 2048 of 8 bytes
+    static constexpr int TILE = 4 * WAVE * VEC * K;
 };
+
+int tune_scan_backoff();        // rk_api.hip
+int tune_scan_blocks_per_cu();  // rk_api.hip
 
 struct ScanArgs {
     int op;
@@ -433,26 +503,39 @@ inline int32_t launch_scan(const ScanArgs& a) {
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
-    constexpr int TILE = ScanTile<T>::TILE;
-    const int64_t tpl = (s.mid + TILE - 1) / TILE;
-    const int64_t ntiles = tpl * nlines;
-    if (ntiles > 0x7fffffff) return RK_ERR_TOO_LARGE;
-    if (tpl == 1) {
-        if (lines_aligned)
-            scan_lookback_kernel<In, T, Op, true, false, 256, 4><<<(unsigned)ntiles, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, nullptr, nullptr, 0, 0);
-        else
-            scan_lookback_kernel<In, T, Op, false, false, 256, 4><<<(unsigned)ntiles, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, nullptr, nullptr, 0, 0);
+    // lines that fit one tile: smallest tile that holds the line
+    if (s.mid <= ScanTile<T, 8>::TILE) {
+        if (nlines > 0x7fffffff) return RK_ERR_TOO_LARGE;
+        const unsigned grid = (unsigned)nlines;
+#define RK_SCAN_TILES(KK)                                                                                             \
+        do {                                                                                                          \
+            if (lines_aligned) scan_tiles_kernel<In, T, Op, true, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op); \
+            else scan_tiles_kernel<In, T, Op, false, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op);            \
+        } while (0)
+        if (s.mid <= ScanTile<T, 2>::TILE) RK_SCAN_TILES(2);
+        else if (s.mid <= ScanTile<T, 4>::TILE) RK_SCAN_TILES(4);
+        else RK_SCAN_TILES(8);
+#undef RK_SCAN_TILES
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
+    constexpr int KT = 8;
+    constexpr int TILE = ScanTile<T, KT>::TILE;
+    const int64_t tpl = (s.mid + TILE - 1) / TILE;
+    const int64_t ntiles = tpl * nlines;
+    if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
     Workspace w{};
-    const size_t need = (size_t)ntiles * Words<T>::N * sizeof(uint64_t);
+    const int64_t gpl = (tpl + WAVE - 1) / WAVE, ngroups = gpl * nlines;
+    const size_t need = (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
+    int64_t grid = (int64_t)device_info().cus * tune_scan_blocks_per_cu();
+    if (grid > ntiles) grid = ntiles;
+    unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     if (lines_aligned)
-        scan_lookback_kernel<In, T, Op, true, true, 256, 4><<<(unsigned)ntiles, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, w.hdr, w.desc, ntiles, cap);
+        scan_chain_kernel<In, T, Op, true, KT><<<(unsigned)grid, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, tune_scan_backoff());
     else
-        scan_lookback_kernel<In, T, Op, false, true, 256, 4><<<(unsigned)ntiles, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, w.hdr, w.desc, ntiles, cap);
+        scan_chain_kernel<In, T, Op, false, KT><<<(unsigned)grid, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, tune_scan_backoff());
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }

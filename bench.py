@@ -1,0 +1,303 @@
+#!/usr/bin/env python3
+"""Benchmark of the ROCArray array-kernel path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--no-cpu]
+
+Prints ONE JSON line.  A *step* is one pass of the headline workload named by the metric -- sum over a
+Float32 vector, eltype-preserving cumsum over an Int32 vector and the fused broadcast
+z .= a .* x .+ y .* exp.(w), each on 2^26 elements -- with every input already resident in HBM.
+`value` = algorithmic bytes of the K timed steps / their wall time (GB/s), measured between two stream
+synchronisations; the buffers of consecutive steps rotate so that no step finds its input in the 256 MB
+Infinity Cache.  `roofline` is the dominant kernel of the step (the broadcast: 16 of the 28 bytes per
+element), timed with HIP events on the launch stream.  `configs` lists every BASELINE configuration at
+its own size (elements/s, GB/s, fraction of the 8 TB/s HBM peak; minimum and mean of the timed repeats).
+`cpu_baseline` times the C restatement of Julia Base (oracle/oracle_c.c, kind "port": no Julia runtime
+exists on this machine) on the host cores for the same step.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+N_HEAD = 1 << 26
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return p.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU; the path has no multi-GPU part "
+              "(every op shards without communication, see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from __graft_entry__ import load_package
+    rk = load_package()
+    L = rk.lazy
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    K, W = args.steps, args.warmup
+
+    def dev_array(t: "torch.Tensor", dims, dtype):
+        """Wrap a device tensor produced by torch's generators as a ROCArray (no copy)."""
+        return rk.ROCArray(buf=t.view(torch.uint8).reshape(-1), dims=dims, dtype=dtype)
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+
+    def rand_f32(n, lo=0.0, hi=1.0):
+        return (torch.rand(n, device=dev, generator=gen, dtype=torch.float32) * (hi - lo) + lo)
+
+    def randn_f32(n):
+        return torch.randn(n, device=dev, generator=gen, dtype=torch.float32)
+
+    def randint_i32(n):
+        return torch.randint(-1000, 1001, (n,), device=dev, generator=gen, dtype=torch.int32)
+
+    def time_launches(fn, reps, warm=3):
+        """Average / minimum duration (ms) of `fn(i)` launches, HIP events on the launch stream."""
+        for i in range(warm):
+            fn(i)
+        torch.cuda.synchronize()
+        # whole batch between two events: average launch-to-launch time with a saturated queue
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        avg = e0.elapsed_time(e1) / reps
+        # individual launches: minimum (the reference reports the minimum, perf/runbenchmarks.jl:81-86)
+        best = float("inf")
+        for i in range(min(reps, 20)):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn(i)
+            b.record()
+            b.synchronize()
+            best = min(best, a.elapsed_time(b))
+        return avg, best
+
+    # ---- headline step: sum f32 + cumsum i32 + broadcast, 2^26 elements each --------------------------
+    n = N_HEAD
+    ROT = 3
+    sum_in = [dev_array(rand_f32(n), (n,), np.float32) for _ in range(ROT)]
+    sum_out = rk.ROCArray(dims=(1,), dtype=np.float32)
+    scan_in = [dev_array(randint_i32(n), (n,), np.int32) for _ in range(ROT)]
+    scan_out = [rk.ROCArray(dims=(n,), dtype=np.int32) for _ in range(ROT)]
+    bx = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+    by = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+    bw = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+    bz = [rk.ROCArray(dims=(n,), dtype=np.float32) for _ in range(2)]
+    a = np.float32(0.5)
+    exprs = [a * L(bx[i]) + L(by[i]) * rk.broadcast.exp(L(bw[i])) for i in range(2)]
+
+    def op_sum(i):
+        rk.mapreducedim_(rk.identity, rk.add, sum_out, sum_in[i % ROT])
+
+    def op_scan(i):
+        rk.accumulate_("add", scan_out[i % ROT], scan_in[i % ROT])
+
+    def op_bcast(i):
+        rk.materialize_(bz[i % 2], exprs[i % 2])
+
+    def step(i):
+        op_sum(i)
+        op_scan(i)
+        op_bcast(i)
+
+    bytes_sum, bytes_scan, bytes_bc = 4 * n, 8 * n, 16 * n
+    step_bytes = bytes_sum + bytes_scan + bytes_bc
+
+    for i in range(W):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / K
+    value = step_bytes / (wall / K) / 1e9
+
+    bc_avg, bc_min = time_launches(op_bcast, K)
+    sum_avg, sum_min = time_launches(op_sum, K)
+    scan_avg, scan_min = time_launches(op_scan, K)
+
+    def entry(name, elems, nbytes, avg_ms, min_ms, **extra):
+        gbs = nbytes / (avg_ms * 1e-3) / 1e9
+        e = {"op": name, "elements": elems, "bytes": nbytes, "avg_us": round(avg_ms * 1e3, 2), "min_us": round(min_ms * 1e3, 2),
+             "elements_per_s": elems / (avg_ms * 1e-3), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+             "GBps_best": round(nbytes / (min_ms * 1e-3) / 1e9, 1)}
+        e.update(extra)
+        return e
+
+    configs = [
+        entry("sum Float32[2^26]", n, bytes_sum, sum_avg, sum_min),
+        entry("cumsum Int32[2^26]", n, bytes_scan, scan_avg, scan_min),
+        entry("z .= a.*x .+ y.*exp.(w) Float32[2^26]", n, bytes_bc, bc_avg, bc_min),
+    ]
+    roofline = {"bound": "hbm", "kernel": "bc_kernel<EvalAxpbyExp,float,4,linear> (z .= a.*x .+ y.*exp.(w), 2^26 elts)",
+                "achieved": round(bytes_bc / (bc_avg * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(bytes_bc / (bc_avg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "bytes_per_launch": bytes_bc, "avg_launch_us": round(bc_avg * 1e3, 2)}
+
+    del sum_in, scan_in, scan_out, bx, by, bw, bz, exprs
+    torch.cuda.empty_cache()
+
+    # ---- every BASELINE configuration at its own size ------------------------------------------------------
+    if not args.no_configs:
+        reps = max(10, min(K, 30))
+
+        def run_cfg(name, elems, nbytes, fn, **extra):
+            avg, best = time_launches(fn, reps)
+            configs.append(entry(name, elems, nbytes, avg, best, **extra))
+
+        # cfg 1: full sums (2^24 fits the Infinity Cache: rotate 8 buffers = 512 MiB)
+        for logn, rot in ((24, 8), (28, 2)):
+            m = 1 << logn
+            xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(rot)]
+            r = rk.ROCArray(dims=(1,), dtype=np.float32)
+            run_cfg(f"cfg1a sum Float32[2^{logn}]", m, 4 * m, lambda i: rk.mapreducedim_(rk.identity, rk.add, r, xs[i % rot]))
+            del xs
+        m = 1 << 24
+        xi = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(8)]
+        ri = rk.ROCArray(dims=(1,), dtype=np.int64)
+        run_cfg("cfg1b sum Int32[2^24] -> Int64", m, 4 * m, lambda i: rk.mapreducedim_(rk.identity, rk.add, ri, xi[i % 8]))
+        del xi
+        # cfg 2: 8192 x 8192
+        d = 8192
+        As = [dev_array(randn_f32(d * d), (d, d), np.float32) for _ in range(3)]
+        r1 = rk.ROCArray(dims=(1, d), dtype=np.float32)
+        r2 = rk.ROCArray(dims=(d, 1), dtype=np.float32)
+        run_cfg("cfg2a mapreduce(abs2,+,A;dims=1) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: rk.mapreducedim_(rk.abs2, rk.add, r1, As[i % 3]))
+        run_cfg("cfg2b mapreduce(abs2,+,A;dims=2) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: rk.mapreducedim_(rk.abs2, rk.add, r2, As[i % 3]))
+        from amdgpu_jl_amd import _lib as RL
+        from amdgpu_jl_amd.array import workspace, stream_ptr
+        fv = rk.ROCArray(dims=(1, d), dtype=np.float32)
+        fi = rk.ROCArray(dims=(2, 1, d), dtype=np.int64)
+        shp = RL.shape_array((d, d))
+
+        def op_findmax(i):
+            ws, wsb = workspace()
+            RL.check(RL.lib.rk_findminmax(1, RL.RK_F32, As[i % 3].ptr, 2, shp, 1, fv.ptr, fi.ptr, ws, wsb, stream_ptr()))
+        run_cfg("cfg2c findmax(A;dims=1) 8192^2", d * d, 4 * d * d + 20 * d, op_findmax)
+        del As
+        # cfg 3
+        m = 1 << 27
+        si = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(2)]
+        so = [rk.ROCArray(dims=(m,), dtype=np.int32) for _ in range(2)]
+        run_cfg("cfg3a cumsum Int32[2^27]", m, 8 * m, lambda i: rk.accumulate_("add", so[i % 2], si[i % 2]))
+        del si, so
+        rows, cols = 4096, 16384
+        Bi = [dev_array(rand_f32(rows * cols), (rows, cols), np.float32) for _ in range(2)]
+        Bo = [rk.ROCArray(dims=(rows, cols), dtype=np.float32) for _ in range(2)]
+        run_cfg("cfg3b cumsum(B;dims=1) 4096x16384 Float32", rows * cols, 8 * rows * cols,
+                lambda i: rk.accumulate_("add", Bo[i % 2], Bi[i % 2], dims=1))
+        run_cfg("cumsum(B;dims=2) 4096x16384 Float32", rows * cols, 8 * rows * cols,
+                lambda i: rk.accumulate_("add", Bo[i % 2], Bi[i % 2], dims=2))
+        del Bi, Bo
+        # cfg 4
+        m = 512 ** 3
+        x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))
+        z4 = rk.ROCArray(dims=(512, 512, 512), dtype=np.float32)
+        e4 = a * L(x4) + L(y4) * rk.broadcast.exp(L(w4))
+        run_cfg("cfg4a z .= a.*x .+ y.*exp.(w) 512^3", m, 16 * m, lambda i: rk.materialize_(z4, e4))
+        del x4, y4, w4, z4, e4
+        d = 16384
+        A4 = dev_array(rand_f32(d * d, -1, 1), (d, d), np.float32)
+        r4 = dev_array(rand_f32(d, -1, 1), (1, d), np.float32)
+        c4 = dev_array(rand_f32(d, -1, 1), (d, 1), np.float32)
+        C4 = rk.ROCArray(dims=(d, d), dtype=np.float32)
+        e4b = L(A4) + L(r4) * L(c4)
+        run_cfg("cfg4b C .= A .+ r .* c 16384^2", d * d, 8 * d * d + 8 * d, lambda i: rk.materialize_(C4, e4b))
+        del A4, C4, e4b
+        # cfg 5
+        for ne, rot in ((4000, 6), (240_000, 1)):
+            Qs = [dev_array(rand_f32(625 * ne, 0.5, 1.5), (5, 5, 5, 5, ne), np.float32) for _ in range(rot)]
+            Vs = [dev_array(rand_f32(1750 * ne, 0.9, 1.1), (5, 5, 5, 14, ne), np.float32) for _ in range(rot)]
+            Rs = [rk.zeros(np.float32, 5, 5, 5, 5, ne) for _ in range(rot)]
+            Dm = dev_array(rand_f32(25), (5, 5), np.float32)
+            run_cfg(f"cfg5 volumerhs! N=4 nelem={ne}", 125 * ne, 13500 * ne,
+                    lambda i: rk.volumerhs_(Rs[i % rot], Qs[i % rot], Vs[i % rot], 9.81, Dm, ne), flops=37_000 * ne)
+            del Qs, Vs, Rs
+        torch.cuda.empty_cache()
+
+    # ---- CPU baseline: C restatement of Julia Base on the host cores, same step -----------------------------
+    cpu = None
+    if not args.no_cpu:
+        so = os.path.join(ROOT, "oracle", "liboracle_c.so")
+        if os.path.exists(so):
+            lib = C.CDLL(so)
+            lib.orc_sum_f32.restype = C.c_double
+            lib.orc_sum_f32.argtypes = [C.c_void_p, C.c_int64, C.c_int]
+            lib.orc_cumsum_i32.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
+            lib.orc_bcast_axpby_exp_f32.argtypes = [C.c_float] + [C.c_void_p] * 4 + [C.c_int64, C.c_int]
+            threads = max(1, min(16, os.cpu_count() or 1))
+            rng = np.random.default_rng(0)
+            hx = rng.random(n, dtype=np.float32)
+            hi = rng.integers(-1000, 1001, n, dtype=np.int32)
+            ho = np.empty_like(hi)
+            hy, hw = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
+            hz = np.empty_like(hx)
+
+            def cpu_step(t):
+                lib.orc_sum_f32(hx.ctypes.data, n, t)
+                lib.orc_cumsum_i32(hi.ctypes.data, n, ho.ctypes.data)
+                lib.orc_bcast_axpby_exp_f32(0.5, hx.ctypes.data, hy.ctypes.data, hw.ctypes.data, hz.ctypes.data, n, t)
+
+            def best_of(t, reps):
+                cpu_step(t)
+                best = float("inf")
+                for _ in range(reps):
+                    t0 = time.perf_counter()
+                    cpu_step(t)
+                    best = min(best, time.perf_counter() - t0)
+                return best
+
+            t1 = best_of(1, 2)
+            tn = best_of(threads, 5) if threads > 1 else t1
+            cpu = {"value": round(step_bytes / tn / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+                   "single_thread_GBps": round(step_bytes / t1 / 1e9, 2),
+                   "sample": "the same step (sum Float32 + accumulate(+) Int32 + z .= a.*x .+ y.*exp.(w), 2^26 elements each), "
+                             "minimum of 5 runs of oracle/oracle_c.c with OpenMP on `cores` threads (the Int32 scan is sequential, "
+                             "as in Julia Base); Julia itself is not installed on this machine, so this is the C port of Base's "
+                             "algorithms (JULIA_NUM_THREADS does not apply; Base's sum/accumulate/broadcast are single-threaded: "
+                             "see single_thread_GBps)"}
+
+    out = {
+        "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for sum/cumsum/broadcast at 2^26 elems",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "step = sum(Float32[2^26]) + accumulate(+, Int32[2^26]) + (z .= a.*x .+ y.*exp.(w), Float32[2^26]); "
+                               "28 algorithmic bytes per element; rotating HBM-resident buffers",
+                   "elements": n, "bytes_per_step": step_bytes, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "configs": configs,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
