@@ -45,9 +45,10 @@ int tune_scan_backoff() {
     return v;
 }
 
-// Persistent workgroups per compute unit of the look-back scan (RK_SCAN_BLOCKS_PER_CU).
+// Persistent 256-thread workgroups per compute unit of the look-back scan; larger workgroups scale it
+// down (RK_SCAN_BLOCKS_PER_CU).
 int tune_scan_blocks_per_cu() {
-    static const int v = env_int("RK_SCAN_BLOCKS_PER_CU", 6, 1, 16);
+    static const int v = env_int("RK_SCAN_BLOCKS_PER_CU", 4, 1, 16);
     return v;
 }
 

@@ -129,10 +129,10 @@ template <typename T, typename Op, int K> struct TileRegs {
     T excl[K];       // exclusive prefix of that vector inside the wave's quarter
 };
 
-template <typename In, typename T, typename Op, bool VECTOR, int K>
+template <typename In, typename T, typename Op, bool VECTOR, int K, int NW = 4>
 __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e0, int valid, Op op, TileRegs<T, Op, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int TILE = 4 * WAVE * VEC * K;
+    constexpr int TILE = NW * WAVE * VEC * K;
     typedef typename VecOf<In, VEC>::type VI;
     const T ident = Op::template identity<T>();
     const int wave = threadIdx.x / WAVE, lane = lane_id();
@@ -165,11 +165,11 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
     return carry;    // total of this wave's quarter
 }
 
-template <typename T, typename Op, bool VECTOR, int K>
+template <typename T, typename Op, bool VECTOR, int K, int NW = 4>
 __device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int valid, int inclusive, T base, Op op,
                                            const TileRegs<T, Op, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int TILE = 4 * WAVE * VEC * K;
+    constexpr int TILE = NW * WAVE * VEC * K;
     typedef typename VecOf<T, VEC>::type VT;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int woff = wave * (WAVE * VEC * K) + lane * VEC;
@@ -222,22 +222,25 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ 
 }
 
 // ---- long contiguous lines: persistent workgroups, single pass, two-level decoupled look-back --------------
-// `counter` packs (epoch << 32 | acquisitions).  A workgroup takes its tiles from it in acquisition order
-// (every predecessor of a tile is therefore already owned by a running workgroup: the look-back cannot wait
-// on work that has not started) and fetches the NEXT id while it works on the current tile, which hides the
-// latency of the device-wide atomic.  Every workgroup makes exactly one acquisition beyond the last tile, so
-// the acquisition number ntiles + gridDim.x - 1 is the last access of the call: its owner advances the epoch
-// and resets the count for the next call, and clears a rotating slice of the descriptor slots this call did
-// not use, so that no slot can keep a tag for more than SWEEP calls (tags are 30-bit epochs).
+// `counter` packs (epoch << 32 | acquisitions).  A workgroup takes its tiles from it in acquisition order:
+// every predecessor of a tile is therefore already owned by a running workgroup, so the look-back never
+// waits on work that has not started.  The id of the next tile is taken only when the workgroup is ready
+// to load it -- ids taken ahead of time would be published late and stall every successor.
+// Device-wide atomics on one address complete at about 14 ns each on MI355X, so the tile is made as large
+// as the problem allows (up to 1024 threads x 8 vectors = 128 KiB of input): 2^27 elements are 4096
+// acquisitions, ~60 us, against ~170 us of streaming.
+// Every workgroup makes exactly one acquisition beyond the last tile, so acquisition number
+// ntiles + gridDim.x - 1 is the last access of the call: its owner advances the epoch and resets the count
+// for the next call, and clears a rotating slice of the descriptor slots this call did not use, so that no
+// slot keeps a tag for more than SWEEP calls (tags are 30-bit epochs).
 constexpr int SCAN_SWEEP = 1024;
 
-template <typename In, typename T, typename Op, bool VECTOR, int K>
-__global__ __launch_bounds__(256) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
+__global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
                                                          int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                          unsigned long long* counter, uint64_t* desc, int64_t ngroups_per_line,
                                                          int64_t ngroups, int64_t desc_capacity, int backoff) {
     constexpr int VEC = 16 / sizeof(T);
-    constexpr int NW = 4;
     constexpr int TILE = NW * WAVE * VEC * K;
     __shared__ T lds_wave[NW];
     __shared__ T lds_prefix;
@@ -248,21 +251,18 @@ __global__ __launch_bounds__(256) void scan_chain_kernel(const In* __restrict__ 
     uint64_t* tile_desc = desc;                                        // [words][ntiles]
     uint64_t* group_desc = desc + (int64_t)Words<T>::N * ntiles;       // [words][ngroups]
 
-    unsigned long long pending = 0;
     if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     unsigned long long cur = lds_id;
     while ((int64_t)(cur & 0xffffffffull) < ntiles) {
         const int64_t tile = (int64_t)(cur & 0xffffffffull);
         const uint32_t epoch = (uint32_t)(cur >> 32);
-        if (tid == 0) pending = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
         const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
         const int64_t e0 = line * line_len + tl * TILE;
         const int64_t left = line_len - tl * TILE;
         const int valid = left < TILE ? (int)left : TILE;
         TileRegs<T, Op, K> r;
-        const T wtot = tile_load_scan<In, T, Op, VECTOR, K>(in, e0, valid, op, r);
+        const T wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, op, r);
         if (lane == 0) lds_wave[wave] = wtot;
         __syncthreads();
         T wave_prefix = ident, tile_agg = ident;
@@ -281,8 +281,8 @@ __global__ __launch_bounds__(256) void scan_chain_kernel(const In* __restrict__ 
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
-        tile_store<T, Op, VECTOR, K>(out, e0, valid, inclusive, op(lds_prefix, wave_prefix), op, r);
-        if (tid == 0) lds_id = pending;
+        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, inclusive, op(lds_prefix, wave_prefix), op, r);
+        if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         cur = lds_id;
     }
@@ -519,8 +519,11 @@ inline int32_t launch_scan(const ScanArgs& a) {
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
+    // long lines: the chained look-back scan; tile = NW waves x 8 vectors, as large as the line length allows
     constexpr int KT = 8;
-    constexpr int TILE = ScanTile<T, KT>::TILE;
+    const int64_t line_bytes = s.mid * (int64_t)sizeof(T);
+    const int nw = line_bytes >= ((int64_t)128 << 20) ? 16 : (line_bytes >= ((int64_t)32 << 20) ? 8 : 4);
+    const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
     const int64_t tpl = (s.mid + TILE - 1) / TILE;
     const int64_t ntiles = tpl * nlines;
     if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
@@ -529,13 +532,20 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const size_t need = (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
-    int64_t grid = (int64_t)device_info().cus * tune_scan_blocks_per_cu();
+    int64_t grid = (int64_t)device_info().cus * tune_scan_blocks_per_cu() * 4 / nw;
     if (grid > ntiles) grid = ntiles;
+    if (grid < 1) grid = 1;
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
-    if (lines_aligned)
-        scan_chain_kernel<In, T, Op, true, KT><<<(unsigned)grid, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, tune_scan_backoff());
-    else
-        scan_chain_kernel<In, T, Op, false, KT><<<(unsigned)grid, 256, 0, a.stream>>>(in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, tune_scan_backoff());
+    const int backoff = tune_scan_backoff();
+#define RK_SCAN_CHAIN(VECF, NWW)                                                                                      \
+    scan_chain_kernel<In, T, Op, VECF, KT, NWW><<<(unsigned)grid, NWW * WAVE, 0, a.stream>>>(                          \
+        in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, backoff)
+    if (lines_aligned) {
+        if (nw == 16) RK_SCAN_CHAIN(true, 16); else if (nw == 8) RK_SCAN_CHAIN(true, 8); else RK_SCAN_CHAIN(true, 4);
+    } else {
+        if (nw == 16) RK_SCAN_CHAIN(false, 16); else if (nw == 8) RK_SCAN_CHAIN(false, 8); else RK_SCAN_CHAIN(false, 4);
+    }
+#undef RK_SCAN_CHAIN
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }
