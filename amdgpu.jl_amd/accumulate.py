@@ -31,14 +31,32 @@ def accumulate_(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusi
         raise ValueError("dims must be >= 1")
     if len(A) == 0:
         return B
+    _launch_accumulate(op, B, A, dims, init, inclusive)()
+    return B
+
+
+def _launch_accumulate(op, B, A, dims, init, inclusive):
     bytes_needed = L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, B.code, A.ndim, L.shape_array(A.dims),
                                             (1 << (dims - 1)) if dims <= A.ndim else 0)
     ws, ws_bytes = workspace(bytes_needed)
     ibuf = _scalar_buffer(init, B.dtype)
-    st = L.lib.rk_accumulate(_OP[op], A.code, B.code, A.ptr, B.ptr, A.ndim, L.shape_array(A.dims), int(dims),
-                             1 if inclusive else 0, ibuf, ws, ws_bytes, stream_ptr())
-    L.check(st, "rk_accumulate")
-    return B
+    args = (_OP[op], A.code, B.code, A.ptr, B.ptr, A.ndim, L.shape_array(A.dims), int(dims), 1 if inclusive else 0,
+            ibuf, ws, ws_bytes)
+    fn = L.lib.rk_accumulate
+
+    def launch():
+        L.check(fn(*args, stream_ptr()), "rk_accumulate")
+    return launch
+
+
+def plan_accumulate(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusive: bool = True):
+    """Validate once, return a callable that repeats ``accumulate!(op, B, A; dims, init)`` with no
+    per-call host work beyond the foreign call."""
+    if op not in ("add", "mul", "max", "min") or B.dims != A.dims or len(A) == 0:
+        raise ValueError("plan_accumulate: unsupported operator, mismatched dims or empty input")
+    if dims is None:
+        dims = 1
+    return _launch_accumulate(op, B, A, dims, init, inclusive)
 
 
 def accumulate(op: str, A: ROCArray, dims=None, init=None, inclusive: bool = True) -> ROCArray:

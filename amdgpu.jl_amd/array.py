@@ -145,6 +145,7 @@ def Array(x: ROCArray) -> np.ndarray:
 
 # ---- per-(device, stream) workspace: the analogue of the reference's per-task library state --------
 _workspaces: dict = {}
+_retired: list = []
 
 
 def workspace(min_bytes: int = 0):
@@ -154,6 +155,8 @@ def workspace(min_bytes: int = 0):
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
         size = max(need, 2 * ws.numel() if ws is not None else 0)
+        if ws is not None:
+            _retired.append(ws)      # prepared calls may still hold its address: never free a workspace
         ws = torch.empty(size, dtype=torch.uint8, device=device())
         assert ws.data_ptr() % 256 == 0
         L.check(L.lib.rk_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr()), "rk_workspace_init")

@@ -190,12 +190,33 @@ def materialize_(dest: ROCArray, bc) -> ROCArray:
         full = full[:-1]
     if full != dest.dims:
         raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"destination {dest.dims} vs broadcast shape {shape}")
-    if len(operands) > 0 and len(dest) == 0:
+    if len(dest) == 0:
         return dest
-    prog = _program(operands, tokens, compute, dest.ndim)
-    st = L.lib.rk_broadcast(prog, dest.ptr, dest.code, dest.ndim, L.shape_array(dest.dims), stream_ptr())
-    L.check(st, "rk_broadcast")
+    _launch_broadcast(dest, operands, tokens, compute)()
     return dest
+
+
+def _launch_broadcast(dest, operands, tokens, compute):
+    prog = _program(operands, tokens, compute, dest.ndim)
+    args = (prog, dest.ptr, dest.code, dest.ndim, L.shape_array(dest.dims))
+    fn = L.lib.rk_broadcast
+    keep = operands          # the program holds raw device pointers: keep the arrays alive with the plan
+
+    def launch(_keep=keep):
+        L.check(fn(*args, stream_ptr()), "rk_broadcast")
+    return launch
+
+
+def plan_materialize(dest: ROCArray, bc):
+    """Flatten and validate ``dest .= bc`` once; the returned callable repeats it with no per-call host
+    work beyond the foreign call (Julia specialises the same tree at compile time)."""
+    operands, tokens, compute, shape = _compile(bc)
+    full = broadcast_shape(shape, dest.dims)
+    while len(full) > dest.ndim and full[-1] == 1:
+        full = full[:-1]
+    if full != dest.dims or len(dest) == 0:
+        raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"destination {dest.dims} vs broadcast shape {shape}")
+    return _launch_broadcast(dest, operands, tokens, compute)
 
 
 def materialize(bc) -> ROCArray:

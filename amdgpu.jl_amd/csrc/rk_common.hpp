@@ -47,7 +47,7 @@ const DeviceInfo& device_info();   // rk_api.hip
 
 // ---- workspace layout -------------------------------------------------------------------
 // [0, 256)                       WsHeader
-// [256, +64 KiB)                 completion tickets of the multi-workgroup reductions
+// [256, +2 MiB)                  completion tickets of the multi-workgroup reductions, one per 128-byte line
 // [.., +WS_PARTIALS_BYTES)       partial results of the reductions
 // [WS_DESC_OFFSET, end)          tile descriptors of the look-back scan (tagged words; kept apart
 //                                from the partials so arbitrary partial bits never look like a tag)
@@ -59,7 +59,9 @@ static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
 
 constexpr size_t WS_HEADER_BYTES = 256;
 constexpr size_t WS_TICKET_COUNT = 16384;
-constexpr size_t WS_TICKET_BYTES = WS_TICKET_COUNT * sizeof(uint32_t);
+constexpr int TICKET_STRIDE = 32;            // uint32 slots between tickets: one 128-byte line each
+constexpr int TICKET_GROUP = 32;             // workgroups that share a first-level ticket
+constexpr size_t WS_TICKET_BYTES = WS_TICKET_COUNT * TICKET_STRIDE * sizeof(uint32_t);
 constexpr size_t WS_PARTIALS_OFFSET = WS_HEADER_BYTES + WS_TICKET_BYTES;
 constexpr size_t WS_PARTIALS_BYTES = (size_t)8 << 20;
 constexpr size_t WS_DESC_OFFSET = WS_PARTIALS_OFFSET + WS_PARTIALS_BYTES;

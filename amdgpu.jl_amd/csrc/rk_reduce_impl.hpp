@@ -155,20 +155,46 @@ __global__ __launch_bounds__(BLOCK) void reduce_split_kernel(const In* __restric
         if (t == 0) sink(line, a);
         return;
     }
+    // Two levels of completion tickets.  Device-wide atomics on ONE address complete at roughly 14 ns each
+    // on MI355X, so thousands of workgroups must not share a ticket: groups of TICKET_GROUP workgroups
+    // share one (each on its own 128-byte line), the last arrival of a group folds the group's partials
+    // in lane order and takes a ticket of the line, the last group folds the group results.  All orders
+    // are fixed, so the result does not depend on arrival order.
+    const int ngroups = (splits + TICKET_GROUP - 1) / TICKET_GROUP;
+    const int grp = s / TICKET_GROUP;
+    const int gsize = (grp == ngroups - 1) ? splits - grp * TICKET_GROUP : TICKET_GROUP;
+    Acc* gpartials = partials + (int64_t)gridDim.y * splits;
+    uint32_t* gticket = tickets + (line * (ngroups + 1) + grp) * TICKET_STRIDE;
+    uint32_t* lticket = tickets + (line * (ngroups + 1) + ngroups) * TICKET_STRIDE;
     if (t == 0) {
         store_agent(&partials[line * splits + s], a);
         publish_barrier();      // the partial is at the coherent level before the ticket moves
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[line], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (old == (uint32_t)splits - 1u);
+        const uint32_t old = __hip_atomic_fetch_add(gticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (old == (uint32_t)gsize - 1u);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __syncthreads();            // everybody has read is_last before it is written again
+    if (t < WAVE) {
+        static_assert(TICKET_GROUP <= WAVE, "a group is folded by one wave");
+        Acc r = t < gsize ? load_agent(&partials[line * splits + grp * TICKET_GROUP + t]) : Op::template identity<Acc>();
+        r = wave_reduce(r, op);
+        if (t == 0) {
+            *gticket = 0;       // leave the workspace clean for the next call
+            store_agent(&gpartials[line * ngroups + grp], r);
+            publish_barrier();
+            const uint32_t old = __hip_atomic_fetch_add(lticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = (old == (uint32_t)ngroups - 1u);
+        }
     }
     __syncthreads();
     if (!is_last) return;
     Acc r = Op::template identity<Acc>();
-    for (int i = t; i < splits; i += BLOCK) r = op(r, load_agent(&partials[line * splits + i]));
+    for (int i = t; i < ngroups; i += BLOCK) r = op(r, load_agent(&gpartials[line * ngroups + i]));
     r = block_reduce<NW>(r, op, lds);
     if (t == 0) {
         sink(line, r);
-        tickets[line] = 0;   // leave the workspace clean for the next call
+        *lticket = 0;
     }
 }
 
@@ -269,7 +295,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     }
     __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
     if (t == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         is_last = (old == (uint32_t)msplits - 1u);
     }
     __syncthreads();
@@ -279,7 +305,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         for (int i = 0; i < msplits; ++i) f = op(f, load_agent(&partials[(tile * msplits + i) * COLS + t]));
         sink(col + o * g.inner, f);
     }
-    if (t == 0) tickets[tile] = 0;
+    if (t == 0) tickets[tile * TICKET_STRIDE] = 0;
 }
 
 // ---- arbitrary masks: one wave per output ------------------------------------------------------------
@@ -368,11 +394,12 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
     int64_t max_splits = (s.mid + 2 * per_pass - 1) / (2 * per_pass);
     if (want > max_splits) want = max_splits;
     if (want > 4096) want = 4096;
-    const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / nlines;
+    const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / (2 * nlines);   // partials + group partials
     if (want > fit) want = fit;
-    if (want < 1 || nlines > (int64_t)WS_TICKET_COUNT) want = 1;
+    const int64_t groups = (want + TICKET_GROUP - 1) / TICKET_GROUP;
+    if (want < 1 || nlines * (groups + 1) > (int64_t)WS_TICKET_COUNT) want = 1;
     p.splits = (int)want;
-    p.payload = want > 1 ? (size_t)(nlines * want) * sizeof(Acc) : 0;
+    p.payload = want > 1 ? (size_t)(nlines * (want + groups)) * sizeof(Acc) : 0;
     return p;
 }
 

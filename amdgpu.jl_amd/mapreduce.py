@@ -88,12 +88,33 @@ def mapreducedim_(f: str, op: str, R: ROCArray, A: ROCArray, init=None) -> ROCAr
         mask |= 1 << d
     if len(A) == 0:
         return R                                        # mapreduce.jl:91
+    _launch_mapreducedim(f, op, R, A, init, mask)()
+    return R
+
+
+def _launch_mapreducedim(f, op, R, A, init, mask):
+    """Zero-argument callable that enqueues the reduction on the current stream."""
     ws, ws_bytes = workspace()
     ibuf = _scalar_buffer(init, R.dtype)
-    st = L.lib.rk_mapreduce(_MAP[f], _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask,
-                            R.ptr, ibuf, ws, ws_bytes, stream_ptr())
-    L.check(st, "rk_mapreduce")
-    return R
+    args = (_MAP[f], _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, R.ptr, ibuf, ws, ws_bytes)
+    fn = L.lib.rk_mapreduce
+
+    def launch():
+        L.check(fn(*args, stream_ptr()), "rk_mapreduce")
+    return launch
+
+
+def plan_mapreducedim(f: str, op: str, R: ROCArray, A: ROCArray, init=None):
+    """Validate once, return a callable that repeats ``mapreducedim!(f, op, R, A; init)`` with no
+    per-call host work beyond the foreign call (what a compiled ``ccall`` site costs in Julia)."""
+    rdims = R.dims + (1,) * (A.ndim - R.ndim)
+    mask = 0
+    for d, (r, a) in enumerate(zip(rdims, A.dims)):
+        if r != a:
+            if r != 1:
+                raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"mapreducedim!: cannot reduce {A.dims} into {R.dims}")
+            mask |= 1 << d
+    return _launch_mapreducedim(f, op, R, A, init, mask)
 
 
 def mapreduce(f: str, op: str, A: ROCArray, dims=None, init=None):
@@ -169,3 +190,15 @@ def findmax(A: ROCArray, dims=None):
 
 def findmin(A: ROCArray, dims=None):
     return _findminmax(A, False, dims)
+
+
+def plan_findmax(A: ROCArray, vals: ROCArray, idx: ROCArray, dims, want_max: bool = True):
+    """Callable that repeats ``findmax(A; dims)`` into preallocated outputs."""
+    mask = _dims_mask(dims, A.ndim)
+    ws, ws_bytes = workspace()
+    args = (1 if want_max else 0, A.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, vals.ptr, idx.ptr, ws, ws_bytes)
+    fn = L.lib.rk_findminmax
+
+    def launch():
+        L.check(fn(*args, stream_ptr()), "rk_findminmax")
+    return launch

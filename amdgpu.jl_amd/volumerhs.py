@@ -26,3 +26,14 @@ def volumerhs_(rhs: ROCArray, Q: ROCArray, vgeo: ROCArray, gravity, D: ROCArray,
     st = L.lib.rk_volumerhs_f32(rhs.ptr, Q.ptr, vgeo.ptr, float(gravity), D.ptr, nelem, stream_ptr())
     L.check(st, "rk_volumerhs_f32")
     return rhs
+
+
+def plan_volumerhs(rhs: ROCArray, Q: ROCArray, vgeo: ROCArray, gravity, D: ROCArray, nelem: int):
+    """Callable that repeats ``volumerhs!`` on fixed arrays with no per-call host work beyond the
+    foreign call (the benchmark loop of perf/volumerhs.jl:199-202)."""
+    args = (rhs.ptr, Q.ptr, vgeo.ptr, float(gravity), D.ptr, int(nelem))
+    fn = L.lib.rk_volumerhs_f32
+
+    def launch():
+        L.check(fn(*args, stream_ptr()), "rk_volumerhs_f32")
+    return launch
