@@ -149,6 +149,12 @@ def main():
     ms_per_step = wall * 1e3 / K
     value = step_bytes / (wall / K) / 1e9
 
+    # plain copy z .= x through the same broadcast entry point: the practical read+write ceiling of the
+    # device, and the kernel of known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters
+    p_copy = [plan_materialize(bz[i], L(bx[i])) for i in range(2)]
+    copy_avg, copy_min = time_launches(lambda i: p_copy[i % 2](), K)
+    del p_copy
+
     bc_avg, bc_min = time_launches(op_bcast, K)
     sum_avg, sum_min = time_launches(op_sum, K)
     scan_avg, scan_min = time_launches(op_scan, K)
@@ -165,6 +171,7 @@ def main():
         entry("sum Float32[2^26]", n, bytes_sum, sum_avg, sum_min),
         entry("cumsum Int32[2^26]", n, bytes_scan, scan_avg, scan_min),
         entry("z .= a.*x .+ y.*exp.(w) Float32[2^26]", n, bytes_bc, bc_avg, bc_min),
+        entry("copy z .= x Float32[2^26] (device read+write ceiling, counter calibration)", n, 8 * n, copy_avg, copy_min),
     ]
     roofline = {"bound": "hbm", "kernel": "bc_kernel<EvalAxpbyExp,float,4,linear> (z .= a.*x .+ y.*exp.(w), 2^26 elts)",
                 "achieved": round(bytes_bc / (bc_avg * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

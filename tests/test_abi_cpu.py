@@ -1,0 +1,179 @@
+"""CPU-only checks of the C ABI: librk.so loads, exports every symbol include/rk.h declares, and rejects
+bad arguments with status codes before touching the GPU (no compute call is made here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rk.h")
+
+
+@pytest.fixture(scope="module")
+def L(rk):
+    from amdgpu_jl_amd import _lib
+    return _lib
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"RK_API\s+[\w\s\*]+?\b(rk_\w+)\s*\(", text)
+
+
+def test_header_symbols_are_exported_and_bound(L):
+    names = _declared_symbols()
+    assert len(names) >= 10 and len(set(names)) == len(names)
+    raw = C.CDLL(L.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"librk.so does not export {n}"
+        assert n in L.PROTOTYPES, f"the ctypes binding lacks {n}"
+    assert set(L.PROTOTYPES) == set(names)
+
+
+def test_only_c_abi_symbols_are_public(L):
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", L.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    public = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    assert {s for s in public if s.startswith("rk_")} == set(_declared_symbols())
+    assert not [s for s in public if "rk" in s and not s.startswith("rk_") and not s.startswith("_")]
+
+
+def test_header_constants_match_binding(L):
+    text = open(HEADER).read()
+    for name in ("RK_ERR_INVALID_ARGUMENT", "RK_ERR_UNSUPPORTED", "RK_ERR_WORKSPACE", "RK_ERR_DIMENSION", "RK_ERR_TOO_LARGE"):
+        assert int(re.search(name + r"\s*=\s*(\d+)", text).group(1)) == getattr(L, name)
+    assert int(re.search(r"#define RK_MAX_DIMS (\d+)", text).group(1)) == L.RK_MAX_DIMS
+    assert int(re.search(r"#define RK_MAX_OPERANDS (\d+)", text).group(1)) == L.RK_MAX_OPERANDS
+    assert int(re.search(r"#define RK_MAX_PROGRAM (\d+)", text).group(1)) == L.RK_MAX_PROGRAM
+    assert int(re.search(r"#define RK_VERSION (\d+)", text).group(1)) == L.lib.rk_version()
+    assert int(re.search(r"RK_BC_ADD = (\d+)", text).group(1)) == L.RK_BC_ADD
+    assert int(re.search(r"RK_BC_NEG = (\d+)", text).group(1)) == L.RK_BC_NEG
+
+
+def test_status_strings(L):
+    assert L.lib.rk_status_string(0) == b"RK_SUCCESS"
+    for code in (L.RK_ERR_INVALID_ARGUMENT, L.RK_ERR_UNSUPPORTED, L.RK_ERR_WORKSPACE, L.RK_ERR_DIMENSION, L.RK_ERR_TOO_LARGE):
+        assert L.lib.rk_status_string(code).startswith(b"RK_ERR_")
+    assert L.lib.rk_status_string(424242) == b"unknown rk status"
+
+
+def test_mapreduce_argument_validation(L):
+    sh = L.shape_array((10,))
+    one = C.c_void_p(0x1000)                  # never dereferenced: validation fails first
+    f = L.lib.rk_mapreduce
+    assert f(0, 0, L.RK_F32, L.RK_F32, None, 1, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # null arrays
+    assert f(0, 9, L.RK_F32, L.RK_F32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # bad op
+    assert f(7, 0, L.RK_F32, L.RK_F32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # bad map
+    assert f(0, 0, 99, L.RK_F32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT           # bad dtype
+    assert f(0, 0, L.RK_F32, L.RK_F32, one, 9, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # ndim > 8
+    assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, L.shape_array((-1,)), 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert f(0, 0, L.RK_F32, L.RK_I32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Float32 -> Int32
+    assert f(0, 0, L.RK_U64, L.RK_U64, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    # zero-length input: success without launching (src/kernels/mapreduce.jl:91), even with null pointers
+    assert f(0, 0, L.RK_F32, L.RK_F32, None, 1, L.shape_array((0,)), 1, None, None, None, 0, None) == L.RK_SUCCESS
+    # a reduction that needs partials but has no workspace
+    big = L.shape_array((1 << 24,))
+    assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, big, 1, one, None, None, 0, None) == L.RK_ERR_WORKSPACE
+    assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, big, 1, one, None, C.c_void_p(0x1001), 1 << 30, None) == L.RK_ERR_WORKSPACE   # misaligned
+
+
+def test_findminmax_and_accumulate_validation(L):
+    sh = L.shape_array((4, 4))
+    one = C.c_void_p(0x1000)
+    g = L.lib.rk_findminmax
+    assert g(1, L.RK_F32, None, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert g(1, L.RK_F32, one, 2, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # no output requested
+    assert g(1, L.RK_U8, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert g(1, L.RK_F32, None, 2, L.shape_array((0, 4)), 1, None, None, None, 0, None) == L.RK_SUCCESS
+    a = L.lib.rk_accumulate
+    assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert a(0, L.RK_F32, L.RK_F32, one, one, 2, sh, 0, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # dim is 1-based
+    assert a(5, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert a(2, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 0, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # exclusive max needs init
+    assert a(0, L.RK_F32, L.RK_F64, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert a(0, L.RK_U8, L.RK_I64, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT    # aliasing with different sizes
+    assert a(0, L.RK_F32, L.RK_F32, None, None, 1, L.shape_array((0,)), 1, 1, None, None, 0, None) == L.RK_SUCCESS
+    # a look-back scan without workspace
+    assert a(0, L.RK_I32, L.RK_I32, one, C.c_void_p(0x2000), 1, L.shape_array((1 << 24,)), 1, 1, None, None, 0, None) == L.RK_ERR_WORKSPACE
+
+
+def _prog(L, tokens, operands, compute=None):
+    p = L.RkProgram()
+    p.compute = L.RK_F32 if compute is None else compute
+    p.n_operands = len(operands)
+    for k, (ptr, dt, shape) in enumerate(operands):
+        p.operands[k].ptr = ptr
+        p.operands[k].dtype = dt
+        p.operands[k].ndim = len(shape)
+        for d, n in enumerate(shape):
+            p.operands[k].shape[d] = n
+    p.n_tokens = len(tokens)
+    for i, t in enumerate(tokens):
+        p.tokens[i] = t
+    return p
+
+
+def test_broadcast_program_validation(L):
+    b = L.lib.rk_broadcast
+    sh = L.shape_array((4, 3))
+    dest = C.c_void_p(0x1000)
+    arr = lambda *s: (0x2000, L.RK_F32, s)
+    assert b(None, dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT
+    ok_ops = [arr(4, 3), arr(4, 3)]
+    assert b(_prog(L, [0, 1], ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT              # two values left
+    assert b(_prog(L, [0, L.RK_BC_ADD], ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT    # stack underflow
+    assert b(_prog(L, [0, 5, L.RK_BC_ADD], ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT  # operand 5 missing
+    assert b(_prog(L, [0, 1, 999], ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT          # unknown token
+    assert b(_prog(L, [0, 1, L.RK_BC_ADD], ok_ops, compute=L.RK_I32), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_UNSUPPORTED
+    assert b(_prog(L, [0, 1, L.RK_BC_ADD], [arr(4, 3), arr(3, 3)]), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_DIMENSION
+    assert b(_prog(L, [0, 1, L.RK_BC_ADD], [arr(4, 3), arr(4, 3, 2)]), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_DIMENSION
+    assert b(_prog(L, [0, 1, L.RK_BC_ADD], ok_ops), None, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT  # null dest
+    deep = [0] * 9 + [L.RK_BC_ADD] * 8
+    assert b(_prog(L, deep, ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_UNSUPPORTED                     # stack deeper than 8
+    assert b(_prog(L, [0, 1, L.RK_BC_ADD], [arr(0, 3), arr(0, 3)]), None, L.RK_F32, 2, L.shape_array((0, 3)), None) == L.RK_SUCCESS
+
+
+def test_volumerhs_and_scatter_validation(L):
+    v = L.lib.rk_volumerhs_f32
+    one = C.c_void_p(0x1000)
+    assert v(None, one, one, 9.81, one, 10, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert v(one, one, one, 9.81, one, -1, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert v(None, None, None, 9.81, None, 0, None) == L.RK_SUCCESS
+    s = L.lib.rk_findall_scatter
+    assert s(None, one, one, 1, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
+    assert s(None, None, None, 1, L.shape_array((0,)), None) == L.RK_SUCCESS
+    assert s(one, one, one, 9, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
+
+
+def test_workspace_queries(L):
+    wb = L.lib.rk_workspace_bytes
+    base = wb(L.RK_KIND_MAPREDUCE, L.RK_F32, 1, L.shape_array((1 << 20,)), 1)
+    assert base % 256 == 0 and base <= (16 << 20)          # RK_WORKSPACE_DEFAULT serves it
+    small = wb(L.RK_KIND_ACCUMULATE, L.RK_I32, 1, L.shape_array((1000,)), 1)
+    big = wb(L.RK_KIND_ACCUMULATE, L.RK_I32, 1, L.shape_array((1 << 27,)), 1)
+    assert small == base and big > base and big <= (16 << 20)
+    assert wb(L.RK_KIND_ACCUMULATE, L.RK_F32, 2, L.shape_array((4096, 16384)), 1) == base     # lines fit one tile: no descriptors
+    assert wb(L.RK_KIND_ACCUMULATE, 99, 1, None, 0) == base                                    # bad arguments: the generic minimum
+    wi = L.lib.rk_workspace_init
+    assert wi(None, 1 << 24, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert wi(C.c_void_p(0x1001), 1 << 24, None) == L.RK_ERR_WORKSPACE
+    assert wi(C.c_void_p(0x1000), 1024, None) == L.RK_ERR_WORKSPACE
+
+
+def test_host_mirror_rules_without_gpu(rk):
+    """Host-side logic of the mirror that needs no device: eltype rules, broadcast shapes, program flattening."""
+    assert rk.reduce_eltype("add_sum", np.int32) == np.int64 and rk.reduce_eltype("add", np.int32) == np.int32
+    assert rk.accumulate_eltype("add", np.bool_) == np.int64 and rk.accumulate_eltype("add", np.int32) == np.int32
+    from amdgpu_jl_amd import broadcast as B
+    assert B.broadcast_shape((2, 3), (2,)) == (2, 3)
+    with pytest.raises(rk.DimensionMismatch):
+        B.broadcast_shape((2, 3), (3,))
+    a = np.float32(0.5)
+    ops, toks = [], []
+    B._flatten(B._leaf(a * B.lazy(1.0) + B.lazy(2.0) * B.exp(B.lazy(3.0))), ops, toks)
+    from amdgpu_jl_amd import _lib as L
+    assert toks == [0, 1, L.RK_BC_MUL, 2, 3, L.RK_BC_EXP, L.RK_BC_MUL, L.RK_BC_ADD]
+    with pytest.raises(rk.UnsupportedError):
+        B.broadcasted("besselj", 1.0)
