@@ -29,6 +29,9 @@ class Broadcasted:
     """Lazy broadcast node: ``f`` applied to ``args`` (leaves: ROCArray or scalar)."""
 
     __slots__ = ("f", "args")
+    # NumPy scalars must hand `np.float32(0.5) * lazy(x)` to __rmul__ untouched; without this NumPy
+    # would treat the node as an object array and pass a Python float (Float64) instead of 0.5f0
+    __array_ufunc__ = None
 
     def __init__(self, f, args):
         self.f = f

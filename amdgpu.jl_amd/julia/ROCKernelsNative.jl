@@ -1,0 +1,319 @@
+# ROCKernelsNative.jl -- the reference-side binding of librk.so.
+#
+# Load AFTER AMDGPU.jl:  `using AMDGPU; include("ROCKernelsNative.jl"); ROCKernelsNative.enable!()`
+# The Julia API surface does not change.  The method families below get a more specific method whose body
+# is a `ccall` into the hand-written gfx950 kernels (C ABI: include/rk.h); whatever the native layer does not
+# enumerate (arbitrary closures, wrapper types, exotic eltypes) falls through to the stock GPUArrays /
+# AcceleratedKernels methods by `invoke`.
+#
+#   replaced method family                                   reference location
+#   GPUArrays.mapreducedim!(f, op, R::AnyROCArray, A; init)  src/kernels/mapreduce.jl:86-173
+#   Base.accumulate!/accumulate/cumsum/cumprod               src/kernels/accumulate.jl:1-8
+#   Base.copyto!(dest, ::Broadcasted{<:ROCArrayStyle})       src/broadcast.jl:3-35 (+ GPUArrays _copyto!)
+#   findmax/findmin(A; dims)                                 GPUArrays findminmax -> mapreducedim!
+#   volumerhs!(rhs, Q, vgeo, gravity, D, nelem)              perf/volumerhs.jl:200-201
+#
+# This file is shipped as text: no Julia runtime exists where this repository is built and tested, so it is
+# exercised only where `julia` and AMDGPU.jl are installed.  The Python host mirror in this package makes
+# exactly the same calls and is what the test-suite drives.
+module ROCKernelsNative
+
+using AMDGPU
+using AMDGPU: ROCArray, AnyROCArray, ROCArrayStyle, HIP
+import GPUArrays
+import Base.Broadcast: Broadcasted
+
+const librk = Ref{String}(joinpath(@__DIR__, "..", "librk.so"))
+
+# ---- status handling: integer status -> exception, like AMDGPU's @check (src/utils.jl:226-242) -------------
+struct RKError <: Exception
+    code::Int32
+end
+function Base.showerror(io::IO, e::RKError)
+    msg = unsafe_string(ccall((:rk_status_string, librk[]), Cstring, (Int32,), e.code))
+    print(io, "RKError($(e.code)): $msg")
+end
+const RK_ERR_UNSUPPORTED = Int32(10002)
+const RK_ERR_DIMENSION = Int32(10004)
+@inline function check(status::Int32)
+    status == 0 && return nothing
+    status == RK_ERR_DIMENSION && throw(DimensionMismatch("librk: array extents do not agree"))
+    throw(RKError(status))
+end
+
+# ---- enums of include/rk.h ----------------------------------------------------------------------------------
+rk_dtype(::Type{Float32}) = Cint(0); rk_dtype(::Type{Float64}) = Cint(1)
+rk_dtype(::Type{Int32}) = Cint(2);   rk_dtype(::Type{Int64}) = Cint(3)
+rk_dtype(::Type{Bool}) = Cint(4);    rk_dtype(::Type{UInt8}) = Cint(4)
+rk_dtype(::Type{UInt32}) = Cint(5);  rk_dtype(::Type{UInt64}) = Cint(6)
+rk_dtype(::Type) = nothing
+rk_map(::typeof(identity)) = Cint(0); rk_map(::typeof(abs2)) = Cint(1); rk_map(::typeof(abs)) = Cint(2)
+rk_map(_) = nothing
+rk_op(::typeof(+)) = Cint(0); rk_op(::typeof(Base.add_sum)) = Cint(0)
+rk_op(::typeof(*)) = Cint(1); rk_op(::typeof(Base.mul_prod)) = Cint(1)
+rk_op(::typeof(max)) = Cint(2); rk_op(::typeof(min)) = Cint(3)
+rk_op(_) = nothing
+
+# ---- one workspace per (device, stream): the analogue of the per-task library handles (src/cache.jl) --------
+const WORKSPACE_BYTES = 16 << 20
+const workspaces = Dict{Tuple{Int,Ptr{Cvoid}},ROCArray{UInt8,1}}()
+const workspaces_lock = ReentrantLock()
+stream_ptr() = Base.unsafe_convert(Ptr{Cvoid}, AMDGPU.stream().stream)     # hipStream_t of the task-local stream
+function workspace(minbytes::Integer = 0)
+    key = (AMDGPU.device_id(AMDGPU.device()), stream_ptr())
+    lock(workspaces_lock) do
+        ws = get(workspaces, key, nothing)
+        if ws === nothing || length(ws) < minbytes
+            ws = ROCArray{UInt8}(undef, max(WORKSPACE_BYTES, 2minbytes))
+            check(ccall((:rk_workspace_init, librk[]), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                        pointer(ws), length(ws), stream_ptr()))
+            workspaces[key] = ws
+        end
+        ws
+    end
+end
+
+dense(A::ROCArray) = true          # dense column-major storage: (pointer, dims) describes it completely
+dense(_) = false
+
+# ---- mapreducedim! ------------------------------------------------------------------------------------------
+function native_mapreducedim!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N}, init) where {TR,TA,N}
+    Base.check_reducedims(R, A)
+    isempty(A) && return true
+    mask = UInt32(0)
+    for d in 1:N
+        size(R, d) == size(A, d) || (mask |= UInt32(1) << (d - 1))
+    end
+    ws = workspace()
+    shape = Int64[size(A)...]
+    initref = init === nothing ? C_NULL : Ref(convert(TR, init))
+    GC.@preserve R A ws shape initref begin
+        st = ccall((:rk_mapreduce, librk[]), Int32,
+                   (Cint, Cint, Cint, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Cvoid},
+                    Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   rk_map(f), rk_op(op), rk_dtype(TA), rk_dtype(TR), pointer(A), N, shape, mask, pointer(R),
+                   initref === C_NULL ? C_NULL : Base.unsafe_convert(Ptr{Cvoid}, initref),
+                   pointer(ws), length(ws), stream_ptr())
+    end
+    st == RK_ERR_UNSUPPORTED && return false
+    check(st)
+    return true
+end
+
+function enable_mapreduce!()
+    @eval function GPUArrays.mapreducedim!(f::F, op::OP, R::ROCArray{TR}, A::ROCArray{TA}; init=nothing) where {F,OP,TR,TA}
+        if rk_map(f) !== nothing && rk_op(op) !== nothing && rk_dtype(TR) !== nothing && rk_dtype(TA) !== nothing &&
+           ndims(R) <= ndims(A)
+            # with init === nothing the reference combines with R's own contents, which must already be the
+            # neutral element (mapreduce.jl:161-164): overwriting R gives the same result
+            Rn = ndims(R) < ndims(A) ? reshape(R, Base.fill_to_length(size(R), 1, Val(ndims(A)))) : R
+            native_mapreducedim!(f, op, Rn, A, init) && return R
+        end
+        return invoke(GPUArrays.mapreducedim!, Tuple{F,OP,AnyROCArray{TR},Union{AbstractArray,Broadcasted}}, f, op, R, A; init)
+    end
+end
+
+# ---- findmax / findmin ----------------------------------------------------------------------------------------
+function native_findminmax(wantmax::Bool, A::ROCArray{T,N}, dims) where {T,N}
+    mask = UInt32(0)
+    for d in (dims === Colon() ? (1:N) : dims)
+        d <= N && (mask |= UInt32(1) << (d - 1))
+    end
+    rdims = ntuple(d -> (mask >> (d - 1)) & 1 == 1 ? 1 : size(A, d), N)
+    vals = similar(A, T, rdims)
+    idx = similar(A, CartesianIndex{N}, rdims)      # N Int64 per element, the layout the kernel writes
+    ws = workspace()
+    shape = Int64[size(A)...]
+    GC.@preserve A vals idx ws shape begin
+        check(ccall((:rk_findminmax, librk[]), Int32,
+                    (Int32, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Int64}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                    wantmax, rk_dtype(T), pointer(A), N, shape, mask, pointer(vals),
+                    convert(Ptr{Int64}, pointer(idx)), pointer(ws), length(ws), stream_ptr()))
+    end
+    return vals, idx
+end
+function enable_findminmax!()
+    for (fn, wantmax) in ((:findmax, true), (:findmin, false))
+        @eval function Base.$fn(A::ROCArray{T,N}; dims=:) where {T<:Union{Float32,Float64,Int32,Int64},N}
+            vals, idx = native_findminmax($wantmax, A, dims)
+            dims === Colon() || return vals, idx
+            v = AMDGPU.@allowscalar vals[1]
+            i = AMDGPU.@allowscalar idx[1]
+            return v, (N == 1 ? i[1] : i)
+        end
+    end
+end
+
+# ---- accumulate -------------------------------------------------------------------------------------------------
+function native_accumulate!(op, B::ROCArray{TB,N}, A::ROCArray{TA,N}; init, dims, inclusive::Bool) where {TB,TA,N}
+    size(B) == size(A) || throw(DimensionMismatch("accumulate!: $(size(B)) vs $(size(A))"))
+    isempty(A) && return true
+    dim = dims === nothing ? (N == 1 ? 1 : throw(ArgumentError("accumulate on N-d arrays needs dims"))) : Int(dims)
+    shape = Int64[size(A)...]
+    need = ccall((:rk_workspace_bytes, librk[]), Csize_t, (Cint, Cint, Cint, Ptr{Int64}, UInt32),
+                 2, rk_dtype(TB), N, shape, dim <= N ? UInt32(1) << (dim - 1) : UInt32(0))
+    ws = workspace(need)
+    initref = Ref(convert(TB, init))
+    GC.@preserve A B ws shape initref begin
+        st = ccall((:rk_accumulate, librk[]), Int32,
+                   (Cint, Cint, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cint, Ptr{Int64}, Cint, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   rk_op(op), rk_dtype(TA), rk_dtype(TB), pointer(A), pointer(B), N, shape, dim, inclusive,
+                   Base.unsafe_convert(Ptr{Cvoid}, initref), pointer(ws), length(ws), stream_ptr())
+    end
+    st == RK_ERR_UNSUPPORTED && return false
+    check(st)
+    return true
+end
+
+function enable_accumulate!()
+    @eval function Base.accumulate!(op, B::ROCArray, A::ROCArray; init=zero(eltype(A)), dims=nothing, inclusive::Bool=true, kwargs...)
+        if isempty(kwargs) && rk_op(op) !== nothing && rk_dtype(eltype(A)) !== nothing && rk_dtype(eltype(B)) !== nothing
+            native_accumulate!(op, B, A; init, dims, inclusive) && return B
+        end
+        return AMDGPU.AK.accumulate!(op, B, A, AMDGPU.ROCBackend(); init, dims, inclusive, kwargs...)
+    end
+    @eval function Base.accumulate(op, A::ROCArray; init=zero(eltype(A)), kwargs...)
+        B = similar(A, Base.promote_op(op, eltype(A), typeof(init)))
+        return accumulate!(op, B, A; init, kwargs...)
+    end
+    @eval Base.cumsum(A::ROCArray; kwargs...) = accumulate(+, A; kwargs...)
+    @eval Base.cumprod(A::ROCArray; kwargs...) = accumulate(*, A; init=one(eltype(A)), kwargs...)
+end
+
+# ---- fused broadcast: flatten the Broadcasted tree into the postfix program of rk_broadcast -----------------------
+const RK_MAX_DIMS, RK_MAX_OPERANDS, RK_MAX_PROGRAM = 8, 8, 48
+struct RkOperand
+    ptr::Ptr{Cvoid}; dtype::Int32; ndim::Int32; shape::NTuple{8,Int64}; scalar_f::Float64; scalar_i::Int64
+end
+struct RkProgram
+    compute::Int32; n_operands::Int32; operands::NTuple{8,RkOperand}; n_tokens::Int32; tokens::NTuple{48,Int32}
+end
+const BINARY = IdDict{Any,Int32}(+ => 32, - => 33, * => 34, / => 35, max => 36, min => 37, ^ => 38)
+const UNARY = IdDict{Any,Int32}(abs => 65, abs2 => 66, sqrt => 67, exp => 68, log => 69, sin => 70, cos => 71,
+                                tanh => 72, inv => 73, identity => 74)
+struct Unsupported <: Exception end
+
+function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
+    if x isa Broadcasted
+        f, args = x.f, x.args
+        if length(args) == 1 && f === (-)
+            flatten!(ops, toks, args[1]); push!(toks, Int32(64))
+        elseif length(args) == 1 && haskey(UNARY, f)
+            flatten!(ops, toks, args[1]); push!(toks, UNARY[f])
+        elseif length(args) == 2 && haskey(BINARY, f)
+            flatten!(ops, toks, args[1]); flatten!(ops, toks, args[2]); push!(toks, BINARY[f])
+        elseif length(args) == 3 && f === muladd
+            foreach(a -> flatten!(ops, toks, a), args); push!(toks, Int32(39))
+        elseif f === Base.literal_pow && args[3] isa Val{2}          # x .^ 2
+            flatten!(ops, toks, args[2]); push!(toks, Int32(66))
+        else
+            throw(Unsupported())
+        end
+    elseif x isa ROCArray || x isa Union{Float32,Float64,Int32,Int64,Bool}
+        k = findfirst(o -> o === x, ops)
+        k === nothing && (push!(ops, x); k = length(ops))
+        k > RK_MAX_OPERANDS && throw(Unsupported())
+        push!(toks, Int32(k - 1))
+    elseif x isa Base.RefValue && x[] isa Number                    # Ref(scalar)
+        flatten!(ops, toks, x[])
+    else
+        throw(Unsupported())                                        # views, transposes, closures, ...
+    end
+end
+
+function native_copyto!(dest::ROCArray{TD,N}, bc::Broadcasted) where {TD,N}
+    ops, toks = Any[], Int32[]
+    flatten!(ops, toks, bc)
+    length(toks) <= RK_MAX_PROGRAM || throw(Unsupported())
+    CT = promote_type(map(o -> o isa ROCArray ? eltype(o) : typeof(o), ops)...)
+    CT <: Union{Float32,Float64} || length(toks) == 1 || throw(Unsupported())
+    CT <: Union{Float32,Float64} || (CT = Float64)
+    zero_op = RkOperand(C_NULL, 0, 0, ntuple(_ -> Int64(0), 8), 0.0, 0)
+    operands = ntuple(RK_MAX_OPERANDS) do k
+        k > length(ops) && return zero_op
+        o = ops[k]
+        if o isa ROCArray
+            rk_dtype(eltype(o)) === nothing && throw(Unsupported())
+            RkOperand(pointer(o), rk_dtype(eltype(o)), ndims(o), ntuple(d -> d <= ndims(o) ? Int64(size(o, d)) : Int64(0), 8), 0.0, 0)
+        else
+            RkOperand(C_NULL, rk_dtype(typeof(o)), 0, ntuple(_ -> Int64(0), 8), Float64(o), o isa AbstractFloat ? 0 : Int64(o))
+        end
+    end
+    prog = Ref(RkProgram(rk_dtype(CT), length(ops), operands, length(toks),
+                         ntuple(i -> i <= length(toks) ? toks[i] : Int32(0), 48)))
+    shape = Int64[size(dest)...]
+    GC.@preserve dest ops prog shape begin
+        check(ccall((:rk_broadcast, librk[]), Int32, (Ptr{RkProgram}, Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Cvoid}),
+                    prog, pointer(dest), rk_dtype(TD), N, shape, stream_ptr()))
+    end
+    return dest
+end
+
+function enable_broadcast!()
+    @eval function Base.copyto!(dest::ROCArray{TD}, bc::Broadcasted{<:ROCArrayStyle}) where {TD}
+        axes(dest) == axes(bc) || Broadcast.throwdm(axes(dest), axes(bc))
+        isempty(dest) && return dest
+        if rk_dtype(TD) !== nothing
+            try
+                return native_copyto!(dest, bc)
+            catch e
+                e isa Unsupported || rethrow()
+            end
+        end
+        return invoke(Base.copyto!, Tuple{AnyROCArray,Broadcasted{<:GPUArrays.AbstractGPUArrayStyle}}, dest, bc)
+    end
+end
+
+# ---- volumerhs -----------------------------------------------------------------------------------------------------
+"""
+    volumerhs!(rhs, Q, vgeo, gravity, D, nelem)
+
+Drop-in for `@roc groupsize=(5,5) gridsize=nelem volumerhs!(rhs, Q, vgeo, gravity, D, nelem)` (perf/volumerhs.jl:200-201).
+"""
+function volumerhs!(rhs::ROCArray{Float32,5}, Q::ROCArray{Float32,5}, vgeo::ROCArray{Float32,5}, gravity, D::ROCArray{Float32,2}, nelem)
+    size(Q) == size(rhs) == (5, 5, 5, 5, nelem) && size(vgeo) == (5, 5, 5, 14, nelem) && size(D) == (5, 5) ||
+        throw(DimensionMismatch("volumerhs!: N = 4 layouts expected"))
+    GC.@preserve rhs Q vgeo D begin
+        check(ccall((:rk_volumerhs_f32, librk[]), Int32,
+                    (Ptr{Float32}, Ptr{Float32}, Ptr{Float32}, Float32, Ptr{Float32}, Int64, Ptr{Cvoid}),
+                    pointer(rhs), pointer(Q), pointer(vgeo), Float32(gravity), pointer(D), nelem, stream_ptr()))
+    end
+    return nothing
+end
+
+# ---- findall: the scan of this path + the scatter kernel (src/kernels/indexing.jl:8-36) -----------------------------
+function enable_findall!()
+    @eval function Base.findall(bools::ROCArray{Bool,N}) where {N}
+        I = keytype(bools)
+        n = length(bools)
+        n == 0 && return ROCArray{I}(undef, 0)
+        indices = accumulate(+, reshape(bools, n))                   # Bool -> Int64 inclusive scan
+        cnt = AMDGPU.@allowscalar indices[end]
+        ys = ROCArray{I}(undef, cnt)
+        if cnt > 0
+            shape = Int64[size(bools)...]
+            GC.@preserve bools indices ys shape begin
+                check(ccall((:rk_findall_scatter, librk[]), Int32,
+                            (Ptr{UInt8}, Ptr{Int64}, Ptr{Int64}, Cint, Ptr{Int64}, Ptr{Cvoid}),
+                            convert(Ptr{UInt8}, pointer(bools)), pointer(indices), convert(Ptr{Int64}, pointer(ys)),
+                            N, shape, stream_ptr()))
+            end
+        end
+        AMDGPU.unsafe_free!(indices)
+        return ys
+    end
+end
+
+"""
+    enable!()
+
+Install the native methods.  Call once after `using AMDGPU`.
+"""
+function enable!()
+    isfile(librk[]) || error("librk.so not found at $(librk[]); build it with `python amdgpu.jl_amd/build.py`")
+    ccall((:rk_version, librk[]), Int32, ()) >= 100 || error("librk.so is too old")
+    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!()
+    return nothing
+end
+
+end # module

@@ -177,3 +177,6 @@ def test_host_mirror_rules_without_gpu(rk):
     assert toks == [0, 1, L.RK_BC_MUL, 2, 3, L.RK_BC_EXP, L.RK_BC_MUL, L.RK_BC_ADD]
     with pytest.raises(rk.UnsupportedError):
         B.broadcasted("besselj", 1.0)
+    # a NumPy Float32 scalar on the left keeps its type (0.5f0 .* x computes in Float32, not Float64)
+    assert B._compile(np.float32(0.5) * B.lazy(np.float32(2.0)))[2] == np.float32
+    assert B._compile(0.5 * B.lazy(np.float32(2.0)))[2] == np.float64
