@@ -39,6 +39,12 @@ int tune_reduce_blocks_per_cu() {
     return v;
 }
 
+// Workgroups per compute unit of the lanes-along-inner reduction (RK_REDUCE_STRIDED_BLOCKS_PER_CU).
+int tune_reduce_strided_blocks_per_cu() {
+    static const int v = env_int("RK_REDUCE_STRIDED_BLOCKS_PER_CU", 1, 1, 64);
+    return v;
+}
+
 // Look-back polling back-off of the scan, in units of 512 clocks (RK_SCAN_BACKOFF).
 int tune_scan_backoff() {
     static const int v = env_int("RK_SCAN_BACKOFF", 1, 0, 64);

@@ -361,6 +361,7 @@ struct OpMin {
 template <typename T> struct OrderKey;
 template <> struct OrderKey<float> {
     typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
     static __device__ __forceinline__ Key make(float v, bool want_max) {
         const int32_t b = __builtin_bit_cast(int32_t, v);
         const int32_t k = b ^ ((b >> 31) & 0x7fffffff);       // sign-magnitude -> two's complement
@@ -374,6 +375,7 @@ template <> struct OrderKey<float> {
 };
 template <> struct OrderKey<double> {
     typedef int64_t Key;
+    static constexpr bool LOWEST_FREE = true;
     static __device__ __forceinline__ Key make(double v, bool want_max) {
         const int64_t b = __builtin_bit_cast(int64_t, v);
         const int64_t k = b ^ ((b >> 63) & INT64_MAX);
@@ -387,35 +389,49 @@ template <> struct OrderKey<double> {
 };
 template <> struct OrderKey<int32_t> {
     typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = false;
     static __device__ __forceinline__ Key make(int32_t v, bool want_max) { return want_max ? v : ~v; }
     static __device__ __forceinline__ int32_t value(Key k, bool want_max) { return want_max ? k : ~k; }
 };
 template <> struct OrderKey<int64_t> {
     typedef int64_t Key;
+    static constexpr bool LOWEST_FREE = false;
     static __device__ __forceinline__ Key make(int64_t v, bool want_max) { return want_max ? v : ~v; }
     static __device__ __forceinline__ int64_t value(Key k, bool want_max) { return want_max ? k : ~k; }
 };
 
-template <typename K> struct KeyIdx {
-    K       k;
-    int64_t i;     // 0-based column-major linear index into A; -1 = nothing yet
+// `i` is the position of the element along its line (0-based), 32-bit whenever the line is shorter than
+// 2^31 so that key and position travel as one 64-bit word; -1 = nothing yet.
+// LOWEST_FREE: no element maps to the lowest key (true for float keys: the smallest is that of -Inf), so
+// an accumulator that starts at the lowest key takes its first element on a plain "greater than".
+template <typename K, typename P, bool LOWEST_FREE> struct KeyIdx {
+    K k;
+    P i;
 };
 
 struct OpArgKey {
-    template <typename K> __host__ __device__ __forceinline__ KeyIdx<K> operator()(KeyIdx<K> a, KeyIdx<K> b) const {
+    template <typename K, typename P, bool LF>
+    __host__ __device__ __forceinline__ KeyIdx<K, P, LF> operator()(KeyIdx<K, P, LF> a, KeyIdx<K, P, LF> b) const {
         if (a.i < 0) return b;
         if (b.i < 0) return a;
         if (a.k != b.k) return a.k > b.k ? a : b;
         return a.i < b.i ? a : b;
     }
-    template <typename P> static __host__ __device__ __forceinline__ P identity() { P p; p.k = 0; p.i = -1; return p; }
+    template <typename A> static __host__ __device__ __forceinline__ A identity() {
+        A p;
+        p.k = Limits<decltype(p.k)>::lowest();
+        p.i = -1;
+        return p;
+    }
 };
 
 // One step of a streaming accumulation: `x` comes later in index order than everything already in
 // `acc`.  Generic operators just combine; the argmax only replaces on a strictly larger key.
 template <typename Op, typename A> __device__ __forceinline__ A acc_step(Op op, const A& acc, const A& x) { return op(acc, x); }
-template <typename K> __device__ __forceinline__ KeyIdx<K> acc_step(OpArgKey, const KeyIdx<K>& acc, const KeyIdx<K>& x) {
-    return (acc.i < 0 || x.k > acc.k) ? x : acc;
+template <typename K, typename P, bool LF>
+__device__ __forceinline__ KeyIdx<K, P, LF> acc_step(OpArgKey, const KeyIdx<K, P, LF>& acc, const KeyIdx<K, P, LF>& x) {
+    if constexpr (LF) return x.k > acc.k ? x : acc;
+    else return (acc.i < 0 || x.k > acc.k) ? x : acc;
 }
 
 }  // namespace rk

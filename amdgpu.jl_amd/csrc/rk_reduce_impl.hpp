@@ -35,33 +35,39 @@ __device__ __forceinline__ int64_t line_base(const LineGeom& g, int64_t q) {
 }
 
 // ---- element transforms ---------------------------------------------------------------------
-// f is applied in the input type, then converted (Julia: add_sum(widen(f(x)))).
+// Called as xf(value, position along the line).  f is applied in the input type, then converted
+// (Julia: add_sum(widen(f(x)))).
 template <typename In, typename Acc, typename Map> struct MapXform {
+    typedef int64_t Pos;
     __device__ __forceinline__ Acc operator()(In x, int64_t) const { return (Acc)Map()(x); }
 };
-template <typename T> struct ArgXform {
-    bool want_max;
-    typedef KeyIdx<typename OrderKey<T>::Key> P;
-    __device__ __forceinline__ P operator()(T x, int64_t idx) const { P p; p.k = OrderKey<T>::make(x, want_max); p.i = idx; return p; }
+template <typename T, typename P> using ArgAcc = KeyIdx<typename OrderKey<T>::Key, P, OrderKey<T>::LOWEST_FREE>;
+template <typename T, typename P, bool WANT_MAX> struct ArgXform {
+    typedef P Pos;
+    typedef ArgAcc<T, P> A;
+    __device__ __forceinline__ A operator()(T x, P pos) const { A p; p.k = OrderKey<T>::make(x, WANT_MAX); p.i = pos; return p; }
 };
 
 // ---- result sinks ---------------------------------------------------------------------------
+// Called as sink(output index q, reduced value).
 template <typename Acc, typename Op> struct ReduceSink {
     Acc* R;
     Acc  init;
     int  has_init;
     __device__ __forceinline__ void operator()(int64_t q, Acc t) const { R[q] = has_init ? Op()(init, t) : t; }
 };
-template <typename T> struct ArgSink {
+template <typename T, typename P> struct ArgSink {
     T*       vals;
     int64_t* cart;
     int      ndim;
     int64_t  shape[RK_MAX_DIMS];
     bool     want_max;
-    __device__ __forceinline__ void operator()(int64_t q, KeyIdx<typename OrderKey<T>::Key> t) const {
+    bool     absolute;   // positions are already linear offsets into A (the generic kernel)
+    LineGeom g;
+    __device__ __forceinline__ void operator()(int64_t q, ArgAcc<T, P> t) const {
         if (vals) vals[q] = OrderKey<T>::value(t.k, want_max);
         if (cart) {
-            int64_t rem = t.i;
+            int64_t rem = absolute ? (int64_t)t.i : line_base(g, q) + (int64_t)t.i * g.inner;
             for (int d = 0; d < ndim; ++d) {
                 const int64_t c = rem % shape[d];
                 rem /= shape[d];
@@ -77,6 +83,7 @@ template <typename T> struct ArgSink {
 template <typename In, typename Acc, typename Xf, typename Op, bool VECTOR, int GROUP, int UNROLL>
 __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t base, int64_t n, int64_t stride,
                                                int s, int splits, int t, Xf xf, Op op) {
+    typedef typename Xf::Pos Pos;
     if constexpr (VECTOR) {
         constexpr int VEC = 16 / sizeof(In);
         typedef typename VecOf<In, VEC>::type V;
@@ -91,8 +98,8 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
         const int64_t tail = head + nvec * VEC;
         Acc edge = Op::template identity<Acc>();   // kept apart: the vector body below must see increasing indices
         if (s == 0) {   // fewer than VEC (<= 16 <= GROUP) scalars on either side
-            if (t < head) edge = op(edge, xf(p[t], base + t));
-            if (tail + t < n) edge = op(edge, xf(p[tail + t], base + tail + t));
+            if (t < head) edge = op(edge, xf(p[t], (Pos)t));
+            if (tail + t < n) edge = op(edge, xf(p[tail + t], (Pos)(tail + t)));
         }
         constexpr int64_t CHUNK = (int64_t)GROUP * UNROLL;
         const int64_t nchunks = nvec / CHUNK;
@@ -103,16 +110,16 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
             for (int u = 0; u < UNROLL; ++u) v[u] = load_nt(pv + i0 + (int64_t)u * GROUP);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
-                const int64_t e0 = base + head + (i0 + (int64_t)u * GROUP) * VEC;
+                const Pos e0 = (Pos)(head + (i0 + (int64_t)u * GROUP) * VEC);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0 + j));
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], (Pos)(e0 + j)));
             }
         }
         for (int64_t i = nchunks * CHUNK + (int64_t)s * GROUP + t; i < nvec; i += (int64_t)splits * GROUP) {
             const V v = load_nt(pv + i);
-            const int64_t e0 = base + head + i * VEC;
+            const Pos e0 = (Pos)(head + i * VEC);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0 + j));
+            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], (Pos)(e0 + j)));
         }
         Acc a = edge;
 #pragma unroll
@@ -129,9 +136,9 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) v[u] = A[base + (k + u * step) * stride];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], base + (k + u * step) * stride));
+            for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], (Pos)(k + u * step)));
         }
-        for (; k < n; k += step) acc[0] = acc_step(op, acc[0], xf(A[base + k * stride], base + k * stride));
+        for (; k < n; k += step) acc[0] = acc_step(op, acc[0], xf(A[base + k * stride], (Pos)k));
         Acc a = acc[0];
 #pragma unroll
         for (int u = 1; u < UNROLL; ++u) a = op(a, acc[u]);
@@ -216,7 +223,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
     if (line >= g.nlines) return;
     const int64_t base = line_base(g, line);
     Acc a = Op::template identity<Acc>();
-    for (int64_t k = 0; k < g.mid; ++k) a = acc_step(op, a, xf(A[base + k * g.inner], base + k * g.inner));
+    for (int64_t k = 0; k < g.mid; ++k) a = acc_step(op, a, xf(A[base + k * g.inner], (typename Xf::Pos)k));
     sink(line, a);
 }
 
@@ -254,21 +261,21 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
             for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(A + slab + (m + u * NW) * g.inner + col0));
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
-                const int64_t e0 = slab + (m + u * NW) * g.inner + col0;
+                const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
                 if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
                 else {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0 + j));
+                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0));
                 }
             }
         }
         for (; m < m1; m += NW) {
             const V v = load_nt((const V*)(A + slab + m * g.inner + col0));
-            const int64_t e0 = slab + m * g.inner + col0;
+            const typename Xf::Pos e0 = (typename Xf::Pos)m;
             if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v, e0));
             else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0 + j));
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0));
             }
         }
     }
@@ -300,9 +307,39 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     }
     __syncthreads();
     if (!is_last) return;
+    // Last arrival of the strip: fold the msplits rows of partials.  The partials were written through to the
+    // coherent level; one acquire (cache invalidate) in this single workgroup lets it read them with plain,
+    // batched loads.  Wave w folds rows w, w+4, ... for the same columns it streamed; fixed order.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    {
+        const Acc* prow = partials + tile * msplits * COLS + lane * VEC;
+        Acc f[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) f[j] = Op::template identity<Acc>();
+        int i = wave;
+        for (; i + 3 * NW < msplits; i += 4 * NW) {
+            Acc v[4][VEC];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[u][j] = prow[(int64_t)(i + u * NW) * COLS + j];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) f[j] = op(f[j], v[u][j]);
+        }
+        for (; i < msplits; i += NW)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) f[j] = op(f[j], prow[(int64_t)i * COLS + j]);
+        __syncthreads();     // lds is free again
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = f[j];
+        __syncthreads();
+    }
     if (t < COLS && col < g.inner) {
-        Acc f = Op::template identity<Acc>();
-        for (int i = 0; i < msplits; ++i) f = op(f, load_agent(&partials[(tile * msplits + i) * COLS + t]));
+        Acc f = lds[0][t];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) f = op(f, lds[w][t]);
         sink(col + o * g.inner, f);
     }
     if (t == 0) tickets[tile * TICKET_STRIDE] = 0;
@@ -332,7 +369,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restr
             off += (r % g.red_size[d]) * g.red_stride[d];
             r /= g.red_size[d];
         }
-        a = op(a, xf(A[off], off));
+        a = op(a, xf(A[off], (typename Xf::Pos)off));
     }
     a = wave_reduce(a, op);
     if (lane_id() == 0) sink(q, a);
@@ -348,7 +385,8 @@ struct ReducePlan {
 };
 
 // Tunables (workgroups per compute unit the streaming kernels aim for).
-int tune_reduce_blocks_per_cu();   // rk_api.hip
+int tune_reduce_blocks_per_cu();           // rk_api.hip
+int tune_reduce_strided_blocks_per_cu();   // rk_api.hip
 
 template <typename In, typename Acc>
 inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
@@ -366,8 +404,11 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
         p.strips = (int)strips;
         int64_t tiles = strips * s.outer;
         int64_t ms = 1;
-        if (tiles < target_blocks && tiles <= (int64_t)WS_TICKET_COUNT) {
-            ms = (target_blocks + tiles - 1) / tiles;
+        // Few, deep workgroups win here: each lane keeps 4 x 16 B in flight, and every extra slice of
+        // `mid` costs a row of partials plus a longer fold (measured: 8 slices beat 64 by 20 %).
+        const int64_t strided_target = (int64_t)cus * tune_reduce_strided_blocks_per_cu();
+        if (tiles < strided_target && tiles <= (int64_t)WS_TICKET_COUNT) {
+            ms = (strided_target + tiles - 1) / tiles;
             const int64_t max_ms = (s.mid + 31) / 32;      // at least 32 rows per workgroup
             if (ms > max_ms) ms = max_ms;
             if (ms > 1024) ms = 1024;
@@ -510,17 +551,29 @@ inline int32_t mapreduce_typed(const MapreduceArgs& a) {
     }
 }
 
-template <typename T>
-inline int32_t findminmax_typed(const FindArgs& a) {
-    ArgSink<T> sink{};
+template <typename T, typename P>
+inline int32_t findminmax_pos(const FindArgs& a, const Shape3& s) {
+    ArgSink<T, P> sink{};
     sink.vals = (T*)a.vals;
     sink.cart = a.cart;
     sink.ndim = a.ndim;
     for (int d = 0; d < a.ndim; ++d) sink.shape[d] = a.shape[d];
     sink.want_max = a.want_max != 0;
-    ArgXform<T> xf{a.want_max != 0};
-    return launch_reduce<T, KeyIdx<typename OrderKey<T>::Key>>((const T*)a.A, a.ndim, a.shape, a.mask, xf, OpArgKey(), sink, a.ws,
-                                                               a.ws_bytes, a.stream);
+    sink.absolute = !s.single_run;
+    sink.g = LineGeom{s.inner, s.mid, s.inner * s.outer};
+    if (a.want_max)
+        return launch_reduce<T, ArgAcc<T, P>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T, P, true>(), OpArgKey(), sink, a.ws,
+                                              a.ws_bytes, a.stream);
+    return launch_reduce<T, ArgAcc<T, P>>((const T*)a.A, a.ndim, a.shape, a.mask, ArgXform<T, P, false>(), OpArgKey(), sink, a.ws,
+                                          a.ws_bytes, a.stream);
+}
+
+template <typename T>
+inline int32_t findminmax_typed(const FindArgs& a) {
+    const Shape3 s = collapse3(a.ndim, a.shape, a.mask);
+    // 32-bit positions along the line whenever they fit (key + position = one 64-bit word)
+    if (s.single_run && s.mid < ((int64_t)1 << 31)) return findminmax_pos<T, int32_t>(a, s);
+    return findminmax_pos<T, int64_t>(a, s);
 }
 
 // one translation unit per type pair (keeps compile times parallel)
