@@ -22,11 +22,14 @@ namespace rk {
 
 constexpr int BC_BLOCK = 256;
 constexpr int BC_MAX_DEPTH = 8;
+constexpr int BC_RPT = 4;            // rows per thread in rows mode
 
 struct BcOperand {
     const void* ptr;        // nullptr: scalar
     int32_t     dtype;
     int32_t     stride0;    // 0 or 1 (elements) along merged dim 0
+    int32_t     reused;     // has an extruded dim: elements are read many times -> cached loads, not streaming
+    int32_t     row_invariant;   // every stride of dims 1.. is 0: the value depends on the dim-0 index only
     int64_t     stride[RK_MAX_DIMS];   // element strides of merged dims 1.. (index d-1)
     double      sf;
     int64_t     si;
@@ -47,14 +50,16 @@ struct BcArgs {
 };
 
 // ---- typed loads / stores --------------------------------------------------------------------------
-template <typename CT, typename S, int VEC>
+template <typename CT, typename S, int VEC, bool CACHED>
 __device__ __forceinline__ void load_as(const void* p, int64_t off, bool contiguous, CT (&v)[VEC]) {
     const S* q = (const S*)p + off;
     if (contiguous) {
         if constexpr (VEC == 1) v[0] = (CT)q[0];
         else {
             typedef typename VecOf<S, VEC>::type V;
-            const V x = load_nt((const V*)q);
+            V x;
+            if constexpr (CACHED) x = *(const V*)q;
+            else x = load_nt((const V*)q);       // single-use data streams past the caches
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[j] = (CT)x[j];
         }
@@ -65,7 +70,25 @@ __device__ __forceinline__ void load_as(const void* p, int64_t off, bool contigu
     }
 }
 
-template <typename CT, int VEC>
+// HOMOG: every array operand and the destination already have the compute type -- no dispatch on the
+// element type anywhere in the kernel (the common all-Float32 / all-Float64 case).
+template <typename CT, int VEC, bool CACHED, bool HOMOG>
+__device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool contiguous, CT (&v)[VEC]) {
+    if constexpr (HOMOG) { load_as<CT, CT, VEC, CACHED>(o.ptr, off, contiguous, v); return; }
+    switch (o.dtype) {
+        case RK_F32: load_as<CT, float, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_F64: load_as<CT, double, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_I32: load_as<CT, int32_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_I64: load_as<CT, int64_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_U32: load_as<CT, uint32_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_U64: load_as<CT, uint64_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        default:     load_as<CT, uint8_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+    }
+}
+
+// MAY_REUSE: rows mode, where an extruded operand is read again and again and should stay cached; the flat
+// mode reads every dense operand exactly once and always streams (one branch less per operand).
+template <typename CT, int VEC, bool MAY_REUSE, bool HOMOG>
 __device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT (&v)[VEC]) {
     if (o.ptr == nullptr) {
         const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64) ? (CT)o.sf : (CT)o.si;
@@ -74,15 +97,8 @@ __device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT
         return;
     }
     const bool contiguous = o.stride0 != 0;
-    switch (o.dtype) {
-        case RK_F32: load_as<CT, float, VEC>(o.ptr, off, contiguous, v); break;
-        case RK_F64: load_as<CT, double, VEC>(o.ptr, off, contiguous, v); break;
-        case RK_I32: load_as<CT, int32_t, VEC>(o.ptr, off, contiguous, v); break;
-        case RK_I64: load_as<CT, int64_t, VEC>(o.ptr, off, contiguous, v); break;
-        case RK_U32: load_as<CT, uint32_t, VEC>(o.ptr, off, contiguous, v); break;
-        case RK_U64: load_as<CT, uint64_t, VEC>(o.ptr, off, contiguous, v); break;
-        default:     load_as<CT, uint8_t, VEC>(o.ptr, off, contiguous, v); break;
-    }
+    if (MAY_REUSE && o.reused != 0) load_typed<CT, VEC, true, HOMOG>(o, off, contiguous, v);
+    else load_typed<CT, VEC, false, HOMOG>(o, off, contiguous, v);
 }
 
 template <typename CT, typename D, int VEC>
@@ -98,8 +114,9 @@ __device__ __forceinline__ void store_as(void* p, int64_t off, const CT (&v)[VEC
     }
 }
 
-template <typename CT, int VEC>
+template <typename CT, int VEC, bool HOMOG>
 __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, const CT (&v)[VEC]) {
+    if constexpr (HOMOG) { store_as<CT, CT, VEC>(p, off, v); return; }
     switch (dtype) {
         case RK_F32: store_as<CT, float, VEC>(p, off, v); break;
         case RK_F64: store_as<CT, double, VEC>(p, off, v); break;
@@ -238,7 +255,7 @@ struct EvalBinary {
 // ---- kernels --------------------------------------------------------------------------------------------
 extern __shared__ __align__(16) unsigned char bc_lds_raw[];
 
-template <typename Eval, typename CT, int VEC, bool ROWS>
+template <typename Eval, typename CT, int VEC, bool ROWS, bool HOMOG>
 __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
     CT* lds = (CT*)bc_lds_raw;
     const int t = threadIdx.x;
@@ -250,47 +267,95 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
 #pragma unroll
         for (int k = 0; k < Eval::NOPS; ++k) off[k] = dest_off * a.op[k].stride0;
     } else {
-        const int64_t rb = (int64_t)blockIdx.x / a.nxb, xb = (int64_t)blockIdx.x - rb * a.nxb;
+        // A thread keeps its dim-0 position and walks BC_RPT consecutive rows: operands that do not depend
+        // on the row (a column vector against a matrix) are loaded once, and the index arithmetic is paid
+        // once per BC_RPT vectors.
+        // The fused evaluators issue the loads of all BC_RPT rows before the first use (rows past the end
+        // are clamped for the loads and skipped for the store); the interpreter goes row by row.
+        const int64_t xb = blockIdx.x, rb = (int64_t)blockIdx.y + (int64_t)blockIdx.z * gridDim.y;
         const int tx = t & ((1 << a.tx_log2) - 1), ty = t >> a.tx_log2;
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
-        const int64_t row = rb * (BC_BLOCK >> a.tx_log2) + ty;
-        if (i0 >= a.shape[0] || row >= a.nrows) return;
-        dest_off = row * a.shape[0] + i0;
+        const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
+        if (i0 >= a.shape[0] || row0 >= a.nrows) return;
+        constexpr int NB = Eval::USES_LDS ? 1 : (Eval::NOPS >= 3 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
+        for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
+            CT in[NB][RK_MAX_OPERANDS][VEC];
 #pragma unroll
-        for (int k = 0; k < Eval::NOPS; ++k) off[k] = i0 * a.op[k].stride0;
-        int64_t rem = row;
-        for (int d = 1; d < a.ndim; ++d) {
-            int64_t c;
-            if (d == a.ndim - 1) c = rem;
-            else { c = rem % a.shape[d]; rem /= a.shape[d]; }
+            for (int b = 0; b < NB; ++b) {
+                int64_t row = row0 + r0 + b;
+                if (row >= a.nrows) row = a.nrows - 1;
 #pragma unroll
-            for (int k = 0; k < Eval::NOPS; ++k) off[k] += c * a.op[k].stride[d - 1];
+                for (int k = 0; k < Eval::NOPS; ++k) off[k] = i0 * a.op[k].stride0;
+                int64_t rem = row;
+                for (int d = 1; d < a.ndim; ++d) {
+                    int64_t c;
+                    if (d == a.ndim - 1) c = rem;
+                    else { c = rem % a.shape[d]; rem /= a.shape[d]; }
+#pragma unroll
+                    for (int k = 0; k < Eval::NOPS; ++k) off[k] += c * a.op[k].stride[d - 1];
+                }
+#pragma unroll
+                for (int k = 0; k < Eval::NOPS; ++k) {
+                    if (k >= a.n_operands) continue;
+                    if (b == 0 || !a.op[k].row_invariant) load_operand<CT, VEC, true, HOMOG>(a.op[k], off[k], in[b][k]);
+                    else {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) in[b][k][j] = in[0][k][j];
+                    }
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const int64_t row = row0 + r0 + b;
+                if (row < a.nrows) {
+                    CT out[VEC];
+                    Eval::template run<CT, VEC>(a, in[b], out, lds);
+                    store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, row * a.shape[0] + i0, out);
+                }
+            }
         }
+        return;
     }
     CT in[RK_MAX_OPERANDS][VEC];
 #pragma unroll
     for (int k = 0; k < Eval::NOPS; ++k)
-        if (k < a.n_operands) load_operand<CT, VEC>(a.op[k], off[k], in[k]);
+        if (k < a.n_operands) load_operand<CT, VEC, false, HOMOG>(a.op[k], off[k], in[k]);
     CT out[VEC];
     Eval::template run<CT, VEC>(a, in, out, lds);
-    store_dest<CT, VEC>(a.dest, a.dest_dtype, dest_off, out);
+    store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, dest_off, out);
 }
 
 template <typename Eval, typename CT>
 static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
     const int VECN = vec ? 4 : 1;
-    int64_t blocks;
-    if (!rows) blocks = (a.total / VECN + BC_BLOCK - 1) / BC_BLOCK;
-    else blocks = a.nxb * ((a.nrows + (BC_BLOCK >> a.tx_log2) - 1) / (BC_BLOCK >> a.tx_log2));
-    if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - 1) * VECN * BC_BLOCK * sizeof(CT) : 0;
-    if (vec) {
-        if (rows) bc_kernel<Eval, CT, 4, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
-        else      bc_kernel<Eval, CT, 4, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+    dim3 grid(1, 1, 1);
+    if (!rows) {
+        const int64_t blocks = (a.total / VECN + BC_BLOCK - 1) / BC_BLOCK;
+        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+        grid.x = (unsigned)blocks;
     } else {
-        if (rows) bc_kernel<Eval, CT, 1, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
-        else      bc_kernel<Eval, CT, 1, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        // x: workgroups along dim 0; (y, z): row blocks -- no division to recover them in the kernel
+        const int64_t rows_per_block = (int64_t)(BC_BLOCK >> a.tx_log2) * BC_RPT;
+        const int64_t row_blocks = (a.nrows + rows_per_block - 1) / rows_per_block;
+        const int64_t gy = row_blocks < 32768 ? row_blocks : 32768;
+        const int64_t gz = (row_blocks + gy - 1) / gy;
+        if (a.nxb > 0x7fffffff || gz > 65535) return RK_ERR_TOO_LARGE;
+        grid = dim3((unsigned)a.nxb, (unsigned)gy, (unsigned)gz);
     }
+    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - 1) * VECN * BC_BLOCK * sizeof(CT) : 0;
+    // homogeneous element types: a kernel without any dispatch on the element type
+    bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : RK_F64);
+    for (int k = 0; k < a.n_operands; ++k)
+        if (a.op[k].ptr != nullptr && a.op[k].dtype != a.dest_dtype) homog = false;
+#define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
+    if (vec) {
+        if (rows) { if (homog) RK_BC_LAUNCH(4, true, true); else RK_BC_LAUNCH(4, true, false); }
+        else      { if (homog) RK_BC_LAUNCH(4, false, true); else RK_BC_LAUNCH(4, false, false); }
+    } else {
+        if (rows) { if (homog) RK_BC_LAUNCH(1, true, true); else RK_BC_LAUNCH(1, true, false); }
+        else      { if (homog) RK_BC_LAUNCH(1, false, true); else RK_BC_LAUNCH(1, false, false); }
+    }
+#undef RK_BC_LAUNCH
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }
@@ -414,7 +479,13 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
         b.sf = o.scalar_f;
         b.si = o.scalar_i;
         b.stride0 = (int32_t)mstride[k][0];
-        for (int d = 1; d < m; ++d) b.stride[d - 1] = mstride[k][d];
+        b.row_invariant = 1;
+        b.reused = (mstride[k][0] == 0) ? 1 : 0;
+        for (int d = 1; d < m; ++d) {
+            b.stride[d - 1] = mstride[k][d];
+            if (mstride[k][d] != 0) b.row_invariant = 0;
+            else b.reused = 1;
+        }
         if (o.ptr != nullptr) {
             if (m > 1 || mstride[k][0] != 1) linear = false;
             if (mstride[k][0] == 1 && !is_aligned(o.ptr, 4 * dtype_size(o.dtype))) vec = false;

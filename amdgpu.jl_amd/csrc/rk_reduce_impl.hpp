@@ -422,7 +422,7 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
     }
     if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
     const bool contiguous = (s.inner == 1);
-    if (nlines >= target_blocks * 2) {
+    if (nlines >= (int64_t)cus * 16) {            // a wave per line already fills every compute unit
         p.kind = ReducePlan::WAVE_LINES;
         p.vector = contiguous && s.mid >= 2 * VEC;
         return p;
