@@ -47,6 +47,12 @@ int tune_reduce_strided_blocks_per_cu() {
     return v;
 }
 
+// Longest line (bytes) still reduced by one wave; longer lines get a workgroup each (RK_REDUCE_WAVE_MAX_BYTES).
+int tune_reduce_wave_max_bytes() {
+    static const int v = env_int("RK_REDUCE_WAVE_MAX_BYTES", 8192, 1, 1 << 30);
+    return v;
+}
+
 // Look-back polling back-off of the scan, in units of 512 clocks (RK_SCAN_BACKOFF).
 int tune_scan_backoff() {
     static const int v = env_int("RK_SCAN_BACKOFF", 1, 0, 64);
@@ -58,6 +64,12 @@ int tune_scan_backoff() {
 int tune_scan_blocks_per_cu() {
     static const int v = env_int("RK_SCAN_BLOCKS_PER_CU", 4, 1, 16);
     return v;
+}
+
+// Waves per workgroup of the look-back scan: 0 = by line length, else 4, 8 or 16 (RK_SCAN_WAVES).
+int tune_scan_waves() {
+    static const int v = env_int("RK_SCAN_WAVES", 0, 0, 16);
+    return (v == 4 || v == 8 || v == 16) ? v : 0;
 }
 
 static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_U64; }

@@ -387,6 +387,7 @@ struct ReducePlan {
 // Tunables (workgroups per compute unit the streaming kernels aim for).
 int tune_reduce_blocks_per_cu();           // rk_api.hip
 int tune_reduce_strided_blocks_per_cu();   // rk_api.hip
+int tune_reduce_wave_max_bytes();          // rk_api.hip
 
 template <typename In, typename Acc>
 inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
@@ -422,7 +423,11 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
     }
     if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
     const bool contiguous = (s.inner == 1);
-    if (nlines >= (int64_t)cus * 16) {            // a wave per line already fills every compute unit
+    // Plenty of lines: a wave per line fills every compute unit -- but only for short lines.  With a wave per
+    // 32 KiB line all 8192 resident waves stream different DRAM pages at once; a workgroup per line keeps the
+    // active region contiguous (measured on 8192 x 8192 Float32: 6.4 -> 6.65 TB/s, findmax 5.7 -> 6.2 TB/s).
+    if (nlines >= (int64_t)cus * 16 &&
+        (s.mid * (int64_t)sizeof(In) <= tune_reduce_wave_max_bytes() || nlines > 65535)) {
         p.kind = ReducePlan::WAVE_LINES;
         p.vector = contiguous && s.mid >= 2 * VEC;
         return p;

@@ -449,6 +449,7 @@ template <typename T, int K> struct ScanTile {     // geometry of the tile kerne
 
 int tune_scan_backoff();        // rk_api.hip
 int tune_scan_blocks_per_cu();  // rk_api.hip
+int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
 
 struct ScanArgs {
     int op;
@@ -522,7 +523,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
     // long lines: the chained look-back scan; tile = NW waves x 8 vectors, as large as the line length allows
     constexpr int KT = 8;
     const int64_t line_bytes = s.mid * (int64_t)sizeof(T);
-    const int nw = line_bytes >= ((int64_t)128 << 20) ? 16 : (line_bytes >= ((int64_t)32 << 20) ? 8 : 4);
+    // measured (Int32, 2^22 .. 2^27 elements): 16 waves beat 8 and 4 at every size -- fewer, larger tiles mean
+    // fewer serialised acquisitions and fewer look-backs; lines that barely exceed one small tile use 8 or 4
+    int nw = line_bytes > ((int64_t)64 << 10) ? 16 : (line_bytes > ((int64_t)32 << 10) ? 8 : 4);
+    if (tune_scan_waves() != 0) nw = tune_scan_waves();
     const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
     const int64_t tpl = (s.mid + TILE - 1) / TILE;
     const int64_t ntiles = tpl * nlines;
