@@ -370,11 +370,16 @@ __global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict
 }
 
 // ---- inner >= 64: lanes along `inner`, 4 waves share the rows of a chunk -----------------------------
-// grid (strips, outer).  A wave keeps R consecutive rows of its 64 * VEC columns in registers, scans
-// them downwards, and the four waves exchange their column totals through LDS.
+// grid (strips, slices, outer).  A workgroup scans the rows [slice * rows_per_slice, +rows_per_slice) of its
+// 64 * VEC columns: a wave keeps R consecutive rows in registers, scans them downwards, and the four waves
+// exchange their column totals through LDS.  With one slice the scan starts from `init`; with several, the
+// exclusive prefix of every (slice, column) comes from `carry_in` (scan_strided_totals_kernel + a scan of the
+// totals), which makes the slices independent: 12 instead of 8 bytes per element, but thousands of workgroups
+// instead of one per strip.
 template <typename In, typename T, typename Op, bool VECTOR, int R>
 __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
-                                                           int inclusive, Op op) {
+                                                           int inclusive, Op op, int64_t rows_per_slice,
+                                                           const T* __restrict__ carry_in, int64_t carry_pitch) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     constexpr int COLS = WAVE * VEC;
     constexpr int NW = 4;
@@ -384,17 +389,20 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int64_t col0 = (int64_t)blockIdx.x * COLS + (int64_t)lane * VEC;
     const bool live = col0 < g.inner;
-    const int64_t slab = (int64_t)blockIdx.y * g.inner * g.mid;
+    const int64_t slab = (int64_t)blockIdx.z * g.inner * g.mid;
+    const int64_t m_begin = (int64_t)blockIdx.y * rows_per_slice;
+    const int64_t m_end = m_begin + rows_per_slice < g.mid ? m_begin + rows_per_slice : g.mid;
     const T ident = Op::template identity<T>();
     T carry[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) carry[j] = init;
-    for (int64_t m0 = 0; m0 < g.mid; m0 += NW * R) {
+    for (int j = 0; j < VEC; ++j)
+        carry[j] = (carry_in != nullptr && live) ? carry_in[((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * carry_pitch + col0 + j] : init;
+    for (int64_t m0 = m_begin; m0 < m_end; m0 += NW * R) {
         const int64_t row0 = m0 + (int64_t)wave * R;
         T v[R][VEC];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (live && row0 + r < g.mid) {
+            if (live && row0 + r < m_end) {
                 const VI x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
                 if constexpr (VEC == 1) v[r][0] = (T)x;
                 else {
@@ -427,7 +435,7 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
         __syncthreads();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (live && row0 + r < g.mid) {
+            if (live && row0 + r < m_end) {
                 VT o;
                 if constexpr (VEC == 1) o = inclusive ? op(pre[0], v[r][0]) : (r == 0 ? pre[0] : op(pre[0], v[r - 1][0]));
                 else {
@@ -438,6 +446,62 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
                 store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o);
             }
         }
+    }
+}
+
+// Column totals of every (slice, column): totals[(o * slices + slice) * pitch + column].
+template <typename In, typename T, typename Op, bool VECTOR, int UNROLL>
+__global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __restrict__ in, T* __restrict__ totals, ScanGeom g, Op op,
+                                                                  int64_t rows_per_slice, int64_t pitch) {
+    constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
+    constexpr int COLS = WAVE * VEC;
+    constexpr int NW = 4;
+    typedef typename VecOf<In, VEC>::type VI;
+    __shared__ T lds[NW][COLS];
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int64_t col0 = (int64_t)blockIdx.x * COLS + (int64_t)lane * VEC;
+    const bool live = col0 < g.inner;
+    const int64_t slab = (int64_t)blockIdx.z * g.inner * g.mid;
+    const int64_t m_begin = (int64_t)blockIdx.y * rows_per_slice;
+    const int64_t m_end = m_begin + rows_per_slice < g.mid ? m_begin + rows_per_slice : g.mid;
+    T acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = Op::template identity<T>();
+    if (live) {
+        // wave w takes the rows of its quarter of the slice in order (the same grouping as the scan kernel is
+        // not required: only the totals matter, and they are combined in a fixed order)
+        int64_t m = m_begin + wave;
+        for (; m + (UNROLL - 1) * NW < m_end; m += UNROLL * NW) {
+            VI x[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) x[u] = load_nt((const VI*)(in + slab + (m + u * NW) * g.inner + col0));
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if constexpr (VEC == 1) acc[0] = op(acc[0], (T)x[u]);
+                else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], (T)x[u][j]);
+                }
+            }
+        }
+        for (; m < m_end; m += NW) {
+            const VI x = load_nt((const VI*)(in + slab + m * g.inner + col0));
+            if constexpr (VEC == 1) acc[0] = op(acc[0], (T)x);
+            else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = op(acc[j], (T)x[j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = acc[j];
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < COLS) {
+        T r = lds[0][t];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) r = op(r, lds[w][t]);
+        totals[((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * pitch + (int64_t)blockIdx.x * COLS + t] = r;
     }
 }
 
@@ -478,9 +542,45 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const int cols = WAVE * (vec ? VEC : 1);
         const int64_t strips = (s.inner + cols - 1) / cols;
         if (strips > 0x7fffffff || s.outer > 65535) return RK_ERR_TOO_LARGE;
-        dim3 grid((unsigned)strips, (unsigned)s.outer);
-        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op);
-        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op);
+        // One workgroup per strip walks all of `mid`; when that leaves most of the device idle, cut `mid` into
+        // slices: totals per slice, an exclusive scan of the totals (a small strided scan in place), then the
+        // slices scan independently from their carry-in.
+        const int64_t pitch = strips * cols;
+        int64_t slices = 1;
+        const int64_t want_blocks = (int64_t)device_info().cus * 4;
+        if (strips * s.outer < want_blocks) {
+            slices = (want_blocks + strips * s.outer - 1) / (strips * s.outer);
+            const int64_t max_slices = s.mid / 64;                       // at least two register tiles of rows per slice
+            if (slices > max_slices) slices = max_slices;
+            const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(T)) / (pitch * s.outer);
+            if (slices > fit) slices = fit;
+            if (slices > 65535) slices = 65535;
+        }
+        Workspace w{};
+        if (slices > 1 && !carve_workspace(a.ws, a.ws_bytes, 0, &w)) slices = 1;   // no workspace: the single-slice kernel still works
+        if (slices <= 1) {
+            dim3 grid((unsigned)strips, 1, (unsigned)s.outer);
+            if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, s.mid, nullptr, 0);
+            else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, s.mid, nullptr, 0);
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
+        }
+        int64_t rps = (s.mid + slices - 1) / slices;
+        rps = (rps + 31) / 32 * 32;                                      // whole register tiles (4 waves x 8 rows)
+        slices = (s.mid + rps - 1) / rps;
+        T* totals = (T*)w.partials;
+        dim3 grid((unsigned)strips, (unsigned)slices, (unsigned)s.outer);
+        if (vec) scan_strided_totals_kernel<In, T, Op, true, 4><<<grid, 256, 0, a.stream>>>(in, totals, g, op, rps, pitch);
+        else     scan_strided_totals_kernel<In, T, Op, false, 4><<<grid, 256, 0, a.stream>>>(in, totals, g, op, rps, pitch);
+        RK_LAUNCH_CHECK();
+        // exclusive scan of the totals along the slice axis, in place, seeded with init: (pitch, slices, outer)
+        ScanGeom tg{pitch, slices, s.outer};
+        const int tcols = WAVE * VEC;                                    // the totals are 16-byte aligned and pitch % VEC == 0
+        dim3 tgrid((unsigned)((pitch + tcols - 1) / tcols), 1, (unsigned)s.outer);
+        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, a.stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0);
+        RK_LAUNCH_CHECK();
+        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
+        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }

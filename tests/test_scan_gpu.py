@@ -97,6 +97,35 @@ def test_exclusive_with_init_dims(rk, orc, shape, dims):
     assert np.array_equal(got, orc.accumulate("add", x, dims=dims, init=7, inclusive=False))
 
 
+SLICED_CASES = [((128, 4096), 2), ((100, 5001), 2), ((67, 3000, 2), 2), ((256, 1 << 14), 2), ((64, 200, 3), 2), ((1000, 777), 2),
+                ((8, 16, 2500), 3)]
+
+
+@pytest.mark.parametrize("shape,dims", SLICED_CASES)
+@pytest.mark.parametrize("op,inclusive", [("add", True), ("add", False), ("max", True), ("min", False)])
+def test_long_scans_across_rows(rk, orc, shape, dims, op, inclusive):
+    # few columns, many rows: the rows are cut into slices that scan independently from carried-in prefixes
+    x = _rng(31).integers(-10**6, 10**6, shape, dtype=np.int32)
+    got = rk.Array(rk.accumulate(op, rk.ROCArray(x), dims=dims, init=-5, inclusive=inclusive))
+    assert np.array_equal(got, orc.accumulate(op, x, dims=dims, init=-5, inclusive=inclusive))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.int64, np.bool_])
+def test_long_scans_across_rows_dtypes(rk, orc, dtype):
+    rng = _rng(32)
+    x = (rng.random((192, 5000)) < 0.3) if dtype == np.bool_ else (rng.standard_normal((192, 5000)) * 100).astype(dtype)
+    d = rk.ROCArray(x)
+    got = rk.Array(rk.cumsum(d, dims=2))
+    want = orc.cumsum(x, dims=2)
+    if dtype == np.float64:
+        np.testing.assert_allclose(got, want, rtol=1e-11, atol=1e-9)
+    else:
+        assert np.array_equal(got, want)
+    if dtype != np.bool_:
+        rk.accumulate_("add", d, d, dims=2)                         # in place
+        assert np.array_equal(rk.Array(d), got)
+
+
 def test_in_place(rk, orc):
     # test/core/rocarray_base.jl:216-220
     x = _rng(25).random(2)
