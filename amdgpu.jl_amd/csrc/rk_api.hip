@@ -72,6 +72,13 @@ int tune_scan_waves() {
     return (v == 4 || v == 8 || v == 16) ? v : 0;
 }
 
+// Workgroups per compute unit the scan across rows aims for when it cuts the rows into slices
+// (RK_SCAN_SLICE_BLOCKS_PER_CU).
+int tune_scan_slice_blocks_per_cu() {
+    static const int v = env_int("RK_SCAN_SLICE_BLOCKS_PER_CU", 32, 1, 256);
+    return v;
+}
+
 static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_U64; }
 
 static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {

@@ -48,7 +48,7 @@ const DeviceInfo& device_info();   // rk_api.hip
 // ---- workspace layout -------------------------------------------------------------------
 // [0, 256)                       WsHeader
 // [256, +2 MiB)                  completion tickets of the multi-workgroup reductions, one per 128-byte line
-// [.., +WS_PARTIALS_BYTES)       partial results of the reductions
+// [.., +WS_PARTIALS_BYTES)       partial results of the reductions, slice totals of the scans across rows
 // [WS_DESC_OFFSET, end)          tile descriptors of the look-back scan (tagged words; kept apart
 //                                from the partials so arbitrary partial bits never look like a tag)
 struct WsHeader {
@@ -63,7 +63,7 @@ constexpr int TICKET_STRIDE = 32;            // uint32 slots between tickets: on
 constexpr int TICKET_GROUP = 32;             // workgroups that share a first-level ticket
 constexpr size_t WS_TICKET_BYTES = WS_TICKET_COUNT * TICKET_STRIDE * sizeof(uint32_t);
 constexpr size_t WS_PARTIALS_OFFSET = WS_HEADER_BYTES + WS_TICKET_BYTES;
-constexpr size_t WS_PARTIALS_BYTES = (size_t)8 << 20;
+constexpr size_t WS_PARTIALS_BYTES = (size_t)10 << 20;
 constexpr size_t WS_DESC_OFFSET = WS_PARTIALS_OFFSET + WS_PARTIALS_BYTES;
 constexpr uint32_t WS_EPOCH_FIRST = 1;
 

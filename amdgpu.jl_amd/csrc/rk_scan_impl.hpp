@@ -514,6 +514,7 @@ template <typename T, int K> struct ScanTile {     // geometry of the tile kerne
 int tune_scan_backoff();        // rk_api.hip
 int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
+int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
 struct ScanArgs {
     int op;
@@ -522,6 +523,67 @@ struct ScanArgs {
     const void* init;
     void* ws; size_t ws_bytes; hipStream_t stream;
 };
+
+// Scan along `mid` with lanes along `inner` (inner >= 64).  With enough strips one workgroup per strip walks all
+// of `mid` (8 bytes per element).  Otherwise `mid` is cut into slices: totals per slice, an exclusive scan of
+// the totals seeded with init (in place in `scratch`; by this function again when there are many slices), then
+// the slices scan independently from their carried-in prefix: 12 bytes per element, but the whole device works.
+// Short slices are deliberate: workgroups that are resident together then cover a compact range of rows, which
+// the memory system serves faster than many rows far apart (measured with power-of-two row strides).
+template <typename In, typename T, typename Op>
+inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, bool aligned, char* scratch,
+                                size_t scratch_bytes, hipStream_t stream) {
+    constexpr int VEC = 16 / sizeof(T);
+    const bool vec = aligned && (g.inner % VEC == 0);
+    const int cols = WAVE * (vec ? VEC : 1);
+    const int64_t strips = (g.inner + cols - 1) / cols;
+    if (strips > 0x7fffffff || g.outer > 65535) return RK_ERR_TOO_LARGE;
+    const int64_t pitch = strips * cols;
+    const int64_t cus = device_info().cus;
+    int64_t slices = 1;
+    if (strips * g.outer < cus * 4) {
+        const int64_t want = cus * tune_scan_slice_blocks_per_cu();
+        slices = (want + strips * g.outer - 1) / (strips * g.outer);
+        const int64_t max_slices = g.mid / 32;                           // at least one register tile of rows per slice
+        if (slices > max_slices) slices = max_slices;
+        const int64_t fit = (int64_t)(scratch_bytes / 33 * 32 / sizeof(T)) / (pitch * g.outer);   // leave room for the scan of the totals
+        if (slices > fit) slices = fit;
+        if (slices > 65535) slices = 65535;
+    }
+    if (slices <= 1) {
+        dim3 grid((unsigned)strips, 1, (unsigned)g.outer);
+        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0);
+        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0);
+        RK_LAUNCH_CHECK();
+        return RK_SUCCESS;
+    }
+    int64_t rps = (g.mid + slices - 1) / slices;
+    rps = (rps + 31) / 32 * 32;                                          // whole register tiles (4 waves x 8 rows)
+    slices = (g.mid + rps - 1) / rps;
+    T* totals = (T*)scratch;
+    const size_t used = ((size_t)(pitch * slices * g.outer) * sizeof(T) + 255) & ~(size_t)255;
+    dim3 grid((unsigned)strips, (unsigned)slices, (unsigned)g.outer);
+    if (vec) scan_strided_totals_kernel<In, T, Op, true, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch);
+    else     scan_strided_totals_kernel<In, T, Op, false, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch);
+    RK_LAUNCH_CHECK();
+    // exclusive scan of the totals along the slice axis, in place, seeded with init: (pitch, slices, outer); the
+    // totals are 16-byte aligned and pitch % VEC == 0
+    const ScanGeom tg{pitch, slices, g.outer};
+    if (slices > 128) {
+        const int32_t st = scan_across_rows<T, T, Op>(totals, totals, tg, init, 0, op, true, scratch + used,
+                                                      used < scratch_bytes ? scratch_bytes - used : 0, stream);
+        if (st != RK_SUCCESS) return st;
+    } else {
+        const int tcols = WAVE * VEC;
+        dim3 tgrid((unsigned)((pitch + tcols - 1) / tcols), 1, (unsigned)g.outer);
+        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0);
+        RK_LAUNCH_CHECK();
+    }
+    if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
+    else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
 
 template <typename In, typename T, typename Op>
 inline int32_t launch_scan(const ScanArgs& a) {
@@ -538,51 +600,11 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const int inclusive = a.inclusive ? 1 : 0;
 
     if (s.inner >= 64) {
-        const bool vec = aligned && (s.inner % VEC == 0);
-        const int cols = WAVE * (vec ? VEC : 1);
-        const int64_t strips = (s.inner + cols - 1) / cols;
-        if (strips > 0x7fffffff || s.outer > 65535) return RK_ERR_TOO_LARGE;
-        // One workgroup per strip walks all of `mid`; when that leaves most of the device idle, cut `mid` into
-        // slices: totals per slice, an exclusive scan of the totals (a small strided scan in place), then the
-        // slices scan independently from their carry-in.
-        const int64_t pitch = strips * cols;
-        int64_t slices = 1;
-        const int64_t want_blocks = (int64_t)device_info().cus * 4;
-        if (strips * s.outer < want_blocks) {
-            slices = (want_blocks + strips * s.outer - 1) / (strips * s.outer);
-            const int64_t max_slices = s.mid / 64;                       // at least two register tiles of rows per slice
-            if (slices > max_slices) slices = max_slices;
-            const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(T)) / (pitch * s.outer);
-            if (slices > fit) slices = fit;
-            if (slices > 65535) slices = 65535;
-        }
         Workspace w{};
-        if (slices > 1 && !carve_workspace(a.ws, a.ws_bytes, 0, &w)) slices = 1;   // no workspace: the single-slice kernel still works
-        if (slices <= 1) {
-            dim3 grid((unsigned)strips, 1, (unsigned)s.outer);
-            if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, s.mid, nullptr, 0);
-            else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, s.mid, nullptr, 0);
-            RK_LAUNCH_CHECK();
-            return RK_SUCCESS;
-        }
-        int64_t rps = (s.mid + slices - 1) / slices;
-        rps = (rps + 31) / 32 * 32;                                      // whole register tiles (4 waves x 8 rows)
-        slices = (s.mid + rps - 1) / rps;
-        T* totals = (T*)w.partials;
-        dim3 grid((unsigned)strips, (unsigned)slices, (unsigned)s.outer);
-        if (vec) scan_strided_totals_kernel<In, T, Op, true, 4><<<grid, 256, 0, a.stream>>>(in, totals, g, op, rps, pitch);
-        else     scan_strided_totals_kernel<In, T, Op, false, 4><<<grid, 256, 0, a.stream>>>(in, totals, g, op, rps, pitch);
-        RK_LAUNCH_CHECK();
-        // exclusive scan of the totals along the slice axis, in place, seeded with init: (pitch, slices, outer)
-        ScanGeom tg{pitch, slices, s.outer};
-        const int tcols = WAVE * VEC;                                    // the totals are 16-byte aligned and pitch % VEC == 0
-        dim3 tgrid((unsigned)((pitch + tcols - 1) / tcols), 1, (unsigned)s.outer);
-        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, a.stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0);
-        RK_LAUNCH_CHECK();
-        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
-        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
-        RK_LAUNCH_CHECK();
-        return RK_SUCCESS;
+        char* scratch = nullptr;
+        size_t scratch_bytes = 0;
+        if (carve_workspace(a.ws, a.ws_bytes, 0, &w)) { scratch = (char*)w.partials; scratch_bytes = WS_PARTIALS_BYTES; }
+        return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream);
     }
     const int64_t nlines = s.inner * s.outer;
     if (s.inner > 1 || s.mid <= 16) {
