@@ -42,8 +42,9 @@ int tune_reduce_blocks_per_cu() {
 }
 
 // Workgroups per compute unit of the lanes-along-inner reduction (RK_REDUCE_STRIDED_BLOCKS_PER_CU).
+// Measured for mapreduce(abs2, +, 8192 x 8192 Float32; dims=2): 1 -> 5.3, 2 -> 6.5, 4 -> 6.3, 8 -> 6.0 TB/s.
 int tune_reduce_strided_blocks_per_cu() {
-    static const int v = env_int("RK_REDUCE_STRIDED_BLOCKS_PER_CU", 1, 1, 64);
+    static const int v = env_int("RK_REDUCE_STRIDED_BLOCKS_PER_CU", 2, 1, 64);
     return v;
 }
 

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
 
 // ---- inner >= 64: lanes along `inner` -------------------------------------------------------------
 // grid (strips, msplits, outer); workgroup = 4 waves; a wave owns 64 * VEC adjacent columns of a
-// strip and every 4th row of the workgroup's slice of `mid`.
+// strip and every 4th row of the row batches dealt to its workgroup.
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int UNROLL>
 __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
                                                              Acc* partials, uint32_t* tickets) {
@@ -249,33 +249,39 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     Acc acc[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) acc[j] = Op::template identity<Acc>();
-    // rows of this workgroup: contiguous slice [m0, m1) of mid
-    const int64_t per = (g.mid + msplits - 1) / msplits;
-    const int64_t m0 = (int64_t)ms * per;
-    const int64_t m1 = (m0 + per < g.mid) ? m0 + per : g.mid;
+    // Rows are dealt out in batches of UNROLL * 4: batch b goes to workgroup b % msplits, so at any moment the
+    // workgroups of a strip (and, strip by strip, the whole grid) read one compact band of rows.  Giving every
+    // workgroup one long contiguous slice instead spreads the reads over rows megabytes apart, which the
+    // memory system serves up to 20 % slower when the row pitch is a power of two.
+    constexpr int64_t BATCH = (int64_t)UNROLL * NW;
+    const int64_t nbatches = (g.mid + BATCH - 1) / BATCH;
     if (live) {
-        int64_t m = m0 + wave;
-        for (; m + (UNROLL - 1) * NW < m1; m += UNROLL * NW) {
+        const In* p = A + slab + col0;
+        for (int64_t b = ms; b < nbatches; b += msplits) {
+            const int64_t m = b * BATCH + wave;
             V v[UNROLL];
+            if (m + (UNROLL - 1) * NW < g.mid) {
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(A + slab + (m + u * NW) * g.inner + col0));
+                for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(p + (m + u * NW) * g.inner));
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
-                if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
-                else {
+                for (int u = 0; u < UNROLL; ++u) {
+                    const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
+                    if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
+                    else {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0));
+                        for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0));
+                    }
                 }
-            }
-        }
-        for (; m < m1; m += NW) {
-            const V v = load_nt((const V*)(A + slab + m * g.inner + col0));
-            const typename Xf::Pos e0 = (typename Xf::Pos)m;
-            if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v, e0));
-            else {
+            } else {
+                for (int64_t r = m; r < g.mid; r += NW) {
+                    const V x = load_nt((const V*)(p + r * g.inner));
+                    const typename Xf::Pos e0 = (typename Xf::Pos)r;
+                    if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(x, e0));
+                    else {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], e0));
+                        for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(x[j], e0));
+                    }
+                }
             }
         }
     }
@@ -405,8 +411,8 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
         p.strips = (int)strips;
         int64_t tiles = strips * s.outer;
         int64_t ms = 1;
-        // Few, deep workgroups win here: each lane keeps 4 x 16 B in flight, and every extra slice of
-        // `mid` costs a row of partials plus a longer fold (measured: 8 slices beat 64 by 20 %).
+        // Few, deep workgroups win here: each lane keeps 4 x 16 B in flight, and every extra share of
+        // `mid` costs a row of partials plus a longer fold.
         const int64_t strided_target = (int64_t)cus * tune_reduce_strided_blocks_per_cu();
         if (tiles < strided_target && tiles <= (int64_t)WS_TICKET_COUNT) {
             ms = (strided_target + tiles - 1) / tiles;
