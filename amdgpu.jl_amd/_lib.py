@@ -38,7 +38,7 @@ RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
 # rk_op
 RK_OP_ADD, RK_OP_MUL, RK_OP_MAX, RK_OP_MIN = range(4)
 # rk_opkind
-RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE = range(3)
+RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE, RK_KIND_FINDALL = range(4)
 # rk_bc_token
 (RK_BC_ADD, RK_BC_SUB, RK_BC_MUL, RK_BC_DIV, RK_BC_MAX, RK_BC_MIN, RK_BC_POW, RK_BC_FMA) = range(32, 40)
 (RK_BC_NEG, RK_BC_ABS, RK_BC_ABS2, RK_BC_SQRT, RK_BC_EXP, RK_BC_LOG, RK_BC_SIN, RK_BC_COS, RK_BC_TANH,
@@ -83,6 +83,7 @@ PROTOTYPES = {
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
                                      C.c_void_p]),
     "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),
+    "rk_findall": (C.c_int32, [C.c_void_p, C.c_int, _I64P, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
 }
 
 

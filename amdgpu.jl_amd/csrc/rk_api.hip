@@ -95,6 +95,8 @@ static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {
     return true;
 }
 
+size_t findall_workspace_need(int64_t n);   // rk_select.hip
+
 }  // namespace rk
 
 using namespace rk;
@@ -128,6 +130,7 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
         const int64_t tpl = (s.mid + tile - 1) / tile, gpl = (tpl + WAVE - 1) / WAVE;
         if (s.inner == 1 && tpl > 1) need += (size_t)((tpl + gpl) * s.outer) * (esz / 4) * sizeof(uint64_t);
     }
+    if (kind == RK_KIND_FINDALL && valid_shape(ndim, shape, &total) && total > 0) need += findall_workspace_need(total);
     return (need + 255) & ~(size_t)255;
 }
 

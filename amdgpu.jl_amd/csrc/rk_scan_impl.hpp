@@ -229,11 +229,26 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ 
 // Device-wide atomics on one address complete at about 14 ns each on MI355X, so the tile is made as large
 // as the problem allows (up to 1024 threads x 8 vectors = 128 KiB of input): 2^27 elements are 4096
 // acquisitions, ~60 us, against ~170 us of streaming.
-// Every workgroup makes exactly one acquisition beyond the last tile, so acquisition number
-// ntiles + gridDim.x - 1 is the last access of the call: its owner advances the epoch and resets the count
-// for the next call, and clears a rotating slice of the descriptor slots this call did not use, so that no
-// slot keeps a tag for more than SWEEP calls (tags are 30-bit epochs).
 constexpr int SCAN_SWEEP = 1024;
+
+// Every workgroup of a chained kernel makes exactly one acquisition beyond the last tile, so acquisition number
+// ntiles + gridDim.x - 1 is the last access of the call.  Its owner (wave 0 runs this) advances the epoch and
+// resets the count for the next call, and clears a rotating slice of the descriptor slots this call did not
+// use, so that no slot keeps a tag for more than SCAN_SWEEP calls (tags are 30-bit epochs).
+__device__ __forceinline__ void chain_finish(unsigned long long cur, int64_t ntiles, int64_t used, unsigned long long* counter,
+                                             uint64_t* desc, int64_t desc_capacity) {
+    if (threadIdx.x >= WAVE || (int64_t)(cur & 0xffffffffull) != ntiles + (int64_t)gridDim.x - 1) return;
+    const int lane = lane_id();
+    uint32_t epoch = (uint32_t)(cur >> 32);
+    const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
+    int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
+    if (lo < used) lo = used;
+    if (hi > desc_capacity) hi = desc_capacity;
+    for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
+    epoch = (epoch + 1u) & 0x3fffffffu;
+    if (epoch == 0u) epoch = 1u;          // tag 0 marks a cleared slot
+    if (lane == 0) *counter = (unsigned long long)epoch << 32;
+}
 
 template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
 __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
@@ -286,19 +301,7 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
         __syncthreads();
         cur = lds_id;
     }
-    // `cur` is this workgroup's one acquisition past the end
-    if (wave == 0 && (int64_t)(cur & 0xffffffffull) == ntiles + (int64_t)gridDim.x - 1) {
-        uint32_t epoch = (uint32_t)(cur >> 32);
-        const int64_t used = (int64_t)Words<T>::N * (ntiles + ngroups);
-        const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
-        int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
-        if (lo < used) lo = used;
-        if (hi > desc_capacity) hi = desc_capacity;
-        for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
-        epoch = (epoch + 1u) & 0x3fffffffu;
-        if (epoch == 0u) epoch = 1u;          // tag 0 marks a cleared slot
-        if (lane == 0) *counter = (unsigned long long)epoch << 32;
-    }
+    chain_finish(cur, ntiles, (int64_t)Words<T>::N * (ntiles + ngroups), counter, desc, desc_capacity);
 }
 
 // ---- contiguous lines shorter than a tile: one wave per line -------------------------------------

@@ -1,0 +1,231 @@
+// findall(::ROCArray{Bool}) in one pass over the mask: stream compaction with the chained look-back of the
+// scan.  Replaces the cumsum + `_ker!` pair of src/kernels/indexing.jl:8-36 (9 bytes per element for the Int64
+// cumsum, 9 more for the scatter) by 1 byte per element read plus the indices written.
+#include <cstdlib>
+
+#include "rk_common.hpp"
+#include "rk_scan_impl.hpp"
+
+namespace rk {
+
+constexpr int SEL_CHUNK = WAVE * 16;                         // Bools one wave covers with one 16-byte load per lane
+
+struct SelShape {
+    int64_t s[RK_MAX_DIMS];
+    int ndim;
+};
+
+// Writes the 1-based index of element `i` (0-based, column-major) as entry `pos` of ys.
+template <bool LINEAR, bool SMALL>
+__device__ __forceinline__ void emit_index(int64_t* __restrict__ ys, int64_t pos, int64_t i, const SelShape& shp) {
+    if constexpr (LINEAR) {
+        ys[pos] = i + 1;
+    } else if constexpr (SMALL) {                            // every extent and the length fit 32 bits
+        uint32_t rem = (uint32_t)i;
+        for (int d = 0; d < shp.ndim; ++d) {
+            const uint32_t e = (uint32_t)shp.s[d], q = rem / e;
+            ys[pos * shp.ndim + d] = (int64_t)(rem - q * e) + 1;
+            rem = q;
+        }
+    } else {
+        int64_t rem = i;
+        for (int d = 0; d < shp.ndim; ++d) {
+            const int64_t q = rem / shp.s[d];
+            ys[pos * shp.ndim + d] = rem - q * shp.s[d] + 1;
+            rem = q;
+        }
+    }
+}
+
+// Persistent workgroups take tiles of SEL_NW * SEL_K * 1024 Bools in acquisition order (see scan_chain_kernel).
+// A lane counts the set bytes of its SEL_K 16-byte loads, the counts are scanned across the wave (DPP) and the
+// workgroup (LDS), the tile total is published and the tile's offset resolved by the two-level look-back.
+// Output: per load, the lanes drop the in-chunk offsets of their set bytes into the wave's LDS strip at their
+// scanned positions; the wave then reads the strip back in order and writes indices with coalesced stores (a
+// lane writing its own run directly makes every store instruction touch 64 different lines: 4x slower at high
+// density).  Only bit 0 of a byte is looked at (Julia's Bool).
+template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K>
+__global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uint8_t* __restrict__ bools, int64_t n, int64_t* __restrict__ ys,
+                                                                       int64_t* __restrict__ count_out, SelShape shp, int aligned,
+                                                                       unsigned long long* counter, uint64_t* desc, int64_t ntiles,
+                                                                       int64_t ngroups, int64_t desc_capacity, int backoff) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int SEL_TILE = SEL_NW * SEL_CHUNK * SEL_K;
+    __shared__ uint16_t lds_strip[SEL_NW][SEL_CHUNK];
+    __shared__ int32_t lds_wave[SEL_NW];
+    __shared__ int64_t lds_prefix;
+    __shared__ unsigned long long lds_id;
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    uint64_t* tile_desc = desc;                                          // [2 words][ntiles]
+    uint64_t* group_desc = desc + (int64_t)Words<int64_t>::N * ntiles;   // [2 words][ngroups]
+    const OpAdd op;
+
+    if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    unsigned long long cur = lds_id;
+    while ((int64_t)(cur & 0xffffffffull) < ntiles) {
+        const int64_t tile = (int64_t)(cur & 0xffffffffull);
+        const uint32_t epoch = (uint32_t)(cur >> 32);
+        const int64_t e0 = tile * SEL_TILE;
+        const int64_t left = n - e0;
+        const int valid = left < SEL_TILE ? (int)left : SEL_TILE;
+        const int woff = wave * (SEL_CHUNK * SEL_K) + lane * 16;
+        // per 16-byte load: bit b of `hits` = byte b of the lane's 16 is set; `pk` packs the lane's first output
+        // position inside the chunk (high half) with the hits (low half), so a tile costs one register per load
+        uint32_t pk[SEL_K];
+        int32_t ktot[SEL_K];                     // hits of the whole chunk (wave-uniform)
+        int32_t carry = 0;
+#pragma unroll
+        for (int k0 = 0; k0 < SEL_K; k0 += 4) {
+            u32x4 x[4];
+            if (aligned && valid == SEL_TILE) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) x[k] = load_nt((const u32x4*)(bools + e0 + woff + (k0 + k) * SEL_CHUNK));
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        uint32_t word = 0;
+#pragma unroll
+                        for (int b = 0; b < 4; ++b) {
+                            const int idx = woff + (k0 + k) * SEL_CHUNK + q * 4 + b;
+                            if (idx < valid) word |= (uint32_t)bools[e0 + idx] << (8 * b);
+                        }
+                        x[k][q] = word;
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                // bit 0 of the four bytes of a word -> bits 24..27 (the partial products land on distinct bits)
+                x[k] &= 0x01010101u;
+                const uint32_t hits = ((x[k][0] * 0x01020408u) >> 24) | ((x[k][1] * 0x01020408u) >> 20 & 0xf0u) |
+                                      ((x[k][2] * 0x01020408u) >> 16 & 0xf00u) | ((x[k][3] * 0x01020408u) >> 12 & 0xf000u);
+                const int32_t c = __popc(hits);
+                const int32_t inc = wave_scan_inclusive(c, op, 0);
+                pk[k0 + k] = ((uint32_t)(inc - c) << 16) | hits;
+                ktot[k0 + k] = read_lane(inc, WAVE - 1);
+                carry += ktot[k0 + k];
+            }
+        }
+        if (lane == 0) lds_wave[wave] = carry;
+        __syncthreads();
+        int32_t wave_prefix = 0, tile_count = 0;
+#pragma unroll
+        for (int w = 0; w < SEL_NW; ++w) {
+            const int32_t c = lds_wave[w];
+            if (w < wave) wave_prefix += c;
+            tile_count += c;
+        }
+        if (wave == 0) {
+            int64_t tile_prefix = 0;
+            if (lane == 0) desc_publish(tile_desc, ntiles, tile, (int64_t)tile_count, (epoch << 2) | DESC_A);
+            if (tile > 0)
+                tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
+                                             (int64_t)0, op, (int64_t)0, backoff);
+            if (lane == 0) {
+                lds_prefix = tile_prefix;
+                if (tile == ntiles - 1 && count_out != nullptr) *count_out = tile_prefix + tile_count;
+            }
+        }
+        __syncthreads();
+        int64_t base = lds_prefix + wave_prefix;
+        uint16_t* strip = lds_strip[wave];
+#pragma unroll
+        for (int k = 0; k < SEL_K; ++k) {
+            if (ktot[k] == 0) continue;                                   // wave-uniform
+            int32_t p = (int32_t)(pk[k] >> 16);
+            for (uint32_t m = pk[k] & 0xffffu; m != 0u; m &= m - 1u) strip[p++] = (uint16_t)(lane * 16 + __ffs(m) - 1);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int64_t i0 = e0 + wave * (SEL_CHUNK * SEL_K) + k * SEL_CHUNK;
+            for (int i = lane; i < ktot[k]; i += WAVE) emit_index<LINEAR, SMALL>(ys, base + i, i0 + strip[i], shp);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();                              // the strip is reused by the next chunk
+            base += ktot[k];
+        }
+        if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        cur = lds_id;
+    }
+    chain_finish(cur, ntiles, (int64_t)Words<int64_t>::N * (ntiles + ngroups), counter, desc, desc_capacity);
+}
+
+__global__ void store_count_kernel(int64_t* p, int64_t v) { *p = v; }
+
+// 16-byte loads per lane and tile (RK_SELECT_LOADS: 4, 8 or 16).  Measured on MI355X, 2^28 Bools, 1 % / 25 % / 100 %
+// set: 4 loads 96 / 179 / 417 us, 8 loads 76 / 161 / 465 us, 16 loads 72 / 167 / 466 us: tile acquisitions are
+// serialised device-wide (one atomic each), so larger tiles win until the output dominates.
+int tune_select_loads() {
+    static const int v = [] { const char* s = std::getenv("RK_SELECT_LOADS"); const int x = s ? std::atoi(s) : 0; return (x == 4 || x == 8 || x == 16) ? x : 16; }();
+    return v;
+}
+int tune_select_blocks_per_cu() {
+    static const int v = [] { const char* s = std::getenv("RK_SELECT_BLOCKS_PER_CU"); const int x = s ? std::atoi(s) : 0; return (x >= 1 && x <= 2) ? x : 2; }();
+    return v;
+}
+
+size_t findall_workspace_need(int64_t n) {
+    const int64_t SEL_TILE = 16 * SEL_CHUNK * 4;                           // the smallest tile any configuration uses
+    const int64_t ntiles = (n + SEL_TILE - 1) / SEL_TILE, ngroups = (ntiles + WAVE - 1) / WAVE;
+    return (size_t)(ntiles + ngroups) * Words<int64_t>::N * sizeof(uint64_t);
+}
+
+}  // namespace rk
+
+using namespace rk;
+
+extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* shape, int64_t* ys, int64_t* count_out, void* ws,
+                              size_t ws_bytes, void* stream) {
+    if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
+    SelShape shp{};
+    shp.ndim = ndim;
+    int64_t n = 1;
+    bool small = true;
+    for (int d = 0; d < RK_MAX_DIMS; ++d) {
+        shp.s[d] = d < ndim ? shape[d] : 1;
+        if (shp.s[d] < 0) return RK_ERR_INVALID_ARGUMENT;
+        if (shp.s[d] != 0 && n > INT64_MAX / shp.s[d]) return RK_ERR_INVALID_ARGUMENT;
+        n *= shp.s[d];
+    }
+    if (n == 0) {
+        if (count_out != nullptr) {
+            store_count_kernel<<<1, 1, 0, (hipStream_t)stream>>>(count_out, 0);
+            RK_LAUNCH_CHECK();
+        }
+        return RK_SUCCESS;
+    }
+    if (bools == nullptr || ys == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (n > 0xffffffffll) small = false;
+    const int nw = 16, kl = tune_select_loads();
+    const int64_t SEL_TILE = (int64_t)nw * SEL_CHUNK * kl;
+    const int64_t ntiles = (n + SEL_TILE - 1) / SEL_TILE, ngroups = (ntiles + WAVE - 1) / WAVE;
+    if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
+    Workspace w{};
+    if (!carve_workspace(ws, ws_bytes, findall_workspace_need(n), &w)) return RK_ERR_WORKSPACE;
+    const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
+    int64_t grid = (int64_t)device_info().cus * tune_select_blocks_per_cu();
+    if (grid > ntiles) grid = ntiles;
+    unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
+    const int aligned = is_aligned(bools, 16) ? 1 : 0;
+    const int backoff = tune_scan_backoff();
+    hipStream_t st = (hipStream_t)stream;
+#define RK_SELECT2(LIN, SM, NWW, KK)                                                                                             \
+    findall_select_kernel<LIN, SM, NWW, KK><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned, counter,  \
+                                                                                   w.desc, ntiles, ngroups, cap, backoff)
+#define RK_SELECT(LIN, SM)                                                                                                       \
+    do {                                                                                                                         \
+        if (kl == 4) RK_SELECT2(LIN, SM, 16, 4);                                                                                 \
+        else if (kl == 8) RK_SELECT2(LIN, SM, 16, 8);                                                                            \
+        else RK_SELECT2(LIN, SM, 16, 16);                                                                                        \
+    } while (0)
+    if (ndim <= 1) RK_SELECT(true, true);
+    else if (small) RK_SELECT(false, true);
+    else RK_SELECT(false, false);
+#undef RK_SELECT
+#undef RK_SELECT2
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}

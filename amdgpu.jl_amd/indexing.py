@@ -1,12 +1,21 @@
-"""Host mirror of ``Base.findall(::AnyROCArray{Bool})`` (src/kernels/indexing.jl:8-36): a cumsum over
-the flattened Bool array (the scan of this path), a scalar fetch of the count, then the scatter kernel."""
+"""Host mirror of ``Base.findall(::AnyROCArray{Bool})`` (src/kernels/indexing.jl:8-36).
+
+``findall`` is the one-pass form: count the true entries (a U8 -> Int64 reduction), fetch the count,
+allocate, then one stream-compaction pass (``rk_findall``).  ``findall_two_pass`` keeps the reference's
+own structure -- Int64 cumsum of the flattened mask, scalar fetch of its last entry, scatter kernel -- on
+the native scan and ``rk_findall_scatter``."""
 from __future__ import annotations
 
 import numpy as np
 
 from . import _lib as L
 from .accumulate import accumulate
-from .array import ROCArray, stream_ptr
+from .array import ROCArray, stream_ptr, workspace
+from .mapreduce import count
+
+
+def _empty(nd: int) -> ROCArray:
+    return ROCArray(dims=(0,) if nd == 1 else (nd, 0), dtype=np.int64)
 
 
 def findall(bools: ROCArray) -> ROCArray:
@@ -14,16 +23,29 @@ def findall(bools: ROCArray) -> ROCArray:
     Int64 ``(N, count)`` array of CartesianIndex columns for N-d arrays (``keytype(bools)``)."""
     if bools.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findall needs a Bool array")
-    n = len(bools)
-    nd = bools.ndim
+    n, nd = len(bools), bools.ndim
     if n == 0:
-        return ROCArray(dims=(0,) if nd == 1 else (nd, 0), dtype=np.int64)
-    flat = bools.reshape(n)
-    indices = accumulate("add", flat)                       # indexing.jl:10
-    count = int(indices.view_range(n, n).item())            # indexing.jl:12 (@allowscalar indices[end])
-    ys = ROCArray(dims=(count,) if nd == 1 else (nd, count), dtype=np.int64)
-    if count > 0:
+        return _empty(nd)
+    total = int(count(bools))                                # indexing.jl:12 (the scalar fetch)
+    ys = ROCArray(dims=(total,) if nd == 1 else (nd, total), dtype=np.int64)
+    if total > 0:
+        shape = L.shape_array(bools.dims)
+        ws, ws_bytes = workspace(L.lib.rk_workspace_bytes(L.RK_KIND_FINDALL, L.RK_U8, nd, shape, 0))
+        L.check(L.lib.rk_findall(bools.ptr, nd, shape, ys.ptr, None, ws, ws_bytes, stream_ptr()), "rk_findall")
+    return ys
+
+
+def findall_two_pass(bools: ROCArray) -> ROCArray:
+    """The reference's sequence of kernels: cumsum (indexing.jl:10), count fetch (:12), scatter (:16-31)."""
+    if bools.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findall needs a Bool array")
+    n, nd = len(bools), bools.ndim
+    if n == 0:
+        return _empty(nd)
+    indices = accumulate("add", bools.reshape(n))
+    total = int(indices.view_range(n, n).item())
+    ys = ROCArray(dims=(total,) if nd == 1 else (nd, total), dtype=np.int64)
+    if total > 0:
         st = L.lib.rk_findall_scatter(bools.ptr, indices.ptr, ys.ptr, nd, L.shape_array(bools.dims), stream_ptr())
         L.check(st, "rk_findall_scatter")
     return ys
-

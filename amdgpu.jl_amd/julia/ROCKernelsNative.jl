@@ -281,25 +281,26 @@ function volumerhs!(rhs::ROCArray{Float32,5}, Q::ROCArray{Float32,5}, vgeo::ROCA
     return nothing
 end
 
-# ---- findall: the scan of this path + the scatter kernel (src/kernels/indexing.jl:8-36) -----------------------------
+# ---- findall: count, then one stream-compaction pass (replaces src/kernels/indexing.jl:8-36) ---------------------------
 function enable_findall!()
     @eval function Base.findall(bools::ROCArray{Bool,N}) where {N}
         I = keytype(bools)
         n = length(bools)
         n == 0 && return ROCArray{I}(undef, 0)
-        indices = accumulate(+, reshape(bools, n))                   # Bool -> Int64 inclusive scan
-        cnt = AMDGPU.@allowscalar indices[end]
+        cnt = sum(reshape(bools, n))                                 # Bool -> Int64 reduction (rk_mapreduce), scalar fetch
         ys = ROCArray{I}(undef, cnt)
         if cnt > 0
             shape = Int64[size(bools)...]
-            GC.@preserve bools indices ys shape begin
-                check(ccall((:rk_findall_scatter, librk[]), Int32,
-                            (Ptr{UInt8}, Ptr{Int64}, Ptr{Int64}, Cint, Ptr{Int64}, Ptr{Cvoid}),
-                            convert(Ptr{UInt8}, pointer(bools)), pointer(indices), convert(Ptr{Int64}, pointer(ys)),
-                            N, shape, stream_ptr()))
+            need = ccall((:rk_workspace_bytes, librk[]), Csize_t, (Cint, Cint, Cint, Ptr{Int64}, UInt32),
+                         3, rk_dtype(Bool), N, shape, UInt32(0))     # 3 = RK_KIND_FINDALL
+            ws = workspace(need)
+            GC.@preserve bools ys shape ws begin
+                check(ccall((:rk_findall, librk[]), Int32,
+                            (Ptr{UInt8}, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                            convert(Ptr{UInt8}, pointer(bools)), N, shape, convert(Ptr{Int64}, pointer(ys)), C_NULL,
+                            pointer(ws), sizeof(ws), stream_ptr()))
             end
         end
-        AMDGPU.unsafe_free!(indices)
         return ys
     end
 end

@@ -118,6 +118,8 @@ def main():
     from amdgpu_jl_amd.accumulate import plan_accumulate
     from amdgpu_jl_amd.broadcast import plan_materialize
     from amdgpu_jl_amd.volumerhs import plan_volumerhs
+    from amdgpu_jl_amd import _lib as RL
+    from amdgpu_jl_amd.array import workspace, stream_ptr
     p_sum = [plan_mapreducedim(rk.identity, rk.add, sum_out, x) for x in sum_in]
     p_scan = [plan_accumulate("add", o, x) for o, x in zip(scan_out, scan_in)]
     p_bc = [plan_materialize(bz[i], exprs[i]) for i in range(2)]
@@ -236,6 +238,17 @@ def main():
         run_cfg("cfg3b cumsum(B;dims=1) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pa[i % 2]())
         run_cfg("cumsum(B;dims=2) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pb[i % 2]())
         del Bi, Bo, pa, pb
+        # findall: the scan's direct consumer (src/kernels/indexing.jl:8-36); one pass: 1 B/elt read + 8 B per index written
+        m = 1 << 26
+        masks = [dev_array((rand_f32(m) < 0.25), (m,), np.bool_) for _ in range(2)]
+        cnts = [int(rk.count(b)) for b in masks]
+        ysel = [rk.ROCArray(dims=(c,), dtype=np.int64) for c in cnts]
+        shp = RL.shape_array((m,))
+        wsp, wsb = workspace(RL.lib.rk_workspace_bytes(RL.RK_KIND_FINDALL, RL.RK_U8, 1, shp, 0))
+        def run_findall(i):
+            RL.check(RL.lib.rk_findall(masks[i % 2].ptr, 1, shp, ysel[i % 2].ptr, None, wsp, wsb, stream_ptr()), "rk_findall")
+        run_cfg("findall(Bool[2^26], 25 % true) one pass, count known", m, m + 8 * cnts[0], run_findall)
+        del masks, ysel
         # cfg 4
         m = 512 ** 3
         x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))

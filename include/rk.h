@@ -78,7 +78,7 @@ typedef enum { RK_OP_ADD = 0, RK_OP_MUL = 1, RK_OP_MAX = 2, RK_OP_MIN = 3 } rk_o
 
 /* which entry point a workspace is sized for */
 typedef enum {
-    RK_KIND_MAPREDUCE = 0, RK_KIND_FINDMINMAX = 1, RK_KIND_ACCUMULATE = 2
+    RK_KIND_MAPREDUCE = 0, RK_KIND_FINDMINMAX = 1, RK_KIND_ACCUMULATE = 2, RK_KIND_FINDALL = 3
 } rk_opkind;
 
 /* ---- library ------------------------------------------------------------------- */
@@ -199,6 +199,19 @@ RK_API int32_t rk_volumerhs_f32(float* rhs, const float* Q, const float* vgeo, f
  * index when ndim == 1) to ys[indices[i]-1]. */
 RK_API int32_t rk_findall_scatter(const uint8_t* bools, const int64_t* indices, int64_t* ys,
                            int ndim, const int64_t* shape, void* stream);
+
+/* ---- findall in one pass ------------------------------------------------------------------
+ * Replaces the whole body of Base.findall(::AnyROCArray{Bool})  src/kernels/indexing.jl:8-36
+ * after the count is known: the Int64 cumsum (`:10`), the scatter kernel (`:16-31`) and the
+ * temporary they share (`:33`) become one pass that reads each Bool once and writes the indices.
+ * `ys` must hold count(bools) entries (the caller gets the count from
+ * rk_mapreduce(RK_MAP_IDENTITY, RK_OP_ADD, RK_U8 -> RK_I64), the `indices[end]` of `:12`):
+ * `ndim` Int64 per entry (1-based CartesianIndex, column-major), or the linear index when
+ * ndim <= 1; entries are in column-major order of the elements.  Only bit 0 of a Bool byte is
+ * looked at.  If `count_out` is not NULL it receives the number of entries written (device
+ * pointer, Int64).  Needs the workspace (RK_KIND_FINDALL). */
+RK_API int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* shape, int64_t* ys,
+                   int64_t* count_out, void* ws, size_t ws_bytes, void* stream);
 
 #ifdef __cplusplus
 }

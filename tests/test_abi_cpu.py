@@ -145,6 +145,14 @@ def test_volumerhs_and_scatter_validation(L):
     assert s(None, one, one, 1, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
     assert s(None, None, None, 1, L.shape_array((0,)), None) == L.RK_SUCCESS
     assert s(one, one, one, 9, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
+    f = L.lib.rk_findall
+    two = C.c_void_p(0x2000)
+    assert f(None, 1, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert f(one, 1, L.shape_array((5,)), None, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert f(one, 9, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert f(one, 1, L.shape_array((-5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert f(one, 1, L.shape_array((5,)), one, None, None, 0, None) == L.RK_ERR_WORKSPACE
+    assert f(None, 1, L.shape_array((0,)), None, None, None, 0, None) == L.RK_SUCCESS
 
 
 def test_workspace_queries(L):
@@ -155,6 +163,8 @@ def test_workspace_queries(L):
     big = wb(L.RK_KIND_ACCUMULATE, L.RK_I32, 1, L.shape_array((1 << 27,)), 1)
     assert small == base and big > base and big <= (16 << 20)
     assert wb(L.RK_KIND_ACCUMULATE, L.RK_F32, 2, L.shape_array((4096, 16384)), 1) == base     # lines fit one tile: no descriptors
+    assert wb(L.RK_KIND_FINDALL, L.RK_U8, 1, L.shape_array((1 << 31,)), 0) <= (16 << 20)
+    assert wb(L.RK_KIND_FINDALL, L.RK_U8, 1, L.shape_array((1 << 26,)), 0) > base
     assert wb(L.RK_KIND_ACCUMULATE, 99, 1, None, 0) == base                                    # bad arguments: the generic minimum
     wi = L.lib.rk_workspace_init
     assert wi(None, 1 << 24, None) == L.RK_ERR_INVALID_ARGUMENT
