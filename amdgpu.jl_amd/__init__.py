@@ -15,5 +15,7 @@ from . import broadcast                                                         
 from .broadcast import lazy, materialize, materialize_, fill_, Broadcasted             # noqa: F401
 from .volumerhs import volumerhs_                                                     # noqa: F401
 from .indexing import findall                                                         # noqa: F401
+from .reverse import reverse, reverse_                                                # noqa: F401
+from .permutedims import permutedims, permutedims_                                    # noqa: F401
 
 __version__ = "0.1.0"

@@ -83,6 +83,8 @@ PROTOTYPES = {
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
                                      C.c_void_p]),
     "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),
+    "rk_permutedims": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, _I64P, C.POINTER(C.c_int32), C.c_void_p]),
+    "rk_reverse": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, _I64P, C.c_uint32, C.c_void_p]),
     "rk_findall": (C.c_int32, [C.c_void_p, C.c_int, _I64P, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
 }
 

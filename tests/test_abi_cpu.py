@@ -145,8 +145,22 @@ def test_volumerhs_and_scatter_validation(L):
     assert s(None, one, one, 1, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
     assert s(None, None, None, 1, L.shape_array((0,)), None) == L.RK_SUCCESS
     assert s(one, one, one, 9, L.shape_array((5,)), None) == L.RK_ERR_INVALID_ARGUMENT
-    f = L.lib.rk_findall
     two = C.c_void_p(0x2000)
+    r = L.lib.rk_reverse
+    assert r(None, one, 4, 1, L.shape_array((5,)), 1, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert r(one, one, 3, 1, L.shape_array((5,)), 1, None) == L.RK_ERR_UNSUPPORTED
+    assert r(one, one, 4, 9, L.shape_array((5,)), 1, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert r(C.c_void_p(0x1002), one, 4, 1, L.shape_array((5,)), 1, None) == L.RK_ERR_INVALID_ARGUMENT   # misaligned for the element
+    assert r(None, None, 4, 1, L.shape_array((0,)), 1, None) == L.RK_SUCCESS
+    assert r(one, one, 4, 2, L.shape_array((5, 1)), 2, None) == L.RK_SUCCESS          # reverse! of an extent of 1: nothing to do
+    pm = L.lib.rk_permutedims
+    i32 = lambda *v: (C.c_int32 * len(v))(*v)
+    assert pm(one, two, 4, 2, L.shape_array((5, 6)), i32(2, 2), None) == L.RK_ERR_INVALID_ARGUMENT     # not a permutation
+    assert pm(one, two, 4, 2, L.shape_array((5, 6)), i32(0, 1), None) == L.RK_ERR_INVALID_ARGUMENT
+    assert pm(one, one, 4, 2, L.shape_array((5, 6)), i32(2, 1), None) == L.RK_ERR_INVALID_ARGUMENT     # in place is not defined
+    assert pm(one, two, 5, 2, L.shape_array((5, 6)), i32(2, 1), None) == L.RK_ERR_UNSUPPORTED
+    assert pm(None, None, 4, 2, L.shape_array((0, 6)), i32(2, 1), None) == L.RK_SUCCESS
+    f = L.lib.rk_findall
     assert f(None, 1, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(one, 1, L.shape_array((5,)), None, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(one, 9, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT

@@ -367,3 +367,36 @@ def test_golden_fixtures_unchanged():
     assert set(now) == set(gold)
     for k in gold:
         np.testing.assert_allclose(np.array(now[k], dtype=np.float64), np.array(gold[k], dtype=np.float64), rtol=1e-12, err_msg=k)
+
+
+def test_reverse_matches_definition(orc):
+    # element-by-element definition of reverse.jl:73-80: y[ref - idx on flipped dims] = x[idx]
+    rng = np.random.default_rng(7)
+    x = rng.integers(-100, 100, (3, 4, 5)).astype(np.int16)
+    for dims in (None, 1, 2, 3, (1, 3), (2, 3), (1, 2, 3)):
+        flip = {1, 2, 3} if dims is None else ({dims} if isinstance(dims, int) else set(dims))
+        want = np.empty_like(x)
+        for i in range(3):
+            for j in range(4):
+                for k in range(5):
+                    want[2 - i if 1 in flip else i, 3 - j if 2 in flip else j, 4 - k if 3 in flip else k] = x[i, j, k]
+        assert np.array_equal(orc.reverse(x, dims=dims), want)
+    v = np.arange(1, 11)
+    assert orc.reverse(v).tolist() == list(range(10, 0, -1))
+    assert orc.reverse(v, 3, 6).tolist() == [1, 2, 6, 5, 4, 3, 7, 8, 9, 10]          # Base: reverse(1:10 |> collect, 3, 6)
+    assert orc.reverse(v, 4).tolist() == [1, 2, 3, 10, 9, 8, 7, 6, 5, 4]
+
+
+def test_permutedims_matches_definition(orc):
+    rng = np.random.default_rng(8)
+    x = rng.integers(-100, 100, (2, 3, 4)).astype(np.int32)
+    for perm in ((1, 2, 3), (2, 1, 3), (3, 1, 2), (3, 2, 1), (1, 3, 2), (2, 3, 1)):
+        out = orc.permutedims(x, perm)
+        assert out.shape == tuple(x.shape[p - 1] for p in perm)
+        for i in range(2):
+            for j in range(3):
+                for k in range(4):
+                    idx = (i, j, k)
+                    assert out[tuple(idx[p - 1] for p in perm)] == x[i, j, k]
+    m = np.array([[1, 2, 3], [4, 5, 6]])
+    assert orc.permutedims(m, (2, 1)).tolist() == [[1, 4], [2, 5], [3, 6]]       # Base docs: permutedims of a matrix
