@@ -32,7 +32,7 @@ RK_ERR_DIMENSION = 10004
 RK_ERR_TOO_LARGE = 10005
 
 # rk_dtype
-RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64 = range(7)
+RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16 = range(9)
 # rk_map
 RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
 # rk_op
@@ -83,6 +83,9 @@ PROTOTYPES = {
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
                                      C.c_void_p]),
     "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),
+    "rk_sort_tmp_bytes": (C.c_size_t, [C.c_int, C.c_int64, C.c_int32]),
+    "rk_sort": (C.c_int32, [C.c_int, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_sortperm": (C.c_int32, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_permutedims": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, _I64P, C.POINTER(C.c_int32), C.c_void_p]),
     "rk_reverse": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, _I64P, C.c_uint32, C.c_void_p]),
     "rk_findall": (C.c_int32, [C.c_void_p, C.c_int, _I64P, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -80,7 +80,7 @@ int tune_scan_slice_blocks_per_cu() {
     return v;
 }
 
-static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_U64; }
+static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_I16; }   // unsupported combinations fail in the dispatch
 
 static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {
     if (ndim < 0 || ndim > RK_MAX_DIMS) return false;

@@ -33,6 +33,7 @@ inline size_t dtype_size(int dt) {
         case RK_F32: case RK_I32: case RK_U32: return 4;
         case RK_F64: case RK_I64: case RK_U64: return 8;
         case RK_U8: return 1;
+        case RK_F16: case RK_I16: return 2;
         default: return 0;
     }
 }

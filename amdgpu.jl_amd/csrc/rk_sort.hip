@@ -1,0 +1,666 @@
+// sort! / sortperm! of vectors (src/kernels/sorting.jl:1-3, which forwards to AcceleratedKernels' merge sort):
+// least-significant-digit radix sort, 8 bits per pass, one kernel per pass.
+//
+//   sort_init_kernel     clears the histograms, the tile tickets and the tile descriptors (no memset: graph-safe)
+//   sort_min_kernel      one read of the keys: the smallest mapped key, which every key is taken relative to
+//   sort_hist_kernel     one read of the keys: the 256-bin histogram of every digit at once
+//   sort_plan_kernel     exclusive scan of every histogram = first output slot of each digit value; passes whose
+//                        digit is the same for all keys are skipped (small-range integers need 1-2 passes);
+//                        records which buffer each remaining pass reads
+//   sort_pass_kernel     a tile ranks its keys by digit (wave-level match by ballots, counts in LDS), learns how
+//                        many keys of each digit the earlier tiles hold, reorders the tile in LDS and writes runs of
+//                        equal digits.  Up to 1024 tiles (a tunable) the counts of the earlier tiles come from a
+//                        chained look-back (tiles in ticket order publish their 256 counts, one lane per digit walks
+//                        back): a pass reads and writes every key once.  Beyond that the walk is the bottleneck --
+//                        a descriptor is 2 KiB per step against 16 KiB of keys per tile, and the thousand tiles in
+//                        flight resolve their prefixes nearly one after the other (measured: half of the pass) --
+//                        so large sorts count first:
+//   sort_upsweep_kernel  the 256 digit counts of every tile (one more read of the keys), then an exclusive scan
+//                        down the tiles (the strided scan of the accumulate path) gives every tile its offsets.
+//   sort_finish_kernel   moves the result into the caller's array when an odd number of passes ran
+//
+// Keys are mapped to unsigned integers that sort like Base.isless (-0.0 < 0.0, NaN last; every NaN becomes the
+// canonical one), complemented for rev=true; the mapping is applied on the first read and undone on the last
+// write.  The sort is stable, so sortperm keeps equal keys in index order (also with rev=true, as Base does).
+#include <cstdlib>
+
+#include "rk_common.hpp"
+#include "rk_scan_impl.hpp"
+
+namespace rk {
+
+constexpr int SORT_BLOCK = 256;
+constexpr size_t SORT_SCAN_SCRATCH = (size_t)2 << 20;
+constexpr int SORT_NW = SORT_BLOCK / WAVE;
+constexpr int SORT_MAX_PASSES = 8;
+
+struct SortCtl {                                  // head of the caller's temporary buffer
+    uint32_t hist[SORT_MAX_PASSES][256];          // counts, then (sort_plan_kernel) exclusive prefix sums
+    uint32_t ticket[SORT_MAX_PASSES];
+    uint32_t skip[SORT_MAX_PASSES];
+    uint32_t src_is_b[SORT_MAX_PASSES];           // the pass reads buffer B (1) or A (0)
+    uint32_t first_pass, last_pass, nexec, pad;
+    unsigned long long inv_min;                   // ~(smallest mapped key), kept as a maximum so that zero is its identity
+};
+
+// ---- key <-> ordered unsigned integer -----------------------------------------------------------------
+template <typename T> struct SortKey;
+template <> struct SortKey<int16_t> {
+    typedef uint16_t U;
+    static __device__ __forceinline__ U enc(int16_t v) { return (U)((uint16_t)v ^ 0x8000u); }
+    static __device__ __forceinline__ int16_t dec(U u) { return (int16_t)(u ^ 0x8000u); }
+};
+template <> struct SortKey<int32_t> {
+    typedef uint32_t U;
+    static __device__ __forceinline__ U enc(int32_t v) { return (U)v ^ 0x80000000u; }
+    static __device__ __forceinline__ int32_t dec(U u) { return (int32_t)(u ^ 0x80000000u); }
+};
+template <> struct SortKey<int64_t> {
+    typedef uint64_t U;
+    static __device__ __forceinline__ U enc(int64_t v) { return (U)v ^ 0x8000000000000000ull; }
+    static __device__ __forceinline__ int64_t dec(U u) { return (int64_t)(u ^ 0x8000000000000000ull); }
+};
+struct half_bits { uint16_t b; };                 // Float16 travels as its bit pattern
+template <> struct SortKey<half_bits> {
+    typedef uint16_t U;
+    static __device__ __forceinline__ U enc(half_bits v) {
+        uint16_t b = v.b;
+        if ((b & 0x7fffu) > 0x7c00u) b = 0x7e00u;                 // NaN -> canonical, sorts after +Inf
+        return (U)((b & 0x8000u) ? ~b : (b ^ 0x8000u));
+    }
+    static __device__ __forceinline__ half_bits dec(U u) { return half_bits{(uint16_t)((u & 0x8000u) ? (u ^ 0x8000u) : ~u)}; }
+};
+template <> struct SortKey<float> {
+    typedef uint32_t U;
+    static __device__ __forceinline__ U enc(float v) {
+        uint32_t b = __builtin_bit_cast(uint32_t, v);
+        if (v != v) b = 0x7fc00000u;
+        return (b & 0x80000000u) ? ~b : (b ^ 0x80000000u);
+    }
+    static __device__ __forceinline__ float dec(U u) { return __builtin_bit_cast(float, (u & 0x80000000u) ? (u ^ 0x80000000u) : ~u); }
+};
+template <> struct SortKey<double> {
+    typedef uint64_t U;
+    static __device__ __forceinline__ U enc(double v) {
+        uint64_t b = __builtin_bit_cast(uint64_t, v);
+        if (v != v) b = 0x7ff8000000000000ull;
+        return (b & 0x8000000000000000ull) ? ~b : (b ^ 0x8000000000000000ull);
+    }
+    static __device__ __forceinline__ double dec(U u) {
+        return __builtin_bit_cast(double, (u & 0x8000000000000000ull) ? (u ^ 0x8000000000000000ull) : ~u);
+    }
+};
+
+// the same mapping on the raw bit pattern: one load path serves the first pass (caller's keys) and the later ones
+// and relative to the smallest mapped key of the array: small-range integers (and floats of one binade) then have
+// constant high digits, whose passes are skipped
+template <typename T> __device__ __forceinline__ typename SortKey<T>::U enc_bits(typename SortKey<T>::U raw, int rev, typename SortKey<T>::U umin) {
+    typedef typename SortKey<T>::U U;
+    const U u = SortKey<T>::enc(__builtin_bit_cast(T, raw));
+    return (U)((rev ? (U)~u : u) - umin);
+}
+template <typename T> __device__ __forceinline__ T dec_bits(typename SortKey<T>::U k, int rev, typename SortKey<T>::U umin) {
+    typedef typename SortKey<T>::U U;
+    const U u = (U)(k + umin);
+    return SortKey<T>::dec(rev ? (U)~u : u);
+}
+
+template <typename U> __device__ __forceinline__ uint32_t digit_of(U u, int pass) { return (uint32_t)(u >> (8 * pass)) & 0xffu; }
+
+// Mask of the lanes of `valid` whose digit equals this lane's.  Per bit of the digit: e = all ones where the bit is
+// set, m = ballot of the bit; (m ^ e) has a one exactly for the lanes that differ from this lane in that bit.
+__device__ __forceinline__ uint64_t match_digit(uint32_t d, uint64_t valid) {
+    uint32_t diff_lo = 0, diff_hi = 0;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const uint32_t e = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1);
+        const uint64_t m = __ballot(e != 0u);
+        diff_lo |= (uint32_t)m ^ e;
+        diff_hi |= (uint32_t)(m >> 32) ^ e;
+    }
+    return ~(((uint64_t)diff_hi << 32) | diff_lo) & valid;
+}
+
+// Histogram updates in LDS.  Evenly spread digits go in with one LDS atomic per lane.  When many lanes hold the same
+// digit (exponent bytes, the high bytes of small integers) those atomics would queue up on one LDS word, so the
+// lanes are matched first and one lane per digit value adds the whole group.  digits_skewed() is the wave-uniform
+// test: do at least 8 lanes share the first lane's digit?
+__device__ __forceinline__ bool digits_skewed(uint32_t d, bool valid) {
+    const uint64_t active = __ballot(valid);
+    if (active == 0ull) return false;
+    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d, __ffsll((unsigned long long)active) - 1);
+    return __popcll(__ballot(valid && d == d0)) >= 8;
+}
+__device__ __forceinline__ void count_digit(uint32_t* row, uint32_t d, bool valid, bool skewed) {
+    if (skewed) {
+        const uint64_t active = __ballot(valid);
+        if (active == 0ull) return;
+        const int first = __ffsll((unsigned long long)active) - 1;
+        const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d, first);
+        if (__ballot(valid && d == d0) == active) {                       // one value in the whole wave
+            if (lane_id() == first) atomicAdd(&row[d0], (uint32_t)__popcll(active));
+            return;
+        }
+        const uint64_t peers = match_digit(d, active);
+        if (valid && lane_id() == __ffsll((unsigned long long)peers) - 1) atomicAdd(&row[d], (uint32_t)__popcll(peers));
+    } else if (valid) atomicAdd(&row[d], 1u);
+}
+
+// ---- init: clear control block and descriptors ------------------------------------------------------------
+__global__ __launch_bounds__(256) void sort_init_kernel(uint64_t* words, int64_t nwords) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * 256) words[i] = 0;
+}
+
+// The two whole-array reads below take 16-byte vectors from the aligned body [head, head + nvec * VEC) of the keys
+// and single elements from the few keys in front of and behind it.
+template <typename T, typename F>
+__device__ __forceinline__ void for_each_key(const T* __restrict__ keys, int64_t n, int64_t head, int64_t nvec, F&& f) {
+    typedef typename SortKey<T>::U U;
+    constexpr int VEC = 16 / sizeof(T);
+    typedef typename VecOf<U, VEC>::type VU;
+    const VU* body = (const VU*)(keys + head);
+    constexpr int UNR = 4;                                   // loads in flight per lane
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + (UNR - 1) * stride < nvec; i += UNR * stride) {
+        VU v[UNR];
+#pragma unroll
+        for (int r = 0; r < UNR; ++r) v[r] = load_nt(body + i + r * stride);
+#pragma unroll
+        for (int r = 0; r < UNR; ++r) {
+            U k[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) k[j] = (U)v[r][j];
+            f(k, VEC);
+        }
+    }
+    for (; i < nvec; i += stride) {
+        const VU v = load_nt(body + i);
+        U k[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) k[j] = (U)v[j];
+        f(k, VEC);
+    }
+    if (blockIdx.x == 0) {
+        const int64_t tail0 = head + nvec * VEC, extra = head + (n - tail0);     // at most 2 * (VEC - 1) keys
+        for (int64_t i = threadIdx.x; i < extra; i += 256) {
+            const int64_t e = i < head ? i : tail0 + (i - head);
+            U k[VEC];
+            k[0] = __builtin_bit_cast(U, keys[e]);
+            f(k, 1);
+        }
+    }
+}
+
+// ---- smallest mapped key ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void sort_min_kernel(const T* __restrict__ keys, int64_t n, int64_t head, int64_t nvec, int rev,
+                                                       SortCtl* ctl) {
+    typedef typename SortKey<T>::U U;
+    constexpr int VEC = 16 / sizeof(T);
+    __shared__ unsigned long long part[SORT_NW];
+    unsigned long long inv = 0;                  // max of ~u
+    for_each_key<T>(keys, n, head, nvec, [&](const U (&k)[VEC], int cnt) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if (j < cnt) {
+                const unsigned long long x = (unsigned long long)(U)~enc_bits<T>(k[j], rev, (U)0);
+                inv = x > inv ? x : inv;
+            }
+        }
+    });
+    // one device-wide atomic per workgroup: atomics on one address complete one after the other
+    inv = wave_reduce(inv, OpMax());
+    if (lane_id() == 0) part[threadIdx.x / WAVE] = inv;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < SORT_NW; ++w) inv = part[w] > inv ? part[w] : inv;
+        if (inv != 0ull) atomicMax(&ctl->inv_min, inv);
+    }
+}
+
+// ---- all digit histograms in one read -------------------------------------------------------------------------
+template <typename T, int PASSES>
+__global__ __launch_bounds__(256) void sort_hist_kernel(const T* __restrict__ keys, int64_t n, int64_t head, int64_t nvec, int rev,
+                                                        SortCtl* ctl) {
+    typedef typename SortKey<T>::U U;
+    __shared__ uint32_t h[PASSES][256];
+    const U umin = (U)~ctl->inv_min;
+    for (int i = threadIdx.x; i < PASSES * 256; i += 256) (&h[0][0])[i] = 0;
+    __syncthreads();
+    constexpr int VEC = 16 / sizeof(T);
+    for_each_key<T>(keys, n, head, nvec, [&](const U (&k)[VEC], int cnt) {
+        U u[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) u[j] = enc_bits<T>(k[j], rev, umin);
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const bool skewed = digits_skewed(digit_of(u[0], p), true);       // judged on the first key of the vector
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) count_digit(h[p], digit_of(u[j], p), j < cnt, skewed);
+        }
+    });
+    __syncthreads();
+    for (int i = threadIdx.x; i < PASSES * 256; i += 256) {
+        const uint32_t c = (&h[0][0])[i];
+        if (c) atomicAdd(&ctl->hist[0][0] + i, c);
+    }
+}
+
+// ---- plan: scan the histograms, decide which passes run and what they read ---------------------------------------
+// one workgroup of 256 threads; lane d owns digit value d
+__global__ __launch_bounds__(256) void sort_plan_kernel(SortCtl* ctl, int passes, uint32_t n, int first_reads_b) {
+    __shared__ uint32_t wsum[SORT_NW];
+    __shared__ int any_full;
+    const int d = threadIdx.x, wave = d / WAVE, lane = d % WAVE;
+    for (int p = 0; p < passes; ++p) {
+        const uint32_t c = ctl->hist[p][d];
+        if (d == 0) any_full = 0;
+        __syncthreads();
+        if (c == n) any_full = 1;
+        const uint32_t inc = wave_scan_inclusive(c, OpAdd(), 0u);
+        if (lane == WAVE - 1) wsum[wave] = inc;
+        __syncthreads();
+        uint32_t base = 0;
+        for (int w = 0; w < wave; ++w) base += wsum[w];
+        ctl->hist[p][d] = base + inc - c;
+        if (d == 0) ctl->skip[p] = any_full ? 1u : 0u;
+        __syncthreads();
+    }
+    if (d == 0) {
+        uint32_t src_b = first_reads_b ? 1u : 0u, nexec = 0, first = 0xffffffffu, last = 0xffffffffu;
+        for (int p = 0; p < passes; ++p) {
+            if (ctl->skip[p]) continue;
+            ctl->src_is_b[p] = src_b;
+            src_b ^= 1u;
+            if (first == 0xffffffffu) first = (uint32_t)p;
+            last = (uint32_t)p;
+            ++nexec;
+        }
+        ctl->first_pass = first;
+        ctl->last_pass = last;
+        ctl->nexec = nexec;
+    }
+}
+
+// ---- digit counts of every tile (large sorts) ---------------------------------------------------------------------
+// Same tiles as sort_pass_kernel, one per workgroup.  Lanes with the same digit find each other as in the pass
+// kernel, so skewed digits (exponent bytes, the high bytes of small integers) cost the same as uniform ones.
+template <typename T, int ITEMS>
+__global__ __launch_bounds__(SORT_BLOCK) void sort_upsweep_kernel(const T* __restrict__ orig, const typename SortKey<T>::U* buf_a,
+                                                                  const typename SortKey<T>::U* buf_b, uint32_t n, int pass, int rev,
+                                                                  const SortCtl* ctl, uint32_t* __restrict__ tile_count) {
+    typedef typename SortKey<T>::U U;
+    constexpr int TILE = SORT_BLOCK * ITEMS;
+    __shared__ uint32_t cnt[SORT_NW][256];
+    if (ctl->skip[pass]) return;
+    const bool first = (uint32_t)pass == ctl->first_pass;
+    const U* in = first ? (const U*)orig : (ctl->src_is_b[pass] != 0u ? buf_b : buf_a);
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    for (int i = tid; i < SORT_NW * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
+    __syncthreads();
+    const uint32_t tile = blockIdx.x;
+    const uint32_t woff = tile * (uint32_t)TILE + (uint32_t)wave * (WAVE * ITEMS) + lane;
+    U key[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const uint32_t e = woff + i * WAVE;
+        key[i] = (U)~(U)0;
+        if (e < n) key[i] = in[e];
+    }
+    if (first) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) key[i] = enc_bits<T>(key[i], rev, (U)~ctl->inv_min);   // padding keys are never counted
+    }
+    bool skewed = false;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const bool valid = woff + i * WAVE < n;
+        const uint32_t d = digit_of(key[i], pass);
+        if ((i & 3) == 0) skewed = digits_skewed(d, valid);                     // judged on every fourth round
+        count_digit(cnt[wave], d, valid, skewed);
+    }
+    __syncthreads();
+    uint32_t c = 0;
+#pragma unroll
+    for (int w = 0; w < SORT_NW; ++w) c += cnt[w][tid];
+    tile_count[(uint64_t)tile * 256 + tid] = c;
+}
+
+// ---- one pass ----------------------------------------------------------------------------------------------------
+// Tile = 256 threads x ITEMS keys.  Wave w owns the w-th quarter of the tile; its item i of lane l is key
+// i * 64 + l of that quarter (coalesced loads; the order (i, l) is memory order, which the ranking keeps).
+// desc[tile][digit]: low half = count, high half = (pass + 1) << 2 | status (1 = count of this tile only,
+// 2 = count of this and all earlier tiles); written and read with relaxed device-scope atomics, so the count
+// always travels with its tag.
+template <typename T, int ITEMS, bool PERM, bool COUNTED>
+__global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restrict__ orig, typename SortKey<T>::U* buf_a,
+                                                               typename SortKey<T>::U* buf_b, uint32_t* val_a, uint32_t* val_b,
+                                                               int64_t* __restrict__ perm_out, uint32_t n, int pass, int rev, SortCtl* ctl,
+                                                               uint64_t* desc, const uint32_t* __restrict__ tile_before, uint32_t ntiles) {
+    typedef typename SortKey<T>::U U;
+    constexpr int TILE = SORT_BLOCK * ITEMS;
+    __shared__ U lds_keys[TILE];
+    __shared__ uint32_t lds_vals[PERM ? TILE : 1];
+    __shared__ uint32_t cnt[SORT_NW][256];        // per wave and digit: count, then offset of the wave inside the digit
+    __shared__ uint32_t tile_start[256];          // first slot of the digit in the sorted tile
+    __shared__ uint32_t goff[256];                // global slot of the digit's first key of this tile, minus tile_start
+    __shared__ uint32_t wsum[SORT_NW];
+    __shared__ uint32_t lds_tile;
+
+    if (ctl->skip[pass]) return;
+    const bool first = (uint32_t)pass == ctl->first_pass, last = (uint32_t)pass == ctl->last_pass;
+    const U umin = (U)~ctl->inv_min;
+    const bool src_b = ctl->src_is_b[pass] != 0u;
+    const U* in = first ? (const U*)orig : (src_b ? buf_b : buf_a);
+    U* dst = src_b ? buf_a : buf_b;
+    const uint32_t* vsrc = src_b ? val_b : val_a;
+    uint32_t* vdst = src_b ? val_a : val_b;
+    const uint32_t tag_a = ((uint32_t)(pass + 1) << 2) | 1u, tag_p = ((uint32_t)(pass + 1) << 2) | 2u;
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+
+    for (uint32_t round = 0;; ++round) {
+        if (!COUNTED && tid == 0) lds_tile = atomicAdd(&ctl->ticket[pass], 1u);
+        for (int i = tid; i < SORT_NW * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
+        __syncthreads();
+        const uint32_t tile = COUNTED ? blockIdx.x + round * gridDim.x : lds_tile;
+        if (tile >= ntiles) return;
+        const uint32_t e0 = tile * (uint32_t)TILE;
+        const uint32_t woff = e0 + (uint32_t)wave * (WAVE * ITEMS) + lane;
+
+        // load (and map on the first pass)
+        U key[ITEMS];
+        uint32_t val[PERM ? ITEMS : 1];
+        uint32_t rank[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t e = woff + i * WAVE;
+            key[i] = (U)~(U)0;
+            if (e < n) key[i] = in[e];
+        }
+        if constexpr (PERM) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) val[i] = woff + i * WAVE;              // first pass: the key's own index
+            if (!first) {
+#pragma unroll
+                for (int i = 0; i < ITEMS; ++i)
+                    if (woff + i * WAVE < n) val[i] = vsrc[woff + i * WAVE];
+            }
+        }
+        if (first) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) key[i] = enc_bits<T>(key[i], rev, umin);    // padding keys are never counted
+        }
+        // rank inside the wave: lanes with the same digit find each other with 8 ballots; the lowest of them adds
+        // their number to the wave's counter of that digit.  The adds are LDS atomics that return the old value:
+        // LDS serves a wave's requests in order, so the 16 rounds queue up back to back with no wait in between
+        // (a plain read-modify-write needs a round trip per round).
+        uint32_t who[ITEMS];                     // leader lane | lanes below with the same digit << 8
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const bool valid = woff + i * WAVE < n;
+            const uint32_t d = digit_of(key[i], pass);
+            const uint64_t peers = match_digit(d, __ballot(valid));
+            const int leader = valid ? __ffsll((unsigned long long)peers) - 1 : 0;
+            const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
+            who[i] = (uint32_t)leader | (below << 8);
+            rank[i] = 0;
+            if (valid && lane == leader) rank[i] = atomicAdd(&cnt[wave][d], (uint32_t)__popcll(peers));
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) rank[i] = (uint32_t)__shfl((int)rank[i], (int)(who[i] & 0xffu)) + (who[i] >> 8);
+        __syncthreads();
+        // digit d = tid: count of the tile, offsets of the waves inside the digit
+        uint32_t count = 0;
+#pragma unroll
+        for (int w = 0; w < SORT_NW; ++w) {
+            const uint32_t c = cnt[w][tid];
+            cnt[w][tid] = count;
+            count += c;
+        }
+        // publish the count, then look back over the earlier tiles for this digit
+        uint64_t* my = desc + (uint64_t)tile * 256 + tid;
+        uint32_t excl = 0;
+        if constexpr (COUNTED) {
+            excl = tile_before[(uint64_t)tile * 256 + tid];
+        } else if (tile == 0) {
+            __hip_atomic_store(my, ((uint64_t)tag_p << 32) | count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            __hip_atomic_store(my, ((uint64_t)tag_a << 32) | count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // walk back over the earlier tiles, LB descriptors per round trip: sum counts until one that already
+            // includes its own predecessors; a descriptor that is not written yet is polled again
+            constexpr int LB = 8;
+            int64_t t = (int64_t)tile - 1;
+            bool done = false;
+            while (!done) {
+                uint64_t w[LB];
+#pragma unroll
+                for (int j = 0; j < LB; ++j) {
+                    w[j] = ((uint64_t)tag_p << 32);                       // in front of tile 0: nothing, and final
+                    if (t - j >= 0) w[j] = __hip_atomic_load(desc + (uint64_t)(t - j) * 256 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                int j = 0;
+#pragma unroll
+                for (; j < LB; ++j) {
+                    const uint32_t tg = (uint32_t)(w[j] >> 32);
+                    if (tg != tag_a && tg != tag_p) break;
+                    excl += (uint32_t)w[j];
+                    if (tg == tag_p) { done = true; break; }
+                }
+                t -= j;
+                if (!done && j == 0) __builtin_amdgcn_s_sleep(2);
+            }
+            __hip_atomic_store(my, ((uint64_t)tag_p << 32) | (uint64_t)(excl + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // first slot of every digit inside the sorted tile: exclusive scan of the counts over the 256 digits
+        const uint32_t inc = wave_scan_inclusive(count, OpAdd(), 0u);
+        if (lane == WAVE - 1) wsum[wave] = inc;
+        __syncthreads();
+        uint32_t start = inc - count;
+        for (int w = 0; w < wave; ++w) start += wsum[w];
+        tile_start[tid] = start;
+        goff[tid] = ctl->hist[pass][tid] + excl - start;
+        __syncthreads();
+        // reorder the tile in LDS
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            if (woff + i * WAVE < n) {
+                const uint32_t d = digit_of(key[i], pass);
+                const uint32_t pos = tile_start[d] + cnt[wave][d] + rank[i];
+                lds_keys[pos] = key[i];
+                if constexpr (PERM) lds_vals[pos] = val[i];
+            }
+        }
+        __syncthreads();
+        const uint32_t valid_n = n - e0 < (uint32_t)TILE ? n - e0 : (uint32_t)TILE;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t q = (uint32_t)tid + i * SORT_BLOCK;
+            if (q < valid_n) {
+                const U u = lds_keys[q];
+                const uint32_t slot = goff[digit_of(u, pass)] + q;
+                if constexpr (PERM) {
+                    if (last) perm_out[slot] = (int64_t)lds_vals[q] + 1;
+                    else { dst[slot] = u; vdst[slot] = lds_vals[q]; }
+                } else {
+                    if (last) ((T*)dst)[slot] = dec_bits<T>(u, rev, umin);
+                    else dst[slot] = u;
+                }
+            }
+        }
+        __syncthreads();      // LDS is reused by the next tile
+    }
+}
+
+// ---- finish ------------------------------------------------------------------------------------------------------
+// sort: after an odd number of passes the result sits in buffer B.  sortperm: no pass ran = identity permutation.
+template <typename W>
+__global__ __launch_bounds__(256) void sort_finish_kernel(const SortCtl* ctl, W* a, const W* b, int64_t nwords, int64_t* perm_out, int64_t n) {
+    const uint32_t nexec = ctl->nexec;
+    if (perm_out != nullptr) {
+        if (nexec != 0u) return;
+        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) perm_out[i] = i + 1;
+        return;
+    }
+    if ((nexec & 1u) == 0u) return;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * 256) a[i] = b[i];
+}
+
+// ---- host --------------------------------------------------------------------------------------------------------
+struct SortLayout {
+    size_t desc_off, clear_end, scratch_off, keys_b_off, keys_a_off, val_a_off, val_b_off, total;
+    uint32_t ntiles;
+    bool counted;          // large sort: desc_off holds the per-tile digit counts (uint32) instead of descriptors
+};
+
+template <typename T> constexpr int sort_items() { return sizeof(T) == 8 ? 8 : 16; }
+
+// More tiles than this: count first, no look-back (RK_SORT_LOOKBACK_TILES).
+static uint32_t sort_lookback_tiles() {
+    static const uint32_t v = [] { const char* e = std::getenv("RK_SORT_LOOKBACK_TILES"); const long x = e ? std::atol(e) : 0; return x > 0 ? (uint32_t)x : 1024u; }();
+    return v;
+}
+
+static SortLayout sort_layout(size_t key_size, int items, int64_t n, bool perm) {
+    SortLayout l{};
+    const int64_t tile = (int64_t)SORT_BLOCK * items;
+    l.ntiles = (uint32_t)((n + tile - 1) / tile);
+    size_t off = (sizeof(SortCtl) + 255) & ~(size_t)255;
+    l.counted = l.ntiles > sort_lookback_tiles();
+    l.desc_off = off;
+    if (l.counted) {
+        l.clear_end = off;                                   // only the control block needs clearing
+        off += (size_t)l.ntiles * 256 * sizeof(uint32_t);
+        l.scratch_off = off;
+        off += SORT_SCAN_SCRATCH;
+    } else {
+        off += (size_t)l.ntiles * 256 * sizeof(uint64_t);
+        l.clear_end = off;
+    }
+    const size_t kbytes = ((size_t)n * key_size + 255) & ~(size_t)255, vbytes = ((size_t)n * 4 + 255) & ~(size_t)255;
+    l.keys_b_off = off; off += kbytes;
+    if (perm) {
+        l.keys_a_off = off; off += kbytes;
+        l.val_a_off = off; off += vbytes;
+        l.val_b_off = off; off += vbytes;
+    }
+    l.total = off;
+    return l;
+}
+
+template <typename T>
+static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, void* tmp, size_t tmp_bytes, hipStream_t stream) {
+    typedef typename SortKey<T>::U U;
+    constexpr int ITEMS = sort_items<T>();
+    constexpr int PASSES = (int)sizeof(T);
+    const bool perm = perm_out != nullptr;
+    const SortLayout l = sort_layout(sizeof(T), ITEMS, n, perm);
+    if (tmp == nullptr || !is_aligned(tmp, 256) || tmp_bytes < l.total) return RK_ERR_WORKSPACE;
+    char* base = (char*)tmp;
+    SortCtl* ctl = (SortCtl*)base;
+    uint64_t* desc = (uint64_t*)(base + l.desc_off);
+    U* buf_b = (U*)(base + l.keys_b_off);
+    U* buf_a = perm ? (U*)(base + l.keys_a_off) : (U*)keys;
+    uint32_t* val_a = perm ? (uint32_t*)(base + l.val_a_off) : nullptr;
+    uint32_t* val_b = perm ? (uint32_t*)(base + l.val_b_off) : nullptr;
+    const int cus = device_info().cus;
+
+    const int64_t init_words = (int64_t)(l.clear_end / sizeof(uint64_t));
+    int64_t g = (init_words + 255) / 256;
+    if (g > cus * 16) g = cus * 16;
+    sort_init_kernel<<<(unsigned)g, 256, 0, stream>>>((uint64_t*)base, init_words);
+    RK_LAUNCH_CHECK();
+    g = (n + 256 * 16 - 1) / (256 * 16);
+    if (g > cus * 8) g = cus * 8;
+    constexpr int KVEC = 16 / (int)sizeof(T);
+    int64_t head = (int64_t)(((16 - ((uintptr_t)keys & 15)) & 15) / sizeof(T));
+    if (head > n) head = n;
+    const int64_t nvec = (n - head) / KVEC;
+    // few workgroups: each ends with device-wide atomics on shared words (1 for the minimum, 256 per digit position)
+    const unsigned gmin = (unsigned)(g < cus * 2 ? g : cus * 2), ghist = (unsigned)(g < cus * 4 ? g : cus * 4);
+    sort_min_kernel<T><<<gmin, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+    RK_LAUNCH_CHECK();
+    sort_hist_kernel<T, PASSES><<<ghist, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+    RK_LAUNCH_CHECK();
+    // sortperm: the first pass reads the caller's keys and should write buffer A, i.e. "reads B"
+    sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0);
+    RK_LAUNCH_CHECK();
+    unsigned pgrid = l.ntiles < (unsigned)(cus * 4) ? l.ntiles : (unsigned)(cus * 4);
+    uint32_t* tile_count = (uint32_t*)desc;
+    for (int p = 0; p < PASSES; ++p) {
+        if (l.counted) {
+            sort_upsweep_kernel<T, ITEMS><<<l.ntiles, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, (uint32_t)n, p, rev, ctl, tile_count);
+            RK_LAUNCH_CHECK();
+            // counts -> keys of the digit in earlier tiles: exclusive scan down the tiles, in place.  A skipped pass
+            // scans stale numbers that nobody reads (the host cannot know which passes are skipped).
+            const ScanGeom sg{256, (int64_t)l.ntiles, 1};
+            const int32_t st = scan_across_rows<uint32_t, uint32_t, OpAdd>(tile_count, tile_count, sg, 0u, 0, OpAdd(), true,
+                                                                          base + l.scratch_off, SORT_SCAN_SCRATCH, stream);
+            if (st != RK_SUCCESS) return st;
+            if (perm) sort_pass_kernel<T, ITEMS, true, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles);
+            else sort_pass_kernel<T, ITEMS, false, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles);
+        } else {
+            if (perm) sort_pass_kernel<T, ITEMS, true, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles);
+            else sort_pass_kernel<T, ITEMS, false, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles);
+        }
+        RK_LAUNCH_CHECK();
+    }
+    const int64_t nwords = ((int64_t)n * (int64_t)sizeof(T) + 3) / 4;
+    g = ((perm ? n : nwords) + 255) / 256;
+    if (g > cus * 16) g = cus * 16;
+    // whole 32-bit words: buffers are 256-byte padded, the caller's array is at least element-aligned; 16-bit keys
+    // with an odd count copy one element more than n only inside buffer padding on the source side -- so copy by element there
+    if (sizeof(T) == 2) sort_finish_kernel<uint16_t><<<(unsigned)g, 256, 0, stream>>>(ctl, (uint16_t*)keys, (const uint16_t*)buf_b, perm ? 0 : n, perm_out, n);
+    else sort_finish_kernel<uint32_t><<<(unsigned)g, 256, 0, stream>>>(ctl, (uint32_t*)keys, (const uint32_t*)buf_b, perm ? 0 : nwords, perm_out, n);
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+static bool sort_dtype_size(int dt, size_t* size) {
+    switch (dt) {
+        case RK_F32: case RK_I32: *size = 4; return true;
+        case RK_F64: case RK_I64: *size = 8; return true;
+        case RK_F16: case RK_I16: *size = 2; return true;
+        default: return false;
+    }
+}
+
+}  // namespace rk
+
+using namespace rk;
+
+extern "C" size_t rk_sort_tmp_bytes(rk_dtype dt, int64_t n, int32_t with_perm) {
+    size_t ks = 0;
+    if (!sort_dtype_size((int)dt, &ks) || n <= 0) return 256;
+    return sort_layout(ks, ks == 8 ? 8 : 16, n, with_perm != 0).total;
+}
+
+static int32_t sort_dispatch(rk_dtype dt, void* keys, int64_t* perm_out, int64_t n, int32_t rev, void* tmp, size_t tmp_bytes, void* stream) {
+    size_t ks = 0;
+    if (!sort_dtype_size((int)dt, &ks)) return ((int)dt >= RK_F32 && (int)dt <= RK_I16) ? RK_ERR_UNSUPPORTED : RK_ERR_INVALID_ARGUMENT;
+    if (n < 0) return RK_ERR_INVALID_ARGUMENT;
+    if (n == 0) return RK_SUCCESS;
+    if (keys == nullptr || !is_aligned(keys, ks)) return RK_ERR_INVALID_ARGUMENT;
+    if (n >= ((int64_t)1 << 31)) return RK_ERR_TOO_LARGE;
+    hipStream_t st = (hipStream_t)stream;
+    const int r = rev ? 1 : 0;
+    switch ((int)dt) {
+        case RK_F32: return sort_typed<float>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+        case RK_F64: return sort_typed<double>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+        case RK_I32: return sort_typed<int32_t>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+        case RK_I64: return sort_typed<int64_t>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+        case RK_F16: return sort_typed<half_bits>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+        default:     return sort_typed<int16_t>(keys, perm_out, n, r, tmp, tmp_bytes, st);
+    }
+}
+
+extern "C" int32_t rk_sort(rk_dtype dt, void* keys, int64_t n, int32_t rev, void* tmp, size_t tmp_bytes, void* stream) {
+    return sort_dispatch(dt, keys, nullptr, n, rev, tmp, tmp_bytes, stream);
+}
+
+extern "C" int32_t rk_sortperm(rk_dtype dt, const void* keys, int64_t* perm_out, int64_t n, int32_t rev, void* tmp, size_t tmp_bytes,
+                               void* stream) {
+    if (n > 0 && perm_out == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    return sort_dispatch(dt, (void*)keys, perm_out, n, rev, tmp, tmp_bytes, stream);
+}

@@ -352,6 +352,38 @@ function enable_permutedims!()
     end
 end
 
+# ---- sort! / sortperm! (src/kernels/sorting.jl:1-3): default order and rev natively, closures stay with AK -------------
+rk_dtype(::Type{Float16}) = Cint(7); rk_dtype(::Type{Int16}) = Cint(8)
+const SORTABLE = Union{Float16,Float32,Float64,Int16,Int32,Int64}
+
+function enable_sort!()
+    @eval function Base.sort!(x::ROCVector{T}; rev::Bool=false, lt=isless, by=identity, kwargs...) where {T<:SORTABLE}
+        (lt === isless && by === identity && isempty(kwargs)) || return (AMDGPU.AK.sort!(x; rev, lt, by, kwargs...); x)
+        n = length(x)
+        n > 1 || return x
+        tmp = ROCVector{UInt8}(undef, ccall((:rk_sort_tmp_bytes, librk[]), Csize_t, (Cint, Int64, Int32), rk_dtype(T), n, 0))
+        GC.@preserve x tmp begin
+            check(ccall((:rk_sort, librk[]), Int32, (Cint, Ptr{Cvoid}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                        rk_dtype(T), pointer(x), n, rev, pointer(tmp), sizeof(tmp), stream_ptr()))
+        end
+        AMDGPU.unsafe_free!(tmp)
+        return x
+    end
+    @eval function Base.sortperm!(ix::ROCVector{Int}, x::ROCVector{T}; rev::Bool=false, lt=isless, by=identity, kwargs...) where {T<:SORTABLE}
+        (lt === isless && by === identity && isempty(kwargs)) || return (AMDGPU.AK.sortperm!(ix, x; rev, lt, by, kwargs...); ix)
+        n = length(x)
+        length(ix) == n || throw(DimensionMismatch("sortperm!: index vector of length $(length(ix)) for $n keys"))
+        n > 0 || return ix
+        tmp = ROCVector{UInt8}(undef, ccall((:rk_sort_tmp_bytes, librk[]), Csize_t, (Cint, Int64, Int32), rk_dtype(T), n, 1))
+        GC.@preserve ix x tmp begin
+            check(ccall((:rk_sortperm, librk[]), Int32, (Cint, Ptr{Cvoid}, Ptr{Int64}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                        rk_dtype(T), pointer(x), pointer(ix), n, rev, pointer(tmp), sizeof(tmp), stream_ptr()))
+        end
+        AMDGPU.unsafe_free!(tmp)
+        return ix
+    end
+end
+
 """
     enable!()
 
@@ -360,7 +392,7 @@ Install the native methods.  Call once after `using AMDGPU`.
 function enable!()
     isfile(librk[]) || error("librk.so not found at $(librk[]); build it with `python amdgpu.jl_amd/build.py`")
     ccall((:rk_version, librk[]), Int32, ()) >= 100 || error("librk.so is too old")
-    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!(); enable_reverse!(); enable_permutedims!()
+    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!(); enable_reverse!(); enable_permutedims!(); enable_sort!()
     return nothing
 end
 

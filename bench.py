@@ -262,6 +262,17 @@ def main():
         run_cfg("reverse(A; dims=1) 8192^2 Float32", d * d, 8 * d * d, run_reverse)
         run_cfg("permutedims(A, (2,1)) 8192^2 Float32", d * d, 8 * d * d, run_permute)
         del ra, rb
+        # sort! (src/kernels/sorting.jl:1; perf/array.jl:143-149 sorts a Float32 vector): 8 B/key is the floor of
+        # any out-of-place permutation (one read, one write); the radix sort makes 4 digit passes plus 3 reads
+        m = 1 << 26
+        ssrc = randn_f32(m)
+        skeys = dev_array(ssrc.clone(), (m,), np.float32)
+        stmp = torch.empty(int(RL.lib.rk_sort_tmp_bytes(RL.RK_F32, m, 0)), dtype=torch.uint8, device=dev)
+        def run_sort(i):
+            skeys.buf.copy_(ssrc.view(torch.uint8))                      # unsorted input every time (the copy is timed too)
+            RL.check(RL.lib.rk_sort(RL.RK_F32, skeys.ptr, m, 0, stmp.data_ptr(), stmp.numel(), stream_ptr()), "rk_sort")
+        run_cfg("sort!(Float32[2^26]) incl. 85 us refill copy; GB/s at 8 B/key", m, 8 * m, run_sort)
+        del ssrc, skeys, stmp
         # cfg 4
         m = 512 ** 3
         x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))

@@ -66,7 +66,9 @@ typedef enum {
     RK_I64 = 3,  /* Int64   */
     RK_U8  = 4,  /* Bool / UInt8 (one byte per element) */
     RK_U32 = 5,  /* UInt32  */
-    RK_U64 = 6   /* UInt64  */
+    RK_U64 = 6,  /* UInt64  */
+    RK_F16 = 7,  /* Float16 (sort / sortperm only; reverse and permutedims take any 2-byte element) */
+    RK_I16 = 8   /* Int16   (sort / sortperm only) */
 } rk_dtype;
 
 /* f of mapreduce(f, op, A) */
@@ -232,6 +234,25 @@ RK_API int32_t rk_reverse(const void* x, void* y, size_t elsize, int ndim, const
  * bytes); src and dst are dense, column-major and must not overlap.  No workspace. */
 RK_API int32_t rk_permutedims(const void* src, void* dst, size_t elsize, int ndim,
                        const int64_t* shape, const int32_t* perm, void* stream);
+
+/* ---- sort! / sortperm! of vectors ------------------------------------------------------------
+ * Replace AK.sort! / AK.sortperm! behind  src/kernels/sorting.jl:1-3  for the default order
+ * (`lt = isless`, `by = identity`) and `rev`; custom `lt` / `by` closures cannot cross a C ABI
+ * (the caller keeps its own path for them).  Element types: Float16/32/64, Int16/32/64 (the types
+ * of test/hip_rocarray/sorting.jl).  Order = Base.isless: -0.0 before 0.0, NaN last (every NaN
+ * comes back as the canonical NaN).  Stable: sortperm keeps equal keys in index order, also with
+ * rev != 0, like Base.
+ *   rk_sort      sorts `keys` in place.
+ *   rk_sortperm  leaves `keys` untouched and writes the 1-based permutation (Int64) to
+ *                `perm_out`; unlike `sortperm!(ix, x)` it does not read an initial `ix`
+ *                (the reference always passes 1:n, src/kernels/sorting.jl:3).
+ * `tmp`: caller-owned, 256-byte aligned, at least rk_sort_tmp_bytes(dt, n, with_perm) bytes, any
+ * contents; it is the ping-pong buffer plus bookkeeping, cleared by the call itself.  n < 2^31. */
+RK_API size_t  rk_sort_tmp_bytes(rk_dtype dt, int64_t n, int32_t with_perm);
+RK_API int32_t rk_sort(rk_dtype dt, void* keys, int64_t n, int32_t rev, void* tmp, size_t tmp_bytes,
+                void* stream);
+RK_API int32_t rk_sortperm(rk_dtype dt, const void* keys, int64_t* perm_out, int64_t n, int32_t rev,
+                    void* tmp, size_t tmp_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -438,6 +438,33 @@ def reverse(x: np.ndarray, start=None, stop=None, dims=None) -> np.ndarray:
     return x[tuple(idx)].copy()
 
 
+def _isless_rank(x: np.ndarray) -> np.ndarray:
+    """Unsigned integers that order like ``Base.isless`` on ``x`` (floats: -0.0 < 0.0, every NaN equal and last)."""
+    x = np.asarray(x)
+    if x.dtype.kind == "f":
+        ut = {2: np.uint16, 4: np.uint32, 8: np.uint64}[x.dtype.itemsize]
+        b = np.where(np.isnan(x), np.array(np.nan, dtype=x.dtype), x).view(ut)     # one NaN pattern for all NaNs
+        sign = ut(1) << ut(8 * x.dtype.itemsize - 1)
+        return np.where(b & sign != 0, ~b, b | sign)
+    ut = np.dtype(f"u{x.dtype.itemsize}").type
+    return x.view(ut) ^ (ut(1) << ut(8 * x.dtype.itemsize - 1))
+
+
+def sortperm(x: np.ndarray, rev: bool = False) -> np.ndarray:
+    """``sortperm(x; rev)`` (src/kernels/sorting.jl:3, Base semantics): 1-based, stable -- equal keys stay in
+    index order, with ``rev=true`` too (Base reverses the ordering, not the result)."""
+    r = _isless_rank(x)
+    if rev:
+        r = ~r
+    return np.argsort(r, kind="stable").astype(np.int64) + 1
+
+
+def sort(x: np.ndarray, rev: bool = False) -> np.ndarray:
+    """``sort(x; rev)`` (src/kernels/sorting.jl:1): ``x[sortperm(x; rev)]``."""
+    x = np.asarray(x)
+    return x[sortperm(x, rev) - 1]
+
+
 def permutedims(x: np.ndarray, perm) -> np.ndarray:
     """``permutedims(x, perm)`` (Base; 1-based perm): ``size(out, k) == size(x, perm[k])`` and
     ``out[i_perm[1], ..., i_perm[N]] == x[i_1, ..., i_N]``."""

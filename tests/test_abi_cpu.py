@@ -160,6 +160,20 @@ def test_volumerhs_and_scatter_validation(L):
     assert pm(one, one, 4, 2, L.shape_array((5, 6)), i32(2, 1), None) == L.RK_ERR_INVALID_ARGUMENT     # in place is not defined
     assert pm(one, two, 5, 2, L.shape_array((5, 6)), i32(2, 1), None) == L.RK_ERR_UNSUPPORTED
     assert pm(None, None, 4, 2, L.shape_array((0, 6)), i32(2, 1), None) == L.RK_SUCCESS
+    so, sp, tb = L.lib.rk_sort, L.lib.rk_sortperm, L.lib.rk_sort_tmp_bytes
+    big = C.c_void_p(0x10000)
+    assert so(L.RK_F32, None, 10, 0, big, 1 << 30, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert so(L.RK_U8, one, 10, 0, big, 1 << 30, None) == L.RK_ERR_UNSUPPORTED
+    assert so(99, one, 10, 0, big, 1 << 30, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert so(L.RK_F32, one, -1, 0, big, 1 << 30, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert so(L.RK_F32, one, 10, 0, None, 0, None) == L.RK_ERR_WORKSPACE
+    assert so(L.RK_F32, one, 10, 0, big, 16, None) == L.RK_ERR_WORKSPACE
+    assert so(L.RK_F32, one, 1 << 31, 0, big, 1 << 40, None) == L.RK_ERR_TOO_LARGE
+    assert so(L.RK_F32, None, 0, 0, None, 0, None) == L.RK_SUCCESS
+    assert sp(L.RK_I64, one, None, 10, 0, big, 1 << 30, None) == L.RK_ERR_INVALID_ARGUMENT
+    n = 1 << 20
+    assert tb(L.RK_F32, n, 0) >= 4 * n and tb(L.RK_F32, n, 1) >= 16 * n and tb(L.RK_F32, n, 0) < 5 * n
+    assert tb(L.RK_I64, n, 0) >= 8 * n and tb(L.RK_I16, n, 0) >= 2 * n and tb(L.RK_U8, n, 0) == 256
     f = L.lib.rk_findall
     assert f(None, 1, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(one, 1, L.shape_array((5,)), None, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT

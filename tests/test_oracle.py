@@ -400,3 +400,47 @@ def test_permutedims_matches_definition(orc):
                     assert out[tuple(idx[p - 1] for p in perm)] == x[i, j, k]
     m = np.array([[1, 2, 3], [4, 5, 6]])
     assert orc.permutedims(m, (2, 1)).tolist() == [[1, 4], [2, 5], [3, 6]]       # Base docs: permutedims of a matrix
+
+
+def test_sort_matches_isless_insertion_sort(orc):
+    # Base.isless restated as a comparison, then a textbook stable insertion sort: pins order of signed zeros,
+    # NaNs, infinities and the stability of sortperm (also with rev=true)
+    import math
+
+    def isless(a, b):
+        if isinstance(a, float) or isinstance(b, float):
+            if math.isnan(a):
+                return False
+            if math.isnan(b):
+                return True
+            if a == b == 0.0:
+                return math.copysign(1.0, a) < math.copysign(1.0, b)
+        return a < b
+
+    def insertion_perm(v, rev):
+        lt = (lambda a, b: isless(b, a)) if rev else isless
+        p = []
+        for i, e in enumerate(v):
+            k = len(p)
+            while k > 0 and lt(e, v[p[k - 1]]):
+                k -= 1
+            p.insert(k, i)
+        return [i + 1 for i in p]
+
+    rng = np.random.default_rng(9)
+    specials = [0.0, -0.0, np.nan, np.inf, -np.inf, 1.5, -1.5, 0.0, -0.0, np.nan, 1.5]
+    for dtype in (np.float16, np.float32, np.float64):
+        v = np.array(specials + list(rng.integers(-3, 4, 20).astype(float)), dtype=dtype)
+        for rev in (False, True):
+            assert orc.sortperm(v, rev).tolist() == insertion_perm([float(e) for e in v], rev)
+            s = orc.sort(v, rev)
+            assert np.array_equal(s.view(f"u{v.itemsize}"), v[np.array(insertion_perm([float(e) for e in v], rev)) - 1].view(f"u{v.itemsize}"))
+    for dtype in (np.int16, np.int32, np.int64):
+        info = np.iinfo(dtype)
+        v = np.array([0, -1, info.min, info.max, 5, 5, -1, info.min] + list(rng.integers(-5, 6, 20)), dtype=dtype)
+        for rev in (False, True):
+            assert orc.sortperm(v, rev).tolist() == insertion_perm([int(e) for e in v], rev)
+    x = rng.standard_normal(1000).astype(np.float32)
+    assert np.array_equal(orc.sort(x), np.sort(x)) and np.array_equal(orc.sort(x, rev=True), np.sort(x)[::-1])
+    assert orc.sort(np.array([3, 1, 2])).tolist() == [1, 2, 3]
+    assert orc.sortperm(np.array([3, 1, 2])).tolist() == [2, 3, 1]                 # Base docs: sortperm([3, 1, 2])

@@ -1,0 +1,109 @@
+"""GPU parity of sort / sort! / sortperm / sortperm! (src/kernels/sorting.jl:1-3) against the oracle, through the
+C ABI: the sizes and element types of test/hip_rocarray/sorting.jl:5-28 for the default order and rev=true
+(values and permutations bit-exact, NaNs compared as equal), plus sizes that span many tiles, special floats,
+duplicates (stability) and small-range integers (skipped passes).  `lt` / `by` closures have no native form."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+TYPES = [np.float16, np.float32, np.float64, np.int16, np.int32, np.int64]
+
+
+def _rand(rng, dtype, n):
+    dt = np.dtype(dtype)
+    if dt.kind == "f":
+        return rng.random(n).astype(dt)                       # rand(T, sz)
+    return rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, n, dtype=dt, endpoint=True)
+
+
+def _check(rk, orc, x):
+    xd = rk.ROCArray(x)
+    for rev in (False, True):
+        want, wperm = orc.sort(x, rev), orc.sortperm(x, rev)
+        got = rk.Array(rk.sort(xd, rev=rev))
+        assert got.dtype == x.dtype and np.array_equal(got, want, equal_nan=x.dtype.kind == "f"), rev
+        if x.dtype.kind == "f":
+            assert np.array_equal(np.signbit(got[~np.isnan(got)]), np.signbit(want[~np.isnan(want)]))
+        p = rk.Array(rk.sortperm(xd, rev=rev))
+        assert p.dtype == np.int64 and np.array_equal(p, wperm), rev
+    assert np.array_equal(rk.Array(xd), x, equal_nan=x.dtype.kind == "f")          # sort / sortperm leave x alone
+    assert rk.sort_(xd) is xd
+    assert np.array_equal(rk.Array(xd), orc.sort(x), equal_nan=x.dtype.kind == "f")
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("sz", [1, 2, 3, 4, 33, 333, 3333, 4096])
+def test_reference_sizes_and_types(rk, orc, dtype, sz):
+    _check(rk, orc, _rand(np.random.default_rng(sz), dtype, sz))
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("n", [4097, 65_537, 1_000_003])
+def test_many_tiles(rk, orc, dtype, n):
+    _check(rk, orc, _rand(np.random.default_rng(n), dtype, n))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32, np.float64])
+def test_special_floats_and_stability(rk, orc, dtype):
+    rng = np.random.default_rng(5)
+    base = np.array([0.0, -0.0, np.nan, np.inf, -np.inf, 1.0, -1.0, 65504.0, -65504.0, 6e-8, -6e-8], dtype=dtype)
+    x = rng.choice(base, 50_000)
+    x[::7] = -x[::7]
+    _check(rk, orc, x)
+
+
+@pytest.mark.parametrize("dtype", [np.int16, np.int32, np.int64])
+def test_small_range_integers_skip_passes(rk, orc, dtype):
+    rng = np.random.default_rng(6)
+    _check(rk, orc, rng.integers(-10, 11, 300_000).astype(dtype))                  # perf/array.jl:16 rand(-10:10, ...)
+    _check(rk, orc, np.full(10_000, 7, dtype=dtype))                               # every pass skipped
+    _check(rk, orc, (rng.integers(0, 2, 100_000) * 256).astype(dtype))             # only the second digit varies
+    _check(rk, orc, np.arange(100_000, 0, -1).astype(dtype) if dtype != np.int16 else np.arange(30_000, 0, -1).astype(dtype))
+
+
+def test_perf_suite_size_and_in_place_outputs(rk, orc):
+    x = np.random.default_rng(7).random(512 * 1000).astype(np.float32)             # sort(gpu_vec), perf/array.jl:145
+    _check(rk, orc, x)
+    ix = rk.ROCArray(dims=(x.size,), dtype=np.int64)
+    assert rk.sortperm_(ix, rk.ROCArray(x)) is ix
+    assert np.array_equal(x[rk.Array(ix) - 1], np.sort(x))                         # y == xd[sortperm(xd)], sorting.jl:14
+
+
+def test_full_size_sort(rk, orc):
+    x = np.random.default_rng(8).standard_normal(1 << 24).astype(np.float32)
+    got = rk.Array(rk.sort(rk.ROCArray(x)))
+    assert np.array_equal(got, np.sort(x))
+    k = np.random.default_rng(9).integers(-2**62, 2**62, 1 << 22, dtype=np.int64)
+    p = rk.Array(rk.sortperm(rk.ROCArray(k), rev=True))
+    assert np.array_equal(p, orc.sortperm(k, True))
+
+
+@pytest.mark.parametrize("dtype", [np.int16, np.float32, np.float64])
+def test_unaligned_views(rk, orc, dtype):
+    # keys that start 1 .. 9 elements into a buffer: the vector body of the whole-array reads starts later
+    x = _rand(np.random.default_rng(10), dtype, 70_010)
+    d = rk.ROCArray(x)
+    for first in (2, 3, 4, 6, 10):
+        v = d.view_range(first, 70_005)
+        want = orc.sort(x[first - 1:70_005])
+        assert np.array_equal(rk.Array(rk.sort(v)), want)
+        assert np.array_equal(rk.Array(rk.sortperm(v)), orc.sortperm(x[first - 1:70_005]))
+    v = d.view_range(3, 70_001)
+    rk.sort_(v, rev=True)
+    got = rk.Array(d)
+    assert np.array_equal(got[2:70_001], orc.sort(x[2:70_001], rev=True))
+    assert np.array_equal(got[:2], x[:2]) and np.array_equal(got[70_001:], x[70_001:])      # neighbours untouched
+
+
+def test_unsupported_forms(rk):
+    xd = rk.ROCArray(np.arange(10, dtype=np.float32))
+    with pytest.raises(rk.UnsupportedError):
+        rk.sort(xd, lt=lambda a, b: a > b)
+    with pytest.raises(rk.UnsupportedError):
+        rk.sortperm(xd, by=lambda k: 2 * k)
+    with pytest.raises(rk.UnsupportedError):
+        rk.sort(rk.ROCArray(np.zeros((3, 4), dtype=np.float32)))
+    with pytest.raises(rk.UnsupportedError):
+        rk.sort(rk.ROCArray(np.zeros(5, dtype=np.uint8)))
+    assert len(rk.sort(rk.ROCArray(np.zeros(0, dtype=np.float32)))) == 0
