@@ -164,6 +164,7 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
             case RK_F64: return mapreduce_f64(a);
             case RK_I32: return mapreduce_i32(a);
             case RK_I64: return mapreduce_i64(a);
+            case RK_U8:  return mapreduce_u8(a);
             default: return RK_ERR_UNSUPPORTED;
         }
     }
@@ -186,6 +187,7 @@ int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, co
         case RK_F64: return findminmax_f64(a);
         case RK_I32: return findminmax_i32(a);
         case RK_I64: return findminmax_i64(a);
+        case RK_U8:  return findminmax_u8(a);
         default: return RK_ERR_UNSUPPORTED;
     }
 }

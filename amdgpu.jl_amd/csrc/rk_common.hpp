@@ -237,8 +237,12 @@ __device__ __forceinline__ int lane_id() { return (int)__lane_id(); }
 // workgroups it costs more than the streaming kernel it sits in.  The writer orders
 // "value, then flag/ticket" with publish_barrier() (waits until its own stores have completed).
 template <typename T> __device__ __forceinline__ void store_agent(T* p, const T& v) {
-    static_assert(sizeof(T) % 4 == 0, "whole words only");
-    if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
+    static_assert(sizeof(T) % 4 == 0 || sizeof(T) == 1 || sizeof(T) == 2, "whole words, or one scalar of 1 or 2 bytes");
+    if constexpr (sizeof(T) == 1) {
+        __hip_atomic_store((uint8_t*)p, __builtin_bit_cast(uint8_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (sizeof(T) == 2) {
+        __hip_atomic_store((uint16_t*)p, __builtin_bit_cast(uint16_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
         uint64_t w[sizeof(T) / 8];
         __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
@@ -253,9 +257,13 @@ template <typename T> __device__ __forceinline__ void store_agent(T* p, const T&
     }
 }
 template <typename T> __device__ __forceinline__ T load_agent(const T* p) {
-    static_assert(sizeof(T) % 4 == 0, "whole words only");
+    static_assert(sizeof(T) % 4 == 0 || sizeof(T) == 1 || sizeof(T) == 2, "whole words, or one scalar of 1 or 2 bytes");
     T v;
-    if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
+    if constexpr (sizeof(T) == 1) {
+        return __builtin_bit_cast(T, __hip_atomic_load((const uint8_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    } else if constexpr (sizeof(T) == 2) {
+        return __builtin_bit_cast(T, __hip_atomic_load((const uint16_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    } else if constexpr (sizeof(T) % 8 == 0 && alignof(T) >= 8) {
         uint64_t w[sizeof(T) / 8];
 #pragma unroll
         for (unsigned i = 0; i < sizeof(T) / 8; ++i)
@@ -399,6 +407,13 @@ template <> struct OrderKey<int64_t> {
     static constexpr bool LOWEST_FREE = false;
     static __device__ __forceinline__ Key make(int64_t v, bool want_max) { return want_max ? v : ~v; }
     static __device__ __forceinline__ int64_t value(Key k, bool want_max) { return want_max ? k : ~k; }
+};
+
+template <> struct OrderKey<uint8_t> {            // Bool / UInt8: findfirst(bools) is findmax's index
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
+    static __device__ __forceinline__ Key make(uint8_t v, bool want_max) { return want_max ? (Key)v : ~(Key)v; }
+    static __device__ __forceinline__ uint8_t value(Key k, bool want_max) { return (uint8_t)(want_max ? k : ~k); }
 };
 
 // `i` is the position of the element along its line (0-based), 32-bit whenever the line is shorter than

@@ -19,7 +19,10 @@ int32_t findminmax_i64(const FindArgs& a) { return findminmax_typed<int64_t>(a);
 int32_t mapreduce_i32_i64(const MapreduceArgs& a) { return mapreduce_typed<int32_t, int64_t>(a); }
 #elif RK_INST == 5
 int32_t mapreduce_u8_i64(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, int64_t>(a); }
+#elif RK_INST == 6
+int32_t mapreduce_u8(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, uint8_t>(a); }      // any / all of Bool arrays
+int32_t findminmax_u8(const FindArgs& a) { return findminmax_typed<uint8_t>(a); }                   // findfirst of Bool arrays
 #else
-#error "RK_INST must be 0..5"
+#error "RK_INST must be 0..6"
 #endif
 }  // namespace rk

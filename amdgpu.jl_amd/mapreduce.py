@@ -162,6 +162,37 @@ def count(A: ROCArray, dims=None):
     return mapreduce(identity, add_sum, A, dims=dims)
 
 
+def any(A: ROCArray, dims=None):                             # noqa: A001 - mirrors Base.any
+    """``any(::ROCArray{Bool}; dims)``: ``|`` over Bools is ``max`` over their bytes."""
+    if A.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "any needs a Bool array (predicates are closures)")
+    if len(A) == 0:
+        return False if dims is None else ROCArray(np.zeros(_reduced_dims(A.dims, _dims_mask(dims, A.ndim)), dtype=np.bool_))
+    r = mapreduce(identity, max_, A, dims=dims)
+    return bool(r) if dims is None else r
+
+
+def all(A: ROCArray, dims=None):                             # noqa: A001 - mirrors Base.all
+    """``all(::ROCArray{Bool}; dims)``: ``&`` over Bools is ``min`` over their bytes."""
+    if A.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "all needs a Bool array (predicates are closures)")
+    if len(A) == 0:
+        return True if dims is None else ROCArray(np.ones(_reduced_dims(A.dims, _dims_mask(dims, A.ndim)), dtype=np.bool_))
+    r = mapreduce(identity, min_, A, dims=dims)
+    return bool(r) if dims is None else r
+
+
+def findfirst(A: ROCArray):
+    """``findfirst(::ROCArray{Bool})``: index of the first true entry in column-major order (an Int for
+    vectors, a CartesianIndex tuple otherwise) or ``None``: the argmax of the bytes, ties to the smallest index."""
+    if A.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findfirst needs a Bool array (predicates are closures)")
+    if len(A) == 0:
+        return None
+    v, i = _findminmax(A, True, None)
+    return i if v else None
+
+
 def _findminmax(A: ROCArray, want_max: bool, dims):
     if len(A) == 0:
         raise ValueError("reducing over an empty collection is not allowed")

@@ -225,3 +225,29 @@ def test_repeated_calls_reuse_clean_workspace(rk, orc):
     r0 = rk.Array(rk.sum(dA, dims=2))
     for _ in range(3):
         assert np.array_equal(rk.Array(rk.sum(dA, dims=2)), r0)
+
+
+@pytest.mark.parametrize("shape", [(1,), (1000,), (1 << 20,), (300, 70), (70, 300), (17, 5, 33)])
+def test_any_all_findfirst_bool(rk, orc, shape):
+    # Bool reductions run on the bytes: any = max, all = min, findfirst = argmax with ties to the smallest index
+    rng = _rng(40)
+    for p in (0.0, 1e-4, 0.5, 1.0):
+        b = rng.random(shape) < p
+        d = rk.ROCArray(b)
+        assert rk.any(d) == bool(b.any()) and rk.all(d) == bool(b.all())
+        flat = b.reshape(-1, order="F")
+        want = None if not flat.any() else int(np.argmax(flat)) + 1
+        got = rk.findfirst(d)
+        if want is None or b.ndim == 1:
+            assert got == want
+        else:
+            assert tuple(got) == tuple(int(i) + 1 for i in np.unravel_index(want - 1, b.shape, order="F"))
+        for dims in range(1, b.ndim + 1):
+            ra, rl = rk.any(d, dims=dims), rk.all(d, dims=dims)
+            assert ra.dtype == np.bool_ and rl.dtype == np.bool_
+            assert np.array_equal(rk.Array(ra), b.any(axis=dims - 1, keepdims=True))
+            assert np.array_equal(rk.Array(rl), b.all(axis=dims - 1, keepdims=True))
+    one = np.zeros(shape, dtype=bool)
+    one[(-1,) * one.ndim] = True                                  # the last element in column-major order too
+    got = rk.findfirst(rk.ROCArray(one))
+    assert (got if one.ndim == 1 else int(np.ravel_multi_index(tuple(i - 1 for i in got), one.shape, order="F")) + 1) == one.size
