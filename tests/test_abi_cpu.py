@@ -85,7 +85,7 @@ def test_findminmax_and_accumulate_validation(L):
     g = L.lib.rk_findminmax
     assert g(1, L.RK_F32, None, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert g(1, L.RK_F32, one, 2, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # no output requested
-    assert g(1, L.RK_U8, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert g(1, L.RK_U32, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
     assert g(1, L.RK_F32, None, 2, L.shape_array((0, 4)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     a = L.lib.rk_accumulate
     assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
