@@ -73,3 +73,55 @@ def test_graph_replays_match_oracle(rk, orc):
         assert np.array_equal(rk.Array(r_row)[:, 0], h2.astype(np.int64).sum(axis=1)), replay
         # eager work through the default stream's workspace between the replays
         assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(hi[:300_000]))), np.cumsum(hi[:300_000], dtype=np.int32))
+
+
+def test_graph_replays_of_findall_reverse_permutedims_sort(rk, orc):
+    import ctypes as C
+    from amdgpu_jl_amd import _lib as L
+    from amdgpu_jl_amd.array import workspace, stream_ptr
+
+    n, shape2 = 300_007, (130, 257)
+    rng = np.random.default_rng(43)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        mask = rk.ROCArray(dims=(n,), dtype=np.bool_)
+        ys = rk.ROCArray(dims=(n,), dtype=np.int64)                # room for every element
+        cnt = rk.ROCArray(dims=(1,), dtype=np.int64)
+        keys = rk.ROCArray(dims=(n,), dtype=np.float32)
+        perm = rk.ROCArray(dims=(n,), dtype=np.int64)
+        m2 = rk.ROCArray(dims=shape2, dtype=np.int32)
+        rev = rk.ROCArray(dims=shape2, dtype=np.int32)
+        tr = rk.ROCArray(dims=shape2[::-1], dtype=np.int32)
+        shp1, shp2 = L.shape_array((n,)), L.shape_array(shape2)
+        p21 = (C.c_int32 * 2)(2, 1)
+        ws, wsb = workspace(L.lib.rk_workspace_bytes(L.RK_KIND_FINDALL, L.RK_U8, 1, shp1, 0))
+        tmp = torch.empty(int(L.lib.rk_sort_tmp_bytes(L.RK_F32, n, 1)), dtype=torch.uint8, device="cuda")
+
+        def calls():
+            s = stream_ptr()
+            L.check(L.lib.rk_findall(mask.ptr, 1, shp1, ys.ptr, cnt.ptr, ws, wsb, s), "rk_findall")
+            L.check(L.lib.rk_sortperm(L.RK_F32, keys.ptr, perm.ptr, n, 0, tmp.data_ptr(), tmp.numel(), s), "rk_sortperm")
+            L.check(L.lib.rk_sort(L.RK_F32, keys.ptr, n, 1, tmp.data_ptr(), tmp.numel(), s), "rk_sort")
+            L.check(L.lib.rk_reverse(m2.ptr, rev.ptr, 4, 2, shp2, 1, s), "rk_reverse")
+            L.check(L.lib.rk_permutedims(m2.ptr, tr.ptr, 4, 2, shp2, p21, s), "rk_permutedims")
+        mask.buf.zero_(); keys.buf.zero_(); m2.buf.zero_()
+        calls()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        calls()
+    for replay in range(3):
+        hm = rng.random(n) < 0.3
+        hk = rng.standard_normal(n).astype(np.float32)
+        h2 = rng.integers(-10**6, 10**6, shape2, dtype=np.int32)
+        _upload(mask, hm); _upload(keys, hk); _upload(m2, h2)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        c = int(rk.Array(cnt)[0])
+        assert c == int(hm.sum()), replay
+        assert np.array_equal(rk.Array(ys)[:c], np.nonzero(hm)[0] + 1), replay
+        assert np.array_equal(rk.Array(perm), orc.sortperm(hk)), replay
+        assert np.array_equal(rk.Array(keys), orc.sort(hk, rev=True)), replay
+        assert np.array_equal(rk.Array(rev), h2[::-1, :]), replay
+        assert np.array_equal(rk.Array(tr), h2.T), replay
