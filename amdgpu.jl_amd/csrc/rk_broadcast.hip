@@ -128,85 +128,83 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
     }
 }
 
-// ---- scalar math in the compute type ---------------------------------------------------------------
-template <typename CT> __device__ __forceinline__ CT bc_unary(int tok, CT a) {
-    switch (tok) {
-        case RK_BC_NEG: return -a;
-        case RK_BC_ABS: return a < CT(0) ? -a : (a == CT(0) ? CT(0) : a);
-        case RK_BC_ABS2: return a * a;
-        case RK_BC_SQRT: return sqrt(a);
-        case RK_BC_EXP: return exp(a);
-        case RK_BC_LOG: return log(a);
-        case RK_BC_SIN: return sin(a);
-        case RK_BC_COS: return cos(a);
-        case RK_BC_TANH: return tanh(a);
-        case RK_BC_INV: return CT(1) / a;
-        default: return a;   // RK_BC_IDENTITY
-    }
-}
-template <typename CT> __device__ __forceinline__ CT bc_binary(int tok, CT a, CT b) {
-    switch (tok) {
-        case RK_BC_ADD: return a + b;
-        case RK_BC_SUB: return a - b;
-        case RK_BC_MUL: return a * b;
-        case RK_BC_DIV: return a / b;
-        case RK_BC_MAX: return OpMax()(a, b);
-        case RK_BC_MIN: return OpMin()(a, b);
-        default: return pow(a, b);   // RK_BC_POW
-    }
-}
-
 // ---- evaluators ---------------------------------------------------------------------------------------
-// Postfix interpreter.  Stack slot s of thread t, component j lives at lds[(s * VEC + j) * BLOCK + t]
-// (conflict-free); the top of the stack stays in registers.
+// Postfix interpreter.  The program is the same for every lane, so every token is one scalar branch (a switch
+// outside the per-component loops: inside them the compiler turns it into selects that evaluate exp, log, sin ...
+// for every element).  The four topmost stack entries live in registers and move by one place on push / pop;
+// deeper entries (rare) spill to LDS: entry e of thread t, component j at lds[(e * VEC + j) * BLOCK + t].
+constexpr int BC_REG_DEPTH = 4;
 struct EvalInterp {
     static constexpr int NOPS = RK_MAX_OPERANDS;   // load what the program declares
     static constexpr bool USES_LDS = true;
     template <typename CT, int VEC>
     static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
         const int t = threadIdx.x;
-        CT top[VEC];
+        CT s0[VEC], s1[VEC], s2[VEC], s3[VEC];     // s0 = top of the stack
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) top[j] = CT(0);
-        int depth = 0;   // values on the stack, including `top`
+        for (int j = 0; j < VEC; ++j) s0[j] = s1[j] = s2[j] = s3[j] = CT(0);
+        int depth = 0;
+        auto push = [&](const CT (&v)[VEC]) {
+            if (depth >= BC_REG_DEPTH) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) lds[((depth - BC_REG_DEPTH) * VEC + j) * BC_BLOCK + t] = s3[j];
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { s3[j] = s2[j]; s2[j] = s1[j]; s1[j] = s0[j]; s0[j] = v[j]; }
+            ++depth;
+        };
+        auto drop_second = [&]() {                 // the entry under the top has been consumed
+            --depth;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { s1[j] = s2[j]; s2[j] = s3[j]; }
+            if (depth >= BC_REG_DEPTH) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) s3[j] = lds[((depth - BC_REG_DEPTH) * VEC + j) * BC_BLOCK + t];
+            }
+        };
+#define RK_BC_UN(EXPR)  { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = s0[j]; s0[j] = (EXPR); } } break
+#define RK_BC_BIN(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = s1[j], y = s0[j]; s0[j] = (EXPR); } drop_second(); } break
         for (int i = 0; i < a.n_tokens; ++i) {
             const int tok = a.tokens[i];
-            if (tok < RK_MAX_OPERANDS) {
-                if (depth > 0) {
+            switch (tok) {
+                case 0: push(in[0]); break;
+                case 1: push(in[1]); break;
+                case 2: push(in[2]); break;
+                case 3: push(in[3]); break;
+                case 4: push(in[4]); break;
+                case 5: push(in[5]); break;
+                case 6: push(in[6]); break;
+                case 7: push(in[7]); break;
+                case RK_BC_ADD: RK_BC_BIN(x + y);
+                case RK_BC_SUB: RK_BC_BIN(x - y);
+                case RK_BC_MUL: RK_BC_BIN(x * y);
+                case RK_BC_DIV: RK_BC_BIN(x / y);
+                case RK_BC_MAX: RK_BC_BIN(OpMax()(x, y));
+                case RK_BC_MIN: RK_BC_BIN(OpMin()(x, y));
+                case RK_BC_POW: RK_BC_BIN(pow(x, y));
+                case RK_BC_FMA: {                   // x * y + top with x the deepest of the three
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) lds[((depth - 1) * VEC + j) * BC_BLOCK + t] = top[j];
-                }
-                ++depth;
-                // static register indices: select the operand with a uniform branch
-#pragma unroll
-                for (int k = 0; k < RK_MAX_OPERANDS; ++k)
-                    if (tok == k) {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) top[j] = in[k][j];
-                    }
-            } else if (tok >= RK_BC_NEG) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) top[j] = bc_unary<CT>(tok, top[j]);
-            } else if (tok == RK_BC_FMA) {
-                CT x[VEC], y[VEC];
-                depth -= 2;
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    y[j] = lds[((depth) * VEC + j) * BC_BLOCK + t];
-                    x[j] = lds[((depth - 1) * VEC + j) * BC_BLOCK + t];
-                    top[j] = x[j] * y[j] + top[j];
-                }
-            } else {
-                --depth;
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) {
-                    const CT x = lds[((depth - 1) * VEC + j) * BC_BLOCK + t];
-                    top[j] = bc_binary<CT>(tok, x, top[j]);
-                }
+                    for (int j = 0; j < VEC; ++j) s0[j] = s2[j] * s1[j] + s0[j];
+                    drop_second();
+                    drop_second();
+                } break;
+                case RK_BC_NEG: RK_BC_UN(-x);
+                case RK_BC_ABS: RK_BC_UN(x < CT(0) ? -x : (x == CT(0) ? CT(0) : x));
+                case RK_BC_ABS2: RK_BC_UN(x * x);
+                case RK_BC_SQRT: RK_BC_UN(sqrt(x));
+                case RK_BC_EXP: RK_BC_UN(exp(x));
+                case RK_BC_LOG: RK_BC_UN(log(x));
+                case RK_BC_SIN: RK_BC_UN(sin(x));
+                case RK_BC_COS: RK_BC_UN(cos(x));
+                case RK_BC_TANH: RK_BC_UN(tanh(x));
+                case RK_BC_INV: RK_BC_UN(CT(1) / x);
+                default: break;                     // RK_BC_IDENTITY
             }
         }
+#undef RK_BC_UN
+#undef RK_BC_BIN
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) out[j] = top[j];
+        for (int j = 0; j < VEC; ++j) out[j] = s0[j];
     }
 };
 
@@ -246,9 +244,19 @@ struct EvalBinary {
     static constexpr bool USES_LDS = false;
     template <typename CT, int VEC>
     static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
-        const int tok = a.tokens[2];
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) out[j] = bc_binary<CT>(tok, in[0][j], in[1][j]);
+        // one scalar branch on the operator, then the component loop (the other way round every element
+        // would evaluate pow)
+#define RK_BC_BIN2(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = in[0][j], y = in[1][j]; out[j] = (EXPR); } } break
+        switch (a.tokens[2]) {
+            case RK_BC_ADD: RK_BC_BIN2(x + y);
+            case RK_BC_SUB: RK_BC_BIN2(x - y);
+            case RK_BC_MUL: RK_BC_BIN2(x * y);
+            case RK_BC_DIV: RK_BC_BIN2(x / y);
+            case RK_BC_MAX: RK_BC_BIN2(OpMax()(x, y));
+            case RK_BC_MIN: RK_BC_BIN2(OpMin()(x, y));
+            default:        RK_BC_BIN2(pow(x, y));      // RK_BC_POW
+        }
+#undef RK_BC_BIN2
     }
 };
 
@@ -277,7 +285,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
         const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
-        constexpr int NB = Eval::USES_LDS ? 1 : (Eval::NOPS >= 3 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
+        constexpr int NB = Eval::USES_LDS ? 1 : (Eval::NOPS >= 4 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
 #pragma unroll
@@ -342,7 +350,7 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
         if (a.nxb > 0x7fffffff || gz > 65535) return RK_ERR_TOO_LARGE;
         grid = dim3((unsigned)a.nxb, (unsigned)gy, (unsigned)gz);
     }
-    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - 1) * VECN * BC_BLOCK * sizeof(CT) : 0;
+    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - BC_REG_DEPTH) * VECN * BC_BLOCK * sizeof(CT) : 0;
     // homogeneous element types: a kernel without any dispatch on the element type
     bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : RK_F64);
     for (int k = 0; k < a.n_operands; ++k)
