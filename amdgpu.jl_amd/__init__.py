@@ -14,7 +14,7 @@ from .accumulate import accumulate, accumulate_, cumsum, cumprod, accumulate_elt
 from . import broadcast                                                               # noqa: F401
 from .broadcast import lazy, materialize, materialize_, fill_, Broadcasted             # noqa: F401
 from .volumerhs import volumerhs_                                                     # noqa: F401
-from .indexing import findall                                                         # noqa: F401
+from .indexing import findall, getindex_mask                                                         # noqa: F401
 from .reverse import reverse, reverse_                                                # noqa: F401
 from .permutedims import permutedims, permutedims_                                    # noqa: F401
 from .sorting import sort, sort_, sortperm, sortperm_                                 # noqa: F401

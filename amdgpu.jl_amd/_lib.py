@@ -83,6 +83,7 @@ PROTOTYPES = {
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
                                      C.c_void_p]),
     "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),
+    "rk_gather_slices": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "rk_sort_tmp_bytes": (C.c_size_t, [C.c_int, C.c_int64, C.c_int32]),
     "rk_sort": (C.c_int32, [C.c_int, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_sortperm": (C.c_int32, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_size_t, C.c_void_p]),

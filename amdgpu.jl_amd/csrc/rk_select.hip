@@ -229,3 +229,50 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }
+
+// ---- x[.., indices]: the gather behind logical indexing ------------------------------------------------------------
+// y[i, j] = x[i, idx[j] - 1] for i < inner: `x[mask]`, `x[:, mask]`, `x[:, :, mask]` (test/hip_rocarray/indexing.jl:5-18)
+// after Base.to_index has turned the mask into findall(mask) (src/kernels/indexing.jl:1).  Elements are opaque.
+namespace rk {
+
+template <typename E> struct GatherElem { typedef E type; };
+struct Bytes16 { uint64_t lo, hi; };
+
+template <typename E>
+__global__ __launch_bounds__(256) void gather_slices_kernel(const E* __restrict__ x, const int64_t* __restrict__ idx, E* __restrict__ y,
+                                                            int64_t inner, int64_t total, int64_t nsrc) {
+    const int64_t f = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (f >= total) return;
+    int64_t i = 0, j = f;
+    if (inner != 1) { j = f / inner; i = f - j * inner; }
+    const int64_t s = idx[j] - 1;
+    if (s < 0 || s >= nsrc) return;          // an index outside x selects nothing (the caller checks bounds)
+    y[f] = x[s * inner + i];
+}
+
+}  // namespace rk
+
+extern "C" int32_t rk_gather_slices(const void* x, const int64_t* idx, void* y, size_t elsize, int64_t inner, int64_t nidx, int64_t nsrc,
+                                    void* stream) {
+    if (inner < 0 || nidx < 0 || nsrc < 0) return RK_ERR_INVALID_ARGUMENT;
+    if (elsize != 1 && elsize != 2 && elsize != 4 && elsize != 8 && elsize != 16) return RK_ERR_UNSUPPORTED;
+    if (inner == 0 || nidx == 0) return RK_SUCCESS;
+    if (x == nullptr || idx == nullptr || y == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    const size_t align = elsize < 16 ? elsize : 8;
+    if (!is_aligned(x, align) || !is_aligned(y, align)) return RK_ERR_INVALID_ARGUMENT;
+    if (nidx > INT64_MAX / inner) return RK_ERR_TOO_LARGE;
+    const int64_t total = inner * nidx, blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+    hipStream_t st = (hipStream_t)stream;
+#define RK_GATHER(E) rk::gather_slices_kernel<E><<<(unsigned)blocks, 256, 0, st>>>((const E*)x, idx, (E*)y, inner, total, nsrc)
+    switch (elsize) {
+        case 1: RK_GATHER(uint8_t); break;
+        case 2: RK_GATHER(uint16_t); break;
+        case 4: RK_GATHER(uint32_t); break;
+        case 8: RK_GATHER(uint64_t); break;
+        default: RK_GATHER(rk::Bytes16); break;
+    }
+#undef RK_GATHER
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}

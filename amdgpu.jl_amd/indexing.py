@@ -49,3 +49,25 @@ def findall_two_pass(bools: ROCArray) -> ROCArray:
         st = L.lib.rk_findall_scatter(bools.ptr, indices.ptr, ys.ptr, nd, L.shape_array(bools.dims), stream_ptr())
         L.check(st, "rk_findall_scatter")
     return ys
+
+
+def getindex_mask(x: ROCArray, mask: ROCArray) -> ROCArray:
+    """``x[mask]`` for a mask of x's shape, or ``x[:, ..., :, mask]`` for a Bool vector along the last dim
+    (test/hip_rocarray/indexing.jl:5-18): ``Base.to_index`` turns the mask into ``findall(mask)``
+    (indexing.jl:1), then the selected slices are gathered."""
+    if mask.dtype != np.bool_:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "logical indexing needs a Bool mask")
+    if mask.dims == x.dims:
+        inner, nsrc, lead = 1, len(x), ()
+        idx = findall(mask.reshape(len(mask)))
+    elif mask.ndim == 1 and x.ndim >= 1 and mask.dims[0] == x.dims[-1]:
+        lead = x.dims[:-1]
+        inner, nsrc = int(np.prod(lead, dtype=np.int64)), x.dims[-1]
+        idx = findall(mask)
+    else:
+        raise IndexError(f"BoundsError: mask {mask.dims} against array {x.dims}")       # Base.checkbounds
+    n = len(idx)
+    y = ROCArray(dims=lead + (n,), dtype=x.dtype)
+    if n > 0 and inner > 0:
+        L.check(L.lib.rk_gather_slices(x.ptr, idx.ptr, y.ptr, x.dtype.itemsize, inner, n, nsrc, stream_ptr()), "rk_gather_slices")
+    return y

@@ -215,6 +215,15 @@ RK_API int32_t rk_findall_scatter(const uint8_t* bools, const int64_t* indices, 
 RK_API int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* shape, int64_t* ys,
                    int64_t* count_out, void* ws, size_t ws_bytes, void* stream);
 
+/* ---- gather along the last dimension ---------------------------------------------------------
+ * y[i, j] = x[i, idx[j]] for i in 1:inner, j in 1:nidx (idx 1-based, Int64; x has `nsrc` slices
+ * of `inner` elements).  Serves logical indexing `x[mask]`, `x[:, mask]`, `x[:, :, mask]`
+ * (test/hip_rocarray/indexing.jl:5-18) once  Base.to_index(::ROCArray, ::AbstractArray{Bool})
+ * src/kernels/indexing.jl:1  has produced idx = findall(mask); the reference leaves the gather to
+ * GPUArrays' generic indexing kernel.  Elements are opaque (`elsize` = 1, 2, 4, 8 or 16). */
+RK_API int32_t rk_gather_slices(const void* x, const int64_t* idx, void* y, size_t elsize,
+                         int64_t inner, int64_t nidx, int64_t nsrc, void* stream);
+
 /* ---- reverse / reverse! -------------------------------------------------------------------
  * Replaces both `_reverse!` kernels of src/kernels/reverse.jl: out of place (`:59-88`, y != x)
  * and in place (`:92-122`, y == x; partially overlapping x and y are not allowed).

@@ -174,6 +174,11 @@ def test_volumerhs_and_scatter_validation(L):
     n = 1 << 20
     assert tb(L.RK_F32, n, 0) >= 4 * n and tb(L.RK_F32, n, 1) >= 16 * n and tb(L.RK_F32, n, 0) < 5 * n
     assert tb(L.RK_I64, n, 0) >= 8 * n and tb(L.RK_I16, n, 0) >= 2 * n and tb(L.RK_U8, n, 0) == 256
+    ga = L.lib.rk_gather_slices
+    assert ga(None, one, two, 4, 3, 5, 7, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert ga(one, one, two, 3, 3, 5, 7, None) == L.RK_ERR_UNSUPPORTED
+    assert ga(one, one, two, 4, -1, 5, 7, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert ga(None, None, None, 4, 3, 0, 7, None) == L.RK_SUCCESS
     f = L.lib.rk_findall
     assert f(None, 1, L.shape_array((5,)), one, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(one, 1, L.shape_array((5,)), None, None, two, 16 << 20, None) == L.RK_ERR_INVALID_ARGUMENT

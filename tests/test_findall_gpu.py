@@ -68,3 +68,25 @@ def test_findall_full_size_and_count_out(rk, orc):
     m = np.random.default_rng(7).random(1 << 20) < 0.5
     idx = rk.Array(rk.findall(rk.ROCArray(m)))
     assert np.array_equal(x[idx - 1], x[m])
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.float64, np.int16, np.bool_, np.complex128])
+def test_selection_by_mask(rk, orc, dtype):
+    # test/hip_rocarray/indexing.jl:5-18: x[m], x[:, m], x[:, :, m]
+    rng = np.random.default_rng(12)
+    def rand(shape):
+        return (rng.random(shape) * 1000).astype(dtype) if np.dtype(dtype).kind != "b" else rng.random(shape) < 0.5
+    for n in (16, 100_003):
+        m = rng.random(n) < 0.5
+        md = rk.ROCArray(m)
+        for shape in ((n,), (1, n), (3, 1, n), (7, n)):
+            x = rand(shape)
+            got = rk.Array(rk.getindex_mask(rk.ROCArray(x), md))
+            assert np.array_equal(got, x[..., m])
+    x = rand((33, 65))
+    m2 = rng.random((33, 65)) < 0.3
+    got = rk.Array(rk.getindex_mask(rk.ROCArray(x), rk.ROCArray(m2)))
+    assert np.array_equal(got, x.reshape(-1, order="F")[m2.reshape(-1, order="F")])        # column-major order of the hits
+    with pytest.raises(IndexError):
+        rk.getindex_mask(rk.ROCArray(x), rk.ROCArray(np.ones(5, dtype=bool)))
+    assert rk.getindex_mask(rk.ROCArray(x), rk.ROCArray(np.zeros((33, 65), dtype=bool))).dims == (0,)
