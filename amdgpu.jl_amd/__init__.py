@@ -13,6 +13,7 @@ from .mapreduce import (mapreduce, mapreducedim_, sum, prod, maximum, minimum, c
 from .accumulate import accumulate, accumulate_, cumsum, cumprod, accumulate_eltype    # noqa: F401
 from . import broadcast                                                               # noqa: F401
 from .broadcast import lazy, materialize, materialize_, fill_, Broadcasted             # noqa: F401
+from .views import ROCView, view, transpose, PermutedDimsArray                         # noqa: F401
 from .volumerhs import volumerhs_                                                     # noqa: F401
 from .indexing import findall, getindex_mask                                                         # noqa: F401
 from .reverse import reverse, reverse_                                                # noqa: F401

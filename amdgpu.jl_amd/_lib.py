@@ -53,6 +53,9 @@ class RkOperand(C.Structure):
         ("shape", C.c_int64 * RK_MAX_DIMS),
         ("scalar_f", C.c_double),
         ("scalar_i", C.c_int64),
+        ("strided", C.c_int32),
+        ("reserved", C.c_int32),
+        ("strides", C.c_int64 * RK_MAX_DIMS),
     ]
 
 
@@ -80,6 +83,7 @@ PROTOTYPES = {
     "rk_accumulate": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,
                                   C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_broadcast": (C.c_int32, [C.POINTER(RkProgram), C.c_void_p, C.c_int, C.c_int, _I64P, C.c_void_p]),
+    "rk_broadcast_strided": (C.c_int32, [C.POINTER(RkProgram), C.c_void_p, C.c_int, C.c_int, _I64P, _I64P, C.c_void_p]),
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,
                                      C.c_void_p]),
     "rk_findall_scatter": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_void_p]),

@@ -140,7 +140,11 @@ def zeros(dtype, *dims) -> ROCArray:
     return out
 
 
-def Array(x: ROCArray) -> np.ndarray:
+def Array(x) -> np.ndarray:
+    """``Array(x)`` of a ROCArray, or of a strided wrapper (copied to a dense array on the device first)."""
+    if not isinstance(x, ROCArray):
+        from .views import copy
+        x = copy(x)
     return x.to_host()
 
 

@@ -17,6 +17,9 @@ import numpy as np
 
 from . import _lib as L
 from .array import ROCArray, dtype_code, stream_ptr
+from .views import ROCView
+
+_ARRAYS = (ROCArray, ROCView)
 
 _BINARY = {"+": L.RK_BC_ADD, "-": L.RK_BC_SUB, "*": L.RK_BC_MUL, "/": L.RK_BC_DIV, "max": L.RK_BC_MAX,
            "min": L.RK_BC_MIN, "^": L.RK_BC_POW}
@@ -141,7 +144,7 @@ def _compile(bc: Broadcasted):
     _flatten(_leaf(bc), operands, tokens)
     if len(tokens) > L.RK_MAX_PROGRAM:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "broadcast expression too long")
-    dts = [o.dtype if isinstance(o, ROCArray) else _scalar_dtype(o) for o in operands]
+    dts = [o.dtype if isinstance(o, _ARRAYS) else _scalar_dtype(o) for o in operands]
     compute = np.result_type(*dts) if dts else np.dtype(np.float64)
     only_leaf = len(tokens) == 1
     if compute.kind != "f":
@@ -151,7 +154,7 @@ def _compile(bc: Broadcasted):
             raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "integer broadcast arithmetic is not in the native op set")
     if compute == np.float16:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "Float16 broadcast")
-    shapes = [o.dims for o in operands if isinstance(o, ROCArray)]
+    shapes = [o.dims for o in operands if isinstance(o, _ARRAYS)]
     return operands, tokens, compute, broadcast_shape(*shapes)
 
 
@@ -161,8 +164,8 @@ def _program(operands, tokens, compute, dest_ndim) -> L.RkProgram:
     p.n_operands = len(operands)
     for k, o in enumerate(operands):
         ro = p.operands[k]
-        if isinstance(o, ROCArray):
-            ro.ptr = o.ptr
+        if isinstance(o, _ARRAYS):
+            ro.ptr = o.sptr if isinstance(o, ROCView) else o.ptr
             ro.dtype = o.code
             dims = o.dims
             while len(dims) > dest_ndim and dims[-1] == 1:     # trailing singleton dims carry nothing
@@ -170,6 +173,10 @@ def _program(operands, tokens, compute, dest_ndim) -> L.RkProgram:
             ro.ndim = len(dims)
             for d, n in enumerate(dims):
                 ro.shape[d] = n
+            if isinstance(o, ROCView):                         # SubArray / Transpose / PermutedDimsArray operand
+                ro.strided = 1
+                for d in range(len(dims)):
+                    ro.strides[d] = o.strides[d]
         else:
             dt = _scalar_dtype(o)
             ro.ptr = None
@@ -201,12 +208,16 @@ def materialize_(dest: ROCArray, bc) -> ROCArray:
 
 def _launch_broadcast(dest, operands, tokens, compute):
     prog = _program(operands, tokens, compute, dest.ndim)
-    args = (prog, dest.ptr, dest.code, dest.ndim, L.shape_array(dest.dims))
-    fn = L.lib.rk_broadcast
     keep = operands          # the program holds raw device pointers: keep the arrays alive with the plan
+    if isinstance(dest, ROCView):                  # `@view(C[...]) .= bc`, `transpose(C) .= bc`
+        args = (prog, dest.sptr, dest.code, dest.ndim, L.shape_array(dest.dims), L.shape_array(dest.strides))
+        fn, name = L.lib.rk_broadcast_strided, "rk_broadcast_strided"
+    else:
+        args = (prog, dest.ptr, dest.code, dest.ndim, L.shape_array(dest.dims))
+        fn, name = L.lib.rk_broadcast, "rk_broadcast"
 
     def launch(_keep=keep):
-        L.check(fn(*args, stream_ptr()), "rk_broadcast")
+        L.check(fn(*args, stream_ptr()), name)
     return launch
 
 
@@ -225,7 +236,7 @@ def plan_materialize(dest: ROCArray, bc):
 def materialize(bc) -> ROCArray:
     """``Broadcast.materialize(bc)``: allocates the result (``similar(bc, T, dims)``, broadcast.jl:26-30)."""
     operands, tokens, compute, shape = _compile(bc)
-    dts = [o.dtype if isinstance(o, ROCArray) else _scalar_dtype(o) for o in operands]
+    dts = [o.dtype if isinstance(o, _ARRAYS) else _scalar_dtype(o) for o in operands]
     out_dt = np.result_type(*dts) if len(tokens) == 1 else compute
     dest = ROCArray(dims=shape, dtype=out_dt)
     return materialize_(dest, bc)

@@ -27,7 +27,7 @@ constexpr int BC_RPT = 4;            // rows per thread in rows mode
 struct BcOperand {
     const void* ptr;        // nullptr: scalar
     int32_t     dtype;
-    int32_t     stride0;    // 0 or 1 (elements) along merged dim 0
+    int64_t     stride0;    // element stride along merged dim 0: 0 (extruded), 1 (dense) or any other (views; scalar lanes only)
     int32_t     reused;     // has an extruded dim: elements are read many times -> cached loads, not streaming
     int32_t     row_invariant;   // every stride of dims 1.. is 0: the value depends on the dim-0 index only
     int64_t     stride[RK_MAX_DIMS];   // element strides of merged dims 1.. (index d-1)
@@ -47,6 +47,8 @@ struct BcArgs {
     int64_t   nxb;                     // rows mode: workgroups along dim 0
     void*     dest;
     int32_t   dest_dtype;
+    int64_t   dest_stride0;            // element strides of the destination over the merged dims (dense: 1, shape[0], ...)
+    int64_t   dest_stride[RK_MAX_DIMS];
 };
 
 // ---- typed loads / stores --------------------------------------------------------------------------
@@ -96,7 +98,7 @@ __device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT
         for (int j = 0; j < VEC; ++j) v[j] = x;
         return;
     }
-    const bool contiguous = o.stride0 != 0;
+    const bool contiguous = o.stride0 != 0;     // on the vector path stride0 is 0 or 1; scalar lanes carry any stride in `off`
     if (MAY_REUSE && o.reused != 0) load_typed<CT, VEC, true, HOMOG>(o, off, contiguous, v);
     else load_typed<CT, VEC, false, HOMOG>(o, off, contiguous, v);
 }
@@ -288,12 +290,14 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         constexpr int NB = Eval::USES_LDS ? 1 : (Eval::NOPS >= 4 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
+            int64_t doff[NB];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
                 int64_t row = row0 + r0 + b;
                 if (row >= a.nrows) row = a.nrows - 1;
 #pragma unroll
                 for (int k = 0; k < Eval::NOPS; ++k) off[k] = i0 * a.op[k].stride0;
+                doff[b] = i0 * a.dest_stride0;
                 int64_t rem = row;
                 for (int d = 1; d < a.ndim; ++d) {
                     int64_t c;
@@ -301,6 +305,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
                     else { c = rem % a.shape[d]; rem /= a.shape[d]; }
 #pragma unroll
                     for (int k = 0; k < Eval::NOPS; ++k) off[k] += c * a.op[k].stride[d - 1];
+                    doff[b] += c * a.dest_stride[d - 1];
                 }
 #pragma unroll
                 for (int k = 0; k < Eval::NOPS; ++k) {
@@ -318,7 +323,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
                 if (row < a.nrows) {
                     CT out[VEC];
                     Eval::template run<CT, VEC>(a, in[b], out, lds);
-                    store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, row * a.shape[0] + i0, out);
+                    store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, doff[b], out);
                 }
             }
         }
@@ -389,8 +394,8 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
 
 using namespace rk;
 
-extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
-                                void* stream) {
+static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
+                              const int64_t* dest_strides, void* stream) {
     if (prog == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
     if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
@@ -425,7 +430,16 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
         total *= shape[d];
     }
     // operand shapes against dest (Julia: DimensionMismatch), per-dim strides with 0 on extruded dims
-    int64_t stride[RK_MAX_OPERANDS][RK_MAX_DIMS];
+    // slot n_operands holds the destination, so that dims merge only where it is dense as well
+    const int KD = prog->n_operands;
+    int64_t stride[RK_MAX_OPERANDS + 1][RK_MAX_DIMS];
+    {
+        int64_t s = 1;
+        for (int d = 0; d < ndim; ++d) {
+            stride[KD][d] = dest_strides ? dest_strides[d] : s;
+            s *= shape[d];
+        }
+    }
     for (int k = 0; k < prog->n_operands; ++k) {
         const rk_operand& o = prog->operands[k];
         if (o.dtype < RK_F32 || o.dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
@@ -439,7 +453,7 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
         for (int d = 0; d < ndim; ++d) {
             const int64_t n = d < o.ndim ? o.shape[d] : 1;
             if (n != shape[d] && n != 1) return RK_ERR_DIMENSION;
-            stride[k][d] = (n == 1) ? 0 : s;
+            stride[k][d] = (n == 1) ? 0 : (o.strided ? o.strides[d] : s);
             s *= n;
         }
     }
@@ -451,22 +465,22 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
     BcArgs a;
     std::memset(&a, 0, sizeof(a));
     int64_t mshape[RK_MAX_DIMS];
-    int64_t mstride[RK_MAX_OPERANDS][RK_MAX_DIMS];
+    int64_t mstride[RK_MAX_OPERANDS + 1][RK_MAX_DIMS];
     int m = 0;
     for (int d = 0; d < ndim; ++d) {
         if (shape[d] == 1) continue;
         bool merge = m > 0;
         if (merge)
-            for (int k = 0; k < prog->n_operands; ++k)
+            for (int k = 0; k <= KD; ++k)
                 if (stride[k][d] != mstride[k][m - 1] * mshape[m - 1]) { merge = false; break; }
         if (merge) mshape[m - 1] *= shape[d];
         else {
             mshape[m] = shape[d];
-            for (int k = 0; k < prog->n_operands; ++k) mstride[k][m] = stride[k][d];
+            for (int k = 0; k <= KD; ++k) mstride[k][m] = stride[k][d];
             ++m;
         }
     }
-    if (m == 0) { mshape[0] = 1; for (int k = 0; k < prog->n_operands; ++k) mstride[k][0] = 0; m = 1; }
+    if (m == 0) { mshape[0] = 1; for (int k = 0; k < KD; ++k) mstride[k][0] = 0; mstride[KD][0] = 1; m = 1; }
 
     a.n_operands = prog->n_operands;
     a.n_tokens = prog->n_tokens;
@@ -477,8 +491,13 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
     for (int d = 0; d < m; ++d) { a.shape[d] = mshape[d]; if (d > 0) a.nrows *= mshape[d]; }
     a.dest = dest;
     a.dest_dtype = (int32_t)dest_dtype;
-    bool linear = true;     // every array operand dense over the merged shape
-    bool vec = (mshape[0] % 4 == 0) && is_aligned(dest, 4 * dtype_size(dest_dtype));
+    a.dest_stride0 = mstride[KD][0];
+    for (int d = 1; d < m; ++d) a.dest_stride[d - 1] = mstride[KD][d];
+    bool linear = (m == 1 && mstride[KD][0] == 1);     // the destination and every array operand dense over the merged shape
+    // 16-byte lanes: whole vectors along dim 0, dense there, and every row start of every array 16-byte aligned
+    bool vec = (mshape[0] % 4 == 0) && is_aligned(dest, 4 * dtype_size(dest_dtype)) && mstride[KD][0] == 1;
+    for (int d = 1; d < m; ++d)
+        if (mstride[KD][d] % 4 != 0) vec = false;
     for (int k = 0; k < prog->n_operands; ++k) {
         const rk_operand& o = prog->operands[k];
         BcOperand& b = a.op[k];
@@ -486,7 +505,7 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
         b.dtype = o.dtype;
         b.sf = o.scalar_f;
         b.si = o.scalar_i;
-        b.stride0 = (int32_t)mstride[k][0];
+        b.stride0 = mstride[k][0];
         b.row_invariant = 1;
         b.reused = (mstride[k][0] == 0) ? 1 : 0;
         for (int d = 1; d < m; ++d) {
@@ -495,14 +514,14 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
             else b.reused = 1;
         }
         if (o.ptr != nullptr) {
-            if (m > 1 || mstride[k][0] != 1) linear = false;
-            if (mstride[k][0] == 1 && !is_aligned(o.ptr, 4 * dtype_size(o.dtype))) vec = false;
+            // one merged dim: the flat kernel takes operands that are dense (stride 1) or fully extruded (stride 0)
+            if (mstride[k][0] != 0 && mstride[k][0] != 1) { linear = false; vec = false; }
+            if (mstride[k][0] == 1) {
+                if (!is_aligned(o.ptr, 4 * dtype_size(o.dtype))) vec = false;
+                for (int d = 1; d < m; ++d)
+                    if (mstride[k][d] % 4 != 0) vec = false;
+            }
         }
-    }
-    if (m > 1) linear = false;
-    if (m == 1) {
-        // one merged dim: operands are dense (stride 1) or fully extruded (stride 0, same as a scalar load)
-        linear = true;
     }
     if (!linear) {
         // lanes along dim 0: TX = smallest power of two covering shape[0] / VEC, at most the workgroup
@@ -514,4 +533,14 @@ extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype des
     }
     if (prog->compute == RK_F32) return bc_dispatch<float>(a, vec, !linear, (hipStream_t)stream);
     return bc_dispatch<double>(a, vec, !linear, (hipStream_t)stream);
+}
+
+extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
+                                void* stream) {
+    return broadcast_impl(prog, dest, dest_dtype, ndim, shape, nullptr, stream);
+}
+
+extern "C" int32_t rk_broadcast_strided(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
+                                        const int64_t* dest_strides, void* stream) {
+    return broadcast_impl(prog, dest, dest_dtype, ndim, shape, dest_strides, stream);
 }

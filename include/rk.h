@@ -171,6 +171,10 @@ typedef struct {
     int64_t     shape[RK_MAX_DIMS];
     double      scalar_f;         /* scalar value when dtype is F32/F64                  */
     int64_t     scalar_i;         /* scalar value when dtype is an integer type          */
+    int32_t     strided;          /* != 0: `strides` below describe the array (a view, a
+                                   * transpose, a PermutedDimsArray); 0: dense column-major */
+    int32_t     reserved;
+    int64_t     strides[RK_MAX_DIMS]; /* element strides per dim; may be negative          */
 } rk_operand;
 
 typedef struct {
@@ -183,6 +187,12 @@ typedef struct {
 
 RK_API int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype,
                      int ndim, const int64_t* shape, void* stream);
+/* The same with a destination that is a strided view (`@view(C[2:5, :]) .= ...`,
+ * `transpose(C) .= ...`): `dest` points at its first element, `dest_strides` are its element
+ * strides per dim (NULL = dense).  Distinct index tuples must address distinct elements. */
+RK_API int32_t rk_broadcast_strided(const rk_program* prog, void* dest, rk_dtype dest_dtype,
+                             int ndim, const int64_t* shape, const int64_t* dest_strides,
+                             void* stream);
 
 /* ---- volumerhs -----------------------------------------------------------------------
  * Replaces `@roc groupsize=(5,5) gridsize=nelem volumerhs!(rhs, Q, vgeo, gravity, D, nelem)`

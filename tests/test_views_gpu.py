@@ -1,0 +1,93 @@
+"""Broadcast with wrapper operands and destinations -- views, transposes, PermutedDimsArrays (the reference's
+ROCArrayStyle covers "any ROCArray or wrapper", src/broadcast.jl:7-10) -- against NumPy slicing, through the C ABI.
+`+ - *` results are bit-exact (same Float32 operations in the same order)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _f32(rng, shape):
+    return rng.standard_normal(shape).astype(np.float32)
+
+
+def test_view_operands(rk):
+    rng = np.random.default_rng(1)
+    A = _f32(rng, (40, 30)); B = _f32(rng, (40, 30)); v = _f32(rng, 40)
+    dA, dB, dv = rk.ROCArray(A), rk.ROCArray(B), rk.ROCArray(v)
+    L = rk.lazy
+    # rows 3:22, columns 2:2:30 of A plus a dense block
+    got = rk.Array(rk.materialize(L(rk.view(dA, (3, 22), (2, 2, 30))) + L(rk.ROCArray(np.ascontiguousarray(B[2:22, 1:30:2])))))
+    assert np.array_equal(got, A[2:22, 1:30:2] + B[2:22, 1:30:2])
+    # a column view and a reversed row range
+    got = rk.Array(rk.materialize(L(rk.view(dA, None, 7)) * L(dv)))
+    assert np.array_equal(got, A[:, 6] * v)
+    got = rk.Array(rk.materialize(L(rk.view(dA, (40, -1, 1), None)) - L(dB)))
+    assert np.array_equal(got, A[::-1, :] - B)
+    # a row view (stride 40 along its only dim)
+    got = rk.Array(rk.materialize(np.float32(2) * L(rk.view(dA, 5, None))))
+    assert np.array_equal(got, np.float32(2) * A[4, :])
+    assert np.array_equal(rk.Array(rk.view(dA, (2, 39), (1, 30))), A[1:39, :])
+
+
+def test_transpose_and_permuteddims_operands(rk):
+    rng = np.random.default_rng(2)
+    A = _f32(rng, (64, 48)); B = _f32(rng, (48, 64)); T3 = _f32(rng, (8, 12, 20))
+    L = rk.lazy
+    got = rk.Array(rk.materialize(L(rk.transpose(rk.ROCArray(A))) + L(rk.ROCArray(B))))
+    assert np.array_equal(got, A.T + B)
+    v = _f32(rng, 48)
+    got = rk.Array(rk.materialize(L(rk.ROCArray(A)) * L(rk.transpose(rk.ROCArray(v)))))       # 64x48 .* 1x48
+    assert np.array_equal(got, A * v[None, :])
+    P = rk.PermutedDimsArray(rk.ROCArray(T3), (3, 1, 2))
+    assert P.dims == (20, 8, 12)
+    assert np.array_equal(rk.Array(P), np.transpose(T3, (2, 0, 1)))
+    assert np.array_equal(rk.Array(rk.materialize(L(P) * np.float32(3))), np.transpose(T3, (2, 0, 1)) * np.float32(3))
+    # against the dense permutedims kernel
+    assert np.array_equal(rk.Array(P), rk.Array(rk.permutedims(rk.ROCArray(T3), (3, 1, 2))))
+
+
+def test_view_destinations(rk):
+    rng = np.random.default_rng(3)
+    C = _f32(rng, (50, 37)); X = _f32(rng, (20, 37)); Y = _f32(rng, (37, 50))
+    L = rk.lazy
+    dC = rk.ROCArray(C)
+    rk.materialize_(rk.view(dC, (11, 30), None), L(rk.ROCArray(X)) * np.float32(2))            # @view(C[11:30, :]) .= 2X
+    want = C.copy(); want[10:30, :] = X * np.float32(2)
+    assert np.array_equal(rk.Array(dC), want)
+    rk.materialize_(rk.transpose(dC), L(rk.ROCArray(Y)) + np.float32(1))                        # transpose(C) .= Y .+ 1
+    assert np.array_equal(rk.Array(dC), (Y + np.float32(1)).T)
+    rk.fill_(rk.view(dC, (1, 2, 49), (37, -3, 1)), 7.0)                                          # C[1:2:49, 37:-3:1] .= 7
+    want = (Y + np.float32(1)).T.copy(); want[0:49:2, 36::-3] = 7.0
+    assert np.array_equal(rk.Array(dC), want)
+    # in-place update of a view from itself and a row vector: v .= v .+ r
+    r = _f32(rng, 37)
+    vw = rk.view(dC, (5, 44), None)
+    rk.materialize_(vw, L(vw) + L(rk.transpose(rk.ROCArray(r))))
+    want[4:44, :] = want[4:44, :] + r[None, :]
+    assert np.array_equal(rk.Array(dC), want)
+
+
+def test_large_strided_shapes_and_vector_path(rk):
+    rng = np.random.default_rng(4)
+    A = _f32(rng, (1024, 513))
+    dA = rk.ROCArray(A)
+    L = rk.lazy
+    # aligned row range with whole 16-byte vectors: the vector lanes stay on
+    got = rk.Array(rk.materialize(L(rk.view(dA, (257, 768), (2, 512))) * np.float32(0.5)))
+    assert np.array_equal(got, A[256:768, 1:512] * np.float32(0.5))
+    # unaligned start, odd extents
+    got = rk.Array(rk.materialize(L(rk.view(dA, (2, 1000), (3, 511))) + L(rk.view(dA, (3, 1001), (1, 509)))))
+    assert np.array_equal(got, A[1:1000, 2:511] + A[2:1001, 0:509])
+    # matrix transpose through the broadcast kernel equals the tiled transpose
+    assert np.array_equal(rk.Array(rk.transpose(dA)), A.T)
+
+
+def test_views_are_refused_by_dense_ops(rk):
+    d = rk.ROCArray(np.arange(12, dtype=np.float32).reshape(3, 4))
+    with pytest.raises(rk.UnsupportedError):
+        rk.sum(rk.view(d, (1, 2), None))
+    with pytest.raises(IndexError):
+        rk.view(d, (1, 5), None)
+    with pytest.raises(IndexError):
+        rk.view(d, 4, None)
