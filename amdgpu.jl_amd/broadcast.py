@@ -139,23 +139,45 @@ def _flatten(bc: Broadcasted, operands: list, tokens: list):
         tokens.append(_UNARY[bc.f])
 
 
+_INT_SAFE = None
+
+
+def _int_safe_tokens():
+    global _INT_SAFE
+    if _INT_SAFE is None:
+        _INT_SAFE = {L.RK_BC_ADD, L.RK_BC_SUB, L.RK_BC_MUL, L.RK_BC_MAX, L.RK_BC_MIN, L.RK_BC_FMA,
+                     L.RK_BC_NEG, L.RK_BC_ABS, L.RK_BC_ABS2, L.RK_BC_IDENTITY}
+    return _INT_SAFE
+
+
 def _compile(bc: Broadcasted):
+    """Flatten ``bc``; returns (operands, tokens, compute type, shape, result eltype).  Floating-point programs compute
+    in the promoted float type.  All-integer programs of ``+ - * max min muladd - abs abs2`` compute in Int64 and keep
+    Julia's result eltype (Int32 .+ Int32 is an Int32 that wraps); with ``/`` or a math function Julia's result is a
+    Float64, and so is the compute type here."""
     operands, tokens = [], []
     _flatten(_leaf(bc), operands, tokens)
     if len(tokens) > L.RK_MAX_PROGRAM:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "broadcast expression too long")
     dts = [o.dtype if isinstance(o, _ARRAYS) else _scalar_dtype(o) for o in operands]
-    compute = np.result_type(*dts) if dts else np.dtype(np.float64)
-    only_leaf = len(tokens) == 1
-    if compute.kind != "f":
-        if only_leaf:                      # copy / fill / convert: exact for |x| < 2^53
-            compute = np.dtype(np.float64)
+    eltype = np.result_type(*dts) if dts else np.dtype(np.float64)
+    compute = eltype
+    ops = [t for t in tokens if t >= L.RK_MAX_OPERANDS]
+    if eltype.kind != "f":
+        if eltype.kind not in "iub":
+            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"broadcast over eltype {eltype}")
+        if all(t in _int_safe_tokens() for t in ops):
+            if eltype == np.uint64 and any(t in (L.RK_BC_MAX, L.RK_BC_MIN) for t in ops):
+                raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "max / min of UInt64 values")
+            compute = np.dtype(np.int64)
+            if eltype == np.bool_ and ops:             # true + true isa Int
+                eltype = np.dtype(np.int64)
         else:
-            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "integer broadcast arithmetic is not in the native op set")
+            compute = eltype = np.dtype(np.float64)
     if compute == np.float16:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "Float16 broadcast")
     shapes = [o.dims for o in operands if isinstance(o, _ARRAYS)]
-    return operands, tokens, compute, broadcast_shape(*shapes)
+    return operands, tokens, compute, broadcast_shape(*shapes), eltype
 
 
 def _program(operands, tokens, compute, dest_ndim) -> L.RkProgram:
@@ -194,7 +216,7 @@ def _program(operands, tokens, compute, dest_ndim) -> L.RkProgram:
 
 def materialize_(dest: ROCArray, bc) -> ROCArray:
     """``Broadcast.materialize!(dest, bc)`` / ``copyto!(dest, bc)``: one fused kernel, returns dest."""
-    operands, tokens, compute, shape = _compile(bc)
+    operands, tokens, compute, shape, _ = _compile(bc)
     full = broadcast_shape(shape, dest.dims)
     while len(full) > dest.ndim and full[-1] == 1:
         full = full[:-1]
@@ -224,7 +246,7 @@ def _launch_broadcast(dest, operands, tokens, compute):
 def plan_materialize(dest: ROCArray, bc):
     """Flatten and validate ``dest .= bc`` once; the returned callable repeats it with no per-call host
     work beyond the foreign call (Julia specialises the same tree at compile time)."""
-    operands, tokens, compute, shape = _compile(bc)
+    operands, tokens, compute, shape, _ = _compile(bc)
     full = broadcast_shape(shape, dest.dims)
     while len(full) > dest.ndim and full[-1] == 1:
         full = full[:-1]
@@ -235,10 +257,8 @@ def plan_materialize(dest: ROCArray, bc):
 
 def materialize(bc) -> ROCArray:
     """``Broadcast.materialize(bc)``: allocates the result (``similar(bc, T, dims)``, broadcast.jl:26-30)."""
-    operands, tokens, compute, shape = _compile(bc)
-    dts = [o.dtype if isinstance(o, _ARRAYS) else _scalar_dtype(o) for o in operands]
-    out_dt = np.result_type(*dts) if len(tokens) == 1 else compute
-    dest = ROCArray(dims=shape, dtype=out_dt)
+    operands, tokens, compute, shape, eltype = _compile(bc)
+    dest = ROCArray(dims=shape, dtype=eltype)
     return materialize_(dest, bc)
 
 

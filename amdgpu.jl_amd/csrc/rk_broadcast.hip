@@ -180,10 +180,8 @@ struct EvalInterp {
                 case RK_BC_ADD: RK_BC_BIN(x + y);
                 case RK_BC_SUB: RK_BC_BIN(x - y);
                 case RK_BC_MUL: RK_BC_BIN(x * y);
-                case RK_BC_DIV: RK_BC_BIN(x / y);
                 case RK_BC_MAX: RK_BC_BIN(OpMax()(x, y));
                 case RK_BC_MIN: RK_BC_BIN(OpMin()(x, y));
-                case RK_BC_POW: RK_BC_BIN(pow(x, y));
                 case RK_BC_FMA: {                   // x * y + top with x the deepest of the three
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) s0[j] = s2[j] * s1[j] + s0[j];
@@ -193,14 +191,22 @@ struct EvalInterp {
                 case RK_BC_NEG: RK_BC_UN(-x);
                 case RK_BC_ABS: RK_BC_UN(x < CT(0) ? -x : (x == CT(0) ? CT(0) : x));
                 case RK_BC_ABS2: RK_BC_UN(x * x);
-                case RK_BC_SQRT: RK_BC_UN(sqrt(x));
-                case RK_BC_EXP: RK_BC_UN(exp(x));
-                case RK_BC_LOG: RK_BC_UN(log(x));
-                case RK_BC_SIN: RK_BC_UN(sin(x));
-                case RK_BC_COS: RK_BC_UN(cos(x));
-                case RK_BC_TANH: RK_BC_UN(tanh(x));
-                case RK_BC_INV: RK_BC_UN(CT(1) / x);
-                default: break;                     // RK_BC_IDENTITY
+                default:                            // RK_BC_IDENTITY, or a token of the floating-point programs
+                    if constexpr (std::is_floating_point<CT>::value) {
+                        switch (tok) {
+                            case RK_BC_DIV: RK_BC_BIN(x / y);
+                            case RK_BC_POW: RK_BC_BIN(pow(x, y));
+                            case RK_BC_SQRT: RK_BC_UN(sqrt(x));
+                            case RK_BC_EXP: RK_BC_UN(exp(x));
+                            case RK_BC_LOG: RK_BC_UN(log(x));
+                            case RK_BC_SIN: RK_BC_UN(sin(x));
+                            case RK_BC_COS: RK_BC_UN(cos(x));
+                            case RK_BC_TANH: RK_BC_UN(tanh(x));
+                            case RK_BC_INV: RK_BC_UN(CT(1) / x);
+                            default: break;
+                        }
+                    }
+                    break;
             }
         }
 #undef RK_BC_UN
@@ -253,10 +259,19 @@ struct EvalBinary {
             case RK_BC_ADD: RK_BC_BIN2(x + y);
             case RK_BC_SUB: RK_BC_BIN2(x - y);
             case RK_BC_MUL: RK_BC_BIN2(x * y);
-            case RK_BC_DIV: RK_BC_BIN2(x / y);
             case RK_BC_MAX: RK_BC_BIN2(OpMax()(x, y));
             case RK_BC_MIN: RK_BC_BIN2(OpMin()(x, y));
-            default:        RK_BC_BIN2(pow(x, y));      // RK_BC_POW
+            default:
+                if constexpr (std::is_floating_point<CT>::value) {
+                    if (a.tokens[2] == RK_BC_DIV) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) out[j] = in[0][j] / in[1][j];
+                    } else {                        // RK_BC_POW
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) out[j] = pow(in[0][j], in[1][j]);
+                    }
+                }
+                break;
         }
 #undef RK_BC_BIN2
     }
@@ -357,7 +372,7 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
     }
     const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - BC_REG_DEPTH) * VECN * BC_BLOCK * sizeof(CT) : 0;
     // homogeneous element types: a kernel without any dispatch on the element type
-    bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : RK_F64);
+    bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : (std::is_same<CT, double>::value ? RK_F64 : RK_I64));
     for (int k = 0; k < a.n_operands; ++k)
         if (a.op[k].ptr != nullptr && a.op[k].dtype != a.dest_dtype) homog = false;
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
@@ -382,7 +397,9 @@ static bool tokens_are(const BcArgs& a, std::initializer_list<int> want) {
 
 template <typename CT>
 static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
-    if (tokens_are(a, {0, 1, RK_BC_MUL, 2, 3, RK_BC_EXP, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAxpbyExp, CT>(a, vec, rows, stream);
+    if constexpr (std::is_floating_point<CT>::value) {
+        if (tokens_are(a, {0, 1, RK_BC_MUL, 2, 3, RK_BC_EXP, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAxpbyExp, CT>(a, vec, rows, stream);
+    }
     if (tokens_are(a, {0, 1, 2, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAddMul, CT>(a, vec, rows, stream);
     if (tokens_are(a, {0})) return bc_launch<EvalCopy, CT>(a, vec, rows, stream);
     if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 && a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW)
@@ -399,7 +416,8 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
     if (prog == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
     if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
-    if (prog->compute != RK_F32 && prog->compute != RK_F64) return RK_ERR_UNSUPPORTED;
+    if (prog->compute != RK_F32 && prog->compute != RK_F64 && prog->compute != RK_I64) return RK_ERR_UNSUPPORTED;
+    const bool int_compute = prog->compute == RK_I64;
     if (prog->n_operands < 0 || prog->n_operands > RK_MAX_OPERANDS) return RK_ERR_INVALID_ARGUMENT;
     if (prog->n_tokens < 1 || prog->n_tokens > RK_MAX_PROGRAM) return RK_ERR_INVALID_ARGUMENT;
 
@@ -412,12 +430,14 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
             ++depth;
         } else if (tok >= RK_BC_ADD && tok <= RK_BC_POW) {
             if (depth < 2) return RK_ERR_INVALID_ARGUMENT;
+            if (int_compute && (tok == RK_BC_DIV || tok == RK_BC_POW)) return RK_ERR_UNSUPPORTED;   // Julia: Int / Int is a Float64
             --depth;
         } else if (tok == RK_BC_FMA) {
             if (depth < 3) return RK_ERR_INVALID_ARGUMENT;
             depth -= 2;
         } else if (tok >= RK_BC_NEG && tok <= RK_BC_IDENTITY) {
             if (depth < 1) return RK_ERR_INVALID_ARGUMENT;
+            if (int_compute && tok != RK_BC_NEG && tok != RK_BC_ABS && tok != RK_BC_ABS2 && tok != RK_BC_IDENTITY) return RK_ERR_UNSUPPORTED;
         } else return RK_ERR_INVALID_ARGUMENT;
         if (depth > max_depth) max_depth = depth;
     }
@@ -532,6 +552,7 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
         a.nxb = (n0v + (1ll << l2) - 1) >> l2;
     }
     if (prog->compute == RK_F32) return bc_dispatch<float>(a, vec, !linear, (hipStream_t)stream);
+    if (int_compute) return bc_dispatch<int64_t>(a, vec, !linear, (hipStream_t)stream);
     return bc_dispatch<double>(a, vec, !linear, (hipStream_t)stream);
 }
 

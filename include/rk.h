@@ -178,7 +178,10 @@ typedef struct {
 } rk_operand;
 
 typedef struct {
-    int32_t    compute;           /* rk_dtype every operand is converted to: F32 or F64 */
+    int32_t    compute;           /* rk_dtype every operand is converted to: F32, F64, or
+                                   * I64 for integer programs (+ - * max min muladd neg abs
+                                   * abs2 only; the store keeps the low bits, i.e. Int32
+                                   * results wrap as in Julia)                             */
     int32_t    n_operands;
     rk_operand operands[RK_MAX_OPERANDS];
     int32_t    n_tokens;

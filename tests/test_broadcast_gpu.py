@@ -129,3 +129,51 @@ def test_unaligned_and_f64(rk, orc):
     got = rk.materialize(L(v) * 3.0 + 1.0)
     assert got.dtype == np.float64
     assert np.array_equal(rk.Array(got), x[1:] * 3.0 + 1.0)
+
+
+def test_integer_programs_are_exact_and_wrap(rk):
+    # all-integer + - * max min abs compute in Int64 and keep Julia's result eltype; Int32 results wrap
+    rng = np.random.default_rng(50)
+    L = rk.lazy
+    a32 = rng.integers(-2**31, 2**31 - 1, (300, 70), dtype=np.int32)
+    b32 = rng.integers(-2**31, 2**31 - 1, (300, 70), dtype=np.int32)
+    got = rk.materialize(L(rk.ROCArray(a32)) + L(rk.ROCArray(b32)) * L(rk.ROCArray(a32)))
+    assert got.dtype == np.int32
+    with np.errstate(over="ignore"):
+        assert np.array_equal(rk.Array(got), a32 + b32 * a32)                   # NumPy wraps Int32 like Julia
+    a64 = rng.integers(-2**62, 2**62, 100_003, dtype=np.int64)
+    b64 = rng.integers(-2**62, 2**62, 100_003, dtype=np.int64)
+    got = rk.materialize(L(rk.ROCArray(a64)) * 3 - L(rk.ROCArray(b64)))         # beyond 2^53: a Float64 detour would lose bits
+    assert got.dtype == np.int64
+    with np.errstate(over="ignore"):
+        assert np.array_equal(rk.Array(got), a64 * 3 - b64)
+    got = rk.materialize(rk.broadcast.max_(L(rk.ROCArray(a64)), L(rk.ROCArray(b64))) + rk.broadcast.abs_(L(rk.ROCArray(a32[:, 0].astype(np.int64)[:1]))))
+    assert np.array_equal(rk.Array(got), np.maximum(a64, b64) + abs(np.int64(a32[0, 0])))
+    # Int32 matrix .+ Int64 column: promotes to Int64; row/column extrusion
+    col = rng.integers(-1000, 1000, (300, 1), dtype=np.int64)
+    got = rk.materialize(L(rk.ROCArray(a32)) + L(rk.ROCArray(col)))
+    assert got.dtype == np.int64 and np.array_equal(rk.Array(got), a32.astype(np.int64) + col)
+    # gpu_mat_ints .+ 1 (perf/array.jl:16 arrays) and Bool + Bool
+    ints = rng.integers(-10, 11, (512, 1000), dtype=np.int64)
+    assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(ints)) + 1)), ints + 1)
+    m1, m2 = rng.random(1000) < 0.5, rng.random(1000) < 0.5
+    got = rk.materialize(L(rk.ROCArray(m1)) + L(rk.ROCArray(m2)))
+    assert got.dtype == np.int64 and np.array_equal(rk.Array(got), m1.astype(np.int64) + m2)
+    # `/` and math functions of integers are Float64 in Julia
+    got = rk.materialize(L(rk.ROCArray(ints)) / L(rk.ROCArray(ints + 20)))
+    assert got.dtype == np.float64 and np.array_equal(rk.Array(got), ints / (ints + 20))
+    got = rk.materialize(rk.broadcast.sqrt(L(rk.ROCArray(ints + 10))))
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(rk.Array(got), np.sqrt(ints + 10), rtol=1e-15)
+    # an Int64 program into an Int32 destination keeps the low bits; into a Float32 destination converts
+    d32 = rk.ROCArray(dims=(100_003,), dtype=np.int32)
+    rk.materialize_(d32, L(rk.ROCArray(a64)) + L(rk.ROCArray(b64)))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(rk.Array(d32), (a64 + b64).astype(np.int32))
+    small = rng.integers(-1000, 1000, 5000, dtype=np.int64)
+    f32 = rk.ROCArray(dims=(5000,), dtype=np.float32)
+    rk.materialize_(f32, L(rk.ROCArray(small)) * 2)
+    assert np.array_equal(rk.Array(f32), (small * 2).astype(np.float32))
+    # copies of Int64 beyond 2^53 are exact
+    big = np.array([2**62 + 1, -(2**62) - 3, 2**53 + 1], dtype=np.int64)
+    assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(big)))), big)
