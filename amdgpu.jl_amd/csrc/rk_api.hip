@@ -165,11 +165,14 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
             case RK_I32: return mapreduce_i32(a);
             case RK_I64: return mapreduce_i64(a);
             case RK_U8:  return mapreduce_u8(a);
+            case RK_U32: return mapreduce_u32(a);
+            case RK_U64: return mapreduce_u64(a);
             default: return RK_ERR_UNSUPPORTED;
         }
     }
     if (in == RK_I32 && out == RK_I64) return mapreduce_i32_i64(a);
-    if (in == RK_U8 && out == RK_I64) return mapreduce_u8_i64(a);
+    if (in == RK_U8 && (out == RK_I64 || out == RK_U64)) return mapreduce_u8_i64(a);   // sums of bytes: the same bits either way
+    if (in == RK_U32 && out == RK_U64) return mapreduce_u32_u64(a);
     return RK_ERR_UNSUPPORTED;
 }
 
@@ -188,6 +191,8 @@ int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, co
         case RK_I32: return findminmax_i32(a);
         case RK_I64: return findminmax_i64(a);
         case RK_U8:  return findminmax_u8(a);
+        case RK_U32: return findminmax_u32(a);
+        case RK_U64: return findminmax_u64(a);
         default: return RK_ERR_UNSUPPORTED;
     }
 }
@@ -209,6 +214,8 @@ int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, v
             case RK_F64: return scan_f64(a);
             case RK_I32: return scan_i32(a);
             case RK_I64: return scan_i64(a);
+            case RK_U32: return scan_u32(a);
+            case RK_U64: return scan_u64(a);
             default: return RK_ERR_UNSUPPORTED;
         }
     }

@@ -409,6 +409,18 @@ template <> struct OrderKey<int64_t> {
     static __device__ __forceinline__ int64_t value(Key k, bool want_max) { return want_max ? k : ~k; }
 };
 
+template <> struct OrderKey<uint32_t> {
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = false;
+    static __device__ __forceinline__ Key make(uint32_t v, bool want_max) { const Key k = (Key)(v ^ 0x80000000u); return want_max ? k : ~k; }
+    static __device__ __forceinline__ uint32_t value(Key k, bool want_max) { return (uint32_t)(want_max ? k : ~k) ^ 0x80000000u; }
+};
+template <> struct OrderKey<uint64_t> {
+    typedef int64_t Key;
+    static constexpr bool LOWEST_FREE = false;
+    static __device__ __forceinline__ Key make(uint64_t v, bool want_max) { const Key k = (Key)(v ^ 0x8000000000000000ull); return want_max ? k : ~k; }
+    static __device__ __forceinline__ uint64_t value(Key k, bool want_max) { return (uint64_t)(want_max ? k : ~k) ^ 0x8000000000000000ull; }
+};
 template <> struct OrderKey<uint8_t> {            // Bool / UInt8: findfirst(bools) is findmax's index
     typedef int32_t Key;
     static constexpr bool LOWEST_FREE = true;

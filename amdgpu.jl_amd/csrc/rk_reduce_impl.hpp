@@ -595,6 +595,11 @@ int32_t mapreduce_i64(const MapreduceArgs&);
 int32_t mapreduce_i32_i64(const MapreduceArgs&);
 int32_t mapreduce_u8_i64(const MapreduceArgs&);
 int32_t mapreduce_u8(const MapreduceArgs&);
+int32_t mapreduce_u32(const MapreduceArgs&);
+int32_t mapreduce_u32_u64(const MapreduceArgs&);
+int32_t mapreduce_u64(const MapreduceArgs&);
+int32_t findminmax_u32(const FindArgs&);
+int32_t findminmax_u64(const FindArgs&);
 int32_t findminmax_u8(const FindArgs&);
 int32_t findminmax_f32(const FindArgs&);
 int32_t findminmax_f64(const FindArgs&);

@@ -22,7 +22,14 @@ int32_t mapreduce_u8_i64(const MapreduceArgs& a) { return mapreduce_typed<uint8_
 #elif RK_INST == 6
 int32_t mapreduce_u8(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, uint8_t>(a); }      // any / all of Bool arrays
 int32_t findminmax_u8(const FindArgs& a) { return findminmax_typed<uint8_t>(a); }                   // findfirst of Bool arrays
+#elif RK_INST == 7
+int32_t mapreduce_u32(const MapreduceArgs& a) { return mapreduce_typed<uint32_t, uint32_t>(a); }
+int32_t mapreduce_u32_u64(const MapreduceArgs& a) { return mapreduce_typed<uint32_t, uint64_t>(a); }   // add_sum widens UInt32 to UInt64
+int32_t findminmax_u32(const FindArgs& a) { return findminmax_typed<uint32_t>(a); }
+#elif RK_INST == 8
+int32_t mapreduce_u64(const MapreduceArgs& a) { return mapreduce_typed<uint64_t, uint64_t>(a); }
+int32_t findminmax_u64(const FindArgs& a) { return findminmax_typed<uint64_t>(a); }
 #else
-#error "RK_INST must be 0..6"
+#error "RK_INST must be 0..8"
 #endif
 }  // namespace rk

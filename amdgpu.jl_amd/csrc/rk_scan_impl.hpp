@@ -696,5 +696,7 @@ int32_t scan_i32(const ScanArgs&);
 int32_t scan_i64(const ScanArgs&);
 int32_t scan_u8_i64(const ScanArgs&);
 int32_t scan_u8_i32(const ScanArgs&);
+int32_t scan_u32(const ScanArgs&);
+int32_t scan_u64(const ScanArgs&);
 
 }  // namespace rk

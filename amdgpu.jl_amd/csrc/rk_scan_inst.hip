@@ -15,7 +15,11 @@ int32_t scan_i64(const ScanArgs& a) { return scan_typed<int64_t, int64_t>(a); }
 int32_t scan_u8_i64(const ScanArgs& a) { return scan_typed<uint8_t, int64_t>(a); }
 #elif RK_INST == 5
 int32_t scan_u8_i32(const ScanArgs& a) { return scan_typed<uint8_t, int32_t>(a); }
+#elif RK_INST == 6
+int32_t scan_u32(const ScanArgs& a) { return scan_typed<uint32_t, uint32_t>(a); }
+#elif RK_INST == 7
+int32_t scan_u64(const ScanArgs& a) { return scan_typed<uint64_t, uint64_t>(a); }
 #else
-#error "RK_INST must be 0..5"
+#error "RK_INST must be 0..7"
 #endif
 }  // namespace rk

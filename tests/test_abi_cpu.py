@@ -70,7 +70,7 @@ def test_mapreduce_argument_validation(L):
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 9, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # ndim > 8
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, L.shape_array((-1,)), 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(0, 0, L.RK_F32, L.RK_I32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Float32 -> Int32
-    assert f(0, 0, L.RK_U64, L.RK_U64, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert f(0, 0, L.RK_F16, L.RK_F16, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
     # zero-length input: success without launching (src/kernels/mapreduce.jl:91), even with null pointers
     assert f(0, 0, L.RK_F32, L.RK_F32, None, 1, L.shape_array((0,)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     # a reduction that needs partials but has no workspace
@@ -85,7 +85,7 @@ def test_findminmax_and_accumulate_validation(L):
     g = L.lib.rk_findminmax
     assert g(1, L.RK_F32, None, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert g(1, L.RK_F32, one, 2, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # no output requested
-    assert g(1, L.RK_U32, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert g(1, L.RK_I16, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
     assert g(1, L.RK_F32, None, 2, L.shape_array((0, 4)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     a = L.lib.rk_accumulate
     assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT

@@ -251,3 +251,29 @@ def test_any_all_findfirst_bool(rk, orc, shape):
     one[(-1,) * one.ndim] = True                                  # the last element in column-major order too
     got = rk.findfirst(rk.ROCArray(one))
     assert (got if one.ndim == 1 else int(np.ravel_multi_index(tuple(i - 1 for i in got), one.shape, order="F")) + 1) == one.size
+
+
+@pytest.mark.parametrize("dtype", [np.uint32, np.uint64, np.uint8])
+def test_unsigned_reductions(rk, orc, dtype):
+    rng = _rng(41)
+    info = np.iinfo(dtype)
+    for shape, dims in [((100_003,), None), ((300, 70), 1), ((300, 70), 2), ((17, 5, 33), (1, 3))]:
+        A = rng.integers(0, info.max, shape, dtype=dtype, endpoint=True)
+        d = rk.ROCArray(A)
+        s = rk.sum(d, dims=dims)                                       # add_sum widens UInt8 / UInt32 to UInt64
+        want = orc.mapreduce("identity", "add_sum", A, dims=dims)
+        if dims is None:
+            assert s == want and np.asarray(s).dtype == np.uint64
+        else:
+            assert s.dtype == np.uint64 and np.array_equal(rk.Array(s), want)
+        if dtype == np.uint8:
+            continue
+        assert np.array_equal(np.asarray(rk.Array(rk.maximum(d, dims=dims)) if dims else rk.maximum(d)), orc.maximum(A, dims=dims))
+        assert np.array_equal(np.asarray(rk.Array(rk.minimum(d, dims=dims)) if dims else rk.minimum(d)), orc.minimum(A, dims=dims))
+        if dims in (None, 1, 2):
+            _check_findminmax(rk, orc, A, dims)
+        # plain + keeps the eltype and wraps
+        r = rk.mapreduce(rk.identity, rk.add, d, dims=dims)
+        with np.errstate(over="ignore"):
+            want = A.sum(dtype=dtype) if dims is None else A.sum(axis=tuple(x - 1 for x in ((dims,) if isinstance(dims, int) else dims)), keepdims=True, dtype=dtype)
+        assert np.array_equal(np.asarray(r if dims is None else rk.Array(r)), want)

@@ -184,3 +184,16 @@ def test_bool_scan_and_findall(rk, orc):
         want = orc.findall(m)
         assert np.array_equal(got if m.ndim == 1 else got.T, want)
     assert len(rk.findall(rk.ROCArray(np.zeros(100, dtype=bool)))) == 0
+
+
+@pytest.mark.parametrize("dtype", [np.uint32, np.uint64])
+def test_unsigned_scans_wrap(rk, orc, dtype):
+    rng = _rng(33)
+    info = np.iinfo(dtype)
+    for shape, dims in [((300_001,), 1), ((300, 70), 1), ((300, 70), 2), ((64, 3000), 2)]:
+        x = rng.integers(0, info.max, shape, dtype=dtype, endpoint=True)
+        got = rk.accumulate("add", rk.ROCArray(x), dims=dims)
+        assert got.dtype == dtype
+        with np.errstate(over="ignore"):
+            assert np.array_equal(rk.Array(got), np.cumsum(x, axis=dims - 1, dtype=dtype))
+        assert np.array_equal(rk.Array(rk.accumulate("max", rk.ROCArray(x), dims=dims)), np.maximum.accumulate(x, axis=dims - 1))
