@@ -21,6 +21,7 @@ module ROCKernelsNative
 using AMDGPU
 using AMDGPU: ROCArray, AnyROCArray, ROCArrayStyle, HIP
 import GPUArrays
+import LinearAlgebra
 import Base.Broadcast: Broadcasted
 
 const librk = Ref{String}(joinpath(@__DIR__, "..", "librk.so"))
@@ -184,7 +185,13 @@ end
 const RK_MAX_DIMS, RK_MAX_OPERANDS, RK_MAX_PROGRAM = 8, 8, 48
 struct RkOperand
     ptr::Ptr{Cvoid}; dtype::Int32; ndim::Int32; shape::NTuple{8,Int64}; scalar_f::Float64; scalar_i::Int64
+    strided::Int32; reserved::Int32; strides::NTuple{8,Int64}
 end
+# wrappers over a ROCArray that are (pointer, size, strides) triples: operands / destinations of rk_broadcast_strided
+const ROCWrapper{T,N} = Union{SubArray{T,N,<:ROCArray}, LinearAlgebra.Transpose{T,<:ROCArray{T}},
+                              PermutedDimsArray{T,N,<:Any,<:Any,<:ROCArray}}
+is_strided_wrapper(x) = x isa ROCWrapper && eltype(x) <: Real && applicable(strides, x)
+const INT_SAFE = (Int32(32), Int32(33), Int32(34), Int32(36), Int32(37), Int32(39), Int32(64), Int32(65), Int32(66), Int32(74))
 struct RkProgram
     compute::Int32; n_operands::Int32; operands::NTuple{8,RkOperand}; n_tokens::Int32; tokens::NTuple{48,Int32}
 end
@@ -209,7 +216,7 @@ function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
         else
             throw(Unsupported())
         end
-    elseif x isa ROCArray || x isa Union{Float32,Float64,Int32,Int64,Bool}
+    elseif x isa ROCArray || is_strided_wrapper(x) || x isa Union{Float32,Float64,Int32,Int64,Bool}
         k = findfirst(o -> o === x, ops)
         k === nothing && (push!(ops, x); k = length(ops))
         k > RK_MAX_OPERANDS && throw(Unsupported())
@@ -217,43 +224,55 @@ function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
     elseif x isa Base.RefValue && x[] isa Number                    # Ref(scalar)
         flatten!(ops, toks, x[])
     else
-        throw(Unsupported())                                        # views, transposes, closures, ...
+        throw(Unsupported())                                        # non-strided wrappers, closures, ...
     end
 end
 
-function native_copyto!(dest::ROCArray{TD,N}, bc::Broadcasted) where {TD,N}
+function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadcasted) where {TD,N}
     ops, toks = Any[], Int32[]
     flatten!(ops, toks, bc)
     length(toks) <= RK_MAX_PROGRAM || throw(Unsupported())
-    CT = promote_type(map(o -> o isa ROCArray ? eltype(o) : typeof(o), ops)...)
-    CT <: Union{Float32,Float64} || length(toks) == 1 || throw(Unsupported())
-    CT <: Union{Float32,Float64} || (CT = Float64)
-    zero_op = RkOperand(C_NULL, 0, 0, ntuple(_ -> Int64(0), 8), 0.0, 0)
+    CT = promote_type(map(o -> o isa AbstractArray ? eltype(o) : typeof(o), ops)...)
+    if !(CT <: Union{Float32,Float64})
+        # integer programs of + - * max min muladd - abs abs2 compute in Int64 (the store keeps the low bits);
+        # with `/` or a math function Julia's result is a Float64 and so is the compute type
+        CT = all(t -> t < RK_MAX_OPERANDS || t in INT_SAFE, toks) && CT <: Union{Bool,Int32,Int64,UInt8,UInt32} ? Int64 : Float64
+    end
+    zeros8 = ntuple(_ -> Int64(0), 8)
+    zero_op = RkOperand(C_NULL, 0, 0, zeros8, 0.0, 0, 0, 0, zeros8)
     operands = ntuple(RK_MAX_OPERANDS) do k
         k > length(ops) && return zero_op
         o = ops[k]
-        if o isa ROCArray
+        if o isa AbstractArray
             rk_dtype(eltype(o)) === nothing && throw(Unsupported())
-            RkOperand(pointer(o), rk_dtype(eltype(o)), ndims(o), ntuple(d -> d <= ndims(o) ? Int64(size(o, d)) : Int64(0), 8), 0.0, 0)
+            shape = ntuple(d -> d <= ndims(o) ? Int64(size(o, d)) : Int64(0), 8)
+            if o isa ROCArray
+                RkOperand(pointer(o), rk_dtype(eltype(o)), ndims(o), shape, 0.0, 0, 0, 0, zeros8)
+            else                                                     # SubArray / Transpose / PermutedDimsArray
+                st = strides(o)
+                RkOperand(pointer(o), rk_dtype(eltype(o)), ndims(o), shape, 0.0, 0, 1, 0, ntuple(d -> d <= ndims(o) ? Int64(st[d]) : Int64(0), 8))
+            end
         else
-            RkOperand(C_NULL, rk_dtype(typeof(o)), 0, ntuple(_ -> Int64(0), 8), Float64(o), o isa AbstractFloat ? 0 : Int64(o))
+            RkOperand(C_NULL, rk_dtype(typeof(o)), 0, zeros8, Float64(o), o isa AbstractFloat ? 0 : Int64(o), 0, 0, zeros8)
         end
     end
     prog = Ref(RkProgram(rk_dtype(CT), length(ops), operands, length(toks),
                          ntuple(i -> i <= length(toks) ? toks[i] : Int32(0), 48)))
     shape = Int64[size(dest)...]
-    GC.@preserve dest ops prog shape begin
-        check(ccall((:rk_broadcast, librk[]), Int32, (Ptr{RkProgram}, Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Cvoid}),
-                    prog, pointer(dest), rk_dtype(TD), N, shape, stream_ptr()))
+    dstrides = dest isa ROCArray ? C_NULL : Int64[strides(dest)...]     # NULL = dense
+    GC.@preserve dest ops prog shape dstrides begin
+        check(ccall((:rk_broadcast_strided, librk[]), Int32,
+                    (Ptr{RkProgram}, Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}),
+                    prog, pointer(dest), rk_dtype(TD), N, shape, dstrides, stream_ptr()))
     end
     return dest
 end
 
 function enable_broadcast!()
-    @eval function Base.copyto!(dest::ROCArray{TD}, bc::Broadcasted{<:ROCArrayStyle}) where {TD}
+    @eval function Base.copyto!(dest::Union{ROCArray{TD},ROCWrapper{TD}}, bc::Broadcasted{<:ROCArrayStyle}) where {TD}
         axes(dest) == axes(bc) || Broadcast.throwdm(axes(dest), axes(bc))
         isempty(dest) && return dest
-        if rk_dtype(TD) !== nothing
+        if rk_dtype(TD) !== nothing && (dest isa ROCArray || is_strided_wrapper(dest))
             try
                 return native_copyto!(dest, bc)
             catch e
