@@ -10,7 +10,8 @@
 //       scan_wave_lines_kernel lines shorter than a tile: one wave per line with a running carry
 //   inner  > 1 : strided lines, lanes run along the contiguous `inner` axis
 //       scan_strided_kernel    4 waves x register tiles of rows, column totals through LDS
-//   scan_thread_kernel         one lane per line (tiny lines / narrow inner)
+//       scan_narrow_kernel     1 < inner < 64 with long lines: tiles of whole rows through LDS
+//   scan_thread_kernel         one lane per line (tiny lines)
 #pragma once
 
 #include "rk_common.hpp"
@@ -372,6 +373,63 @@ __global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict
     }
 }
 
+// ---- 1 < inner < 64 with long lines: tiles of whole rows through LDS ----------------------------------
+// Lanes along `inner` would leave most of a wave idle, and one lane per line (scan_thread_kernel) walks the line
+// alone.  Here a workgroup takes a tile of consecutive rows -- contiguous memory, loaded and stored coalesced --
+// into LDS.  Thread t owns column t % inner and the (t / inner)-th segment of the tile's rows; neighbouring threads
+// touch neighbouring LDS words.  Pass TOTALS: column totals of every tile.  After an exclusive scan of the totals
+// along the tiles (seeded with init) the second pass scans every tile from its carried-in prefix.
+// grid (tiles, outer); totals / carry: [(o * tiles + tile) * inner + column].
+template <typename T> struct NarrowTile { static constexpr int ELEMS = sizeof(T) >= 8 ? 4096 : 8192; };
+
+template <typename In, typename T, typename Op, bool TOTALS>
+__global__ __launch_bounds__(256) void scan_narrow_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, int inclusive, Op op,
+                                                          int64_t rows_per_tile, T* __restrict__ carry) {
+    constexpr int ELEMS = NarrowTile<T>::ELEMS;
+    __shared__ T tile[ELEMS];
+    __shared__ T seg_total[256];
+    const int tid = threadIdx.x;
+    const int inner = (int)g.inner;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_tile;
+    const int nrows = (int)(r0 + rows_per_tile <= g.mid ? rows_per_tile : g.mid - r0);
+    const int count = nrows * inner;
+    const int64_t base = (int64_t)blockIdx.y * g.inner * g.mid + r0 * g.inner;
+    for (int e = tid; e < count; e += 256) tile[e] = (T)in[base + e];
+    __syncthreads();
+    const int nseg = 256 / inner;                                  // segments of rows per column
+    const int c = tid % inner, sgm = tid / inner;
+    const bool active = sgm < nseg;
+    const int seg_rows = (nrows + nseg - 1) / nseg;
+    const int row_lo = sgm * seg_rows, row_hi = row_lo + seg_rows < nrows ? row_lo + seg_rows : nrows;
+    const T ident = Op::template identity<T>();
+    T tot = ident;
+    if (active)
+        for (int r = row_lo; r < row_hi; ++r) tot = op(tot, tile[r * inner + c]);
+    seg_total[tid] = tot;                                          // index sgm * inner + c == tid for active threads
+    __syncthreads();
+    const int64_t slot = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * inner + c;
+    if constexpr (TOTALS) {
+        if (active && sgm == 0) {
+            T t = ident;
+            for (int q = 0; q < nseg; ++q) t = op(t, seg_total[q * inner + c]);
+            carry[slot] = t;
+        }
+    } else {
+        if (active) {
+            T run = carry[slot];
+            for (int q = 0; q < sgm; ++q) run = op(run, seg_total[q * inner + c]);
+            for (int r = row_lo; r < row_hi; ++r) {
+                const T x = tile[r * inner + c];
+                const T nxt = op(run, x);
+                tile[r * inner + c] = inclusive ? nxt : run;
+                run = nxt;
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < count; e += 256) out[base + e] = tile[e];
+    }
+}
+
 // ---- inner >= 64: lanes along `inner`, 4 waves share the rows of a chunk -----------------------------
 // grid (strips, slices, outer).  A workgroup scans the rows [slice * rows_per_slice, +rows_per_slice) of its
 // 64 * VEC columns: a wave keeps R consecutive rows in registers, scans them downwards, and the four waves
@@ -588,6 +646,40 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     return RK_SUCCESS;
 }
 
+// Scan along `mid` for 1 < inner < 64 (see scan_narrow_kernel).  Returns false when the tile totals do not fit the
+// scratch area: the caller then takes another path.
+template <typename In, typename T, typename Op>
+inline int32_t scan_narrow(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, char* scratch, size_t scratch_bytes,
+                           hipStream_t stream, bool* done) {
+    *done = false;
+    const int64_t rows_per_tile = NarrowTile<T>::ELEMS / g.inner;
+    const int64_t tiles = (g.mid + rows_per_tile - 1) / rows_per_tile;
+    if (tiles > 0x7fffffff || g.outer > 65535) return RK_SUCCESS;
+    const size_t need = (size_t)(tiles * g.outer * g.inner) * sizeof(T);
+    const size_t used = (need + 255) & ~(size_t)255;
+    if (scratch == nullptr || used > scratch_bytes) return RK_SUCCESS;
+    T* totals = (T*)scratch;
+    dim3 grid((unsigned)tiles, (unsigned)g.outer);
+    scan_narrow_kernel<In, T, Op, true><<<grid, 256, 0, stream>>>(in, nullptr, g, inclusive, op, rows_per_tile, totals);
+    RK_LAUNCH_CHECK();
+    // exclusive scan of the totals along the tiles, seeded with init: the (inner, tiles, outer) problem again
+    const ScanGeom tg{g.inner, tiles, g.outer};
+    bool sub = false;
+    if (tiles > 32) {                  // a lane per column walking more tiles than this is slower than three small launches
+        const int32_t st = scan_narrow<T, T, Op>(totals, totals, tg, init, 0, op, scratch + used, scratch_bytes - used, stream, &sub);
+        if (st != RK_SUCCESS) return st;
+    }
+    if (!sub) {
+        const int64_t blocks = (g.inner * g.outer + 255) / 256;
+        scan_thread_kernel<T, T, Op, 256><<<(unsigned)blocks, 256, 0, stream>>>(totals, totals, tg, init, 0, op);
+        RK_LAUNCH_CHECK();
+    }
+    scan_narrow_kernel<In, T, Op, false><<<grid, 256, 0, stream>>>(in, out, g, inclusive, op, rows_per_tile, totals);
+    RK_LAUNCH_CHECK();
+    *done = true;
+    return RK_SUCCESS;
+}
+
 template <typename In, typename T, typename Op>
 inline int32_t launch_scan(const ScanArgs& a) {
     const Op op;
@@ -610,6 +702,16 @@ inline int32_t launch_scan(const ScanArgs& a) {
         return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream);
     }
     const int64_t nlines = s.inner * s.outer;
+    if (s.inner > 1 && s.mid > 64) {
+        // narrow inner, long lines: whole-row tiles through LDS (one lane per line would walk each line alone:
+        // 127 ms for accumulate(+, 3 x 1_000_000; dims=2))
+        Workspace w{};
+        if (carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
+            bool done = false;
+            const int32_t st = scan_narrow<In, T, Op>(in, out, g, init, inclusive, op, (char*)w.partials, WS_PARTIALS_BYTES, a.stream, &done);
+            if (st != RK_SUCCESS || done) return st;
+        }
+    }
     if (s.inner > 1 || s.mid <= 16) {
         const int64_t blocks = (nlines + 255) / 256;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;

@@ -197,3 +197,24 @@ def test_unsigned_scans_wrap(rk, orc, dtype):
         with np.errstate(over="ignore"):
             assert np.array_equal(rk.Array(got), np.cumsum(x, axis=dims - 1, dtype=dtype))
         assert np.array_equal(rk.Array(rk.accumulate("max", rk.ROCArray(x), dims=dims)), np.maximum.accumulate(x, axis=dims - 1))
+
+
+NARROW_CASES = [((3, 1_000_000), 2), ((2, 70_001), 2), ((5, 9000, 3), 2), ((17, 33_333), 2), ((63, 20_000), 2), ((7, 3, 40_000), 3),
+                ((3, 5, 9001, 2), 3), ((63, 65), 2), ((2, 2_100_000), 2)]
+
+
+@pytest.mark.parametrize("shape,dims", NARROW_CASES)
+def test_narrow_inner_long_lines(rk, orc, shape, dims):
+    # accumulate(+, 3 x 1_000_000; dims=2) of perf/array.jl:77,84: few columns, very long lines
+    rng = _rng(34)
+    x = rng.integers(-1000, 1000, shape, dtype=np.int32)
+    d = rk.ROCArray(x)
+    assert np.array_equal(rk.Array(rk.accumulate("add", d, dims=dims)), orc.accumulate("add", x, dims=dims))
+    assert np.array_equal(rk.Array(rk.accumulate("max", d, dims=dims, init=5, inclusive=False)),
+                          orc.accumulate("max", x, dims=dims, init=5, inclusive=False))
+    xf = rng.random(shape)
+    np.testing.assert_allclose(rk.Array(rk.cumsum(rk.ROCArray(xf), dims=dims)), orc.cumsum(xf, dims=dims), rtol=1e-11)
+    b = rng.random(shape) < 0.5
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=dims)), orc.cumsum(b, dims=dims))       # Bool -> Int64
+    rk.accumulate_("add", d, d, dims=dims)                                                             # in place
+    assert np.array_equal(rk.Array(d), orc.accumulate("add", x, dims=dims))
