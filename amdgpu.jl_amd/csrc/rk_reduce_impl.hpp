@@ -396,7 +396,7 @@ int tune_reduce_strided_blocks_per_cu();   // rk_api.hip
 int tune_reduce_wave_max_bytes();          // rk_api.hip
 
 template <typename In, typename Acc>
-inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
+inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, size_t cap = WS_PARTIALS_BYTES) {
     ReducePlan p{};
     const int cus = device_info().cus;
     const int64_t target_blocks = (int64_t)cus * tune_reduce_blocks_per_cu();
@@ -419,7 +419,7 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
             const int64_t max_ms = (s.mid + 31) / 32;      // at least 32 rows per workgroup
             if (ms > max_ms) ms = max_ms;
             if (ms > 1024) ms = 1024;
-            const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / (tiles * cols);
+            const int64_t fit = (int64_t)(cap / sizeof(Acc)) / (tiles * cols);
             if (ms > fit) ms = fit;
             if (ms < 1) ms = 1;
         }
@@ -446,7 +446,7 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
     int64_t max_splits = (s.mid + 2 * per_pass - 1) / (2 * per_pass);
     if (want > max_splits) want = max_splits;
     if (want > 4096) want = 4096;
-    const int64_t fit = (int64_t)(WS_PARTIALS_BYTES / sizeof(Acc)) / (2 * nlines);   // partials + group partials
+    const int64_t fit = (int64_t)(cap / sizeof(Acc)) / (2 * nlines);   // partials + group partials
     if (want > fit) want = fit;
     const int64_t groups = (want + TICKET_GROUP - 1) / TICKET_GROUP;
     if (want < 1 || nlines * (groups + 1) > (int64_t)WS_TICKET_COUNT) want = 1;
@@ -457,11 +457,11 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run) {
 
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink>
 inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32_t mask, Xf xf, Op op, Sink sink,
-                             void* ws, size_t ws_bytes, hipStream_t stream) {
+                             void* ws, size_t ws_bytes, hipStream_t stream, size_t cap = WS_PARTIALS_BYTES) {
     const Shape3 s = collapse3(ndim, shape, mask);
-    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run);
+    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap);
     Workspace w{};
-    if (p.payload > WS_PARTIALS_BYTES) return RK_ERR_WORKSPACE;   // the planner never asks for more
+    if (p.payload > cap) return RK_ERR_WORKSPACE;   // the planner never asks for more
     if (p.payload > 0 && !carve_workspace(ws, ws_bytes, 0, &w)) return RK_ERR_WORKSPACE;
     LineGeom g{s.inner, s.mid, s.inner * s.outer};
     constexpr int UNROLL = sizeof(In) >= 4 ? 4 : 2;
@@ -534,9 +534,43 @@ struct FindArgs {
     void* ws; size_t ws_bytes; hipStream_t stream;
 };
 
+// Reduced dims that are not neighbours (dims=(1,3); the (1,2,4) of a batch norm): the generic kernel walks every
+// output's elements with a stride pattern and reaches a tenth of the bandwidth.  Since op is associative and
+// commutative, the lowest run of reduced dims is folded first -- a plain single-run reduction of all the data into
+// a temporary at the top of the partials area -- and the remaining dims are reduced from that much smaller array.
+constexpr size_t REDUCE_TEMP_MAX = WS_PARTIALS_BYTES / 2;
+
 template <typename In, typename Acc, typename Map, typename Op>
 inline int32_t mapreduce_one(const MapreduceArgs& a) {
     ReduceSink<Acc, Op> sink{(Acc*)a.R, a.init ? *(const Acc*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
+    const Shape3 s = collapse3(a.ndim, a.shape, a.mask);
+    if (!s.single_run && s.total > 0) {
+        uint32_t mask1 = 0;                       // the lowest run of reduced dims (extents of 1 do not break a run)
+        int64_t shape1[RK_MAX_DIMS], rest = 1;
+        bool in_run = false, closed = false;
+        for (int d = 0; d < a.ndim; ++d) {
+            shape1[d] = a.shape[d];
+            const bool red = (a.mask >> d) & 1u;
+            if (a.shape[d] == 1) continue;
+            if (red && !closed) { mask1 |= 1u << d; shape1[d] = 1; in_run = true; }
+            else {
+                if (in_run) closed = true;
+                rest *= a.shape[d];
+            }
+        }
+        const size_t temp_bytes = ((size_t)rest * sizeof(Acc) + 255) & ~(size_t)255;
+        Workspace w{};
+        if (mask1 != 0 && temp_bytes <= REDUCE_TEMP_MAX && carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
+            Acc* temp = (Acc*)((char*)w.partials + WS_PARTIALS_BYTES - temp_bytes);
+            const size_t cap = WS_PARTIALS_BYTES - temp_bytes;
+            ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
+            const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, mask1, MapXform<In, Acc, Map>(), Op(), to_temp,
+                                                      a.ws, a.ws_bytes, a.stream, cap);
+            if (st != RK_SUCCESS) return st;
+            return launch_reduce<Acc, Acc>((const Acc*)temp, a.ndim, shape1, a.mask & ~mask1, MapXform<Acc, Acc, MapIdentity>(), Op(), sink,
+                                           a.ws, a.ws_bytes, a.stream, cap);
+        }
+    }
     return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, MapXform<In, Acc, Map>(), Op(), sink,
                                   a.ws, a.ws_bytes, a.stream);
 }
