@@ -373,6 +373,54 @@ __global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict
     }
 }
 
+// ---- short contiguous lines: a group of lanes per line, one 16-byte vector per lane ------------------------------
+// (line length a multiple of the vector and at most 32 vectors, 16-byte aligned).  Lane l of a wave takes vector l of
+// the wave's chunk, so loads and stores are fully coalesced whatever the line length; line = l / L, position = l % L
+// with L vectors per line, and the 64 % L lanes past the last whole line idle.  Each lane scans its vector, the
+// vector totals are scanned over the lanes of the line by shuffles that never cross a line start.  One lane per
+// line with whole vectors reaches 1 TB/s on the same shape, one lane per line with scalars half of that
+// (cumsum of 16 x 1_000_000 Float32 along dim 1: 231 us -> 128 us -> 42 us).
+template <typename In, typename T, typename Op, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int L, int64_t nlines,
+                                                                 T init, int inclusive, Op op) {
+    constexpr int VEC = 16 / sizeof(T), U = 4;
+    typedef typename VecOf<In, VEC>::type VI;
+    typedef typename VecOf<T, VEC>::type VT;
+    const int lane = threadIdx.x & 63;
+    const int lpw = 64 / L;                                  // whole lines per wave and step
+    const int ln = lane / L, pos = lane - ln * L;
+    const int64_t wave_id = (int64_t)blockIdx.x * (BLOCK / 64) + (threadIdx.x >> 6);
+    VI x[U];
+    bool live[U];
+    int64_t vecidx[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t line = (wave_id * U + u) * lpw + ln;
+        live[u] = ln < lpw && line < nlines;
+        vecidx[u] = line * L + pos;
+        x[u] = VI{};
+        if (live[u]) x[u] = load_nt((const VI*)in + vecidx[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        T loc[VEC];
+        loc[0] = (T)x[u][0];
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) loc[j] = op(loc[j - 1], (T)x[u][j]);
+        T tot = loc[VEC - 1];
+        for (int d = 1; d < L; d <<= 1) {
+            const T v = __shfl_up(tot, d, 64);
+            if (pos >= d) tot = op(v, tot);
+        }
+        const T prev = __shfl_up(tot, 1, 64);
+        const T base = pos > 0 ? op(init, prev) : init;
+        VT o;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = inclusive ? op(base, loc[j]) : (j == 0 ? base : op(base, loc[j > 0 ? j - 1 : 0]));
+        if (live[u]) store_nt((VT*)out + vecidx[u], o);
+    }
+}
+
 // ---- 1 < inner < 64 with long lines: tiles of whole rows through LDS ----------------------------------
 // Lanes along `inner` would leave most of a wave idle, and one lane per line (scan_thread_kernel) walks the line
 // alone.  Here a workgroup takes a tile of consecutive rows -- contiguous memory, loaded and stored coalesced --
@@ -711,6 +759,15 @@ inline int32_t launch_scan(const ScanArgs& a) {
             const int32_t st = scan_narrow<In, T, Op>(in, out, g, init, inclusive, op, (char*)w.partials, WS_PARTIALS_BYTES, a.stream, &done);
             if (st != RK_SUCCESS || done) return st;
         }
+    }
+    if (s.inner == 1 && s.mid % VEC == 0 && s.mid / VEC <= 32 && aligned) {
+        const int L = (int)(s.mid / VEC);
+        const int64_t per_block = (int64_t)4 * 4 * (64 / L);            // waves x steps x lines per wave and step
+        const int64_t blocks = (nlines + per_block - 1) / per_block;
+        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+        scan_short_lines_kernel<In, T, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, L, nlines, init, inclusive, op);
+        RK_LAUNCH_CHECK();
+        return RK_SUCCESS;
     }
     if (s.inner > 1 || s.mid <= 16) {
         const int64_t blocks = (nlines + 255) / 256;

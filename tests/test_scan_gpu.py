@@ -218,3 +218,19 @@ def test_narrow_inner_long_lines(rk, orc, shape, dims):
     assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=dims)), orc.cumsum(b, dims=dims))       # Bool -> Int64
     rk.accumulate_("add", d, d, dims=dims)                                                             # in place
     assert np.array_equal(rk.Array(d), orc.accumulate("add", x, dims=dims))
+
+
+@pytest.mark.parametrize("shape", [(16, 100_000), (4, 50_001), (8, 3, 7000), (12, 1000), (2, 100_000), (16, 1), (6, 999), (20, 3001), (128, 500), (100, 777), (64, 1000), (36, 5, 41)])
+def test_short_contiguous_lines(rk, orc, shape):
+    rng = _rng(35)
+    for dtype in (np.float32, np.float64, np.int32, np.int64):
+        x = (rng.standard_normal(shape) * 100).astype(dtype)
+        got = rk.Array(rk.accumulate("add", rk.ROCArray(x), dims=1, init=3, inclusive=False))
+        want = orc.accumulate("add", x, dims=1, init=3, inclusive=False)
+        if np.dtype(dtype).kind == "f":
+            np.testing.assert_allclose(got, want, rtol=RTOL if dtype == np.float32 else 1e-12, atol=1e-3 if dtype == np.float32 else 1e-9)
+        else:
+            assert np.array_equal(got, want)
+        assert np.array_equal(rk.Array(rk.accumulate("max", rk.ROCArray(x), dims=1)), orc.accumulate("max", x, dims=1))
+    b = rng.random(shape) < 0.5
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=1)), orc.cumsum(b, dims=1))
