@@ -12,7 +12,8 @@ from .mapreduce import (mapreduce, mapreducedim_, sum, prod, maximum, minimum, c
                         add_sum, mul_prod, add, mul, max_, min_)
 from .accumulate import accumulate, accumulate_, cumsum, cumprod, accumulate_eltype    # noqa: F401
 from . import broadcast                                                               # noqa: F401
-from .broadcast import lazy, materialize, materialize_, fill_, Broadcasted             # noqa: F401
+from .broadcast import (lazy, materialize, materialize_, fill_, Broadcasted,            # noqa: F401
+                        isodd, iseven, isnan, ifelse)
 from .views import ROCView, view, transpose, PermutedDimsArray                         # noqa: F401
 from .volumerhs import volumerhs_                                                     # noqa: F401
 from .indexing import findall, getindex_mask                                                         # noqa: F401

@@ -35,6 +35,7 @@ RK_ERR_TOO_LARGE = 10005
 RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16 = range(9)
 # rk_map
 RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
+RK_MAP_MAX_TOKENS, RK_MAP_MAX_CONSTS = 16, 4
 # rk_op
 RK_OP_ADD, RK_OP_MUL, RK_OP_MAX, RK_OP_MIN = range(4)
 # rk_opkind
@@ -43,6 +44,9 @@ RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE, RK_KIND_FINDALL = ran
 (RK_BC_ADD, RK_BC_SUB, RK_BC_MUL, RK_BC_DIV, RK_BC_MAX, RK_BC_MIN, RK_BC_POW, RK_BC_FMA) = range(32, 40)
 (RK_BC_NEG, RK_BC_ABS, RK_BC_ABS2, RK_BC_SQRT, RK_BC_EXP, RK_BC_LOG, RK_BC_SIN, RK_BC_COS, RK_BC_TANH,
  RK_BC_INV, RK_BC_IDENTITY) = range(64, 75)
+(RK_BC_LT, RK_BC_LE, RK_BC_GT, RK_BC_GE, RK_BC_EQ, RK_BC_NE, RK_BC_AND, RK_BC_OR) = range(96, 104)
+RK_BC_IFELSE = 112
+(RK_BC_NOT, RK_BC_ISODD, RK_BC_ISEVEN, RK_BC_ISNAN, RK_BC_WRAP_I32, RK_BC_WRAP_U32) = range(128, 134)
 
 
 class RkOperand(C.Structure):
@@ -69,6 +73,16 @@ class RkProgram(C.Structure):
     ]
 
 
+class RkMapProgram(C.Structure):
+    _fields_ = [
+        ("n_tokens", C.c_int32),
+        ("tokens", C.c_int32 * RK_MAP_MAX_TOKENS),
+        ("n_consts", C.c_int32),
+        ("const_f", C.c_double * RK_MAP_MAX_CONSTS),
+        ("const_i", C.c_int64 * RK_MAP_MAX_CONSTS),
+    ]
+
+
 _I64P = C.POINTER(C.c_int64)
 
 PROTOTYPES = {
@@ -78,6 +92,8 @@ PROTOTYPES = {
     "rk_workspace_init": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_mapreduce_program": (C.c_int32, [C.POINTER(RkMapProgram), C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
+                                         C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_findminmax": (C.c_int32, [C.c_int32, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_accumulate": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,

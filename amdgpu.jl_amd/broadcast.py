@@ -13,6 +13,8 @@ are Float64 and Python ints Int64, as in Julia.
 """
 from __future__ import annotations
 
+import builtins
+
 import numpy as np
 
 from . import _lib as L
@@ -26,6 +28,10 @@ _BINARY = {"+": L.RK_BC_ADD, "-": L.RK_BC_SUB, "*": L.RK_BC_MUL, "/": L.RK_BC_DI
 _UNARY = {"neg": L.RK_BC_NEG, "abs": L.RK_BC_ABS, "abs2": L.RK_BC_ABS2, "sqrt": L.RK_BC_SQRT, "exp": L.RK_BC_EXP,
           "log": L.RK_BC_LOG, "sin": L.RK_BC_SIN, "cos": L.RK_BC_COS, "tanh": L.RK_BC_TANH, "inv": L.RK_BC_INV,
           "identity": L.RK_BC_IDENTITY}
+_COMPARE = {"<": L.RK_BC_LT, "<=": L.RK_BC_LE, ">": L.RK_BC_GT, ">=": L.RK_BC_GE, "==": L.RK_BC_EQ, "!=": L.RK_BC_NE}
+_LOGIC = {"&": L.RK_BC_AND, "|": L.RK_BC_OR}
+_PREDICATE = {"!": L.RK_BC_NOT, "isodd": L.RK_BC_ISODD, "iseven": L.RK_BC_ISEVEN, "isnan": L.RK_BC_ISNAN}
+_MATH = ("sqrt", "exp", "log", "sin", "cos", "tanh", "inv")
 
 
 class Broadcasted:
@@ -51,6 +57,19 @@ class Broadcasted:
     def __rtruediv__(self, o): return Broadcasted("/", (_leaf(o), self))
     def __pow__(self, o): return Broadcasted("^", (self, _leaf(o)))
     def __neg__(self): return Broadcasted("neg", (self,))
+    # comparisons and logic (.<  .==  .&  .!): Bool-valued nodes
+    def __lt__(self, o): return Broadcasted("<", (self, _leaf(o)))
+    def __le__(self, o): return Broadcasted("<=", (self, _leaf(o)))
+    def __gt__(self, o): return Broadcasted(">", (self, _leaf(o)))
+    def __ge__(self, o): return Broadcasted(">=", (self, _leaf(o)))
+    def __eq__(self, o): return Broadcasted("==", (self, _leaf(o)))
+    def __ne__(self, o): return Broadcasted("!=", (self, _leaf(o)))
+    __hash__ = object.__hash__
+    def __and__(self, o): return Broadcasted("&", (self, _leaf(o)))
+    def __rand__(self, o): return Broadcasted("&", (_leaf(o), self))
+    def __or__(self, o): return Broadcasted("|", (self, _leaf(o)))
+    def __ror__(self, o): return Broadcasted("|", (_leaf(o), self))
+    def __invert__(self): return Broadcasted("!", (self,))
 
 
 def _leaf(x):
@@ -68,7 +87,9 @@ def broadcasted(f: str, *args) -> Broadcasted:
     """``Broadcast.broadcasted(f, args...)`` for an enumerated ``f``."""
     if f == "muladd":
         return Broadcasted("muladd", tuple(_leaf(a) for a in args))
-    if f not in _BINARY and f not in _UNARY:
+    if f == "ifelse":
+        return ifelse(*args)
+    if f not in _BINARY and f not in _UNARY and f not in _COMPARE and f not in _LOGIC and f not in _PREDICATE:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"broadcast function {f!r}")
     return Broadcasted(f, tuple(_leaf(a) for a in args))
 
@@ -84,6 +105,10 @@ exp, log, sin, cos, tanh, sqrt, abs_, abs2, inv = (_unary(n) for n in
                                                     ("exp", "log", "sin", "cos", "tanh", "sqrt", "abs", "abs2", "inv"))
 
 
+isodd, iseven, isnan, not_ = (_unary(n) for n in ("isodd", "iseven", "isnan", "!"))
+
+
+def ifelse(c, a, b): return Broadcasted("ifelse", (_leaf(c), _leaf(a), _leaf(b)))
 def max_(a, b): return Broadcasted("max", (_leaf(a), _leaf(b)))
 def min_(a, b): return Broadcasted("min", (_leaf(a), _leaf(b)))
 def muladd(a, b, c): return Broadcasted("muladd", (_leaf(a), _leaf(b), _leaf(c)))
@@ -117,7 +142,65 @@ def broadcast_shape(*shapes):
     return tuple(out)
 
 
-def _flatten(bc: Broadcasted, operands: list, tokens: list):
+class MapVar:
+    """Stands for the element in ``mapreduce(f, op, A)``: ``f(lazy(MapVar(eltype)))`` traces f into a tree."""
+    __slots__ = ("dtype",)
+
+    def __init__(self, dtype):
+        self.dtype = np.dtype(dtype)
+
+
+def _leaf_dtype(o) -> np.dtype:
+    return o.dtype if isinstance(o, _ARRAYS + (MapVar,)) else _scalar_dtype(o)
+
+
+def promote_type(a, b) -> np.dtype:
+    """Julia's ``promote_type`` on the element types in use here: a float beats any integer and the wider float
+    wins; Bool yields to integers; the wider integer wins, the unsigned one at equal width."""
+    a, b = np.dtype(a), np.dtype(b)
+    if a == b:
+        return a
+    if a.kind == "f" or b.kind == "f":
+        return max((d for d in (a, b) if d.kind == "f"), key=lambda d: d.itemsize)
+    if a.kind == "b":
+        return b
+    if b.kind == "b":
+        return a
+    if a.itemsize != b.itemsize:
+        return a if a.itemsize > b.itemsize else b
+    return a if a.kind == "u" else b
+
+
+def _infer(bc: Broadcasted, types: dict) -> np.dtype:
+    """Julia's result eltype of every node of the tree (``Broadcast.combine_eltypes``), by node identity."""
+    if bc.f is None:
+        t = _leaf_dtype(bc.args[0])
+    else:
+        ats = [_infer(a, types) for a in bc.args]
+        t = ats[0]
+        for u in ats[1:]:
+            t = promote_type(t, u)
+        if bc.f in _COMPARE or bc.f in _LOGIC or bc.f in _PREDICATE:
+            if bc.f in ("isodd", "iseven") and ats[0].kind == "f":
+                raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"{bc.f} of floating-point values")
+            t = np.dtype(np.bool_)
+        elif bc.f == "ifelse":
+            t = promote_type(ats[1], ats[2])
+        elif bc.f in ("/", "^") or bc.f in _MATH:
+            if t.kind != "f":
+                t = np.dtype(np.float64)               # Int / Int and sqrt(Int) are Float64
+        elif bc.f in ("+", "-", "*", "muladd", "neg") and t.kind == "b":
+            t = np.dtype(np.int64)                     # true + true isa Int
+    if t.kind not in "fiub":
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"broadcast over eltype {t}")
+    types[id(bc)] = t
+    return t
+
+
+_ORDER_SENSITIVE = set(_COMPARE) | set(_LOGIC) | {"!", "max", "min"}
+
+
+def _emit(bc: Broadcasted, operands: list, tokens: list, types: dict, int_program: bool):
     if bc.f is None:
         leaf = bc.args[0]
         for k, o in enumerate(operands):           # the same array object appears once
@@ -130,54 +213,85 @@ def _flatten(bc: Broadcasted, operands: list, tokens: list):
         tokens.append(len(operands) - 1)
         return
     for a in bc.args:
-        _flatten(a, operands, tokens)
+        _emit(a, operands, tokens, types, int_program)
+        # integer programs compute in Int64: where the order or the zero-ness of a 32-bit intermediate matters,
+        # bring it back to the value Julia holds (Int32 arithmetic wraps)
+        if int_program and bc.f in _ORDER_SENSITIVE and a.f is not None:
+            _wrap(types[id(a)], tokens)
     if bc.f == "muladd":
         tokens.append(L.RK_BC_FMA)
-    elif bc.f in _BINARY:
-        tokens.append(_BINARY[bc.f])
+    elif bc.f == "ifelse":
+        tokens.append(L.RK_BC_IFELSE)
     else:
-        tokens.append(_UNARY[bc.f])
+        for table in (_BINARY, _UNARY, _COMPARE, _LOGIC, _PREDICATE):
+            if bc.f in table:
+                tokens.append(table[bc.f])
+                break
 
 
-_INT_SAFE = None
+def _wrap(t: np.dtype, tokens: list):
+    if t == np.int32:
+        tokens.append(L.RK_BC_WRAP_I32)
+    elif t == np.uint32:
+        tokens.append(L.RK_BC_WRAP_U32)
 
 
-def _int_safe_tokens():
-    global _INT_SAFE
-    if _INT_SAFE is None:
-        _INT_SAFE = {L.RK_BC_ADD, L.RK_BC_SUB, L.RK_BC_MUL, L.RK_BC_MAX, L.RK_BC_MIN, L.RK_BC_FMA,
-                     L.RK_BC_NEG, L.RK_BC_ABS, L.RK_BC_ABS2, L.RK_BC_IDENTITY}
-    return _INT_SAFE
+def _compile_tree(tree: Broadcasted, operands: list):
+    """Type the tree and flatten it after the operands already listed; returns (tokens, compute type, result eltype).
+    Floating-point programs compute in the promoted float type.  All-integer programs compute in Int64 and keep
+    Julia's result eltype (Int32 .+ Int32 is an Int32 that wraps); with ``/`` or a math function Julia's result is
+    a Float64, and so is the compute type here."""
+    types: dict = {}
+    eltype = _infer(tree, types)
+    kinds = list(types.values())
+    floats = [t for t in kinds if t.kind == "f"]
+    if floats:
+        compute = max(floats, key=lambda d: d.itemsize)
+        if compute == np.float16:
+            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "Float16 broadcast")
+    else:
+        compute = np.dtype(np.int64)
+    tokens: list = []
+    _emit(tree, operands, tokens, types, not floats)
+    if not floats:
+        # an order-sensitive token over UInt64 values cannot be computed in Int64
+        def visit(n):
+            if n.f in _ORDER_SENSITIVE and builtins.any(types[id(a)] == np.uint64 for a in n.args):
+                raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"{n.f} of UInt64 values")
+            if n.f is not None:
+                for a in n.args:
+                    visit(a)
+        visit(tree)
+    return tokens, compute, eltype, types
 
 
 def _compile(bc: Broadcasted):
-    """Flatten ``bc``; returns (operands, tokens, compute type, shape, result eltype).  Floating-point programs compute
-    in the promoted float type.  All-integer programs of ``+ - * max min muladd - abs abs2`` compute in Int64 and keep
-    Julia's result eltype (Int32 .+ Int32 is an Int32 that wraps); with ``/`` or a math function Julia's result is a
-    Float64, and so is the compute type here."""
-    operands, tokens = [], []
-    _flatten(_leaf(bc), operands, tokens)
+    """Flatten ``bc``; returns (operands, tokens, compute type, shape, result eltype)."""
+    operands: list = []
+    tokens, compute, eltype, _ = _compile_tree(_leaf(bc), operands)
     if len(tokens) > L.RK_MAX_PROGRAM:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "broadcast expression too long")
-    dts = [o.dtype if isinstance(o, _ARRAYS) else _scalar_dtype(o) for o in operands]
-    eltype = np.result_type(*dts) if dts else np.dtype(np.float64)
-    compute = eltype
-    ops = [t for t in tokens if t >= L.RK_MAX_OPERANDS]
-    if eltype.kind != "f":
-        if eltype.kind not in "iub":
-            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"broadcast over eltype {eltype}")
-        if all(t in _int_safe_tokens() for t in ops):
-            if eltype == np.uint64 and any(t in (L.RK_BC_MAX, L.RK_BC_MIN) for t in ops):
-                raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "max / min of UInt64 values")
-            compute = np.dtype(np.int64)
-            if eltype == np.bool_ and ops:             # true + true isa Int
-                eltype = np.dtype(np.int64)
-        else:
-            compute = eltype = np.dtype(np.float64)
-    if compute == np.float16:
-        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "Float16 broadcast")
     shapes = [o.dims for o in operands if isinstance(o, _ARRAYS)]
     return operands, tokens, compute, broadcast_shape(*shapes), eltype
+
+
+def compile_map(f, dtype):
+    """Trace the unary closure ``f`` of ``mapreduce(f, op, A)`` on a symbolic element: returns
+    (tokens, constants, Julia's eltype of f(x), compute type).  Token 0 is the element, tokens 1.. the constants;
+    a closure that captures an array, needs more than RK_MAP_MAX_CONSTS constants, RK_MAP_MAX_TOKENS tokens or a
+    deeper value stack than the kernels keep in registers is unsupported."""
+    var = MapVar(dtype)
+    tree = _leaf(f(lazy(var)))
+    operands: list = [var]
+    tokens, compute, eltype, types = _compile_tree(tree, operands)
+    consts = operands[1:]
+    if builtins.any(isinstance(c, _ARRAYS + (MapVar,)) for c in consts):
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "mapreduce closure over an array")
+    if compute.kind != "f" and tree.f is not None:
+        _wrap(eltype, tokens)                          # the reduction sees the Int32 Julia would hand it
+    if len(tokens) > L.RK_MAP_MAX_TOKENS or len(consts) > L.RK_MAP_MAX_CONSTS:
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "mapreduce closure too long")
+    return tokens, consts, eltype, compute
 
 
 def _program(operands, tokens, compute, dest_ndim) -> L.RkProgram:

@@ -157,7 +157,7 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
     if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91
     if (A == nullptr || R == nullptr) return RK_ERR_INVALID_ARGUMENT;
     reduce_mask &= (1u << ndim) - 1u;       // dims beyond ndim reduce nothing
-    MapreduceArgs a{(int)f, (int)op, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream};
+    MapreduceArgs a{(int)f, (int)op, nullptr, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream};
     if (in == out) {
         switch (in) {
             case RK_F32: return mapreduce_f32(a);
@@ -173,6 +173,34 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
     if (in == RK_I32 && out == RK_I64) return mapreduce_i32_i64(a);
     if (in == RK_U8 && (out == RK_I64 || out == RK_U64)) return mapreduce_u8_i64(a);   // sums of bytes: the same bits either way
     if (in == RK_U32 && out == RK_U64) return mapreduce_u32_u64(a);
+    return RK_ERR_UNSUPPORTED;
+}
+
+int32_t rk_mapreduce_program(const rk_map_program* f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim,
+                             const int64_t* shape, uint32_t reduce_mask, void* R, const void* init, void* ws, size_t ws_bytes,
+                             void* stream) {
+    int64_t total = 0;
+    if (f == nullptr || !valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
+    if (f->n_tokens < 1 || f->n_tokens > RK_MAP_MAX_TOKENS || f->n_consts < 0 || f->n_consts > RK_MAP_MAX_CONSTS) return RK_ERR_INVALID_ARGUMENT;
+    const bool int_compute = in != RK_F32 && in != RK_F64;
+    {   // operand 0 = the element, 1 .. n_consts = the constants; the value stack stays in registers
+        const int32_t st = validate_tokens(f->tokens, f->n_tokens, 1 + f->n_consts, int_compute, INTERP_REG_DEPTH);
+        if (st != RK_SUCCESS) return st;
+    }
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91
+    if (A == nullptr || R == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    reduce_mask &= (1u << ndim) - 1u;
+    MapreduceArgs a{RK_MAP_PROGRAM, (int)op, f, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream};
+    if (in == RK_F32 && out == RK_F32) return mapreduce_prog_f32(a);
+    if (in == RK_F32 && out == RK_I64) return mapreduce_prog_f32_i64(a);
+    if (in == RK_F64 && out == RK_F64) return mapreduce_prog_f64(a);
+    if (in == RK_F64 && out == RK_I64) return mapreduce_prog_f64_i64(a);
+    if (in == RK_I32 && out == RK_I32) return mapreduce_prog_i32(a);
+    if (in == RK_I32 && out == RK_I64) return mapreduce_prog_i32_i64(a);
+    if (in == RK_I64 && out == RK_I64) return mapreduce_prog_i64(a);
+    if (in == RK_U8 && out == RK_I64) return mapreduce_prog_u8_i64(a);
     return RK_ERR_UNSUPPORTED;
 }
 

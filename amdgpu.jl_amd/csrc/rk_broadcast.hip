@@ -15,6 +15,7 @@
 #include <cstring>
 
 #include "rk_common.hpp"
+#include "rk_interp.hpp"
 
 #pragma clang fp contract(off)
 
@@ -131,88 +132,20 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
 }
 
 // ---- evaluators ---------------------------------------------------------------------------------------
-// Postfix interpreter.  The program is the same for every lane, so every token is one scalar branch (a switch
-// outside the per-component loops: inside them the compiler turns it into selects that evaluate exp, log, sin ...
-// for every element).  The four topmost stack entries live in registers and move by one place on push / pop;
-// deeper entries (rare) spill to LDS: entry e of thread t, component j at lds[(e * VEC + j) * BLOCK + t].
-constexpr int BC_REG_DEPTH = 4;
+// Postfix interpreter (rk_interp.hpp) over the loaded operands.
+template <typename CT, int VEC> struct BcFetch {
+    const CT (&in)[RK_MAX_OPERANDS][VEC];
+    template <int K> __device__ __forceinline__ void get(CT (&v)[VEC]) const {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = in[K][j];
+    }
+};
 struct EvalInterp {
     static constexpr int NOPS = RK_MAX_OPERANDS;   // load what the program declares
     static constexpr bool USES_LDS = true;
     template <typename CT, int VEC>
     static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
-        const int t = threadIdx.x;
-        CT s0[VEC], s1[VEC], s2[VEC], s3[VEC];     // s0 = top of the stack
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) s0[j] = s1[j] = s2[j] = s3[j] = CT(0);
-        int depth = 0;
-        auto push = [&](const CT (&v)[VEC]) {
-            if (depth >= BC_REG_DEPTH) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) lds[((depth - BC_REG_DEPTH) * VEC + j) * BC_BLOCK + t] = s3[j];
-            }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) { s3[j] = s2[j]; s2[j] = s1[j]; s1[j] = s0[j]; s0[j] = v[j]; }
-            ++depth;
-        };
-        auto drop_second = [&]() {                 // the entry under the top has been consumed
-            --depth;
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) { s1[j] = s2[j]; s2[j] = s3[j]; }
-            if (depth >= BC_REG_DEPTH) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) s3[j] = lds[((depth - BC_REG_DEPTH) * VEC + j) * BC_BLOCK + t];
-            }
-        };
-#define RK_BC_UN(EXPR)  { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = s0[j]; s0[j] = (EXPR); } } break
-#define RK_BC_BIN(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = s1[j], y = s0[j]; s0[j] = (EXPR); } drop_second(); } break
-        for (int i = 0; i < a.n_tokens; ++i) {
-            const int tok = a.tokens[i];
-            switch (tok) {
-                case 0: push(in[0]); break;
-                case 1: push(in[1]); break;
-                case 2: push(in[2]); break;
-                case 3: push(in[3]); break;
-                case 4: push(in[4]); break;
-                case 5: push(in[5]); break;
-                case 6: push(in[6]); break;
-                case 7: push(in[7]); break;
-                case RK_BC_ADD: RK_BC_BIN(x + y);
-                case RK_BC_SUB: RK_BC_BIN(x - y);
-                case RK_BC_MUL: RK_BC_BIN(x * y);
-                case RK_BC_MAX: RK_BC_BIN(OpMax()(x, y));
-                case RK_BC_MIN: RK_BC_BIN(OpMin()(x, y));
-                case RK_BC_FMA: {                   // x * y + top with x the deepest of the three
-#pragma unroll
-                    for (int j = 0; j < VEC; ++j) s0[j] = s2[j] * s1[j] + s0[j];
-                    drop_second();
-                    drop_second();
-                } break;
-                case RK_BC_NEG: RK_BC_UN(-x);
-                case RK_BC_ABS: RK_BC_UN(x < CT(0) ? -x : (x == CT(0) ? CT(0) : x));
-                case RK_BC_ABS2: RK_BC_UN(x * x);
-                default:                            // RK_BC_IDENTITY, or a token of the floating-point programs
-                    if constexpr (std::is_floating_point<CT>::value) {
-                        switch (tok) {
-                            case RK_BC_DIV: RK_BC_BIN(x / y);
-                            case RK_BC_POW: RK_BC_BIN(pow(x, y));
-                            case RK_BC_SQRT: RK_BC_UN(sqrt(x));
-                            case RK_BC_EXP: RK_BC_UN(exp(x));
-                            case RK_BC_LOG: RK_BC_UN(log(x));
-                            case RK_BC_SIN: RK_BC_UN(sin(x));
-                            case RK_BC_COS: RK_BC_UN(cos(x));
-                            case RK_BC_TANH: RK_BC_UN(tanh(x));
-                            case RK_BC_INV: RK_BC_UN(CT(1) / x);
-                            default: break;
-                        }
-                    }
-                    break;
-            }
-        }
-#undef RK_BC_UN
-#undef RK_BC_BIN
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) out[j] = s0[j];
+        interp_run<CT, VEC, BC_BLOCK>(a.tokens, a.n_tokens, BcFetch<CT, VEC>{in}, out, lds);
     }
 };
 
@@ -370,7 +303,7 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
         if (a.nxb > 0x7fffffff || gz > 65535) return RK_ERR_TOO_LARGE;
         grid = dim3((unsigned)a.nxb, (unsigned)gy, (unsigned)gz);
     }
-    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - BC_REG_DEPTH) * VECN * BC_BLOCK * sizeof(CT) : 0;
+    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - INTERP_REG_DEPTH) * VECN * BC_BLOCK * sizeof(CT) : 0;
     // homogeneous element types: a kernel without any dispatch on the element type
     bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : (std::is_same<CT, double>::value ? RK_F64 : RK_I64));
     for (int k = 0; k < a.n_operands; ++k)
@@ -421,28 +354,10 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
     if (prog->n_operands < 0 || prog->n_operands > RK_MAX_OPERANDS) return RK_ERR_INVALID_ARGUMENT;
     if (prog->n_tokens < 1 || prog->n_tokens > RK_MAX_PROGRAM) return RK_ERR_INVALID_ARGUMENT;
 
-    // the program must be a well-formed postfix expression that leaves exactly one value
-    int depth = 0, max_depth = 0;
-    for (int i = 0; i < prog->n_tokens; ++i) {
-        const int tok = prog->tokens[i];
-        if (tok >= 0 && tok < RK_MAX_OPERANDS) {
-            if (tok >= prog->n_operands) return RK_ERR_INVALID_ARGUMENT;
-            ++depth;
-        } else if (tok >= RK_BC_ADD && tok <= RK_BC_POW) {
-            if (depth < 2) return RK_ERR_INVALID_ARGUMENT;
-            if (int_compute && (tok == RK_BC_DIV || tok == RK_BC_POW)) return RK_ERR_UNSUPPORTED;   // Julia: Int / Int is a Float64
-            --depth;
-        } else if (tok == RK_BC_FMA) {
-            if (depth < 3) return RK_ERR_INVALID_ARGUMENT;
-            depth -= 2;
-        } else if (tok >= RK_BC_NEG && tok <= RK_BC_IDENTITY) {
-            if (depth < 1) return RK_ERR_INVALID_ARGUMENT;
-            if (int_compute && tok != RK_BC_NEG && tok != RK_BC_ABS && tok != RK_BC_ABS2 && tok != RK_BC_IDENTITY) return RK_ERR_UNSUPPORTED;
-        } else return RK_ERR_INVALID_ARGUMENT;
-        if (depth > max_depth) max_depth = depth;
+    {
+        const int32_t st = validate_tokens(prog->tokens, prog->n_tokens, prog->n_operands, int_compute, BC_MAX_DEPTH);
+        if (st != RK_SUCCESS) return st;
     }
-    if (depth != 1) return RK_ERR_INVALID_ARGUMENT;
-    if (max_depth > BC_MAX_DEPTH) return RK_ERR_UNSUPPORTED;
 
     int64_t total = 1;
     for (int d = 0; d < ndim; ++d) {

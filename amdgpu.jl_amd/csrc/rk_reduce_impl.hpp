@@ -19,6 +19,7 @@
 #pragma once
 
 #include "rk_common.hpp"
+#include "rk_interp.hpp"
 
 namespace rk {
 
@@ -47,6 +48,57 @@ template <typename T, typename P, bool WANT_MAX> struct ArgXform {
     typedef ArgAcc<T, P> A;
     __device__ __forceinline__ A operator()(T x, P pos) const { A p; p.k = OrderKey<T>::make(x, WANT_MAX); p.i = pos; return p; }
 };
+
+// f given as a postfix program over the element (operand token 0) and up to RK_MAP_MAX_CONSTS constants (tokens
+// 1 ..): mapreduce(x -> x + 1, +, A), count(isodd, A).  Floating-point elements compute in their own type, integers
+// in Int64 (the program wraps to 32 bits itself where Julia's value would).  The interpreter costs one scalar
+// branch per token, so the kernels hand it the values of one or two vector loads at a time (`batch`).
+struct PackedTokens {                        // 16 tokens of 8 bits in two scalar registers: no memory behind tokens[i]
+    uint64_t lo, hi;
+    __device__ __forceinline__ int operator[](int i) const { return (int)(((i < 8 ? lo : hi) >> ((i & 7) * 8)) & 0xffu); }
+};
+template <typename In, typename Acc> struct ProgXform {
+    typedef int64_t Pos;
+    typedef typename std::conditional<std::is_floating_point<In>::value, In, int64_t>::type CT;
+    static constexpr int CHUNK = 32 / sizeof(CT);        // components per interpreter run: 8 Float32, 4 Float64 / Int64
+    PackedTokens tokens;
+    int32_t n_tokens;
+    CT c[RK_MAP_MAX_CONSTS];
+    template <int N> struct Fetch {
+        const In* x;
+        const CT (&c)[RK_MAP_MAX_CONSTS];
+        template <int K> __device__ __forceinline__ void get(CT (&v)[N]) const {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                if constexpr (K == 0) v[j] = (CT)x[j];
+                else if constexpr (K <= RK_MAP_MAX_CONSTS) v[j] = c[K - 1];
+                else v[j] = CT(0);
+            }
+        }
+    };
+    template <int N> __device__ __forceinline__ void batch(const In* x, Acc* y) const {
+        CT out[N];
+        interp_run<CT, N, 0>(tokens, n_tokens, Fetch<N>{x, c}, out, (CT*)nullptr);
+#pragma unroll
+        for (int j = 0; j < N; ++j) y[j] = (Acc)out[j];
+    }
+    __device__ __forceinline__ Acc operator()(In x, int64_t) const {
+        Acc y;
+        batch<1>(&x, &y);
+        return y;
+    }
+};
+template <typename Xf> struct XfIsBatch : std::false_type {};
+template <typename In, typename Acc> struct XfIsBatch<ProgXform<In, Acc>> : std::true_type {};
+
+// m[i] = xf(x[i]) for TOTAL loaded values, CHUNK at a time
+template <int TOTAL, typename In, typename Acc, typename Xf>
+__device__ __forceinline__ void map_batch(const In (&x)[TOTAL], Acc (&m)[TOTAL], const Xf& xf) {
+    constexpr int C = TOTAL < Xf::CHUNK ? TOTAL : Xf::CHUNK;
+    static_assert(TOTAL % C == 0, "loaded values split into whole chunks");
+#pragma unroll
+    for (int c0 = 0; c0 < TOTAL; c0 += C) xf.template batch<C>(&x[c0], &m[c0]);
+}
 
 // ---- result sinks ---------------------------------------------------------------------------
 // Called as sink(output index q, reduced value).
@@ -108,18 +160,42 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
             const int64_t i0 = c * CHUNK + t;
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) v[u] = load_nt(pv + i0 + (int64_t)u * GROUP);
+            if constexpr (XfIsBatch<Xf>::value) {
+                In x[UNROLL * VEC];
+                Acc m[UNROLL * VEC];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const Pos e0 = (Pos)(head + (i0 + (int64_t)u * GROUP) * VEC);
+                for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], (Pos)(e0 + j)));
+                    for (int j = 0; j < VEC; ++j) x[u * VEC + j] = v[u][j];
+                map_batch<UNROLL * VEC>(x, m, xf);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], m[u * VEC + j]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const Pos e0 = (Pos)(head + (i0 + (int64_t)u * GROUP) * VEC);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], (Pos)(e0 + j)));
+                }
             }
         }
         for (int64_t i = nchunks * CHUNK + (int64_t)s * GROUP + t; i < nvec; i += (int64_t)splits * GROUP) {
             const V v = load_nt(pv + i);
             const Pos e0 = (Pos)(head + i * VEC);
+            if constexpr (XfIsBatch<Xf>::value) {
+                In x[VEC];
+                Acc m[VEC];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], (Pos)(e0 + j)));
+                for (int j = 0; j < VEC; ++j) x[j] = v[j];
+                map_batch<VEC>(x, m, xf);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], m[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], (Pos)(e0 + j)));
+            }
         }
         Acc a = edge;
 #pragma unroll
@@ -135,8 +211,15 @@ __device__ __forceinline__ Acc accumulate_line(const In* __restrict__ A, int64_t
             In v[UNROLL];
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) v[u] = A[base + (k + u * step) * stride];
+            if constexpr (XfIsBatch<Xf>::value) {
+                Acc m[UNROLL];
+                map_batch<UNROLL>(v, m, xf);
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], (Pos)(k + u * step)));
+                for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], m[u]);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], (Pos)(k + u * step)));
+            }
         }
         for (; k < n; k += step) acc[0] = acc_step(op, acc[0], xf(A[base + k * stride], (Pos)k));
         Acc a = acc[0];
@@ -263,13 +346,31 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
             if (m + (UNROLL - 1) * NW < g.mid) {
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(p + (m + u * NW) * g.inner));
+                if constexpr (XfIsBatch<Xf>::value) {
+                    In x[UNROLL * VEC];
+                    Acc y[UNROLL * VEC];
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
-                    if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
-                    else {
+                    for (int u = 0; u < UNROLL; ++u) {
+                        if constexpr (VEC == 1) x[u] = v[u];
+                        else {
 #pragma unroll
-                        for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0));
+                            for (int j = 0; j < VEC; ++j) x[u * VEC + j] = v[u][j];
+                        }
+                    }
+                    map_batch<UNROLL * VEC>(x, y, xf);
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], y[u * VEC + j]);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
+                        if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
+                        else {
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], e0));
+                        }
                     }
                 }
             } else {
@@ -522,7 +623,8 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
 
 // ---- typed entry points instantiated once per (in, out) pair ---------------------------------------
 struct MapreduceArgs {
-    int f, op;
+    int f, op;                   // f: rk_map, or RK_MAP_PROGRAM with `prog`
+    const rk_map_program* prog;
     const void* A; int ndim; const int64_t* shape; uint32_t mask;
     void* R; const void* init;
     void* ws; size_t ws_bytes; hipStream_t stream;
@@ -540,8 +642,8 @@ struct FindArgs {
 // a temporary at the top of the partials area -- and the remaining dims are reduced from that much smaller array.
 constexpr size_t REDUCE_TEMP_MAX = WS_PARTIALS_BYTES / 2;
 
-template <typename In, typename Acc, typename Map, typename Op>
-inline int32_t mapreduce_one(const MapreduceArgs& a) {
+template <typename In, typename Acc, typename Xf, typename Op>
+inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
     ReduceSink<Acc, Op> sink{(Acc*)a.R, a.init ? *(const Acc*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
     const Shape3 s = collapse3(a.ndim, a.shape, a.mask);
     if (!s.single_run && s.total > 0) {
@@ -564,24 +666,52 @@ inline int32_t mapreduce_one(const MapreduceArgs& a) {
             Acc* temp = (Acc*)((char*)w.partials + WS_PARTIALS_BYTES - temp_bytes);
             const size_t cap = WS_PARTIALS_BYTES - temp_bytes;
             ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
-            const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, mask1, MapXform<In, Acc, Map>(), Op(), to_temp,
+            const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, mask1, xf, Op(), to_temp,
                                                       a.ws, a.ws_bytes, a.stream, cap);
             if (st != RK_SUCCESS) return st;
             return launch_reduce<Acc, Acc>((const Acc*)temp, a.ndim, shape1, a.mask & ~mask1, MapXform<Acc, Acc, MapIdentity>(), Op(), sink,
                                            a.ws, a.ws_bytes, a.stream, cap);
         }
     }
-    return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, MapXform<In, Acc, Map>(), Op(), sink,
-                                  a.ws, a.ws_bytes, a.stream);
+    return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream);
 }
 
 template <typename In, typename Acc, typename Map>
 inline int32_t mapreduce_op(const MapreduceArgs& a) {
+    const MapXform<In, Acc, Map> xf;
     switch (a.op) {
-        case RK_OP_ADD: return mapreduce_one<In, Acc, Map, OpAdd>(a);
-        case RK_OP_MUL: return mapreduce_one<In, Acc, Map, OpMul>(a);
-        case RK_OP_MAX: return mapreduce_one<In, Acc, Map, OpMax>(a);
-        case RK_OP_MIN: return mapreduce_one<In, Acc, Map, OpMin>(a);
+        case RK_OP_ADD: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpAdd>(a, xf);
+        case RK_OP_MUL: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMul>(a, xf);
+        case RK_OP_MAX: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMax>(a, xf);
+        case RK_OP_MIN: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMin>(a, xf);
+        default: return RK_ERR_INVALID_ARGUMENT;
+    }
+}
+
+// f as a program (validated by the caller: at most RK_MAP_MAX_TOKENS tokens, stack depth within the registers)
+template <typename In, typename Acc>
+inline ProgXform<In, Acc> make_prog_xform(const rk_map_program& p) {
+    ProgXform<In, Acc> xf{};
+    for (int i = 0; i < p.n_tokens; ++i) {
+        const uint64_t t = (uint64_t)(p.tokens[i] & 0xff) << ((i & 7) * 8);
+        if (i < 8) xf.tokens.lo |= t; else xf.tokens.hi |= t;
+    }
+    xf.n_tokens = p.n_tokens;
+    typedef typename ProgXform<In, Acc>::CT CT;
+    for (int k = 0; k < RK_MAP_MAX_CONSTS; ++k)
+        xf.c[k] = k < p.n_consts ? (std::is_floating_point<CT>::value ? (CT)p.const_f[k] : (CT)p.const_i[k]) : CT(0);
+    return xf;
+}
+template <typename In, typename Acc, bool ADD_ONLY = false>
+inline int32_t mapreduce_prog(const MapreduceArgs& a) {
+    typedef ProgXform<In, Acc> Xf;
+    const Xf xf = make_prog_xform<In, Acc>(*a.prog);
+    if constexpr (ADD_ONLY) return a.op == RK_OP_ADD ? mapreduce_one<In, Acc, Xf, OpAdd>(a, xf) : (int32_t)RK_ERR_UNSUPPORTED;
+    else switch (a.op) {
+        case RK_OP_ADD: return mapreduce_one<In, Acc, Xf, OpAdd>(a, xf);
+        case RK_OP_MUL: return mapreduce_one<In, Acc, Xf, OpMul>(a, xf);
+        case RK_OP_MAX: return mapreduce_one<In, Acc, Xf, OpMax>(a, xf);
+        case RK_OP_MIN: return mapreduce_one<In, Acc, Xf, OpMin>(a, xf);
         default: return RK_ERR_INVALID_ARGUMENT;
     }
 }
@@ -622,6 +752,14 @@ inline int32_t findminmax_typed(const FindArgs& a) {
 }
 
 // one translation unit per type pair (keeps compile times parallel)
+int32_t mapreduce_prog_f32(const MapreduceArgs&);
+int32_t mapreduce_prog_f32_i64(const MapreduceArgs&);      // count(pred, A): + only
+int32_t mapreduce_prog_f64(const MapreduceArgs&);
+int32_t mapreduce_prog_f64_i64(const MapreduceArgs&);
+int32_t mapreduce_prog_i32(const MapreduceArgs&);
+int32_t mapreduce_prog_i64(const MapreduceArgs&);
+int32_t mapreduce_prog_i32_i64(const MapreduceArgs&);
+int32_t mapreduce_prog_u8_i64(const MapreduceArgs&);
 int32_t mapreduce_f32(const MapreduceArgs&);
 int32_t mapreduce_f64(const MapreduceArgs&);
 int32_t mapreduce_i32(const MapreduceArgs&);

@@ -6,19 +6,27 @@ namespace rk {
 #if RK_INST == 0
 int32_t mapreduce_f32(const MapreduceArgs& a) { return mapreduce_typed<float, float>(a); }
 int32_t findminmax_f32(const FindArgs& a) { return findminmax_typed<float>(a); }
+int32_t mapreduce_prog_f32(const MapreduceArgs& a) { return mapreduce_prog<float, float>(a); }
+int32_t mapreduce_prog_f32_i64(const MapreduceArgs& a) { return mapreduce_prog<float, int64_t, true>(a); }
 #elif RK_INST == 1
 int32_t mapreduce_f64(const MapreduceArgs& a) { return mapreduce_typed<double, double>(a); }
 int32_t findminmax_f64(const FindArgs& a) { return findminmax_typed<double>(a); }
+int32_t mapreduce_prog_f64(const MapreduceArgs& a) { return mapreduce_prog<double, double>(a); }
+int32_t mapreduce_prog_f64_i64(const MapreduceArgs& a) { return mapreduce_prog<double, int64_t, true>(a); }
 #elif RK_INST == 2
 int32_t mapreduce_i32(const MapreduceArgs& a) { return mapreduce_typed<int32_t, int32_t>(a); }
 int32_t findminmax_i32(const FindArgs& a) { return findminmax_typed<int32_t>(a); }
+int32_t mapreduce_prog_i32(const MapreduceArgs& a) { return mapreduce_prog<int32_t, int32_t>(a); }
 #elif RK_INST == 3
 int32_t mapreduce_i64(const MapreduceArgs& a) { return mapreduce_typed<int64_t, int64_t>(a); }
 int32_t findminmax_i64(const FindArgs& a) { return findminmax_typed<int64_t>(a); }
+int32_t mapreduce_prog_i64(const MapreduceArgs& a) { return mapreduce_prog<int64_t, int64_t>(a); }
 #elif RK_INST == 4
 int32_t mapreduce_i32_i64(const MapreduceArgs& a) { return mapreduce_typed<int32_t, int64_t>(a); }
+int32_t mapreduce_prog_i32_i64(const MapreduceArgs& a) { return mapreduce_prog<int32_t, int64_t>(a); }
 #elif RK_INST == 5
 int32_t mapreduce_u8_i64(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, int64_t>(a); }
+int32_t mapreduce_prog_u8_i64(const MapreduceArgs& a) { return mapreduce_prog<uint8_t, int64_t>(a); }
 #elif RK_INST == 6
 int32_t mapreduce_u8(const MapreduceArgs& a) { return mapreduce_typed<uint8_t, uint8_t>(a); }      // any / all of Bool arrays
 int32_t findminmax_u8(const FindArgs& a) { return findminmax_typed<uint8_t>(a); }                   // findfirst of Bool arrays

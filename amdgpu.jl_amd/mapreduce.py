@@ -67,11 +67,33 @@ def _scalar_buffer(value, dtype: np.dtype):
     return C.create_string_buffer(np.array(value, dtype=dtype).tobytes(), dtype.itemsize)
 
 
-def mapreducedim_(f: str, op: str, R: ROCArray, A: ROCArray, init=None) -> ROCArray:
+def _map_program(f, dtype):
+    """A closure for f -> (rk_map_program, Julia's eltype of f(x)); traced by calling it on a symbolic element."""
+    from .broadcast import compile_map
+    tokens, consts, eltype, compute = compile_map(f, dtype)
+    dt = np.dtype(dtype)
+    if (compute.kind == "f") != (dt.kind == "f") or (compute.kind == "f" and compute != dt):
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"mapreduce closure computing in {compute} over {dt} elements "
+                                                       "(a Python float is a Float64: use np.float32 constants)")
+    p = L.RkMapProgram()
+    p.n_tokens = len(tokens)
+    for i, t in enumerate(tokens):
+        p.tokens[i] = t
+    p.n_consts = len(consts)
+    for k, c in enumerate(consts):
+        if compute.kind == "f":
+            p.const_f[k] = float(c)
+        else:
+            p.const_i[k] = int(c)
+    return p, eltype
+
+
+def mapreducedim_(f, op: str, R: ROCArray, A: ROCArray, init=None) -> ROCArray:
     """``GPUArrays.mapreducedim!(f, op, R, A; init)``: reduces A into R over every dimension in which
     R has extent 1 and A does not; returns the R object it was given (mapreduce.jl:93,172;
-    test/core/rocarray_base.jl:263-267).  With ``init=None`` the neutral element of ``op`` is used."""
-    if f not in _MAP:
+    test/core/rocarray_base.jl:263-267).  With ``init=None`` the neutral element of ``op`` is used.
+    ``f`` is one of the enumerated maps or a closure of the element (``lambda x: x + 1``)."""
+    if not callable(f) and f not in _MAP:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"map {f!r}")
     if op not in _OP:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"reduction operator {op!r}")
@@ -96,11 +118,16 @@ def _launch_mapreducedim(f, op, R, A, init, mask):
     """Zero-argument callable that enqueues the reduction on the current stream."""
     ws, ws_bytes = workspace()
     ibuf = _scalar_buffer(init, R.dtype)
-    args = (_MAP[f], _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, R.ptr, ibuf, ws, ws_bytes)
-    fn = L.lib.rk_mapreduce
+    if callable(f):
+        prog, _ = _map_program(f, A.dtype)
+        args = (prog, _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, R.ptr, ibuf, ws, ws_bytes)
+        fn, name = L.lib.rk_mapreduce_program, "rk_mapreduce_program"
+    else:
+        args = (_MAP[f], _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, R.ptr, ibuf, ws, ws_bytes)
+        fn, name = L.lib.rk_mapreduce, "rk_mapreduce"
 
     def launch():
-        L.check(fn(*args, stream_ptr()), "rk_mapreduce")
+        L.check(fn(*args, stream_ptr()), name)
     return launch
 
 
@@ -117,12 +144,21 @@ def plan_mapreducedim(f: str, op: str, R: ROCArray, A: ROCArray, init=None):
     return _launch_mapreducedim(f, op, R, A, init, mask)
 
 
-def mapreduce(f: str, op: str, A: ROCArray, dims=None, init=None):
+def mapreduce(f, op: str, A: ROCArray, dims=None, init=None):
     """``mapreduce(f, op, A; dims, init)``.  ``dims=None`` is Julia's ``:`` and returns a host scalar
     (a blocking 4/8-byte read, like ``@allowscalar R[]`` in GPUArrays); otherwise a ROCArray whose
-    reduced dims have extent 1."""
+    reduced dims have extent 1.  ``f``: "identity" / "abs2" / "abs", or a closure of the element built from
+    arithmetic, comparisons and this package's functions (``lambda x: x + 1``, ``lambda x: isodd(x)``): it is
+    traced into a program that the reduction kernels evaluate on the loaded values (one pass over A); the result
+    eltype is ``promote_op(op, T, T)`` with T the eltype of ``f(x)``, as GPUArrays infers it."""
     mask = _dims_mask(dims, A.ndim)
-    out_dt = reduce_eltype(op, A.dtype)
+    if callable(f):
+        _, mapped = _map_program(f, A.dtype)
+        if mapped == np.bool_ and op in ("max", "min"):
+            return _reduce_predicate(f, op, A, dims, mask)
+        out_dt = reduce_eltype(op, mapped)
+    else:
+        out_dt = reduce_eltype(op, A.dtype)
     if len(A) == 0:
         if op in ("max", "min"):
             raise ValueError("reducing over an empty collection is not allowed")
@@ -139,54 +175,109 @@ def mapreduce(f: str, op: str, A: ROCArray, dims=None, init=None):
     return R
 
 
-def sum(A: ROCArray, dims=None, f: str = identity):          # noqa: A001 - mirrors Base.sum
-    return mapreduce(f, add_sum, A, dims=dims)
+def _reduce_predicate(pred, op, A, dims, mask):
+    """``any(pred, A; dims)`` / ``all(pred, A; dims)``: | and & of Bools are max and min of 0 / 1, accumulated in A's
+    own element type (Int64 for Bool arrays) and turned into Bools at the end."""
+    from .broadcast import lazy, materialize
+    acc_dt = A.dtype if A.dtype in (np.float32, np.float64, np.int32, np.int64) else np.dtype(np.int64)
+    if len(A) == 0:
+        neutral = op == "min"
+        return neutral if dims is None else ROCArray(np.full(_reduced_dims(A.dims, mask), neutral, dtype=np.bool_))
+    rshape = (1,) * A.ndim if dims is None else _reduced_dims(A.dims, mask)
+    R = ROCArray(dims=rshape, dtype=acc_dt)
+    mapreducedim_(pred, op, R, A)
+    if dims is None:
+        return bool(R.item() != 0)
+    return materialize(lazy(R) != acc_dt.type(0))
 
 
-def prod(A: ROCArray, dims=None):
-    return mapreduce(identity, mul_prod, A, dims=dims)
+def _split(args, name):
+    """(f, A) from Julia's two call forms ``name(A)`` and ``name(f, A)``."""
+    if len(args) == 1:
+        return None, args[0]
+    if len(args) == 2 and callable(args[0]):
+        return args
+    raise TypeError(f"{name}(A) or {name}(f, A)")
 
 
-def maximum(A: ROCArray, dims=None):
-    return mapreduce(identity, max_, A, dims=dims)
+def sum(*args, dims=None, f=identity):          # noqa: A001 - mirrors Base.sum
+    """``sum(A; dims)`` / ``sum(f, A; dims)``."""
+    g, A = _split(args, "sum")
+    return mapreduce(g if g is not None else f, add_sum, A, dims=dims)
 
 
-def minimum(A: ROCArray, dims=None):
-    return mapreduce(identity, min_, A, dims=dims)
+def prod(*args, dims=None):
+    g, A = _split(args, "prod")
+    return mapreduce(g if g is not None else identity, mul_prod, A, dims=dims)
 
 
-def count(A: ROCArray, dims=None):
-    """``count(::ROCArray{Bool})`` == sum of the Bool array in Int64."""
+def maximum(*args, dims=None):
+    g, A = _split(args, "maximum")
+    return mapreduce(g if g is not None else identity, max_, A, dims=dims)
+
+
+def minimum(*args, dims=None):
+    g, A = _split(args, "minimum")
+    return mapreduce(g if g is not None else identity, min_, A, dims=dims)
+
+
+def _check_predicate(pred, A, name):
+    _, mapped = _map_program(pred, A.dtype)
+    if mapped != np.bool_:
+        raise TypeError(f"{name}: non-boolean ({mapped}) used in boolean context")     # Julia's TypeError
+
+
+def count(*args, dims=None):
+    """``count(::ROCArray{Bool}; dims)`` == sum of the Bool array in Int64; ``count(pred, A; dims)`` sums the
+    predicate's Bools in the same single pass over A."""
+    pred, A = _split(args, "count")
+    if pred is not None:
+        _check_predicate(pred, A, "count")
+        return mapreduce(pred, add_sum, A, dims=dims)
     if A.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "count needs a Bool array")
     return mapreduce(identity, add_sum, A, dims=dims)
 
 
-def any(A: ROCArray, dims=None):                             # noqa: A001 - mirrors Base.any
-    """``any(::ROCArray{Bool}; dims)``: ``|`` over Bools is ``max`` over their bytes."""
+def any(*args, dims=None):                             # noqa: A001 - mirrors Base.any
+    """``any(::ROCArray{Bool}; dims)``: ``|`` over Bools is ``max`` over their bytes.  ``any(pred, A; dims)``."""
+    pred, A = _split(args, "any")
+    if pred is not None:
+        _check_predicate(pred, A, "any")
+        return mapreduce(pred, max_, A, dims=dims)
     if A.dtype != np.bool_:
-        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "any needs a Bool array (predicates are closures)")
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "any needs a Bool array or a predicate")
     if len(A) == 0:
         return False if dims is None else ROCArray(np.zeros(_reduced_dims(A.dims, _dims_mask(dims, A.ndim)), dtype=np.bool_))
     r = mapreduce(identity, max_, A, dims=dims)
     return bool(r) if dims is None else r
 
 
-def all(A: ROCArray, dims=None):                             # noqa: A001 - mirrors Base.all
-    """``all(::ROCArray{Bool}; dims)``: ``&`` over Bools is ``min`` over their bytes."""
+def all(*args, dims=None):                             # noqa: A001 - mirrors Base.all
+    """``all(::ROCArray{Bool}; dims)``: ``&`` over Bools is ``min`` over their bytes.  ``all(pred, A; dims)``."""
+    pred, A = _split(args, "all")
+    if pred is not None:
+        _check_predicate(pred, A, "all")
+        return mapreduce(pred, min_, A, dims=dims)
     if A.dtype != np.bool_:
-        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "all needs a Bool array (predicates are closures)")
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "all needs a Bool array or a predicate")
     if len(A) == 0:
         return True if dims is None else ROCArray(np.ones(_reduced_dims(A.dims, _dims_mask(dims, A.ndim)), dtype=np.bool_))
     r = mapreduce(identity, min_, A, dims=dims)
     return bool(r) if dims is None else r
 
 
-def findfirst(A: ROCArray):
+def findfirst(*args):
     """``findfirst(::ROCArray{Bool})``: index of the first true entry in column-major order (an Int for
-    vectors, a CartesianIndex tuple otherwise) or ``None``: the argmax of the bytes, ties to the smallest index."""
+    vectors, a CartesianIndex tuple otherwise) or ``None``: the argmax of the bytes, ties to the smallest index.
+    ``findfirst(pred, A)`` searches ``pred.(A)`` (benchmarked in perf/array.jl:44-47)."""
+    pred, A = _split(args, "findfirst")
+    if pred is not None:
+        from .broadcast import lazy, materialize
+        _check_predicate(pred, A, "findfirst")
+        A = materialize(pred(lazy(A)))
     if A.dtype != np.bool_:
-        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findfirst needs a Bool array (predicates are closures)")
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findfirst needs a Bool array or a predicate")
     if len(A) == 0:
         return None
     v, i = _findminmax(A, True, None)

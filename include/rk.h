@@ -115,6 +115,34 @@ RK_API int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
                      void* R, const void* init,
                      void* ws, size_t ws_bytes, void* stream);
 
+/* ---- mapreduce with f given as a program -----------------------------------------------
+ * Replaces GPUArrays.mapreducedim!(f, op, R, A) for an f outside the rk_map list
+ *                                                        src/kernels/mapreduce.jl:86-89
+ * e.g. mapreduce(x -> x + 1, +, A; dims) (benchmarked in perf/array.jl:107-122), sum(f, A),
+ * count(isodd, A), any(x -> x > 0, A).  f is a postfix program of rk_bc_token (declared with
+ * the broadcast below) over the element -- operand token 0 -- and up to RK_MAP_MAX_CONSTS
+ * constants -- operand tokens 1 ..; at most RK_MAP_MAX_TOKENS tokens and a value stack of
+ * depth 4.  Float32 / Float64 elements compute in their own type, integer elements in Int64
+ * (constants from const_i; the program holds RK_BC_WRAP_* where a 32-bit intermediate
+ * matters), and the result is converted to `out`.
+ * Supported (in -> out): F32 -> F32, F64 -> F64, I32 -> I32, I64 -> I64, I32 -> I64,
+ * U8 -> I64; F32 -> I64 and F64 -> I64 with RK_OP_ADD only (counts).
+ * Everything else as rk_mapreduce. */
+#define RK_MAP_MAX_TOKENS 16
+#define RK_MAP_MAX_CONSTS 4
+#define RK_MAP_PROGRAM 3          /* the f of these calls, next to the rk_map values */
+typedef struct {
+    int32_t n_tokens;
+    int32_t tokens[RK_MAP_MAX_TOKENS];
+    int32_t n_consts;
+    double  const_f[RK_MAP_MAX_CONSTS];   /* used when the elements are F32 / F64 */
+    int64_t const_i[RK_MAP_MAX_CONSTS];   /* used when they are integers          */
+} rk_map_program;
+RK_API int32_t rk_mapreduce_program(const rk_map_program* f, rk_op op, rk_dtype in, rk_dtype out,
+                      const void* A, int ndim, const int64_t* shape, uint32_t reduce_mask,
+                      void* R, const void* init,
+                      void* ws, size_t ws_bytes, void* stream);
+
 /* ---- findmax / findmin -----------------------------------------------------------
  * Replaces the (value, CartesianIndex) tuple reduction that GPUArrays' findminmax sends
  * through mapreducedim!                                    src/kernels/mapreduce.jl:86
@@ -161,7 +189,16 @@ typedef enum {
     RK_BC_ADD = 32, RK_BC_SUB, RK_BC_MUL, RK_BC_DIV, RK_BC_MAX, RK_BC_MIN, RK_BC_POW,
     RK_BC_FMA,                 /* muladd(a, b, c): pops c, b, a                         */
     RK_BC_NEG = 64, RK_BC_ABS, RK_BC_ABS2, RK_BC_SQRT, RK_BC_EXP, RK_BC_LOG, RK_BC_SIN,
-    RK_BC_COS, RK_BC_TANH, RK_BC_INV, RK_BC_IDENTITY
+    RK_BC_COS, RK_BC_TANH, RK_BC_INV, RK_BC_IDENTITY,
+    /* predicates and logic: the result is 1 or 0 in the compute type (a Bool once stored to a U8 dest);
+     * AND / OR / NOT / IFELSE read "nonzero" as true */
+    RK_BC_LT = 96, RK_BC_LE, RK_BC_GT, RK_BC_GE, RK_BC_EQ, RK_BC_NE, RK_BC_AND, RK_BC_OR,
+    RK_BC_IFELSE = 112,        /* ifelse(c, a, b): pops b, a, c                          */
+    RK_BC_NOT = 128, RK_BC_ISODD, RK_BC_ISEVEN,     /* ISODD / ISEVEN: integer programs     */
+    RK_BC_ISNAN,
+    RK_BC_WRAP_I32,            /* integer programs: sign-extend the low 32 bits, i.e. the Int32 value Julia
+                                * holds at this point (needed before order-sensitive tokens only)      */
+    RK_BC_WRAP_U32             /* the same, zero-extending (UInt32)                                    */
 } rk_bc_token;
 
 typedef struct {
@@ -179,9 +216,9 @@ typedef struct {
 
 typedef struct {
     int32_t    compute;           /* rk_dtype every operand is converted to: F32, F64, or
-                                   * I64 for integer programs (+ - * max min muladd neg abs
-                                   * abs2 only; the store keeps the low bits, i.e. Int32
-                                   * results wrap as in Julia)                             */
+                                   * I64 for integer programs (no / ^ or math functions; the
+                                   * store keeps the low bits, i.e. Int32 results wrap as in
+                                   * Julia)                                                */
     int32_t    n_operands;
     rk_operand operands[RK_MAX_OPERANDS];
     int32_t    n_tokens;

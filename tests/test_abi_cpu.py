@@ -132,7 +132,38 @@ def test_broadcast_program_validation(L):
     assert b(_prog(L, [0, 1, L.RK_BC_ADD], ok_ops), None, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT  # null dest
     deep = [0] * 9 + [L.RK_BC_ADD] * 8
     assert b(_prog(L, deep, ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_UNSUPPORTED                     # stack deeper than 8
+    assert b(_prog(L, [0, L.RK_BC_ISODD], ok_ops), dest, L.RK_U8, 2, sh, None) == L.RK_ERR_UNSUPPORTED        # isodd in a Float32 program
+    assert b(_prog(L, [0, 1, L.RK_BC_IFELSE], ok_ops), dest, L.RK_F32, 2, sh, None) == L.RK_ERR_INVALID_ARGUMENT   # ifelse pops three
     assert b(_prog(L, [0, 1, L.RK_BC_ADD], [arr(0, 3), arr(0, 3)]), None, L.RK_F32, 2, L.shape_array((0, 3)), None) == L.RK_SUCCESS
+
+
+def test_mapreduce_program_validation(L):
+    m = L.lib.rk_mapreduce_program
+    sh = L.shape_array((4, 3))
+    A, R = C.c_void_p(0x1000), C.c_void_p(0x2000)
+
+    def prog(tokens, n_consts=1):
+        p = L.RkMapProgram()
+        p.n_tokens = len(tokens)
+        for i, t in enumerate(tokens):
+            p.tokens[i] = t
+        p.n_consts = n_consts
+        return p
+    plus1 = [0, 1, L.RK_BC_ADD]
+    assert m(None, L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert m(prog([]), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert m(prog(plus1, 5), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert m(prog([0, 2, L.RK_BC_ADD]), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # constant 2 missing
+    assert m(prog([0, L.RK_BC_ADD]), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # stack underflow
+    assert m(prog([0, 1]), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT                # two values left
+    assert m(prog(plus1), 7, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    deep = [0, 0, 0, 0, 0] + [L.RK_BC_ADD] * 4
+    assert m(prog(deep), L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_UNSUPPORTED      # value stack deeper than 4
+    assert m(prog([0, L.RK_BC_SQRT]), L.RK_OP_ADD, L.RK_I64, L.RK_I64, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_UNSUPPORTED   # sqrt(Int) is a Float64
+    assert m(prog([0, L.RK_BC_ISODD]), L.RK_OP_ADD, L.RK_F32, L.RK_I64, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert m(prog(plus1), L.RK_OP_ADD, L.RK_F32, L.RK_F64, A, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_UNSUPPORTED     # no such type pair
+    assert m(prog(plus1), L.RK_OP_ADD, L.RK_F32, L.RK_F32, None, 2, sh, 1, R, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert m(prog(plus1), L.RK_OP_ADD, L.RK_F32, L.RK_F32, None, 2, L.shape_array((0, 3)), 1, None, None, None, 0, None) == L.RK_SUCCESS   # mapreduce.jl:91
 
 
 def test_volumerhs_and_scatter_validation(L):
@@ -214,8 +245,7 @@ def test_host_mirror_rules_without_gpu(rk):
     with pytest.raises(rk.DimensionMismatch):
         B.broadcast_shape((2, 3), (3,))
     a = np.float32(0.5)
-    ops, toks = [], []
-    B._flatten(B._leaf(a * B.lazy(1.0) + B.lazy(2.0) * B.exp(B.lazy(3.0))), ops, toks)
+    toks = B._compile(a * B.lazy(1.0) + B.lazy(2.0) * B.exp(B.lazy(3.0)))[1]
     from amdgpu_jl_amd import _lib as L
     assert toks == [0, 1, L.RK_BC_MUL, 2, 3, L.RK_BC_EXP, L.RK_BC_MUL, L.RK_BC_ADD]
     with pytest.raises(rk.UnsupportedError):
@@ -223,3 +253,20 @@ def test_host_mirror_rules_without_gpu(rk):
     # a NumPy Float32 scalar on the left keeps its type (0.5f0 .* x computes in Float32, not Float64)
     assert B._compile(np.float32(0.5) * B.lazy(np.float32(2.0)))[2] == np.float32
     assert B._compile(0.5 * B.lazy(np.float32(2.0)))[2] == np.float64
+    # Julia's promotion, not NumPy's: Int64 with Float32 is Float32; Int32 with UInt32 is UInt32
+    assert B.promote_type(np.int64, np.float32) == np.float32 and B.promote_type(np.int32, np.uint32) == np.uint32
+    assert B.promote_type(np.bool_, np.int32) == np.int32 and B.promote_type(np.int64, np.uint32) == np.int64
+    # closures of mapreduce(f, op, A) traced on a symbolic element: tokens, constants, eltype of f(x), compute type
+    toks, consts, elt, comp = B.compile_map(lambda x: x + 1, np.float32)
+    assert toks == [0, 1, L.RK_BC_ADD] and consts == [1] and elt == np.float32 and comp == np.float32
+    toks, consts, elt, comp = B.compile_map(lambda x: x + 1, np.int32)
+    assert elt == np.int64 and comp == np.int64 and toks == [0, 1, L.RK_BC_ADD]
+    toks, consts, elt, comp = B.compile_map(lambda x: x * x > 0, np.int32)          # the comparison needs the wrapped square
+    assert elt == np.bool_ and toks == [0, 0, L.RK_BC_MUL, L.RK_BC_WRAP_I32, 1, L.RK_BC_GT]
+    toks, _, elt, _ = B.compile_map(lambda x: x * x, np.int32)                      # and so does a widening reduction
+    assert elt == np.int32 and toks == [0, 0, L.RK_BC_MUL, L.RK_BC_WRAP_I32]
+    assert B.compile_map(lambda x: B.isodd(x), np.int64)[2] == np.bool_
+    assert B.compile_map(lambda x: x, np.float64)[0] == [0]
+    with pytest.raises(rk.UnsupportedError):
+        B.compile_map(lambda x: B.isodd(x), np.float32)
+    assert B._compile(B.lazy(np.float32(1)) > B.lazy(2))[4] == np.bool_
