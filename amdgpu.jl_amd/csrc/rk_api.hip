@@ -187,6 +187,8 @@ int32_t rk_mapreduce_program(const rk_map_program* f, rk_op op, rk_dtype in, rk_
     {   // operand 0 = the element, 1 .. n_consts = the constants; the value stack stays in registers
         const int32_t st = validate_tokens(f->tokens, f->n_tokens, 1 + f->n_consts, int_compute, INTERP_REG_DEPTH);
         if (st != RK_SUCCESS) return st;
+        for (int i = 0; i < f->n_tokens; ++i)
+            if (!token_basic(f->tokens[i])) return RK_ERR_UNSUPPORTED;      // pow, sin, cos, tanh: map first, then reduce
     }
     if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
     if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91

@@ -134,6 +134,7 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
 // ---- evaluators ---------------------------------------------------------------------------------------
 // Postfix interpreter (rk_interp.hpp) over the loaded operands.
 template <typename CT, int VEC> struct BcFetch {
+    static constexpr int NOPS = RK_MAX_OPERANDS;
     const CT (&in)[RK_MAX_OPERANDS][VEC];
     template <int K> __device__ __forceinline__ void get(CT (&v)[VEC]) const {
 #pragma unroll
@@ -145,7 +146,7 @@ struct EvalInterp {
     static constexpr bool USES_LDS = true;
     template <typename CT, int VEC>
     static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
-        interp_run<CT, VEC, BC_BLOCK>(a.tokens, a.n_tokens, BcFetch<CT, VEC>{in}, out, lds);
+        interp_run<CT, VEC, BC_BLOCK, true>(a.tokens, a.n_tokens, BcFetch<CT, VEC>{in}, out, lds);
     }
 };
 

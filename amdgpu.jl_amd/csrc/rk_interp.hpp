@@ -30,6 +30,11 @@ __host__ __device__ constexpr bool token_float_ok(int tok) {
     return tok != RK_BC_ISODD && tok != RK_BC_ISEVEN && tok != RK_BC_WRAP_I32 && tok != RK_BC_WRAP_U32;
 }
 
+// pow and the trigonometric / hyperbolic functions exist in the full interpreter only
+__host__ __device__ constexpr bool token_basic(int tok) {
+    return tok != RK_BC_POW && tok != RK_BC_SIN && tok != RK_BC_COS && tok != RK_BC_TANH;
+}
+
 // A well-formed postfix expression that leaves exactly one value; operand tokens are 0 .. n_operands-1.
 inline int32_t validate_tokens(const int32_t* tokens, int n_tokens, int n_operands, bool int_compute, int max_allowed_depth) {
     int depth = 0, max_depth = 0;
@@ -56,10 +61,16 @@ inline int32_t validate_tokens(const int32_t* tokens, int n_tokens, int n_operan
 // N components are evaluated together.  The four topmost stack entries live in registers and move by one place on
 // push / pop; deeper entries (rare) spill to LDS when SPILL_BLOCK > 0 (entry e of thread t, component j at
 // lds[(e * N + j) * SPILL_BLOCK + t]); with SPILL_BLOCK == 0 the host limits programs to depth INTERP_REG_DEPTH.
-// fetch.template get<K>(v) delivers operand K; tokens[i] is token i (an array in kernel arguments, or packed bits).
+// FULL = false leaves out pow, sin, cos and tanh (the reductions instantiate the interpreter in every kernel variant;
+// the host keeps such programs away from them).
+// fetch.template get<K>(v) delivers operand K < Fetch::NOPS; tokens[i] is token i (an array in kernel arguments, or
+// packed bits).
+// Measured alternative: slots as fixed registers selected by a second switch over the (uniform) depth, so that
+// nothing moves on push / pop -- more scalar branches per token and just as many moves (the register allocator
+// reconciles the cases with copies): no faster, 4 MB more code.
 constexpr int INTERP_REG_DEPTH = 4;
 
-template <typename CT, int N, int SPILL_BLOCK, typename Tokens, typename Fetch>
+template <typename CT, int N, int SPILL_BLOCK, bool FULL, typename Tokens, typename Fetch>
 __device__ __forceinline__ void interp_run(const Tokens& tokens, int n_tokens, const Fetch& fetch, CT (&out)[N], CT* lds) {
     const int t = threadIdx.x;
     CT s0[N], s1[N], s2[N], s3[N];     // s0 = top of the stack
@@ -88,7 +99,7 @@ __device__ __forceinline__ void interp_run(const Tokens& tokens, int n_tokens, c
             }
         }
     };
-#define RK_BC_OPERAND(K) case K: { CT v[N]; fetch.template get<K>(v); push(v); } break
+#define RK_BC_OPERAND(K) case K: { CT v[N]; if constexpr (K < Fetch::NOPS) fetch.template get<K>(v); push(v); } break
 #define RK_BC_UN(EXPR)  { _Pragma("unroll") for (int j = 0; j < N; ++j) { const CT x = s0[j]; s0[j] = (EXPR); } } break
 #define RK_BC_BIN(EXPR) { _Pragma("unroll") for (int j = 0; j < N; ++j) { const CT x = s1[j], y = s0[j]; s0[j] = (EXPR); } drop_second(); } break
     for (int i = 0; i < n_tokens; ++i) {
@@ -135,16 +146,22 @@ __device__ __forceinline__ void interp_run(const Tokens& tokens, int n_tokens, c
                 if constexpr (std::is_floating_point<CT>::value) {
                     switch (tok) {
                         case RK_BC_DIV: RK_BC_BIN(x / y);
-                        case RK_BC_POW: RK_BC_BIN(pow(x, y));
                         case RK_BC_SQRT: RK_BC_UN(sqrt(x));
                         case RK_BC_EXP: RK_BC_UN(exp(x));
                         case RK_BC_LOG: RK_BC_UN(log(x));
-                        case RK_BC_SIN: RK_BC_UN(sin(x));
-                        case RK_BC_COS: RK_BC_UN(cos(x));
-                        case RK_BC_TANH: RK_BC_UN(tanh(x));
                         case RK_BC_INV: RK_BC_UN(CT(1) / x);
                         case RK_BC_ISNAN: RK_BC_UN(x != x ? CT(1) : CT(0));
-                        default: break;
+                        default:
+                            if constexpr (FULL) {
+                                switch (tok) {
+                                    case RK_BC_POW: RK_BC_BIN(pow(x, y));
+                                    case RK_BC_SIN: RK_BC_UN(sin(x));
+                                    case RK_BC_COS: RK_BC_UN(cos(x));
+                                    case RK_BC_TANH: RK_BC_UN(tanh(x));
+                                    default: break;
+                                }
+                            }
+                            break;
                     }
                 } else {
                     switch (tok) {
