@@ -101,6 +101,80 @@ function native_mapreducedim!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N}, init) w
     return true
 end
 
+# ---- closures for f: traced on a symbolic element into an rk_map_program -----------------------------------------------
+# f(MapSym) runs ordinary Julia code; every operator on a MapSym appends rk_bc_token values instead of computing.
+# Token 0 is the element, tokens 1.. the scalars f closes over.  What the tracer cannot follow -- `if` on a value,
+# functions without a method for MapSym -- throws, and the stock mapreducedim! runs instead.
+struct RKMapProgram
+    n_tokens::Int32; tokens::NTuple{16,Int32}; n_consts::Int32; const_f::NTuple{4,Float64}; const_i::NTuple{4,Int64}
+end
+struct MapSym{T} <: Real                # T: the Julia type the value would have
+    toks::Vector{Int32}
+    consts::Vector{Any}                 # shared by every node of one trace
+end
+operand!(s::MapSym, c::Union{Float32,Float64,Int32,Int64,Bool}) = begin
+    k = findfirst(==(c), s.consts)
+    k === nothing && (push!(s.consts, c); k = length(s.consts))
+    k > 4 && throw(Unsupported())
+    Int32[k]
+end
+for (f, tok) in ((:+, 32), (:-, 33), (:*, 34), (:/, 35), (:max, 36), (:min, 37), (:<, 96), (:<=, 97), (:>, 98), (:>=, 99),
+                 (:(==), 100), (:!=, 101), (:&, 102), (:|, 103))
+    R = tok >= 96 ? :(Bool) : tok == 35 ? :(typeof(one(A) / one(B))) : :(Base.promote_op($f, A, B))
+    @eval Base.$f(a::MapSym{A}, b::MapSym{B}) where {A,B} = MapSym{$R}(vcat(a.toks, b.toks, Int32($tok)), a.consts)
+    @eval Base.$f(a::MapSym{A}, b::B) where {A,B<:Union{Float32,Float64,Int32,Int64,Bool}} =
+        MapSym{$R}(vcat(a.toks, operand!(a, b), Int32($tok)), a.consts)
+    @eval Base.$f(a::A, b::MapSym{B}) where {A<:Union{Float32,Float64,Int32,Int64,Bool},B} =
+        MapSym{$R}(vcat(operand!(b, a), b.toks, Int32($tok)), b.consts)
+end
+for (f, tok) in ((:-, 64), (:abs, 65), (:abs2, 66), (:sqrt, 67), (:exp, 68), (:log, 69), (:inv, 73), (:!, 128), (:isodd, 129),
+                 (:iseven, 130), (:isnan, 131))
+    R = tok >= 128 ? :(Bool) : :(Base.promote_op($f, A))
+    @eval Base.$f(a::MapSym{A}) where {A} = MapSym{$R}(vcat(a.toks, Int32($tok)), a.consts)
+end
+Base.ifelse(c::MapSym{Bool}, a::MapSym{A}, b::MapSym{B}) where {A,B} =
+    MapSym{promote_type(A, B)}(vcat(c.toks, a.toks, b.toks, Int32(112)), c.consts)
+
+function trace_map(f, ::Type{T}) where {T}
+    consts = Any[]
+    y = f(MapSym{T}(Int32[0], consts))
+    y isa MapSym || throw(Unsupported())
+    R = typeof(y).parameters[1]
+    toks = y.toks
+    # integer programs run in Int64: only Int64 / Bool values may reach an order-sensitive token or the reduction unwrapped
+    T <: Union{Int32,UInt32} && throw(Unsupported())
+    T <: AbstractFloat && !all(c -> c isa T || c isa Integer, consts) && throw(Unsupported())      # 0.5 over Float32: a Float64 map
+    length(toks) <= 16 || throw(Unsupported())
+    cf = ntuple(k -> k <= length(consts) ? Float64(consts[k]) : 0.0, 4)
+    ci = ntuple(k -> k <= length(consts) && !(consts[k] isa AbstractFloat) ? Int64(consts[k]) : Int64(0), 4)
+    return Ref(RKMapProgram(length(toks), ntuple(i -> i <= length(toks) ? toks[i] : Int32(0), 16), length(consts), cf, ci)), R
+end
+
+function native_mapreducedim_closure!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N}, init) where {TR,TA,N}
+    prog, TM = try trace_map(f, TA) catch; return false end
+    TR === Base.promote_op(op, TM, TM) || return false
+    Base.check_reducedims(R, A)
+    isempty(A) && return true
+    mask = UInt32(0)
+    for d in 1:N
+        size(R, d) == size(A, d) || (mask |= UInt32(1) << (d - 1))
+    end
+    ws = workspace()
+    shape = Int64[size(A)...]
+    initref = init === nothing ? C_NULL : Ref(convert(TR, init))
+    GC.@preserve R A ws shape initref prog begin
+        st = ccall((:rk_mapreduce_program, librk[]), Int32,
+                   (Ref{RKMapProgram}, Cint, Cint, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Cvoid},
+                    Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   prog, rk_op(op), rk_dtype(TA), rk_dtype(TR), pointer(A), N, shape, mask, pointer(R),
+                   initref === C_NULL ? C_NULL : Base.unsafe_convert(Ptr{Cvoid}, initref),
+                   pointer(ws), length(ws), stream_ptr())
+    end
+    st == RK_ERR_UNSUPPORTED && return false
+    check(st)
+    return true
+end
+
 function enable_mapreduce!()
     @eval function GPUArrays.mapreducedim!(f::F, op::OP, R::ROCArray{TR}, A::ROCArray{TA}; init=nothing) where {F,OP,TR,TA}
         if rk_map(f) !== nothing && rk_op(op) !== nothing && rk_dtype(TR) !== nothing && rk_dtype(TA) !== nothing &&
@@ -109,6 +183,10 @@ function enable_mapreduce!()
             # neutral element (mapreduce.jl:161-164): overwriting R gives the same result
             Rn = ndims(R) < ndims(A) ? reshape(R, Base.fill_to_length(size(R), 1, Val(ndims(A)))) : R
             native_mapreducedim!(f, op, Rn, A, init) && return R
+        elseif rk_op(op) !== nothing && rk_dtype(TR) !== nothing && rk_dtype(TA) !== nothing && ndims(R) <= ndims(A)
+            # f is a closure: mapreduce(x -> x + 1, +, A), count(isodd, A), ...
+            Rn = ndims(R) < ndims(A) ? reshape(R, Base.fill_to_length(size(R), 1, Val(ndims(A)))) : R
+            native_mapreducedim_closure!(f, op, Rn, A, init) && return R
         end
         return invoke(GPUArrays.mapreducedim!, Tuple{F,OP,AnyROCArray{TR},Union{AbstractArray,Broadcasted}}, f, op, R, A; init)
     end
@@ -191,13 +269,18 @@ end
 const ROCWrapper{T,N} = Union{SubArray{T,N,<:ROCArray}, LinearAlgebra.Transpose{T,<:ROCArray{T}},
                               PermutedDimsArray{T,N,<:Any,<:Any,<:ROCArray}}
 is_strided_wrapper(x) = x isa ROCWrapper && eltype(x) <: Real && applicable(strides, x)
-const INT_SAFE = (Int32(32), Int32(33), Int32(34), Int32(36), Int32(37), Int32(39), Int32(64), Int32(65), Int32(66), Int32(74))
+const INT_SAFE = (Int32(32), Int32(33), Int32(34), Int32(36), Int32(37), Int32(39), Int32(64), Int32(65), Int32(66), Int32(74),
+                  Int32.(96:103)..., Int32(112), Int32.(128:131)...)     # + comparisons, & |, ifelse, ! isodd iseven isnan
+# comparisons, max and min of 32-bit intermediates need RK_BC_WRAP_I32 (132) first; this binding keeps such programs
+# (an order-sensitive token over a non-leaf Int32 / UInt32 argument) on the stock path instead of typing the tree
+const ORDER_SENSITIVE = (Int32(36), Int32(37), Int32.(96:103)..., Int32(128))
 struct RkProgram
     compute::Int32; n_operands::Int32; operands::NTuple{8,RkOperand}; n_tokens::Int32; tokens::NTuple{48,Int32}
 end
-const BINARY = IdDict{Any,Int32}(+ => 32, - => 33, * => 34, / => 35, max => 36, min => 37, ^ => 38)
+const BINARY = IdDict{Any,Int32}(+ => 32, - => 33, * => 34, / => 35, max => 36, min => 37, ^ => 38,
+                                 < => 96, <= => 97, > => 98, >= => 99, == => 100, != => 101, & => 102, | => 103)
 const UNARY = IdDict{Any,Int32}(abs => 65, abs2 => 66, sqrt => 67, exp => 68, log => 69, sin => 70, cos => 71,
-                                tanh => 72, inv => 73, identity => 74)
+                                tanh => 72, inv => 73, identity => 74, ! => 128, isodd => 129, iseven => 130, isnan => 131)
 struct Unsupported <: Exception end
 
 function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
@@ -211,6 +294,8 @@ function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
             flatten!(ops, toks, args[1]); flatten!(ops, toks, args[2]); push!(toks, BINARY[f])
         elseif length(args) == 3 && f === muladd
             foreach(a -> flatten!(ops, toks, a), args); push!(toks, Int32(39))
+        elseif length(args) == 3 && f === ifelse
+            foreach(a -> flatten!(ops, toks, a), args); push!(toks, Int32(112))
         elseif f === Base.literal_pow && args[3] isa Val{2}          # x .^ 2
             flatten!(ops, toks, args[2]); push!(toks, Int32(66))
         else
@@ -237,6 +322,10 @@ function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadc
         # integer programs of + - * max min muladd - abs abs2 compute in Int64 (the store keeps the low bits);
         # with `/` or a math function Julia's result is a Float64 and so is the compute type
         CT = all(t -> t < RK_MAX_OPERANDS || t in INT_SAFE, toks) && CT <: Union{Bool,Int32,Int64,UInt8,UInt32} ? Int64 : Float64
+        if CT === Int64 && any(t -> t in ORDER_SENSITIVE, toks) &&
+           any(o -> (o isa AbstractArray ? eltype(o) : typeof(o)) <: Union{Int32,UInt32}, ops) && count(t -> t >= RK_MAX_OPERANDS, toks) > 1
+            throw(Unsupported())                 # would need RK_BC_WRAP_I32 after the 32-bit intermediates
+        end
     end
     zeros8 = ntuple(_ -> Int64(0), 8)
     zero_op = RkOperand(C_NULL, 0, 0, zeros8, 0.0, 0, 0, 0, zeros8)

@@ -8,6 +8,7 @@ through the C ABI.  No arithmetic happens on the host.
 """
 from __future__ import annotations
 
+import builtins
 import ctypes as C
 
 import numpy as np
@@ -71,6 +72,8 @@ def _map_program(f, dtype):
     """A closure for f -> (rk_map_program, Julia's eltype of f(x)); traced by calling it on a symbolic element."""
     from .broadcast import compile_map
     tokens, consts, eltype, compute = compile_map(f, dtype)
+    if builtins.any(t in (L.RK_BC_POW, L.RK_BC_SIN, L.RK_BC_COS, L.RK_BC_TANH) for t in tokens):
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "pow / sin / cos / tanh inside a reduction kernel")
     dt = np.dtype(dtype)
     if (compute.kind == "f") != (dt.kind == "f") or (compute.kind == "f" and compute != dt):
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"mapreduce closure computing in {compute} over {dt} elements "
@@ -153,7 +156,13 @@ def mapreduce(f, op: str, A: ROCArray, dims=None, init=None):
     eltype is ``promote_op(op, T, T)`` with T the eltype of ``f(x)``, as GPUArrays infers it."""
     mask = _dims_mask(dims, A.ndim)
     if callable(f):
-        _, mapped = _map_program(f, A.dtype)
+        try:
+            _, mapped = _map_program(f, A.dtype)
+        except L.UnsupportedError:
+            # a closure the reduction kernels do not interpret (too long, pow or trigonometry, another array, a result
+            # in another float type): map first -- one fused broadcast kernel -- then reduce the mapped array
+            from .broadcast import lazy, materialize
+            return mapreduce(identity, op, materialize(f(lazy(A))), dims=dims, init=init)
         if mapped == np.bool_ and op in ("max", "min"):
             return _reduce_predicate(f, op, A, dims, mask)
         out_dt = reduce_eltype(op, mapped)
@@ -221,10 +230,18 @@ def minimum(*args, dims=None):
     return mapreduce(g if g is not None else identity, min_, A, dims=dims)
 
 
-def _check_predicate(pred, A, name):
-    _, mapped = _map_program(pred, A.dtype)
+def _predicate_or_bools(pred, A, name):
+    """(pred, A) when the reduction kernels interpret ``pred``; (None, pred.(A)) -- the Bools materialized by one
+    broadcast kernel -- when they do not."""
+    try:
+        _, mapped = _map_program(pred, A.dtype)
+    except L.UnsupportedError:
+        from .broadcast import lazy, materialize
+        pred, A = None, materialize(pred(lazy(A)))
+        mapped = A.dtype
     if mapped != np.bool_:
         raise TypeError(f"{name}: non-boolean ({mapped}) used in boolean context")     # Julia's TypeError
+    return pred, A
 
 
 def count(*args, dims=None):
@@ -232,7 +249,8 @@ def count(*args, dims=None):
     predicate's Bools in the same single pass over A."""
     pred, A = _split(args, "count")
     if pred is not None:
-        _check_predicate(pred, A, "count")
+        pred, A = _predicate_or_bools(pred, A, "count")
+    if pred is not None:
         return mapreduce(pred, add_sum, A, dims=dims)
     if A.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "count needs a Bool array")
@@ -243,7 +261,8 @@ def any(*args, dims=None):                             # noqa: A001 - mirrors Ba
     """``any(::ROCArray{Bool}; dims)``: ``|`` over Bools is ``max`` over their bytes.  ``any(pred, A; dims)``."""
     pred, A = _split(args, "any")
     if pred is not None:
-        _check_predicate(pred, A, "any")
+        pred, A = _predicate_or_bools(pred, A, "any")
+    if pred is not None:
         return mapreduce(pred, max_, A, dims=dims)
     if A.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "any needs a Bool array or a predicate")
@@ -257,7 +276,8 @@ def all(*args, dims=None):                             # noqa: A001 - mirrors Ba
     """``all(::ROCArray{Bool}; dims)``: ``&`` over Bools is ``min`` over their bytes.  ``all(pred, A; dims)``."""
     pred, A = _split(args, "all")
     if pred is not None:
-        _check_predicate(pred, A, "all")
+        pred, A = _predicate_or_bools(pred, A, "all")
+    if pred is not None:
         return mapreduce(pred, min_, A, dims=dims)
     if A.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "all needs a Bool array or a predicate")
@@ -274,8 +294,9 @@ def findfirst(*args):
     pred, A = _split(args, "findfirst")
     if pred is not None:
         from .broadcast import lazy, materialize
-        _check_predicate(pred, A, "findfirst")
         A = materialize(pred(lazy(A)))
+        if A.dtype != np.bool_:
+            raise TypeError(f"findfirst: non-boolean ({A.dtype}) used in boolean context")
     if A.dtype != np.bool_:
         raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "findfirst needs a Bool array or a predicate")
     if len(A) == 0:

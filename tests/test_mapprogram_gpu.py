@@ -189,15 +189,30 @@ def test_bool_valued_broadcasts(rk):
         assert np.array_equal(rk.Array(got), (big + big) > 0)
 
 
+def test_closures_outside_the_kernel_set_map_first(rk, orc):
+    """Closures the reduction kernels do not interpret take two kernels (broadcast, then reduce): same results."""
+    x = _rng(9).standard_normal((33, 1000)).astype(np.float32)
+    y = _rng(10).standard_normal((33, 1000)).astype(np.float32)
+    a, b = rk.ROCArray(x), rk.ROCArray(y)
+    for dims in (None, 1, 2):
+        got = rk.sum(lambda v: rk.broadcast.sin(v) * rk.broadcast.cos(v), a, dims=dims)        # trigonometry
+        want = orc.mapreduce("identity", "add_sum", (np.sin(x.astype(np.float64)) * np.cos(x.astype(np.float64))).astype(np.float32), dims=dims)
+        np.testing.assert_allclose(np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape), want, rtol=1e-4, atol=1e-3)
+        got = rk.sum(lambda v: (v - rk.lazy(b)) * (v - rk.lazy(b)), a, dims=dims)              # captures an array
+        want = orc.mapreduce("identity", "add_sum", (x - y) * (x - y), dims=dims)
+        np.testing.assert_allclose(np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape), want, rtol=2e-5, atol=1e-3)
+        got = rk.sum(lambda v: v * 0.5, a, dims=dims)                                           # Float64 constant: a Float64 sum
+        want = (x.astype(np.float64) * 0.5).sum(axis=None if dims is None else dims - 1, keepdims=dims is not None)
+        assert (got.dtype if dims is not None else np.asarray(got).dtype) == np.float64
+        np.testing.assert_allclose(np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape), want, rtol=1e-12, atol=1e-9)
+        got = rk.sum(lambda v: ((((v + 1) * v + 2) * v + 3) * v + 4) * v + 5, a, dims=dims)   # five constants
+        x64 = x.astype(np.float64)
+        want = (((((x64 + 1) * x64 + 2) * x64 + 3) * x64 + 4) * x64 + 5).sum(axis=None if dims is None else dims - 1, keepdims=dims is not None)
+        np.testing.assert_allclose(np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape), want, rtol=1e-4, atol=1e-2)
+
+
 def test_unsupported_closures(rk):
     x = rk.ROCArray(np.ones((4, 4), dtype=np.float32))
-    other = rk.ROCArray(np.ones((4, 4), dtype=np.float32))
-    with pytest.raises(rk.UnsupportedError):
-        rk.mapreduce(lambda v: v + rk.lazy(other), "add", x)                    # captures an array
-    with pytest.raises(rk.UnsupportedError):
-        rk.mapreduce(lambda v: v * 0.5, "add", x)                                # Float64 constant over Float32 elements
-    with pytest.raises(rk.UnsupportedError):
-        rk.mapreduce(lambda v: ((((v + 1) * v + 2) * v + 3) * v + 4) * v + 5, "add", x)   # six constants
     with pytest.raises(rk.UnsupportedError):
         rk.mapreduce(lambda v: rk.isodd(v), "add", x)                            # isodd of a Float32
     with pytest.raises(TypeError):
