@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 N_HEAD = 1 << 26
-TRAFFIC_BC_2_26 = 1_073_369_088   # measured HBM bytes per launch of the dominant kernel (algorithmic: 2^30)
+TRAFFIC_BC_2_26 = 1_073_341_440   # measured HBM bytes per launch of the dominant kernel (algorithmic: 2^30)
 
 
 def parse():
@@ -203,6 +203,13 @@ def main():
             ps = [plan_mapreducedim(rk.identity, rk.add, r, x) for x in xs]
             run_cfg(f"cfg1a sum Float32[2^{logn}]", m, 4 * m, lambda i: ps[i % rot]())
             del xs, ps
+        # f as a closure, traced into a program the reduction kernels interpret (perf/array.jl:107-122)
+        m = 1 << 28
+        xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(2)]
+        r = rk.ROCArray(dims=(1,), dtype=np.float32)
+        ps = [plan_mapreducedim(lambda v: v + 1, rk.add, r, x) for x in xs]
+        run_cfg("mapreduce(x -> x + 1, +, Float32[2^28])", m, 4 * m, lambda i: ps[i % 2]())
+        del xs, ps
         m = 1 << 24
         xi = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(8)]
         ri = rk.ROCArray(dims=(1,), dtype=np.int64)
