@@ -8,6 +8,7 @@ build in parallel.  hipcc cross-compiles: no GPU is needed to build.
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -23,6 +24,8 @@ FLAGS = [
     # packed FP32 instructions are kept out of every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # per-kernel register / private-memory report of the device pass, checked below
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 # (source, object suffix, extra flags)
@@ -38,11 +41,48 @@ def _compile(unit):
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
     cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
-    # the host pass does not know the gfx feature flag and says so once per file: harmless
-    err = "\n".join(l for l in r.stderr.splitlines() if "not a recognized feature" not in l)
+    # No kernel of this library may keep an array in private memory: the ones that did (operand registers indexed with a
+    # computed address, a tile the optimizer failed to split into registers) ran 1.8-16x slower.  The report of the
+    # device pass gives private bytes per lane and spilled registers; a few spilled registers at the 128-register cap
+    # of the 1024-thread kernels are tolerated, anything beyond them is not.
+    private, lines, skip = [], [], 0
+    cur = {}
+
+    def close():
+        if cur and cur.get("scratch", 0) > 4 * cur.get("vspill", 0) + 8 or cur.get("vspill", 0) > 16:
+            private.append(f"{cur['name']}: {cur['scratch']} bytes of private memory per lane, {cur.get('vspill', 0)} spilled registers")
+    pending = []                     # "In file included from" lines belong to the diagnostic that follows them
+    for l in r.stderr.splitlines():
+        if l.startswith("In file included from"):
+            pending.append(l)
+            continue
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            pending = []
+            m = re.search(r"remark:\s+Function Name: (\S+)", l)
+            if m:
+                close()
+                cur = {"name": m.group(1)}
+            m = re.search(r"remark:\s+ScratchSize \[bytes/lane\]: (\d+)", l)
+            if m:
+                cur["scratch"] = int(m.group(1))
+            m = re.search(r"remark:\s+VGPRs Spill: (\d+)", l)
+            if m:
+                cur["vspill"] = int(m.group(1))
+            skip = 2 if "Function Name" in l else 0      # the remark's source line and caret follow
+            continue
+        if skip > 0:
+            skip -= 1
+            continue
+        # the host pass does not know the gfx feature flag and says so once per file: harmless
+        if "not a recognized feature" not in l:
+            lines.extend(pending)
+            lines.append(l)
+        pending = []
+    close()
+    err = "\n".join(lines)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}{suffix}:\n{err}")
-    return obj, err
+    return obj, err, [f"{src}{suffix}: {p}" for p in private]
 
 
 def build(jobs: int | None = None, verbose: bool = True) -> str:
@@ -50,10 +90,13 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
     jobs = jobs or min(8, os.cpu_count() or 1)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(_compile, UNITS))
-    for obj, err in results:
+    for obj, err, _ in results:
         if err.strip() and verbose:
             print(err, file=sys.stderr)
-    objs = [o for o, _ in results]
+    private = [p for _, _, ps in results for p in ps]
+    if private:
+        raise RuntimeError("kernels using private memory:\n  " + "\n  ".join(private))
+    objs = [o for o, _, _ in results]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -38,6 +38,7 @@ struct BcOperand {
 
 struct BcArgs {
     int32_t   n_operands, n_tokens;
+    int32_t   max_depth;               // of the value stack (entries beyond the registers live in LDS)
     int32_t   tokens[RK_MAX_PROGRAM];
     BcOperand op[RK_MAX_OPERANDS];
     int32_t   ndim;                    // merged rank (>= 1)
@@ -132,23 +133,30 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
 }
 
 // ---- evaluators ---------------------------------------------------------------------------------------
-// Postfix interpreter (rk_interp.hpp) over the loaded operands.
-template <typename CT, int VEC> struct BcFetch {
-    static constexpr int NOPS = RK_MAX_OPERANDS;
+// Postfix interpreter (rk_interp.hpp) over the loaded operands, one vector per run.  Two vectors (or rows) per run
+// would halve the scalar branches per element, but the kernel then needs 210-250 registers and loses more to
+// occupancy than it gains (sqrt(x*x+y*y)-w on 512^3: 500 -> 636 us).
+template <typename CT, int VEC, int NOPS_> struct BcFetch {
+    static constexpr int NOPS = NOPS_;
     const CT (&in)[RK_MAX_OPERANDS][VEC];
     template <int K> __device__ __forceinline__ void get(CT (&v)[VEC]) const {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = in[K][j];
     }
 };
-struct EvalInterp {
-    static constexpr int NOPS = RK_MAX_OPERANDS;   // load what the program declares
+template <int NOPS_> struct EvalInterpN {
+    static constexpr int NOPS = NOPS_;             // operand slots: load what the program declares, up to this many
     static constexpr bool USES_LDS = true;
     template <typename CT, int VEC>
     static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
-        interp_run<CT, VEC, BC_BLOCK, true>(a.tokens, a.n_tokens, BcFetch<CT, VEC>{in}, out, lds);
+        interp_run<CT, VEC, BC_BLOCK, true>(a.tokens, a.n_tokens, BcFetch<CT, VEC, NOPS_>{in}, out, lds);
     }
 };
+// Programs over at most 4 operands (most) run a copy with half the operand registers: in rows mode it can then keep
+// the loads of all of a thread's rows in flight at the occupancy of the general one, which goes row by row and is
+// bound by load latency ((A .- r) .* c .+ A on 16384^2: 1.6 TB/s).
+typedef EvalInterpN<RK_MAX_OPERANDS> EvalInterp;
+typedef EvalInterpN<4> EvalInterp4;
 
 // z = a * x + y * exp(w)            tokens: 0 1 MUL 2 3 EXP MUL ADD
 struct EvalAxpbyExp {
@@ -211,6 +219,65 @@ struct EvalBinary {
     }
 };
 
+// dest = (u op1 v) op2 w             tokens: u v <op1> w <op2>      (x .- m) ./ s,  a .* x .+ y,  x .* x .+ y
+// dest = u op1 (v op2 w)             tokens: u v w <op2> <op1>      x .+ y .* z with any arithmetic operators
+// Two scalar branches and no value stack: the three-operand trees that the interpreter would run at a third to
+// two thirds of the bandwidth.  The host renumbers the operands to u = 0, v = 1, w = 2 (an array that appears twice
+// gets two slots): choosing among the loaded operands in the kernel, by switch or by select, makes the compiler
+// index the operand registers with a computed address, i.e. move them to private memory (4x slower).
+struct EvalChain2 {
+    static constexpr int NOPS = 3;
+    static constexpr bool USES_LDS = false;
+    static bool chain_op(int t, bool int_compute) { return t >= RK_BC_ADD && t <= RK_BC_MIN && !(int_compute && t == RK_BC_DIV); }
+    // true: `c` is `a` with the operands in the order u, v, w and tokens 0 1 <op1> 2 <op2> or 0 1 2 <op2> <op1>
+    static bool canonical(const BcArgs& a, bool int_compute, BcArgs& c) {
+        if (a.n_tokens != 5) return false;
+        const int32_t* t = a.tokens;
+        auto opnd = [&](int i) { return t[i] >= 0 && t[i] < a.n_operands; };
+        if (!opnd(0) || !opnd(1) || !chain_op(t[4], int_compute)) return false;
+        const bool left = opnd(3);                  // (u op1 v) op2 w
+        if (left ? !chain_op(t[2], int_compute) : !(opnd(2) && chain_op(t[3], int_compute))) return false;
+        c = a;
+        c.n_operands = 3;
+        c.op[0] = a.op[t[0]];
+        c.op[1] = a.op[t[1]];
+        c.op[2] = a.op[left ? t[3] : t[2]];
+        c.tokens[0] = 0;
+        c.tokens[1] = 1;
+        if (left) { c.tokens[3] = 2; } else { c.tokens[2] = 2; }
+        return true;
+    }
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void apply(int tok, const CT (&x)[VEC], const CT (&y)[VEC], CT (&r)[VEC]) {
+#define RK_BC_BIN3(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT p = x[j], q = y[j]; r[j] = (EXPR); } } break
+        switch (tok) {
+            case RK_BC_ADD: RK_BC_BIN3(p + q);
+            case RK_BC_SUB: RK_BC_BIN3(p - q);
+            case RK_BC_MUL: RK_BC_BIN3(p * q);
+            case RK_BC_MAX: RK_BC_BIN3(OpMax()(p, q));
+            case RK_BC_MIN: RK_BC_BIN3(OpMin()(p, q));
+            default:
+                if constexpr (std::is_floating_point<CT>::value) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) r[j] = x[j] / y[j];
+                }
+                break;
+        }
+#undef RK_BC_BIN3
+    }
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        CT t[VEC];
+        if (a.tokens[3] == 2) {                     // (u op1 v) op2 w
+            apply<CT, VEC>(a.tokens[2], in[0], in[1], t);
+            apply<CT, VEC>(a.tokens[4], t, in[2], out);
+        } else {                                    // u op1 (v op2 w)
+            apply<CT, VEC>(a.tokens[3], in[1], in[2], t);
+            apply<CT, VEC>(a.tokens[4], in[0], t, out);
+        }
+    }
+};
+
 // ---- kernels --------------------------------------------------------------------------------------------
 extern __shared__ __align__(16) unsigned char bc_lds_raw[];
 
@@ -236,7 +303,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
         const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
-        constexpr int NB = Eval::USES_LDS ? 1 : (Eval::NOPS >= 4 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
+        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? (HOMOG ? BC_RPT : 2) : 1) : (Eval::NOPS >= 4 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
             int64_t doff[NB];
@@ -244,8 +311,11 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
             for (int b = 0; b < NB; ++b) {
                 int64_t row = row0 + r0 + b;
                 if (row >= a.nrows) row = a.nrows - 1;
+                // (the interpreter declares room for every operand slot: skip the 64-bit index arithmetic of the
+                // slots the program does not use -- it was most of that kernel's instructions in this mode)
 #pragma unroll
-                for (int k = 0; k < Eval::NOPS; ++k) off[k] = i0 * a.op[k].stride0;
+                for (int k = 0; k < Eval::NOPS; ++k)
+                    if (!Eval::USES_LDS || k < a.n_operands) off[k] = i0 * a.op[k].stride0;
                 doff[b] = i0 * a.dest_stride0;
                 int64_t rem = row;
                 for (int d = 1; d < a.ndim; ++d) {
@@ -253,7 +323,8 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
                     if (d == a.ndim - 1) c = rem;
                     else { c = rem % a.shape[d]; rem /= a.shape[d]; }
 #pragma unroll
-                    for (int k = 0; k < Eval::NOPS; ++k) off[k] += c * a.op[k].stride[d - 1];
+                    for (int k = 0; k < Eval::NOPS; ++k)
+                        if (!Eval::USES_LDS || k < a.n_operands) off[k] += c * a.op[k].stride[d - 1];
                     doff[b] += c * a.dest_stride[d - 1];
                 }
 #pragma unroll
@@ -304,7 +375,9 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
         if (a.nxb > 0x7fffffff || gz > 65535) return RK_ERR_TOO_LARGE;
         grid = dim3((unsigned)a.nxb, (unsigned)gy, (unsigned)gz);
     }
-    const size_t lds = Eval::USES_LDS ? (size_t)(BC_MAX_DEPTH - INTERP_REG_DEPTH) * VECN * BC_BLOCK * sizeof(CT) : 0;
+    // LDS only for the stack entries below the registers, i.e. for programs deeper than INTERP_REG_DEPTH
+    const int spill = Eval::USES_LDS && a.max_depth > INTERP_REG_DEPTH ? a.max_depth - INTERP_REG_DEPTH : 0;
+    const size_t lds = (size_t)spill * VECN * BC_BLOCK * sizeof(CT);
     // homogeneous element types: a kernel without any dispatch on the element type
     bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : (std::is_same<CT, double>::value ? RK_F64 : RK_I64));
     for (int k = 0; k < a.n_operands; ++k)
@@ -338,6 +411,11 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
     if (tokens_are(a, {0})) return bc_launch<EvalCopy, CT>(a, vec, rows, stream);
     if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 && a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW)
         return bc_launch<EvalBinary, CT>(a, vec, rows, stream);
+    {
+        BcArgs c;
+        if (EvalChain2::canonical(a, !std::is_floating_point<CT>::value, c)) return bc_launch<EvalChain2, CT>(c, vec, rows, stream);
+    }
+    if (a.n_operands <= EvalInterp4::NOPS) return bc_launch<EvalInterp4, CT>(a, vec, rows, stream);
     return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
 }
 
@@ -355,8 +433,9 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
     if (prog->n_operands < 0 || prog->n_operands > RK_MAX_OPERANDS) return RK_ERR_INVALID_ARGUMENT;
     if (prog->n_tokens < 1 || prog->n_tokens > RK_MAX_PROGRAM) return RK_ERR_INVALID_ARGUMENT;
 
+    int max_depth = 0;
     {
-        const int32_t st = validate_tokens(prog->tokens, prog->n_tokens, prog->n_operands, int_compute, BC_MAX_DEPTH);
+        const int32_t st = validate_tokens(prog->tokens, prog->n_tokens, prog->n_operands, int_compute, BC_MAX_DEPTH, &max_depth);
         if (st != RK_SUCCESS) return st;
     }
 
@@ -420,6 +499,7 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
 
     a.n_operands = prog->n_operands;
     a.n_tokens = prog->n_tokens;
+    a.max_depth = max_depth;
     for (int i = 0; i < prog->n_tokens; ++i) a.tokens[i] = prog->tokens[i];
     a.ndim = m;
     a.total = total;

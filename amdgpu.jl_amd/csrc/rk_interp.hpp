@@ -36,7 +36,8 @@ __host__ __device__ constexpr bool token_basic(int tok) {
 }
 
 // A well-formed postfix expression that leaves exactly one value; operand tokens are 0 .. n_operands-1.
-inline int32_t validate_tokens(const int32_t* tokens, int n_tokens, int n_operands, bool int_compute, int max_allowed_depth) {
+inline int32_t validate_tokens(const int32_t* tokens, int n_tokens, int n_operands, bool int_compute, int max_allowed_depth,
+                               int* depth_out = nullptr) {
     int depth = 0, max_depth = 0;
     for (int i = 0; i < n_tokens; ++i) {
         const int tok = tokens[i];
@@ -53,6 +54,7 @@ inline int32_t validate_tokens(const int32_t* tokens, int n_tokens, int n_operan
     }
     if (depth != 1) return RK_ERR_INVALID_ARGUMENT;
     if (max_depth > max_allowed_depth) return RK_ERR_UNSUPPORTED;
+    if (depth_out) *depth_out = max_depth;
     return RK_SUCCESS;
 }
 

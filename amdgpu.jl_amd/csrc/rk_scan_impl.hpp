@@ -126,8 +126,10 @@ struct ScanGeom {
 // scan inside the lane, DPP scan across the wave, carry to the next load; wave totals meet in LDS.
 template <typename T, typename Op, int K> struct TileRegs {
     static constexpr int VEC = 16 / sizeof(T);
-    T v[K][VEC];     // inclusive scan inside each lane's vector
-    T excl[K];       // exclusive prefix of that vector inside the wave's quarter
+    // vector values, not T v[K][VEC]: with the array form the 64-bit integer instantiations kept the tile in private
+    // memory (a store and a load per element: cumsum of Int64[2^26] 342 us against 191 us for Float64)
+    typename VecOf<T, VEC>::type v[K];     // inclusive scan inside each lane's vector
+    T excl[K];                             // exclusive prefix of that vector inside the wave's quarter
 };
 
 template <typename In, typename T, typename Op, bool VECTOR, int K, int NW = 4>

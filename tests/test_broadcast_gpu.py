@@ -177,3 +177,38 @@ def test_integer_programs_are_exact_and_wrap(rk):
     # copies of Int64 beyond 2^53 are exact
     big = np.array([2**62 + 1, -(2**62) - 3, 2**53 + 1], dtype=np.int64)
     assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(big)))), big)
+
+
+def test_three_operand_trees_all_operator_pairs(rk):
+    """(u op1 v) op2 w and u op1 (v op2 w) run on a fused evaluator: every operator pair, both shapes, repeated and
+    scalar and extruded operands; Float32 results equal NumPy's un-fused Float32 arithmetic bit for bit."""
+    rng = _rng(21)
+    shape = (132, 77)
+    x = (rng.random(shape, dtype=np.float32) + np.float32(0.5))
+    y = (rng.random(shape, dtype=np.float32) + np.float32(0.5))
+    col = (rng.random((132, 1), dtype=np.float32) + np.float32(0.5))
+    row = (rng.random((1, 77), dtype=np.float32) + np.float32(0.5))
+    X, Y, Cc, R = (rk.ROCArray(a) for a in (x, y, col, row))
+    B = rk.broadcast
+    ops = {"+": (lambda a, b: a + b, np.add), "-": (lambda a, b: a - b, np.subtract), "*": (lambda a, b: a * b, np.multiply),
+           "/": (lambda a, b: a / b, np.divide), "max": (B.max_, np.maximum), "min": (B.min_, np.minimum)}
+    two = np.float32(2)
+    triples = [((X, x), (Y, y), (Cc, col)), ((X, x), (X, x), (Y, y)), ((two, two), (X, x), (R, row)), ((Cc, col), (R, row), (X, x))]
+    lz = rk.lazy
+    for (u, hu), (v, hv), (w, hw) in triples:
+        for n1, (f1, g1) in ops.items():
+            for n2, (f2, g2) in ops.items():
+                got = rk.Array(rk.materialize(f2(f1(lz(u), lz(v)), lz(w))))
+                np.testing.assert_array_equal(got, g2(g1(hu, hv), hw).astype(np.float32), err_msg=f"({n1}) {n2}")
+                got = rk.Array(rk.materialize(f1(lz(u), f2(lz(v), lz(w)))))
+                np.testing.assert_array_equal(got, g1(hu, g2(hv, hw)).astype(np.float32), err_msg=f"{n1} ({n2})")
+    k = rng.integers(-2**31, 2**31, shape).astype(np.int32)
+    j = rng.integers(-2**31, 2**31, shape).astype(np.int32)
+    K, J = rk.ROCArray(k), rk.ROCArray(j)
+    with np.errstate(over="ignore"):
+        for n1 in ("+", "-", "*"):
+            for n2 in ("+", "-", "*"):
+                f1, g1 = ops[n1]
+                f2, g2 = ops[n2]
+                got = rk.materialize(f2(f1(lz(K), lz(J)), lz(K)))
+                assert got.dtype == np.int32 and np.array_equal(rk.Array(got), g2(g1(k, j), k)), (n1, n2)
