@@ -343,11 +343,19 @@ def accumulate(op: str, A: np.ndarray, dims=None, init=None, inclusive: bool = T
             raise ValueError("dims must be >= 1")
         axis = dims - 1
     if axis >= A.ndim:
-        out = a.copy()
+        out = a.copy()                        # every element is a line of length 1: out[i] = op(init, A[i])
         if init is not None:
+            seed = a.dtype.type(init)
             with np.errstate(over="ignore"):
-                out = out + a.dtype.type(init) if op == "add" else out * a.dtype.type(init)
+                if op == "add":
+                    out = out + seed
+                elif op == "mul":
+                    out = out * seed
+                else:
+                    out = (np.maximum if op == "max" else np.minimum)(out, seed)
         if not inclusive:
+            if init is None and op in ("max", "min"):
+                raise ValueError("exclusive max/min scans need init")
             neutral = a.dtype.type(0 if op == "add" else 1)
             out = np.full_like(a, neutral if init is None else a.dtype.type(init))
         return out

@@ -196,6 +196,11 @@ def test_accumulate_exclusive_and_ops():
     assert orc.accumulate("max", x).tolist() == [3, 3, 4, 4, 5]
     assert orc.accumulate("min", x, init=2).tolist() == [2, 1, 1, 1, 1]
     assert orc.cumprod(np.array([1.5, 2.0])).tolist() == [1.5, 3.0]                                  # :224
+    # a dim beyond ndims: every element is a line of length one, out[i] = op(init, x[i]) for every operator
+    assert orc.accumulate("min", x, dims=2, init=2).tolist() == [2, 1, 2, 1, 2]
+    assert orc.accumulate("max", x, dims=2, init=2).tolist() == [3, 2, 4, 2, 5]
+    assert orc.accumulate("mul", x, dims=3, init=2).tolist() == [6, 2, 8, 2, 10]
+    assert orc.accumulate("add", x, dims=2, init=2, inclusive=False).tolist() == [2, 2, 2, 2, 2]
 
 
 def test_findall_matches_definition():
