@@ -175,3 +175,38 @@ def test_random_broadcasts(rk):
             assert got.dtype == np.bool_ and np.array_equal(got, want)
         else:
             np.testing.assert_array_equal(got, want.astype(np.float32))      # un-fused Float32 arithmetic: bit for bit
+
+
+def test_random_sorts_and_selections(rk, orc):
+    rng = np.random.default_rng(1006 + SEED)
+    sizes = EXTENTS + [65_536, 100_003, 300_000, (1 << 20) + 5]
+    for case in range(80):
+        n = int(rng.choice(sizes))
+        dtype = [np.float32, np.float64, np.int32, np.int64, np.int16, np.float16][int(rng.integers(6))]
+        rev = bool(rng.random() < 0.4)
+        spread = [3, 1000, 2**15 - 1][int(rng.integers(3))]           # many ties / few ties
+        _say("sort", case, n, np.dtype(dtype).name, "rev" if rev else "fwd", spread)
+        if np.dtype(dtype).kind == "f":
+            with np.errstate(over="ignore"):                          # Float16 overflows to +-Inf: fine, Inf sorts too
+                x = (rng.standard_normal(n) * spread).astype(dtype)
+            x[rng.random(n) < 0.01] = np.nan
+            x[rng.random(n) < 0.01] = -0.0
+            x[rng.random(n) < 0.01] = 0.0
+        else:
+            x = rng.integers(-spread, spread + 1, n).astype(dtype)
+        dx = rk.ROCArray(x)
+        got = rk.Array(rk.sort(dx, rev=rev))
+        want = orc.sort(x, rev=rev)
+        assert got.dtype == x.dtype and np.array_equal(got, want, equal_nan=True)
+        if x.dtype.kind == "f":
+            assert np.array_equal(np.signbit(got[~np.isnan(got)]), np.signbit(want[~np.isnan(want)]))
+        assert np.array_equal(rk.Array(rk.sortperm(dx, rev=rev)), orc.sortperm(x, rev=rev))       # stable: one answer
+    for case in range(80):
+        shape = _shape(rng)
+        density = [0.0, 0.001, 0.3, 0.9, 1.0][int(rng.integers(5))]
+        _say("findall", case, shape, density)
+        m = rng.random(shape) < density
+        got = rk.Array(rk.findall(rk.ROCArray(m)))
+        want = orc.findall(m)
+        assert np.array_equal(got, want if len(shape) == 1 else want.T)
+        assert rk.count(rk.ROCArray(m)) == int(m.sum())
