@@ -278,6 +278,53 @@ struct EvalChain2 {
     }
 };
 
+// dest = (((u0 op1 u1) op2 u2) ... opn un)      tokens: u0 u1 <op1> u2 <op2> ... un <opn>, up to 8 operands
+// e.g. (x .- m) ./ s .* g .+ b.  One scalar branch per operator and no value stack; operands renumbered on the host
+// to u_k = slot k, like EvalChain2.  In rows mode the interpreter is instruction-bound (1.9 TB/s on 16384^2).
+// Instantiated for 4, 6 and 8 operand slots: in rows mode every slot costs scalar registers for its pointer and
+// strides, and the 8-slot kernel spills some sixty of them ((A .- m) ./ s .* g .+ b with four row vectors on
+// 16384^2: 2.0 TB/s with 8 slots, 2.6 with 6; a four-operand chain: 2.2 -> 3.9).  An array that appears twice is
+// loaded twice.
+template <int NOPS_> struct EvalLeftChainN {
+    static constexpr int NOPS = NOPS_;
+    static constexpr bool USES_LDS = false;
+    static bool canonical(const BcArgs& a, bool int_compute, BcArgs& c) {
+        const int n = (a.n_tokens + 1) / 2;         // operands of the chain
+        if (a.n_tokens < 7 || a.n_tokens % 2 == 0 || n > RK_MAX_OPERANDS) return false;
+        const int32_t* t = a.tokens;
+        auto opnd = [&](int i) { return t[i] >= 0 && t[i] < a.n_operands; };
+        if (!opnd(0)) return false;
+        for (int k = 1; k < n; ++k)
+            if (!opnd(2 * k - 1) || !EvalChain2::chain_op(t[2 * k], int_compute)) return false;
+        c = a;
+        c.n_operands = n;
+        c.op[0] = a.op[t[0]];
+        c.tokens[0] = 0;
+        for (int k = 1; k < n; ++k) {
+            c.op[k] = a.op[t[2 * k - 1]];
+            c.tokens[2 * k - 1] = k;
+        }
+        return true;
+    }
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        CT acc[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = in[0][j];
+#pragma unroll
+        for (int k = 1; k < NOPS_; ++k) {
+            if (k < a.n_operands) {
+                CT r[VEC];
+                EvalChain2::apply<CT, VEC>(a.tokens[2 * k], acc, in[k], r);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = r[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = acc[j];
+    }
+};
+
 // ---- kernels --------------------------------------------------------------------------------------------
 extern __shared__ __align__(16) unsigned char bc_lds_raw[];
 
@@ -303,7 +350,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
         const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
-        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? (HOMOG ? BC_RPT : 2) : 1) : (Eval::NOPS >= 4 ? 2 : BC_RPT);   // keeps the kernel under 64 VGPRs
+        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? (HOMOG ? BC_RPT : 2) : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
             int64_t doff[NB];
@@ -414,13 +461,32 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
     {
         BcArgs c;
         if (EvalChain2::canonical(a, !std::is_floating_point<CT>::value, c)) return bc_launch<EvalChain2, CT>(c, vec, rows, stream);
+        if (EvalLeftChainN<8>::canonical(a, !std::is_floating_point<CT>::value, c)) {
+            if (c.n_operands <= 4) return bc_launch<EvalLeftChainN<4>, CT>(c, vec, rows, stream);
+            if (c.n_operands <= 6) return bc_launch<EvalLeftChainN<6>, CT>(c, vec, rows, stream);
+            return bc_launch<EvalLeftChainN<8>, CT>(c, vec, rows, stream);
+        }
     }
     if (a.n_operands <= EvalInterp4::NOPS) return bc_launch<EvalInterp4, CT>(a, vec, rows, stream);
     return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
 }
 
+// This file is compiled once per compute type (-DRK_BC_INST=0, 1, 2: Float32, Float64, Int64 kernels) and once
+// without the macro for the C entry points, so that the kernel sets build in parallel.
+int32_t bc_dispatch_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+int32_t bc_dispatch_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+int32_t bc_dispatch_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+#if defined(RK_BC_INST) && RK_BC_INST == 0
+int32_t bc_dispatch_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<float>(a, vec, rows, stream); }
+#elif defined(RK_BC_INST) && RK_BC_INST == 1
+int32_t bc_dispatch_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<double>(a, vec, rows, stream); }
+#elif defined(RK_BC_INST) && RK_BC_INST == 2
+int32_t bc_dispatch_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<int64_t>(a, vec, rows, stream); }
+#endif
+
 }  // namespace rk
 
+#ifndef RK_BC_INST
 using namespace rk;
 
 static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
@@ -547,9 +613,9 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
         a.tx_log2 = l2;
         a.nxb = (n0v + (1ll << l2) - 1) >> l2;
     }
-    if (prog->compute == RK_F32) return bc_dispatch<float>(a, vec, !linear, (hipStream_t)stream);
-    if (int_compute) return bc_dispatch<int64_t>(a, vec, !linear, (hipStream_t)stream);
-    return bc_dispatch<double>(a, vec, !linear, (hipStream_t)stream);
+    if (prog->compute == RK_F32) return bc_dispatch_f32(a, vec, !linear, (hipStream_t)stream);
+    if (int_compute) return bc_dispatch_i64(a, vec, !linear, (hipStream_t)stream);
+    return bc_dispatch_f64(a, vec, !linear, (hipStream_t)stream);
 }
 
 extern "C" int32_t rk_broadcast(const rk_program* prog, void* dest, rk_dtype dest_dtype, int ndim, const int64_t* shape,
@@ -561,3 +627,4 @@ extern "C" int32_t rk_broadcast_strided(const rk_program* prog, void* dest, rk_d
                                         const int64_t* dest_strides, void* stream) {
     return broadcast_impl(prog, dest, dest_dtype, ndim, shape, dest_strides, stream);
 }
+#endif  // RK_BC_INST

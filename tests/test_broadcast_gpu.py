@@ -212,3 +212,32 @@ def test_three_operand_trees_all_operator_pairs(rk):
                 f2, g2 = ops[n2]
                 got = rk.materialize(f2(f1(lz(K), lz(J)), lz(K)))
                 assert got.dtype == np.int32 and np.array_equal(rk.Array(got), g2(g1(k, j), k)), (n1, n2)
+
+
+def test_left_deep_chains(rk):
+    """((u0 op u1) op u2) ... up to eight operands run without a value stack; same bits as NumPy's Float32."""
+    rng = _rng(22)
+    shape = (260, 37)
+    full = [rng.random(shape, dtype=np.float32) + np.float32(0.5) for _ in range(3)]
+    col = rng.random((260, 1), dtype=np.float32) + np.float32(0.5)
+    row = rng.random((1, 37), dtype=np.float32) + np.float32(0.5)
+    row2 = rng.random((1, 37), dtype=np.float32) + np.float32(0.5)
+    hosts = [full[0], row, row2, col, full[1], np.float32(1.5), full[2], full[0]]
+    devs = [rk.ROCArray(h) if isinstance(h, np.ndarray) else h for h in hosts]
+    lz = rk.lazy
+    B = rk.broadcast
+    gpu_ops = [lambda a, b: a - b, lambda a, b: a / b, lambda a, b: a * b, lambda a, b: a + b, B.max_, B.min_, lambda a, b: a - b]
+    cpu_ops = [np.subtract, np.divide, np.multiply, np.add, np.maximum, np.minimum, np.subtract]
+    for n in range(4, 9):                                     # 4 .. 8 operands (3 have their own evaluator)
+        for shift in range(3):
+            g, c = lz(devs[0]), hosts[0]
+            for k in range(1, n):
+                j = (k - 1 + shift) % len(gpu_ops)
+                g = gpu_ops[j](g, lz(devs[k]))
+                c = cpu_ops[j](c, hosts[k])
+            np.testing.assert_array_equal(rk.Array(rk.materialize(g)), c.astype(np.float32), err_msg=f"{n} operands, shift {shift}")
+    k = rng.integers(-2**31, 2**31, (4, 1000)).astype(np.int32)
+    K = rk.ROCArray(k)
+    with np.errstate(over="ignore"):
+        got = rk.materialize(((lz(K) * lz(K) - lz(K)) * np.int32(3) + lz(K)) * lz(K))
+        assert got.dtype == np.int32 and np.array_equal(rk.Array(got), ((k * k - k) * np.int32(3) + k) * k)
