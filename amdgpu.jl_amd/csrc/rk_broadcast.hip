@@ -54,8 +54,22 @@ struct BcArgs {
 };
 
 // ---- typed loads / stores --------------------------------------------------------------------------
+// One element at an address that is the same in every lane of the wave (an operand extruded along dim 0 -- a row
+// vector against a matrix -- when a wave's lanes share their row), from memory the kernel does not write (an operand
+// with an extruded dim cannot be the destination): a scalar load.  As a vector load the same request occupies the
+// texture path like a full 64-lane access, once per row and operand.
+template <typename S> __device__ __forceinline__ S load_wave_uniform(const S* q) {
+    const uint64_t p = (uint64_t)q;
+    // (the builtin returns a signed int: without the casts the low word is sign-extended over the high one)
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));
+    const uint64_t u = ((uint64_t)hi << 32) | (uint64_t)lo;
+    typedef const S __attribute__((address_space(4))) * ConstPtr;
+    return *(ConstPtr)u;
+}
+
 template <typename CT, typename S, int VEC, bool CACHED>
-__device__ __forceinline__ void load_as(const void* p, int64_t off, bool contiguous, CT (&v)[VEC]) {
+__device__ __forceinline__ void load_as(const void* p, int64_t off, bool contiguous, bool wave_uniform, CT (&v)[VEC]) {
     const S* q = (const S*)p + off;
     if (contiguous) {
         if constexpr (VEC == 1) v[0] = (CT)q[0];
@@ -68,7 +82,9 @@ __device__ __forceinline__ void load_as(const void* p, int64_t off, bool contigu
             for (int j = 0; j < VEC; ++j) v[j] = (CT)x[j];
         }
     } else {
-        const CT x = (CT)q[0];
+        CT x;
+        if constexpr (sizeof(S) >= 4) x = wave_uniform ? (CT)load_wave_uniform(q) : (CT)q[0];
+        else x = (CT)q[0];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = x;
     }
@@ -77,23 +93,23 @@ __device__ __forceinline__ void load_as(const void* p, int64_t off, bool contigu
 // HOMOG: every array operand and the destination already have the compute type -- no dispatch on the
 // element type anywhere in the kernel (the common all-Float32 / all-Float64 case).
 template <typename CT, int VEC, bool CACHED, bool HOMOG>
-__device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool contiguous, CT (&v)[VEC]) {
-    if constexpr (HOMOG) { load_as<CT, CT, VEC, CACHED>(o.ptr, off, contiguous, v); return; }
+__device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool contiguous, bool wave_uniform, CT (&v)[VEC]) {
+    if constexpr (HOMOG) { load_as<CT, CT, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); return; }
     switch (o.dtype) {
-        case RK_F32: load_as<CT, float, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        case RK_F64: load_as<CT, double, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        case RK_I32: load_as<CT, int32_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        case RK_I64: load_as<CT, int64_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        case RK_U32: load_as<CT, uint32_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        case RK_U64: load_as<CT, uint64_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
-        default:     load_as<CT, uint8_t, VEC, CACHED>(o.ptr, off, contiguous, v); break;
+        case RK_F32: load_as<CT, float, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_F64: load_as<CT, double, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_I32: load_as<CT, int32_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_I64: load_as<CT, int64_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_U32: load_as<CT, uint32_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_U64: load_as<CT, uint64_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        default:     load_as<CT, uint8_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
     }
 }
 
 // MAY_REUSE: rows mode, where an extruded operand is read again and again and should stay cached; the flat
 // mode reads every dense operand exactly once and always streams (one branch less per operand).
 template <typename CT, int VEC, bool MAY_REUSE, bool HOMOG>
-__device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT (&v)[VEC]) {
+__device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, bool wave_rows, CT (&v)[VEC]) {
     if (o.ptr == nullptr) {
         const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64) ? (CT)o.sf : (CT)o.si;
 #pragma unroll
@@ -101,8 +117,8 @@ __device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, CT
         return;
     }
     const bool contiguous = o.stride0 != 0;     // on the vector path stride0 is 0 or 1; scalar lanes carry any stride in `off`
-    if (MAY_REUSE && o.reused != 0) load_typed<CT, VEC, true, HOMOG>(o, off, contiguous, v);
-    else load_typed<CT, VEC, false, HOMOG>(o, off, contiguous, v);
+    if (MAY_REUSE && o.reused != 0) load_typed<CT, VEC, true, HOMOG>(o, off, contiguous, wave_rows, v);
+    else load_typed<CT, VEC, false, HOMOG>(o, off, contiguous, false, v);
 }
 
 template <typename CT, typename D, int VEC>
@@ -350,6 +366,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
         const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
+        const bool wave_rows = a.tx_log2 >= 6;     // 64 or more lanes along dim 0: the lanes of a wave share their rows
         constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? (HOMOG ? BC_RPT : 2) : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
@@ -377,7 +394,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
 #pragma unroll
                 for (int k = 0; k < Eval::NOPS; ++k) {
                     if (k >= a.n_operands) continue;
-                    if (b == 0 || !a.op[k].row_invariant) load_operand<CT, VEC, true, HOMOG>(a.op[k], off[k], in[b][k]);
+                    if (b == 0 || !a.op[k].row_invariant) load_operand<CT, VEC, true, HOMOG>(a.op[k], off[k], wave_rows, in[b][k]);
                     else {
 #pragma unroll
                         for (int j = 0; j < VEC; ++j) in[b][k][j] = in[0][k][j];
@@ -399,7 +416,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
     CT in[RK_MAX_OPERANDS][VEC];
 #pragma unroll
     for (int k = 0; k < Eval::NOPS; ++k)
-        if (k < a.n_operands) load_operand<CT, VEC, false, HOMOG>(a.op[k], off[k], in[k]);
+        if (k < a.n_operands) load_operand<CT, VEC, false, HOMOG>(a.op[k], off[k], false, in[k]);
     CT out[VEC];
     Eval::template run<CT, VEC>(a, in, out, lds);
     store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, dest_off, out);
