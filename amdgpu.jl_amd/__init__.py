@@ -8,7 +8,7 @@ without the built library raises.
 from ._lib import (RKError, DimensionMismatch, UnsupportedError, lib, LIB_PATH)       # noqa: F401
 from .array import ROCArray, Array, similar, zeros, workspace                         # noqa: F401
 from .mapreduce import (mapreduce, mapreducedim_, sum, prod, maximum, minimum, count, # noqa: F401,A004
-                        findmax, findmin, any, all, findfirst, reduce_eltype, identity, abs2, abs_,
+                        findmax, findmin, argmax, argmin, extrema, any, all, findfirst, reduce_eltype, identity, abs2, abs_,
                         add_sum, mul_prod, add, mul, max_, min_)
 from .accumulate import accumulate, accumulate_, cumsum, cumprod, accumulate_eltype    # noqa: F401
 from . import broadcast                                                               # noqa: F401

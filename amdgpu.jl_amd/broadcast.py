@@ -342,7 +342,46 @@ def materialize_(dest: ROCArray, bc) -> ROCArray:
     return dest
 
 
-def _launch_broadcast(dest, operands, tokens, compute):
+def _extent(a):
+    """(first byte, one past the last byte, identity of the layout) of the memory an array or wrapper addresses."""
+    size = a.dtype.itemsize
+    if isinstance(a, ROCView):
+        lo = hi = a.sptr
+        for n, st in zip(a.dims, a.strides):
+            if n == 0:
+                return a.sptr, a.sptr, None
+            span = (n - 1) * st * size
+            lo, hi = (lo + span, hi) if span < 0 else (lo, hi + span)
+        return lo, hi + size, (a.sptr, a.dims, a.strides)
+    dense, st = [], 1
+    for n in a.dims:
+        dense.append(st)
+        st *= n
+    return a.ptr, a.ptr + len(a) * size, (a.ptr, a.dims, tuple(dense))
+
+
+def _unalias(dest, operands):
+    """``Broadcast.broadcast_unalias``: an operand that may share memory with the destination without being the very
+    same elements in the same places (``x .= x .+ 1`` is fine; ``@view(A[1:4, :]) .= @view(A[2:5, :])`` is not) is
+    copied first, so the kernel never reads an element another lane has already overwritten."""
+    from .views import copy as copy_view
+    dlo, dhi, dident = _extent(dest)
+    out = []
+    for o in operands:
+        if isinstance(o, _ARRAYS) and len(o) > 0 and dhi > dlo:
+            lo, hi, ident = _extent(o)
+            if lo < dhi and dlo < hi and ident != dident:
+                o = copy_view(o) if isinstance(o, ROCView) else o.copy()
+        out.append(o)
+    return out
+
+
+def _launch_broadcast(dest, operands, tokens, compute, repeatable=False):
+    fresh = _unalias(dest, operands)
+    if repeatable and builtins.any(a is not b for a, b in zip(fresh, operands)):
+        # a plan would keep reading the copy made now
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "a prepared broadcast whose operand aliases the destination")
+    operands = fresh
     prog = _program(operands, tokens, compute, dest.ndim)
     keep = operands          # the program holds raw device pointers: keep the arrays alive with the plan
     if isinstance(dest, ROCView):                  # `@view(C[...]) .= bc`, `transpose(C) .= bc`
@@ -366,7 +405,7 @@ def plan_materialize(dest: ROCArray, bc):
         full = full[:-1]
     if full != dest.dims or len(dest) == 0:
         raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"destination {dest.dims} vs broadcast shape {shape}")
-    return _launch_broadcast(dest, operands, tokens, compute)
+    return _launch_broadcast(dest, operands, tokens, compute, repeatable=True)
 
 
 def materialize(bc) -> ROCArray:

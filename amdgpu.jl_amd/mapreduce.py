@@ -335,6 +335,21 @@ def findmin(A: ROCArray, dims=None):
     return _findminmax(A, False, dims)
 
 
+def argmax(A: ROCArray, dims=None):
+    """``argmax(A; dims)`` = the index half of ``findmax`` (the kernel skips the value output)."""
+    return _findminmax(A, True, dims)[1]
+
+
+def argmin(A: ROCArray, dims=None):
+    return _findminmax(A, False, dims)[1]
+
+
+def extrema(*args, dims=None):
+    """``extrema(A; dims)`` / ``extrema(f, A; dims)``: (minimum, maximum) -- host scalars, or two ROCArrays with
+    ``dims`` (Julia returns one array of tuples; the pair of arrays holds the same values)."""
+    return minimum(*args, dims=dims), maximum(*args, dims=dims)
+
+
 def plan_findmax(A: ROCArray, vals: ROCArray, idx: ROCArray, dims, want_max: bool = True):
     """Callable that repeats ``findmax(A; dims)`` into preallocated outputs."""
     mask = _dims_mask(dims, A.ndim)

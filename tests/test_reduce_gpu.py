@@ -277,3 +277,18 @@ def test_unsigned_reductions(rk, orc, dtype):
         with np.errstate(over="ignore"):
             want = A.sum(dtype=dtype) if dims is None else A.sum(axis=tuple(x - 1 for x in ((dims,) if isinstance(dims, int) else dims)), keepdims=True, dtype=dtype)
         assert np.array_equal(np.asarray(r if dims is None else rk.Array(r)), want)
+
+
+def test_argmax_argmin_extrema(rk, orc):
+    rng = _rng(41)
+    A = rng.integers(-50, 51, (37, 1001)).astype(np.float32)
+    dA = rk.ROCArray(A)
+    assert rk.argmax(dA) == orc.findmax(A)[1] and rk.argmin(dA) == orc.findmin(A)[1]
+    for dims in (1, 2):
+        assert np.array_equal(np.moveaxis(rk.Array(rk.argmax(dA, dims=dims)), 0, -1), orc.findmax(A, dims=dims)[1])
+        assert np.array_equal(np.moveaxis(rk.Array(rk.argmin(dA, dims=dims)), 0, -1), orc.findmin(A, dims=dims)[1])
+        lo, hi = rk.extrema(dA, dims=dims)
+        assert np.array_equal(rk.Array(lo), A.min(axis=dims - 1, keepdims=True)) and np.array_equal(rk.Array(hi), A.max(axis=dims - 1, keepdims=True))
+    assert rk.extrema(dA) == (A.min(), A.max())
+    lo, hi = rk.extrema(lambda v: v * v, dA)
+    assert (lo, hi) == ((A * A).min(), (A * A).max())

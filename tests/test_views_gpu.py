@@ -91,3 +91,29 @@ def test_views_are_refused_by_dense_ops(rk):
         rk.view(d, (1, 5), None)
     with pytest.raises(IndexError):
         rk.view(d, 4, None)
+
+
+def test_operands_that_alias_the_destination_are_copied_first(rk):
+    """``Broadcast.broadcast_unalias``: the right-hand side is evaluated as if no element had been written yet."""
+    rng = np.random.default_rng(31)
+    a = rng.standard_normal((300, 257)).astype(np.float32)
+    A = rk.ROCArray(a)
+    rk.materialize_(rk.view(A, (1, 299), None), rk.lazy(rk.view(A, (2, 300), None)) + np.float32(1))     # rows move up by one
+    want = a.copy()
+    want[0:299, :] = a[1:300, :] + np.float32(1)
+    assert np.array_equal(rk.Array(A), want)
+    s = rng.standard_normal((129, 129)).astype(np.float32)
+    S = rk.ROCArray(s)
+    rk.materialize_(S, rk.lazy(rk.transpose(S)) * np.float32(2))                                       # S .= 2 .* transpose(S)
+    assert np.array_equal(rk.Array(S), s.T * np.float32(2))
+    x = rng.standard_normal(10_001).astype(np.float32)
+    X = rk.ROCArray(x)
+    rk.materialize_(X, rk.lazy(X) * rk.lazy(X) + np.float32(1))                                         # the same elements in place
+    assert np.array_equal(rk.Array(X), x * x + np.float32(1))
+    rk.materialize_(rk.view(X, (1, 5000)), rk.lazy(rk.view(X, (5001, -1, 2))))                          # reversed overlapping range
+    want = x * x + np.float32(1)
+    want[0:5000] = want[1:5001][::-1].copy()
+    assert np.array_equal(rk.Array(X), want)
+    from amdgpu_jl_amd.broadcast import plan_materialize
+    with pytest.raises(rk.UnsupportedError):
+        plan_materialize(rk.view(A, (1, 299), None), rk.lazy(rk.view(A, (2, 300), None)))
