@@ -47,7 +47,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU; the path has no multi-GPU part "
-              "(every op shards without communication, see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "(every op shards along its non-reduced extent without communication). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
