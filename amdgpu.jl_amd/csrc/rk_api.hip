@@ -161,6 +161,7 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
     if (in == out) {
         switch (in) {
             case RK_F32: return mapreduce_f32(a);
+            case RK_F16: return mapreduce_f16(a);
             case RK_F64: return mapreduce_f64(a);
             case RK_I32: return mapreduce_i32(a);
             case RK_I64: return mapreduce_i64(a);
@@ -217,6 +218,7 @@ int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, co
     FindArgs a{want_max ? 1 : 0, A, ndim, shape, reduce_mask, vals, cart_idx, ws, ws_bytes, (hipStream_t)stream};
     switch (in) {
         case RK_F32: return findminmax_f32(a);
+        case RK_F16: return findminmax_f16(a);
         case RK_F64: return findminmax_f64(a);
         case RK_I32: return findminmax_i32(a);
         case RK_I64: return findminmax_i64(a);

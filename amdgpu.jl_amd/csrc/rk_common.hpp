@@ -382,6 +382,13 @@ template <> struct OrderKey<float> {
         return __builtin_bit_cast(float, kk ^ ((kk >> 31) & 0x7fffffff));
     }
 };
+typedef _Float16 half_t;
+template <> struct OrderKey<half_t> {             // through Float32: exact both ways
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
+    static __device__ __forceinline__ Key make(half_t v, bool want_max) { return OrderKey<float>::make((float)v, want_max); }
+    static __device__ __forceinline__ half_t value(Key k, bool want_max) { return (half_t)OrderKey<float>::value(k, want_max); }
+};
 template <> struct OrderKey<double> {
     typedef int64_t Key;
     static constexpr bool LOWEST_FREE = true;

@@ -102,11 +102,12 @@ __device__ __forceinline__ void map_batch(const In (&x)[TOTAL], Acc (&m)[TOTAL],
 
 // ---- result sinks ---------------------------------------------------------------------------
 // Called as sink(output index q, reduced value).
-template <typename Acc, typename Op> struct ReduceSink {
-    Acc* R;
+// Out differs from Acc for Float16 arrays (accumulated in Float32, rounded once at the end).
+template <typename Acc, typename Op, typename Out = Acc> struct ReduceSink {
+    Out* R;
     Acc  init;
     int  has_init;
-    __device__ __forceinline__ void operator()(int64_t q, Acc t) const { R[q] = has_init ? Op()(init, t) : t; }
+    __device__ __forceinline__ void operator()(int64_t q, Acc t) const { R[q] = (Out)(has_init ? Op()(init, t) : t); }
 };
 template <typename T, typename P> struct ArgSink {
     T*       vals;
@@ -646,9 +647,9 @@ struct FindArgs {
 // a temporary at the top of the partials area -- and the remaining dims are reduced from that much smaller array.
 constexpr size_t REDUCE_TEMP_MAX = WS_PARTIALS_BYTES / 2;
 
-template <typename In, typename Acc, typename Xf, typename Op>
+template <typename In, typename Acc, typename Xf, typename Op, typename Out = Acc>
 inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
-    ReduceSink<Acc, Op> sink{(Acc*)a.R, a.init ? *(const Acc*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
+    ReduceSink<Acc, Op, Out> sink{(Out*)a.R, a.init ? (Acc)*(const Out*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
     const Shape3 s = collapse3(a.ndim, a.shape, a.mask);
     if (!s.single_run && s.total > 0) {
         uint32_t mask1 = 0;                       // the lowest run of reduced dims (extents of 1 do not break a run)
@@ -680,14 +681,14 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
     return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream);
 }
 
-template <typename In, typename Acc, typename Map>
+template <typename In, typename Acc, typename Map, typename Out = Acc>
 inline int32_t mapreduce_op(const MapreduceArgs& a) {
     const MapXform<In, Acc, Map> xf;
     switch (a.op) {
-        case RK_OP_ADD: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpAdd>(a, xf);
-        case RK_OP_MUL: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMul>(a, xf);
-        case RK_OP_MAX: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMax>(a, xf);
-        case RK_OP_MIN: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMin>(a, xf);
+        case RK_OP_ADD: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpAdd, Out>(a, xf);
+        case RK_OP_MUL: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMul, Out>(a, xf);
+        case RK_OP_MAX: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMax, Out>(a, xf);
+        case RK_OP_MIN: return mapreduce_one<In, Acc, MapXform<In, Acc, Map>, OpMin, Out>(a, xf);
         default: return RK_ERR_INVALID_ARGUMENT;
     }
 }
@@ -720,12 +721,12 @@ inline int32_t mapreduce_prog(const MapreduceArgs& a) {
     }
 }
 
-template <typename In, typename Acc>
+template <typename In, typename Acc, typename Out = Acc>
 inline int32_t mapreduce_typed(const MapreduceArgs& a) {
     switch (a.f) {
-        case RK_MAP_IDENTITY: return mapreduce_op<In, Acc, MapIdentity>(a);
-        case RK_MAP_ABS2:     return mapreduce_op<In, Acc, MapAbs2>(a);
-        case RK_MAP_ABS:      return mapreduce_op<In, Acc, MapAbs>(a);
+        case RK_MAP_IDENTITY: return mapreduce_op<In, Acc, MapIdentity, Out>(a);
+        case RK_MAP_ABS2:     return mapreduce_op<In, Acc, MapAbs2, Out>(a);
+        case RK_MAP_ABS:      return mapreduce_op<In, Acc, MapAbs, Out>(a);
         default: return RK_ERR_INVALID_ARGUMENT;
     }
 }
@@ -765,6 +766,8 @@ int32_t mapreduce_prog_i64(const MapreduceArgs&);
 int32_t mapreduce_prog_i32_i64(const MapreduceArgs&);
 int32_t mapreduce_prog_u8_i64(const MapreduceArgs&);
 int32_t mapreduce_f32(const MapreduceArgs&);
+int32_t mapreduce_f16(const MapreduceArgs&);
+int32_t findminmax_f16(const FindArgs&);
 int32_t mapreduce_f64(const MapreduceArgs&);
 int32_t mapreduce_i32(const MapreduceArgs&);
 int32_t mapreduce_i64(const MapreduceArgs&);

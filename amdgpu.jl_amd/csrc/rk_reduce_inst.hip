@@ -37,7 +37,11 @@ int32_t findminmax_u32(const FindArgs& a) { return findminmax_typed<uint32_t>(a)
 #elif RK_INST == 8
 int32_t mapreduce_u64(const MapreduceArgs& a) { return mapreduce_typed<uint64_t, uint64_t>(a); }
 int32_t findminmax_u64(const FindArgs& a) { return findminmax_typed<uint64_t>(a); }
+#elif RK_INST == 9
+// Float16 arrays: f in Float16 (abs2 rounds like Julia's), accumulation in Float32, one rounding at the end
+int32_t mapreduce_f16(const MapreduceArgs& a) { return mapreduce_typed<half_t, float, half_t>(a); }
+int32_t findminmax_f16(const FindArgs& a) { return findminmax_typed<half_t>(a); }
 #else
-#error "RK_INST must be 0..8"
+#error "RK_INST must be 0..9"
 #endif
 }  // namespace rk

@@ -108,8 +108,10 @@ RK_API int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream);
  * size 1 (mapreduce.jl:95-107) and element type `out`.  R is OVERWRITTEN with
  * op(init, reduction); `init` = host pointer to one `out` element, or NULL for op's
  * neutral element (0, 1, typemin, typemax).  One launch, no recursion, no allocation.
- * Supported (in -> out): same type; I32/U8 -> I64 and U32 -> U64 (add_sum widening);
- * F32 -> F64.  MAX/MIN on floats follow Base.max/min (NaN propagates, -0.0 < 0.0). */
+ * Supported (in -> out): same type for F32, F64, F16, I32, I64, U8, U32, U64 (Float16:
+ * f in Float16, accumulation in Float32, one rounding at the end); I32/U8 -> I64 and
+ * U32 -> U64 (add_sum widening).  MAX/MIN on floats follow Base.max/min (NaN propagates,
+ * -0.0 < 0.0). */
 RK_API int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
                      const void* A, int ndim, const int64_t* shape, uint32_t reduce_mask,
                      void* R, const void* init,

@@ -250,6 +250,8 @@ def _order_score(A: np.ndarray, want_max: bool) -> np.ndarray:
     """
     A = np.asarray(A)
     if A.dtype.kind == "f":
+        if A.dtype == np.float16:
+            A = A.astype(np.float32)                    # exact, and order-preserving
         if A.dtype == np.float32:
             bits = A.view(np.int32).astype(np.int64)
             mag = bits & np.int64(0x7FFFFFFF)

@@ -70,7 +70,7 @@ def test_mapreduce_argument_validation(L):
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 9, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # ndim > 8
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, L.shape_array((-1,)), 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(0, 0, L.RK_F32, L.RK_I32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Float32 -> Int32
-    assert f(0, 0, L.RK_F16, L.RK_F16, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert f(0, 0, L.RK_I16, L.RK_I16, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Int16 reductions
     # zero-length input: success without launching (src/kernels/mapreduce.jl:91), even with null pointers
     assert f(0, 0, L.RK_F32, L.RK_F32, None, 1, L.shape_array((0,)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     # a reduction that needs partials but has no workspace

@@ -292,3 +292,37 @@ def test_argmax_argmin_extrema(rk, orc):
     assert rk.extrema(dA) == (A.min(), A.max())
     lo, hi = rk.extrema(lambda v: v * v, dA)
     assert (lo, hi) == ((A * A).min(), (A * A).max())
+
+
+@pytest.mark.parametrize("shape,dims", [((1000,), None), ((257, 129), 1), ((257, 129), 2), ((33, 65, 17), (1, 3)), ((1 << 20,), None), ((8, 100_000), 2)])
+def test_float16_reductions(rk, orc, shape, dims):
+    """Float16 arrays: f applied in Float16, accumulated in Float32, rounded once to Float16.  Sums within one Float16
+    rounding (2^-11 relative) plus the Float32 accumulation error of the Float64 result; max / min / findmax exact."""
+    rng = _rng(61)
+    x = rng.standard_normal(shape).astype(np.float16)
+    dx = rk.ROCArray(x)
+    x64 = x.astype(np.float64)
+    ax = None if dims is None else tuple(d - 1 for d in ((dims,) if isinstance(dims, int) else dims))
+    for f, mapped in (("identity", x64), ("abs2", (x * x).astype(np.float64)), ("abs", np.abs(x64))):
+        got = rk.mapreduce(f, "add_sum", dx, dims=dims)
+        want = mapped.sum(axis=ax, keepdims=dims is not None)
+        mag = np.abs(mapped).sum(axis=ax, keepdims=dims is not None)
+        got = np.asarray(got if dims is None else rk.Array(got))
+        assert got.dtype == np.float16
+        got = got.astype(np.float64).reshape(want.shape)
+        with np.errstate(over="ignore"):
+            over = np.isinf(want.astype(np.float16))              # beyond 65504: Inf, as in Julia
+        assert np.array_equal(np.isinf(got), over)
+        assert np.all(over | (np.abs(got - want) <= 2.0**-10 * np.abs(want) + 1e-6 * mag + 1e-7))
+        for op, ref in (("max", np.max), ("min", np.min)):
+            got = rk.mapreduce(f, op, dx, dims=dims)
+            got = np.asarray(got if dims is None else rk.Array(got))
+            want = ref(mapped, axis=ax, keepdims=dims is not None).astype(np.float16)
+            assert got.dtype == np.float16 and np.array_equal(got.reshape(want.shape), want)
+    if dims is None or isinstance(dims, int):
+        _check_findminmax(rk, orc, rng.integers(-4, 5, shape).astype(np.float16), dims)
+        _check_findminmax(rk, orc, x, dims)
+    init = rk.mapreduce("identity", "add", dx, dims=dims, init=np.float16(2.5))
+    init = np.asarray(init if dims is None else rk.Array(init)).astype(np.float64)
+    want = x64.sum(axis=ax, keepdims=dims is not None) + 2.5
+    assert np.all(np.abs(init.reshape(want.shape) - want) <= 2.0**-10 * np.abs(want) + 1e-6 * np.abs(x64).sum(axis=ax, keepdims=dims is not None) + 1e-7)
