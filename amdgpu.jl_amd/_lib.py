@@ -46,7 +46,7 @@ RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE, RK_KIND_FINDALL = ran
  RK_BC_INV, RK_BC_IDENTITY) = range(64, 75)
 (RK_BC_LT, RK_BC_LE, RK_BC_GT, RK_BC_GE, RK_BC_EQ, RK_BC_NE, RK_BC_AND, RK_BC_OR) = range(96, 104)
 RK_BC_IFELSE = 112
-(RK_BC_NOT, RK_BC_ISODD, RK_BC_ISEVEN, RK_BC_ISNAN, RK_BC_WRAP_I32, RK_BC_WRAP_U32) = range(128, 134)
+(RK_BC_NOT, RK_BC_ISODD, RK_BC_ISEVEN, RK_BC_ISNAN, RK_BC_WRAP_I32, RK_BC_WRAP_U32, RK_BC_ROUND_F16) = range(128, 135)
 
 
 class RkOperand(C.Structure):

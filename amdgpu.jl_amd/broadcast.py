@@ -227,6 +227,9 @@ def _emit(bc: Broadcasted, operands: list, tokens: list, types: dict, int_progra
             if bc.f in table:
                 tokens.append(table[bc.f])
                 break
+    # Julia computes Float16 arithmetic in Float32 and rounds every result: so does the program
+    if types[id(bc)] == np.float16 and (bc.f in ("+", "-", "*", "/", "^", "muladd", "abs2") or bc.f in _MATH):
+        tokens.append(L.RK_BC_ROUND_F16)
 
 
 def _wrap(t: np.dtype, tokens: list):
@@ -248,7 +251,7 @@ def _compile_tree(tree: Broadcasted, operands: list):
     if floats:
         compute = max(floats, key=lambda d: d.itemsize)
         if compute == np.float16:
-            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "Float16 broadcast")
+            compute = np.dtype(np.float32)             # with RK_BC_ROUND_F16 after every Float16-typed operation
     else:
         compute = np.dtype(np.int64)
     tokens: list = []

@@ -102,6 +102,7 @@ __device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool
         case RK_I64: load_as<CT, int64_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         case RK_U32: load_as<CT, uint32_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         case RK_U64: load_as<CT, uint64_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_F16: load_as<CT, half_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         default:     load_as<CT, uint8_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
     }
 }
@@ -111,7 +112,7 @@ __device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool
 template <typename CT, int VEC, bool MAY_REUSE, bool HOMOG>
 __device__ __forceinline__ void load_operand(const BcOperand& o, int64_t off, bool wave_rows, CT (&v)[VEC]) {
     if (o.ptr == nullptr) {
-        const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64) ? (CT)o.sf : (CT)o.si;
+        const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64 || o.dtype == RK_F16) ? (CT)o.sf : (CT)o.si;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = x;
         return;
@@ -144,6 +145,7 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
         case RK_I64: store_as<CT, int64_t, VEC>(p, off, v); break;
         case RK_U32: store_as<CT, uint32_t, VEC>(p, off, v); break;
         case RK_U64: store_as<CT, uint64_t, VEC>(p, off, v); break;
+        case RK_F16: store_as<CT, half_t, VEC>(p, off, v); break;
         default:     store_as<CT, uint8_t, VEC>(p, off, v); break;
     }
 }
@@ -367,7 +369,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
         const bool wave_rows = a.tx_log2 >= 6;     // 64 or more lanes along dim 0: the lanes of a wave share their rows
-        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? (HOMOG ? BC_RPT : 2) : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
+        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? 2 : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
             int64_t doff[NB];
@@ -510,9 +512,11 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
                               const int64_t* dest_strides, void* stream) {
     if (prog == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
-    if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_I16) return RK_ERR_INVALID_ARGUMENT;
+    if (dest_dtype == RK_I16) return RK_ERR_UNSUPPORTED;
     if (prog->compute != RK_F32 && prog->compute != RK_F64 && prog->compute != RK_I64) return RK_ERR_UNSUPPORTED;
     const bool int_compute = prog->compute == RK_I64;
+    if (dest_dtype == RK_F16 && int_compute) return RK_ERR_UNSUPPORTED;
     if (prog->n_operands < 0 || prog->n_operands > RK_MAX_OPERANDS) return RK_ERR_INVALID_ARGUMENT;
     if (prog->n_tokens < 1 || prog->n_tokens > RK_MAX_PROGRAM) return RK_ERR_INVALID_ARGUMENT;
 
@@ -540,7 +544,8 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
     }
     for (int k = 0; k < prog->n_operands; ++k) {
         const rk_operand& o = prog->operands[k];
-        if (o.dtype < RK_F32 || o.dtype > RK_U64) return RK_ERR_INVALID_ARGUMENT;
+        if (o.dtype < RK_F32 || o.dtype > RK_I16) return RK_ERR_INVALID_ARGUMENT;
+        if (o.dtype == RK_I16 || (o.dtype == RK_F16 && int_compute)) return RK_ERR_UNSUPPORTED;
         if (o.ptr == nullptr) {
             if (o.ndim != 0) return RK_ERR_INVALID_ARGUMENT;
             for (int d = 0; d < ndim; ++d) stride[k][d] = 0;

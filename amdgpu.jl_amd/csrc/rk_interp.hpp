@@ -15,7 +15,7 @@ __host__ __device__ constexpr int token_arity(int tok) {
            : (tok >= RK_BC_NEG && tok <= RK_BC_IDENTITY) ? 1
            : (tok >= RK_BC_LT && tok <= RK_BC_OR)      ? 2
            : (tok == RK_BC_IFELSE)                     ? 3
-           : (tok >= RK_BC_NOT && tok <= RK_BC_WRAP_U32) ? 1
+           : (tok >= RK_BC_NOT && tok <= RK_BC_ROUND_F16) ? 1
                                                        : -1;
 }
 
@@ -153,6 +153,7 @@ __device__ __forceinline__ void interp_run(const Tokens& tokens, int n_tokens, c
                         case RK_BC_LOG: RK_BC_UN(log(x));
                         case RK_BC_INV: RK_BC_UN(CT(1) / x);
                         case RK_BC_ISNAN: RK_BC_UN(x != x ? CT(1) : CT(0));
+                        case RK_BC_ROUND_F16: RK_BC_UN((CT)(half_t)x);
                         default:
                             if constexpr (FULL) {
                                 switch (tok) {

@@ -283,7 +283,18 @@ const UNARY = IdDict{Any,Int32}(abs => 65, abs2 => 66, sqrt => 67, exp => 68, lo
                                 tanh => 72, inv => 73, identity => 74, ! => 128, isodd => 129, iseven => 130, isnan => 131)
 struct Unsupported <: Exception end
 
+# Julia computes Float16 arithmetic in Float32 and rounds every result; a Float16 tree runs as a Float32 program with
+# RK_BC_ROUND_F16 (134) after every operation whose eltype is Float16
+rounds_f16(f) = f in (+, -, *, /, ^, muladd, abs2, sqrt, exp, log, sin, cos, tanh, inv)
 function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
+    if x isa Broadcasted
+        flatten_node!(ops, toks, x)
+        Broadcast.combine_eltypes(x.f, x.args) === Float16 && rounds_f16(x.f) && push!(toks, Int32(134))
+    else
+        flatten_node!(ops, toks, x)
+    end
+end
+function flatten_node!(ops::Vector{Any}, toks::Vector{Int32}, x)
     if x isa Broadcasted
         f, args = x.f, x.args
         if length(args) == 1 && f === (-)
@@ -301,7 +312,7 @@ function flatten!(ops::Vector{Any}, toks::Vector{Int32}, x)
         else
             throw(Unsupported())
         end
-    elseif x isa ROCArray || is_strided_wrapper(x) || x isa Union{Float32,Float64,Int32,Int64,Bool}
+    elseif x isa ROCArray || is_strided_wrapper(x) || x isa Union{Float16,Float32,Float64,Int32,Int64,Bool}
         k = findfirst(o -> o === x, ops)
         k === nothing && (push!(ops, x); k = length(ops))
         k > RK_MAX_OPERANDS && throw(Unsupported())
@@ -318,6 +329,7 @@ function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadc
     flatten!(ops, toks, bc)
     length(toks) <= RK_MAX_PROGRAM || throw(Unsupported())
     CT = promote_type(map(o -> o isa AbstractArray ? eltype(o) : typeof(o), ops)...)
+    CT === Float16 && (CT = Float32)
     if !(CT <: Union{Float32,Float64})
         # integer programs of + - * max min muladd - abs abs2 compute in Int64 (the store keeps the low bits);
         # with `/` or a math function Julia's result is a Float64 and so is the compute type

@@ -200,7 +200,10 @@ typedef enum {
     RK_BC_ISNAN,
     RK_BC_WRAP_I32,            /* integer programs: sign-extend the low 32 bits, i.e. the Int32 value Julia
                                 * holds at this point (needed before order-sensitive tokens only)      */
-    RK_BC_WRAP_U32             /* the same, zero-extending (UInt32)                                    */
+    RK_BC_WRAP_U32,            /* the same, zero-extending (UInt32)                                    */
+    RK_BC_ROUND_F16            /* Float32 programs over Float16 arrays: round to Float16 and back, after every
+                                * operation whose Julia result is a Float16 (Julia computes Float16 arithmetic in
+                                * Float32 and rounds each result)                                       */
 } rk_bc_token;
 
 typedef struct {

@@ -241,3 +241,42 @@ def test_left_deep_chains(rk):
     with np.errstate(over="ignore"):
         got = rk.materialize(((lz(K) * lz(K) - lz(K)) * np.int32(3) + lz(K)) * lz(K))
         assert got.dtype == np.int32 and np.array_equal(rk.Array(got), ((k * k - k) * np.int32(3) + k) * k)
+
+
+def test_float16_arrays(rk):
+    """Float16 operands and destinations: Float32 arithmetic with a rounding to Float16 after every operation whose Julia
+    type is Float16 -- what Julia (and NumPy) do -- so results are bit-identical to NumPy's Float16 arithmetic."""
+    rng = _rng(23)
+    shape = (130, 67)
+    x = rng.standard_normal(shape).astype(np.float16)
+    y = (rng.random(shape) + 0.5).astype(np.float16)
+    col = rng.standard_normal((130, 1)).astype(np.float16)
+    f = rng.standard_normal(shape).astype(np.float32)
+    X, Y, Cc, F = (rk.ROCArray(a) for a in (x, y, col, f))
+    lz = rk.lazy
+    h = np.float16
+    cases = [
+        (lz(X) + lz(Y), x + y), (lz(X) * lz(Y) - lz(Cc), x * y - col), (lz(X) / lz(Y), x / y),
+        ((lz(X) + lz(Y)) * (lz(X) - lz(Y)) / lz(Y), (x + y) * (x - y) / y),
+        (h(1.5) * lz(X) + lz(Cc), h(1.5) * x + col), (rk.broadcast.abs2(lz(X)) + lz(Y), x * x + y),
+        (rk.broadcast.max_(lz(X), lz(Cc)) - rk.broadcast.min_(lz(X), lz(Y)), np.maximum(x, col) - np.minimum(x, y)),
+        (lz(X) + 2, x + h(2)),                                   # an Int literal keeps Float16
+    ]
+    for bc, want in cases:
+        got = rk.materialize(bc)
+        assert got.dtype == np.float16
+        np.testing.assert_array_equal(rk.Array(got), want.astype(np.float16))
+    got = rk.materialize(lz(X) * lz(F) + lz(Y))                  # Float16 with Float32: a Float32 program, nothing rounded
+    assert got.dtype == np.float32
+    np.testing.assert_array_equal(rk.Array(got), x.astype(np.float32) * f + y.astype(np.float32))
+    got = rk.materialize((lz(X) + lz(Y)) * lz(F))                # the Float16 sum is rounded before it meets the Float32
+    np.testing.assert_array_equal(rk.Array(got), (x + y).astype(np.float32) * f)
+    dest = rk.ROCArray(dims=shape, dtype=np.float16)              # Float32 program into a Float16 destination
+    rk.materialize_(dest, lz(F) * np.float32(0.5))
+    np.testing.assert_array_equal(rk.Array(dest), (f * np.float32(0.5)).astype(np.float16))
+    got = rk.materialize(rk.broadcast.exp(lz(X)))
+    assert got.dtype == np.float16
+    np.testing.assert_allclose(rk.Array(got).astype(np.float64), np.exp(x.astype(np.float64)), rtol=2.0**-10)
+    assert np.array_equal(rk.Array(rk.materialize(lz(X) > lz(Y))), x > y)
+    s = rk.sum(lambda v: v * v, X)                               # closures over Float16 arrays: map first, then reduce
+    assert isinstance(s, np.float16) and abs(float(s) - float((x * x).astype(np.float64).sum())) <= 2.0**-9 * float((x * x).astype(np.float64).sum())
