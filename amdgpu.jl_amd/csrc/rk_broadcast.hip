@@ -415,6 +415,8 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         }
         return;
     }
+    // one vector per thread: two (loads of both issued first, half the workgroups) measured 4 % slower on
+    // z .= a.*x .+ y.*exp.(w) and on the plain copy
     CT in[RK_MAX_OPERANDS][VEC];
 #pragma unroll
     for (int k = 0; k < Eval::NOPS; ++k)
