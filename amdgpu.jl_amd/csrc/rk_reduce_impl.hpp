@@ -13,6 +13,7 @@
 //                          fixed order (deterministic, single launch)
 //   reduce_wave_kernel     many medium lines: one wave per line, no LDS, no barrier
 //   reduce_thread_kernel   very many tiny lines: one lane per line
+//   reduce_narrow_kernel   1 < inner < 64 with long lines: contiguous runs of whole rows
 //   reduce_strided_kernel  inner >= 64: lanes run along the contiguous `inner` axis (128-bit
 //                          loads), waves and workgroups split `mid`
 // plus reduce_generic_kernel for masks that are not one run (e.g. dims=(1,3)).
@@ -311,6 +312,87 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
     sink(line, a);
 }
 
+// ---- 1 < inner < 64 with long lines: contiguous runs of whole rows ---------------------------------------
+// (sum(A; dims=2) of a 3 x 1_000_000 array, perf/array.jl:91,96; the fold over the long dim of a 2 x 3 x N array.)
+// A wave per line reads one element in `inner`, a quarter or less of every cache line at a time.  Here thread t of
+// the inner * R threads (R = 256 / inner whole rows) reads element t of the workgroup's current run of R rows:
+// consecutive lanes, consecutive addresses, and because a pass advances by whole rows the thread's column t % inner
+// never changes.  The R threads of a column meet in LDS.  grid (msplits, outer): a workgroup takes rows_per_split
+// rows of one slab; partials[(o * msplits + ms) * inner + column], one ticket per slab, the last arrival folds.
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink>
+__global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
+                                                            Acc* partials, uint32_t* tickets, int64_t rows_per_split) {
+    typedef typename Xf::Pos Pos;
+    __shared__ Acc lds[256];
+    __shared__ int is_last;
+    const int t = threadIdx.x;
+    const int inner = (int)g.inner;
+    const int R = 256 / inner, T = R * inner;
+    const int ms = blockIdx.x, msplits = gridDim.x;
+    const int64_t o = blockIdx.y;
+    const int64_t r0 = (int64_t)ms * rows_per_split;
+    int64_t r1 = r0 + rows_per_split;
+    if (r1 > g.mid) r1 = g.mid;
+    const In* slab = A + o * g.inner * g.mid;
+    constexpr int NU = 8;                  // loads in flight per thread
+    Acc acc[NU];
+#pragma unroll
+    for (int u = 0; u < NU; ++u) acc[u] = Op::template identity<Acc>();
+    if (t < T) {
+        const int rt = t / inner;
+        int64_t row = r0 + rt;
+        const In* p = slab + r0 * inner + t;       // = slab + row * inner + column; a pass advances by T elements
+        for (; row + (NU - 1) * R < r1; row += NU * R, p += NU * T) {
+            In v[NU];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) v[u] = p[u * T];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) acc[u] = acc_step(op, acc[u], xf(v[u], (Pos)(row + u * R)));
+        }
+        for (; row < r1; row += R, p += T) acc[0] = acc_step(op, acc[0], xf(p[0], (Pos)row));
+    }
+    Acc all = acc[0];
+#pragma unroll
+    for (int u = 1; u < NU; ++u) all = op(all, acc[u]);
+    lds[t] = all;
+    __syncthreads();
+    Acc r = Op::template identity<Acc>();
+    if (t < inner)
+        for (int k = 0; k < R; ++k) r = op(r, lds[t + k * inner]);
+    if (msplits == 1) {
+        if (t < inner) sink(t + o * g.inner, r);
+        return;
+    }
+    if (t < inner) {
+        store_agent(&partials[(o * msplits + ms) * inner + t], r);
+        publish_barrier();
+    }
+    __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
+    if (t == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[o * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = (old == (uint32_t)msplits - 1u);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    // the last arrival folds the msplits rows of partials the way it folded its own rows: thread t takes column
+    // t % inner of rows t / inner, t / inner + R, ...; the R threads of a column meet in LDS
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    Acc f = Op::template identity<Acc>();
+    if (t < T) {
+        const int rt = t / inner, c = t - rt * inner;
+        for (int i = rt; i < msplits; i += R) f = op(f, partials[(o * msplits + i) * inner + c]);
+    }
+    __syncthreads();     // lds is free again
+    lds[t] = f;
+    __syncthreads();
+    if (t < inner) {
+        Acc r2 = Op::template identity<Acc>();
+        for (int k = 0; k < R; ++k) r2 = op(r2, lds[t + k * inner]);
+        sink(t + o * g.inner, r2);
+    }
+    if (t == 0) tickets[o * TICKET_STRIDE] = 0;
+}
+
 // ---- inner >= 64: lanes along `inner` -------------------------------------------------------------
 // grid (strips, msplits, outer); workgroup = 4 waves; a wave owns 64 * VEC adjacent columns of a
 // strip and every 4th row of the row batches dealt to its workgroup.
@@ -485,9 +567,10 @@ __global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restr
 
 // ---- host side: pick a kernel and launch -------------------------------------------------------------
 struct ReducePlan {
-    enum Kind { SPLIT, WAVE_LINES, THREAD_LINES, STRIDED, GENERIC } kind;
+    enum Kind { SPLIT, WAVE_LINES, THREAD_LINES, STRIDED, NARROW, GENERIC } kind;
     bool    vector;
-    int     splits;      // SPLIT: workgroups per line; STRIDED: slices of mid
+    int     splits;      // SPLIT: workgroups per line; STRIDED, NARROW: slices of mid
+    int64_t rows_per_split;   // NARROW
     int     strips;      // STRIDED
     size_t  payload;     // bytes of partials
 };
@@ -530,6 +613,23 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
         return p;
     }
     if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
+    if (s.inner > 1 && s.mid >= 1024 && s.outer <= 65535 && s.outer <= (int64_t)WS_TICKET_COUNT) {
+        p.kind = ReducePlan::NARROW;
+        const int64_t rows_per_pass = 256 / s.inner;
+        // every extra workgroup costs a row of partials and a longer fold: two per compute unit measured best
+        // (63 x 1048576 Float32: 1024 workgroups 107 us, 512 73 us), each with at least 16 passes of its own
+        int64_t want = (target_blocks + s.outer - 1) / s.outer;
+        const int64_t max_splits = (s.mid + 16 * rows_per_pass - 1) / (16 * rows_per_pass);
+        if (want > max_splits) want = max_splits;
+        if (want > 4096) want = 4096;
+        const int64_t fit = (int64_t)(cap / sizeof(Acc)) / (s.outer * s.inner);
+        if (want > fit) want = fit;
+        if (want < 1) want = 1;
+        p.splits = (int)want;
+        p.rows_per_split = (s.mid + want - 1) / want;
+        p.payload = want > 1 ? (size_t)(s.outer * want * s.inner) * sizeof(Acc) : 0;
+        return p;
+    }
     const bool contiguous = (s.inner == 1);
     // Plenty of lines: a wave per line fills every compute unit -- but only for short lines.  With a wave per
     // 32 KiB line all 8192 resident waves stream different DRAM pages at once; a workgroup per line keeps the
@@ -605,6 +705,11 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
                 reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
             break;
         }
+        case ReducePlan::NARROW: {
+            dim3 grid(p.splits, (unsigned)s.outer);
+            reduce_narrow_kernel<In, Acc, Xf, Op, Sink><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.rows_per_split);
+            break;
+        }
         case ReducePlan::GENERIC: {
             GenericGeom gg{};
             int64_t stride = 1;
@@ -652,30 +757,44 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
     ReduceSink<Acc, Op, Out> sink{(Out*)a.R, a.init ? (Acc)*(const Out*)a.init : Op::template identity<Acc>(), a.init ? 1 : 0};
     const Shape3 s = collapse3(a.ndim, a.shape, a.mask);
     if (!s.single_run && s.total > 0) {
-        uint32_t mask1 = 0;                       // the lowest run of reduced dims (extents of 1 do not break a run)
-        int64_t shape1[RK_MAX_DIMS], rest = 1;
-        bool in_run = false, closed = false;
+        // the runs of reduced dims (extents of 1 do not break a run), lowest first
+        uint32_t run_mask[RK_MAX_DIMS];
+        int64_t run_ext[RK_MAX_DIMS];
+        int nruns = 0;
+        bool in_run = false;
         for (int d = 0; d < a.ndim; ++d) {
-            shape1[d] = a.shape[d];
-            const bool red = (a.mask >> d) & 1u;
             if (a.shape[d] == 1) continue;
-            if (red && !closed) { mask1 |= 1u << d; shape1[d] = 1; in_run = true; }
-            else {
-                if (in_run) closed = true;
-                rest *= a.shape[d];
-            }
+            if ((a.mask >> d) & 1u) {
+                if (!in_run) { run_mask[nruns] = 0; run_ext[nruns] = 1; ++nruns; in_run = true; }
+                run_mask[nruns - 1] |= 1u << d;
+                run_ext[nruns - 1] *= a.shape[d];
+            } else in_run = false;
         }
-        const size_t temp_bytes = ((size_t)rest * sizeof(Acc) + 255) & ~(size_t)255;
+        // Fold one run first into a temporary of total / extent elements: the lowest run if that fits (the
+        // rest is then reduced from a compact array), else the longest one (sum of 2 x 3 x 2097152 over dims (1, 3):
+        // folding dim 1 leaves 25 MB, folding dim 3 leaves six numbers -- the generic kernel, one thread per output,
+        // took 41 ms there).
+        int longest = 0;
+        for (int r = 1; r < nruns; ++r)
+            if (run_ext[r] > run_ext[longest]) longest = r;
+        const int candidates[2] = {0, longest};
         Workspace w{};
-        if (mask1 != 0 && temp_bytes <= REDUCE_TEMP_MAX && carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
-            Acc* temp = (Acc*)((char*)w.partials + WS_PARTIALS_BYTES - temp_bytes);
-            const size_t cap = WS_PARTIALS_BYTES - temp_bytes;
-            ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
-            const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, mask1, xf, Op(), to_temp,
-                                                      a.ws, a.ws_bytes, a.stream, cap);
-            if (st != RK_SUCCESS) return st;
-            return launch_reduce<Acc, Acc>((const Acc*)temp, a.ndim, shape1, a.mask & ~mask1, MapXform<Acc, Acc, MapIdentity>(), Op(), sink,
-                                           a.ws, a.ws_bytes, a.stream, cap);
+        if (nruns > 0 && carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
+            for (int c = 0; c < 2; ++c) {
+                const int r = candidates[c];
+                const size_t temp_bytes = ((size_t)(s.total / run_ext[r]) * sizeof(Acc) + 255) & ~(size_t)255;
+                if (temp_bytes > REDUCE_TEMP_MAX) continue;
+                int64_t shape1[RK_MAX_DIMS];
+                for (int d = 0; d < a.ndim; ++d) shape1[d] = ((run_mask[r] >> d) & 1u) ? 1 : a.shape[d];
+                Acc* temp = (Acc*)((char*)w.partials + WS_PARTIALS_BYTES - temp_bytes);
+                const size_t cap = WS_PARTIALS_BYTES - temp_bytes;
+                ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
+                const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, run_mask[r], xf, Op(), to_temp,
+                                                          a.ws, a.ws_bytes, a.stream, cap);
+                if (st != RK_SUCCESS) return st;
+                return launch_reduce<Acc, Acc>((const Acc*)temp, a.ndim, shape1, a.mask & ~run_mask[r], MapXform<Acc, Acc, MapIdentity>(),
+                                               Op(), sink, a.ws, a.ws_bytes, a.stream, cap);
+            }
         }
     }
     return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream);

@@ -326,3 +326,27 @@ def test_float16_reductions(rk, orc, shape, dims):
     init = np.asarray(init if dims is None else rk.Array(init)).astype(np.float64)
     want = x64.sum(axis=ax, keepdims=dims is not None) + 2.5
     assert np.all(np.abs(init.reshape(want.shape) - want) <= 2.0**-10 * np.abs(want) + 1e-6 * np.abs(x64).sum(axis=ax, keepdims=dims is not None) + 1e-7)
+
+
+@pytest.mark.parametrize("shape,dims", [((3, 100_000), 2), ((7, 52_429, 5), 2), ((2, 3, 200_001), 3), ((63, 4099), 2), ((5, 5, 5, 5, 2000), 5),
+                                        ((2, 3, 200_001), (1, 3)), ((5, 5, 5, 5, 2000), (1, 5)), ((33, 1025, 2), 2), ((16, 1024), 2), ((2, 1_000_003), 2)])
+def test_long_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
+    """1 < inner < 64 along a long reduced dim (sum(A; dims=2) of a 3 x N array), alone and as the first fold of a
+    reduction over non-adjacent dims."""
+    rng = _rng(71)
+    for dtype in (np.float32, np.int32, np.int64, np.float64):
+        x = rng.integers(-1000, 1001, shape).astype(dtype)
+        dx = rk.ROCArray(x)
+        for f, op in (("identity", "add_sum"), ("abs2", "max"), ("identity", "min")):
+            got = rk.Array(rk.mapreduce(f, op, dx, dims=dims))
+            want = orc.mapreduce(f, op, x, dims=dims)
+            if np.dtype(dtype).kind == "f" and op == "add_sum":
+                np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-2)
+            else:
+                assert np.array_equal(got, want.astype(got.dtype))
+    if isinstance(dims, int):
+        _check_findminmax(rk, orc, rng.integers(-4, 5, shape).astype(np.float32), dims)
+        _check_findminmax(rk, orc, rng.standard_normal(shape).astype(np.float64), dims)
+    c = rk.count(lambda v: v > 0, rk.ROCArray(x), dims=dims)
+    ax = tuple(d - 1 for d in ((dims,) if isinstance(dims, int) else dims))
+    assert np.array_equal(rk.Array(c), (x > 0).sum(axis=ax, keepdims=True))
