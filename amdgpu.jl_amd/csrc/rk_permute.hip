@@ -3,8 +3,9 @@
 // perf/array.jl:151-155); here:
 //   * dims that stay neighbours in the same order are merged, extents of 1 dropped;
 //   * if the first dim stays first, rows move whole: 16-byte units (or elements), coalesced on both sides;
-//   * if the source's or the destination's contiguous dim is short (<= 8 elements: (N, 3) <-> (3, N), batches of tiny
-//     matrices), a lane moves one run of that dim (rk_permute_small.hpp);
+//   * if the leading dims of the source (up to the one that becomes the destination's first) or of the destination
+//     (up to the source's first) hold at most 8 elements -- (N, 3) <-> (3, N), (2, 3, N) <-> (N, 3, 2), batches of
+//     tiny matrices -- a lane moves one such run (rk_permute_small.hpp);
 //   * otherwise 64 x 64 tiles over (src dim 1, the src dim that becomes dst dim 1) go through LDS, so that loads
 //     run along the source's contiguous axis and stores along the destination's.
 // 2 x elsize bytes per element, no workspace.
@@ -154,10 +155,10 @@ __global__ __launch_bounds__(256) void permute_small_kernel(const T* __restrict_
     T v[PERM_SMALL_MAX];
 #pragma unroll
     for (int j = 0; j < PERM_SMALL_MAX; ++j)
-        if (j < g.small) v[j] = src[so + j * g.small_sstride];
+        if (j < g.small) v[j] = src[so + g.run_soff[j]];
 #pragma unroll
     for (int j = 0; j < PERM_SMALL_MAX; ++j)
-        if (j < g.small) dst[dofs + j * g.small_dstride] = v[j];
+        if (j < g.small) dst[dofs + g.run_doff[j]] = v[j];
 }
 
 template <int E>
@@ -190,7 +191,7 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
         // a short contiguous dim on either side: tiles would be mostly empty
         // ((4194304, 3) -> (3, 4194304) Float32: 0.68 TB/s with tiles)
         PermSmallGeom sg;
-        if (perm_small_geometry(g.ext, g.dstride, g.nd, g.p, g.total, &sg) && sg.small <= 8) {
+        if (perm_small_geometry(g.ext, g.dstride, g.nd, g.p, g.total, 8, &sg)) {
             const int64_t blocks = (sg.n_threads + 255) / 256;
             if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
             permute_small_kernel<T><<<(unsigned)blocks, 256, 0, stream>>>((const T*)src, (T*)dst, sg);

@@ -1,10 +1,10 @@
-// permutedims when the source's or the destination's contiguous dim is short (at most PERM_SMALL_MAX elements): the
-// (N, 3) <-> (3, N) and (N, 4) <-> (4, N) conversions between arrays of structures and structures of arrays, batches of
-// tiny matrices.  64 x 64 tiles through LDS leave most of every tile empty there.  Here a lane owns one run of the short
-// dim: it reads the run's elements (stride 1 when the short dim is the source's first, else the source stride of that
-// dim) and writes them (the destination stride of that dim, 1 when it is the destination's first).  Lanes advance along
-// the long dim that is contiguous on the other side, so every load (or store) instruction of a wave covers consecutive
-// addresses, and the runs of neighbouring lanes are neighbours in memory on the short side.
+// permutedims when a short block of dims leads the source or the destination (at most PERM_SMALL_MAX elements): the
+// (N, 3) <-> (3, N) and (N, 4) <-> (4, N) conversions between arrays of structures and structures of arrays,
+// (2, 3, N) <-> (N, 3, 2), batches of tiny matrices.  64 x 64 tiles through LDS leave most of every tile empty there.
+// Here a lane owns one run = one instance of the short block: contiguous on the side the block leads, scattered by the
+// other side's strides.  Lanes advance along the long dim that is contiguous on the other side, so every load (or
+// store) instruction of a wave covers consecutive addresses, and the runs of neighbouring lanes are neighbours in
+// memory on the run's contiguous side.
 //
 // The index mapping is host-callable: a brute-force check over every thread of many shapes runs on the CPU.
 #pragma once
@@ -25,12 +25,13 @@ constexpr int PERM_MAX_DIMS = 8;
 
 struct PermSmallGeom {
     int64_t n_threads;                 // runs = elements / small
-    int nd;                            // looped dims: every merged dim except the short one, the lane dim first
+    int nd;                            // looped dims: every merged dim outside the short block, the lane dim first
     int64_t ext[PERM_MAX_DIMS];
     int64_t sstride[PERM_MAX_DIMS];    // source / destination strides (elements) of the looped dims
     int64_t dstride[PERM_MAX_DIMS];
-    int32_t small;                     // extent of the short dim
-    int64_t small_sstride, small_dstride;
+    int32_t small;                     // elements of a run (the product of the short block's extents)
+    int64_t run_soff[PERM_SMALL_MAX];  // source / destination offset of element j of a run; one of the two is j
+    int64_t run_doff[PERM_SMALL_MAX];
 };
 
 // Source and destination offsets (elements) of the first element of run `idx`.
@@ -48,29 +49,67 @@ RK_HD void perm_small_offsets(const PermSmallGeom& g, int64_t idx, int64_t* soff
 }
 
 // Geometry from merged source extents `ext[0..nd)`, the destination stride of every merged source dim, and p = the
-// merged source dim that is contiguous in the destination (p != 0).  Returns false when neither side is short.
-inline bool perm_small_geometry(const int64_t* ext, const int64_t* dstride, int nd, int p, int64_t total, PermSmallGeom* out) {
-    if (nd < 2 || nd > PERM_MAX_DIMS || p <= 0 || p >= nd) return false;
+// merged source dim that is contiguous in the destination (p != 0).  Two shapes qualify:
+//   * the source's leading dims 0 .. p-1 hold at most max_run elements together (2 x 3 x N -> N x 3 x 2, 3 x N -> N x 3):
+//     a run is that block, contiguous in the source, its elements scattered by the destination strides; lanes along p;
+//   * the destination's leading dims, up to the one that is the source's dim 0, hold at most max_run elements
+//     (N x 3 x 2 -> 2 x 3 x N, N x 4 -> 4 x N): a run is contiguous in the destination, gathered by source strides;
+//     lanes along dim 0.
+// In both the runs of neighbouring lanes are neighbours in memory on the run's contiguous side.  Returns false otherwise.
+inline bool perm_small_geometry(const int64_t* ext, const int64_t* dstride, int nd, int p, int64_t total, int max_run, PermSmallGeom* out) {
+    if (nd < 2 || nd > PERM_MAX_DIMS || p <= 0 || p >= nd || max_run > PERM_SMALL_MAX) return false;
     int64_t sstr[PERM_MAX_DIMS];
     int64_t s = 1;
     for (int d = 0; d < nd; ++d) { sstr[d] = s; s *= ext[d]; }
-    int small_dim, lane_dim;
-    // prefer the short destination run (its stores become one contiguous piece per lane); else the short source run
-    // and only when the runs of neighbouring lanes are neighbours in memory on the short side (the lane dim follows the
-    // short dim directly there); otherwise every access of a run is a scattered 4- or 8-byte piece
-    // ((1048576, 2, 8) -> (8, 2, 1048576): 145 us this way, 62 us with tiles)
-    if (ext[p] <= PERM_SMALL_MAX && dstride[0] == ext[p]) { small_dim = p; lane_dim = 0; }
-    else if (ext[0] <= PERM_SMALL_MAX && p == 1) { small_dim = 0; lane_dim = p; }
-    else return false;
+    bool in_block[PERM_MAX_DIMS] = {};
+    int block[PERM_MAX_DIMS], nb = 0;      // dims of the short block, fastest first on the run's contiguous side
+    int lane_dim = -1;
+    bool src_run = false;
+    // destination order of the merged source dims: increasing dstride
+    int dorder[PERM_MAX_DIMS];
+    for (int d = 0; d < nd; ++d) dorder[d] = d;
+    for (int i = 1; i < nd; ++i)
+        for (int j = i; j > 0 && dstride[dorder[j]] < dstride[dorder[j - 1]]; --j) { const int t = dorder[j]; dorder[j] = dorder[j - 1]; dorder[j - 1] = t; }
+    {   // destination-leading block: dorder[0] = p, ..., until source dim 0 appears
+        int64_t prod = 1;
+        int k = 0;
+        while (k < nd && dorder[k] != 0) { prod *= ext[dorder[k]]; ++k; }
+        if (k >= 1 && k < nd && prod <= max_run) {
+            for (int i = 0; i < k; ++i) { block[nb++] = dorder[i]; in_block[dorder[i]] = true; }
+            lane_dim = 0;
+        }
+    }
+    if (lane_dim < 0) {   // source-leading block: dims 0 .. p-1
+        int64_t prod = 1;
+        for (int d = 0; d < p; ++d) prod *= ext[d];
+        if (prod <= max_run) {
+            for (int d = 0; d < p; ++d) { block[nb++] = d; in_block[d] = true; }
+            lane_dim = p;
+            src_run = true;
+        }
+    }
+    if (lane_dim < 0) return false;
     PermSmallGeom g{};
-    g.small = (int32_t)ext[small_dim];
-    g.small_sstride = sstr[small_dim];
-    g.small_dstride = dstride[small_dim];
-    g.n_threads = total / ext[small_dim];
+    int64_t run = 1;
+    for (int i = 0; i < nb; ++i) run *= ext[block[i]];
+    g.small = (int32_t)run;
+    for (int64_t j = 0; j < run; ++j) {    // coordinates of element j inside the block, the first block dim fastest
+        int64_t rem = j, so = 0, dof = 0;
+        for (int i = 0; i < nb; ++i) {
+            const int64_t c = rem % ext[block[i]];
+            rem /= ext[block[i]];
+            so += c * sstr[block[i]];
+            dof += c * dstride[block[i]];
+        }
+        g.run_soff[j] = so;
+        g.run_doff[j] = dof;
+    }
+    (void)src_run;
+    g.n_threads = total / run;
     int k = 0;
     g.ext[k] = ext[lane_dim]; g.sstride[k] = sstr[lane_dim]; g.dstride[k] = dstride[lane_dim]; ++k;
     for (int d = 0; d < nd; ++d) {
-        if (d == small_dim || d == lane_dim) continue;
+        if (in_block[d] || d == lane_dim) continue;
         g.ext[k] = ext[d]; g.sstride[k] = sstr[d]; g.dstride[k] = dstride[d]; ++k;
     }
     g.nd = k;

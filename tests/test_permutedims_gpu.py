@@ -73,7 +73,8 @@ def test_front_end(rk, orc):
 @pytest.mark.parametrize("dtype", [np.bool_, np.int16, np.float32, np.float64, np.complex128])
 @pytest.mark.parametrize("shape,perm", [((100_003, 3), (2, 1)), ((3, 100_003), (2, 1)), ((65_537, 4), (2, 1)), ((4, 65_537), (2, 1)),
                                         ((8, 8, 5000), (2, 1, 3)), ((2, 7, 3001), (2, 1, 3)), ((1000, 5, 7, 3), (2, 1, 4, 3)),
-                                        ((6, 1000, 4), (3, 2, 1)), ((1, 5, 4099), (3, 2, 1)), ((8, 257, 2, 9), (3, 1, 4, 2)), ((2, 2, 2, 2, 70_001), (4, 3, 2, 1, 5))])
+                                        ((6, 1000, 4), (3, 2, 1)), ((1, 5, 4099), (3, 2, 1)), ((8, 257, 2, 9), (3, 1, 4, 2)), ((2, 2, 2, 2, 70_001), (4, 3, 2, 1, 5)),
+                                        ((2, 3, 100_001), (3, 2, 1)), ((100_001, 3, 2), (3, 2, 1)), ((2, 2, 2, 50_001, 3), (4, 3, 2, 1, 5)), ((4, 2, 70_001), (3, 1, 2))])
 def test_short_contiguous_dims(rk, orc, dtype, shape, perm):
     """A short contiguous dim on either side (arrays of structures <-> structures of arrays, batches of tiny matrices)."""
     _check(rk, orc, _rand(np.random.default_rng(71), dtype, shape), perm)
