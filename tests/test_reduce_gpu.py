@@ -350,3 +350,32 @@ def test_long_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
     c = rk.count(lambda v: v > 0, rk.ROCArray(x), dims=dims)
     ax = tuple(d - 1 for d in ((dims,) if isinstance(dims, int) else dims))
     assert np.array_equal(rk.Array(c), (x > 0).sum(axis=ax, keepdims=True))
+
+
+@pytest.mark.parametrize("m", [2, 3, 5, 8, 15, 16, 17, 20, 31, 32, 33, 48, 63, 64, 65, 100, 128, 129, 200, 255, 256])
+def test_many_short_contiguous_lines(rk, orc, m):
+    """dims=1 with 2 .. 256 elements a line and many lines (sum(A; dims=1) of a 32 x N array): whole lines staged through
+    LDS, 1 .. 16 lanes a line.  Line counts that fill a block exactly, leave a ragged last block, and an offset view
+    (no 16-byte alignment: the scalar loads)."""
+    rng = _rng(83 + m)
+    for n in (1024, 4111, 70_001):
+        for dtype in (np.float32, np.int64, np.float64, np.uint8):
+            x = rng.integers(0 if dtype == np.uint8 else -1000, 200 if dtype == np.uint8 else 1001, (m, n)).astype(dtype)
+            dx = rk.ROCArray(x)
+            for f, op in (("identity", "add_sum"), ("abs2", "max"), ("identity", "min")):
+                if dtype == np.uint8 and f == "abs2":
+                    continue
+                got = rk.Array(rk.mapreduce(f, op, dx, dims=1))
+                want = orc.mapreduce(f, op, x, dims=1)
+                if np.dtype(dtype).kind == "f" and op == "add_sum":
+                    np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-2)
+                else:
+                    assert np.array_equal(got, want.astype(got.dtype))
+        _check_findminmax(rk, orc, rng.integers(-2, 3, (m, n)).astype(np.float32), 1)        # ties: the first index wins
+        _check_findminmax(rk, orc, rng.standard_normal((m, n)), 1)
+        c = rk.count(lambda v: v > 0, dx, dims=1)
+        assert np.array_equal(rk.Array(c), (x > 0).sum(axis=0, keepdims=True))
+    flat = rng.standard_normal(m * 2000 + 3).astype(np.float32)
+    v = rk.ROCArray(flat).view_range(4, 3 + m * 2000).reshape(m, 2000)
+    got = rk.Array(rk.mapreduce("identity", "add_sum", v, dims=1))
+    np.testing.assert_allclose(got, flat[3:3 + m * 2000].reshape(2000, m).sum(axis=1, dtype=np.float64)[None, :], rtol=1e-5, atol=1e-4)
