@@ -234,3 +234,28 @@ def test_short_contiguous_lines(rk, orc, shape):
         assert np.array_equal(rk.Array(rk.accumulate("max", rk.ROCArray(x), dims=1)), orc.accumulate("max", x, dims=1))
     b = rng.random(shape) < 0.5
     assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=1)), orc.cumsum(b, dims=1))
+
+
+@pytest.mark.parametrize("m", [3, 5, 6, 7, 9, 13, 15, 17, 18, 31, 33, 63, 65, 101, 127, 129, 130, 255, 256])
+def test_short_contiguous_lines_of_any_length(rk, orc, m):
+    """dims=1 with lines of 3 .. 256 elements that are no whole number of 16-byte vectors (cumsum of a 15 x N array):
+    whole lines staged through LDS, 1 .. 16 lanes a line; exact and ragged last blocks, inclusive and exclusive, an
+    unaligned view, a Bool source."""
+    rng = _rng(91 + m)
+    for n in (1024, 4111, 30_001):
+        for dtype in (np.float32, np.float64, np.int32, np.int64):
+            x = rng.integers(-100, 101, (m, n)).astype(dtype)
+            dx = rk.ROCArray(x)
+            for op, init, inclusive in (("add", None, True), ("add", 3, False), ("max", None, True), ("min", -5, True)):
+                got = rk.Array(rk.accumulate(op, dx, dims=1, init=init, inclusive=inclusive))
+                want = orc.accumulate(op, x, dims=1, init=init, inclusive=inclusive)
+                assert np.array_equal(got, want.astype(got.dtype))          # small integers: Float32 sums are exact too
+        xf = rng.standard_normal((m, n)).astype(np.float32)
+        got = rk.Array(rk.cumsum(rk.ROCArray(xf), dims=1))
+        np.testing.assert_allclose(got, orc.cumsum(xf, dims=1), rtol=RTOL, atol=1e-4)
+        b = rng.random((m, n)) < 0.5
+        assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=1)), orc.cumsum(b, dims=1))
+    flat = rng.integers(-50, 51, m * 1500 + 3).astype(np.float32)
+    v = rk.ROCArray(flat).view_range(4, 3 + m * 1500).reshape(m, 1500)
+    got = rk.Array(rk.cumsum(v, dims=1))
+    assert np.array_equal(got, np.cumsum(flat[3:3 + m * 1500].reshape(1500, m), axis=1).T)
