@@ -13,7 +13,7 @@
 //                          fixed order (deterministic, single launch)
 //   reduce_wave_kernel     many medium lines: one wave per line, no LDS, no barrier
 //   reduce_thread_kernel   very many tiny lines: one lane per line
-//   reduce_short_lines_kernel  many contiguous lines of 2 .. 256 elements: whole lines through LDS
+//   reduce_short_lines_kernel  many short lines (contiguous, or inner < 64): whole inner x mid slabs through LDS
 //   reduce_narrow_kernel   1 < inner < 64 with long lines: contiguous runs of whole rows
 //   reduce_strided_kernel  inner >= 64: lanes run along the contiguous `inner` axis (128-bit
 //                          loads), waves and workgroups split `mid`
@@ -313,32 +313,35 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
     sink(line, a);
 }
 
-// ---- many contiguous lines of 2 .. 256 elements: whole lines through LDS -----------------------------------------
-// (sum(A; dims=1) of a 32 x 1_000_000 array.)  A wave per line leaves most lanes idle or gives each wave too little to
-// keep loads in flight, and a lane per line reads with a stride; here a workgroup copies a run of whole lines --
-// contiguous memory, 16-byte vectors -- into LDS, and a group of tpl = 1, 2, .. 16 lanes folds each line from there
-// (lane `part` takes the elements e = part (mod tpl), then a DPP fold across the group).  f is applied on the way out
-// of LDS, so LDS holds 1 .. 8 bytes an element whatever the accumulator is (16 for findmax).
-// Line l is walked from element rot(l) with wrap-around (the operators are commutative, and the index rule of
-// findmax / findmin does not depend on the order): rot(l) = l * (tpl - m) mod P, P the largest power of two <= min(m, 64),
-// puts lane (l, part) at an address = l * tpl + part (mod P), which spreads the lanes of a wave over the banks for
-// every m (a common start is a 32-way conflict for m = 32; l mod m is one for m = 31).
-// The host picks lines_per_block so that a block's first element is 16-byte aligned when the array is (VECTOR).
+// ---- many short lines, contiguous or with a narrow inner extent: whole slabs through LDS -----------------------
+// (sum(A; dims=1) of a 32 x 1_000_000 array; sum(A; dims=2) of a 4 x 32 x 250_000 array.)  A slab is the inner x mid
+// block of one outer index, contiguous in memory.  A wave per line leaves most lanes idle or gives each wave too
+// little to keep loads in flight, and a lane per line reads with a stride; here a workgroup copies a run of whole
+// slabs -- contiguous memory, 16-byte vectors -- into LDS, and a group of tpl = 1, 2, .. 16 lanes folds each line from
+// there (lane `part` takes the elements k = part (mod tpl), then a DPP fold across the group).  f is applied on the
+// way out of LDS, so LDS holds 1 .. 8 bytes an element whatever the accumulator is (16 for findmax).
+// The lines of slab s are walked from element rot(s) with wrap-around (the operators are commutative, and the index
+// rule of findmax / findmin does not depend on the order): rot(s) = s * (tpl - m) mod P, P the largest power of two
+// <= min(m, 64), puts lane (s, i, part) at an address = inner * (s * tpl + part) + i (mod inner * P), which spreads the
+// lanes of a wave over the banks for every m (with inner = 1 a common start is a 32-way conflict for m = 32; s mod m
+// is one for m = 31).
+// The host picks slabs_per_block so that a block's first element is 16-byte aligned when the array is (VECTOR).
 template <typename In> struct ShortLinesTile { static constexpr int ELEMS = 16384 / sizeof(In); };
-constexpr int SHORT_LINES_MAX = 256;
+constexpr int SHORT_LINES_MAX = 256;          // contiguous lines beyond this do as well with a wave each
 
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR>
-__global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __restrict__ A, int m, int64_t nlines, int lines_per_block,
+__global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __restrict__ A, int inner, int m, int64_t nslabs, int slabs_per_block,
                                                                  int tpl_log2, int rot_mask, Xf xf, Op op, Sink sink) {
     typedef typename Xf::Pos Pos;
     constexpr int TE = ShortLinesTile<In>::ELEMS;
     __shared__ __attribute__((aligned(16))) In lds[TE];
     const int t = threadIdx.x;
-    const int64_t line0 = (int64_t)blockIdx.x * lines_per_block;
-    int64_t left = nlines - line0;
-    const int nl = left < lines_per_block ? (int)left : lines_per_block;     // > 0 by the grid size
-    const int ne = nl * m;                                                    // <= TE by the choice of lines_per_block
-    const In* p = A + line0 * m;
+    const int slab = inner * m;
+    const int64_t slab0 = (int64_t)blockIdx.x * slabs_per_block;
+    const int64_t left = nslabs - slab0;
+    const int ns = left < slabs_per_block ? (int)left : slabs_per_block;     // > 0 by the grid size
+    const int ne = ns * slab;                                                 // <= TE by the choice of slabs_per_block
+    const In* p = A + slab0 * slab;
     constexpr int VEC = VECTOR ? 16 / sizeof(In) : 1;
     typedef typename VecOf<In, VEC>::type V;
     const int nv = ne / VEC;
@@ -349,18 +352,20 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
     for (int e = nv * VEC + t; e < ne; e += 256) lds[e] = p[e];             // fewer than VEC elements
     __syncthreads();
     const int tpl = 1 << tpl_log2;                       // <= 16 and <= m
+    const int nl = ns * inner;
     const int items = nl << tpl_log2;
     for (int base = 0; base < items; base += 256) {      // uniform trip count: the DPP fold below needs every lane
         const int idx = base + t;
         const int l = idx >> tpl_log2, part = idx & (tpl - 1);
         Acc acc = Op::template identity<Acc>();
         if (l < nl) {
-            const In* row = lds + l * m;
-            const int count = (m - part + tpl - 1) >> tpl_log2;          // elements e = part (mod tpl) of 0 .. m-1
-            int k = part + ((l * (tpl - m)) & rot_mask);                  // < tpl + P <= 2 m
+            const int sl = l / inner;
+            const In* line = lds + sl * slab + (l - sl * inner);
+            const int count = (m - part + tpl - 1) >> tpl_log2;          // elements k = part (mod tpl) of 0 .. m-1
+            int k = part + ((sl * (tpl - m)) & rot_mask);                 // < tpl + P <= 2 m
             if (k >= m) k -= m;
             for (int c = 0; c < count; ++c) {
-                acc = op(acc, xf(row[k], (Pos)k));
+                acc = op(acc, xf(line[k * inner], (Pos)k));
                 k += tpl;
                 if (k >= m) k -= m;
             }
@@ -369,7 +374,7 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
         if (tpl_log2 >= 2) acc = op(acc, dpp_move<DPP_QUAD_XOR2>(acc, acc));
         if (tpl_log2 >= 3) acc = op(acc, dpp_move<DPP_ROW_HALF_MIRROR>(acc, acc));
         if (tpl_log2 >= 4) acc = op(acc, dpp_move<DPP_ROW_MIRROR>(acc, acc));
-        if (l < nl && part == 0) sink(line0 + l, acc);
+        if (l < nl && part == 0) sink(slab0 * inner + l, acc);
     }
 }
 
@@ -633,6 +638,7 @@ struct ReducePlan {
     int     splits;      // SPLIT: workgroups per line; STRIDED, NARROW: slices of mid
     int64_t rows_per_split;   // NARROW
     int     strips;      // STRIDED
+    int     slabs_per_block, tpl_log2, rot_mask;      // SHORT_LINES
     size_t  payload;     // bytes of partials
 };
 
@@ -649,6 +655,33 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
     constexpr int VEC = 16 / sizeof(In);
     if (!single_run) { p.kind = ReducePlan::GENERIC; return p; }
     const int64_t nlines = s.inner * s.outer;
+    const int64_t slab = s.inner * s.mid;
+    // (rows of 64 elements or more that are whole vectors stream as well through the strided kernel)
+    if (s.mid >= 2 && nlines >= 1024 && slab <= ShortLinesTile<In>::ELEMS && (s.inner > 1 || s.mid <= SHORT_LINES_MAX) &&
+        (s.inner < 64 || s.inner % VEC != 0 || !is_aligned(A, 16))) {
+        // whole slabs per block, and (for the vector loads) a block size in bytes that is a multiple of 16
+        int spb = ShortLinesTile<In>::ELEMS / (int)slab;
+        bool vector = is_aligned(A, 16);
+        if (vector) {
+            int q = 16;                                                      // 16 / gcd(slab bytes, 16)
+            for (size_t bytes = (size_t)slab * sizeof(In); q > 1 && bytes % 2 == 0; bytes /= 2) q /= 2;
+            if (spb / q > 0) spb -= spb % q;
+            else vector = false;
+        }
+        const int lines = spb * (int)s.inner;
+        int tl = 0;
+        while (tl < 4 && (lines << tl) < 256 && (2 << tl) <= s.mid) ++tl;
+        if ((lines << tl) >= 128) {                                          // else too few lanes would fold
+            int pow2 = 1;
+            while (pow2 * 2 <= s.mid && pow2 < 64) pow2 *= 2;
+            p.kind = ReducePlan::SHORT_LINES;
+            p.vector = vector;
+            p.slabs_per_block = spb;
+            p.tpl_log2 = tl;
+            p.rot_mask = pow2 - 1;
+            return p;
+        }
+    }
     if (s.inner >= 64) {
         p.kind = ReducePlan::STRIDED;
         p.vector = (s.inner % VEC == 0) && is_aligned(A, 16);
@@ -671,11 +704,6 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
         }
         p.splits = (int)ms;
         p.payload = ms > 1 ? (size_t)(tiles * ms * cols) * sizeof(Acc) : 0;
-        return p;
-    }
-    if (s.inner == 1 && s.mid >= 2 && s.mid <= SHORT_LINES_MAX && nlines >= 1024) {
-        p.kind = ReducePlan::SHORT_LINES;
-        p.vector = is_aligned(A, 16);
         return p;
     }
     if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
@@ -763,26 +791,14 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
             break;
         }
         case ReducePlan::SHORT_LINES: {
-            // whole lines per block, and (for the vector loads) a block size in bytes that is a multiple of 16
-            const int m = (int)s.mid;
-            int lpb = ShortLinesTile<In>::ELEMS / m;                             // >= 8
-            bool vector = p.vector;
-            if (vector) {
-                int q = 16;                                                      // 16 / gcd(line bytes, 16)
-                for (size_t bytes = (size_t)m * sizeof(In); q > 1 && bytes % 2 == 0; bytes /= 2) q /= 2;
-                if (lpb / q > 0) lpb -= lpb % q;
-                else vector = false;
-            }
-            int tpl_log2 = 0;
-            while (tpl_log2 < 4 && (lpb << tpl_log2) < 256) ++tpl_log2;           // 2^tpl_log2 <= 16 < m whenever lpb < 256
-            int pow2 = 1;
-            while (pow2 * 2 <= m && pow2 < 64) pow2 *= 2;
-            const int64_t blocks = (g.nlines + lpb - 1) / lpb;
+            const int64_t blocks = (s.outer + p.slabs_per_block - 1) / p.slabs_per_block;
             if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-            if (vector)
-                reduce_short_lines_kernel<In, Acc, Xf, Op, Sink, true><<<(unsigned)blocks, 256, 0, stream>>>(A, m, g.nlines, lpb, tpl_log2, pow2 - 1, xf, op, sink);
+            if (p.vector)
+                reduce_short_lines_kernel<In, Acc, Xf, Op, Sink, true><<<(unsigned)blocks, 256, 0, stream>>>(
+                    A, (int)s.inner, (int)s.mid, s.outer, p.slabs_per_block, p.tpl_log2, p.rot_mask, xf, op, sink);
             else
-                reduce_short_lines_kernel<In, Acc, Xf, Op, Sink, false><<<(unsigned)blocks, 256, 0, stream>>>(A, m, g.nlines, lpb, tpl_log2, pow2 - 1, xf, op, sink);
+                reduce_short_lines_kernel<In, Acc, Xf, Op, Sink, false><<<(unsigned)blocks, 256, 0, stream>>>(
+                    A, (int)s.inner, (int)s.mid, s.outer, p.slabs_per_block, p.tpl_log2, p.rot_mask, xf, op, sink);
             break;
         }
         case ReducePlan::STRIDED: {

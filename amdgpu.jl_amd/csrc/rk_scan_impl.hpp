@@ -12,7 +12,7 @@
 //       scan_strided_kernel    4 waves x register tiles of rows, column totals through LDS
 //       scan_narrow_kernel     1 < inner < 64 with long lines: tiles of whole rows through LDS
 //   scan_thread_kernel         one lane per line (tiny lines)
-//   scan_lds_lines_kernel      short contiguous lines of any length: whole lines through LDS
+//   scan_lds_lines_kernel      short lines of any length (contiguous, or short along a narrow inner): whole slabs through LDS
 #pragma once
 
 #include "rk_common.hpp"
@@ -424,27 +424,30 @@ __global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __res
     }
 }
 
-// ---- short contiguous lines of any length: whole lines through LDS ------------------------------------------------
+// ---- short lines of any length, contiguous or with a narrow inner extent: whole slabs through LDS -----------------
 // (cumsum(A; dims=1) of a 15 x 2_000_000 array: the line length is no multiple of the 16-byte vector, so lines start
-// at odd addresses; a lane per line reads with a stride of 60 bytes -- 425 us -- and a wave per line idles 49 lanes.)
-// A workgroup copies a 16 KiB run of whole lines into LDS with 16-byte loads (the host picks the lines per block so
-// that every block starts at a whole vector), a group of tpl = 1, 2 .. 16 lanes scans each line in place -- lane `part`
-// owns a segment of ceil(m / tpl) elements, the segment totals are scanned over the group's lanes by shuffles that
-// never cross a group -- and the tile leaves with 16-byte stores.
-constexpr int SCAN_LDS_LINES_MAX = 128;     // beyond, and for whole vectors beyond 64, a wave per line does as well or better
+// at odd addresses; a lane per line reads with a stride of 60 bytes -- 425 us -- and a wave per line idles 49 lanes.
+// cumsum(A; dims=2) of a 4 x 32 x 250_000 array: a lane per line walks 32 rows of 16 bytes.)
+// A slab is the inner x mid block of one outer index, contiguous in memory.  A workgroup copies a 16 KiB run of whole
+// slabs into LDS with 16-byte loads (the host picks the slabs per block so that every block starts at a whole vector),
+// a group of tpl = 1, 2 .. 16 lanes scans each line in place -- lane `part` owns a segment of ceil(m / tpl) elements,
+// the segment totals are scanned over the group's lanes by shuffles that never cross a group -- and the tile leaves
+// with 16-byte stores.
+constexpr int SCAN_LDS_LINES_MAX = 128;     // contiguous lines beyond, and whole vectors beyond 64: a wave per line does as well or better
 
 template <typename In, typename T, typename Op, bool VECTOR>
-__global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int m, int64_t nlines,
-                                                             int lines_per_block, int tpl_log2, T init, int inclusive, Op op) {
+__global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int inner, int m, int64_t nslabs,
+                                                             int slabs_per_block, int tpl_log2, T init, int inclusive, Op op) {
     constexpr int TE = 16384 / sizeof(T);
     __shared__ __attribute__((aligned(16))) T lds[TE];
     const int t = threadIdx.x;
-    const int64_t line0 = (int64_t)blockIdx.x * lines_per_block;
-    const int64_t left = nlines - line0;
-    const int nl = left < lines_per_block ? (int)left : lines_per_block;     // > 0 by the grid size
-    const int ne = nl * m;                                                    // <= TE by the choice of lines_per_block
-    const In* p = in + line0 * m;
-    T* q = out + line0 * m;
+    const int slab = inner * m;
+    const int64_t slab0 = (int64_t)blockIdx.x * slabs_per_block;
+    const int64_t left = nslabs - slab0;
+    const int ns = left < slabs_per_block ? (int)left : slabs_per_block;     // > 0 by the grid size
+    const int ne = ns * slab;                                                 // <= TE by the choice of slabs_per_block
+    const In* p = in + slab0 * slab;
+    T* q = out + slab0 * slab;
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     typedef typename VecOf<In, VEC>::type VI;
     typedef typename VecOf<T, VEC>::type VT;
@@ -464,6 +467,7 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
     __syncthreads();
     const int tpl = 1 << tpl_log2;
     const int seg = (m + tpl - 1) >> tpl_log2;
+    const int nl = ns * inner;
     const int items = nl << tpl_log2;
     for (int base = 0; base < items; base += 256) {       // uniform trip count: the shuffles below need every lane
         const int idx = base + t;
@@ -471,13 +475,14 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
         const int k0 = part * seg;
         const int k1 = k0 + seg < m ? k0 + seg : m;
         const bool live = l < nl && k0 < m;                // empty segments sit at the end of a group: nothing reads them
-        T* row = lds + (live ? l * m : 0);
+        const int sl = live ? l / inner : 0;
+        T* line = lds + (live ? sl * slab + (l - sl * inner) : 0);
         T tot = init;
         if (live) {
-            tot = row[k0];
+            tot = line[k0 * inner];
             for (int k = k0 + 1; k < k1; ++k) {
-                tot = op(tot, row[k]);
-                row[k] = tot;
+                tot = op(tot, line[k * inner]);
+                line[k * inner] = tot;
             }
         }
         for (int d = 1; d < tpl; d <<= 1) {
@@ -488,16 +493,16 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
         const T before = part > 0 ? op(init, prev) : init;
         if (live) {
             if (inclusive) {
-                for (int k = k0; k < k1; ++k) row[k] = op(before, row[k]);
+                for (int k = k0; k < k1; ++k) line[k * inner] = op(before, line[k * inner]);
             } else {
-                for (int k = k1 - 1; k > k0; --k) row[k] = op(before, row[k - 1]);
-                row[k0] = before;
+                for (int k = k1 - 1; k > k0; --k) line[k * inner] = op(before, line[(k - 1) * inner]);
+                line[k0 * inner] = before;
             }
         }
     }
     __syncthreads();
     for (int i = t; i < nv; i += 256) {
-        if constexpr (VEC == 1) out[line0 * m + i] = lds[i];
+        if constexpr (VEC == 1) q[i] = lds[i];
         else store_nt((VT*)q + i, ((const VT*)lds)[i]);
     }
     for (int e = nv * VEC + t; e < ne; e += 256) q[e] = lds[e];
@@ -827,6 +832,38 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const bool aligned = is_aligned(in, VEC * sizeof(In)) && is_aligned(out, 16);
     const int inclusive = a.inclusive ? 1 : 0;
 
+    {
+        // short lines whose inner x mid slabs fit an LDS tile.  Contiguous lines that are whole vectors have their own
+        // kernel below (up to 32 vectors) or do as well with a wave each (beyond 64 elements); with 16 .. 63 elements in
+        // a row a lane per line reads whole 64-byte pieces and is faster (32 x 32 x 32768 Float32: 44 against 52 us).
+        const int64_t slab = s.inner * s.mid;
+        const int64_t all_lines = s.inner * s.outer;
+        const bool whole_vectors = aligned && s.inner == 1 && s.mid % VEC == 0 && (s.mid / VEC <= 32 || s.mid > 64);
+        if (s.mid >= 2 && all_lines >= 1024 && slab <= (int64_t)(16384 / sizeof(T)) && !whole_vectors &&
+            (s.inner > 1 ? (s.inner < 16 || s.inner >= 64) : (s.mid >= 3 && s.mid <= SCAN_LDS_LINES_MAX))) {
+            int spb = (int)(16384 / sizeof(T)) / (int)slab;
+            bool vector = aligned;
+            if (vector) {
+                int q = VEC;                                                  // VEC / gcd(slab, VEC)
+                for (int64_t e = slab; q > 1 && e % 2 == 0; e /= 2) q /= 2;
+                if (spb / q > 0) spb -= spb % q;
+                else vector = false;
+            }
+            const int lines = spb * (int)s.inner;
+            int tl = 0;
+            while (tl < 4 && (lines << tl) < 256 && (2 << tl) <= s.mid) ++tl;
+            if ((lines << tl) >= 128) {                                       // else too few lanes would scan
+                const int64_t blocks = (s.outer + spb - 1) / spb;
+                if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+                if (vector)
+                    scan_lds_lines_kernel<In, T, Op, true><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
+                else
+                    scan_lds_lines_kernel<In, T, Op, false><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
+                RK_LAUNCH_CHECK();
+                return RK_SUCCESS;
+            }
+        }
+    }
     if (s.inner >= 64) {
         Workspace w{};
         char* scratch = nullptr;
@@ -851,27 +888,6 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const int64_t blocks = (nlines + per_block - 1) / per_block;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
         scan_short_lines_kernel<In, T, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, L, nlines, init, inclusive, op);
-        RK_LAUNCH_CHECK();
-        return RK_SUCCESS;
-    }
-    if (s.inner == 1 && s.mid >= 3 && s.mid <= SCAN_LDS_LINES_MAX && nlines >= 1024 && !(aligned && s.mid % VEC == 0 && s.mid > 64)) {
-        // whole lines per block and, for the vector path, a whole number of vectors
-        const int m = (int)s.mid;
-        int lpb = (int)(16384 / sizeof(T)) / m;                           // >= 8
-        bool vector = aligned;
-        if (vector) {
-            int q = VEC;                                                  // VEC / gcd(m, VEC)
-            for (int mm = m; q > 1 && mm % 2 == 0; mm /= 2) q /= 2;
-            lpb -= lpb % q;                                               // q <= VEC <= lpb
-        }
-        int tpl_log2 = 0;
-        while (tpl_log2 < 4 && (lpb << tpl_log2) < 256) ++tpl_log2;
-        const int64_t blocks = (nlines + lpb - 1) / lpb;
-        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-        if (vector)
-            scan_lds_lines_kernel<In, T, Op, true><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, m, nlines, lpb, tpl_log2, init, inclusive, op);
-        else
-            scan_lds_lines_kernel<In, T, Op, false><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, m, nlines, lpb, tpl_log2, init, inclusive, op);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }

@@ -379,3 +379,30 @@ def test_many_short_contiguous_lines(rk, orc, m):
     v = rk.ROCArray(flat).view_range(4, 3 + m * 2000).reshape(m, 2000)
     got = rk.Array(rk.mapreduce("identity", "add_sum", v, dims=1))
     np.testing.assert_allclose(got, flat[3:3 + m * 2000].reshape(2000, m).sum(axis=1, dtype=np.float64)[None, :], rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("shape,dims", [((2, 8, 5000), 2), ((4, 32, 3001), 2), ((4, 100, 1025), 2), ((16, 20, 2000), 2), ((3, 17, 4099), 2),
+                                        ((8, 300, 500), 2), ((32, 32, 1000), 2), ((5, 5, 30_001), 2), ((48, 64, 333), 2), ((63, 65, 129), 2),
+                                        ((2, 8, 5, 1000), 2), ((3, 2, 7, 4000), 3), ((2, 2, 2, 2, 9000), (3, 4)), ((7, 2, 100_000), 2)])
+def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
+    """1 < inner < 64 with a short reduced dim and many slabs (sum(A; dims=2) of a 4 x 32 x N array): whole inner x mid
+    slabs staged through LDS."""
+    rng = _rng(97)
+    for dtype in (np.float32, np.int32, np.int64, np.float64, np.uint8):
+        x = rng.integers(0 if dtype == np.uint8 else -1000, 200 if dtype == np.uint8 else 1001, shape).astype(dtype)
+        dx = rk.ROCArray(x)
+        for f, op in (("identity", "add_sum"), ("abs2", "max"), ("identity", "min")):
+            if dtype == np.uint8 and f == "abs2":
+                continue
+            got = rk.Array(rk.mapreduce(f, op, dx, dims=dims))
+            want = orc.mapreduce(f, op, x, dims=dims)
+            if np.dtype(dtype).kind == "f" and op == "add_sum":
+                np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-2)
+            else:
+                assert np.array_equal(got, want.astype(got.dtype))
+    if isinstance(dims, int):
+        _check_findminmax(rk, orc, rng.integers(-2, 3, shape).astype(np.float32), dims)
+        _check_findminmax(rk, orc, rng.standard_normal(shape), dims)
+    c = rk.count(lambda v: v > 100, dx, dims=dims)
+    ax = tuple(d - 1 for d in ((dims,) if isinstance(dims, int) else dims))
+    assert np.array_equal(rk.Array(c), (x > 100).sum(axis=ax, keepdims=True))

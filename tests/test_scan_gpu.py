@@ -259,3 +259,23 @@ def test_short_contiguous_lines_of_any_length(rk, orc, m):
     v = rk.ROCArray(flat).view_range(4, 3 + m * 1500).reshape(m, 1500)
     got = rk.Array(rk.cumsum(v, dims=1))
     assert np.array_equal(got, np.cumsum(flat[3:3 + m * 1500].reshape(1500, m), axis=1).T)
+
+
+@pytest.mark.parametrize("shape,dims", [((2, 8, 5000), 2), ((4, 32, 3001), 2), ((4, 100, 1025), 2), ((16, 20, 2000), 2), ((3, 17, 4099), 2),
+                                        ((8, 300, 500), 2), ((32, 32, 1000), 2), ((5, 5, 30_001), 2), ((48, 64, 333), 2), ((63, 65, 129), 2),
+                                        ((2, 8, 5, 1000), 2), ((3, 2, 7, 4000), 3), ((64, 16, 300), 2), ((100, 7, 1000), 2), ((7, 2, 100_000), 2)])
+def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
+    """A short scanned dim behind a narrow inner extent, many slabs (cumsum(A; dims=2) of a 4 x 32 x N array): whole
+    inner x mid slabs staged through LDS."""
+    rng = _rng(101)
+    for dtype in (np.float32, np.float64, np.int32, np.int64):
+        x = rng.integers(-100, 101, shape).astype(dtype)
+        dx = rk.ROCArray(x)
+        for op, init, inclusive in (("add", None, True), ("add", 3, False), ("max", None, True), ("min", -5, True)):
+            got = rk.Array(rk.accumulate(op, dx, dims=dims, init=init, inclusive=inclusive))
+            want = orc.accumulate(op, x, dims=dims, init=init, inclusive=inclusive)
+            assert np.array_equal(got, want.astype(got.dtype))              # small integers: Float32 sums are exact too
+    xf = rng.standard_normal(shape).astype(np.float32)
+    np.testing.assert_allclose(rk.Array(rk.cumsum(rk.ROCArray(xf), dims=dims)), orc.cumsum(xf, dims=dims), rtol=RTOL, atol=1e-4)
+    b = rng.random(shape) < 0.5
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=dims)), orc.cumsum(b, dims=dims))
