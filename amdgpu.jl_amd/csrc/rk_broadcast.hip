@@ -31,6 +31,7 @@ struct BcOperand {
     int64_t     stride0;    // element stride along merged dim 0: 0 (extruded), 1 (dense) or any other (views; scalar lanes only)
     int32_t     reused;     // has an extruded dim: elements are read many times -> cached loads, not streaming
     int32_t     row_invariant;   // every stride of dims 1.. is 0: the value depends on the dim-0 index only
+    int32_t     flat_dense;      // dense over the whole merged shape: the element offset is the destination's linear index
     int64_t     stride[RK_MAX_DIMS];   // element strides of merged dims 1.. (index d-1)
     double      sf;
     int64_t     si;
@@ -45,6 +46,7 @@ struct BcArgs {
     int64_t   shape[RK_MAX_DIMS];      // merged dest shape
     int64_t   total;
     int64_t   nrows;                   // product of shape[1..]
+    int32_t   indexed;                 // indexed mode (bc_indexed_kernel) instead of rows mode
     int32_t   tx_log2;                 // rows mode: lanes along dim 0 = 1 << tx_log2
     int64_t   nxb;                     // rows mode: workgroups along dim 0
     void*     dest;
@@ -358,15 +360,18 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
 #pragma unroll
         for (int k = 0; k < Eval::NOPS; ++k) off[k] = dest_off * a.op[k].stride0;
     } else {
-        // A thread keeps its dim-0 position and walks BC_RPT consecutive rows: operands that do not depend
-        // on the row (a column vector against a matrix) are loaded once, and the index arithmetic is paid
-        // once per BC_RPT vectors.
+        // A thread keeps its dim-0 position and takes BC_RPT rows: operands that do not depend on the row (a
+        // column vector against a matrix) are loaded once.  The rows of a thread lie TY = BC_BLOCK >> tx_log2
+        // apart, so that the threads of a workgroup cover TY consecutive rows with every load: with a short
+        // dim 0 (4 x 32 x 262144 .+ 4 x 1 x 262144: one 16-byte vector a row) consecutive rows per thread made
+        // every load touch 16 bytes in 64 (216 us; 49 us this way).
         // The fused evaluators issue the loads of all BC_RPT rows before the first use (rows past the end
         // are clamped for the loads and skipped for the store); the interpreter goes row by row.
         const int64_t xb = blockIdx.x, rb = (int64_t)blockIdx.y + (int64_t)blockIdx.z * gridDim.y;
         const int tx = t & ((1 << a.tx_log2) - 1), ty = t >> a.tx_log2;
         const int64_t i0 = ((xb << a.tx_log2) + tx) * VEC;
-        const int64_t row0 = (rb * (BC_BLOCK >> a.tx_log2) + ty) * BC_RPT;
+        const int rows_apart = BC_BLOCK >> a.tx_log2;
+        const int64_t row0 = rb * (rows_apart * BC_RPT) + ty;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
         const bool wave_rows = a.tx_log2 >= 6;     // 64 or more lanes along dim 0: the lanes of a wave share their rows
         constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? 2 : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
@@ -375,7 +380,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
             int64_t doff[NB];
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                int64_t row = row0 + r0 + b;
+                int64_t row = row0 + (int64_t)(r0 + b) * rows_apart;
                 if (row >= a.nrows) row = a.nrows - 1;
                 // (the interpreter declares room for every operand slot: skip the 64-bit index arithmetic of the
                 // slots the program does not use -- it was most of that kernel's instructions in this mode)
@@ -405,7 +410,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
             }
 #pragma unroll
             for (int b = 0; b < NB; ++b) {
-                const int64_t row = row0 + r0 + b;
+                const int64_t row = row0 + (int64_t)(r0 + b) * rows_apart;
                 if (row < a.nrows) {
                     CT out[VEC];
                     Eval::template run<CT, VEC>(a, in[b], out, lds);
@@ -424,6 +429,74 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
     CT out[VEC];
     Eval::template run<CT, VEC>(a, in, out, lds);
     store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, dest_off, out);
+}
+
+// Indexed mode: a dense destination whose rows are no whole number of 16-byte vectors (3 x N .+ 1 x N, 17 x N .* 17 x 1,
+// 8191 x 4099 .+ 1 x 4099) and at most BC_INDEXED_DIMS merged dims.  Lanes along dim 0 move one element each there (and
+// idle when dim 0 is short: 3 x 11184810 .+ 1 x 11184810 Float32 144 us, 63 us here); a thread owns VEC consecutive
+// elements of the destination's linear order: one 16-byte store, one 16-byte load per dense operand, and for every
+// other operand VEC single loads at offsets found by splitting the linear index once (three 32-bit divisions) and
+// counting up with carries.
+constexpr int BC_INDEXED_DIMS = 4;
+
+template <typename Eval, typename CT, int VEC, bool HOMOG>
+__global__ __launch_bounds__(BC_BLOCK) void bc_indexed_kernel(const BcArgs a) {
+    CT* lds = (CT*)bc_lds_raw;
+    const int64_t e0 = ((int64_t)blockIdx.x * BC_BLOCK + threadIdx.x) * VEC;
+    if (e0 >= a.total) return;
+    const int valid = a.total - e0 < VEC ? (int)(a.total - e0) : VEC;      // < VEC in the last thread of a ragged total
+    const uint32_t s0 = (uint32_t)a.shape[0], s1 = (uint32_t)a.shape[1], s2 = (uint32_t)a.shape[2];    // 1 beyond the rank
+    uint32_t c[VEC][BC_INDEXED_DIMS];
+    {
+        uint32_t r = (uint32_t)e0;           // total < 2^32
+        c[0][0] = r % s0; r /= s0;
+        c[0][1] = r % s1; r /= s1;
+        c[0][2] = r % s2;
+        c[0][3] = r / s2;
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) {
+            uint32_t c0 = c[j - 1][0] + 1, c1 = c[j - 1][1], c2 = c[j - 1][2], c3 = c[j - 1][3];
+            if (c0 == s0) {
+                c0 = 0;
+                if (++c1 == s1) {
+                    c1 = 0;
+                    if (++c2 == s2) { c2 = 0; ++c3; }
+                }
+            }
+            c[j][0] = c0; c[j][1] = c1; c[j][2] = c2; c[j][3] = c3;
+        }
+    }
+    CT in[RK_MAX_OPERANDS][VEC];
+#pragma unroll
+    for (int k = 0; k < Eval::NOPS; ++k) {
+        if (k >= a.n_operands) continue;
+        const BcOperand& o = a.op[k];
+        if (o.ptr == nullptr || (o.flat_dense != 0 && valid == VEC)) {
+            load_operand<CT, VEC, false, HOMOG>(o, e0, false, in[k]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                if (j >= valid) { in[k][j] = in[k][0]; continue; }          // past the end: any value, never stored
+                const int64_t off = (int64_t)c[j][0] * o.stride0 + (int64_t)c[j][1] * o.stride[0] + (int64_t)c[j][2] * o.stride[1] +
+                                    (int64_t)c[j][3] * o.stride[2];
+                CT one[1];
+                load_typed<CT, 1, true, HOMOG>(o, off, true, false, one);
+                in[k][j] = one[0];
+            }
+        }
+    }
+    CT out[VEC];
+    Eval::template run<CT, VEC>(a, in, out, lds);
+    if (valid == VEC) {
+        store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, e0, out);
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC - 1; ++j) {
+            if (j >= valid) break;
+            const CT one[1] = {out[j]};
+            store_dest<CT, 1, HOMOG>(a.dest, a.dest_dtype, e0 + j, one);
+        }
+    }
 }
 
 template <typename Eval, typename CT>
@@ -451,7 +524,12 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
     for (int k = 0; k < a.n_operands; ++k)
         if (a.op[k].ptr != nullptr && a.op[k].dtype != a.dest_dtype) homog = false;
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
-    if (vec) {
+    if (a.indexed != 0) {            // the planner sets it together with vec and rows
+        const int64_t blocks = ((a.total + 3) / 4 + BC_BLOCK - 1) / BC_BLOCK;
+        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+        if (homog) bc_indexed_kernel<Eval, CT, 4, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        else bc_indexed_kernel<Eval, CT, 4, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+    } else if (vec) {
         if (rows) { if (homog) RK_BC_LAUNCH(4, true, true); else RK_BC_LAUNCH(4, true, false); }
         else      { if (homog) RK_BC_LAUNCH(4, false, true); else RK_BC_LAUNCH(4, false, false); }
     } else {
@@ -627,6 +705,26 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
                 for (int d = 1; d < m; ++d)
                     if (mstride[k][d] % 4 != 0) vec = false;
             }
+        }
+    }
+    if (!linear && !vec && m <= BC_INDEXED_DIMS && total < (1ll << 32) &&
+        is_aligned(dest, 4 * dtype_size(dest_dtype))) {
+        // rows that are no whole number of vectors, dense destination: threads along the linear index
+        bool ok = mstride[KD][0] == 1;
+        int64_t dense = mshape[0];
+        for (int d = 1; d < m && ok; ++d) { ok = mstride[KD][d] == dense; dense *= mshape[d]; }
+        for (int k = 0; k < prog->n_operands && ok; ++k) {
+            if (prog->operands[k].ptr == nullptr) continue;
+            bool fd = mstride[k][0] == 1;
+            int64_t ds = mshape[0];
+            for (int d = 1; d < m && fd; ++d) { fd = mstride[k][d] == ds; ds *= mshape[d]; }
+            a.op[k].flat_dense = fd ? 1 : 0;
+            if (fd && !is_aligned(prog->operands[k].ptr, 4 * dtype_size(prog->operands[k].dtype))) ok = false;
+        }
+        if (ok) {
+            a.indexed = 1;
+            vec = true;
+            for (int d = m; d < BC_INDEXED_DIMS; ++d) a.shape[d] = 1;
         }
     }
     if (!linear) {

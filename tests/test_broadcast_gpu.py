@@ -280,3 +280,35 @@ def test_float16_arrays(rk):
     assert np.array_equal(rk.Array(rk.materialize(lz(X) > lz(Y))), x > y)
     s = rk.sum(lambda v: v * v, X)                               # closures over Float16 arrays: map first, then reduce
     assert isinstance(s, np.float16) and abs(float(s) - float((x * x).astype(np.float64).sum())) <= 2.0**-9 * float((x * x).astype(np.float64).sum())
+
+
+@pytest.mark.parametrize("shape,others", [((3, 40_000), [(3, 1), (1, 40_000)]), ((17, 4000), [(17, 1), (1, 4000)]), ((5, 7, 800), [(5, 1, 800), (1, 7, 1)]),
+                                          ((2, 2, 2, 30_000), [(2, 1, 2, 1), (1, 2, 1, 30_000)]), ((6, 10_002), [(1, 10_002), (6, 10_002)]),
+                                          ((63, 4, 100), [(63, 1, 100), (1, 4, 1)]), ((3, 40_001), [(1, 40_001), (3, 1)]), ((17, 4001), [(17, 1), (1, 4001)]),
+                                          ((5, 3, 333), [(1, 3, 333), (5, 1, 1)]), ((3, 3, 3, 3, 1000), [(3, 1, 3, 1, 1000), (1, 3, 1, 3, 1)])])
+def test_short_odd_first_dim(rk, shape, others):
+    """A dense destination whose dim 0 is short and no whole number of 16-byte vectors (3 x N .+ 1 x N): threads along
+    the linear index, extruded operands gathered; totals that are no multiple of 4 end in a partial vector.  Float32, mixed element types (Float64 and Int32 operands into a
+    Float32 / Float64 destination), an integer program, a deep tree (the interpreter), and five merged dims (lanes
+    along dim 0 again)."""
+    rng = np.random.default_rng(211)
+    L = rk.lazy
+    A = rng.standard_normal(shape).astype(np.float32)
+    u = rng.standard_normal(others[0]).astype(np.float32)
+    v = rng.standard_normal(others[1]).astype(np.float32)
+    dA, du, dv = rk.ROCArray(A), rk.ROCArray(u), rk.ROCArray(v)
+    np.testing.assert_array_equal(rk.Array(rk.materialize(L(dA) + L(du))), A + u)
+    np.testing.assert_array_equal(rk.Array(rk.materialize((L(dA) - L(du)) * L(dv))), (A - u) * v)
+    np.testing.assert_array_equal(rk.Array(rk.materialize(L(du) * L(dv))), (u * v).astype(np.float32) + np.zeros(shape, np.float32))
+    deep = rk.materialize(rk.broadcast.max_(L(dA) * L(du) + L(dv), L(dA) - np.float32(0.25)) * (L(du) + L(dv)) - L(dA) * L(dA))
+    np.testing.assert_array_equal(rk.Array(deep), np.maximum(A * u + v, A - np.float32(0.25)) * (u + v) - A * A)
+    u64 = rng.standard_normal(others[0])
+    np.testing.assert_array_equal(rk.Array(rk.materialize(L(dA) + L(rk.ROCArray(u64)))), A + u64)             # Float64 result
+    iA = rng.integers(-1000, 1000, shape).astype(np.int32)
+    iu = rng.integers(-1000, 1000, others[0]).astype(np.int32)
+    got = rk.Array(rk.materialize(L(rk.ROCArray(iA)) * L(rk.ROCArray(iu)) - L(rk.ROCArray(iA))))
+    assert got.dtype == np.int32 and np.array_equal(got, iA * iu - iA)
+    dest = rk.ROCArray(dims=shape, dtype=np.float32)                                                            # in place: dest is an operand
+    rk.materialize_(dest, L(dA) + np.float32(0))
+    rk.materialize_(dest, L(dest) * L(dv) + L(du))
+    np.testing.assert_array_equal(rk.Array(dest), A * v + u)
