@@ -26,10 +26,11 @@ namespace rk {
 constexpr int PERM_SLAB_MAX_DIMS = 8;
 constexpr int PERM_SLAB_THREADS = 256;
 constexpr int PERM_SLAB_SHORT = 32;        // a leading extent below this counts as short
-constexpr int PERM_SLAB_LONG_CHUNK = 64;   // elements of a long leading dim in a box
+constexpr int PERM_SLAB_LONG_CHUNK = 64;   // elements of a long leading dim in a box ...
+constexpr int PERM_SLAB_LONG_MAX = 256;    // ... and when the third dim is used up and the budget is not
 
 // Elements of LDS the kernel needs for a box budget of `budget` elements (zpitch rounds up to odd: at most TZ more).
-constexpr int perm_slab_lds_elems(int budget) { return budget + PERM_SLAB_LONG_CHUNK; }
+constexpr int perm_slab_lds_elems(int budget) { return budget + PERM_SLAB_LONG_MAX; }
 
 struct PermSlabGeom {
     int nd;                                 // merged dims
@@ -47,8 +48,12 @@ struct PermSlabBox {
 };
 
 // Chooses the box; false when this mapping does not apply (then the tiles do the work).
-inline bool perm_slab_geometry(const int64_t* ext, const int64_t* dstride, int nd, int p, int budget, PermSlabGeom* out) {
-    if (nd < 3 || nd > PERM_SLAB_MAX_DIMS || p == 0) return false;
+inline bool perm_slab_geometry(const int64_t* ext_in, const int64_t* dstride_in, int nd, int p, int budget, PermSlabGeom* out) {
+    if (nd < 2 || nd > PERM_SLAB_MAX_DIMS || p == 0) return false;
+    // a plain transpose with a short side (17 x N <-> N x 17) is the same box with a third dim of extent 1
+    int64_t ext[PERM_SLAB_MAX_DIMS + 1], dstride[PERM_SLAB_MAX_DIMS + 1];
+    for (int d = 0; d < nd; ++d) { ext[d] = ext_in[d]; dstride[d] = dstride_in[d]; }
+    if (nd == 2) { ext[2] = 1; dstride[2] = 0; nd = 3; }
     const int64_t a = ext[0], b = ext[p];
     const bool short_x = a < PERM_SLAB_SHORT, short_z = b < PERM_SLAB_SHORT;
     if (!short_x && !short_z) return false;
@@ -79,6 +84,13 @@ inline bool perm_slab_geometry(const int64_t* ext, const int64_t* dstride, int n
     if (ty < 1) return false;
     if (ty > ext[y]) ty = ext[y];
     g.TY = (int32_t)ty;
+    if (ty == ext[y]) {
+        // the third dim is used up: spend the rest of the budget on the long side
+        int64_t room = budget / ((int64_t)(short_x ? g.TX : g.TZ) * g.TY);
+        if (room > PERM_SLAB_LONG_MAX) room = PERM_SLAB_LONG_MAX;
+        if (!short_x && room > g.TX) g.TX = (int32_t)(room < a ? room : a);
+        if (!short_z && room > g.TZ) g.TZ = (int32_t)(room < b ? room : b);
+    }
     g.zpitch = (g.TX * g.TY) | 1;
     g.tilesx = (a + g.TX - 1) / g.TX;
     g.tilesy = (ext[y] + g.TY - 1) / g.TY;
@@ -146,14 +158,35 @@ struct PermSlabWalk {
     }
 };
 
-// Thread t of the box: copies its share of the source into LDS (source order: x fastest).
+// Thread t of the box: copies its share of the source into LDS (source order: x fastest).  Four elements a round:
+// their loads are issued together (one for 16-byte elements: the compiler keeps a round of those in private memory).
+template <typename T> struct PermSlabRound { static constexpr int N = sizeof(T) >= 16 ? 1 : 4; };
+
 template <typename T>
 RK_HD void perm_slab_load(const PermSlabGeom& g, const PermSlabBox& box, int32_t t, const T* src, T* lds) {
     const int64_t ssy = g.sstride[g.y], ssz = g.sstride[g.p];
     PermSlabWalk w;
     w.start(t, box.nx, box.ny);
-    for (; w.c2 < box.nz; w.next())
-        lds[w.c0 + g.TX * w.c1 + g.zpitch * w.c2] = src[box.sbase + w.c0 + w.c1 * ssy + w.c2 * ssz];
+    while (w.c2 < box.nz) {
+        constexpr int U = PermSlabRound<T>::N;
+        T v[U];
+        int32_t at[U];
+        bool live[U];
+#ifdef __HIPCC__
+#pragma unroll
+#endif
+        for (int u = 0; u < U; ++u) {
+            live[u] = w.c2 < box.nz;
+            at[u] = w.c0 + g.TX * w.c1 + g.zpitch * w.c2;
+            if (live[u]) v[u] = src[box.sbase + w.c0 + w.c1 * ssy + w.c2 * ssz];
+            w.next();
+        }
+#ifdef __HIPCC__
+#pragma unroll
+#endif
+        for (int u = 0; u < U; ++u)
+            if (live[u]) lds[at[u]] = v[u];
+    }
 }
 
 // Thread t of the box: writes its share of LDS to the destination (destination order: z fastest).
@@ -162,8 +195,26 @@ RK_HD void perm_slab_store(const PermSlabGeom& g, const PermSlabBox& box, int32_
     const int64_t dsy = g.dstride[g.y], dsx = g.dstride[0];
     PermSlabWalk w;
     w.start(t, box.nz, box.ny);
-    for (; w.c2 < box.nx; w.next())
-        dst[box.dbase + w.c0 + w.c1 * dsy + w.c2 * dsx] = lds[w.c2 + g.TX * w.c1 + g.zpitch * w.c0];
+    while (w.c2 < box.nx) {
+        constexpr int U = PermSlabRound<T>::N;
+        T v[U];
+        int64_t at[U];
+        bool live[U];
+#ifdef __HIPCC__
+#pragma unroll
+#endif
+        for (int u = 0; u < U; ++u) {
+            live[u] = w.c2 < box.nx;
+            at[u] = box.dbase + w.c0 + w.c1 * dsy + w.c2 * dsx;
+            if (live[u]) v[u] = lds[w.c2 + g.TX * w.c1 + g.zpitch * w.c0];
+            w.next();
+        }
+#ifdef __HIPCC__
+#pragma unroll
+#endif
+        for (int u = 0; u < U; ++u)
+            if (live[u]) dst[at[u]] = v[u];
+    }
 }
 
 }  // namespace rk

@@ -83,7 +83,8 @@ def test_short_contiguous_dims(rk, orc, dtype, shape, perm):
 @pytest.mark.parametrize("dtype", [np.bool_, np.int16, np.float32, np.float64, np.complex128])
 @pytest.mark.parametrize("shape,perm", [((2, 100_001, 2), (3, 2, 1)), ((8, 5000, 8), (3, 2, 1)), ((4, 32, 3001), (3, 2, 1)), ((3001, 32, 4), (3, 2, 1)),
                                         ((17, 33, 65), (3, 2, 1)), ((3, 700, 5, 31), (4, 2, 3, 1)), ((31, 9, 1000), (3, 2, 1)), ((1000, 9, 31), (3, 2, 1)),
-                                        ((5, 40, 6, 300), (3, 4, 2, 1)), ((16, 2, 3, 4, 500), (5, 2, 4, 3, 1)), ((12, 1025, 20), (3, 2, 1)), ((2, 3, 4, 5, 6, 700), (6, 5, 4, 3, 2, 1))])
+                                        ((5, 40, 6, 300), (3, 4, 2, 1)), ((16, 2, 3, 4, 500), (5, 2, 4, 3, 1)), ((12, 1025, 20), (3, 2, 1)), ((2, 3, 4, 5, 6, 700), (6, 5, 4, 3, 2, 1)),
+                                        ((17, 20_001), (2, 1)), ((20_001, 17), (2, 1)), ((31, 5000), (2, 1)), ((9, 70_000), (2, 1)), ((70_000, 9), (2, 1)), ((12, 7, 3000), (3, 1, 2))])
 def test_short_first_dims_with_a_third_dim(rk, orc, dtype, shape, perm):
     """The source's or the destination's first dim is short and neither side is a run of at most 8 elements: boxes of
     three dims through LDS ((2, N, 2) with perm (3, 2, 1): a tile per 4 elements otherwise)."""
