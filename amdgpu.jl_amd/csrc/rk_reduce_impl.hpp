@@ -609,26 +609,36 @@ struct GenericGeom {
     int64_t nout, nred_total;
 };
 
-template <typename In, typename Acc, typename Xf, typename Op, typename Sink, int BLOCK>
+// GROUP lanes share an output: 1 (a handful of elements per output and many outputs: maximum(A; dims=(1, 3)) of a
+// 4 x 1_000_000 x 4 array -- a wave per output would idle 48 lanes and there are a million outputs), 64, or the whole
+// workgroup (few outputs with many elements each: findmax(A; dims=(1, 3)) of a 256^3 array has 256 outputs).
+// I is the type the index of a reduced element is split in: 32-bit division is several times cheaper than 64-bit.
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, int BLOCK, int GROUP, typename I>
 __global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restrict__ A, GenericGeom g, Xf xf, Op op, Sink sink) {
-    const int64_t q = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
-    if (q >= g.nout) return;
+    __shared__ Acc lds[BLOCK / WAVE];
+    const int64_t q = GROUP == BLOCK ? (int64_t)blockIdx.x : ((int64_t)blockIdx.x * BLOCK + threadIdx.x) / GROUP;
+    if (q >= g.nout) return;                 // uniform over the lanes that share an output
     int64_t base = 0, rem = q;
     for (int d = 0; d < g.nkeep; ++d) {
         base += (rem % g.keep_size[d]) * g.keep_stride[d];
         rem /= g.keep_size[d];
     }
     Acc a = Op::template identity<Acc>();
-    for (int64_t k = lane_id(); k < g.nred_total; k += WAVE) {
-        int64_t off = base, r = k;
+    const I total = (I)g.nred_total;
+    for (I k = (I)(threadIdx.x % GROUP); k < total; k += (I)GROUP) {
+        int64_t off = base;
+        I r = k;
         for (int d = 0; d < g.nred; ++d) {
-            off += (r % g.red_size[d]) * g.red_stride[d];
-            r /= g.red_size[d];
+            const I n = (I)g.red_size[d];
+            const I c = d == g.nred - 1 ? r : r % n;
+            off += (int64_t)c * g.red_stride[d];
+            r /= n;
         }
         a = op(a, xf(A[off], (typename Xf::Pos)off));
     }
-    a = wave_reduce(a, op);
-    if (lane_id() == 0) sink(q, a);
+    if constexpr (GROUP == BLOCK) a = block_reduce<BLOCK / WAVE>(a, op, lds);
+    else if constexpr (GROUP == WAVE) a = wave_reduce(a, op);
+    if (threadIdx.x % GROUP == 0) sink(q, a);
 }
 
 // ---- host side: pick a kernel and launch -------------------------------------------------------------
@@ -826,9 +836,18 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
                 }
                 stride *= shape[d];
             }
-            const int64_t blocks = (gg.nout + 3) / 4;
-            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-            reduce_generic_kernel<In, Acc, Xf, Op, Sink, 256><<<(unsigned)blocks, 256, 0, stream>>>(A, gg, xf, op, sink);
+            const bool narrow = gg.nred_total < (1ll << 31);        // element indices fit 32 bits (with the group's stride added)
+#define RK_GENERIC(GROUP, BLOCKS)                                                                                            \
+    do {                                                                                                                     \
+        const int64_t blocks = (BLOCKS);                                                                                     \
+        if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;                                                                    \
+        if (narrow) reduce_generic_kernel<In, Acc, Xf, Op, Sink, 256, GROUP, uint32_t><<<(unsigned)blocks, 256, 0, stream>>>(A, gg, xf, op, sink); \
+        else reduce_generic_kernel<In, Acc, Xf, Op, Sink, 256, GROUP, int64_t><<<(unsigned)blocks, 256, 0, stream>>>(A, gg, xf, op, sink);         \
+    } while (0)
+            if (gg.nred_total <= 64 && gg.nout >= 16384) RK_GENERIC(1, (gg.nout + 255) / 256);
+            else if (gg.nout <= 2048 && gg.nred_total >= 4096) RK_GENERIC(256, gg.nout);
+            else RK_GENERIC(64, (gg.nout + 3) / 4);
+#undef RK_GENERIC
             break;
         }
     }

@@ -406,3 +406,25 @@ def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
     c = rk.count(lambda v: v > 100, dx, dims=dims)
     ax = tuple(d - 1 for d in ((dims,) if isinstance(dims, int) else dims))
     assert np.array_equal(rk.Array(c), (x > 100).sum(axis=ax, keepdims=True))
+
+
+@pytest.mark.parametrize("shape,dims", [((4, 20_000, 4), (1, 3)), ((64, 16, 64), (1, 3)), ((8, 300, 8), (1, 3)), ((3, 5, 7, 2000), (1, 3)),
+                                        ((2, 17_000, 3, 2), (1, 3, 4)), ((100, 3, 100, 5), (1, 3)), ((2, 2, 2, 2, 2, 5000), (1, 3, 5))])
+def test_reduced_dims_that_are_no_single_run(rk, orc, shape, dims):
+    """Reduced dims separated by kept ones (dims=(1, 3)) in the kernel for arbitrary masks: a lane, a wave or a workgroup
+    per output by the number of outputs and of elements each.  findmax / findmin always take it; the reductions take it
+    when the intermediate of a two-step fold would not fit the workspace (the last case below)."""
+    rng = _rng(131)
+    _check_findminmax(rk, orc, rng.integers(-3, 4, shape).astype(np.float32), dims)       # ties: the first index wins
+    _check_findminmax(rk, orc, rng.standard_normal(shape), dims)
+    _check_findminmax(rk, orc, rng.integers(-1000, 1000, shape).astype(np.int32), dims)
+    x = rng.integers(-1000, 1001, shape).astype(np.int64)
+    for op in ("add_sum", "max", "min"):
+        assert np.array_equal(rk.Array(rk.mapreduce("identity", op, rk.ROCArray(x), dims=dims)), orc.mapreduce("identity", op, x, dims=dims))
+
+
+def test_two_step_fold_that_does_not_fit(rk, orc):
+    x = _rng(137).integers(-1000, 1001, (4, 1_400_000, 4)).astype(np.float32)           # either fold leaves 22 MB
+    dx = rk.ROCArray(x)
+    assert np.array_equal(rk.Array(rk.maximum(dx, dims=(1, 3))), x.max(axis=(0, 2), keepdims=True))
+    np.testing.assert_allclose(rk.Array(rk.sum(dx, dims=(1, 3))), x.sum(axis=(0, 2), keepdims=True, dtype=np.float64), rtol=1e-5, atol=1e-2)
