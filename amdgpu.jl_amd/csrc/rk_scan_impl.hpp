@@ -430,7 +430,7 @@ __global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __res
 // cumsum(A; dims=2) of a 4 x 32 x 250_000 array: a lane per line walks 32 rows of 16 bytes.)
 // A slab is the inner x mid block of one outer index, contiguous in memory.  A workgroup copies a 16 KiB run of whole
 // slabs into LDS with 16-byte loads (the host picks the slabs per block so that every block starts at a whole vector),
-// a group of tpl = 1, 2 .. 16 lanes scans each line in place -- lane `part` owns a segment of ceil(m / tpl) elements,
+// a group of tpl = 1, 2 .. 64 lanes scans each line in place -- lane `part` owns a segment of ceil(m / tpl) elements,
 // the segment totals are scanned over the group's lanes by shuffles that never cross a group -- and the tile leaves
 // with 16-byte stores.
 constexpr int SCAN_LDS_LINES_MAX = 128;     // contiguous lines beyond, and whole vectors beyond 64: a wave per line does as well or better
@@ -466,7 +466,9 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
     for (int e = nv * VEC + t; e < ne; e += 256) lds[e] = (T)p[e];           // fewer than VEC elements
     __syncthreads();
     const int tpl = 1 << tpl_log2;
-    const int seg = (m + tpl - 1) >> tpl_log2;
+    // an odd segment length: the lanes of a group start inner * seg elements apart, and an even pitch folds them onto
+    // few banks (2 x 1000 x 16777 Float32 with 64 lanes a line: segments of 16 put 32 lanes on one bank, 234 us; of 17, 51 us)
+    const int seg = ((m + tpl - 1) >> tpl_log2) | 1;
     const int nl = ns * inner;
     const int items = nl << tpl_log2;
     for (int base = 0; base < items; base += 256) {       // uniform trip count: the shuffles below need every lane
@@ -851,7 +853,7 @@ inline int32_t launch_scan(const ScanArgs& a) {
             }
             const int lines = spb * (int)s.inner;
             int tl = 0;
-            while (tl < 4 && (lines << tl) < 256 && (2 << tl) <= s.mid) ++tl;
+            while (tl < 6 && (lines << tl) < 256 && (2 << tl) <= s.mid) ++tl;            // up to a wave per line
             if ((lines << tl) >= 128) {                                       // else too few lanes would scan
                 const int64_t blocks = (s.outer + spb - 1) / spb;
                 if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;

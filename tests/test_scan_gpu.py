@@ -263,7 +263,7 @@ def test_short_contiguous_lines_of_any_length(rk, orc, m):
 
 @pytest.mark.parametrize("shape,dims", [((2, 8, 5000), 2), ((4, 32, 3001), 2), ((4, 100, 1025), 2), ((16, 20, 2000), 2), ((3, 17, 4099), 2),
                                         ((8, 300, 500), 2), ((32, 32, 1000), 2), ((5, 5, 30_001), 2), ((48, 64, 333), 2), ((63, 65, 129), 2),
-                                        ((2, 8, 5, 1000), 2), ((3, 2, 7, 4000), 3), ((64, 16, 300), 2), ((100, 7, 1000), 2), ((7, 2, 100_000), 2)])
+                                        ((2, 8, 5, 1000), 2), ((3, 2, 7, 4000), 3), ((64, 16, 300), 2), ((100, 7, 1000), 2), ((7, 2, 100_000), 2), ((2, 1000, 600), 2), ((3, 333, 400), 2), ((1, 4001, 1), 2)])
 def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
     """A short scanned dim behind a narrow inner extent, many slabs (cumsum(A; dims=2) of a 4 x 32 x N array): whole
     inner x mid slabs staged through LDS."""
