@@ -326,15 +326,21 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
 // lanes of a wave over the banks for every m (with inner = 1 a common start is a 32-way conflict for m = 32; s mod m
 // is one for m = 31).
 // The host picks slabs_per_block so that a block's first element is 16-byte aligned when the array is (VECTOR).
-template <typename In> struct ShortLinesTile { static constexpr int ELEMS = 16384 / sizeof(In); };
+// A traced f (a postfix program) runs while the tile is loaded, and LDS holds its values: Acc-sized slots then.
+template <typename In, typename Acc, typename Xf> struct ShortLinesTile {
+    static constexpr bool MAPPED_IN_LDS = XfIsBatch<Xf>::value && sizeof(Acc) >= sizeof(In) && sizeof(Acc) <= 8;
+    static constexpr int BYTES = 16384;
+    static constexpr int ELEMS = BYTES / (MAPPED_IN_LDS ? sizeof(Acc) : sizeof(In));
+};
 constexpr int SHORT_LINES_MAX = 256;          // contiguous lines beyond this do as well with a wave each
 
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR>
 __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __restrict__ A, int inner, int m, int64_t nslabs, int slabs_per_block,
                                                                  int tpl_log2, int rot_mask, Xf xf, Op op, Sink sink) {
     typedef typename Xf::Pos Pos;
-    constexpr int TE = ShortLinesTile<In>::ELEMS;
-    __shared__ __attribute__((aligned(16))) In lds[TE];
+    typedef ShortLinesTile<In, Acc, Xf> Tile;
+    __shared__ __attribute__((aligned(16))) char lds_raw[Tile::BYTES];
+    In* lds = (In*)lds_raw;
     const int t = threadIdx.x;
     const int slab = inner * m;
     const int64_t slab0 = (int64_t)blockIdx.x * slabs_per_block;
@@ -345,11 +351,48 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
     constexpr int VEC = VECTOR ? 16 / sizeof(In) : 1;
     typedef typename VecOf<In, VEC>::type V;
     const int nv = ne / VEC;
-    for (int i = t; i < nv; i += 256) {
-        if constexpr (VEC == 1) lds[i] = p[i];
-        else ((V*)lds)[i] = load_nt((const V*)p + i);
+    // A traced f (a postfix program) costs scalar control flow per call, whatever the number of values: it runs here,
+    // on two vectors at a time; the fold then reads f's values.
+    constexpr bool MAPPED_IN_LDS = Tile::MAPPED_IN_LDS;
+    if constexpr (MAPPED_IN_LDS) {
+        Acc* mapped = (Acc*)lds_raw;
+        if constexpr (VEC == 1) {
+            for (int i = t; i < ne; i += 256) mapped[i] = xf(p[i], (Pos)0);
+        } else {
+            constexpr int AV = 16 / sizeof(Acc);              // <= VEC
+            typedef typename VecOf<Acc, AV>::type VA;
+            for (int i = t; i < nv; i += 512) {
+                const bool second = i + 256 < nv;
+                const V v0 = load_nt((const V*)p + i);
+                V v1 = v0;
+                if (second) v1 = load_nt((const V*)p + i + 256);
+                In x[2 * VEC];
+                Acc y[2 * VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) { x[j] = v0[j]; x[VEC + j] = v1[j]; }
+                map_batch<2 * VEC>(x, y, xf);
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    if (h == 1 && !second) break;
+                    Acc* to = mapped + (i + h * 256) * VEC;
+#pragma unroll
+                    for (int j0 = 0; j0 < VEC; j0 += AV) {
+                        VA w;
+#pragma unroll
+                        for (int j = 0; j < AV; ++j) w[j] = y[h * VEC + j0 + j];
+                        *(VA*)(to + j0) = w;
+                    }
+                }
+            }
+            for (int e = nv * VEC + t; e < ne; e += 256) mapped[e] = xf(p[e], (Pos)0);
+        }
+    } else {
+        for (int i = t; i < nv; i += 256) {
+            if constexpr (VEC == 1) lds[i] = p[i];
+            else ((V*)lds)[i] = load_nt((const V*)p + i);
+        }
+        for (int e = nv * VEC + t; e < ne; e += 256) lds[e] = p[e];             // fewer than VEC elements
     }
-    for (int e = nv * VEC + t; e < ne; e += 256) lds[e] = p[e];             // fewer than VEC elements
     __syncthreads();
     const int tpl = 1 << tpl_log2;                       // <= 16 and <= m
     const int nl = ns * inner;
@@ -361,11 +404,13 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
         if (l < nl) {
             const int sl = l / inner;
             const In* line = lds + sl * slab + (l - sl * inner);
+            const Acc* mapped_line = (const Acc*)lds_raw + sl * slab + (l - sl * inner);
             const int count = (m - part + tpl - 1) >> tpl_log2;          // elements k = part (mod tpl) of 0 .. m-1
             int k = part + ((sl * (tpl - m)) & rot_mask);                 // < tpl + P <= 2 m
             if (k >= m) k -= m;
             for (int c = 0; c < count; ++c) {
-                acc = op(acc, xf(line[k * inner], (Pos)k));
+                if constexpr (MAPPED_IN_LDS) acc = op(acc, mapped_line[k * inner]);
+                else acc = op(acc, xf(line[k * inner], (Pos)k));
                 k += tpl;
                 if (k >= m) k -= m;
             }
@@ -658,7 +703,8 @@ int tune_reduce_strided_blocks_per_cu();   // rk_api.hip
 int tune_reduce_wave_max_bytes();          // rk_api.hip
 
 template <typename In, typename Acc>
-inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, size_t cap = WS_PARTIALS_BYTES, int grid_scale = 1) {
+inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, size_t cap = WS_PARTIALS_BYTES, int grid_scale = 1,
+                              int short_lines_tile = 16384 / (int)sizeof(In)) {
     ReducePlan p{};
     const int cus = device_info().cus;
     const int64_t target_blocks = (int64_t)cus * tune_reduce_blocks_per_cu() * grid_scale;
@@ -667,10 +713,10 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
     const int64_t nlines = s.inner * s.outer;
     const int64_t slab = s.inner * s.mid;
     // (rows of 64 elements or more that are whole vectors stream as well through the strided kernel)
-    if (s.mid >= 2 && nlines >= 1024 && slab <= ShortLinesTile<In>::ELEMS && (s.inner > 1 || s.mid <= SHORT_LINES_MAX) &&
+    if (s.mid >= 2 && nlines >= 1024 && slab <= short_lines_tile && (s.inner > 1 || s.mid <= SHORT_LINES_MAX) &&
         (s.inner < 64 || s.inner % VEC != 0 || !is_aligned(A, 16))) {
         // whole slabs per block, and (for the vector loads) a block size in bytes that is a multiple of 16
-        int spb = ShortLinesTile<In>::ELEMS / (int)slab;
+        int spb = short_lines_tile / (int)slab;
         bool vector = is_aligned(A, 16);
         if (vector) {
             int q = 16;                                                      // 16 / gcd(slab bytes, 16)
@@ -769,7 +815,7 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
     // (2^26 Float32, x -> x + 1: 3.4 -> 5.2 TB/s with twice the workgroups; 9 tokens: 2.3 -> 2.6 TB/s with four times)
     int grid_scale = 1;
     if constexpr (XfIsBatch<Xf>::value) grid_scale = xf.n_tokens > 4 ? 4 : 2;
-    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap, grid_scale);
+    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap, grid_scale, ShortLinesTile<In, Acc, Xf>::ELEMS);
     Workspace w{};
     if (p.payload > cap) return RK_ERR_WORKSPACE;   // the planner never asks for more
     if (p.payload > 0 && !carve_workspace(ws, ws_bytes, 0, &w)) return RK_ERR_WORKSPACE;
