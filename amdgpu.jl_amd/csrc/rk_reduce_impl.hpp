@@ -670,16 +670,30 @@ __global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restr
     }
     Acc a = Op::template identity<Acc>();
     const I total = (I)g.nred_total;
-    for (I k = (I)(threadIdx.x % GROUP); k < total; k += (I)GROUP) {
-        int64_t off = base;
-        I r = k;
-        for (int d = 0; d < g.nred; ++d) {
-            const I n = (I)g.red_size[d];
-            const I c = d == g.nred - 1 ? r : r % n;
-            off += (int64_t)c * g.red_stride[d];
-            r /= n;
+    // NU elements a round, their loads issued together (few outputs mean few waves: 256 workgroups for findmax(A; dims=(1, 3))
+    // of a 256^3 array, and one load in flight per lane leaves the memory system idle)
+    constexpr int NU = GROUP == 1 ? 1 : 4;
+    for (I k = (I)(threadIdx.x % GROUP); k < total; k += (I)(NU * GROUP)) {       // total < 2^31 when I has 32 bits: no wrap
+        int64_t off[NU];
+        In v[NU];
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            I r = k + (I)(u * GROUP);
+            off[u] = -1;
+            if (r < total) {
+                off[u] = base;
+                for (int d = 0; d < g.nred; ++d) {
+                    const I n = (I)g.red_size[d];
+                    const I c = d == g.nred - 1 ? r : r % n;
+                    off[u] += (int64_t)c * g.red_stride[d];
+                    r /= n;
+                }
+                v[u] = A[off[u]];
+            }
         }
-        a = op(a, xf(A[off], (typename Xf::Pos)off));
+#pragma unroll
+        for (int u = 0; u < NU; ++u)
+            if (off[u] >= 0) a = op(a, xf(v[u], (typename Xf::Pos)off[u]));
     }
     if constexpr (GROUP == BLOCK) a = block_reduce<BLOCK / WAVE>(a, op, lds);
     else if constexpr (GROUP == WAVE) a = wave_reduce(a, op);
