@@ -269,6 +269,41 @@ def main():
         run_cfg("reverse(A; dims=1) 8192^2 Float32", d * d, 8 * d * d, run_reverse)
         run_cfg("permutedims(A, (2,1)) 8192^2 Float32", d * d, 8 * d * d, run_permute)
         del ra, rb
+        # short and narrow extents (arrays of small structures: 3 x N, 4 x 32 x N), 2^25 elements, 3 rotating buffers
+        n25 = 1 << 25
+        def three(shape):
+            return [dev_array(randn_f32(int(np.prod(shape))), shape, np.float32) for _ in range(3)]
+        sa = three((32, n25 // 32))
+        sr = rk.ROCArray(dims=(1, n25 // 32), dtype=np.float32)
+        ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
+        run_cfg("sum(A; dims=1) 32x1048576 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3]())
+        del sa, sr, ps
+        sa = three((4, 32, n25 // 128))
+        sr = rk.ROCArray(dims=(4, 1, n25 // 128), dtype=np.float32)
+        ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
+        run_cfg("sum(A; dims=2) 4x32x262144 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3]())
+        del sa, sr, ps
+        n15 = n25 // 15
+        sa = three((15, n15))
+        so = [rk.ROCArray(dims=(15, n15), dtype=np.float32) for _ in range(3)]
+        ps = [plan_accumulate("add", o, x, dims=1) for o, x in zip(so, sa)]
+        run_cfg(f"cumsum(A; dims=1) 15x{n15} Float32", 15 * n15, 8 * 15 * n15, lambda i: ps[i % 3]())
+        del sa, so, ps
+        n3 = n25 // 3
+        sa = three((3, n3))
+        sv = dev_array(randn_f32(n3), (1, n3), np.float32)
+        so = [rk.ROCArray(dims=(3, n3), dtype=np.float32) for _ in range(3)]
+        ps = [plan_materialize(o, L(x) + L(sv)) for o, x in zip(so, sa)]
+        run_cfg(f"C .= A .+ r 3x{n3} .+ 1x{n3} Float32", 3 * n3, 8 * 3 * n3 + 4 * n3, lambda i: ps[i % 3]())
+        del sa, sv, so, ps
+        sa = three((2, n25 // 4, 2))
+        so = [rk.ROCArray(dims=(2, n25 // 4, 2), dtype=np.float32) for _ in range(3)]
+        shp3 = RL.shape_array((2, n25 // 4, 2))
+        perm321 = (C.c_int32 * 3)(3, 2, 1)
+        def run_permute3(i):
+            RL.check(RL.lib.rk_permutedims(sa[i % 3].ptr, so[i % 3].ptr, 4, 3, shp3, perm321, stream_ptr()), "rk_permutedims")
+        run_cfg("permutedims(A, (3,2,1)) 2x8388608x2 Float32", n25, 8 * n25, run_permute3)
+        del sa, so
         # sort! (src/kernels/sorting.jl:1; perf/array.jl:143-149 sorts a Float32 vector): 8 B/key is the floor of
         # any out-of-place permutation (one read, one write); the radix sort makes 4 digit passes plus 3 reads
         m = 1 << 26
