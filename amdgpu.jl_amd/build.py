@@ -1,6 +1,6 @@
 """Builds librk.so (gfx950 only) in-tree with hipcc.
 
-    python amdgpu.jl_amd/build.py [-j N]
+    python amdgpu.jl_amd/build.py [-j N] [--incremental]
 
 The element-type instantiations are separate objects (one source compiled with -DRK_INST=n) so they
 build in parallel.  hipcc cross-compiles: no GPU is needed to build.
@@ -85,18 +85,41 @@ def _compile(unit):
     return obj, err, [f"{src}{suffix}: {p}" for p in private]
 
 
-def build(jobs: int | None = None, verbose: bool = True) -> str:
+def _stale(unit) -> bool:
+    """True when the unit's object is older than its source or any header of the library."""
+    src, suffix, _ = unit
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [os.path.join(CSRC, src), os.path.join(HERE, "..", "include", "rk.h")]
+    text = open(os.path.join(CSRC, src)).read()
+    seen, todo = set(), re.findall(r'#include "([^"]+)"', text)
+    while todo:                                   # headers of csrc/, transitively
+        h = os.path.basename(todo.pop())
+        if h in seen or not os.path.exists(os.path.join(CSRC, h)):
+            continue
+        seen.add(h)
+        deps.append(os.path.join(CSRC, h))
+        todo += re.findall(r'#include "([^"]+)"', open(os.path.join(CSRC, h)).read())
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(jobs: int | None = None, verbose: bool = True, incremental: bool = False) -> str:
+    """Compile and link.  ``incremental`` recompiles only the units whose sources changed (a developer's
+    shortcut; the private-memory check then covers only those units)."""
     os.makedirs(OBJ, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
+    units = [u for u in UNITS if _stale(u)] if incremental else list(UNITS)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        results = list(pool.map(_compile, UNITS))
+        results = list(pool.map(_compile, units))
     for obj, err, _ in results:
         if err.strip() and verbose:
             print(err, file=sys.stderr)
     private = [p for _, _, ps in results for p in ps]
     if private:
         raise RuntimeError("kernels using private memory:\n  " + "\n  ".join(private))
-    objs = [o for o, _, _ in results]
+    objs = [os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o") for src, suffix, _ in UNITS]
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -110,4 +133,4 @@ if __name__ == "__main__":
     j = None
     if "-j" in sys.argv:
         j = int(sys.argv[sys.argv.index("-j") + 1])
-    build(j)
+    build(j, incremental="--incremental" in sys.argv)
