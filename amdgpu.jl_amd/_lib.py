@@ -30,6 +30,7 @@ RK_ERR_UNSUPPORTED = 10002
 RK_ERR_WORKSPACE = 10003
 RK_ERR_DIMENSION = 10004
 RK_ERR_TOO_LARGE = 10005
+RK_STATIC_SCRATCH_BYTES = 16 << 20
 
 # rk_dtype
 RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16 = range(9)
@@ -98,6 +99,8 @@ PROTOTYPES = {
                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_accumulate": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,
                                   C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_accumulate_static": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,
+                                         C.c_int32, C.c_void_p, C.c_void_p]),
     "rk_broadcast": (C.c_int32, [C.POINTER(RkProgram), C.c_void_p, C.c_int, C.c_int, _I64P, C.c_void_p]),
     "rk_broadcast_strided": (C.c_int32, [C.POINTER(RkProgram), C.c_void_p, C.c_int, C.c_int, _I64P, _I64P, C.c_void_p]),
     "rk_volumerhs_f32": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64,

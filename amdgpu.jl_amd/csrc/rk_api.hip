@@ -1,6 +1,7 @@
 // C ABI entry points of librk.so: argument validation (runs without a GPU), dispatch on the
 // element types, workspace management.  The kernels live in rk_*_impl.hpp / rk_*.hip.
 #include <atomic>
+#include <mutex>
 #include <cstdlib>
 #include <cstddef>
 #include <cstring>
@@ -97,6 +98,57 @@ static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {
 
 size_t findall_workspace_need(int64_t n);   // rk_select.hip
 
+// Prepares a workspace: header, tickets and descriptors to zero (tag 0 = never valid), the scan epoch to
+// WS_EPOCH_FIRST.  A kernel, not hipMemsetAsync: memset nodes recorded into a captured graph have replayed
+// wrongly on this platform, and a fill kernel is safe either way.  64-bit words (what the descriptors are);
+// word 0 is the header's scan_counter = epoch << 32.
+__global__ __launch_bounds__(256) void workspace_init_kernel(uint64_t* ws, size_t head_words, size_t desc_word0, size_t total_words) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total_words; i += stride) {
+        if (i >= head_words && i < desc_word0) continue;          // partials: never read before written
+        ws[i] = i == 0 ? (uint64_t)WS_EPOCH_FIRST << 32 : 0ull;
+    }
+}
+
+static int32_t workspace_init(void* ws, size_t ws_bytes, hipStream_t stream) {
+    static_assert(offsetof(WsHeader, scan_counter) == 0 && WS_PARTIALS_OFFSET % 8 == 0 && WS_DESC_OFFSET % 8 == 0, "layout in 64-bit words");
+    workspace_init_kernel<<<1024, 256, 0, stream>>>((uint64_t*)ws, WS_PARTIALS_OFFSET / 8, WS_DESC_OFFSET / 8, ws_bytes / 8);
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+}  // namespace rk
+
+// ---- bookkeeping of rk_accumulate_static ---------------------------------------------------------------------
+// One array per GPU inside the library image.  In host code its name is only a handle for hipGetSymbolAddress;
+// the device address obtained there (per device: each GPU holds its own copy) is what kernels and fills receive.
+static __device__ __align__(256) unsigned char scratch[RK_STATIC_SCRATCH_BYTES];
+
+namespace rk {
+constexpr int STATIC_MAX_DEVICES = 64;
+static std::mutex g_static_mutex;
+static void* g_static_ptr[STATIC_MAX_DEVICES];      // device address of `scratch` on each device, null until prepared
+
+// Device address of the current device's scratch array, prepared (on `stream`) at the first call on that device.
+static int32_t static_scratch(hipStream_t stream, void** out) {
+    int dev = 0;
+    RK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return RK_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (g_static_ptr[dev] == nullptr) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        RK_HIP(hipStreamIsCapturing(stream, &cap));
+        if (cap != hipStreamCaptureStatusNone) return RK_ERR_WORKSPACE;   // a captured preparation would replay with every graph launch
+        void* ptr = nullptr;
+        RK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr || !is_aligned(ptr, 256)) return RK_ERR_WORKSPACE;
+        const int32_t st = workspace_init(ptr, RK_STATIC_SCRATCH_BYTES, stream);
+        if (st != RK_SUCCESS) return st;
+        g_static_ptr[dev] = ptr;
+    }
+    *out = g_static_ptr[dev];
+    return RK_SUCCESS;
+}
 }  // namespace rk
 
 using namespace rk;
@@ -137,14 +189,7 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
 int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
     if (ws == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (!is_aligned(ws, 256) || ws_bytes < WS_DESC_OFFSET) return RK_ERR_WORKSPACE;
-    // header + tickets to zero, descriptors to zero (tag 0 = never valid), then the scan epoch = 1:
-    // scan_counter = 1 << 32, i.e. byte 4 of the header (little endian)
-    RK_HIP(hipMemsetAsync(ws, 0, WS_PARTIALS_OFFSET, (hipStream_t)stream));
-    if (ws_bytes > WS_DESC_OFFSET)
-        RK_HIP(hipMemsetAsync((char*)ws + WS_DESC_OFFSET, 0, ws_bytes - WS_DESC_OFFSET, (hipStream_t)stream));
-    static_assert(WS_EPOCH_FIRST == 1 && offsetof(WsHeader, scan_counter) == 0, "the byte-wise memset below writes epoch 1");
-    RK_HIP(hipMemsetAsync((char*)ws + 4, 1, 1, (hipStream_t)stream));
-    return RK_SUCCESS;
+    return workspace_init(ws, ws_bytes, (hipStream_t)stream);
 }
 
 int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
@@ -255,6 +300,21 @@ int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, v
     if (in == RK_U8 && out == RK_I64) return scan_u8_i64(a);
     if (in == RK_U8 && out == RK_I32) return scan_u8_i32(a);
     return RK_ERR_UNSUPPORTED;
+}
+
+int32_t rk_accumulate_static(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, void* out_ptr, int ndim, const int64_t* shape,
+                             int dim, int32_t inclusive, const void* init, void* stream) {
+    // size check first: it needs no device, and a request that cannot be served must not prepare anything
+    int64_t total = 0;
+    if (!valid_dtype(in) || !valid_dtype(out) || !valid_shape(ndim, shape, &total) || dim < 1) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    const uint32_t mask = dim <= ndim ? (1u << (dim - 1)) : 0u;
+    if (rk_workspace_bytes(RK_KIND_ACCUMULATE, out, ndim, shape, mask) > RK_STATIC_SCRATCH_BYTES) return RK_ERR_TOO_LARGE;
+    if (in_ptr == nullptr || out_ptr == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    void* ws = nullptr;
+    const int32_t st = static_scratch((hipStream_t)stream, &ws);
+    if (st != RK_SUCCESS) return st;
+    return rk_accumulate(op, in, out, in_ptr, out_ptr, ndim, shape, dim, inclusive, init, ws, RK_STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

@@ -177,6 +177,24 @@ RK_API int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out,
                       const void* init,
                       void* ws, size_t ws_bytes, void* stream);
 
+/* ---- accumulate without a caller workspace ------------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory at all --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc -- and so
+ * cannot bring the workspace rk_accumulate asks for: the same scan, with its bookkeeping
+ * (tile counter, look-back descriptors, slice totals) in a device array of
+ * RK_STATIC_SCRATCH_BYTES that is part of the library image, one copy per GPU, held until the
+ * process ends.  Arguments and results as rk_accumulate.  Calls whose bookkeeping would not fit
+ * (rk_workspace_bytes(RK_KIND_ACCUMULATE, ...) > RK_STATIC_SCRATCH_BYTES) return
+ * RK_ERR_TOO_LARGE.  Calls no hipMalloc / hipFree.  Every call on a GPU uses that GPU's one
+ * array: calls that overlap in time on one GPU (two streams, two threads) race and must be
+ * ordered by the caller.  The first call on each device prepares the array with a small kernel
+ * on `stream`; it must not be made while that stream is being captured (RK_ERR_WORKSPACE). */
+#define RK_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+RK_API int32_t rk_accumulate_static(rk_op op, rk_dtype in, rk_dtype out,
+                             const void* in_ptr, void* out_ptr,
+                             int ndim, const int64_t* shape, int dim, int32_t inclusive,
+                             const void* init, void* stream);
+
 /* ---- fused broadcast ---------------------------------------------------------------
  * Replaces copyto!(dest, ::Broadcasted{<:ROCArrayStyle})              src/broadcast.jl:3-35
  * i.e. GPUArrays' broadcast kernel launched through the KernelAbstractions functor
