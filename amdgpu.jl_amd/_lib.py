@@ -30,6 +30,7 @@ RK_ERR_UNSUPPORTED = 10002
 RK_ERR_WORKSPACE = 10003
 RK_ERR_DIMENSION = 10004
 RK_ERR_TOO_LARGE = 10005
+RK_ERR_WAIT = 10006
 RK_STATIC_SCRATCH_BYTES = 16 << 20
 
 # rk_dtype
@@ -91,6 +92,9 @@ PROTOTYPES = {
     "rk_status_string": (C.c_char_p, [C.c_int32]),
     "rk_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, _I64P, C.c_uint32]),
     "rk_workspace_init": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_set_wait_budget": (C.c_int64, [C.c_int64]),
+    "rk_workspace_status": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_sort_status": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce_program": (C.c_int32, [C.POINTER(RkMapProgram), C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,

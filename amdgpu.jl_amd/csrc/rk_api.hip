@@ -74,10 +74,32 @@ int tune_scan_waves() {
     return (v == 4 || v == 8 || v == 16) ? v : 0;
 }
 
+// 1: the single-pass scan takes its tile ids from a device-wide counter (forward progress whatever the order in which
+// workgroups start) instead of from the launch order (RK_SCAN_DYNAMIC_IDS).
+int tune_scan_dynamic_ids() {
+    static const int v = env_int("RK_SCAN_DYNAMIC_IDS", 0, 0, 1);
+    return v;
+}
+
 // Workgroups per compute unit the scan across rows aims for when it cuts the rows into slices
 // (RK_SCAN_SLICE_BLOCKS_PER_CU).
 int tune_scan_slice_blocks_per_cu() {
     static const int v = env_int("RK_SCAN_SLICE_BLOCKS_PER_CU", 32, 1, 256);
+    return v;
+}
+
+// Unsuccessful poll rounds one bounded wait may spend before it gives up (RK_WAIT_BUDGET, rk_set_wait_budget).
+// A round is one device-coherent load plus the back-off, about a microsecond; correct calls resolve in tens of rounds.
+constexpr long long WAIT_BUDGET_DEFAULT = 1ll << 21;
+static std::atomic<long long> g_wait_budget{0};
+long long wait_budget() {
+    long long v = g_wait_budget.load(std::memory_order_relaxed);
+    if (v <= 0) {
+        const char* s = std::getenv("RK_WAIT_BUDGET");
+        v = (s && *s) ? std::strtoll(s, nullptr, 10) : 0;
+        if (v <= 0) v = WAIT_BUDGET_DEFAULT;
+        g_wait_budget.store(v, std::memory_order_relaxed);
+    }
     return v;
 }
 
@@ -165,6 +187,8 @@ const char* rk_status_string(int32_t status) {
         case RK_ERR_WORKSPACE: return "RK_ERR_WORKSPACE: workspace missing, not 256-byte aligned or too small";
         case RK_ERR_DIMENSION: return "RK_ERR_DIMENSION: array extents do not agree";
         case RK_ERR_TOO_LARGE: return "RK_ERR_TOO_LARGE: an extent exceeds what the kernels can index";
+        case RK_ERR_WAIT: return "RK_ERR_WAIT: a kernel gave up waiting for another workgroup (workspace not prepared, or shared by "
+                                 "concurrent calls); the results of calls on it since the last check are invalid, prepare it again";
         default: break;
     }
     if (status > 0 && status < 10000) return hipGetErrorString((hipError_t)status);
@@ -180,7 +204,8 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
         const size_t esz = dtype_size(dt) < 4 ? 4 : dtype_size(dt);
         const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 8;           // ScanTile<T>::TILE
         const int64_t tpl = (s.mid + tile - 1) / tile, gpl = (tpl + WAVE - 1) / WAVE;
-        if (s.inner == 1 && tpl > 1) need += (size_t)((tpl + gpl) * s.outer) * (esz / 4) * sizeof(uint64_t);
+        // one tagged word per 4 bytes of the value per tile, one 128-byte line per group of 64 tiles
+        if (s.inner == 1 && tpl > 1) need += ((size_t)(tpl * s.outer) * (esz / 4) + (size_t)(gpl * s.outer) * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     }
     if (kind == RK_KIND_FINDALL && valid_shape(ndim, shape, &total) && total > 0) need += findall_workspace_need(total);
     return (need + 255) & ~(size_t)255;
@@ -190,6 +215,21 @@ int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream) {
     if (ws == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (!is_aligned(ws, 256) || ws_bytes < WS_DESC_OFFSET) return RK_ERR_WORKSPACE;
     return workspace_init(ws, ws_bytes, (hipStream_t)stream);
+}
+
+int64_t rk_set_wait_budget(int64_t rounds) {
+    const long long prev = wait_budget();
+    g_wait_budget.store(rounds > 0 ? (long long)rounds : WAIT_BUDGET_DEFAULT, std::memory_order_relaxed);
+    return (int64_t)prev;
+}
+
+int32_t rk_workspace_status(const void* ws, size_t ws_bytes, void* stream) {
+    if (ws == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (!is_aligned(ws, 256) || ws_bytes < WS_DESC_OFFSET) return RK_ERR_WORKSPACE;
+    uint32_t failed = 0;
+    RK_HIP(hipMemcpyAsync(&failed, (const char*)ws + offsetof(WsHeader, wait_failed), sizeof(failed), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    RK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return failed != 0u ? RK_ERR_WAIT : RK_SUCCESS;
 }
 
 int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,

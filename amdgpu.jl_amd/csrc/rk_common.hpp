@@ -54,7 +54,8 @@ const DeviceInfo& device_info();   // rk_api.hip
 //                                from the partials so arbitrary partial bits never look like a tag)
 struct WsHeader {
     uint64_t scan_counter;  // look-back scan: epoch << 32 | tile acquisitions of the running call
-    uint32_t pad[62];
+    uint32_t wait_failed;   // set by a kernel that gave up a bounded wait (see WaitCtl); read by rk_workspace_status
+    uint32_t pad[61];
 };
 static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
 
@@ -279,9 +280,41 @@ template <typename T> __device__ __forceinline__ T load_agent(const T* p) {
     return v;
 }
 // All earlier stores of this thread have completed (s_waitcnt vmcnt(0)) before anything later issues.
+// ASSUMPTION beyond the HIP memory model: the model orders a relaxed store before a later relaxed atomic of the same
+// thread only through a release at the scope of the reader (agent), which here would write back the L2.  What this
+// relies on instead is how gfx950 executes the two: agent-scope atomic stores bypass the non-coherent caches and are
+// performed at the device-coherent level, and vmcnt counts a store as done only when that level has acknowledged it,
+// so a ticket or flag issued after the wait cannot be observed before the value.  The workgroup-scope fence only
+// keeps the compiler from moving memory operations across this point.  True on gfx942 / gfx950; to be re-checked
+// on any other target.
 __device__ __forceinline__ void publish_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
+}
+
+// ---- bounded waits ------------------------------------------------------------------------------------------
+// Every loop that polls memory written by another workgroup (look-back of the scans, of the select and of the
+// sort) counts its unsuccessful rounds.  When one wait has used `budget` rounds -- which only happens when the
+// state it polls is not what the protocol expects: a workspace that was never prepared, or one shared by calls
+// that run at the same time -- it sets the word `failed`, stops waiting and carries on with a meaningless value,
+// so that every workgroup still runs to its end and the kernel exits normally.  All waiters look at `failed`
+// every few rounds and give up with the first one.  The results of such a call are wrong; the host learns of it
+// through rk_workspace_status / rk_sort_status and has to prepare the workspace again.
+struct WaitCtl {
+    uint32_t* failed;
+    long long budget;       // unsuccessful poll rounds one wait may spend (a round is a device-coherent load: ~1 us)
+    int       backoff;      // s_sleep units between rounds
+};
+// Called once per unsuccessful round by (at least) one full wave; true = stop waiting.
+__device__ __forceinline__ bool wait_give_up(const WaitCtl& w, long long& rounds) {
+    ++rounds;
+    if (rounds >= w.budget) {
+        __hip_atomic_store(w.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return true;
+    }
+    if ((rounds & 31) == 0 && __hip_atomic_load(w.failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return true;
+    for (int b = 0; b < w.backoff; ++b) __builtin_amdgcn_s_sleep(8);
+    return false;
 }
 
 // Reduction over a workgroup of NW waves.  Every thread returns the total.  `lds` must

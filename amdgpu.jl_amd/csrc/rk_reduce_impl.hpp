@@ -505,19 +505,22 @@ __global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict
 }
 
 // ---- inner >= 64: lanes along `inner` -------------------------------------------------------------
-// grid (strips, msplits, outer); workgroup = 4 waves; a wave owns 64 * VEC adjacent columns of a
-// strip and every 4th row of the row batches dealt to its workgroup.
+// grid (strips * outer, msplits): the outer index shares the x axis with the strips (the y and z axes of a grid end
+// at 65535, and a 64 x 2 x 70000 array has that many outer indices and more); workgroup = 4 waves; a wave owns
+// 64 * VEC adjacent columns of a strip and every 4th row of the row batches dealt to its workgroup.
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int UNROLL>
 __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
-                                                             Acc* partials, uint32_t* tickets) {
+                                                             Acc* partials, uint32_t* tickets, int strips) {
     constexpr int VEC = VECTOR ? 16 / sizeof(In) : 1;
     constexpr int COLS = WAVE * VEC;   // columns per strip
     constexpr int NW = 4;
     typedef typename VecOf<In, VEC>::type V;
     __shared__ Acc lds[NW][COLS];
     __shared__ int is_last;
-    const int strip = blockIdx.x, ms = blockIdx.y, msplits = gridDim.y;
-    const int64_t o = blockIdx.z;
+    const int ms = blockIdx.y, msplits = gridDim.y;
+    const int64_t tile = blockIdx.x;                    // o * strips + strip
+    const int64_t o = tile / strips;
+    const int strip = (int)(tile - o * strips);
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int64_t col0 = (int64_t)strip * COLS + (int64_t)lane * VEC;
     const bool live = col0 < g.inner;      // inner % VEC == 0 on the vector path
@@ -596,7 +599,6 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         return;
     }
     // partials[(o * strips + strip) * msplits + ms][COLS]
-    const int64_t tile = o * gridDim.x + strip;
     if (t < COLS) {
         store_agent(&partials[(tile * msplits + ms) * COLS + t], r);
         publish_barrier();
@@ -872,12 +874,13 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
             break;
         }
         case ReducePlan::STRIDED: {
-            if (s.outer > 65535) return RK_ERR_TOO_LARGE;
-            dim3 grid(p.strips, p.splits, (unsigned)s.outer);
+            const int64_t tiles = (int64_t)p.strips * s.outer;
+            if (tiles > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            dim3 grid((unsigned)tiles, p.splits);
             if (p.vector)
-                reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips);
             else
-                reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets);
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips);
             break;
         }
         case ReducePlan::NARROW: {

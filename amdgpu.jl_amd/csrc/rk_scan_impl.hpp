@@ -69,7 +69,8 @@ __device__ __forceinline__ uint32_t desc_read(const uint64_t* desc, int64_t stri
 //   agg  aggregate of this tile (already published by the caller as the tile's descriptor)
 template <typename T, typename Op>
 __device__ __forceinline__ T desc_lookback2(uint64_t* tile_desc, int64_t tstride, uint64_t* group_desc, int64_t gstride,
-                                            int64_t tile, int64_t tl, int64_t gl, uint32_t epoch, T agg, T init, Op op, T ident, int backoff) {
+                                            int64_t tile, int64_t tl, int64_t gl, uint32_t epoch, T agg, T init, Op op, T ident,
+                                            const WaitCtl& wc) {
     const int lane = lane_id();
     const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
     const int r = (int)(tl & (WAVE - 1));           // predecessors inside the group
@@ -78,6 +79,7 @@ __device__ __forceinline__ T desc_lookback2(uint64_t* tile_desc, int64_t tstride
     T local = ident, gacc = ident, gpre = init;
     bool local_done = (r == 0), group_done = (g == 0), ga_published = false;
     int64_t gfirst = gl - 1, grem = g;              // nearest group of the current window, groups left
+    long long rounds = 0;
     while (!(local_done && group_done)) {
         Words<T> tv = to_words(ident), gv = to_words(ident);
         uint32_t tstat = DESC_A, gstat = DESC_P;    // lanes outside the range: terminators holding ident
@@ -109,12 +111,116 @@ __device__ __forceinline__ T desc_lookback2(uint64_t* tile_desc, int64_t tstride
                 }
             }
         }
-        if (!(local_done && group_done))
-            for (int b = 0; b < backoff; ++b) __builtin_amdgcn_s_sleep(8);
+        if (!(local_done && group_done) && wait_give_up(wc, rounds)) break;     // the prefix below is then meaningless
     }
     const T prefix = op(gpre, local);
     if (r == WAVE - 1 && lane == 0) desc_publish(group_desc, gstride, gl, op(prefix, agg), tagP);
     return prefix;
+}
+
+// ---- look-back with group leaders ------------------------------------------------------------------------------
+// In desc_lookback2 every waiting tile polls the descriptors of the nearest groups, so the one or two 128-byte lines
+// that hold them are read by every tile in flight, round after round.  Device-coherent accesses to one line are
+// served one at a time (some 10 ns each on MI355X): with thousands of tiles in flight that line, not HBM, sets the
+// pace -- measured as 7 ns per tile whatever the tile size, occupancy or polling discipline.  Here only the FIRST
+// tile of a group of 64 (its leader) looks at the group level: it sums group aggregates back to the nearest inclusive
+// prefix and publishes the result -- the inclusive prefix through the previous group -- into that group's descriptor;
+// the other 63 tiles sum the aggregates of their predecessors inside the group and wait for that one word.  Every
+// group descriptor has a 128-byte line of its own (word i of group g at g * GROUP_DESC_STRIDE + i), so its readers are
+// the 63 tiles of the next group and the few leaders in flight.  Per tile the cost falls to ~1.5 ns.
+//   tile descriptors   [words][ntiles], DESC_A only           group descriptors   DESC_A: aggregate of the group
+//                                                                                 DESC_P: inclusive prefix through it
+constexpr int GROUP_DESC_STRIDE = 16;      // 64-bit words: one 128-byte line per group
+
+template <typename T>
+__device__ __forceinline__ void gdesc_publish(uint64_t* gd, int64_t g, T value, uint32_t tag) {
+    Words<T> w = to_words(value);
+    static_assert(Words<T>::N <= GROUP_DESC_STRIDE, "a value fits the line of its group");
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i)
+        __hip_atomic_store(&gd[g * GROUP_DESC_STRIDE + i], ((uint64_t)tag << 32) | (uint64_t)w.w[i], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ uint32_t gdesc_read(const uint64_t* gd, int64_t g, uint32_t tagA, uint32_t tagP, Words<T>& val) {
+    uint32_t status = 0;
+#pragma unroll
+    for (int i = 0; i < Words<T>::N; ++i) {
+        const uint64_t d = __hip_atomic_load(&gd[g * GROUP_DESC_STRIDE + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t tag = (uint32_t)(d >> 32);
+        val.w[i] = (uint32_t)d;
+        const uint32_t st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
+        status = (i == 0) ? st : (st == status ? st : 0u);
+    }
+    return status;
+}
+
+// Executed by one full wave; returns the wave-uniform exclusive prefix of `tile` (tl > 0) inside its line.
+//   tl  index of the tile in its line     gl  global index of the tile's group     agg  aggregate of this tile
+template <typename T, typename Op>
+__device__ __forceinline__ T desc_lookback_leader(uint64_t* tile_desc, int64_t tstride, uint64_t* gd, int64_t tile, int64_t tl, int64_t gl,
+                                                  uint32_t epoch, T agg, T init, Op op, T ident, const WaitCtl& wc) {
+    const int lane = lane_id();
+    const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
+    const int r = (int)(tl & (WAVE - 1));           // predecessors inside the group
+    const int64_t g = tl >> 6;                      // groups in front of this one in the line
+    long long rounds = 0;
+    if (r == 0) {
+        // leader (g > 0, since tl > 0): aggregates of the groups in front, back to the nearest inclusive prefix
+        T gacc = ident, base = init;
+        int64_t gfirst = gl - 1, grem = g;
+        for (;;) {
+            Words<T> gv = to_words(ident);
+            uint32_t gstat = DESC_P;                // lanes beyond the line start: terminators holding ident
+            if (lane < grem) gstat = gdesc_read<T>(gd, gfirst - lane, tagA, tagP, gv);
+            const uint64_t ballotP = __ballot(gstat == DESC_P);
+            const uint64_t ballotX = __ballot(gstat == 0u);
+            const int np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
+            const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
+            if ((ballotX & needed) == 0ull) {
+                const T x = (np < 0 || lane <= np) ? from_words<T>(gv) : ident;
+                gacc = op(wave_reduce(x, op), gacc);
+                if (np >= 0) {
+                    base = (np >= grem) ? op(init, gacc) : gacc;     // a real prefix already contains init
+                    break;
+                }
+                gfirst -= WAVE;
+                grem -= WAVE;
+                continue;
+            }
+            if (wait_give_up(wc, rounds)) break;     // `base` is then meaningless
+        }
+        if (lane == 0) gdesc_publish(gd, gl - 1, base, tagP);
+        return base;
+    }
+    const int64_t t0 = tile - r;
+    T local = ident;
+    for (;;) {
+        Words<T> tv = to_words(ident);
+        uint32_t tstat = DESC_A;
+        if (lane < r) tstat = desc_read<T>(tile_desc, tstride, t0 + lane, tagA, tagP, tv);
+        if (__ballot(tstat == 0u) == 0ull) {
+            local = wave_reduce(from_words<T>(tv), op);
+            break;
+        }
+        if (wait_give_up(wc, rounds)) break;
+    }
+    if (r == WAVE - 1 && lane == 0) gdesc_publish(gd, gl, op(local, agg), tagA);
+    T base = init;
+    if (g > 0) {
+        for (;;) {
+            Words<T> gv = to_words(ident);
+            uint32_t st = 0;
+            if (lane == 0) st = gdesc_read<T>(gd, gl - 1, tagA, tagP, gv);
+            st = (uint32_t)__builtin_amdgcn_readfirstlane((int)st);
+            if (st == DESC_P) {
+                base = read_lane(from_words<T>(gv), 0);
+                break;
+            }
+            if (wait_give_up(wc, rounds)) break;
+        }
+    }
+    return op(base, local);
 }
 
 struct ScanGeom {
@@ -122,19 +228,20 @@ struct ScanGeom {
 };
 
 // ---- one tile of a contiguous line, scanned in registers ---------------------------------------------
-// 256 threads x K loads of 16 output bytes.  Wave w owns the w-th quarter of the tile; its k-th load
-// covers 64 * VEC consecutive elements (one fully coalesced 1 KiB request for 4-byte inputs).  Per load:
-// scan inside the lane, DPP scan across the wave, carry to the next load; wave totals meet in LDS.
-template <typename T, typename Op, int K> struct TileRegs {
+// NW waves x K loads of 16 output bytes.  Wave w owns the w-th part of the tile; its k-th load covers 64 * VEC
+// consecutive elements (one fully coalesced 1 KiB request for 4-byte inputs).  Per load: scan inside the lane, DPP scan
+// across the wave, carry to the next load; the prefix inside the wave's part is folded into the values at once, so
+// a tile costs K vector registers and nothing else (a separate array of per-load prefixes cost K more registers and
+// kept the 1024-thread kernel at one workgroup per compute unit).  Exclusive scans shift while folding.
+template <typename T, int K> struct TileRegs {
     static constexpr int VEC = 16 / sizeof(T);
     // vector values, not T v[K][VEC]: with the array form the 64-bit integer instantiations kept the tile in private
     // memory (a store and a load per element: cumsum of Int64[2^26] 342 us against 191 us for Float64)
-    typename VecOf<T, VEC>::type v[K];     // inclusive scan inside each lane's vector
-    T excl[K];                             // exclusive prefix of that vector inside the wave's quarter
+    typename VecOf<T, VEC>::type v[K];     // scan of the wave's part up to and including (inclusive) / excluding the element
 };
 
 template <typename In, typename T, typename Op, bool VECTOR, int K, int NW = 4>
-__device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e0, int valid, Op op, TileRegs<T, Op, K>& r) {
+__device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e0, int valid, int inclusive, Op op, TileRegs<T, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     typedef typename VecOf<In, VEC>::type VI;
@@ -142,9 +249,10 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int woff = wave * (WAVE * VEC * K) + lane * VEC;
     if (VECTOR && valid == TILE) {
+        const In* p = in + e0 + woff;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const VI x = load_nt((const VI*)(in + e0 + woff + k * WAVE * VEC));
+            const VI x = load_nt((const VI*)(p + k * WAVE * VEC));
 #pragma unroll
             for (int j = 0; j < VEC; ++j) r.v[k][j] = (T)x[j];
         }
@@ -163,45 +271,45 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
 #pragma unroll
         for (int j = 1; j < VEC; ++j) r.v[k][j] = op(r.v[k][j - 1], r.v[k][j]);
         const T inc = wave_scan_inclusive(r.v[k][VEC - 1], op, ident);
-        r.excl[k] = op(carry, wave_shift_right(inc, ident));
+        const T excl = op(carry, wave_shift_right(inc, ident));
         carry = op(carry, read_lane(inc, WAVE - 1));
+        if (inclusive) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[k][j] = op(excl, r.v[k][j]);
+        } else {
+#pragma unroll
+            for (int j = VEC - 1; j > 0; --j) r.v[k][j] = op(excl, r.v[k][j - 1]);
+            r.v[k][0] = excl;
+        }
     }
-    return carry;    // total of this wave's quarter
+    return carry;    // total of this wave's part
 }
 
+// `base`: everything in front of this wave's part (init, earlier tiles, earlier waves).
 template <typename T, typename Op, bool VECTOR, int K, int NW = 4>
-__device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int valid, int inclusive, T base, Op op,
-                                           const TileRegs<T, Op, K>& r) {
+__device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int valid, T base, Op op, const TileRegs<T, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     typedef typename VecOf<T, VEC>::type VT;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int woff = wave * (WAVE * VEC * K) + lane * VEC;
     if (VECTOR && valid == TILE) {
+        T* p = out + e0 + woff;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const T off = op(base, r.excl[k]);
             VT o;
-            if (inclusive) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) o[j] = op(off, r.v[k][j]);
-            } else {
-                o[0] = off;
-#pragma unroll
-                for (int j = 1; j < VEC; ++j) o[j] = op(off, r.v[k][j - 1]);
-            }
-            store_nt((VT*)(out + e0 + woff + k * WAVE * VEC), o);
+            for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
+            store_nt((VT*)(p + k * WAVE * VEC), o);
         }
     } else {
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const T off = op(base, r.excl[k]);
+        for (int k = 0; k < K; ++k)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const int idx = woff + k * WAVE * VEC + j;
-                if (idx < valid) out[e0 + idx] = inclusive ? op(off, r.v[k][j]) : (j == 0 ? off : op(off, r.v[k][j - 1]));
+                if (idx < valid) out[e0 + idx] = op(base, r.v[k][j]);
             }
-        }
     }
 }
 
@@ -214,15 +322,15 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ 
     const T ident = Op::template identity<T>();
     const int wave = threadIdx.x / WAVE;
     const int64_t e0 = (int64_t)blockIdx.x * line_len;
-    TileRegs<T, Op, K> r;
-    const T wtot = tile_load_scan<In, T, Op, VECTOR, K>(in, e0, (int)line_len, op, r);
+    TileRegs<T, K> r;
+    const T wtot = tile_load_scan<In, T, Op, VECTOR, K>(in, e0, (int)line_len, inclusive, op, r);
     if (lane_id() == 0) lds_wave[wave] = wtot;
     __syncthreads();
     T wave_prefix = ident;
 #pragma unroll
     for (int w = 0; w < NW; ++w)
         if (w < wave) wave_prefix = op(wave_prefix, lds_wave[w]);
-    tile_store<T, Op, VECTOR, K>(out, e0, (int)line_len, inclusive, op(init, wave_prefix), op, r);
+    tile_store<T, Op, VECTOR, K>(out, e0, (int)line_len, op(init, wave_prefix), op, r);
 }
 
 // ---- long contiguous lines: persistent workgroups, single pass, two-level decoupled look-back --------------
@@ -258,7 +366,7 @@ template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
 __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
                                                          int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                          unsigned long long* counter, uint64_t* desc, int64_t ngroups_per_line,
-                                                         int64_t ngroups, int64_t desc_capacity, int backoff) {
+                                                         int64_t ngroups, int64_t desc_capacity, WaitCtl wc) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     __shared__ T lds_wave[NW];
@@ -280,8 +388,8 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
         const int64_t e0 = line * line_len + tl * TILE;
         const int64_t left = line_len - tl * TILE;
         const int valid = left < TILE ? (int)left : TILE;
-        TileRegs<T, Op, K> r;
-        const T wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, op, r);
+        TileRegs<T, K> r;
+        const T wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, inclusive, op, r);
         if (lane == 0) lds_wave[wave] = wtot;
         __syncthreads();
         T wave_prefix = ident, tile_agg = ident;
@@ -296,16 +404,105 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, tile_agg, (epoch << 2) | DESC_A);
             if (tl > 0)
                 tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tl, line * ngroups_per_line + (tl >> 6),
-                                             epoch, tile_agg, init, op, ident, backoff);
+                                             epoch, tile_agg, init, op, ident, wc);
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
-        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, inclusive, op(lds_prefix, wave_prefix), op, r);
+        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, wave_prefix), op, r);
         if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         cur = lds_id;
     }
     chain_finish(cur, ntiles, (int64_t)Words<T>::N * (ntiles + ngroups), counter, desc, desc_capacity);
+}
+
+// ---- long contiguous lines: one tile per workgroup in launch order, single pass ------------------------------------
+// Tile = blockIdx.x.  No tile counter: device-wide atomics on one address complete at about 14 ns each, which caps a
+// counter-fed kernel at 70 M tiles/s, and the counter's round trip sits in front of every tile's loads.  Forward
+// progress instead rests on the order in which the hardware starts workgroups: each XCD starts the workgroups dealt
+// to it in increasing blockIdx, so the lowest-numbered unfinished tile is always resident (it cannot be waiting for a
+// slot behind higher-numbered tiles of its own XCD, and tiles of other XCDs do not take its slots), and it waits for
+// nobody.  Should a device ever start workgroups out of order with all slots taken by waiting tiles, the bounded
+// waits end the call with RK_ERR_WAIT instead of hanging; RK_SCAN_DYNAMIC_IDS=1 selects scan_chain_kernel, whose
+// counter needs no such assumption.
+// 1024 threads x 8 vectors = 128 KiB of input per tile at <= 64 registers: two workgroups share a compute unit, one
+// loads or stores while the other waits for its prefix (at 112 registers and one workgroup per unit the wait was
+// dead time: 2^26 Int32 95.6 -> 92.5 us, 2^27 187.8 -> 180.5 us).  Smaller tiles stream better on their own (16 KiB
+// tiles without any look-back: 86 us) but lose more to the look-back than they gain.
+// The epoch of the call is read from the workspace header; the workgroup that leaves last (two-level exit tickets)
+// advances it and clears a rotating slice of unused descriptor slots, like chain_finish.
+// Compiled for 8 waves per SIMD (<= 64 registers); only launched for 4-byte values with aligned lines: 8-byte values
+// hold the same 32 registers of data but scan with twice the temporaries and spilled 20 registers at that limit.
+template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
+__global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+                                                                    int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
+                                                                    unsigned long long* counter, uint32_t* tickets, int ticket_group,
+                                                                    uint64_t* desc, int64_t ngroups_per_line, int64_t ngroups,
+                                                                    int64_t desc_capacity, WaitCtl wc) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int TILE = NW * WAVE * VEC * K;
+    __shared__ T lds_wave[NW];
+    __shared__ T lds_prefix;
+    __shared__ int lds_last;
+    const T ident = Op::template identity<T>();
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    uint64_t* tile_desc = desc;                                        // [words][ntiles]
+    uint64_t* group_desc = desc + (int64_t)Words<T>::N * ntiles;       // [ngroups] lines
+    const uint32_t epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+    {
+        const int64_t tile = blockIdx.x;
+        const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
+        const int64_t e0 = line * line_len + tl * TILE;
+        const int64_t left = line_len - tl * TILE;
+        const int valid = left < TILE ? (int)left : TILE;
+        TileRegs<T, K> r;
+        const T wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, inclusive, op, r);
+        if (lane == 0) lds_wave[wave] = wtot;
+        __syncthreads();
+        if (wave == 0) {
+            static_assert(NW <= WAVE, "the wave totals are scanned by one wave");
+            const T x = lane < NW ? lds_wave[lane] : ident;
+            const T inc = wave_scan_inclusive(x, op, ident);
+            const T tile_agg = read_lane(inc, NW - 1);
+            if (lane < NW) lds_wave[lane] = wave_shift_right(inc, ident);       // what lies in front of each wave inside the tile
+            T tile_prefix = init;
+            if (lane == 0) desc_publish(tile_desc, ntiles, tile, tile_agg, (epoch << 2) | DESC_A);
+            if (tl > 0)
+                tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tl, line * ngroups_per_line + (tl >> 6), epoch,
+                                                   tile_agg, init, op, ident, wc);
+            if (lane == 0) lds_prefix = tile_prefix;
+        }
+        __syncthreads();
+        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
+    }
+    // exit tickets: groups of `ticket_group` workgroups share a first-level ticket (each on its own line)
+    if (tid == 0) {
+        const int64_t nb = gridDim.x, ng = (nb + ticket_group - 1) / ticket_group, grp = blockIdx.x / ticket_group;
+        const uint32_t gsize = (uint32_t)(grp == ng - 1 ? nb - grp * ticket_group : ticket_group);
+        int last = 0;
+        uint32_t* gt = tickets + grp * TICKET_STRIDE;
+        if (__hip_atomic_fetch_add(gt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1u) {
+            *gt = 0;                                                            // clean for the next call
+            uint32_t* lt = tickets + ng * TICKET_STRIDE;
+            if (__hip_atomic_fetch_add(lt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)ng - 1u) {
+                *lt = 0;
+                last = 1;
+            }
+        }
+        lds_last = last;
+    }
+    __syncthreads();
+    if (!lds_last || tid >= WAVE) return;
+    // every workgroup has read the epoch and left: advance it, sweep a slice of the slots this call did not use
+    const int64_t used = (int64_t)Words<T>::N * ntiles + ngroups * GROUP_DESC_STRIDE;
+    const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
+    int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
+    if (lo < used) lo = used;
+    if (hi > desc_capacity) hi = desc_capacity;
+    for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
+    uint32_t e = (epoch + 1u) & 0x3fffffffu;
+    if (e == 0u) e = 1u;
+    if (lane == 0) *counter = (unsigned long long)e << 32;
 }
 
 // ---- contiguous lines shorter than a tile: one wave per line -------------------------------------
@@ -568,7 +765,8 @@ __global__ __launch_bounds__(256) void scan_narrow_kernel(const In* __restrict__
 }
 
 // ---- inner >= 64: lanes along `inner`, 4 waves share the rows of a chunk -----------------------------
-// grid (strips, slices, outer).  A workgroup scans the rows [slice * rows_per_slice, +rows_per_slice) of its
+// grid (strips * outer, slices): the outer index shares the x axis with the strips (the other axes end at 65535).
+// A workgroup scans the rows [slice * rows_per_slice, +rows_per_slice) of its
 // 64 * VEC columns: a wave keeps R consecutive rows in registers, scans them downwards, and the four waves
 // exchange their column totals through LDS.  With one slice the scan starts from `init`; with several, the
 // exclusive prefix of every (slice, column) comes from `carry_in` (scan_strided_totals_kernel + a scan of the
@@ -577,7 +775,7 @@ __global__ __launch_bounds__(256) void scan_narrow_kernel(const In* __restrict__
 template <typename In, typename T, typename Op, bool VECTOR, int R>
 __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
                                                            int inclusive, Op op, int64_t rows_per_slice,
-                                                           const T* __restrict__ carry_in, int64_t carry_pitch) {
+                                                           const T* __restrict__ carry_in, int64_t carry_pitch, int64_t strips) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     constexpr int COLS = WAVE * VEC;
     constexpr int NW = 4;
@@ -585,9 +783,10 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     typedef typename VecOf<In, VEC>::type VI;
     __shared__ T lds[NW][COLS];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int64_t col0 = (int64_t)blockIdx.x * COLS + (int64_t)lane * VEC;
+    const int64_t o = (int64_t)blockIdx.x / strips, strip = (int64_t)blockIdx.x - o * strips;
+    const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
     const bool live = col0 < g.inner;
-    const int64_t slab = (int64_t)blockIdx.z * g.inner * g.mid;
+    const int64_t slab = o * g.inner * g.mid;
     // (Running the slices last to first, so that the scan starts with what the totals pass read last, changed nothing.)
     const int64_t slice = (int64_t)blockIdx.y;
     const int64_t m_begin = slice * rows_per_slice;
@@ -596,7 +795,7 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     T carry[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
-        carry[j] = (carry_in != nullptr && live) ? carry_in[((int64_t)blockIdx.z * gridDim.y + slice) * carry_pitch + col0 + j] : init;
+        carry[j] = (carry_in != nullptr && live) ? carry_in[(o * gridDim.y + slice) * carry_pitch + col0 + j] : init;
     for (int64_t m0 = m_begin; m0 < m_end; m0 += NW * R) {
         const int64_t row0 = m0 + (int64_t)wave * R;
         T v[R][VEC];
@@ -652,16 +851,17 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
 // Column totals of every (slice, column): totals[(o * slices + slice) * pitch + column].
 template <typename In, typename T, typename Op, bool VECTOR, int UNROLL>
 __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __restrict__ in, T* __restrict__ totals, ScanGeom g, Op op,
-                                                                  int64_t rows_per_slice, int64_t pitch) {
+                                                                  int64_t rows_per_slice, int64_t pitch, int64_t strips) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     constexpr int COLS = WAVE * VEC;
     constexpr int NW = 4;
     typedef typename VecOf<In, VEC>::type VI;
     __shared__ T lds[NW][COLS];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int64_t col0 = (int64_t)blockIdx.x * COLS + (int64_t)lane * VEC;
+    const int64_t o = (int64_t)blockIdx.x / strips, strip = (int64_t)blockIdx.x - o * strips;
+    const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
     const bool live = col0 < g.inner;
-    const int64_t slab = (int64_t)blockIdx.z * g.inner * g.mid;
+    const int64_t slab = o * g.inner * g.mid;
     const int64_t m_begin = (int64_t)blockIdx.y * rows_per_slice;
     const int64_t m_end = m_begin + rows_per_slice < g.mid ? m_begin + rows_per_slice : g.mid;
     T acc[VEC];
@@ -702,7 +902,7 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
         T r = lds[0][t];
 #pragma unroll
         for (int w = 1; w < NW; ++w) r = op(r, lds[w][t]);
-        totals[((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * pitch + (int64_t)blockIdx.x * COLS + t] = r;
+        totals[(o * gridDim.y + blockIdx.y) * pitch + strip * COLS + t] = r;
     }
 }
 
@@ -713,8 +913,11 @@ template <typename T, int K> struct ScanTile {     // geometry of the tile kerne
 };
 
 int tune_scan_backoff();        // rk_api.hip
+long long wait_budget();        // rk_api.hip: poll rounds a bounded wait may spend (rk_set_wait_budget)
+inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_budget(), tune_scan_backoff()}; }
 int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
+int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
 struct ScanArgs {
@@ -738,7 +941,7 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     const bool vec = aligned && (g.inner % VEC == 0);
     const int cols = WAVE * (vec ? VEC : 1);
     const int64_t strips = (g.inner + cols - 1) / cols;
-    if (strips > 0x7fffffff || g.outer > 65535) return RK_ERR_TOO_LARGE;
+    if (strips * g.outer > 0x7fffffff) return RK_ERR_TOO_LARGE;
     const int64_t pitch = strips * cols;
     const int64_t cus = device_info().cus;
     int64_t slices = 1;
@@ -752,9 +955,9 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
         if (slices > 65535) slices = 65535;
     }
     if (slices <= 1) {
-        dim3 grid((unsigned)strips, 1, (unsigned)g.outer);
-        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0);
-        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0);
+        dim3 grid((unsigned)(strips * g.outer), 1);
+        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
+        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
@@ -763,9 +966,9 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     slices = (g.mid + rps - 1) / rps;
     T* totals = (T*)scratch;
     const size_t used = ((size_t)(pitch * slices * g.outer) * sizeof(T) + 255) & ~(size_t)255;
-    dim3 grid((unsigned)strips, (unsigned)slices, (unsigned)g.outer);
-    if (vec) scan_strided_totals_kernel<In, T, Op, true, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch);
-    else     scan_strided_totals_kernel<In, T, Op, false, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch);
+    dim3 grid((unsigned)(strips * g.outer), (unsigned)slices);
+    if (vec) scan_strided_totals_kernel<In, T, Op, true, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch, strips);
+    else     scan_strided_totals_kernel<In, T, Op, false, 4><<<grid, 256, 0, stream>>>(in, totals, g, op, rps, pitch, strips);
     RK_LAUNCH_CHECK();
     // exclusive scan of the totals along the slice axis, in place, seeded with init: (pitch, slices, outer); the
     // totals are 16-byte aligned and pitch % VEC == 0
@@ -776,12 +979,13 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
         if (st != RK_SUCCESS) return st;
     } else {
         const int tcols = WAVE * VEC;
-        dim3 tgrid((unsigned)((pitch + tcols - 1) / tcols), 1, (unsigned)g.outer);
-        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0);
+        const int64_t tstrips = (pitch + tcols - 1) / tcols;
+        dim3 tgrid((unsigned)(tstrips * g.outer), 1);
+        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0, tstrips);
         RK_LAUNCH_CHECK();
     }
-    if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
-    else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch);
+    if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
+    else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }
@@ -928,11 +1132,11 @@ inline int32_t launch_scan(const ScanArgs& a) {
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
-    // long lines: the chained look-back scan; tile = NW waves x 8 vectors, as large as the line length allows
+    // long lines: single pass with look-back; tile = NW waves x 8 vectors, as large as the line length allows
     constexpr int KT = 8;
     const int64_t line_bytes = s.mid * (int64_t)sizeof(T);
     // measured (Int32, 2^22 .. 2^27 elements): 16 waves beat 8 and 4 at every size -- fewer, larger tiles mean
-    // fewer serialised acquisitions and fewer look-backs; lines that barely exceed one small tile use 8 or 4
+    // fewer look-backs; lines that barely exceed one small tile use 8 or 4
     int nw = line_bytes > ((int64_t)64 << 10) ? 16 : (line_bytes > ((int64_t)32 << 10) ? 8 : 4);
     if (tune_scan_waves() != 0) nw = tune_scan_waves();
     const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
@@ -941,17 +1145,35 @@ inline int32_t launch_scan(const ScanArgs& a) {
     if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
     Workspace w{};
     const int64_t gpl = (tpl + WAVE - 1) / WAVE, ngroups = gpl * nlines;
-    const size_t need = (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t);
+    // 8-byte values and unaligned lines do not fit two workgroups a compute unit; with one, the persistent counter-fed
+    // kernel is the faster of the two (cumsum of Int64[2^25]: 96 against 107 us)
+    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || !lines_aligned;
+    const size_t need = dynamic_ids ? (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t)
+                                    : ((size_t)ntiles * Words<T>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
+    unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
+    const WaitCtl wc = wait_ctl(w.hdr);
+    if constexpr (sizeof(T) <= 4) {
+        if (!dynamic_ids) {
+            // exit tickets: at most half of the ticket lines, at least TICKET_GROUP workgroups a ticket
+            int64_t tg = (ntiles + (int64_t)WS_TICKET_COUNT / 2 - 1) / ((int64_t)WS_TICKET_COUNT / 2);
+            if (tg < TICKET_GROUP) tg = TICKET_GROUP;
+#define RK_SCAN_ORDERED(NWW)                                                                                          \
+            scan_ordered_kernel<In, T, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
+                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, (int)tg, w.desc, gpl, ngroups, cap, wc)
+            if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
+#undef RK_SCAN_ORDERED
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
+        }
+    }
     int64_t grid = (int64_t)device_info().cus * tune_scan_blocks_per_cu() * 4 / nw;
     if (grid > ntiles) grid = ntiles;
     if (grid < 1) grid = 1;
-    unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
-    const int backoff = tune_scan_backoff();
 #define RK_SCAN_CHAIN(VECF, NWW)                                                                                      \
     scan_chain_kernel<In, T, Op, VECF, KT, NWW><<<(unsigned)grid, NWW * WAVE, 0, a.stream>>>(                          \
-        in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, backoff)
+        in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, wc)
     if (lines_aligned) {
         if (nw == 16) RK_SCAN_CHAIN(true, 16); else if (nw == 8) RK_SCAN_CHAIN(true, 8); else RK_SCAN_CHAIN(true, 4);
     } else {

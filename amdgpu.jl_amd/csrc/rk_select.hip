@@ -48,7 +48,7 @@ template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K>
 __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uint8_t* __restrict__ bools, int64_t n, int64_t* __restrict__ ys,
                                                                        int64_t* __restrict__ count_out, SelShape shp, int aligned,
                                                                        unsigned long long* counter, uint64_t* desc, int64_t ntiles,
-                                                                       int64_t ngroups, int64_t desc_capacity, int backoff) {
+                                                                       int64_t ngroups, int64_t desc_capacity, WaitCtl wc) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int SEL_TILE = SEL_NW * SEL_CHUNK * SEL_K;
     __shared__ uint16_t lds_strip[SEL_NW][SEL_CHUNK];
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, (int64_t)tile_count, (epoch << 2) | DESC_A);
             if (tile > 0)
                 tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
-                                             (int64_t)0, op, (int64_t)0, backoff);
+                                             (int64_t)0, op, (int64_t)0, wc);
             if (lane == 0) {
                 lds_prefix = tile_prefix;
                 if (tile == ntiles - 1 && count_out != nullptr) *count_out = tile_prefix + tile_count;
@@ -210,11 +210,11 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     if (grid > ntiles) grid = ntiles;
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const int aligned = is_aligned(bools, 16) ? 1 : 0;
-    const int backoff = tune_scan_backoff();
+    const WaitCtl wc = wait_ctl(w.hdr);
     hipStream_t st = (hipStream_t)stream;
 #define RK_SELECT2(LIN, SM, NWW, KK)                                                                                             \
     findall_select_kernel<LIN, SM, NWW, KK><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned, counter,  \
-                                                                                   w.desc, ntiles, ngroups, cap, backoff)
+                                                                                   w.desc, ntiles, ngroups, cap, wc)
 #define RK_SELECT(LIN, SM)                                                                                                       \
     do {                                                                                                                         \
         if (kl == 4) RK_SELECT2(LIN, SM, 16, 4);                                                                                 \

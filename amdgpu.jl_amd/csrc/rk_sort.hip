@@ -22,6 +22,7 @@
 // Keys are mapped to unsigned integers that sort like Base.isless (-0.0 < 0.0, NaN last; every NaN becomes the
 // canonical one), complemented for rev=true; the mapping is applied on the first read and undone on the last
 // write.  The sort is stable, so sortperm keeps equal keys in index order (also with rev=true, as Base does).
+#include <cstddef>
 #include <cstdlib>
 #include <type_traits>
 
@@ -40,7 +41,8 @@ struct SortCtl {                                  // head of the caller's tempor
     uint32_t ticket[SORT_MAX_PASSES];
     uint32_t skip[SORT_MAX_PASSES];
     uint32_t src_is_b[SORT_MAX_PASSES];           // the pass reads buffer B (1) or A (0)
-    uint32_t first_pass, last_pass, nexec, pad;
+    uint32_t first_pass, last_pass, nexec;
+    uint32_t wait_failed;                         // a look-back gave up its bounded wait (WaitCtl); read by rk_sort_status
     unsigned long long inv_min;                   // ~(smallest mapped key), kept as a maximum so that zero is its identity
 };
 
@@ -339,7 +341,8 @@ template <typename T, int ITEMS, bool PERM, bool COUNTED>
 __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restrict__ orig, typename SortKey<T>::U* buf_a,
                                                                typename SortKey<T>::U* buf_b, uint32_t* val_a, uint32_t* val_b,
                                                                int64_t* __restrict__ perm_out, uint32_t n, int pass, int rev, SortCtl* ctl,
-                                                               uint64_t* desc, const uint32_t* __restrict__ tile_before, uint32_t ntiles) {
+                                                               uint64_t* desc, const uint32_t* __restrict__ tile_before, uint32_t ntiles,
+                                                               long long wait_rounds) {
     typedef typename SortKey<T>::U U;
     constexpr int TILE = SORT_BLOCK * ITEMS;
     __shared__ U lds_keys[TILE];
@@ -438,6 +441,8 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
                 constexpr int LB = 8;
                 int64_t t = (int64_t)tile - 1;
                 bool done = false;
+                const WaitCtl wc{&ctl->wait_failed, wait_rounds, 0};
+                long long rounds = 0;
                 while (!done) {
                     uint64_t w[LB];
     #pragma unroll
@@ -454,7 +459,11 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
                         if (tg == tag_p) { done = true; break; }
                     }
                     t -= j;
-                    if (!done && j == 0) __builtin_amdgcn_s_sleep(2);
+                    if (!done && j == 0) {
+                        // every lane counts its own rounds (a lane per digit); one giving up makes all others follow
+                        if (wait_give_up(wc, rounds)) break;
+                        __builtin_amdgcn_s_sleep(2);
+                    }
                 }
                 __hip_atomic_store(my, ((uint64_t)tag_p << 32) | (uint64_t)(excl + count), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
@@ -607,11 +616,11 @@ static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, voi
             const int32_t st = scan_across_rows<uint32_t, uint32_t, OpAdd>(tile_count, tile_count, sg, 0u, 0, OpAdd(), true,
                                                                           base + l.scratch_off, SORT_SCAN_SCRATCH, stream);
             if (st != RK_SUCCESS) return st;
-            if (perm) sort_pass_kernel<T, ITEMS, true, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles);
-            else sort_pass_kernel<T, ITEMS, false, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles);
+            if (perm) sort_pass_kernel<T, ITEMS, true, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles, wait_budget());
+            else sort_pass_kernel<T, ITEMS, false, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles, wait_budget());
         } else {
-            if (perm) sort_pass_kernel<T, ITEMS, true, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles);
-            else sort_pass_kernel<T, ITEMS, false, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles);
+            if (perm) sort_pass_kernel<T, ITEMS, true, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles, wait_budget());
+            else sort_pass_kernel<T, ITEMS, false, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles, wait_budget());
         }
         RK_LAUNCH_CHECK();
     }
@@ -662,6 +671,15 @@ static int32_t sort_dispatch(rk_dtype dt, void* keys, int64_t* perm_out, int64_t
         case RK_F16: return sort_typed<half_bits>(keys, perm_out, n, r, tmp, tmp_bytes, st);
         default:     return sort_typed<int16_t>(keys, perm_out, n, r, tmp, tmp_bytes, st);
     }
+}
+
+extern "C" int32_t rk_sort_status(const void* tmp, size_t tmp_bytes, void* stream) {
+    if (tmp == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    if (!is_aligned(tmp, 256) || tmp_bytes < sizeof(SortCtl)) return RK_ERR_WORKSPACE;
+    uint32_t failed = 0;
+    RK_HIP(hipMemcpyAsync(&failed, (const char*)tmp + offsetof(SortCtl, wait_failed), sizeof(failed), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    RK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return failed != 0u ? RK_ERR_WAIT : RK_SUCCESS;
 }
 
 extern "C" int32_t rk_sort(rk_dtype dt, void* keys, int64_t n, int32_t rev, void* tmp, size_t tmp_bytes, void* stream) {

@@ -55,7 +55,8 @@ enum {
     RK_ERR_UNSUPPORTED      = 10002, /* legal request outside the enumerated op set      */
     RK_ERR_WORKSPACE        = 10003, /* workspace missing, misaligned or too small       */
     RK_ERR_DIMENSION        = 10004, /* shapes do not agree (Julia: DimensionMismatch)   */
-    RK_ERR_TOO_LARGE        = 10005  /* an extent exceeds what the kernels index         */
+    RK_ERR_TOO_LARGE        = 10005, /* an extent exceeds what the kernels index         */
+    RK_ERR_WAIT             = 10006  /* a kernel gave up a wait on another workgroup     */
 };
 
 /* ---- element types (Julia eltype <-> code) -------------------------------------- */
@@ -98,6 +99,26 @@ RK_API size_t  rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const i
 /* Zero the bookkeeping area of a freshly allocated workspace (asynchronous on `stream`).
  * Call once per allocation, before its first use. */
 RK_API int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream);
+
+/* Bounded waits.  The single-pass scan, the one-pass findall and the sort hand values from
+ * workgroup to workgroup through the workspace (the sort: through its temporary); the
+ * receiving side polls.  With a prepared workspace used by one call at a time such a wait
+ * ends within microseconds.  A workspace that was never prepared, or that two calls use at
+ * the same time, could make it wait for ever -- a hung GPU -- so every wait counts its
+ * unsuccessful polls: after `rounds` of them (default 2^21, a second or two; environment
+ * RK_WAIT_BUDGET) the kernel records the failure in the workspace, stops waiting and runs to
+ * its end with meaningless results.  No counterpart in the reference, whose kernels never
+ * wait on each other (it launches one kernel per pass, src/kernels/mapreduce.jl:158-170).
+ *   rk_set_wait_budget   sets the budget for later calls of this process (<= 0: the default)
+ *                        and returns the previous one.
+ *   rk_workspace_status  SYNCHRONISES `stream`, then returns RK_ERR_WAIT if any call on the
+ *                        workspace gave up a wait since it was last prepared, else
+ *                        RK_SUCCESS.  After RK_ERR_WAIT call rk_workspace_init again.
+ *   rk_sort_status       the same for the temporary of rk_sort / rk_sortperm (no
+ *                        preparation needed afterwards: every sort clears its temporary). */
+RK_API int64_t rk_set_wait_budget(int64_t rounds);
+RK_API int32_t rk_workspace_status(const void* ws, size_t ws_bytes, void* stream);
+RK_API int32_t rk_sort_status(const void* tmp, size_t tmp_bytes, void* stream);
 
 /* ---- mapreduce ------------------------------------------------------------------
  * Replaces GPUArrays.mapreducedim!(f, op, R, A; init)      src/kernels/mapreduce.jl:86-173
