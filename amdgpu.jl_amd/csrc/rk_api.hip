@@ -81,6 +81,13 @@ int tune_scan_dynamic_ids() {
     return v;
 }
 
+// 0: scans across the rows of a wide matrix (few strips of columns) take the three-pass path (totals, scan of the totals,
+// scan) instead of the single-pass kernel with look-back (RK_SCAN_ROWS_ORDERED).
+int tune_scan_rows_ordered() {
+    static const int v = env_int("RK_SCAN_ROWS_ORDERED", 1, 0, 1);
+    return v;
+}
+
 // Workgroups per compute unit the scan across rows aims for when it cuts the rows into slices
 // (RK_SCAN_SLICE_BLOCKS_PER_CU).
 int tune_scan_slice_blocks_per_cu() {

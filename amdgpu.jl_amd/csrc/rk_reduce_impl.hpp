@@ -111,7 +111,10 @@ template <typename Acc, typename Op, typename Out = Acc> struct ReduceSink {
     int  has_init;
     __device__ __forceinline__ void operator()(int64_t q, Acc t) const { R[q] = (Out)(has_init ? Op()(init, t) : t); }
 };
+// The value written is the winning ELEMENT, read back from A at the winner's position: decoding the key would turn
+// every NaN into the canonical one, and Julia returns the element itself (sign and payload of a NaN included).
 template <typename T, typename P> struct ArgSink {
+    const T* A;
     T*       vals;
     int64_t* cart;
     int      ndim;
@@ -120,9 +123,10 @@ template <typename T, typename P> struct ArgSink {
     bool     absolute;   // positions are already linear offsets into A (the generic kernel)
     LineGeom g;
     __device__ __forceinline__ void operator()(int64_t q, ArgAcc<T, P> t) const {
-        if (vals) vals[q] = OrderKey<T>::value(t.k, want_max);
+        const int64_t lin = absolute ? (int64_t)t.i : line_base(g, q) + (int64_t)t.i * g.inner;
+        if (vals) vals[q] = t.i < 0 ? OrderKey<T>::value(t.k, want_max) : A[lin];
         if (cart) {
-            int64_t rem = absolute ? (int64_t)t.i : line_base(g, q) + (int64_t)t.i * g.inner;
+            int64_t rem = lin;
             for (int d = 0; d < ndim; ++d) {
                 const int64_t c = rem % shape[d];
                 rem /= shape[d];
@@ -1040,6 +1044,7 @@ inline int32_t mapreduce_typed(const MapreduceArgs& a) {
 template <typename T, typename P>
 inline int32_t findminmax_pos(const FindArgs& a, const Shape3& s) {
     ArgSink<T, P> sink{};
+    sink.A = (const T*)a.A;
     sink.vals = (T*)a.vals;
     sink.cart = a.cart;
     sink.ndim = a.ndim;

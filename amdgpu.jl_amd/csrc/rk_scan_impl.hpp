@@ -416,6 +416,47 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
     chain_finish(cur, ntiles, (int64_t)Words<T>::N * (ntiles + ngroups), counter, desc, desc_capacity);
 }
 
+// End of a kernel whose workgroups read the epoch from the header instead of acquiring it: the workgroup that leaves
+// last (two levels of exit tickets: groups of `ticket_group` workgroups share a first-level ticket, each ticket on
+// its own 128-byte line) advances the epoch and clears a rotating slice of the descriptor slots this call did not
+// use, like chain_finish.  Every workgroup has read the epoch before it leaves, so nobody can see the new one.
+__device__ __forceinline__ void ordered_finish(uint32_t epoch, int64_t used, unsigned long long* counter, uint32_t* tickets,
+                                               int ticket_group, uint64_t* desc, int64_t desc_capacity) {
+    __shared__ int lds_last;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        const int64_t nb = gridDim.x, ng = (nb + ticket_group - 1) / ticket_group, grp = blockIdx.x / ticket_group;
+        const uint32_t gsize = (uint32_t)(grp == ng - 1 ? nb - grp * ticket_group : ticket_group);
+        int last = 0;
+        uint32_t* gt = tickets + grp * TICKET_STRIDE;
+        if (__hip_atomic_fetch_add(gt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1u) {
+            *gt = 0;                                                            // clean for the next call
+            uint32_t* lt = tickets + ng * TICKET_STRIDE;
+            if (__hip_atomic_fetch_add(lt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)ng - 1u) {
+                *lt = 0;
+                last = 1;
+            }
+        }
+        lds_last = last;
+    }
+    __syncthreads();
+    if (!lds_last || tid >= WAVE) return;
+    const int lane = lane_id();
+    const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
+    int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
+    if (lo < used) lo = used;
+    if (hi > desc_capacity) hi = desc_capacity;
+    for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
+    uint32_t e = (epoch + 1u) & 0x3fffffffu;
+    if (e == 0u) e = 1u;                  // tag 0 marks a cleared slot
+    if (lane == 0) *counter = (unsigned long long)e << 32;
+}
+// Workgroups per first-level exit ticket: at most half of the ticket lines in use, at least TICKET_GROUP a ticket.
+inline int ordered_ticket_group(int64_t nblocks) {
+    int64_t tg = (nblocks + (int64_t)WS_TICKET_COUNT / 2 - 1) / ((int64_t)WS_TICKET_COUNT / 2);
+    return (int)(tg < TICKET_GROUP ? TICKET_GROUP : tg);
+}
+
 // ---- long contiguous lines: one tile per workgroup in launch order, single pass ------------------------------------
 // Tile = blockIdx.x.  No tile counter: device-wide atomics on one address complete at about 14 ns each, which caps a
 // counter-fed kernel at 70 M tiles/s, and the counter's round trip sits in front of every tile's loads.  Forward
@@ -443,7 +484,6 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
     constexpr int TILE = NW * WAVE * VEC * K;
     __shared__ T lds_wave[NW];
     __shared__ T lds_prefix;
-    __shared__ int lds_last;
     const T ident = Op::template identity<T>();
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     uint64_t* tile_desc = desc;                                        // [words][ntiles]
@@ -475,34 +515,7 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
         __syncthreads();
         tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
     }
-    // exit tickets: groups of `ticket_group` workgroups share a first-level ticket (each on its own line)
-    if (tid == 0) {
-        const int64_t nb = gridDim.x, ng = (nb + ticket_group - 1) / ticket_group, grp = blockIdx.x / ticket_group;
-        const uint32_t gsize = (uint32_t)(grp == ng - 1 ? nb - grp * ticket_group : ticket_group);
-        int last = 0;
-        uint32_t* gt = tickets + grp * TICKET_STRIDE;
-        if (__hip_atomic_fetch_add(gt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsize - 1u) {
-            *gt = 0;                                                            // clean for the next call
-            uint32_t* lt = tickets + ng * TICKET_STRIDE;
-            if (__hip_atomic_fetch_add(lt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)ng - 1u) {
-                *lt = 0;
-                last = 1;
-            }
-        }
-        lds_last = last;
-    }
-    __syncthreads();
-    if (!lds_last || tid >= WAVE) return;
-    // every workgroup has read the epoch and left: advance it, sweep a slice of the slots this call did not use
-    const int64_t used = (int64_t)Words<T>::N * ntiles + ngroups * GROUP_DESC_STRIDE;
-    const int64_t slice = (desc_capacity + SCAN_SWEEP - 1) / SCAN_SWEEP;
-    int64_t lo = (int64_t)(epoch % SCAN_SWEEP) * slice, hi = lo + slice;
-    if (lo < used) lo = used;
-    if (hi > desc_capacity) hi = desc_capacity;
-    for (int64_t i = lo + lane; i < hi; i += WAVE) desc[i] = 0;
-    uint32_t e = (epoch + 1u) & 0x3fffffffu;
-    if (e == 0u) e = 1u;
-    if (lane == 0) *counter = (unsigned long long)e << 32;
+    ordered_finish(epoch, (int64_t)Words<T>::N * ntiles + ngroups * GROUP_DESC_STRIDE, counter, tickets, ticket_group, desc, desc_capacity);
 }
 
 // ---- contiguous lines shorter than a tile: one wave per line -------------------------------------
@@ -906,6 +919,220 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
     }
 }
 
+// ---- inner >= 64, few strips: tiles of rows in launch order, single pass --------------------------------------------
+// scan_strided_kernel needs one workgroup per strip of 64 * VEC columns; a 4096 x 16384 matrix scanned along its rows
+// has 16 strips.  Cutting the rows into slices makes the slices depend on each other.  The three-pass answer (column
+// totals per slice, scan of the totals, scan from the carried-in prefix) reads the input twice: 12 bytes per element.
+// Here a tile is NW * R = 120 rows of one strip and the dependency is resolved like in the single-pass scan of long lines,
+// with a VECTOR for payload and two levels: a tile publishes its 64 * VEC column totals (1 KiB) and a flag, and sums
+// the totals of its predecessors inside its group of ROWS_GROUP tiles; the last tile of a group publishes the group's
+// aggregate; the first one (the leader) sums group aggregates back to the nearest published prefix and publishes the
+// prefix through the previous group, which the other tiles of its group wait for.  With one level a tile read the
+// totals of every tile in flight on its chain (32 KiB for 120 KiB of rows on a 4096 x 16384 matrix: 108 us); with two
+// it reads 5 KiB on average.  Tiles are numbered slice-major (tile = slice * chains + chain, a chain
+// being one strip of one outer index), so the workgroups in flight cover a compact band of whole rows and every
+// predecessor has a lower blockIdx (forward progress as in scan_ordered_kernel).  HBM traffic: 8 bytes per element;
+// the look-back reads one payload per tile in flight on the same chain -- a quarter of the tile's own bytes with 16
+// chains -- from the device-coherent level, not from HBM.
+//   flags     desc[tile]: tagged word, DESC_A = totals published; desc[ntiles + group]: DESC_A = aggregate of the
+//             group published, DESC_P = inclusive prefix through the group published
+//   payload   [ntiles + 2 * groups][64 * VEC] values in the partials area: totals; group aggregates; group prefixes
+constexpr int ROWS_GROUP = 8;      // tiles of a chain per group of the two-level look-back
+
+// NW waves hold rows; one more wave holds none and does the publishing and the look-back.  The registers a kernel
+// needs are the maximum over its branches, so the row data (32 registers) and the look-back's working set no longer
+// add up: 64 registers suffice and two workgroups share a compute unit (with wave 0 doing both, 25 registers spilled).
+template <typename In, typename T, typename Op, int NW, int R>
+__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
+                                                                               int inclusive, Op op, int64_t strips, int64_t nchains,
+                                                                               int64_t nslices, T* payload, unsigned long long* counter,
+                                                                               uint32_t* tickets, int ticket_group, uint64_t* desc,
+                                                                               int64_t desc_capacity, WaitCtl wc) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int COLS = WAVE * VEC;
+    typedef typename VecOf<T, VEC>::type VT;
+    typedef typename VecOf<In, VEC>::type VI;
+    __shared__ T lds[NW][COLS];
+    __shared__ T lds_base[COLS];
+    const T ident = Op::template identity<T>();
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const int64_t ntiles = gridDim.x;
+    const int64_t tile = blockIdx.x;
+    const int64_t slice = tile / nchains, chain = tile - slice * nchains;
+    uint32_t epoch = 0;
+    if (wave == NW) {
+        epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+        const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
+        const int64_t ngroups_chain = (nslices + ROWS_GROUP - 1) / ROWS_GROUP;
+        uint64_t* gflag = desc + ntiles;                                    // [group * nchains + chain]
+        T* gpayA = payload + ntiles * COLS;                                  // aggregates of whole groups
+        T* gpayP = gpayA + ngroups_chain * nchains * COLS;                   // inclusive prefixes through a group
+        const int r = (int)(slice % ROWS_GROUP);                             // predecessors inside the group
+        const int64_t grp = slice / ROWS_GROUP;                              // groups in front of this one in the chain
+        __syncthreads();                                 // the row waves have written their column totals
+        T tot[VEC], base[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            tot[j] = ident;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) tot[j] = op(tot[j], lds[w][lane * VEC + j]);
+            base[j] = init;
+        }
+        const bool has_reader = slice + 1 < nslices;     // the last slice of a chain has none
+        if (has_reader && r < ROWS_GROUP - 1) {          // the group's last tile publishes the group aggregate instead
+            VT t;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) t[j] = tot[j];
+            store_agent((VT*)(payload + tile * COLS + lane * VEC), t);
+            publish_barrier();                           // the totals are at the coherent level before the flag
+            if (lane == 0) __hip_atomic_store(&desc[tile], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        long long rounds = 0;
+        if (r == 0) {
+            if (grp > 0) {
+                // leader: aggregates of the groups in front, back to the nearest published prefix; publishes the
+                // prefix through the previous group for the other tiles of its own
+                T acc[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = ident;
+                int64_t first = grp - 1, rem = grp;
+                for (;;) {
+                    uint32_t st = DESC_P;                // lanes beyond the first group: terminators
+                    if (lane < rem) {
+                        const uint32_t tag = (uint32_t)(__hip_atomic_load(&gflag[(first - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+                        st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
+                    }
+                    const uint64_t ballotP = __ballot(st == DESC_P);
+                    const uint64_t ballotX = __ballot(st == 0u);
+                    const int np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
+                    const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
+                    if ((ballotX & needed) == 0ull) {
+                        const int cnt = np >= 0 ? np : WAVE;
+                        for (int d = 0; d < cnt; ++d) {
+                            const VT x = load_agent((const VT*)(gpayA + ((first - d) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) acc[j] = op(x[j], acc[j]);
+                        }
+                        if (np >= 0) {
+                            if (np >= rem) {                                // ran off the first group: nothing but init in front
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j) base[j] = op(init, acc[j]);
+                            } else {
+                                const VT x = load_agent((const VT*)(gpayP + ((first - np) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j) base[j] = op(x[j], acc[j]);   // a published prefix contains init
+                            }
+                            break;
+                        }
+                        first -= WAVE;
+                        rem -= WAVE;
+                        continue;
+                    }
+                    if (wait_give_up(wc, rounds)) break; // `base` is then meaningless
+                }
+                VT t;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) t[j] = base[j];
+                store_agent((VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC), t);
+                publish_barrier();
+                if (lane == 0) __hip_atomic_store(&gflag[(grp - 1) * nchains + chain], (uint64_t)tagP << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        } else {
+            // totals of the predecessors inside the group
+            T local[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) local[j] = ident;
+            for (;;) {
+                uint32_t st = DESC_A;
+                if (lane < r) {
+                    const uint32_t tag = (uint32_t)(__hip_atomic_load(&desc[(slice - 1 - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+                    st = tag == tagA ? DESC_A : 0u;
+                }
+                if (__ballot(st == 0u) == 0ull) break;
+                if (wait_give_up(wc, rounds)) break;
+            }
+            for (int d = 0; d < r; ++d) {
+                const VT x = load_agent((const VT*)(payload + ((slice - 1 - d) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) local[j] = op(x[j], local[j]);
+            }
+            if (r == ROWS_GROUP - 1 && has_reader) {     // aggregate of the whole group, as soon as it is known
+                VT t;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) t[j] = op(local[j], tot[j]);
+                store_agent((VT*)(gpayA + (grp * nchains + chain) * COLS + lane * VEC), t);
+                publish_barrier();
+                if (lane == 0) __hip_atomic_store(&gflag[grp * nchains + chain], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (grp > 0) {                               // the group's base, from its leader
+                for (;;) {
+                    uint32_t st = 0;
+                    if (lane == 0) st = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
+                    if (__builtin_amdgcn_readfirstlane((int)st) != 0) break;
+                    if (wait_give_up(wc, rounds)) break;
+                }
+                const VT x = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) base[j] = op(x[j], local[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) base[j] = op(init, local[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) lds_base[lane * VEC + j] = base[j];
+        __syncthreads();
+    } else {
+        const int64_t o = chain / strips, strip = chain - o * strips;
+        const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
+        const bool live = col0 < g.inner;                    // inner % VEC == 0: a vector is entirely inside or outside
+        const int64_t slab = o * g.inner * g.mid;
+        const int64_t row0 = slice * (NW * R) + (int64_t)wave * R;
+        VT v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (live && row0 + r < g.mid) {
+                const VI x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[r][j] = (T)x[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[r][j] = ident;
+            }
+        }
+#pragma unroll
+        for (int r = 1; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[r][j] = op(v[r - 1][j], v[r][j]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = v[R - 1][j];
+        __syncthreads();
+        T pre[VEC];                                          // the rows of the tile above this wave's
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            pre[j] = ident;
+            for (int w = 0; w < wave; ++w) pre[j] = op(pre[j], lds[w][lane * VEC + j]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) pre[j] = op(lds_base[lane * VEC + j], pre[j]);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (live && row0 + r < g.mid) {
+                VT o4;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o4[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r > 0 ? r - 1 : 0][j]));
+                store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o4);
+            }
+        }
+    }
+    // the helper wave's thread 0 would do as well; ordered_finish wants thread 0 of the workgroup, so hand it the epoch
+    __shared__ uint32_t lds_epoch;
+    if (wave == NW && lane == 0) lds_epoch = epoch;
+    __syncthreads();
+    ordered_finish(lds_epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
+}
+
 // ---- host side ---------------------------------------------------------------------------------------
 template <typename T, int K> struct ScanTile {     // geometry of the tile kernels: 256 threads x K x 16 bytes of output
     static constexpr int VEC = 16 / sizeof(T);
@@ -917,6 +1144,7 @@ long long wait_budget();        // rk_api.hip: poll rounds a bounded wait may sp
 inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_budget(), tune_scan_backoff()}; }
 int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
+int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
@@ -936,7 +1164,7 @@ struct ScanArgs {
 // the memory system serves faster than many rows far apart (measured with power-of-two row strides).
 template <typename In, typename T, typename Op>
 inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, bool aligned, char* scratch,
-                                size_t scratch_bytes, hipStream_t stream) {
+                                size_t scratch_bytes, hipStream_t stream, const Workspace* ws = nullptr) {
     constexpr int VEC = 16 / sizeof(T);
     const bool vec = aligned && (g.inner % VEC == 0);
     const int cols = WAVE * (vec ? VEC : 1);
@@ -944,6 +1172,21 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     if (strips * g.outer > 0x7fffffff) return RK_ERR_TOO_LARGE;
     const int64_t pitch = strips * cols;
     const int64_t cus = device_info().cus;
+    if constexpr (sizeof(T) <= 4) {
+        // single pass over tiles of 120 rows (7 waves of rows: 134 us against 109 for the 4096 x 16384 matrix); the payloads
+        // of all tiles and groups must fit the partials area
+        constexpr int NW = 15, R = 8;              // 15 waves of rows + 1 for the look-back
+        const int64_t nchains = strips * g.outer, nslices = (g.mid + NW * R - 1) / (NW * R), ntiles = nchains * nslices;
+        const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
+        if (vec && ws != nullptr && tune_scan_rows_ordered() != 0 && nchains < cus * 4 && nslices >= 4 &&
+            (size_t)((ntiles + 2 * ngroups) * cols) * sizeof(T) <= scratch_bytes && (size_t)(ntiles + ngroups) * sizeof(uint64_t) <= ws->desc_bytes) {
+            scan_rows_ordered_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
+                in, out, g, init, inclusive, op, strips, nchains, nslices, (T*)scratch, (unsigned long long*)&ws->hdr->scan_counter,
+                ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr));
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
+        }
+    }
     int64_t slices = 1;
     if (strips * g.outer < cus * 4) {
         const int64_t want = cus * tune_scan_slice_blocks_per_cu();
@@ -1074,8 +1317,9 @@ inline int32_t launch_scan(const ScanArgs& a) {
         Workspace w{};
         char* scratch = nullptr;
         size_t scratch_bytes = 0;
-        if (carve_workspace(a.ws, a.ws_bytes, 0, &w)) { scratch = (char*)w.partials; scratch_bytes = WS_PARTIALS_BYTES; }
-        return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream);
+        const bool have_ws = carve_workspace(a.ws, a.ws_bytes, 0, &w);
+        if (have_ws) { scratch = (char*)w.partials; scratch_bytes = WS_PARTIALS_BYTES; }
+        return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream, have_ws ? &w : nullptr);
     }
     const int64_t nlines = s.inner * s.outer;
     if (s.inner > 1 && s.mid > 64) {
@@ -1156,12 +1400,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const WaitCtl wc = wait_ctl(w.hdr);
     if constexpr (sizeof(T) <= 4) {
         if (!dynamic_ids) {
-            // exit tickets: at most half of the ticket lines, at least TICKET_GROUP workgroups a ticket
-            int64_t tg = (ntiles + (int64_t)WS_TICKET_COUNT / 2 - 1) / ((int64_t)WS_TICKET_COUNT / 2);
-            if (tg < TICKET_GROUP) tg = TICKET_GROUP;
+            const int tg = ordered_ticket_group(ntiles);
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
             scan_ordered_kernel<In, T, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
-                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, (int)tg, w.desc, gpl, ngroups, cap, wc)
+                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, tg, w.desc, gpl, ngroups, cap, wc)
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED
             RK_LAUNCH_CHECK();

@@ -19,8 +19,8 @@
 //                        down the tiles (the strided scan of the accumulate path) gives every tile its offsets.
 //   sort_finish_kernel   moves the result into the caller's array when an odd number of passes ran
 //
-// Keys are mapped to unsigned integers that sort like Base.isless (-0.0 < 0.0, NaN last; every NaN becomes the
-// canonical one), complemented for rev=true; the mapping is applied on the first read and undone on the last
+// Keys are mapped to unsigned integers that sort like Base.isless (-0.0 < 0.0, NaN last; sortperm makes every NaN the
+// canonical one so that they are equal keys, sort! keeps their bit patterns), complemented for rev=true; the mapping is applied on the first read and undone on the last
 // write.  The sort is stable, so sortperm keeps equal keys in index order (also with rev=true, as Base does).
 #include <cstddef>
 #include <cstdlib>
@@ -50,62 +50,89 @@ struct SortCtl {                                  // head of the caller's tempor
 template <typename T> struct SortKey;
 template <> struct SortKey<int16_t> {
     typedef uint16_t U;
-    static __device__ __forceinline__ U enc(int16_t v) { return (U)((uint16_t)v ^ 0x8000u); }
-    static __device__ __forceinline__ int16_t dec(U u) { return (int16_t)(u ^ 0x8000u); }
+    static __device__ __forceinline__ U enc(int16_t v, bool) { return (U)((uint16_t)v ^ 0x8000u); }
+    static __device__ __forceinline__ int16_t dec(U u, bool) { return (int16_t)(u ^ 0x8000u); }
 };
 template <> struct SortKey<int32_t> {
     typedef uint32_t U;
-    static __device__ __forceinline__ U enc(int32_t v) { return (U)v ^ 0x80000000u; }
-    static __device__ __forceinline__ int32_t dec(U u) { return (int32_t)(u ^ 0x80000000u); }
+    static __device__ __forceinline__ U enc(int32_t v, bool) { return (U)v ^ 0x80000000u; }
+    static __device__ __forceinline__ int32_t dec(U u, bool) { return (int32_t)(u ^ 0x80000000u); }
 };
 template <> struct SortKey<int64_t> {
     typedef uint64_t U;
-    static __device__ __forceinline__ U enc(int64_t v) { return (U)v ^ 0x8000000000000000ull; }
-    static __device__ __forceinline__ int64_t dec(U u) { return (int64_t)(u ^ 0x8000000000000000ull); }
+    static __device__ __forceinline__ U enc(int64_t v, bool) { return (U)v ^ 0x8000000000000000ull; }
+    static __device__ __forceinline__ int64_t dec(U u, bool) { return (int64_t)(u ^ 0x8000000000000000ull); }
+};
+// Floats: sign-magnitude bits -> unsigned integers in isless order (-0.0 < 0.0), NaN after +Inf.
+//   keep == false (sortperm: the keys are not part of the result): every NaN becomes the canonical one, so all NaNs
+//                 are equal keys and stay in index order, as isless-equal elements must in a stable sort.
+//   keep == true  (sort!): a bijection of the bit patterns, so the sorted array is a permutation of the input, NaN signs
+//                 and payloads included.  The plain mapping puts the negative NaNs below -Inf: NLOW of them, keys
+//                 0 .. NLOW-1; they are moved above the positive NaNs and everything else shifts down by NLOW.  The
+//                 order among NaNs is then by bit pattern, not by index (Base's own float sort moves its NaNs to the
+//                 end without keeping their order either).
+template <typename U, U NLOW> struct FloatKeyMap {
+    static __device__ __forceinline__ U fwd(U std_key) { return std_key < NLOW ? (U)(std_key + (U)(0 - NLOW)) : (U)(std_key - NLOW); }
+    static __device__ __forceinline__ U inv(U k) { return k >= (U)(0 - NLOW) ? (U)(k - (U)(0 - NLOW)) : (U)(k + NLOW); }
 };
 struct half_bits { uint16_t b; };                 // Float16 travels as its bit pattern
 template <> struct SortKey<half_bits> {
     typedef uint16_t U;
-    static __device__ __forceinline__ U enc(half_bits v) {
+    typedef FloatKeyMap<uint16_t, 0x03ffu> Map;    // 0xfc01 .. 0xffff are the negative NaNs
+    static __device__ __forceinline__ U enc(half_bits v, bool keep) {
         uint16_t b = v.b;
-        if ((b & 0x7fffu) > 0x7c00u) b = 0x7e00u;                 // NaN -> canonical, sorts after +Inf
-        return (U)((b & 0x8000u) ? ~b : (b ^ 0x8000u));
+        if (!keep && (b & 0x7fffu) > 0x7c00u) b = 0x7e00u;        // NaN -> canonical, sorts after +Inf
+        const U u = (U)((b & 0x8000u) ? ~b : (b ^ 0x8000u));
+        return keep ? Map::fwd(u) : u;
     }
-    static __device__ __forceinline__ half_bits dec(U u) { return half_bits{(uint16_t)((u & 0x8000u) ? (u ^ 0x8000u) : ~u)}; }
+    static __device__ __forceinline__ half_bits dec(U k, bool keep) {
+        const U u = keep ? Map::inv(k) : k;
+        return half_bits{(uint16_t)((u & 0x8000u) ? (u ^ 0x8000u) : ~u)};
+    }
 };
 template <> struct SortKey<float> {
     typedef uint32_t U;
-    static __device__ __forceinline__ U enc(float v) {
+    typedef FloatKeyMap<uint32_t, 0x007fffffu> Map;
+    static __device__ __forceinline__ U enc(float v, bool keep) {
         uint32_t b = __builtin_bit_cast(uint32_t, v);
-        if (v != v) b = 0x7fc00000u;
-        return (b & 0x80000000u) ? ~b : (b ^ 0x80000000u);
+        if (!keep && v != v) b = 0x7fc00000u;
+        const U u = (b & 0x80000000u) ? ~b : (b ^ 0x80000000u);
+        return keep ? Map::fwd(u) : u;
     }
-    static __device__ __forceinline__ float dec(U u) { return __builtin_bit_cast(float, (u & 0x80000000u) ? (u ^ 0x80000000u) : ~u); }
+    static __device__ __forceinline__ float dec(U k, bool keep) {
+        const U u = keep ? Map::inv(k) : k;
+        return __builtin_bit_cast(float, (u & 0x80000000u) ? (u ^ 0x80000000u) : ~u);
+    }
 };
 template <> struct SortKey<double> {
     typedef uint64_t U;
-    static __device__ __forceinline__ U enc(double v) {
+    typedef FloatKeyMap<uint64_t, 0x000fffffffffffffull> Map;
+    static __device__ __forceinline__ U enc(double v, bool keep) {
         uint64_t b = __builtin_bit_cast(uint64_t, v);
-        if (v != v) b = 0x7ff8000000000000ull;
-        return (b & 0x8000000000000000ull) ? ~b : (b ^ 0x8000000000000000ull);
+        if (!keep && v != v) b = 0x7ff8000000000000ull;
+        const U u = (b & 0x8000000000000000ull) ? ~b : (b ^ 0x8000000000000000ull);
+        return keep ? Map::fwd(u) : u;
     }
-    static __device__ __forceinline__ double dec(U u) {
+    static __device__ __forceinline__ double dec(U k, bool keep) {
+        const U u = keep ? Map::inv(k) : k;
         return __builtin_bit_cast(double, (u & 0x8000000000000000ull) ? (u ^ 0x8000000000000000ull) : ~u);
     }
 };
 
+// `rev` here is a set of flags: bit 0 = descending order, bit 1 = keep NaN bit patterns (SORT_KEEP_NAN).
+constexpr int SORT_REV = 1, SORT_KEEP_NAN = 2;
 // the same mapping on the raw bit pattern: one load path serves the first pass (caller's keys) and the later ones
 // and relative to the smallest mapped key of the array: small-range integers (and floats of one binade) then have
 // constant high digits, whose passes are skipped
 template <typename T> __device__ __forceinline__ typename SortKey<T>::U enc_bits(typename SortKey<T>::U raw, int rev, typename SortKey<T>::U umin) {
     typedef typename SortKey<T>::U U;
-    const U u = SortKey<T>::enc(__builtin_bit_cast(T, raw));
-    return (U)((rev ? (U)~u : u) - umin);
+    const U u = SortKey<T>::enc(__builtin_bit_cast(T, raw), (rev & SORT_KEEP_NAN) != 0);
+    return (U)(((rev & SORT_REV) ? (U)~u : u) - umin);
 }
 template <typename T> __device__ __forceinline__ T dec_bits(typename SortKey<T>::U k, int rev, typename SortKey<T>::U umin) {
     typedef typename SortKey<T>::U U;
     const U u = (U)(k + umin);
-    return SortKey<T>::dec(rev ? (U)~u : u);
+    return SortKey<T>::dec((rev & SORT_REV) ? (U)~u : u, (rev & SORT_KEEP_NAN) != 0);
 }
 
 template <typename U> __device__ __forceinline__ uint32_t digit_of(U u, int pass) { return (uint32_t)(u >> (8 * pass)) & 0xffu; }
@@ -365,7 +392,12 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
 
     for (uint32_t round = 0;; ++round) {
-        if (!COUNTED && tid == 0) lds_tile = atomicAdd(&ctl->ticket[pass], 1u);
+        if (!COUNTED && tid == 0) {
+            // once a look-back of this call has given up its wait the result is lost: no further tile starts
+            const uint32_t failed = __hip_atomic_load(&ctl->wait_failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t ticket = atomicAdd(&ctl->ticket[pass], 1u);
+            lds_tile = failed != 0u ? ntiles : ticket;
+        }
         for (int i = tid; i < SORT_NW * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
         __syncthreads();
         const uint32_t tile = COUNTED ? blockIdx.x + round * gridDim.x : lds_tile;
@@ -494,6 +526,10 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
                 if (FULL || q < valid_n) {
                     const U u = lds_keys[q];
                     const uint32_t slot = goff[digit_of(u, pass)] + q;
+                    // slot < n always holds in a sound sort.  After a look-back has given up its wait (WaitCtl) the
+                    // offsets are too small and this pass leaves holes; the next pass then reads keys the histograms
+                    // never counted, and its slots can lie anywhere: keep every store inside the arrays.
+                    if (slot >= n) continue;
                     if constexpr (PERM) {
                         if (last) perm_out[slot] = (int64_t)lds_vals[q] + 1;
                         else { dst[slot] = u; vdst[slot] = lds_vals[q]; }
@@ -662,7 +698,7 @@ static int32_t sort_dispatch(rk_dtype dt, void* keys, int64_t* perm_out, int64_t
     if (keys == nullptr || !is_aligned(keys, ks)) return RK_ERR_INVALID_ARGUMENT;
     if (n >= ((int64_t)1 << 31)) return RK_ERR_TOO_LARGE;
     hipStream_t st = (hipStream_t)stream;
-    const int r = rev ? 1 : 0;
+    const int r = (rev ? SORT_REV : 0) | (perm_out == nullptr ? SORT_KEEP_NAN : 0);
     switch ((int)dt) {
         case RK_F32: return sort_typed<float>(keys, perm_out, n, r, tmp, tmp_bytes, st);
         case RK_F64: return sort_typed<double>(keys, perm_out, n, r, tmp, tmp_bytes, st);

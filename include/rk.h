@@ -342,9 +342,10 @@ RK_API int32_t rk_permutedims(const void* src, void* dst, size_t elsize, int ndi
  * Replace AK.sort! / AK.sortperm! behind  src/kernels/sorting.jl:1-3  for the default order
  * (`lt = isless`, `by = identity`) and `rev`; custom `lt` / `by` closures cannot cross a C ABI
  * (the caller keeps its own path for them).  Element types: Float16/32/64, Int16/32/64 (the types
- * of test/hip_rocarray/sorting.jl).  Order = Base.isless: -0.0 before 0.0, NaN last (every NaN
- * comes back as the canonical NaN).  Stable: sortperm keeps equal keys in index order, also with
- * rev != 0, like Base.
+ * of test/hip_rocarray/sorting.jl).  Order = Base.isless: -0.0 before 0.0, NaN last.  The sorted
+ * array is a permutation of the input bit for bit: NaNs keep sign and payload (their order among
+ * themselves is by bit pattern).  Stable: sortperm keeps equal keys -- all NaNs count as equal --
+ * in index order, also with rev != 0, like Base.
  *   rk_sort      sorts `keys` in place.
  *   rk_sortperm  leaves `keys` untouched and writes the 1-based permutation (Int64) to
  *                `perm_out`; unlike `sortperm!(ix, x)` it does not read an initial `ix`

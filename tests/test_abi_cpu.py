@@ -42,7 +42,7 @@ def test_only_c_abi_symbols_are_public(L):
 
 def test_header_constants_match_binding(L):
     text = open(HEADER).read()
-    for name in ("RK_ERR_INVALID_ARGUMENT", "RK_ERR_UNSUPPORTED", "RK_ERR_WORKSPACE", "RK_ERR_DIMENSION", "RK_ERR_TOO_LARGE"):
+    for name in ("RK_ERR_INVALID_ARGUMENT", "RK_ERR_UNSUPPORTED", "RK_ERR_WORKSPACE", "RK_ERR_DIMENSION", "RK_ERR_TOO_LARGE", "RK_ERR_WAIT"):
         assert int(re.search(name + r"\s*=\s*(\d+)", text).group(1)) == getattr(L, name)
     assert int(re.search(r"#define RK_MAX_DIMS (\d+)", text).group(1)) == L.RK_MAX_DIMS
     assert int(re.search(r"#define RK_MAX_OPERANDS (\d+)", text).group(1)) == L.RK_MAX_OPERANDS
@@ -54,7 +54,7 @@ def test_header_constants_match_binding(L):
 
 def test_status_strings(L):
     assert L.lib.rk_status_string(0) == b"RK_SUCCESS"
-    for code in (L.RK_ERR_INVALID_ARGUMENT, L.RK_ERR_UNSUPPORTED, L.RK_ERR_WORKSPACE, L.RK_ERR_DIMENSION, L.RK_ERR_TOO_LARGE):
+    for code in (L.RK_ERR_INVALID_ARGUMENT, L.RK_ERR_UNSUPPORTED, L.RK_ERR_WORKSPACE, L.RK_ERR_DIMENSION, L.RK_ERR_TOO_LARGE, L.RK_ERR_WAIT):
         assert L.lib.rk_status_string(code).startswith(b"RK_ERR_")
     assert L.lib.rk_status_string(424242) == b"unknown rk status"
 
@@ -234,6 +234,28 @@ def test_workspace_queries(L):
     assert wi(None, 1 << 24, None) == L.RK_ERR_INVALID_ARGUMENT
     assert wi(C.c_void_p(0x1001), 1 << 24, None) == L.RK_ERR_WORKSPACE
     assert wi(C.c_void_p(0x1000), 1024, None) == L.RK_ERR_WORKSPACE
+
+
+def test_long_outer_extents_are_not_rejected(L):
+    """Shapes whose outer extent exceeds 65535 (the y / z limit of a grid) pass validation and planning: with no device
+    the call then stops at the launch with a HIP error, never with RK_ERR_TOO_LARGE.  Only meaningful -- and only safe,
+    the pointers are made up -- on a machine without a GPU; the GPU suite runs the same shapes on real arrays."""
+    import torch
+    if torch.cuda.device_count() > 0:
+        pytest.skip("a device is present: the same shapes run for real in tests/test_large_gpu.py")
+    ws, A, R = C.c_void_p(0x10000000), C.c_void_p(0x20000000), C.c_void_p(0x30000000)
+    for shape in ((64, 2, 70000), (64, 5, 70000), (100, 3, 111848), (256, 2, 65536)):
+        for dt in (L.RK_F32, L.RK_F64, L.RK_I32):
+            st = L.lib.rk_mapreduce(L.RK_MAP_IDENTITY, L.RK_OP_ADD, dt, dt, A, 3, L.shape_array(shape), 2, R, None, ws, 16 << 20, None)
+            assert 0 < st < 10000, (shape, dt, st)                      # a hipError_t: no device
+        st = L.lib.rk_findminmax(1, L.RK_F32, A, 3, L.shape_array(shape), 2, R, None, ws, 16 << 20, None)
+        assert 0 < st < 10000, (shape, st)
+    for shape in ((64, 64, 70000), (1000, 3, 112625), (2048, 4, 100000)):
+        st = L.lib.rk_accumulate(L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, R, 3, L.shape_array(shape), 2, 1, None, ws, 16 << 20, None)
+        assert 0 < st < 10000, (shape, st)
+    # a U8 -> I64 scan is sized by its OUTPUT type: two descriptor words per tile
+    shp = L.shape_array((1 << 27,))
+    assert L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, L.RK_I64, 1, shp, 1) > L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, L.RK_I32, 1, shp, 1)
 
 
 def test_host_mirror_rules_without_gpu(rk):

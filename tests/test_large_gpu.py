@@ -59,3 +59,34 @@ def test_broadcast_reverse_findall_beyond_2_31(rk):
     torch.cuda.empty_cache()
     idx = rk.Array(rk.findall(_wrap(rk, m, np.bool_)))
     assert np.array_equal(idx, np.arange(5, N, 1 << 20, dtype=np.int64) + 1)
+
+
+# Outer extents beyond 65535 (the limit of a grid's y and z axes) with lanes along the first dim: the shapes an
+# earlier version refused with RK_ERR_TOO_LARGE.  Small arrays, checked against the oracle.
+LONG_OUTER = [(64, 2, 70000), (64, 5, 70000), (100, 3, 111848), (256, 2, 65536)]
+
+
+@pytest.mark.parametrize("shape", LONG_OUTER)
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32])
+def test_reduce_dims2_long_outer(rk, orc, shape, dtype):
+    rng = np.random.default_rng(sum(shape))
+    h = (rng.standard_normal(shape) * 100).astype(dtype)
+    d = rk.ROCArray(h)
+    got = rk.Array(rk.sum(d, dims=2))
+    want = orc.mapreduce("identity", "add", h, dims=2)
+    if np.dtype(dtype).kind == "f":
+        np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-3 if dtype == np.float32 else 1e-9)
+    else:
+        assert np.array_equal(got, want)
+    v, i = rk.findmax(d, dims=2)
+    ov, oi = orc.findmax(h, dims=2)
+    assert np.array_equal(rk.Array(v), ov)
+    assert np.array_equal(np.moveaxis(rk.Array(i), 0, -1), oi)
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 70000), (1000, 3, 112625), (2048, 4, 100000), (64, 300, 66000)])
+def test_accumulate_dims2_long_outer(rk, orc, shape):
+    rng = np.random.default_rng(sum(shape))
+    h = rng.integers(-1000, 1001, shape, dtype=np.int32)
+    got = rk.Array(rk.cumsum(rk.ROCArray(h), dims=2))
+    assert np.array_equal(got, orc.accumulate("add", h, dims=2))

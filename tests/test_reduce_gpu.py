@@ -428,3 +428,34 @@ def test_two_step_fold_that_does_not_fit(rk, orc):
     dx = rk.ROCArray(x)
     assert np.array_equal(rk.Array(rk.maximum(dx, dims=(1, 3))), x.max(axis=(0, 2), keepdims=True))
     np.testing.assert_allclose(rk.Array(rk.sum(dx, dims=(1, 3))), x.sum(axis=(0, 2), keepdims=True, dtype=np.float64), rtol=1e-5, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype,utype", [(np.float32, np.uint32), (np.float64, np.uint64), (np.float16, np.uint16)])
+def test_findmax_findmin_return_the_nan_itself(rk, dtype, utype):
+    # Julia returns the winning ELEMENT: a negative NaN or one with a payload comes back bit for bit (the first NaN wins)
+    bits = {np.float32: (0xffc00001, 0x7fc12345, 0x7f800001), np.float64: (0xfff8000000000001, 0x7ff8000000abcdef, 0x7ff0000000000001),
+            np.float16: (0xfe01, 0x7e55, 0x7c01)}[dtype]
+    rng = _rng(77)
+    for shape, dims in (((5000,), None), ((300, 40), 1), ((300, 40), 2), ((6, 70000), 1)):
+        h = rng.standard_normal(shape).astype(dtype)
+        u = h.view(utype).reshape(-1)
+        pos = rng.choice(u.size, 3, replace=False)
+        for p_, b in zip(pos, bits):
+            u[p_] = b
+        d = rk.ROCArray(h)
+        for fn in (rk.findmax, rk.findmin):
+            if dims is None:
+                v, i = fn(d)
+                first = int(np.flatnonzero(np.isnan(h.reshape(-1)))[0])
+                assert int(i) == first + 1
+                assert np.array(v, dtype=dtype).view(utype) == h.reshape(-1).view(utype)[first]
+            else:
+                v, i = fn(d, dims=dims)
+                gv = rk.Array(v)
+                gi = np.moveaxis(rk.Array(i), 0, -1).reshape(-1, 2) - 1
+                picked = h[gi[:, 0], gi[:, 1]]
+                assert np.array_equal(gv.reshape(-1).view(utype), picked.view(utype))       # value == A[index], bit for bit
+                ax = dims - 1
+                has_nan = np.isnan(h).any(axis=ax)
+                first_nan = np.argmax(np.isnan(h), axis=ax)
+                assert np.array_equal(gi[:, ax][has_nan.reshape(-1)], first_nan.reshape(-1)[has_nan.reshape(-1)])

@@ -107,3 +107,38 @@ def test_unsupported_forms(rk):
     with pytest.raises(rk.UnsupportedError):
         rk.sort(rk.ROCArray(np.zeros(5, dtype=np.uint8)))
     assert len(rk.sort(rk.ROCArray(np.zeros(0, dtype=np.float32)))) == 0
+
+
+@pytest.mark.parametrize("dtype,utype", [(np.float32, np.uint32), (np.float64, np.uint64), (np.float16, np.uint16)])
+@pytest.mark.parametrize("rev", [False, True])
+def test_sort_keeps_nan_bit_patterns(rk, dtype, utype, rev):
+    # sort!: the result is a permutation of the input bit for bit -- negative NaNs and payloads survive -- with the
+    # non-NaN part in isless order and every NaN after it (before it with rev); sortperm: NaNs are equal keys, index order
+    rng = np.random.default_rng(99)
+    n = 300_000
+    h = rng.standard_normal(n).astype(dtype)
+    u = h.view(utype)
+    nan_bits = {np.float32: [0xffc00001, 0x7fc12345, 0x7f800001, 0xff800001, 0x7fffffff, 0x7fc00000],
+                np.float64: [0xfff8000000000001, 0x7ff8000000abcdef, 0x7ff0000000000001, 0xfff0000000000001, 0x7fffffffffffffff, 0x7ff8000000000000],
+                np.float16: [0xfe01, 0x7e55, 0x7c01, 0xfc01, 0x7fff, 0x7e00]}[dtype]
+    pos = rng.choice(n, 600, replace=False)
+    for k, p_ in enumerate(pos):
+        u[p_] = nan_bits[k % len(nan_bits)]
+    h[rng.choice(n, 50)] = np.inf
+    h[rng.choice(n, 50)] = -np.inf
+    h[rng.choice(n, 50)] = -0.0
+    d = rk.ROCArray(h.copy())
+    rk.sort_(d, rev=rev)
+    got = rk.Array(d)
+    assert np.array_equal(np.sort(got.view(utype)), np.sort(h.view(utype)))            # a permutation of the bits
+    nn = int(np.isnan(h).sum())
+    body = got[nn:] if rev else got[:n - nn]
+    tail = got[:nn] if rev else got[n - nn:]
+    assert np.isnan(tail).all() and not np.isnan(body).any()
+    want = np.sort(h[~np.isnan(h)])
+    want = want[::-1] if rev else want
+    assert np.array_equal(body, want) and np.array_equal(np.signbit(body), np.signbit(want))
+    perm = rk.Array(rk.sortperm(rk.ROCArray(h), rev=rev)) - 1
+    nan_part = perm[:nn] if rev else perm[n - nn:]
+    assert np.array_equal(nan_part, np.flatnonzero(np.isnan(h)))                          # stable among the NaNs
+    assert np.array_equal(np.sort(perm), np.arange(n))
