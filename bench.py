@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ROCArray array-kernel path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--no-cpu] [--only SUBSTRING]
 
 Prints ONE JSON line.  A *step* is one pass of the headline workload named by the metric -- sum over a
 Float32 vector, eltype-preserving cumsum over an Int32 vector and the fused broadcast
@@ -9,10 +9,20 @@ z .= a .* x .+ y .* exp.(w), each on 2^26 elements -- with every input already r
 `value` = algorithmic bytes of the K timed steps / their wall time (GB/s), measured between two stream
 synchronisations; the buffers of consecutive steps rotate so that no step finds its input in the 256 MB
 Infinity Cache.  `roofline` is the dominant kernel of the step (the broadcast: 16 of the 28 bytes per
-element), timed with HIP events on the launch stream.  `configs` lists every BASELINE configuration at
-its own size (elements/s, GB/s, fraction of the 8 TB/s HBM peak; minimum and mean of the timed repeats).
-`cpu_baseline` times the C restatement of Julia Base (oracle/oracle_c.c, kind "port": no Julia runtime
-exists on this machine) on the host cores for the same step.
+element): algorithmic bytes / average launch duration over K back-to-back launches, HIP events on the
+launch stream.
+
+`configs` lists every BASELINE configuration at its own size, calibration rows (read-only, write-only and
+copy kernels through the same entry points: the practical ceilings of the device) and a few extra shapes.
+Per row, the PRIMARY figure (`min_us`, `GBps`, `frac_hbm`, `elements_per_s`) is the minimum over individually
+synchronised launches -- the protocol of the reference's own benchmarks (perf/runbenchmarks.jl:18-23,81-86);
+`batch_avg_us` / `GBps_batch` is the average of the same number of launches issued back to back (tails overlap
+heads, so it is the smaller time for short kernels).  `cpu` beside a row is the C restatement of Julia Base
+(oracle/oracle_c.c, kind "port": no Julia runtime exists on this machine) timed on the host cores for the same
+operation on a bounded sample; `cpu_baseline` is the same for the whole headline step.
+
+Every row runs inside a roctx range named like the row, so a `rocprofv3 --kernel-trace --marker-trace` run
+can be summarised per row (bench_trace_summary.py).
 """
 from __future__ import annotations
 
@@ -39,8 +49,32 @@ def parse():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
-    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    p.add_argument("--only", default=None,
+                   help="run only the rows whose name contains this text ('|' separates alternatives); skips the headline step")
     return p.parse_args()
+
+
+class Roctx:
+    """roctx ranges (no-ops when the library is missing): rocprofv3 --marker-trace records them."""
+
+    def __init__(self):
+        self.lib = None
+        for name in ("librocprofiler-sdk-roctx.so", "libroctx64.so"):
+            try:
+                self.lib = C.CDLL(os.path.join("/opt/rocm/lib", name))
+                self.lib.roctxRangePushA.argtypes = [C.c_char_p]
+                break
+            except OSError:
+                self.lib = None
+
+    def push(self, name: str):
+        if self.lib is not None:
+            self.lib.roctxRangePushA(name.encode())
+
+    def pop(self):
+        if self.lib is not None:
+            self.lib.roctxRangePop()
 
 
 def main():
@@ -57,6 +91,7 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
+    roctx = Roctx()
 
     def dev_array(t: "torch.Tensor", dims, dtype):
         """Wrap a device tensor produced by torch's generators as a ROCArray (no copy)."""
@@ -75,326 +110,427 @@ def main():
         return torch.randint(-1000, 1001, (n,), device=dev, generator=gen, dtype=torch.int32)
 
     def time_launches(fn, reps, warm=3):
-        """Average / minimum duration (ms) of `fn(i)` launches, HIP events on the launch stream."""
+        """(minimum of individually synchronised launches, average of back-to-back launches), both in ms;
+        HIP events on the launch stream (the library launches on torch's current stream)."""
         for i in range(warm):
             fn(i)
         torch.cuda.synchronize()
-        # whole batch between two events: average launch-to-launch time with a saturated queue
+        best = float("inf")
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(reps):
+            a.record()
+            fn(i)
+            b.record()
+            b.synchronize()
+            best = min(best, a.elapsed_time(b))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for i in range(reps):
             fn(i)
         e1.record()
         torch.cuda.synchronize()
-        avg = e0.elapsed_time(e1) / reps
-        # individual launches: minimum (the reference reports the minimum, perf/runbenchmarks.jl:81-86)
-        best = float("inf")
-        for i in range(min(reps, 20)):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            fn(i)
-            b.record()
-            b.synchronize()
-            best = min(best, a.elapsed_time(b))
-        return avg, best
+        return best, e0.elapsed_time(e1) / reps
 
-    # ---- headline step: sum f32 + cumsum i32 + broadcast, 2^26 elements each --------------------------
-    n = N_HEAD
-    ROT = 3
-    sum_in = [dev_array(rand_f32(n), (n,), np.float32) for _ in range(ROT)]
-    sum_out = rk.ROCArray(dims=(1,), dtype=np.float32)
-    scan_in = [dev_array(randint_i32(n), (n,), np.int32) for _ in range(ROT)]
-    scan_out = [rk.ROCArray(dims=(n,), dtype=np.int32) for _ in range(ROT)]
-    bx = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
-    by = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
-    bw = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
-    bz = [rk.ROCArray(dims=(n,), dtype=np.float32) for _ in range(2)]
-    a = np.float32(0.5)
-    exprs = [a * L(bx[i]) + L(by[i]) * rk.broadcast.exp(L(bw[i])) for i in range(2)]
+    # ---- CPU side: the C restatement of Julia Base, timed on the host cores ------------------------------------
+    cpu_lib = None
+    threads = max(1, min(16, os.cpu_count() or 1))
+    host = {}
+    if not args.no_cpu:
+        so = os.path.join(ROOT, "oracle", "liboracle_c.so")
+        if os.path.exists(so):
+            cpu_lib = C.CDLL(so)
+            cpu_lib.orc_sum_f32.restype = C.c_double
+            cpu_lib.orc_sum_i32.restype = C.c_int64
+            cpu_lib.orc_maximum_f32.restype = C.c_float
+            rng = np.random.default_rng(0)
+            n = N_HEAD
+            host["x"] = rng.random(n, dtype=np.float32)
+            host["y"] = rng.standard_normal(n, dtype=np.float32)
+            host["w"] = rng.standard_normal(n, dtype=np.float32)
+            host["i"] = rng.integers(-1000, 1001, n, dtype=np.int32)
+            host["z"] = np.empty(n, dtype=np.float32)
+            host["io"] = np.empty(n, dtype=np.int32)
 
-    # prepared calls: arguments are validated and marshalled once, the timed loop only makes the foreign
-    # call (what a compiled `ccall` site costs in the Julia shim)
+    def P(a):
+        return C.c_void_p(a.ctypes.data)
+
+    def cpu_row(fn, nbytes, sample, reps1=1, repsn=3):
+        """fn(threads) runs the operation once; best-of timing single-threaded and on `threads` cores."""
+        if cpu_lib is None:
+            return None
+
+        def best(t, reps):
+            fn(t)
+            b = float("inf")
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn(t)
+                b = min(b, time.perf_counter() - t0)
+            return b
+        t1 = best(1, reps1)
+        tn = best(threads, repsn) if threads > 1 else t1
+        return {"GBps": round(nbytes / tn / 1e9, 2), "cores": threads, "single_thread_GBps": round(nbytes / t1 / 1e9, 2),
+                "sample": sample}
+
+    I64 = C.c_int64
+    configs = []
+
+    def wanted(name):
+        return args.only is None or any(part in name for part in args.only.split("|"))
+
+    def entry(name, elems, nbytes, min_ms, batch_ms, cpu=None, **extra):
+        gbs = nbytes / (min_ms * 1e-3) / 1e9
+        e = {"op": name, "elements": elems, "bytes": nbytes, "min_us": round(min_ms * 1e3, 2),
+             "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "elements_per_s": elems / (min_ms * 1e-3),
+             "batch_avg_us": round(batch_ms * 1e3, 2), "GBps_batch": round(nbytes / (batch_ms * 1e-3) / 1e9, 1)}
+        if cpu is not None:
+            e["cpu"] = cpu
+        e.update(extra)
+        return e
+
+    def run_row(name, elems, nbytes, fn, reps, cpu=None, **extra):
+        if not wanted(name):
+            return None
+        roctx.push(name)
+        best, batch = time_launches(fn, reps)
+        roctx.pop()
+        c = cpu() if (cpu is not None and cpu_lib is not None) else None
+        e = entry(name, elems, nbytes, best, batch, c, **extra)
+        configs.append(e)
+        return e
+
     from amdgpu_jl_amd.mapreduce import plan_mapreducedim, plan_findmax
     from amdgpu_jl_amd.accumulate import plan_accumulate
     from amdgpu_jl_amd.broadcast import plan_materialize
     from amdgpu_jl_amd.volumerhs import plan_volumerhs
     from amdgpu_jl_amd import _lib as RL
     from amdgpu_jl_amd.array import workspace, stream_ptr
-    p_sum = [plan_mapreducedim(rk.identity, rk.add, sum_out, x) for x in sum_in]
-    p_scan = [plan_accumulate("add", o, x) for o, x in zip(scan_out, scan_in)]
-    p_bc = [plan_materialize(bz[i], exprs[i]) for i in range(2)]
 
-    def op_sum(i):
-        p_sum[i % ROT]()
-
-    def op_scan(i):
-        p_scan[i % ROT]()
-
-    def op_bcast(i):
-        p_bc[i % 2]()
-
-    def step(i):
-        op_sum(i)
-        op_scan(i)
-        op_bcast(i)
-
+    # ---- headline step: sum f32 + cumsum i32 + broadcast, 2^26 elements each --------------------------
+    n = N_HEAD
+    ROT = 3
+    a = np.float32(0.5)
     bytes_sum, bytes_scan, bytes_bc = 4 * n, 8 * n, 16 * n
     step_bytes = bytes_sum + bytes_scan + bytes_bc
+    value = ms_per_step = None
+    roofline = None
+    cpu_step = None
+    HEAD_ROWS = ("sum Float32[2^26]", "maximum Float32[2^26]", "cumsum Int32[2^26]", "z .= a.*x .+ y.*exp.(w) Float32[2^26]",
+                 "calibration: copy z .= x Float32[2^26]", "calibration: fill z .= 1.5f0 Float32[2^26]")
+    if args.only is None or any(wanted(r) for r in HEAD_ROWS):
+        sum_in = [dev_array(rand_f32(n), (n,), np.float32) for _ in range(ROT)]
+        sum_out = rk.ROCArray(dims=(1,), dtype=np.float32)
+        scan_in = [dev_array(randint_i32(n), (n,), np.int32) for _ in range(ROT)]
+        scan_out = [rk.ROCArray(dims=(n,), dtype=np.int32) for _ in range(ROT)]
+        bx = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+        by = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+        bw = [dev_array(randn_f32(n), (n,), np.float32) for _ in range(2)]
+        bz = [rk.ROCArray(dims=(n,), dtype=np.float32) for _ in range(2)]
+        exprs = [a * L(bx[i]) + L(by[i]) * rk.broadcast.exp(L(bw[i])) for i in range(2)]
+        # prepared calls: arguments are validated and marshalled once, the timed loop only makes the foreign
+        # call (what a compiled `ccall` site costs in the Julia shim)
+        p_sum = [plan_mapreducedim(rk.identity, rk.add, sum_out, x) for x in sum_in]
+        p_max = [plan_mapreducedim(rk.identity, rk.max_, sum_out, x) for x in sum_in]
+        p_scan = [plan_accumulate("add", o, x) for o, x in zip(scan_out, scan_in)]
+        p_bc = [plan_materialize(bz[i], exprs[i]) for i in range(2)]
+        p_copy = [plan_materialize(bz[i], L(bx[i])) for i in range(2)]
+        p_fill = [plan_materialize(bz[i], L(np.float32(1.5))) for i in range(2)]
 
-    for i in range(W):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        step(i)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / K
-    value = step_bytes / (wall / K) / 1e9
+        def op_sum(i):
+            p_sum[i % ROT]()
 
-    # plain copy z .= x through the same broadcast entry point: the practical read+write ceiling of the
-    # device, and the kernel of known traffic that calibrates the FETCH_SIZE / WRITE_SIZE counters
-    p_copy = [plan_materialize(bz[i], L(bx[i])) for i in range(2)]
-    copy_avg, copy_min = time_launches(lambda i: p_copy[i % 2](), K)
-    del p_copy
+        def op_scan(i):
+            p_scan[i % ROT]()
 
-    bc_avg, bc_min = time_launches(op_bcast, K)
-    sum_avg, sum_min = time_launches(op_sum, K)
-    scan_avg, scan_min = time_launches(op_scan, K)
+        def op_bcast(i):
+            p_bc[i % 2]()
 
-    def entry(name, elems, nbytes, avg_ms, min_ms, **extra):
-        gbs = nbytes / (avg_ms * 1e-3) / 1e9
-        e = {"op": name, "elements": elems, "bytes": nbytes, "avg_us": round(avg_ms * 1e3, 2), "min_us": round(min_ms * 1e3, 2),
-             "elements_per_s": elems / (avg_ms * 1e-3), "GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
-             "GBps_best": round(nbytes / (min_ms * 1e-3) / 1e9, 1)}
-        e.update(extra)
-        return e
+        def step(i):
+            op_sum(i)
+            op_scan(i)
+            op_bcast(i)
 
-    configs = [
-        entry("sum Float32[2^26]", n, bytes_sum, sum_avg, sum_min),
-        entry("cumsum Int32[2^26]", n, bytes_scan, scan_avg, scan_min),
-        entry("z .= a.*x .+ y.*exp.(w) Float32[2^26]", n, bytes_bc, bc_avg, bc_min),
-        entry("copy z .= x Float32[2^26] (device read+write ceiling, counter calibration)", n, 8 * n, copy_avg, copy_min),
-    ]
-    roofline = {"bound": "hbm", "kernel": "bc_kernel<EvalAxpbyExp,float,4,linear> (z .= a.*x .+ y.*exp.(w), 2^26 elts)",
-                "achieved": round(bytes_bc / (bc_avg * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(bytes_bc / (bc_avg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/headline_step_pmc_fetch_write.txt):
-                # (393238.3 KiB x 1.9999 + 262144.0 KiB x 0.9986), factors from the plain copy kernel of the same runs
-                "traffic": TRAFFIC_BC_2_26 if n == N_HEAD else None,
-                "bytes_per_launch": bytes_bc, "avg_launch_us": round(bc_avg * 1e3, 2)}
+        if args.only is None:
+            roctx.push("headline step (sum + cumsum + broadcast, 2^26)")
+            for i in range(W):
+                step(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(K):
+                step(i)
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+            roctx.pop()
+            ms_per_step = wall * 1e3 / K
+            value = step_bytes / (wall / K) / 1e9
 
-    del sum_in, scan_in, scan_out, bx, by, bw, bz, exprs, p_sum, p_scan, p_bc
-    torch.cuda.empty_cache()
+            # the dominant kernel: average duration over K back-to-back launches (what a kernel trace averages, too)
+            roctx.push("roofline kernel: z .= a.*x .+ y.*exp.(w) Float32[2^26], back to back")
+            _, bc_avg = time_launches(op_bcast, K)
+            roctx.pop()
+            roofline = {"bound": "hbm", "kernel": "bc_kernel<EvalAxpbyExp,float,4,linear> (z .= a.*x .+ y.*exp.(w), 2^26 elts)",
+                        "achieved": round(bytes_bc / (bc_avg * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": round(bytes_bc / (bc_avg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/headline_step_pmc_fetch_write.txt):
+                        # (393238.3 KiB x 1.9999 + 262144.0 KiB x 0.9986), factors from the plain copy kernel of the same runs
+                        "traffic": TRAFFIC_BC_2_26,
+                        "bytes_per_launch": bytes_bc, "avg_launch_us": round(bc_avg * 1e3, 2)}
+
+            if cpu_lib is not None:
+                hx, hy, hw, hi, hz, ho = (host[k] for k in ("x", "y", "w", "i", "z", "io"))
+
+                def cpu_step_fn(t):
+                    cpu_lib.orc_sum_f32(P(hx), I64(n), t)
+                    cpu_lib.orc_cumsum_i32(P(hi), I64(n), P(ho))
+                    cpu_lib.orc_bcast_axpby_exp_f32(C.c_float(0.5), P(hx), P(hy), P(hw), P(hz), I64(n), t)
+                c = cpu_row(cpu_step_fn, step_bytes, "", reps1=1, repsn=3)
+                cpu_step = {"value": c["GBps"], "unit": "GB/s", "cores": c["cores"], "kind": "port",
+                            "single_thread_GBps": c["single_thread_GBps"],
+                            "sample": "the same step (sum Float32 + accumulate(+) Int32 + z .= a.*x .+ y.*exp.(w), 2^26 elements each), "
+                                      "minimum of 3 runs of oracle/oracle_c.c with OpenMP on `cores` threads (the Int32 scan is sequential, "
+                                      "as in Julia Base); Julia itself is not installed on this machine, so this is the C port of Base's "
+                                      "algorithms (JULIA_NUM_THREADS does not apply; Base's sum/accumulate/broadcast are single-threaded: "
+                                      "see single_thread_GBps)"}
+
+        if not args.no_configs:
+            reps = max(10, min(K, 30))
+            hx = host.get("x")
+            run_row("sum Float32[2^26]", n, bytes_sum, op_sum, reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_sum_f32(P(hx), I64(n), t), bytes_sum, "full size"))
+            run_row("maximum Float32[2^26]", n, bytes_sum, lambda i: p_max[i % ROT](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_maximum_f32(P(hx), I64(n), t), bytes_sum, "full size"))
+            run_row("cumsum Int32[2^26]", n, bytes_scan, op_scan, reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_i32(P(host["i"]), I64(n), P(host["io"])), bytes_scan,
+                                        "full size; sequential (threads do not apply)", repsn=1))
+            run_row("z .= a.*x .+ y.*exp.(w) Float32[2^26]", n, bytes_bc, op_bcast, reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_bcast_axpby_exp_f32(C.c_float(0.5), P(hx), P(host["y"]), P(host["w"]), P(host["z"]), I64(n), t),
+                                        bytes_bc, "full size"))
+            # calibration: the simplest kernels through the same entry points = what this device delivers for each traffic mix
+            run_row("calibration: copy z .= x Float32[2^26] (1 read + 1 write; FETCH/WRITE counter calibration)", n, 8 * n,
+                    lambda i: p_copy[i % 2](), reps)
+            run_row("calibration: fill z .= 1.5f0 Float32[2^26] (write only)", n, 4 * n, lambda i: p_fill[i % 2](), reps)
+        del sum_in, scan_in, scan_out, bx, by, bw, bz, exprs, p_sum, p_max, p_scan, p_bc, p_copy, p_fill
+        torch.cuda.empty_cache()
 
     # ---- every BASELINE configuration at its own size ------------------------------------------------------
     if not args.no_configs:
         reps = max(10, min(K, 30))
+        hx, hi = host.get("x"), host.get("i")
 
-        def run_cfg(name, elems, nbytes, fn, **extra):
-            avg, best = time_launches(fn, reps)
-            configs.append(entry(name, elems, nbytes, avg, best, **extra))
-
-        # cfg 1: full sums (2^24 fits the Infinity Cache: rotate 8 buffers = 512 MiB)
-        for logn, rot in ((24, 8), (28, 2)):
-            m = 1 << logn
-            xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(rot)]
+        # calibration at 2^28: read only (sum), write only (fill), copy
+        if wanted("2^28"):
+            m = 1 << 28
+            xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(2)]
+            zs = rk.ROCArray(dims=(m,), dtype=np.float32)
             r = rk.ROCArray(dims=(1,), dtype=np.float32)
             ps = [plan_mapreducedim(rk.identity, rk.add, r, x) for x in xs]
-            run_cfg(f"cfg1a sum Float32[2^{logn}]", m, 4 * m, lambda i: ps[i % rot]())
+            run_row("cfg1a sum Float32[2^28] (calibration: read only)", m, 4 * m, lambda i: ps[i % 2](), reps)
+            pc = [plan_materialize(zs, L(x)) for x in xs]
+            run_row("calibration: copy z .= x Float32[2^28]", m, 8 * m, lambda i: pc[i % 2](), reps)
+            pf = plan_materialize(zs, L(np.float32(1.5)))
+            run_row("calibration: fill z .= 1.5f0 Float32[2^28] (write only)", m, 4 * m, lambda i: pf(), reps)
+            # f as a closure, traced into a program the reduction kernels interpret (perf/array.jl:107-122)
+            pp = [plan_mapreducedim(lambda v: v + 1, rk.add, r, x) for x in xs]
+            run_row("mapreduce(x -> x + 1, +, Float32[2^28])", m, 4 * m, lambda i: pp[i % 2](), reps)
+            del xs, zs, ps, pc, pf, pp
+            torch.cuda.empty_cache()
+        # cfg 1: full sums (2^24 fits the Infinity Cache: rotate 8 buffers = 512 MiB)
+        if wanted("cfg1"):
+            m = 1 << 24
+            xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(8)]
+            r = rk.ROCArray(dims=(1,), dtype=np.float32)
+            ps = [plan_mapreducedim(rk.identity, rk.add, r, x) for x in xs]
+            run_row("cfg1a sum Float32[2^24]", m, 4 * m, lambda i: ps[i % 8](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_sum_f32(P(hx), I64(m), t), 4 * m, "full size", reps1=3))
             del xs, ps
-        # f as a closure, traced into a program the reduction kernels interpret (perf/array.jl:107-122)
-        m = 1 << 28
-        xs = [dev_array(rand_f32(m), (m,), np.float32) for _ in range(2)]
-        r = rk.ROCArray(dims=(1,), dtype=np.float32)
-        ps = [plan_mapreducedim(lambda v: v + 1, rk.add, r, x) for x in xs]
-        run_cfg("mapreduce(x -> x + 1, +, Float32[2^28])", m, 4 * m, lambda i: ps[i % 2]())
-        del xs, ps
-        m = 1 << 24
-        xi = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(8)]
-        ri = rk.ROCArray(dims=(1,), dtype=np.int64)
-        ps = [plan_mapreducedim(rk.identity, rk.add, ri, x) for x in xi]
-        run_cfg("cfg1b sum Int32[2^24] -> Int64", m, 4 * m, lambda i: ps[i % 8]())
-        del xi, ps
+            xi = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(8)]
+            ri = rk.ROCArray(dims=(1,), dtype=np.int64)
+            ps = [plan_mapreducedim(rk.identity, rk.add, ri, x) for x in xi]
+            run_row("cfg1b sum Int32[2^24] -> Int64", m, 4 * m, lambda i: ps[i % 8](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_sum_i32(P(hi), I64(m), t), 4 * m, "full size", reps1=3))
+            del xi, ps
         # cfg 2: 8192 x 8192
-        d = 8192
-        As = [dev_array(randn_f32(d * d), (d, d), np.float32) for _ in range(3)]
-        r1 = rk.ROCArray(dims=(1, d), dtype=np.float32)
-        r2 = rk.ROCArray(dims=(d, 1), dtype=np.float32)
-        p1 = [plan_mapreducedim(rk.abs2, rk.add, r1, A) for A in As]
-        p2 = [plan_mapreducedim(rk.abs2, rk.add, r2, A) for A in As]
-        run_cfg("cfg2a mapreduce(abs2,+,A;dims=1) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: p1[i % 3]())
-        run_cfg("cfg2b mapreduce(abs2,+,A;dims=2) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: p2[i % 3]())
-        fv = rk.ROCArray(dims=(1, d), dtype=np.float32)
-        fi = rk.ROCArray(dims=(2, 1, d), dtype=np.int64)
-        p3 = [plan_findmax(A, fv, fi, 1) for A in As]
-        run_cfg("cfg2c findmax(A;dims=1) 8192^2", d * d, 4 * d * d + 20 * d, lambda i: p3[i % 3]())
-        del As, p1, p2, p3
+        if wanted("cfg2"):
+            d = 8192
+            As = [dev_array(randn_f32(d * d), (d, d), np.float32) for _ in range(3)]
+            r1 = rk.ROCArray(dims=(1, d), dtype=np.float32)
+            r2 = rk.ROCArray(dims=(d, 1), dtype=np.float32)
+            p1 = [plan_mapreducedim(rk.abs2, rk.add, r1, A) for A in As]
+            p2 = [plan_mapreducedim(rk.abs2, rk.add, r2, A) for A in As]
+            hA = host.get("y")                      # 2^26 normals = 8192 x 8192, column-major
+            ho = np.empty(d, dtype=np.float32)
+            hrows = np.empty(d, dtype=np.int64)
+            run_row("cfg2a mapreduce(abs2,+,A;dims=1) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: p1[i % 3](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_abs2sum_dims1_f32(P(hA), I64(d), I64(d), P(ho), t), 4 * d * d, "full size"))
+            run_row("cfg2b mapreduce(abs2,+,A;dims=2) 8192^2", d * d, 4 * d * d + 4 * d, lambda i: p2[i % 3](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_abs2sum_dims2_f32(P(hA), I64(d), I64(d), P(ho), t), 4 * d * d, "full size"))
+            fv = rk.ROCArray(dims=(1, d), dtype=np.float32)
+            fi = rk.ROCArray(dims=(2, 1, d), dtype=np.int64)
+            p3 = [plan_findmax(A, fv, fi, 1) for A in As]
+            run_row("cfg2c findmax(A;dims=1) 8192^2", d * d, 4 * d * d + 20 * d, lambda i: p3[i % 3](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_findmax_dims1_f32(P(hA), I64(d), I64(d), P(ho), P(hrows), t), 4 * d * d, "full size"))
+            del As, p1, p2, p3
         # cfg 3
-        m = 1 << 27
-        si = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(2)]
-        so = [rk.ROCArray(dims=(m,), dtype=np.int32) for _ in range(2)]
-        ps = [plan_accumulate("add", o, x) for o, x in zip(so, si)]
-        run_cfg("cfg3a cumsum Int32[2^27]", m, 8 * m, lambda i: ps[i % 2]())
-        del si, so, ps
-        rows, cols = 4096, 16384
-        Bi = [dev_array(rand_f32(rows * cols), (rows, cols), np.float32) for _ in range(2)]
-        Bo = [rk.ROCArray(dims=(rows, cols), dtype=np.float32) for _ in range(2)]
-        pa = [plan_accumulate("add", o, x, dims=1) for o, x in zip(Bo, Bi)]
-        pb = [plan_accumulate("add", o, x, dims=2) for o, x in zip(Bo, Bi)]
-        run_cfg("cfg3b cumsum(B;dims=1) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pa[i % 2]())
-        run_cfg("cumsum(B;dims=2) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pb[i % 2]())
-        del Bi, Bo, pa, pb
+        if wanted("cfg3") or wanted("cumsum(B;dims=2)"):
+            m = 1 << 27
+            si = [dev_array(randint_i32(m), (m,), np.int32) for _ in range(2)]
+            so = [rk.ROCArray(dims=(m,), dtype=np.int32) for _ in range(2)]
+            ps = [plan_accumulate("add", o, x) for o, x in zip(so, si)]
+            run_row("cfg3a cumsum Int32[2^27]", m, 8 * m, lambda i: ps[i % 2](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_i32(P(hi), I64(N_HEAD), P(host["io"])), 8 * N_HEAD,
+                                        "2^26 of the 2^27 elements; sequential (threads do not apply)", repsn=1))
+            del si, so, ps
+            rows, cols = 4096, 16384
+            Bi = [dev_array(rand_f32(rows * cols), (rows, cols), np.float32) for _ in range(2)]
+            Bo = [rk.ROCArray(dims=(rows, cols), dtype=np.float32) for _ in range(2)]
+            pa = [plan_accumulate("add", o, x, dims=1) for o, x in zip(Bo, Bi)]
+            pb = [plan_accumulate("add", o, x, dims=2) for o, x in zip(Bo, Bi)]
+            hz = host.get("z")
+            run_row("cfg3b cumsum(B;dims=1) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pa[i % 2](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_dims1_f32(P(hx), I64(rows), I64(cols), P(hz), t), 8 * rows * cols, "full size"))
+            run_row("cumsum(B;dims=2) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pb[i % 2](), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_dims2_f32(P(hx), I64(rows), I64(cols), P(hz), t), 8 * rows * cols, "full size"))
+            del Bi, Bo, pa, pb
         # findall: the scan's direct consumer (src/kernels/indexing.jl:8-36); one pass: 1 B/elt read + 8 B per index written
-        m = 1 << 26
-        masks = [dev_array((rand_f32(m) < 0.25), (m,), np.bool_) for _ in range(2)]
-        cnts = [int(rk.count(b)) for b in masks]
-        ysel = [rk.ROCArray(dims=(c,), dtype=np.int64) for c in cnts]
-        shp = RL.shape_array((m,))
-        wsp, wsb = workspace(RL.lib.rk_workspace_bytes(RL.RK_KIND_FINDALL, RL.RK_U8, 1, shp, 0))
-        def run_findall(i):
-            RL.check(RL.lib.rk_findall(masks[i % 2].ptr, 1, shp, ysel[i % 2].ptr, None, wsp, wsb, stream_ptr()), "rk_findall")
-        run_cfg("findall(Bool[2^26], 25 % true) one pass, count known", m, m + 8 * cnts[0], run_findall)
-        del masks, ysel
+        if wanted("findall"):
+            m = 1 << 26
+            masks = [dev_array((rand_f32(m) < 0.25), (m,), np.bool_) for _ in range(2)]
+            cnts = [int(rk.count(b)) for b in masks]
+            ysel = [rk.ROCArray(dims=(c,), dtype=np.int64) for c in cnts]
+            shp = RL.shape_array((m,))
+            wsp, wsb = workspace(RL.lib.rk_workspace_bytes(RL.RK_KIND_FINDALL, RL.RK_U8, 1, shp, 0))
+
+            def run_findall(i):
+                RL.check(RL.lib.rk_findall(masks[i % 2].ptr, 1, shp, ysel[i % 2].ptr, None, wsp, wsb, stream_ptr()), "rk_findall")
+            run_row("findall(Bool[2^26], 25 % true) one pass, count known", m, m + 8 * cnts[0], run_findall, reps)
+            del masks, ysel
         # reverse and permutedims (src/kernels/reverse.jl; perf/array.jl:56-65,151-155), at a bandwidth-bound size
-        d = 8192
-        ra = [dev_array(rand_f32(d * d), (d, d), np.float32) for _ in range(2)]
-        rb = [rk.ROCArray(dims=(d, d), dtype=np.float32) for _ in range(2)]
-        shp2 = RL.shape_array((d, d))
-        perm21 = (C.c_int32 * 2)(2, 1)
-        def run_reverse(i):
-            RL.check(RL.lib.rk_reverse(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, 1, stream_ptr()), "rk_reverse")
-        def run_permute(i):
-            RL.check(RL.lib.rk_permutedims(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, perm21, stream_ptr()), "rk_permutedims")
-        run_cfg("reverse(A; dims=1) 8192^2 Float32", d * d, 8 * d * d, run_reverse)
-        run_cfg("permutedims(A, (2,1)) 8192^2 Float32", d * d, 8 * d * d, run_permute)
-        del ra, rb
+        if wanted("reverse") or wanted("permutedims(A, (2,1))"):
+            d = 8192
+            ra = [dev_array(rand_f32(d * d), (d, d), np.float32) for _ in range(2)]
+            rb = [rk.ROCArray(dims=(d, d), dtype=np.float32) for _ in range(2)]
+            shp2 = RL.shape_array((d, d))
+            perm21 = (C.c_int32 * 2)(2, 1)
+
+            def run_reverse(i):
+                RL.check(RL.lib.rk_reverse(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, 1, stream_ptr()), "rk_reverse")
+
+            def run_permute(i):
+                RL.check(RL.lib.rk_permutedims(ra[i % 2].ptr, rb[i % 2].ptr, 4, 2, shp2, perm21, stream_ptr()), "rk_permutedims")
+            run_row("reverse(A; dims=1) 8192^2 Float32", d * d, 8 * d * d, run_reverse, reps)
+            run_row("permutedims(A, (2,1)) 8192^2 Float32", d * d, 8 * d * d, run_permute, reps)
+            del ra, rb
         # short and narrow extents (arrays of small structures: 3 x N, 4 x 32 x N), 2^25 elements, 3 rotating buffers
         n25 = 1 << 25
+
         def three(shape):
             return [dev_array(randn_f32(int(np.prod(shape))), shape, np.float32) for _ in range(3)]
-        sa = three((32, n25 // 32))
-        sr = rk.ROCArray(dims=(1, n25 // 32), dtype=np.float32)
-        ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
-        run_cfg("sum(A; dims=1) 32x1048576 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3]())
-        del sa, sr, ps
-        sa = three((4, 32, n25 // 128))
-        sr = rk.ROCArray(dims=(4, 1, n25 // 128), dtype=np.float32)
-        ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
-        run_cfg("sum(A; dims=2) 4x32x262144 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3]())
-        del sa, sr, ps
-        n15 = n25 // 15
-        sa = three((15, n15))
-        so = [rk.ROCArray(dims=(15, n15), dtype=np.float32) for _ in range(3)]
-        ps = [plan_accumulate("add", o, x, dims=1) for o, x in zip(so, sa)]
-        run_cfg(f"cumsum(A; dims=1) 15x{n15} Float32", 15 * n15, 8 * 15 * n15, lambda i: ps[i % 3]())
-        del sa, so, ps
-        n3 = n25 // 3
-        sa = three((3, n3))
-        sv = dev_array(randn_f32(n3), (1, n3), np.float32)
-        so = [rk.ROCArray(dims=(3, n3), dtype=np.float32) for _ in range(3)]
-        ps = [plan_materialize(o, L(x) + L(sv)) for o, x in zip(so, sa)]
-        run_cfg(f"C .= A .+ r 3x{n3} .+ 1x{n3} Float32", 3 * n3, 8 * 3 * n3 + 4 * n3, lambda i: ps[i % 3]())
-        del sa, sv, so, ps
-        sa = three((2, n25 // 4, 2))
-        so = [rk.ROCArray(dims=(2, n25 // 4, 2), dtype=np.float32) for _ in range(3)]
-        shp3 = RL.shape_array((2, n25 // 4, 2))
-        perm321 = (C.c_int32 * 3)(3, 2, 1)
-        def run_permute3(i):
-            RL.check(RL.lib.rk_permutedims(sa[i % 3].ptr, so[i % 3].ptr, 4, 3, shp3, perm321, stream_ptr()), "rk_permutedims")
-        run_cfg("permutedims(A, (3,2,1)) 2x8388608x2 Float32", n25, 8 * n25, run_permute3)
-        del sa, so
+        if wanted("sum(A; dims=1) 32x"):
+            sa = three((32, n25 // 32))
+            sr = rk.ROCArray(dims=(1, n25 // 32), dtype=np.float32)
+            ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
+            run_row("sum(A; dims=1) 32x1048576 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3](), reps)
+            del sa, sr, ps
+        if wanted("sum(A; dims=2) 4x32x"):
+            sa = three((4, 32, n25 // 128))
+            sr = rk.ROCArray(dims=(4, 1, n25 // 128), dtype=np.float32)
+            ps = [plan_mapreducedim(rk.identity, rk.add, sr, x) for x in sa]
+            run_row("sum(A; dims=2) 4x32x262144 Float32", n25, 4 * n25 + 4 * (n25 // 32), lambda i: ps[i % 3](), reps)
+            del sa, sr, ps
+        if wanted("cumsum(A; dims=1) 15x"):
+            n15 = n25 // 15
+            sa = three((15, n15))
+            so = [rk.ROCArray(dims=(15, n15), dtype=np.float32) for _ in range(3)]
+            ps = [plan_accumulate("add", o, x, dims=1) for o, x in zip(so, sa)]
+            run_row(f"cumsum(A; dims=1) 15x{n15} Float32", 15 * n15, 8 * 15 * n15, lambda i: ps[i % 3](), reps)
+            del sa, so, ps
+        if wanted("C .= A .+ r 3x"):
+            n3 = n25 // 3
+            sa = three((3, n3))
+            sv = dev_array(randn_f32(n3), (1, n3), np.float32)
+            so = [rk.ROCArray(dims=(3, n3), dtype=np.float32) for _ in range(3)]
+            ps = [plan_materialize(o, L(x) + L(sv)) for o, x in zip(so, sa)]
+            run_row(f"C .= A .+ r 3x{n3} .+ 1x{n3} Float32", 3 * n3, 8 * 3 * n3 + 4 * n3, lambda i: ps[i % 3](), reps)
+            del sa, sv, so, ps
+        if wanted("permutedims(A, (3,2,1))"):
+            sa = three((2, n25 // 4, 2))
+            so = [rk.ROCArray(dims=(2, n25 // 4, 2), dtype=np.float32) for _ in range(3)]
+            shp3 = RL.shape_array((2, n25 // 4, 2))
+            perm321 = (C.c_int32 * 3)(3, 2, 1)
+
+            def run_permute3(i):
+                RL.check(RL.lib.rk_permutedims(sa[i % 3].ptr, so[i % 3].ptr, 4, 3, shp3, perm321, stream_ptr()), "rk_permutedims")
+            run_row("permutedims(A, (3,2,1)) 2x8388608x2 Float32", n25, 8 * n25, run_permute3, reps)
+            del sa, so
         # sort! (src/kernels/sorting.jl:1; perf/array.jl:143-149 sorts a Float32 vector): 8 B/key is the floor of
         # any out-of-place permutation (one read, one write); the radix sort makes 4 digit passes plus 3 reads
-        m = 1 << 26
-        ssrc = randn_f32(m)
-        skeys = dev_array(ssrc.clone(), (m,), np.float32)
-        stmp = torch.empty(int(RL.lib.rk_sort_tmp_bytes(RL.RK_F32, m, 0)), dtype=torch.uint8, device=dev)
-        def run_sort(i):
-            skeys.buf.copy_(ssrc.view(torch.uint8))                      # unsorted input every time (the copy is timed too)
-            RL.check(RL.lib.rk_sort(RL.RK_F32, skeys.ptr, m, 0, stmp.data_ptr(), stmp.numel(), stream_ptr()), "rk_sort")
-        run_cfg("sort!(Float32[2^26]) incl. 85 us refill copy; GB/s at 8 B/key", m, 8 * m, run_sort)
-        del ssrc, skeys, stmp
+        if wanted("sort!"):
+            m = 1 << 26
+            ssrc = randn_f32(m)
+            skeys = dev_array(ssrc.clone(), (m,), np.float32)
+            stmp = torch.empty(int(RL.lib.rk_sort_tmp_bytes(RL.RK_F32, m, 0)), dtype=torch.uint8, device=dev)
+
+            def run_sort(i):
+                skeys.buf.copy_(ssrc.view(torch.uint8))                      # unsorted input every time (the copy is timed too)
+                RL.check(RL.lib.rk_sort(RL.RK_F32, skeys.ptr, m, 0, stmp.data_ptr(), stmp.numel(), stream_ptr()), "rk_sort")
+            run_row("sort!(Float32[2^26]) incl. 85 us refill copy; GB/s at 8 B/key", m, 8 * m, run_sort, reps)
+            del ssrc, skeys, stmp
         # cfg 4
-        m = 512 ** 3
-        x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))
-        z4 = rk.ROCArray(dims=(512, 512, 512), dtype=np.float32)
-        e4 = a * L(x4) + L(y4) * rk.broadcast.exp(L(w4))
-        p4 = plan_materialize(z4, e4)
-        run_cfg("cfg4a z .= a.*x .+ y.*exp.(w) 512^3", m, 16 * m, lambda i: p4())
-        del x4, y4, w4, z4, e4, p4
-        d = 16384
-        A4 = dev_array(rand_f32(d * d, -1, 1), (d, d), np.float32)
-        r4 = dev_array(rand_f32(d, -1, 1), (1, d), np.float32)
-        c4 = dev_array(rand_f32(d, -1, 1), (d, 1), np.float32)
-        C4 = rk.ROCArray(dims=(d, d), dtype=np.float32)
-        e4b = L(A4) + L(r4) * L(c4)
-        p4b = plan_materialize(C4, e4b)
-        run_cfg("cfg4b C .= A .+ r .* c 16384^2", d * d, 8 * d * d + 8 * d, lambda i: p4b())
-        del A4, C4, e4b, p4b
+        if wanted("cfg4"):
+            m = 512 ** 3
+            x4, y4, w4 = (dev_array(randn_f32(m), (512, 512, 512), np.float32) for _ in range(3))
+            z4 = rk.ROCArray(dims=(512, 512, 512), dtype=np.float32)
+            e4 = a * L(x4) + L(y4) * rk.broadcast.exp(L(w4))
+            p4 = plan_materialize(z4, e4)
+            run_row("cfg4a z .= a.*x .+ y.*exp.(w) 512^3", m, 16 * m, lambda i: p4(), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_bcast_axpby_exp_f32(C.c_float(0.5), P(hx), P(host["y"]), P(host["w"]), P(host["z"]), I64(N_HEAD), t),
+                                        16 * N_HEAD, "2^26 of the 2^27 elements"))
+            del x4, y4, w4, z4, e4, p4
+            d = 16384
+            A4 = dev_array(rand_f32(d * d, -1, 1), (d, d), np.float32)
+            r4 = dev_array(rand_f32(d, -1, 1), (1, d), np.float32)
+            c4 = dev_array(rand_f32(d, -1, 1), (d, 1), np.float32)
+            C4 = rk.ROCArray(dims=(d, d), dtype=np.float32)
+            e4b = L(A4) + L(r4) * L(c4)
+            p4b = plan_materialize(C4, e4b)
+            dc = 4096                                # CPU sample: 16384 x 4096 columns of the matrix
+            run_row("cfg4b C .= A .+ r .* c 16384^2", d * d, 8 * d * d + 8 * d, lambda i: p4b(), reps,
+                    cpu=lambda: cpu_row(lambda t: cpu_lib.orc_bcast_rowcol_f32(P(hx), P(host["y"]), P(host["w"]), P(host["z"]), I64(d), I64(dc), t),
+                                        8 * d * dc, "16384 x 4096: a quarter of the columns"))
+            del A4, C4, e4b, p4b
         # cfg 5
-        for ne, rot in ((4000, 6), (240_000, 1)):
-            Qs = [dev_array(rand_f32(625 * ne, 0.5, 1.5), (5, 5, 5, 5, ne), np.float32) for _ in range(rot)]
-            Vs = [dev_array(rand_f32(1750 * ne, 0.9, 1.1), (5, 5, 5, 14, ne), np.float32) for _ in range(rot)]
-            Rs = [rk.zeros(np.float32, 5, 5, 5, 5, ne) for _ in range(rot)]
-            Dm = dev_array(rand_f32(25), (5, 5), np.float32)
-            pv = [plan_volumerhs(Rs[j], Qs[j], Vs[j], 9.81, Dm, ne) for j in range(rot)]
-            run_cfg(f"cfg5 volumerhs! N=4 nelem={ne}", 125 * ne, 13500 * ne, lambda i: pv[i % rot](), flops=37_000 * ne)
-            del Qs, Vs, Rs, pv
+        if wanted("cfg5"):
+            for ne, rot, ne_cpu in ((4000, 6, 4000), (240_000, 1, 24_000)):
+                Qs = [dev_array(rand_f32(625 * ne, 0.5, 1.5), (5, 5, 5, 5, ne), np.float32) for _ in range(rot)]
+                Vs = [dev_array(rand_f32(1750 * ne, 0.9, 1.1), (5, 5, 5, 14, ne), np.float32) for _ in range(rot)]
+                Rs = [rk.zeros(np.float32, 5, 5, 5, 5, ne) for _ in range(rot)]
+                Dm = dev_array(rand_f32(25), (5, 5), np.float32)
+                pv = [plan_volumerhs(Rs[j], Qs[j], Vs[j], 9.81, Dm, ne) for j in range(rot)]
+
+                def cpu_vr(ne_cpu=ne_cpu):
+                    hq = (host["x"][:625 * ne_cpu] + np.float32(0.5))
+                    hv = (host["x"][:1750 * ne_cpu] * np.float32(0.2) + np.float32(0.9))
+                    hr = np.zeros(625 * ne_cpu, dtype=np.float32)
+                    hD = host["x"][:25].copy()
+                    return cpu_row(lambda t: cpu_lib.orc_volumerhs_f32(P(hr), P(hq), P(hv), C.c_float(9.81), P(hD), I64(ne_cpu), t),
+                                   13500 * ne_cpu, "full size" if ne_cpu == ne else f"{ne_cpu} of the {ne} elements")
+                run_row(f"cfg5 volumerhs! N=4 nelem={ne}", 125 * ne, 13500 * ne, lambda i: pv[i % rot](), reps, cpu=cpu_vr, flops=37_000 * ne)
+                del Qs, Vs, Rs, pv
         torch.cuda.empty_cache()
-
-    # ---- CPU baseline: C restatement of Julia Base on the host cores, same step -----------------------------
-    cpu = None
-    if not args.no_cpu:
-        so = os.path.join(ROOT, "oracle", "liboracle_c.so")
-        if os.path.exists(so):
-            lib = C.CDLL(so)
-            lib.orc_sum_f32.restype = C.c_double
-            lib.orc_sum_f32.argtypes = [C.c_void_p, C.c_int64, C.c_int]
-            lib.orc_cumsum_i32.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
-            lib.orc_bcast_axpby_exp_f32.argtypes = [C.c_float] + [C.c_void_p] * 4 + [C.c_int64, C.c_int]
-            threads = max(1, min(16, os.cpu_count() or 1))
-            rng = np.random.default_rng(0)
-            hx = rng.random(n, dtype=np.float32)
-            hi = rng.integers(-1000, 1001, n, dtype=np.int32)
-            ho = np.empty_like(hi)
-            hy, hw = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
-            hz = np.empty_like(hx)
-
-            def cpu_step(t):
-                lib.orc_sum_f32(hx.ctypes.data, n, t)
-                lib.orc_cumsum_i32(hi.ctypes.data, n, ho.ctypes.data)
-                lib.orc_bcast_axpby_exp_f32(0.5, hx.ctypes.data, hy.ctypes.data, hw.ctypes.data, hz.ctypes.data, n, t)
-
-            def best_of(t, reps):
-                cpu_step(t)
-                best = float("inf")
-                for _ in range(reps):
-                    t0 = time.perf_counter()
-                    cpu_step(t)
-                    best = min(best, time.perf_counter() - t0)
-                return best
-
-            t1 = best_of(1, 2)
-            tn = best_of(threads, 5) if threads > 1 else t1
-            cpu = {"value": round(step_bytes / tn / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-                   "single_thread_GBps": round(step_bytes / t1 / 1e9, 2),
-                   "sample": "the same step (sum Float32 + accumulate(+) Int32 + z .= a.*x .+ y.*exp.(w), 2^26 elements each), "
-                             "minimum of 5 runs of oracle/oracle_c.c with OpenMP on `cores` threads (the Int32 scan is sequential, "
-                             "as in Julia Base); Julia itself is not installed on this machine, so this is the C port of Base's "
-                             "algorithms (JULIA_NUM_THREADS does not apply; Base's sum/accumulate/broadcast are single-threaded: "
-                             "see single_thread_GBps)"}
 
     out = {
         "metric": "achieved HBM GB/s (% of ~8 TB/s peak) for sum/cumsum/broadcast at 2^26 elems",
-        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "value": round(value, 1) if value is not None else None, "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 4) if ms_per_step is not None else None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "step = sum(Float32[2^26]) + accumulate(+, Int32[2^26]) + (z .= a.*x .+ y.*exp.(w), Float32[2^26]); "
                                "28 algorithmic bytes per element; rotating HBM-resident buffers",
-                   "elements": n, "bytes_per_step": step_bytes, "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+                   "elements": n, "bytes_per_step": step_bytes,
+                   "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4) if value is not None else None},
         "roofline": roofline,
-        "cpu_baseline": cpu,
+        "cpu_baseline": cpu_step,
+        "timing": "configs: min_us / GBps / frac_hbm = minimum of individually synchronised launches (perf/runbenchmarks.jl:81-86); "
+                  "batch_avg_us / GBps_batch = average of back-to-back launches; cpu = oracle/oracle_c.c on the host cores",
         "configs": configs,
     }
     print(json.dumps(out))

@@ -62,6 +62,32 @@ int64_t orc_sum_i32(const int32_t* x, int64_t n, int threads) {
     return s;
 }
 
+/* Base.max on Float32: NaN propagates, max(-0.0, 0.0) == 0.0 */
+static float max_f32(float a, float b) {
+    if (isnan(a)) return a;
+    if (isnan(b)) return b;
+    if (a == b) return signbit(a) ? b : a;
+    return a > b ? a : b;
+}
+
+/* maximum(x::Vector{Float32}); n >= 1.  Threads reduce contiguous shares, combined in order (max is associative). */
+float orc_maximum_f32(const float* x, int64_t n, int threads) {
+    if (threads < 1) threads = 1;
+    if (threads > 256) threads = 256;
+    float parts[256];
+    int64_t per = (n + threads - 1) / threads;
+#pragma omp parallel for num_threads(threads) schedule(static)
+    for (int t = 0; t < threads; ++t) {
+        int64_t lo = t * per, hi = lo + per < n ? lo + per : n;
+        float m = -INFINITY;
+        for (int64_t i = lo; i < hi; ++i) m = max_f32(m, x[i]);
+        parts[t] = m;
+    }
+    float m = parts[0];
+    for (int t = 1; t < threads; ++t) m = max_f32(m, parts[t]);
+    return m;
+}
+
 /* mapreduce(abs2, +, A; dims=1) on an m x n column-major matrix -> out[n] */
 void orc_abs2sum_dims1_f32(const float* A, int64_t m, int64_t n, float* out, int threads) {
 #pragma omp parallel for num_threads(threads) schedule(static)
@@ -125,6 +151,22 @@ void orc_cumsum_dims1_f32(const float* B, int64_t m, int64_t n, float* out, int 
     for (int64_t j = 0; j < n; ++j) {
         float s = 0.0f;
         for (int64_t i = 0; i < m; ++i) { s += B[j * m + i]; out[j * m + i] = s; }
+    }
+}
+
+/* cumsum(B; dims=2) on an m x n column-major Float32 matrix: row i runs over the columns, stride m.  Walked
+ * column by column (cache-friendly), threads split the rows. */
+void orc_cumsum_dims2_f32(const float* B, int64_t m, int64_t n, float* out, int threads) {
+#pragma omp parallel num_threads(threads)
+    {
+        int t = 0, nt = 1;
+#ifdef _OPENMP
+        t = omp_get_thread_num();
+        nt = omp_get_num_threads();
+#endif
+        int64_t per = (m + nt - 1) / nt, lo = t * per, hi = lo + per < m ? lo + per : m;
+        for (int64_t j = 0; j < n; ++j)
+            for (int64_t i = lo; i < hi; ++i) out[j * m + i] = (j == 0 ? 0.0f : out[(j - 1) * m + i]) + B[j * m + i];
     }
 }
 

@@ -312,6 +312,7 @@ def corc():
     lib = C.CDLL(so)
     lib.orc_sum_f32.restype = C.c_double
     lib.orc_sum_i32.restype = C.c_int64
+    lib.orc_maximum_f32.restype = C.c_float
     return lib
 
 
@@ -347,6 +348,16 @@ def test_c_oracle_matches_numpy_oracle(corc, threads):
     Bo = np.empty_like(B)
     corc.orc_cumsum_dims1_f32(_p(B), C.c_int64(m), C.c_int64(n), _p(Bo), threads)
     np.testing.assert_allclose(Bo, orc.cumsum(B, dims=1), rtol=1e-4)
+    Bo2 = np.empty_like(B)
+    corc.orc_cumsum_dims2_f32(_p(B), C.c_int64(m), C.c_int64(n), _p(Bo2), threads)
+    np.testing.assert_allclose(Bo2, np.cumsum(B.astype(np.float64), axis=1), rtol=1e-4)
+    # maximum: Base.max rules -- plain values, a planted NaN, and +0.0 against -0.0
+    assert corc.orc_maximum_f32(_p(x), C.c_int64(x.size), threads) == x.max()
+    xn = x.copy()
+    xn[123_456] = np.nan
+    assert np.isnan(corc.orc_maximum_f32(_p(xn), C.c_int64(xn.size), threads))
+    zs = np.array([-0.0, 0.0, -0.0], dtype=np.float32)
+    assert not np.signbit(np.float32(corc.orc_maximum_f32(_p(zs), C.c_int64(3), 1)))
     y, w = rng.standard_normal(x.size, dtype=np.float32), rng.standard_normal(x.size, dtype=np.float32)
     z = np.empty_like(x)
     corc.orc_bcast_axpby_exp_f32(C.c_float(0.5), _p(x), _p(y), _p(w), _p(z), C.c_int64(x.size), threads)
