@@ -97,6 +97,10 @@ PROTOTYPES = {
     "rk_sort_status": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_mapreduce_strided": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, _I64P, C.c_uint32,
+                                         C.c_void_p, _I64P, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_accumulate_strided": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, _I64P, _I64P, C.c_int,
+                                          C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce_program": (C.c_int32, [C.POINTER(RkMapProgram), C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_findminmax": (C.c_int32, [C.c_int32, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,

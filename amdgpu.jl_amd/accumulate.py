@@ -36,6 +36,21 @@ def accumulate_(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusi
 
 
 def _launch_accumulate(op, B, A, dims, init, inclusive):
+    from .views import ROCView
+    if isinstance(A, ROCView) or isinstance(B, ROCView):
+        # wrapper arrays laid out alike (accumulate!(+, transpose(B), transpose(A))): the dims are renumbered in the ABI
+        from .mapreduce import _dense_strides
+        astr = tuple(A.strides) if isinstance(A, ROCView) else _dense_strides(A.dims)
+        bstr = tuple(B.strides) if isinstance(B, ROCView) else _dense_strides(B.dims)
+        aptr = A.sptr if isinstance(A, ROCView) else A.ptr
+        bptr = B.sptr if isinstance(B, ROCView) else B.ptr
+        ws, ws_bytes = workspace(16 << 20)
+        sargs = (_OP[op], A.code, B.code, aptr, bptr, A.ndim, L.shape_array(A.dims), L.shape_array(astr), L.shape_array(bstr), int(dims),
+                 1 if inclusive else 0, _scalar_buffer(init, B.dtype), ws, ws_bytes)
+
+        def launch_strided():
+            L.check(L.lib.rk_accumulate_strided(*sargs, stream_ptr()), "rk_accumulate_strided")
+        return launch_strided
     bytes_needed = L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, B.code, A.ndim, L.shape_array(A.dims),
                                             (1 << (dims - 1)) if dims <= A.ndim else 0)
     ws, ws_bytes = workspace(bytes_needed)

@@ -239,8 +239,9 @@ int32_t rk_workspace_status(const void* ws, size_t ws_bytes, void* stream) {
     return failed != 0u ? RK_ERR_WAIT : RK_SUCCESS;
 }
 
-int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
-                     uint32_t reduce_mask, void* R, const void* init, void* ws, size_t ws_bytes, void* stream) {
+static int32_t mapreduce_dispatch(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
+                                  uint32_t reduce_mask, void* R, const void* init, void* ws, size_t ws_bytes, void* stream,
+                                  size_t partials_cap) {
     int64_t total = 0;
     if (!valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
     if ((int)f < RK_MAP_IDENTITY || (int)f > RK_MAP_ABS) return RK_ERR_INVALID_ARGUMENT;
@@ -249,7 +250,7 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
     if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91
     if (A == nullptr || R == nullptr) return RK_ERR_INVALID_ARGUMENT;
     reduce_mask &= (1u << ndim) - 1u;       // dims beyond ndim reduce nothing
-    MapreduceArgs a{(int)f, (int)op, nullptr, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream};
+    MapreduceArgs a{(int)f, (int)op, nullptr, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, (hipStream_t)stream, partials_cap};
     if (in == out) {
         switch (in) {
             case RK_F32: return mapreduce_f32(a);
@@ -267,6 +268,109 @@ int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* 
     if (in == RK_U8 && (out == RK_I64 || out == RK_U64)) return mapreduce_u8_i64(a);   // sums of bytes: the same bits either way
     if (in == RK_U32 && out == RK_U64) return mapreduce_u32_u64(a);
     return RK_ERR_UNSUPPORTED;
+}
+
+int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
+                     uint32_t reduce_mask, void* R, const void* init, void* ws, size_t ws_bytes, void* stream) {
+    return mapreduce_dispatch(f, op, in, out, A, ndim, shape, reduce_mask, R, init, ws, ws_bytes, stream, WS_PARTIALS_BYTES);
+}
+
+// ---- wrapper arrays (transpose, PermutedDimsArray, reshape) in reductions and scans ---------------------------------------
+// A permuted-dense array -- its strides are those of a dense column-major array with the dims in another order -- is
+// a dense array once the dims are listed in memory order, and a reduction or scan over some of its dims is the same
+// operation over the same dims of that dense array.  No kernel knows about strides: the entry points renumber the dims.
+struct DenseOrder {
+    int     order[RK_MAX_DIMS];      // order[k] = the logical dim that is k-th in memory (extents of 1 last)
+    int64_t shape[RK_MAX_DIMS];      // extents in memory order
+};
+// false: the strides are not those of a permuted dense array (a view with gaps, a reversed or repeated dim)
+static bool dense_order(int ndim, const int64_t* shape, const int64_t* strides, DenseOrder* o) {
+    bool used[RK_MAX_DIMS] = {};
+    int n = 0;
+    int64_t expect = 1;
+    for (;;) {
+        int pick = -1;
+        for (int d = 0; d < ndim; ++d)
+            if (!used[d] && shape[d] != 1 && (strides ? strides[d] : expect) == expect && (strides || pick < 0)) { pick = d; break; }
+        if (pick < 0) break;
+        used[pick] = true;
+        o->order[n] = pick;
+        o->shape[n] = shape[pick];
+        ++n;
+        expect *= shape[pick];
+    }
+    for (int d = 0; d < ndim; ++d) {
+        if (used[d]) continue;
+        if (shape[d] != 1) return false;
+        o->order[n] = d;
+        o->shape[n] = 1;
+        ++n;
+    }
+    return true;
+}
+
+int32_t rk_mapreduce_strided(rk_map f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim, const int64_t* shape,
+                             const int64_t* a_strides, uint32_t reduce_mask, void* R, const int64_t* r_strides, const void* init,
+                             void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    if (!valid_dtype(in) || !valid_dtype(out) || A == nullptr || R == nullptr) return RK_ERR_INVALID_ARGUMENT;
+    reduce_mask &= (1u << ndim) - 1u;
+    DenseOrder o{};
+    if (!dense_order(ndim, shape, a_strides, &o)) return RK_ERR_UNSUPPORTED;
+    uint32_t mask_mem = 0;
+    for (int k = 0; k < ndim; ++k)
+        if ((reduce_mask >> o.order[k]) & 1u) mask_mem |= 1u << k;
+    // where the kernels put R: the kept dims in memory order, densely.  nat[d] = that stride of logical dim d
+    int64_t nat[RK_MAX_DIMS] = {}, rshape[RK_MAX_DIMS], count = 1;
+    for (int k = 0; k < ndim; ++k) {
+        const int d = o.order[k];
+        if ((reduce_mask >> d) & 1u) continue;
+        nat[d] = count;
+        count *= shape[d];
+    }
+    bool same = true;
+    int64_t dense = 1;
+    for (int d = 0; d < ndim; ++d) {
+        const bool kept = !((reduce_mask >> d) & 1u);
+        rshape[d] = kept ? shape[d] : 1;
+        const int64_t want = r_strides ? r_strides[d] : dense;
+        if (kept && shape[d] > 1 && want != nat[d]) same = false;
+        dense *= rshape[d];
+    }
+    if (same) return mapreduce_dispatch(f, op, in, out, A, ndim, o.shape, mask_mem, R, init, ws, ws_bytes, stream, WS_PARTIALS_BYTES);
+    // R is laid out otherwise (the transpose of mapreducedim!(identity, +, transpose(R), A)): reduce into the top of
+    // the partials area, then one strided copy into R
+    const size_t esz = dtype_size(out);
+    const size_t temp_bytes = ((size_t)count * esz + 255) & ~(size_t)255;
+    Workspace w{};
+    if (temp_bytes > WS_PARTIALS_BYTES / 4) return RK_ERR_UNSUPPORTED;
+    if (!carve_workspace(ws, ws_bytes, 0, &w)) return RK_ERR_WORKSPACE;
+    void* temp = w.partials + WS_PARTIALS_BYTES - temp_bytes;
+    const int32_t st = mapreduce_dispatch(f, op, in, out, A, ndim, o.shape, mask_mem, temp, init, ws, ws_bytes, stream,
+                                          WS_PARTIALS_BYTES - temp_bytes);
+    if (st != RK_SUCCESS) return st;
+    rk_program prog{};
+    prog.compute = (out == RK_F32 || out == RK_F16) ? RK_F32 : (out == RK_F64 ? RK_F64 : RK_I64);
+    prog.n_operands = 1;
+    prog.operands[0].ptr = temp;
+    prog.operands[0].dtype = out;
+    prog.operands[0].ndim = ndim;
+    prog.operands[0].strided = 1;
+    for (int d = 0; d < ndim; ++d) {
+        prog.operands[0].shape[d] = rshape[d];
+        prog.operands[0].strides[d] = rshape[d] > 1 ? nat[d] : 0;
+    }
+    prog.n_tokens = 1;
+    prog.tokens[0] = 0;
+    int64_t rs[RK_MAX_DIMS];
+    dense = 1;
+    for (int d = 0; d < ndim; ++d) {
+        rs[d] = r_strides ? r_strides[d] : dense;
+        dense *= rshape[d];
+    }
+    return rk_broadcast_strided(&prog, R, out, ndim, rshape, rs, stream);
 }
 
 int32_t rk_mapreduce_program(const rk_map_program* f, rk_op op, rk_dtype in, rk_dtype out, const void* A, int ndim,
@@ -347,6 +451,22 @@ int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, v
     if (in == RK_U8 && out == RK_I64) return scan_u8_i64(a);
     if (in == RK_U8 && out == RK_I32) return scan_u8_i32(a);
     return RK_ERR_UNSUPPORTED;
+}
+
+int32_t rk_accumulate_strided(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, void* out_ptr, int ndim, const int64_t* shape,
+                              const int64_t* in_strides, const int64_t* out_strides, int dim, int32_t inclusive, const void* init,
+                              void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_shape(ndim, shape, &total) || dim < 1) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    DenseOrder oi{}, oo{};
+    if (!dense_order(ndim, shape, in_strides, &oi) || !dense_order(ndim, shape, out_strides, &oo)) return RK_ERR_UNSUPPORTED;
+    for (int k = 0; k < ndim; ++k)
+        if (oi.order[k] != oo.order[k]) return RK_ERR_UNSUPPORTED;     // input and output must be laid out alike
+    int dim_mem = dim;                                                 // dim > ndim: a copy, whatever the layout
+    for (int k = 0; k < ndim; ++k)
+        if (oi.order[k] == dim - 1) dim_mem = k + 1;
+    return rk_accumulate(op, in, out, in_ptr, out_ptr, ndim, oi.shape, dim_mem, inclusive, init, ws, ws_bytes, stream);
 }
 
 int32_t rk_accumulate_static(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, void* out_ptr, int ndim, const int64_t* shape,

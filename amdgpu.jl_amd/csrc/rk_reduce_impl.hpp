@@ -929,6 +929,7 @@ struct MapreduceArgs {
     const void* A; int ndim; const int64_t* shape; uint32_t mask;
     void* R; const void* init;
     void* ws; size_t ws_bytes; hipStream_t stream;
+    size_t partials_cap = WS_PARTIALS_BYTES;   // bytes of the partials area this call may use (the caller keeps the rest)
 };
 struct FindArgs {
     int want_max;
@@ -941,7 +942,7 @@ struct FindArgs {
 // output's elements with a stride pattern and reaches a tenth of the bandwidth.  Since op is associative and
 // commutative, the lowest run of reduced dims is folded first -- a plain single-run reduction of all the data into
 // a temporary at the top of the partials area -- and the remaining dims are reduced from that much smaller array.
-constexpr size_t REDUCE_TEMP_MAX = WS_PARTIALS_BYTES / 2;
+// (at most half of the partials area the call may use)
 
 template <typename In, typename Acc, typename Xf, typename Op, typename Out = Acc>
 inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
@@ -974,11 +975,11 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
             for (int c = 0; c < 2; ++c) {
                 const int r = candidates[c];
                 const size_t temp_bytes = ((size_t)(s.total / run_ext[r]) * sizeof(Acc) + 255) & ~(size_t)255;
-                if (temp_bytes > REDUCE_TEMP_MAX) continue;
+                if (temp_bytes > a.partials_cap / 2) continue;
                 int64_t shape1[RK_MAX_DIMS];
                 for (int d = 0; d < a.ndim; ++d) shape1[d] = ((run_mask[r] >> d) & 1u) ? 1 : a.shape[d];
-                Acc* temp = (Acc*)((char*)w.partials + WS_PARTIALS_BYTES - temp_bytes);
-                const size_t cap = WS_PARTIALS_BYTES - temp_bytes;
+                Acc* temp = (Acc*)((char*)w.partials + a.partials_cap - temp_bytes);
+                const size_t cap = a.partials_cap - temp_bytes;
                 ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
                 const int32_t st = launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, run_mask[r], xf, Op(), to_temp,
                                                           a.ws, a.ws_bytes, a.stream, cap);
@@ -988,7 +989,7 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
             }
         }
     }
-    return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream);
+    return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream, a.partials_cap);
 }
 
 template <typename In, typename Acc, typename Map, typename Out = Acc>

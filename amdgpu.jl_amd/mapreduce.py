@@ -61,6 +61,14 @@ def _reduced_dims(dims_in, mask):
     return tuple(1 if (mask >> d) & 1 else n for d, n in enumerate(dims_in))
 
 
+def _dense_strides(dims):
+    out, s = [], 1
+    for n in dims:
+        out.append(s)
+        s *= n
+    return tuple(out)
+
+
 def _scalar_buffer(value, dtype: np.dtype):
     """Host scalar of ``dtype`` as a ctypes buffer (the ABI reads it during the call)."""
     if value is None:
@@ -121,6 +129,25 @@ def _launch_mapreducedim(f, op, R, A, init, mask):
     """Zero-argument callable that enqueues the reduction on the current stream."""
     ws, ws_bytes = workspace()
     ibuf = _scalar_buffer(init, R.dtype)
+    from .views import ROCView
+    if isinstance(R, ROCView) or isinstance(A, ROCView):
+        # wrapper arrays (transpose, PermutedDimsArray): rk_mapreduce_strided renumbers the dims; closures for f and
+        # views with gaps are not native here
+        if callable(f):
+            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "a closure for f over a wrapper array: copy(view) first")
+        rdims = tuple(R.dims) + (1,) * (A.ndim - R.ndim)
+        rstr = (tuple(R.strides) if isinstance(R, ROCView) else _dense_strides(R.dims)) + (0,) * (A.ndim - R.ndim)
+        astr = tuple(A.strides) if isinstance(A, ROCView) else _dense_strides(A.dims)
+        rstr = tuple(s if n > 1 else 0 for s, n in zip(rstr, rdims))
+        aptr = A.sptr if isinstance(A, ROCView) else A.ptr
+        rptr = R.sptr if isinstance(R, ROCView) else R.ptr
+        args = (_MAP[f], _OP[op], A.code, R.code, aptr, A.ndim, L.shape_array(A.dims), L.shape_array(astr), mask, rptr,
+                L.shape_array(rstr), ibuf, ws, ws_bytes)
+        fn, name = L.lib.rk_mapreduce_strided, "rk_mapreduce_strided"
+
+        def launch_strided():
+            L.check(fn(*args, stream_ptr()), name)
+        return launch_strided
     if callable(f):
         prog, _ = _map_program(f, A.dtype)
         args = (prog, _OP[op], A.code, R.code, A.ptr, A.ndim, L.shape_array(A.dims), mask, R.ptr, ibuf, ws, ws_bytes)

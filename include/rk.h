@@ -138,6 +138,21 @@ RK_API int32_t rk_mapreduce(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
                      void* R, const void* init,
                      void* ws, size_t ws_bytes, void* stream);
 
+/* The same for wrapper arrays: `A` and / or `R` a transpose, PermutedDimsArray or reshape of a dense
+ * array, as in the reference's own test  mapreducedim!(identity, +, transpose(R), A) === R
+ *                                                        test/core/rocarray_base.jl:263-267
+ * (the method takes any AnyROCArray destination, src/kernels/mapreduce.jl:86-89,172).
+ * `A`, `R` point at the first element; `a_strides` / `r_strides` are element strides per dim (NULL =
+ * dense column-major; entries of R's reduced dims are ignored).  A must be PERMUTED-DENSE: its strides
+ * those of a dense array with the dims in some order (no gaps, no negative or zero strides); anything
+ * else -- a view with gaps -- is RK_ERR_UNSUPPORTED (copy it first).  R may have any strides; when they
+ * differ from where the kernels put the result, it is reduced into the workspace (at most 2.5 MiB of
+ * results, else RK_ERR_UNSUPPORTED) and copied into R by the strided broadcast kernel. */
+RK_API int32_t rk_mapreduce_strided(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
+                             const void* A, int ndim, const int64_t* shape, const int64_t* a_strides,
+                             uint32_t reduce_mask, void* R, const int64_t* r_strides, const void* init,
+                             void* ws, size_t ws_bytes, void* stream);
+
 /* ---- mapreduce with f given as a program -----------------------------------------------
  * Replaces GPUArrays.mapreducedim!(f, op, R, A) for an f outside the rk_map list
  *                                                        src/kernels/mapreduce.jl:86-89
@@ -197,6 +212,15 @@ RK_API int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out,
                       int ndim, const int64_t* shape, int dim, int32_t inclusive,
                       const void* init,
                       void* ws, size_t ws_bytes, void* stream);
+
+/* The same for wrapper arrays (cumsum!(transpose(B), transpose(A)), accumulate! on a
+ * PermutedDimsArray): input and output permuted-dense (see rk_mapreduce_strided) with the SAME order of
+ * dims in memory; anything else is RK_ERR_UNSUPPORTED.  `dim` is the logical dimension. */
+RK_API int32_t rk_accumulate_strided(rk_op op, rk_dtype in, rk_dtype out,
+                              const void* in_ptr, void* out_ptr,
+                              int ndim, const int64_t* shape, const int64_t* in_strides,
+                              const int64_t* out_strides, int dim, int32_t inclusive,
+                              const void* init, void* ws, size_t ws_bytes, void* stream);
 
 /* ---- accumulate without a caller workspace ------------------------------------------------
  * No counterpart in the reference.  For callers that cannot allocate device memory at all --

@@ -236,6 +236,25 @@ def test_workspace_queries(L):
     assert wi(C.c_void_p(0x1000), 1024, None) == L.RK_ERR_WORKSPACE
 
 
+def test_strided_entry_points_reject_what_is_not_permuted_dense(L):
+    ws, A, R = C.c_void_p(0x10000000), C.c_void_p(0x20000000), C.c_void_p(0x30000000)
+    shp = L.shape_array((40, 30))
+    for strides in ((1, 80), (2, 80), (1, 20), (-1, 40), (0, 1), (1, 1)):          # gaps, steps, overlap, reversal, repetition
+        st = L.lib.rk_mapreduce_strided(L.RK_MAP_IDENTITY, L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, 2, shp, L.shape_array(strides), 1, R, None,
+                                        None, ws, 16 << 20, None)
+        assert st == L.RK_ERR_UNSUPPORTED, strides
+        st = L.lib.rk_accumulate_strided(L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, R, 2, shp, L.shape_array(strides), L.shape_array(strides), 1, 1,
+                                         None, ws, 16 << 20, None)
+        assert st == L.RK_ERR_UNSUPPORTED, strides
+    # input and output of a scan laid out differently
+    st = L.lib.rk_accumulate_strided(L.RK_OP_ADD, L.RK_F32, L.RK_F32, A, R, 2, shp, L.shape_array((30, 1)), None, 1, 1, None, ws, 16 << 20, None)
+    assert st == L.RK_ERR_UNSUPPORTED
+    assert L.lib.rk_mapreduce_strided(L.RK_MAP_IDENTITY, L.RK_OP_ADD, L.RK_F32, L.RK_F32, None, 2, shp, None, 1, R, None, None, ws, 16 << 20,
+                                      None) == L.RK_ERR_INVALID_ARGUMENT
+    assert L.lib.rk_mapreduce_strided(L.RK_MAP_IDENTITY, L.RK_OP_ADD, L.RK_F32, L.RK_F32, None, 1, L.shape_array((0,)), None, 1, None, None, None,
+                                      None, 0, None) == 0
+
+
 def test_long_outer_extents_are_not_rejected(L):
     """Shapes whose outer extent exceeds 65535 (the y / z limit of a grid) pass validation and planning: with no device
     the call then stops at the launch with a HIP error, never with RK_ERR_TOO_LARGE.  Only meaningful -- and only safe,
