@@ -155,7 +155,13 @@ class DimensionMismatch(RKError, ValueError):
 
 
 class UnsupportedError(RKError, NotImplementedError):
-    """The request is legal Julia but outside the enumerated native op set."""
+    """The request is legal Julia but the library declines it: an operation outside the enumerated native set, an
+    extent beyond what the kernels index (RK_ERR_TOO_LARGE), a workspace the call cannot use (RK_ERR_WORKSPACE).
+    A binding inside AMDGPU.jl answers all three by running the stock method; this mirror has no stock method, so
+    it raises the one exception type a caller catches to take another path.  `status` tells the three apart."""
+
+
+DECLINED = (RK_ERR_UNSUPPORTED, RK_ERR_TOO_LARGE, RK_ERR_WORKSPACE)
 
 
 def check(status: int, where: str = "") -> None:
@@ -163,7 +169,7 @@ def check(status: int, where: str = "") -> None:
         return
     if status == RK_ERR_DIMENSION:
         raise DimensionMismatch(status, where)
-    if status == RK_ERR_UNSUPPORTED:
+    if status in DECLINED:
         raise UnsupportedError(status, where)
     raise RKError(status, where)
 

@@ -154,14 +154,24 @@ _retired: list = []
 
 
 def workspace(min_bytes: int = 0):
-    """(pointer, bytes) of the initialised workspace bound to the current device and stream."""
+    """(pointer, bytes) of the initialised workspace bound to the current device and stream.
+
+    A workspace that is too small is replaced by one of at least twice its size.  The outgrown buffers stay
+    allocated -- a prepared launch or a captured graph may hold their address -- which costs less than the size of
+    the live one in total, since sizes double.  No growth happens on a stream that is being captured: the
+    allocation would not belong to the graph's memory.  Run the call once before the capture (as a warm-up
+    does anyway) or ask for the size up front with ``workspace(rk_workspace_bytes(...))``.
+    """
     key = (torch.cuda.current_device(), stream_ptr())
     need = max(int(min_bytes), 16 << 20)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
+        if torch.cuda.is_current_stream_capturing():
+            raise L.RKError(L.RK_ERR_WORKSPACE, f"workspace of {need} bytes requested while the stream is being captured; "
+                            "run the call once before the capture")
         size = max(need, 2 * ws.numel() if ws is not None else 0)
         if ws is not None:
-            _retired.append(ws)      # prepared calls may still hold its address: never free a workspace
+            _retired.append(ws)
         ws = torch.empty(size, dtype=torch.uint8, device=device())
         assert ws.data_ptr() % 256 == 0
         L.check(L.lib.rk_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr()), "rk_workspace_init")

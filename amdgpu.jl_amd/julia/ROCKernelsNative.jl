@@ -35,7 +35,13 @@ function Base.showerror(io::IO, e::RKError)
     print(io, "RKError($(e.code)): $msg")
 end
 const RK_ERR_UNSUPPORTED = Int32(10002)
+const RK_ERR_WORKSPACE = Int32(10003)
 const RK_ERR_DIMENSION = Int32(10004)
+const RK_ERR_TOO_LARGE = Int32(10005)
+const RK_ERR_WAIT = Int32(10006)
+# A legal request the library does not take -- an operation outside its set, an extent beyond what its kernels
+# index, a workspace it cannot size -- is declined, not an error: the caller runs the stock method instead.
+declined(status::Int32) = status == RK_ERR_UNSUPPORTED || status == RK_ERR_TOO_LARGE || status == RK_ERR_WORKSPACE
 @inline function check(status::Int32)
     status == 0 && return nothing
     status == RK_ERR_DIMENSION && throw(DimensionMismatch("librk: array extents do not agree"))
@@ -76,6 +82,12 @@ end
 
 dense(A::ROCArray) = true          # dense column-major storage: (pointer, dims) describes it completely
 dense(_) = false
+# wrappers over a ROCArray that are (pointer, size, strides) triples: operands / destinations of the *_strided entry points
+const ROCWrapper{T,N} = Union{SubArray{T,N,<:ROCArray}, LinearAlgebra.Transpose{T,<:ROCArray{T}},
+                              PermutedDimsArray{T,N,<:Any,<:Any,<:ROCArray}}
+is_strided_wrapper(x) = x isa ROCWrapper && eltype(x) <: Real && applicable(strides, x)
+const ROCStrided{T,N} = Union{ROCArray{T,N},ROCWrapper{T,N}}
+strides64(A, N) = Int64[k <= ndims(A) ? stride(A, k) : 0 for k in 1:N]
 
 # ---- mapreducedim! ------------------------------------------------------------------------------------------
 function native_mapreducedim!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N}, init) where {TR,TA,N}
@@ -96,7 +108,33 @@ function native_mapreducedim!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N}, init) w
                    initref === C_NULL ? C_NULL : Base.unsafe_convert(Ptr{Cvoid}, initref),
                    pointer(ws), length(ws), stream_ptr())
     end
-    st == RK_ERR_UNSUPPORTED && return false
+    declined(st) && return false
+    check(st)
+    return true
+end
+
+# R or A a transpose / PermutedDimsArray / contiguous view, e.g. mapreducedim!(identity, +, transpose(R), A): the
+# library renumbers the dims of permuted-dense arrays and declines (-> stock method) views with gaps
+function native_mapreducedim_strided!(f, op, R::ROCStrided{TR}, A::ROCStrided{TA,N}, init) where {TR,TA,N}
+    Base.check_reducedims(R, A)
+    isempty(A) && return true
+    mask = UInt32(0)
+    for d in 1:N
+        size(R, d) == size(A, d) || (mask |= UInt32(1) << (d - 1))
+    end
+    ws = workspace()
+    shape = Int64[size(A)...]
+    as, rs = strides64(A, N), strides64(R, N)
+    initref = init === nothing ? C_NULL : Ref(convert(TR, init))
+    GC.@preserve R A ws shape as rs initref begin
+        st = ccall((:rk_mapreduce_strided, librk[]), Int32,
+                   (Cint, Cint, Cint, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Int64},
+                    Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   rk_map(f), rk_op(op), rk_dtype(TA), rk_dtype(TR), pointer(A), N, shape, as, mask, pointer(R), rs,
+                   initref === C_NULL ? C_NULL : Base.unsafe_convert(Ptr{Cvoid}, initref),
+                   pointer(ws), length(ws), stream_ptr())
+    end
+    declined(st) && return false
     check(st)
     return true
 end
@@ -170,7 +208,7 @@ function native_mapreducedim_closure!(f, op, R::ROCArray{TR}, A::ROCArray{TA,N},
                    initref === C_NULL ? C_NULL : Base.unsafe_convert(Ptr{Cvoid}, initref),
                    pointer(ws), length(ws), stream_ptr())
     end
-    st == RK_ERR_UNSUPPORTED && return false
+    declined(st) && return false
     check(st)
     return true
 end
@@ -190,6 +228,14 @@ function enable_mapreduce!()
         end
         return invoke(GPUArrays.mapreducedim!, Tuple{F,OP,AnyROCArray{TR},Union{AbstractArray,Broadcasted}}, f, op, R, A; init)
     end
+    # at least one side a wrapper (the dense pair above is more specific)
+    @eval function GPUArrays.mapreducedim!(f::F, op::OP, R::ROCStrided{TR}, A::ROCStrided{TA}; init=nothing) where {F,OP,TR,TA}
+        if rk_map(f) !== nothing && rk_op(op) !== nothing && rk_dtype(TR) !== nothing && rk_dtype(TA) !== nothing &&
+           ndims(R) == ndims(A) && applicable(strides, R) && applicable(strides, A)
+            native_mapreducedim_strided!(f, op, R, A, init) && return R
+        end
+        return invoke(GPUArrays.mapreducedim!, Tuple{F,OP,AnyROCArray{TR},Union{AbstractArray,Broadcasted}}, f, op, R, A; init)
+    end
 end
 
 # ---- findmax / findmin ----------------------------------------------------------------------------------------
@@ -204,17 +250,22 @@ function native_findminmax(wantmax::Bool, A::ROCArray{T,N}, dims) where {T,N}
     ws = workspace()
     shape = Int64[size(A)...]
     GC.@preserve A vals idx ws shape begin
-        check(ccall((:rk_findminmax, librk[]), Int32,
-                    (Int32, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Int64}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
-                    wantmax, rk_dtype(T), pointer(A), N, shape, mask, pointer(vals),
-                    convert(Ptr{Int64}, pointer(idx)), pointer(ws), length(ws), stream_ptr()))
+        st = ccall((:rk_findminmax, librk[]), Int32,
+                   (Int32, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Int64}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   wantmax, rk_dtype(T), pointer(A), N, shape, mask, pointer(vals),
+                   convert(Ptr{Int64}, pointer(idx)), pointer(ws), length(ws), stream_ptr())
     end
+    declined(st) && return nothing
+    check(st)
     return vals, idx
 end
 function enable_findminmax!()
     for (fn, wantmax) in ((:findmax, true), (:findmin, false))
         @eval function Base.$fn(A::ROCArray{T,N}; dims=:) where {T<:Union{Float32,Float64,Int32,Int64},N}
-            vals, idx = native_findminmax($wantmax, A, dims)
+            isempty(A) && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)       # the stock method's error
+            res = native_findminmax($wantmax, A, dims)
+            res === nothing && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
+            vals, idx = res
             dims === Colon() || return vals, idx
             v = AMDGPU.@allowscalar vals[1]
             i = AMDGPU.@allowscalar idx[1]
@@ -239,7 +290,32 @@ function native_accumulate!(op, B::ROCArray{TB,N}, A::ROCArray{TA,N}; init, dims
                    rk_op(op), rk_dtype(TA), rk_dtype(TB), pointer(A), pointer(B), N, shape, dim, inclusive,
                    Base.unsafe_convert(Ptr{Cvoid}, initref), pointer(ws), length(ws), stream_ptr())
     end
-    st == RK_ERR_UNSUPPORTED && return false
+    declined(st) && return false
+    check(st)
+    return true
+end
+
+function native_accumulate_strided!(op, B::ROCStrided{TB,N}, A::ROCStrided{TA,N}; init, dims, inclusive::Bool) where {TB,TA,N}
+    size(B) == size(A) || throw(DimensionMismatch("accumulate!: $(size(B)) vs $(size(A))"))
+    isempty(A) && return true
+    dim = dims === nothing ? (N == 1 ? 1 : throw(ArgumentError("accumulate on N-d arrays needs dims"))) : Int(dims)
+    shape = Int64[size(A)...]
+    as, bs = strides64(A, N), strides64(B, N)
+    # the library scans the array in its order of dims in memory: size the bookkeeping for that numbering
+    order = sortperm(as)
+    mdim = dim <= N ? findfirst(==(dim), order) : N + 1
+    need = ccall((:rk_workspace_bytes, librk[]), Csize_t, (Cint, Cint, Cint, Ptr{Int64}, UInt32),
+                 2, rk_dtype(TB), N, shape[order], mdim <= N ? UInt32(1) << (mdim - 1) : UInt32(0))
+    ws = workspace(need)
+    initref = Ref(convert(TB, init))
+    GC.@preserve A B ws shape as bs initref begin
+        st = ccall((:rk_accumulate_strided, librk[]), Int32,
+                   (Cint, Cint, Cint, Ptr{Cvoid}, Ptr{Cvoid}, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Int64}, Cint, Int32, Ptr{Cvoid},
+                    Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   rk_op(op), rk_dtype(TA), rk_dtype(TB), pointer(A), pointer(B), N, shape, as, bs, dim, inclusive,
+                   Base.unsafe_convert(Ptr{Cvoid}, initref), pointer(ws), length(ws), stream_ptr())
+    end
+    declined(st) && return false
     check(st)
     return true
 end
@@ -248,6 +324,13 @@ function enable_accumulate!()
     @eval function Base.accumulate!(op, B::ROCArray, A::ROCArray; init=zero(eltype(A)), dims=nothing, inclusive::Bool=true, kwargs...)
         if isempty(kwargs) && rk_op(op) !== nothing && rk_dtype(eltype(A)) !== nothing && rk_dtype(eltype(B)) !== nothing
             native_accumulate!(op, B, A; init, dims, inclusive) && return B
+        end
+        return AMDGPU.AK.accumulate!(op, B, A, AMDGPU.ROCBackend(); init, dims, inclusive, kwargs...)
+    end
+    @eval function Base.accumulate!(op, B::ROCStrided, A::ROCStrided; init=zero(eltype(A)), dims=nothing, inclusive::Bool=true, kwargs...)
+        if isempty(kwargs) && rk_op(op) !== nothing && rk_dtype(eltype(A)) !== nothing && rk_dtype(eltype(B)) !== nothing &&
+           applicable(strides, A) && applicable(strides, B)
+            native_accumulate_strided!(op, B, A; init, dims, inclusive) && return B
         end
         return AMDGPU.AK.accumulate!(op, B, A, AMDGPU.ROCBackend(); init, dims, inclusive, kwargs...)
     end
@@ -265,10 +348,6 @@ struct RkOperand
     ptr::Ptr{Cvoid}; dtype::Int32; ndim::Int32; shape::NTuple{8,Int64}; scalar_f::Float64; scalar_i::Int64
     strided::Int32; reserved::Int32; strides::NTuple{8,Int64}
 end
-# wrappers over a ROCArray that are (pointer, size, strides) triples: operands / destinations of rk_broadcast_strided
-const ROCWrapper{T,N} = Union{SubArray{T,N,<:ROCArray}, LinearAlgebra.Transpose{T,<:ROCArray{T}},
-                              PermutedDimsArray{T,N,<:Any,<:Any,<:ROCArray}}
-is_strided_wrapper(x) = x isa ROCWrapper && eltype(x) <: Real && applicable(strides, x)
 const INT_SAFE = (Int32(32), Int32(33), Int32(34), Int32(36), Int32(37), Int32(39), Int32(64), Int32(65), Int32(66), Int32(74),
                   Int32.(96:103)..., Int32(112), Int32.(128:131)...)     # + comparisons, & |, ifelse, ! isodd iseven isnan
 # comparisons, max and min of 32-bit intermediates need RK_BC_WRAP_I32 (132) first; this binding keeps such programs
@@ -362,10 +441,12 @@ function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadc
     shape = Int64[size(dest)...]
     dstrides = dest isa ROCArray ? C_NULL : Int64[strides(dest)...]     # NULL = dense
     GC.@preserve dest ops prog shape dstrides begin
-        check(ccall((:rk_broadcast_strided, librk[]), Int32,
-                    (Ptr{RkProgram}, Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}),
-                    prog, pointer(dest), rk_dtype(TD), N, shape, dstrides, stream_ptr()))
+        st = ccall((:rk_broadcast_strided, librk[]), Int32,
+                   (Ptr{RkProgram}, Ptr{Cvoid}, Cint, Cint, Ptr{Int64}, Ptr{Int64}, Ptr{Cvoid}),
+                   prog, pointer(dest), rk_dtype(TD), N, shape, dstrides, stream_ptr())
     end
+    declined(st) && throw(Unsupported())
+    check(st)
     return dest
 end
 
@@ -450,7 +531,7 @@ function native_reverse!(y::ROCArray{T,N}, x::ROCArray{T,N}, dims) where {T,N}
         st = ccall((:rk_reverse, librk[]), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Cint, Ptr{Int64}, UInt32, Ptr{Cvoid}),
                    pointer(x), pointer(y), sizeof(T), N, shape, mask, stream_ptr())
     end
-    st == RK_ERR_UNSUPPORTED && return false
+    declined(st) && return false
     check(st)
     return true
 end
@@ -465,9 +546,11 @@ function enable_permutedims!()
         shape = Int64[size(src)...]
         p = Int32[perm...]
         GC.@preserve dest src shape p begin
-            check(ccall((:rk_permutedims, librk[]), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Cint, Ptr{Int64}, Ptr{Int32}, Ptr{Cvoid}),
-                        pointer(src), pointer(dest), sizeof(T), N, shape, p, stream_ptr()))
+            st = ccall((:rk_permutedims, librk[]), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Cint, Ptr{Int64}, Ptr{Int32}, Ptr{Cvoid}),
+                       pointer(src), pointer(dest), sizeof(T), N, shape, p, stream_ptr())
         end
+        declined(st) && return invoke(Base.permutedims!, Tuple{AMDGPU.AnyROCArray,AMDGPU.AnyROCArray,Any}, dest, src, perm)
+        check(st)
         return dest
     end
 end
@@ -483,10 +566,12 @@ function enable_sort!()
         n > 1 || return x
         tmp = ROCVector{UInt8}(undef, ccall((:rk_sort_tmp_bytes, librk[]), Csize_t, (Cint, Int64, Int32), rk_dtype(T), n, 0))
         GC.@preserve x tmp begin
-            check(ccall((:rk_sort, librk[]), Int32, (Cint, Ptr{Cvoid}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
-                        rk_dtype(T), pointer(x), n, rev, pointer(tmp), sizeof(tmp), stream_ptr()))
+            st = ccall((:rk_sort, librk[]), Int32, (Cint, Ptr{Cvoid}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                       rk_dtype(T), pointer(x), n, rev, pointer(tmp), sizeof(tmp), stream_ptr())
         end
         AMDGPU.unsafe_free!(tmp)
+        declined(st) && return (AMDGPU.AK.sort!(x; rev); x)          # rk_sort validates before it writes
+        check(st)
         return x
     end
     @eval function Base.sortperm!(ix::ROCVector{Int}, x::ROCVector{T}; rev::Bool=false, lt=isless, by=identity, kwargs...) where {T<:SORTABLE}
@@ -496,10 +581,12 @@ function enable_sort!()
         n > 0 || return ix
         tmp = ROCVector{UInt8}(undef, ccall((:rk_sort_tmp_bytes, librk[]), Csize_t, (Cint, Int64, Int32), rk_dtype(T), n, 1))
         GC.@preserve ix x tmp begin
-            check(ccall((:rk_sortperm, librk[]), Int32, (Cint, Ptr{Cvoid}, Ptr{Int64}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
-                        rk_dtype(T), pointer(x), pointer(ix), n, rev, pointer(tmp), sizeof(tmp), stream_ptr()))
+            st = ccall((:rk_sortperm, librk[]), Int32, (Cint, Ptr{Cvoid}, Ptr{Int64}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                       rk_dtype(T), pointer(x), pointer(ix), n, rev, pointer(tmp), sizeof(tmp), stream_ptr())
         end
         AMDGPU.unsafe_free!(tmp)
+        declined(st) && return (AMDGPU.AK.sortperm!(ix, x; rev); ix)
+        check(st)
         return ix
     end
 end

@@ -68,8 +68,10 @@ typedef enum {
     RK_U8  = 4,  /* Bool / UInt8 (one byte per element) */
     RK_U32 = 5,  /* UInt32  */
     RK_U64 = 6,  /* UInt64  */
-    RK_F16 = 7,  /* Float16 (sort / sortperm only; reverse and permutedims take any 2-byte element) */
-    RK_I16 = 8   /* Int16   (sort / sortperm only) */
+    RK_F16 = 7,  /* Float16: rk_mapreduce (accumulating in Float32), rk_findminmax, rk_broadcast operands and
+                  * destinations, rk_sort / rk_sortperm; not rk_accumulate (RK_ERR_UNSUPPORTED) */
+    RK_I16 = 8   /* Int16: rk_sort / rk_sortperm only.  rk_reverse and rk_permutedims take an element SIZE, not
+                  * a dtype, and so move any 2-byte element */
 } rk_dtype;
 
 /* f of mapreduce(f, op, A) */
@@ -90,7 +92,11 @@ RK_API const char* rk_status_string(int32_t status);
 
 /* Bytes of workspace that a call of `kind` on an array of `ndim`/`shape` with element
  * type `dt` needs (dims_mask: bit d-1 set = Julia dim d is reduced; for accumulate the
- * single scanned dim).  Never fails: bad arguments return the generic minimum.
+ * single scanned dim).  For RK_KIND_ACCUMULATE `dt` is the OUTPUT dtype of the scan -- the
+ * type the prefixes are carried in: cumsum of Bool into Int64 is sized with RK_I64, and
+ * sizing it with the input dtype would give half the descriptor words.  For the *_strided
+ * entry points pass the extents in the array's order of dims in memory.
+ * Never fails: bad arguments return the generic minimum.
  * A buffer of RK_WORKSPACE_DEFAULT bytes serves every call up to 2^31 elements. */
 #define RK_WORKSPACE_DEFAULT ((size_t)16 << 20)
 RK_API size_t  rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* shape,

@@ -311,3 +311,18 @@ def test_host_mirror_rules_without_gpu(rk):
     with pytest.raises(rk.UnsupportedError):
         B.compile_map(lambda x: B.isodd(x), np.float32)
     assert B._compile(B.lazy(np.float32(1)) > B.lazy(2))[4] == np.bool_
+
+
+def test_declined_statuses_raise_the_fallback_exception(L):
+    """Out-of-set operations, extents beyond the kernels' indexing and unusable workspaces are all `declined`: the one
+    exception a caller catches to take another path (the Julia binding runs the stock method for the same three)."""
+    for code in (L.RK_ERR_UNSUPPORTED, L.RK_ERR_TOO_LARGE, L.RK_ERR_WORKSPACE):
+        with pytest.raises(L.UnsupportedError) as e:
+            L.check(code, "probe")
+        assert e.value.status == code
+    for code in (L.RK_ERR_INVALID_ARGUMENT, L.RK_ERR_WAIT):
+        with pytest.raises(L.RKError) as e:
+            L.check(code, "probe")
+        assert not isinstance(e.value, L.UnsupportedError)
+    with pytest.raises(L.DimensionMismatch):
+        L.check(L.RK_ERR_DIMENSION, "probe")
