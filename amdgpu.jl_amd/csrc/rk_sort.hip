@@ -32,7 +32,6 @@
 namespace rk {
 
 constexpr int SORT_BLOCK = 256;
-constexpr size_t SORT_SCAN_SCRATCH = (size_t)2 << 20;
 constexpr int SORT_NW = SORT_BLOCK / WAVE;
 constexpr int SORT_MAX_PASSES = 8;
 
@@ -44,6 +43,8 @@ struct SortCtl {                                  // head of the caller's tempor
     uint32_t first_pass, last_pass, nexec;
     uint32_t wait_failed;                         // a look-back gave up its bounded wait (WaitCtl); read by rk_sort_status
     unsigned long long inv_min;                   // ~(smallest mapped key), kept as a maximum so that zero is its identity
+    unsigned long long key_max;                   // largest mapped key (large integer sorts: range = key_max - smallest)
+    uint32_t scan_ticket[SORT_MAX_PASSES];        // sort_tilescan_kernel: workgroups that have stored their chunk totals
 };
 
 // ---- key <-> ordered unsigned integer -----------------------------------------------------------------
@@ -150,6 +151,21 @@ __device__ __forceinline__ uint64_t match_digit(uint32_t d, uint64_t valid) {
     }
     return ~(((uint64_t)diff_hi << 32) | diff_lo) & valid;
 }
+// The same for the ranking of the pass kernel, which is bound by its vector instructions: four per bit (sign-extended
+// bit, compare into a lane mask, and one three-input bit operation same &= ~(m ^ e) for each half of the wave)
+// instead of the six the compiler makes of the plain form.  Call with all 64 lanes active.
+__device__ __forceinline__ void match_digit_halves(uint32_t d, uint32_t& same_lo, uint32_t& same_hi) {
+    same_lo = ~0u;
+    same_hi = ~0u;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const uint32_t e = (uint32_t)__builtin_amdgcn_sbfe((int)d, b, 1);
+        uint64_t m;
+        asm volatile("v_cmp_ne_u32_e64 %0, 0, %1" : "=s"(m) : "v"(e));
+        same_lo = __builtin_amdgcn_bitop3_b32(same_lo, (uint32_t)m, e, 0x90);             // a & ~(b ^ c)
+        same_hi = __builtin_amdgcn_bitop3_b32(same_hi, (uint32_t)(m >> 32), e, 0x90);
+    }
+}
 
 // Histogram updates in LDS.  Evenly spread digits go in with one LDS atomic per lane.  When many lanes hold the same
 // digit (exponent bytes, the high bytes of small integers) those atomics would queue up on one LDS word, so the
@@ -190,8 +206,8 @@ __device__ __forceinline__ void for_each_key(const T* __restrict__ keys, int64_t
     typedef typename VecOf<U, VEC>::type VU;
     const VU* body = (const VU*)(keys + head);
     constexpr int UNR = 4;                                   // loads in flight per lane
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     for (; i + (UNR - 1) * stride < nvec; i += UNR * stride) {
         VU v[UNR];
 #pragma unroll
@@ -213,7 +229,7 @@ __device__ __forceinline__ void for_each_key(const T* __restrict__ keys, int64_t
     }
     if (blockIdx.x == 0) {
         const int64_t tail0 = head + nvec * VEC, extra = head + (n - tail0);     // at most 2 * (VEC - 1) keys
-        for (int64_t i = threadIdx.x; i < extra; i += 256) {
+        for (int64_t i = threadIdx.x; i < extra; i += blockDim.x) {
             const int64_t e = i < head ? i : tail0 + (i - head);
             U k[VEC];
             k[0] = __builtin_bit_cast(U, keys[e]);
@@ -250,6 +266,39 @@ __global__ __launch_bounds__(256) void sort_min_kernel(const T* __restrict__ key
     }
 }
 
+// ---- smallest and largest mapped key (large integer sorts) ------------------------------------------------------------
+// Keys are taken relative to the smallest one, so their range tells which digits are zero in every key: the passes of
+// those digits are skipped.  One read at streaming speed; the large sorts do without the histogram read below.
+constexpr int MINMAX_BLOCK = 1024;      // few, large workgroups: each ends with two device-wide atomics on shared words
+template <typename T>
+__global__ __launch_bounds__(MINMAX_BLOCK) void sort_minmax_kernel(const T* __restrict__ keys, int64_t n, int64_t head, int64_t nvec, int rev,
+                                                                   SortCtl* ctl) {
+    typedef typename SortKey<T>::U U;
+    constexpr int VEC = 16 / sizeof(T);
+    __shared__ U part[2][MINMAX_BLOCK / WAVE];
+    U mn = (U)~(U)0, mx = 0;
+    for_each_key<T>(keys, n, head, nvec, [&](const U (&k)[VEC], int cnt) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            if (j < cnt) {
+                const U u = enc_bits<T>(k[j], rev, (U)0);
+                mn = u < mn ? u : mn;
+                mx = u > mx ? u : mx;
+            }
+        }
+    });
+    mn = wave_reduce(mn, OpMin());
+    mx = wave_reduce(mx, OpMax());
+    if (lane_id() == 0) { part[0][threadIdx.x / WAVE] = mn; part[1][threadIdx.x / WAVE] = mx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < MINMAX_BLOCK / WAVE; ++w) { mn = part[0][w] < mn ? part[0][w] : mn; mx = part[1][w] > mx ? part[1][w] : mx; }
+        const unsigned long long inv = (unsigned long long)(U)~mn;
+        if (inv != 0ull) atomicMax(&ctl->inv_min, inv);
+        if (mx != 0) atomicMax(&ctl->key_max, (unsigned long long)mx);
+    }
+}
+
 // ---- all digit histograms in one read -------------------------------------------------------------------------
 template <typename T, int PASSES>
 __global__ __launch_bounds__(256) void sort_hist_kernel(const T* __restrict__ keys, int64_t n, int64_t head, int64_t nvec, int rev,
@@ -279,24 +328,33 @@ __global__ __launch_bounds__(256) void sort_hist_kernel(const T* __restrict__ ke
 }
 
 // ---- plan: scan the histograms, decide which passes run and what they read ---------------------------------------
-// one workgroup of 256 threads; lane d owns digit value d
-__global__ __launch_bounds__(256) void sort_plan_kernel(SortCtl* ctl, int passes, uint32_t n, int first_reads_b) {
+// one workgroup of 256 threads; lane d owns digit value d.  mode 0: from the histograms of sort_hist_kernel.
+// mode 1 (large sorts of integers): from the range of the keys, histograms come later, pass by pass.
+// mode 2 (large sorts of floats): every pass runs, keys are not taken relative to the smallest.
+__global__ __launch_bounds__(256) void sort_plan_kernel(SortCtl* ctl, int passes, uint32_t n, int first_reads_b, int mode) {
     __shared__ uint32_t wsum[SORT_NW];
     __shared__ int any_full;
     const int d = threadIdx.x, wave = d / WAVE, lane = d % WAVE;
-    for (int p = 0; p < passes; ++p) {
-        const uint32_t c = ctl->hist[p][d];
-        if (d == 0) any_full = 0;
-        __syncthreads();
-        if (c == n) any_full = 1;
-        const uint32_t inc = wave_scan_inclusive(c, OpAdd(), 0u);
-        if (lane == WAVE - 1) wsum[wave] = inc;
-        __syncthreads();
-        uint32_t base = 0;
-        for (int w = 0; w < wave; ++w) base += wsum[w];
-        ctl->hist[p][d] = base + inc - c;
-        if (d == 0) ctl->skip[p] = any_full ? 1u : 0u;
-        __syncthreads();
+    if (mode == 0) {
+        for (int p = 0; p < passes; ++p) {
+            const uint32_t c = ctl->hist[p][d];
+            if (d == 0) any_full = 0;
+            __syncthreads();
+            if (c == n) any_full = 1;
+            const uint32_t inc = wave_scan_inclusive(c, OpAdd(), 0u);
+            if (lane == WAVE - 1) wsum[wave] = inc;
+            __syncthreads();
+            uint32_t base = 0;
+            for (int w = 0; w < wave; ++w) base += wsum[w];
+            ctl->hist[p][d] = base + inc - c;
+            if (d == 0) ctl->skip[p] = any_full ? 1u : 0u;
+            __syncthreads();
+        }
+    } else if (d == 0) {
+        if (mode == 2) ctl->inv_min = ~0ull;                          // smallest key taken as 0
+        const unsigned long long umin = ~ctl->inv_min;                 // high bits beyond the key width: ones in both, cancel below
+        const unsigned long long range = mode == 2 ? ~0ull : ctl->key_max - (umin & (passes == 8 ? ~0ull : ((1ull << (8 * passes)) - 1ull)));
+        for (int p = 0; p < passes; ++p) ctl->skip[p] = (range >> (8 * p)) == 0ull ? 1u : 0u;
     }
     if (d == 0) {
         uint32_t src_b = first_reads_b ? 1u : 0u, nexec = 0, first = 0xffffffffu, last = 0xffffffffu;
@@ -315,47 +373,179 @@ __global__ __launch_bounds__(256) void sort_plan_kernel(SortCtl* ctl, int passes
 }
 
 // ---- digit counts of every tile (large sorts) ---------------------------------------------------------------------
-// Same tiles as sort_pass_kernel, one per workgroup.  Lanes with the same digit find each other as in the pass
-// kernel, so skewed digits (exponent bytes, the high bytes of small integers) cost the same as uniform ones.
+// Same tiles as sort_pass_kernel, one per workgroup; the order of the keys inside the tile does not matter here, so
+// aligned full tiles are read as 16-byte vectors.  One LDS atomic per key into one of UPS_SUB histograms per wave,
+// chosen by the lane: skewed digits (exponent bytes, the high bytes of small integers) then queue up 16 deep on a
+// counter instead of 64 deep, and no lane has to find out who else holds its digit.
+constexpr int UPS_SUB = 4;
+
 template <typename T, int ITEMS>
-__global__ __launch_bounds__(SORT_BLOCK) void sort_upsweep_kernel(const T* __restrict__ orig, const typename SortKey<T>::U* buf_a,
+__global__ __launch_bounds__(SORT_BLOCK, 8) void sort_upsweep_kernel(const T* __restrict__ orig, const typename SortKey<T>::U* buf_a,
                                                                   const typename SortKey<T>::U* buf_b, uint32_t n, int pass, int rev,
                                                                   const SortCtl* ctl, uint32_t* __restrict__ tile_count) {
     typedef typename SortKey<T>::U U;
     constexpr int TILE = SORT_BLOCK * ITEMS;
-    __shared__ uint32_t cnt[SORT_NW][256];
+    constexpr int VEC = 16 / (int)sizeof(T), NV = ITEMS / VEC;
+    typedef typename VecOf<U, VEC>::type VU;
+    __shared__ uint32_t cnt[SORT_NW * UPS_SUB][256];
     if (ctl->skip[pass]) return;
     const bool first = (uint32_t)pass == ctl->first_pass;
     const U* in = first ? (const U*)orig : (ctl->src_is_b[pass] != 0u ? buf_b : buf_a);
+    const U umin = (U)~ctl->inv_min;
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-    for (int i = tid; i < SORT_NW * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
-    __syncthreads();
+    for (int i = tid; i < SORT_NW * UPS_SUB * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
     const uint32_t tile = blockIdx.x;
-    const uint32_t woff = tile * (uint32_t)TILE + (uint32_t)wave * (WAVE * ITEMS) + lane;
-    U key[ITEMS];
+    const uint32_t e0 = tile * (uint32_t)TILE;
+    const uint32_t woff = e0 + (uint32_t)wave * (WAVE * ITEMS) + lane;
+    uint32_t* row = cnt[wave * UPS_SUB + (lane & (UPS_SUB - 1))];
+    // (the two read paths share no variables: merged into one key array they made the compiler shuffle it through
+    // private memory)
+    if (e0 + (uint32_t)TILE <= n && (((uintptr_t)(in + e0)) & 15) == 0) {
+        const VU* vin = (const VU*)(in + e0);
+        VU v[NV];
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-        const uint32_t e = woff + i * WAVE;
-        key[i] = (U)~(U)0;
-        if (e < n) key[i] = in[e];
-    }
-    if (first) {
+        for (int r = 0; r < NV; ++r) v[r] = vin[r * SORT_BLOCK + tid];
+        __syncthreads();
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) key[i] = enc_bits<T>(key[i], rev, (U)~ctl->inv_min);   // padding keys are never counted
-    }
-    bool skewed = false;
+        for (int r = 0; r < NV; ++r) {
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-        const bool valid = woff + i * WAVE < n;
-        const uint32_t d = digit_of(key[i], pass);
-        if ((i & 3) == 0) skewed = digits_skewed(d, valid);                     // judged on every fourth round
-        count_digit(cnt[wave], d, valid, skewed);
+            for (int j = 0; j < VEC; ++j) {
+                U k = (U)v[r][j];
+                if (first) k = enc_bits<T>(k, rev, umin);
+                atomicAdd(&row[digit_of(k, pass)], 1u);
+            }
+        }
+    } else {
+        U key[ITEMS];
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const uint32_t e = woff + i * WAVE;
+            key[i] = (U)0;
+            if (e < n) key[i] = in[e];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const U k = first ? enc_bits<T>(key[i], rev, umin) : key[i];
+            if (woff + i * WAVE < n) atomicAdd(&row[digit_of(k, pass)], 1u);
+        }
     }
     __syncthreads();
     uint32_t c = 0;
 #pragma unroll
-    for (int w = 0; w < SORT_NW; ++w) c += cnt[w][tid];
+    for (int w = 0; w < SORT_NW * UPS_SUB; ++w) c += cnt[w][tid];
     tile_count[(uint64_t)tile * 256 + tid] = c;
+}
+
+// ---- where every tile's keys go (large sorts) --------------------------------------------------------------------------
+// Input: count[tile][digit].  Output, for sort_pass_kernel: count[tile][digit] becomes the number of keys of the digit in
+// the earlier tiles of the same chunk of `chunk_rows` tiles; chunk_prefix[chunk][digit] the number in all earlier chunks;
+// ctl->hist[pass][digit] the first output slot of the digit (exclusive scan of the digit totals).
+// One workgroup of 1024 threads per chunk: 4 groups of rows x 256 digits.  The workgroup that stores its chunk totals
+// last (a ticket) scans the totals of all chunks; nobody waits for anybody.  At most 256 chunks.
+constexpr int TS_GROUPS = 4, TS_BLOCK = TS_GROUPS * 256, TS_UNROLL = 16, TS_MAX_CHUNKS = 256;
+
+// Rows [first, first + rows) of column d of x (256 words a row), TS_UNROLL loads in flight: their sum; with WRITE,
+// out[row][d] = start + the sum of the rows in front.
+template <bool WRITE, bool COHERENT>
+__device__ __forceinline__ uint32_t ts_rows(const uint32_t* x, uint32_t first, uint32_t rows, uint32_t d, uint32_t start, uint32_t* out) {
+    uint32_t run = start;
+    for (uint32_t r = 0; r < rows; r += TS_UNROLL) {
+        uint32_t v[TS_UNROLL];
+#pragma unroll
+        for (int j = 0; j < TS_UNROLL; ++j) {
+            v[j] = 0;
+            if (r + j < rows) {
+                const uint32_t* q = x + (uint64_t)(first + r + j) * 256 + d;
+                v[j] = COHERENT ? load_agent(q) : *q;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TS_UNROLL; ++j) {
+            if (WRITE && r + j < rows) out[(uint64_t)(first + r + j) * 256 + d] = run;
+            run += v[j];
+        }
+    }
+    return run - start;
+}
+
+// Exclusive scan down rows [a, b) of column d, for the thread of row group g: out[row][d] = sum of the rows of the
+// column in front, over all groups; returns the column total.  Up to MAXR rows a group stay in registers between the
+// two steps (one round trip to memory); longer groups are read twice.
+template <int MAXR, bool COHERENT>
+__device__ __forceinline__ uint32_t ts_scan_groups(const uint32_t* x, uint32_t* out, uint32_t a, uint32_t b, uint32_t d, uint32_t g,
+                                                   uint32_t (*gsum)[256]) {
+    const uint32_t rows = b - a;
+    const bool in_regs = __syncthreads_and(rows <= (uint32_t)MAXR) != 0;
+    uint32_t v[MAXR];
+    uint32_t mine = 0;
+    if (in_regs) {
+#pragma unroll
+        for (int j = 0; j < MAXR; ++j) {
+            v[j] = 0;
+            if ((uint32_t)j < rows) {
+                const uint32_t* q = x + (uint64_t)(a + j) * 256 + d;
+                v[j] = COHERENT ? load_agent(q) : *q;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < MAXR; ++j) mine += v[j];
+    } else {
+        mine = ts_rows<false, COHERENT>(x, a, rows, d, 0u, nullptr);
+    }
+    gsum[g][d] = mine;
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int k = 0; k < TS_GROUPS; ++k) {
+        const uint32_t s = gsum[k][d];
+        if ((uint32_t)k < g) before += s;
+        total += s;
+    }
+    if (in_regs) {
+        uint32_t run = before;
+#pragma unroll
+        for (int j = 0; j < MAXR; ++j) {
+            if ((uint32_t)j < rows) out[(uint64_t)(a + j) * 256 + d] = run;
+            run += v[j];
+        }
+    } else {
+        ts_rows<true, COHERENT>(x, a, rows, d, before, out);
+    }
+    return total;
+}
+
+__global__ __launch_bounds__(TS_BLOCK) void sort_tilescan_kernel(SortCtl* ctl, int pass, uint32_t* count, uint32_t ntiles, uint32_t chunk_rows,
+                                                                 uint32_t* chunk_total, uint32_t* chunk_prefix) {
+    __shared__ uint32_t gsum[2][TS_GROUPS][256];
+    __shared__ uint32_t wsum[SORT_NW];
+    __shared__ uint32_t lds_ticket;
+    if (ctl->skip[pass]) return;
+    const uint32_t d = threadIdx.x & 255u, g = threadIdx.x >> 8, chunk = blockIdx.x, nchunks = gridDim.x;
+    {
+        const uint32_t r0 = chunk * chunk_rows, r1 = r0 + chunk_rows < ntiles ? r0 + chunk_rows : ntiles;
+        const uint32_t per = (r1 - r0 + TS_GROUPS - 1) / TS_GROUPS;
+        const uint32_t a = r0 + g * per < r1 ? r0 + g * per : r1, b = a + per < r1 ? a + per : r1;
+        const uint32_t total = ts_scan_groups<16, false>(count, count, a, b, d, g, gsum[0]);
+        if (g == 0) store_agent(chunk_total + (uint64_t)chunk * 256 + d, total);
+    }
+    publish_barrier();                       // this thread's total is visible device-wide ...
+    __syncthreads();                         // ... and so is every other thread's of this workgroup
+    if (threadIdx.x == 0) lds_ticket = atomicAdd(&ctl->scan_ticket[pass], 1u);
+    __syncthreads();
+    if (lds_ticket != nchunks - 1u) return;
+    // the last one: exclusive scan of the chunk totals down the chunks, then of the digit totals across the digits
+    const uint32_t per = (nchunks + TS_GROUPS - 1) / TS_GROUPS;
+    const uint32_t a = g * per < nchunks ? g * per : nchunks, b = a + per < nchunks ? a + per : nchunks;
+    const uint32_t total = ts_scan_groups<TS_MAX_CHUNKS / TS_GROUPS, true>(chunk_total, chunk_prefix, a, b, d, g, gsum[1]);
+    const uint32_t inc = wave_scan_inclusive(total, OpAdd(), 0u);          // the same in all four groups
+    if (g == 0 && d % WAVE == WAVE - 1) wsum[d / WAVE] = inc;
+    __syncthreads();
+    if (g == 0) {
+        uint32_t start = inc - total;
+        for (uint32_t w = 0; w < d / WAVE; ++w) start += wsum[w];
+        ctl->hist[pass][d] = start;
+    }
 }
 
 // ---- one pass ----------------------------------------------------------------------------------------------------
@@ -364,19 +554,23 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_upsweep_kernel(const T* __res
 // desc[tile][digit]: low half = count, high half = (pass + 1) << 2 | status (1 = count of this tile only,
 // 2 = count of this and all earlier tiles); written and read with relaxed device-scope atomics, so the count
 // always travels with its tag.
+// waves per SIMD the register allocation aims at: the kernel is bound by its vector instructions, and three or four
+// waves hide the latencies (measured: 4 against 6 workgroups a CU differ by 4%)
+template <typename T, bool PERM, bool COUNTED> constexpr int sort_pass_waves() { return (COUNTED && !PERM && sizeof(T) <= 4) ? 4 : 3; }
+
 template <typename T, int ITEMS, bool PERM, bool COUNTED>
-__global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restrict__ orig, typename SortKey<T>::U* buf_a,
+__global__ __launch_bounds__(SORT_BLOCK, (sort_pass_waves<T, PERM, COUNTED>())) void sort_pass_kernel(const T* __restrict__ orig, typename SortKey<T>::U* buf_a,
                                                                typename SortKey<T>::U* buf_b, uint32_t* val_a, uint32_t* val_b,
                                                                int64_t* __restrict__ perm_out, uint32_t n, int pass, int rev, SortCtl* ctl,
-                                                               uint64_t* desc, const uint32_t* __restrict__ tile_before, uint32_t ntiles,
-                                                               long long wait_rounds) {
+                                                               uint64_t* desc, const uint32_t* __restrict__ tile_before,
+                                                               const uint32_t* __restrict__ chunk_prefix, uint32_t chunk_rows,
+                                                               uint32_t ntiles, long long wait_rounds, uint32_t xcd_chunk) {
     typedef typename SortKey<T>::U U;
     constexpr int TILE = SORT_BLOCK * ITEMS;
     __shared__ U lds_keys[TILE];
     __shared__ uint32_t lds_vals[PERM ? TILE : 1];
-    __shared__ uint32_t cnt[SORT_NW][256];        // per wave and digit: count, then offset of the wave inside the digit
-    __shared__ uint32_t tile_start[256];          // first slot of the digit in the sorted tile
-    __shared__ uint32_t goff[256];                // global slot of the digit's first key of this tile, minus tile_start
+    __shared__ uint32_t cnt[SORT_NW][256];        // per wave and digit: count, then slot in the sorted tile of the wave's first key of the digit
+    __shared__ uint32_t goff[256];                // global slot of the digit's first key of this tile, minus its slot in the sorted tile
     __shared__ uint32_t wsum[SORT_NW];
     __shared__ uint32_t lds_tile;
 
@@ -389,9 +583,12 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
     const uint32_t* vsrc = src_b ? val_b : val_a;
     uint32_t* vdst = src_b ? val_a : val_b;
     const uint32_t tag_a = ((uint32_t)(pass + 1) << 2) | 1u, tag_p = ((uint32_t)(pass + 1) << 2) | 2u;
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-
     for (uint32_t round = 0;; ++round) {
+        // everything derived from the thread's index is computed again for every tile: hoisted out of this loop it
+        // would sit in some 35 registers (16 of them tid + i * 256) across the whole kernel
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int wave = tid / WAVE, lane = tid % WAVE;
         if (!COUNTED && tid == 0) {
             // once a look-back of this call has given up its wait the result is lost: no further tile starts
             const uint32_t failed = __hip_atomic_load(&ctl->wait_failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -400,7 +597,11 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
         }
         for (int i = tid; i < SORT_NW * 256; i += SORT_BLOCK) (&cnt[0][0])[i] = 0;
         __syncthreads();
-        const uint32_t tile = COUNTED ? blockIdx.x + round * gridDim.x : lds_tile;
+        uint32_t tile = COUNTED ? blockIdx.x + round * gridDim.x : lds_tile;
+        if (COUNTED && xcd_chunk != 0u) {
+            const uint32_t i = (blockIdx.x >> 3) + round * (gridDim.x >> 3);
+            tile = i < xcd_chunk ? (blockIdx.x & 7u) * xcd_chunk + i : ntiles;
+        }
         if (tile >= ntiles) return;
         const uint32_t e0 = tile * (uint32_t)TILE;
         const uint32_t woff = e0 + (uint32_t)wave * (WAVE * ITEMS) + lane;
@@ -432,38 +633,52 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
     #pragma unroll
                 for (int i = 0; i < ITEMS; ++i) key[i] = enc_bits<T>(key[i], rev, umin);    // padding keys are never counted
             }
-            // rank inside the wave: lanes with the same digit find each other with 8 ballots; the lowest of them adds
-            // their number to the wave's counter of that digit.  The adds are LDS atomics that return the old value:
-            // LDS serves a wave's requests in order, so the 16 rounds queue up back to back with no wait in between
-            // (a plain read-modify-write needs a round trip per round).
-            uint32_t who[ITEMS];                     // leader lane | lanes below with the same digit << 8
+            // rank inside the wave: lanes with the same digit find each other with 8 ballots; every lane reads the
+            // wave's counter of its digit -- the rank of the group's first key -- and then the lowest lane of the group
+            // adds the size of the group to it.  LDS executes the instructions of one wave in order, so the read of
+            // the next round sees this add, and the 16 rounds queue up back to back; a result is used two rounds later.
+            uint32_t* wcnt = cnt[wave];
+            constexpr int DEPTH = 2;                       // counter reads in flight before their result is used
+            uint32_t pend_before[DEPTH], pend_below[DEPTH];
     #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 const bool valid = FULL || woff + i * WAVE < n;
                 const uint32_t d = digit_of(key[i], pass);
-                const uint64_t peers = match_digit(d, __ballot(valid));
-                const int leader = valid ? __ffsll((unsigned long long)peers) - 1 : 0;
-                const uint32_t below = __builtin_amdgcn_mbcnt_hi((uint32_t)(peers >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)peers, 0u));
-                who[i] = (uint32_t)leader | (below << 8);
-                rank[i] = 0;
-                if (valid && lane == leader) rank[i] = atomicAdd(&cnt[wave][d], (uint32_t)__popcll(peers));
+                uint32_t same_lo, same_hi;
+                match_digit_halves(d, same_lo, same_hi);
+                if (!FULL) {
+                    const uint64_t vm = __ballot(valid);
+                    same_lo &= (uint32_t)vm;
+                    same_hi &= (uint32_t)(vm >> 32);
+                }
+                const uint32_t below = __builtin_amdgcn_mbcnt_hi(same_hi, __builtin_amdgcn_mbcnt_lo(same_lo, 0u));
+                const uint32_t before = __hip_atomic_load(&wcnt[d], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                __builtin_amdgcn_wave_barrier();
+                if (valid && below == 0u) {
+                    const uint32_t total = (uint32_t)__builtin_popcount(same_lo) + (uint32_t)__builtin_popcount(same_hi);
+                    __hip_atomic_fetch_add(&wcnt[d], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+                }
+                if (i >= DEPTH) rank[i - DEPTH] = pend_before[i % DEPTH] + pend_below[i % DEPTH];
+                pend_before[i % DEPTH] = before;
+                pend_below[i % DEPTH] = below;
+                __builtin_amdgcn_sched_barrier(0);
             }
     #pragma unroll
-            for (int i = 0; i < ITEMS; ++i) rank[i] = (uint32_t)__shfl((int)rank[i], (int)(who[i] & 0xffu)) + (who[i] >> 8);
+            for (int i = ITEMS; i < ITEMS + DEPTH; ++i) rank[i - DEPTH] = pend_before[i % DEPTH] + pend_below[i % DEPTH];
             __syncthreads();
-            // digit d = tid: count of the tile, offsets of the waves inside the digit
+            // digit d = tid: count of the tile and of each wave
+            uint32_t wave_count[SORT_NW];
             uint32_t count = 0;
     #pragma unroll
             for (int w = 0; w < SORT_NW; ++w) {
-                const uint32_t c = cnt[w][tid];
-                cnt[w][tid] = count;
-                count += c;
+                wave_count[w] = cnt[w][tid];
+                count += wave_count[w];
             }
             // publish the count, then look back over the earlier tiles for this digit
             uint64_t* my = desc + (uint64_t)tile * 256 + tid;
             uint32_t excl = 0;
             if constexpr (COUNTED) {
-                excl = tile_before[(uint64_t)tile * 256 + tid];
+                excl = tile_before[(uint64_t)tile * 256 + tid] + chunk_prefix[(uint64_t)(tile / chunk_rows) * 256 + tid];
             } else if (tile == 0) {
                 __hip_atomic_store(my, ((uint64_t)tag_p << 32) | count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else {
@@ -505,15 +720,20 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
             __syncthreads();
             uint32_t start = inc - count;
             for (int w = 0; w < wave; ++w) start += wsum[w];
-            tile_start[tid] = start;
             goff[tid] = ctl->hist[pass][tid] + excl - start;
+    #pragma unroll
+            for (int w = 0; w < SORT_NW; ++w) {
+                cnt[w][tid] = start;
+                start += wave_count[w];
+            }
             __syncthreads();
             // reorder the tile in LDS
     #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 if (FULL || woff + i * WAVE < n) {
-                    const uint32_t d = digit_of(key[i], pass);
-                    const uint32_t pos = tile_start[d] + cnt[wave][d] + rank[i];
+                    uint32_t d = digit_of(key[i], pass);
+                    asm volatile("" : "+v"(d));            // computed again here: 16 LDS addresses kept from the ranking cost a wave of occupancy
+                    const uint32_t pos = wcnt[d] + rank[i];
                     lds_keys[pos] = key[i];
                     if constexpr (PERM) lds_vals[pos] = val[i];
                 }
@@ -528,8 +748,9 @@ __global__ __launch_bounds__(SORT_BLOCK) void sort_pass_kernel(const T* __restri
                     const uint32_t slot = goff[digit_of(u, pass)] + q;
                     // slot < n always holds in a sound sort.  After a look-back has given up its wait (WaitCtl) the
                     // offsets are too small and this pass leaves holes; the next pass then reads keys the histograms
-                    // never counted, and its slots can lie anywhere: keep every store inside the arrays.
-                    if (slot >= n) continue;
+                    // never counted, and its slots can lie anywhere: keep every store inside the arrays.  (The large
+                    // sorts count every tile of every pass themselves and wait for nobody.)
+                    if (!COUNTED && slot >= n) continue;
                     if constexpr (PERM) {
                         if (last) perm_out[slot] = (int64_t)lds_vals[q] + 1;
                         else { dst[slot] = u; vdst[slot] = lds_vals[q]; }
@@ -561,8 +782,8 @@ __global__ __launch_bounds__(256) void sort_finish_kernel(const SortCtl* ctl, W*
 
 // ---- host --------------------------------------------------------------------------------------------------------
 struct SortLayout {
-    size_t desc_off, clear_end, scratch_off, keys_b_off, keys_a_off, val_a_off, val_b_off, total;
-    uint32_t ntiles;
+    size_t desc_off, clear_end, chunk_total_off, chunk_prefix_off, keys_b_off, keys_a_off, val_a_off, val_b_off, total;
+    uint32_t ntiles, chunk_rows, nchunks;
     bool counted;          // large sort: desc_off holds the per-tile digit counts (uint32) instead of descriptors
 };
 
@@ -586,8 +807,10 @@ static SortLayout sort_layout(size_t key_size, int items, int64_t n, bool perm) 
     if (l.counted) {
         l.clear_end = off;                                   // only the control block needs clearing
         off += (size_t)l.ntiles * 256 * sizeof(uint32_t);
-        l.scratch_off = off;
-        off += SORT_SCAN_SCRATCH;
+        l.chunk_rows = (l.ntiles + TS_MAX_CHUNKS - 1) / TS_MAX_CHUNKS;
+        l.nchunks = (l.ntiles + l.chunk_rows - 1) / l.chunk_rows;
+        l.chunk_total_off = off;  off += (size_t)TS_MAX_CHUNKS * 256 * sizeof(uint32_t);
+        l.chunk_prefix_off = off; off += (size_t)TS_MAX_CHUNKS * 256 * sizeof(uint32_t);
     } else {
         off += (size_t)l.ntiles * 256 * sizeof(uint64_t);
         l.clear_end = off;
@@ -633,30 +856,43 @@ static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, voi
     const int64_t nvec = (n - head) / KVEC;
     // few workgroups: each ends with device-wide atomics on shared words (1 for the minimum, 256 per digit position)
     const unsigned gmin = (unsigned)(g < cus * 2 ? g : cus * 2), ghist = (unsigned)(g < cus * 4 ? g : cus * 4);
-    sort_min_kernel<T><<<gmin, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
-    RK_LAUNCH_CHECK();
-    sort_hist_kernel<T, PASSES><<<ghist, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
-    RK_LAUNCH_CHECK();
     // sortperm: the first pass reads the caller's keys and should write buffer A, i.e. "reads B"
-    sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0);
+    if (!l.counted) {
+        sort_min_kernel<T><<<gmin, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+        RK_LAUNCH_CHECK();
+        sort_hist_kernel<T, PASSES><<<ghist, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+        RK_LAUNCH_CHECK();
+        sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0, 0);
+    } else if (std::is_integral<T>::value) {
+        sort_minmax_kernel<T><<<gmin, MINMAX_BLOCK, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+        RK_LAUNCH_CHECK();
+        sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0, 1);
+    } else {
+        // floats: the digits of a large array are hardly ever constant, so no read is spent on finding out
+        sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0, 2);
+    }
     RK_LAUNCH_CHECK();
-    unsigned pgrid = l.ntiles < (unsigned)(cus * 4) ? l.ntiles : (unsigned)(cus * 4);
+    static const int wgs_per_cu = [] { const char* e = std::getenv("RK_SORT_WGS_PER_CU"); const int x = e ? std::atoi(e) : 0; return x > 0 ? x : 6; }();
+    static const int xcd_map = [] { const char* e = std::getenv("RK_SORT_XCD"); return e ? std::atoi(e) : 1; }();
+    unsigned pgrid = l.ntiles < (unsigned)(cus * wgs_per_cu) ? l.ntiles : (unsigned)(cus * wgs_per_cu);
+    // large sorts: each XCD takes a contiguous eighth of the tiles, so the runs that neighbouring tiles write next to
+    // each other meet in one L2 (workgroups go to the XCDs round-robin by their index)
+    const uint32_t xcd_chunk = (xcd_map != 0 && l.counted && pgrid % 8u == 0u) ? (l.ntiles + 7u) / 8u : 0u;
     uint32_t* tile_count = (uint32_t*)desc;
+    uint32_t* chunk_total = l.counted ? (uint32_t*)(base + l.chunk_total_off) : nullptr;
+    uint32_t* chunk_prefix = l.counted ? (uint32_t*)(base + l.chunk_prefix_off) : nullptr;
+    const long long wb = wait_budget();
     for (int p = 0; p < PASSES; ++p) {
         if (l.counted) {
             sort_upsweep_kernel<T, ITEMS><<<l.ntiles, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, (uint32_t)n, p, rev, ctl, tile_count);
             RK_LAUNCH_CHECK();
-            // counts -> keys of the digit in earlier tiles: exclusive scan down the tiles, in place.  A skipped pass
-            // scans stale numbers that nobody reads (the host cannot know which passes are skipped).
-            const ScanGeom sg{256, (int64_t)l.ntiles, 1};
-            const int32_t st = scan_across_rows<uint32_t, uint32_t, OpAdd>(tile_count, tile_count, sg, 0u, 0, OpAdd(), true,
-                                                                          base + l.scratch_off, SORT_SCAN_SCRATCH, stream);
-            if (st != RK_SUCCESS) return st;
-            if (perm) sort_pass_kernel<T, ITEMS, true, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles, wait_budget());
-            else sort_pass_kernel<T, ITEMS, false, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, tile_count, l.ntiles, wait_budget());
+            sort_tilescan_kernel<<<l.nchunks, TS_BLOCK, 0, stream>>>(ctl, p, tile_count, l.ntiles, l.chunk_rows, chunk_total, chunk_prefix);
+            RK_LAUNCH_CHECK();
+            if (perm) sort_pass_kernel<T, ITEMS, true, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, tile_count, chunk_prefix, l.chunk_rows, l.ntiles, wb, xcd_chunk);
+            else sort_pass_kernel<T, ITEMS, false, true><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, tile_count, chunk_prefix, l.chunk_rows, l.ntiles, wb, xcd_chunk);
         } else {
-            if (perm) sort_pass_kernel<T, ITEMS, true, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles, wait_budget());
-            else sort_pass_kernel<T, ITEMS, false, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, nullptr, l.ntiles, wait_budget());
+            if (perm) sort_pass_kernel<T, ITEMS, true, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, val_a, val_b, perm_out, (uint32_t)n, p, rev, ctl, desc, nullptr, nullptr, 1u, l.ntiles, wb, 0u);
+            else sort_pass_kernel<T, ITEMS, false, false><<<pgrid, SORT_BLOCK, 0, stream>>>((const T*)keys, buf_a, buf_b, nullptr, nullptr, nullptr, (uint32_t)n, p, rev, ctl, desc, nullptr, nullptr, 1u, l.ntiles, wb, 0u);
         }
         RK_LAUNCH_CHECK();
     }

@@ -79,6 +79,46 @@ def test_full_size_sort(rk, orc):
     assert np.array_equal(p, orc.sortperm(k, True))
 
 
+# More than 1024 tiles of 4096 keys: the sort counts the digits of every tile before each pass (no look-back).
+LARGE = 1024 * 4096 + 4096 * 3 + 37
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+def test_large_sorts_all_types(rk, orc, dtype):
+    _check(rk, orc, _rand(np.random.default_rng(11), dtype, LARGE))
+
+
+@pytest.mark.parametrize("dtype", [np.int16, np.int32, np.int64])
+def test_large_small_range_integers(rk, orc, dtype):
+    rng = np.random.default_rng(12)
+    _check(rk, orc, rng.integers(-10, 11, LARGE).astype(dtype))                    # one pass: the range fits a digit
+    _check(rk, orc, rng.integers(-300, 70_000 if dtype != np.int16 else 3_000, LARGE).astype(dtype))
+    _check(rk, orc, np.full(LARGE, -5, dtype=dtype))                               # every pass skipped
+    _check(rk, orc, (rng.integers(0, 2, LARGE) * 256).astype(dtype))               # low digit constant, not skipped
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_large_special_floats(rk, orc, dtype):
+    rng = np.random.default_rng(13)
+    base = np.array([0.0, -0.0, np.nan, np.inf, -np.inf, 1.0, -1.0, 65504.0, -65504.0, 6e-8, -6e-8], dtype=dtype)
+    x = rng.choice(base, LARGE)
+    x[::7] = -x[::7]
+    _check(rk, orc, x)
+    _check(rk, orc, (1.0 + rng.random(LARGE)).astype(dtype))                       # one binade: exponent digits constant
+
+
+def test_large_unaligned_view(rk, orc):
+    x = _rand(np.random.default_rng(14), np.float32, LARGE + 10)
+    d = rk.ROCArray(x)
+    v = d.view_range(4, LARGE + 6)                                                 # starts 12 bytes into the buffer
+    assert np.array_equal(rk.Array(rk.sort(v)), orc.sort(x[3:LARGE + 6]))
+    assert np.array_equal(rk.Array(rk.sortperm(v, rev=True)), orc.sortperm(x[3:LARGE + 6], True))
+    rk.sort_(v)
+    got = rk.Array(d)
+    assert np.array_equal(got[3:LARGE + 6], orc.sort(x[3:LARGE + 6]))
+    assert np.array_equal(got[:3], x[:3]) and np.array_equal(got[LARGE + 6:], x[LARGE + 6:])
+
+
 @pytest.mark.parametrize("dtype", [np.int16, np.float32, np.float64])
 def test_unaligned_views(rk, orc, dtype):
     # keys that start 1 .. 9 elements into a buffer: the vector body of the whole-array reads starts later
