@@ -1,27 +1,33 @@
 // sort! / sortperm! of vectors (src/kernels/sorting.jl:1-3, which forwards to AcceleratedKernels' merge sort):
-// least-significant-digit radix sort, 8 bits per pass, one kernel per pass.
+// least-significant-digit radix sort, 8 bits per pass.
 //
-//   sort_init_kernel     clears the histograms, the tile tickets and the tile descriptors (no memset: graph-safe)
+//   sort_init_kernel     clears the control block (and the tile descriptors of small sorts); no memset: graph-safe
+//   sort_pass_kernel     a tile of 4096 keys ranks its keys by digit (wave-level match by ballots, counts in LDS), learns
+//                        how many keys of each digit the earlier tiles hold, reorders the tile in LDS and writes runs of
+//                        equal digits.  The kernel is bound by its vector instructions (about 75 a key, 32 of them the
+//                        match), not by memory.
+//   sort_finish_kernel   moves the result into the caller's array when an odd number of passes ran
+//
+// Up to 256 tiles (RK_SORT_LOOKBACK_TILES; 2^20 keys) the counts of the earlier tiles come from a chained look-back (tiles in
+// ticket order publish their 256 counts, one lane per digit walks back), and a pass reads and writes every key once:
 //   sort_min_kernel      one read of the keys: the smallest mapped key, which every key is taken relative to
 //   sort_hist_kernel     one read of the keys: the 256-bin histogram of every digit at once
 //   sort_plan_kernel     exclusive scan of every histogram = first output slot of each digit value; passes whose
 //                        digit is the same for all keys are skipped (small-range integers need 1-2 passes);
 //                        records which buffer each remaining pass reads
-//   sort_pass_kernel     a tile ranks its keys by digit (wave-level match by ballots, counts in LDS), learns how
-//                        many keys of each digit the earlier tiles hold, reorders the tile in LDS and writes runs of
-//                        equal digits.  Up to 1024 tiles (a tunable) the counts of the earlier tiles come from a
-//                        chained look-back (tiles in ticket order publish their 256 counts, one lane per digit walks
-//                        back): a pass reads and writes every key once.  Beyond that the walk is the bottleneck --
-//                        a descriptor is 2 KiB per step against 16 KiB of keys per tile, and the thousand tiles in
-//                        flight resolve their prefixes nearly one after the other (measured: half of the pass) --
-//                        so large sorts count first:
-//   sort_upsweep_kernel  the 256 digit counts of every tile (one more read of the keys), then an exclusive scan
-//                        down the tiles (the strided scan of the accumulate path) gives every tile its offsets.
-//   sort_finish_kernel   moves the result into the caller's array when an odd number of passes ran
+// Beyond that the walk becomes the bottleneck -- a descriptor is 2 KiB per step against 16 KiB of keys per tile, and the
+// tiles in flight resolve their prefixes nearly one after the other (2^22 Float32: 388 us against 146 us) -- so large
+// sorts count before every pass instead:
+//   sort_minmax_kernel   integers only: smallest and largest key in one read; passes above the range are skipped
+//   sort_upsweep_kernel  the 256 digit counts of every tile (one more read of the keys, at streaming speed)
+//   sort_tilescan_kernel exclusive scan of the counts down the tiles in one launch (chunks of tiles; the workgroup
+//                        that finishes last scans the chunk totals and the digit totals)
+// and their pass kernel gives each XCD a contiguous eighth of the tiles.
 //
 // Keys are mapped to unsigned integers that sort like Base.isless (-0.0 < 0.0, NaN last; sortperm makes every NaN the
-// canonical one so that they are equal keys, sort! keeps their bit patterns), complemented for rev=true; the mapping is applied on the first read and undone on the last
-// write.  The sort is stable, so sortperm keeps equal keys in index order (also with rev=true, as Base does).
+// canonical one so that they are equal keys, sort! keeps their bit patterns), complemented for rev=true; the mapping is
+// applied on the first read and undone on the last write.  The sort is stable, so sortperm keeps equal keys in index
+// order (also with rev=true, as Base does).
 #include <cstddef>
 #include <cstdlib>
 #include <type_traits>
@@ -398,6 +404,27 @@ __global__ __launch_bounds__(SORT_BLOCK, 8) void sort_upsweep_kernel(const T* __
     const uint32_t e0 = tile * (uint32_t)TILE;
     const uint32_t woff = e0 + (uint32_t)wave * (WAVE * ITEMS) + lane;
     uint32_t* row = cnt[wave * UPS_SUB + (lane & (UPS_SUB - 1))];
+    // When many lanes hold the same digit (judged on every fourth key) the two most frequent values -- as seen from the
+    // first lane still in play -- are taken out with a ballot each and added by that lane alone; uniform floats have
+    // 50% and 37% of their keys in two values of the exponent digit.
+    bool skewed = false;
+    auto count = [&](uint32_t d, bool valid, int i) {
+        if ((i & 3) == 0) skewed = digits_skewed(d, valid);
+        if (skewed) {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint64_t active = __ballot(valid);
+                if (active != 0ull) {
+                    const int head = __ffsll((unsigned long long)active) - 1;
+                    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d, head);
+                    const uint64_t same = __ballot(valid && d == d0);
+                    if (lane == head) atomicAdd(&row[d0], (uint32_t)__popcll(same));
+                    valid = valid && d != d0;
+                }
+            }
+        }
+        if (valid) atomicAdd(&row[d], 1u);
+    };
     // (the two read paths share no variables: merged into one key array they made the compiler shuffle it through
     // private memory)
     if (e0 + (uint32_t)TILE <= n && (((uintptr_t)(in + e0)) & 15) == 0) {
@@ -412,7 +439,7 @@ __global__ __launch_bounds__(SORT_BLOCK, 8) void sort_upsweep_kernel(const T* __
             for (int j = 0; j < VEC; ++j) {
                 U k = (U)v[r][j];
                 if (first) k = enc_bits<T>(k, rev, umin);
-                atomicAdd(&row[digit_of(k, pass)], 1u);
+                count(digit_of(k, pass), true, r * VEC + j);
             }
         }
     } else {
@@ -427,7 +454,7 @@ __global__ __launch_bounds__(SORT_BLOCK, 8) void sort_upsweep_kernel(const T* __
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
             const U k = first ? enc_bits<T>(key[i], rev, umin) : key[i];
-            if (woff + i * WAVE < n) atomicAdd(&row[digit_of(k, pass)], 1u);
+            count(digit_of(k, pass), woff + i * WAVE < n, i);
         }
     }
     __syncthreads();
@@ -727,38 +754,59 @@ __global__ __launch_bounds__(SORT_BLOCK, (sort_pass_waves<T, PERM, COUNTED>())) 
                 start += wave_count[w];
             }
             __syncthreads();
-            // reorder the tile in LDS
+            // reorder the tile in LDS.  Reads first, writes after, so that the 16 table reads are in flight together.
+    #pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                uint32_t d = digit_of(key[i], pass);
+                asm volatile("" : "+v"(d));            // computed again here: 16 LDS addresses kept from the ranking cost a wave of occupancy
+                rank[i] += wcnt[d];
+            }
     #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 if (FULL || woff + i * WAVE < n) {
-                    uint32_t d = digit_of(key[i], pass);
-                    asm volatile("" : "+v"(d));            // computed again here: 16 LDS addresses kept from the ranking cost a wave of occupancy
-                    const uint32_t pos = wcnt[d] + rank[i];
-                    lds_keys[pos] = key[i];
-                    if constexpr (PERM) lds_vals[pos] = val[i];
+                    lds_keys[rank[i]] = key[i];
+                    if constexpr (PERM) lds_vals[rank[i]] = val[i];
                 }
             }
             __syncthreads();
+            // write runs of equal digits: thread q takes the q-th key of the sorted tile.  Again all reads of a kind
+            // together; `last` is decided once, not per key.
             const uint32_t valid_n = n - e0 < (uint32_t)TILE ? n - e0 : (uint32_t)TILE;
+            U out_key[ITEMS];
+            uint32_t slot[ITEMS];
     #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
                 const uint32_t q = (uint32_t)tid + i * SORT_BLOCK;
-                if (FULL || q < valid_n) {
-                    const U u = lds_keys[q];
-                    const uint32_t slot = goff[digit_of(u, pass)] + q;
-                    // slot < n always holds in a sound sort.  After a look-back has given up its wait (WaitCtl) the
-                    // offsets are too small and this pass leaves holes; the next pass then reads keys the histograms
-                    // never counted, and its slots can lie anywhere: keep every store inside the arrays.  (The large
-                    // sorts count every tile of every pass themselves and wait for nobody.)
-                    if (!COUNTED && slot >= n) continue;
-                    if constexpr (PERM) {
-                        if (last) perm_out[slot] = (int64_t)lds_vals[q] + 1;
-                        else { dst[slot] = u; vdst[slot] = lds_vals[q]; }
-                    } else {
-                        if (last) ((T*)dst)[slot] = dec_bits<T>(u, rev, umin);
-                        else dst[slot] = u;
-                    }
+                out_key[i] = (U)0;
+                if (FULL || q < valid_n) out_key[i] = lds_keys[q];
+            }
+    #pragma unroll
+            for (int i = 0; i < ITEMS; ++i) slot[i] = goff[digit_of(out_key[i], pass)] + (uint32_t)tid + i * SORT_BLOCK;
+            // slot < n always holds in a sound sort.  After a look-back has given up its wait (WaitCtl) the offsets are
+            // too small and this pass leaves holes; the next pass then reads keys the histograms never counted, and
+            // its slots can lie anywhere: keep every store inside the arrays.  (The large sorts count every tile of
+            // every pass themselves and wait for nobody.)
+            auto writable = [&](int i) { return (FULL || (uint32_t)tid + i * SORT_BLOCK < valid_n) && (COUNTED || slot[i] < n); };
+            if constexpr (PERM) {
+                uint32_t out_val[ITEMS];
+    #pragma unroll
+                for (int i = 0; i < ITEMS; ++i) {
+                    out_val[i] = 0;
+                    if (FULL || (uint32_t)tid + i * SORT_BLOCK < valid_n) out_val[i] = lds_vals[(uint32_t)tid + i * SORT_BLOCK];
                 }
+                if (last) {
+    #pragma unroll
+                    for (int i = 0; i < ITEMS; ++i) if (writable(i)) perm_out[slot[i]] = (int64_t)out_val[i] + 1;
+                } else {
+    #pragma unroll
+                    for (int i = 0; i < ITEMS; ++i) if (writable(i)) { dst[slot[i]] = out_key[i]; vdst[slot[i]] = out_val[i]; }
+                }
+            } else if (last) {
+    #pragma unroll
+                for (int i = 0; i < ITEMS; ++i) if (writable(i)) ((T*)dst)[slot[i]] = dec_bits<T>(out_key[i], rev, umin);
+            } else {
+    #pragma unroll
+                for (int i = 0; i < ITEMS; ++i) if (writable(i)) dst[slot[i]] = out_key[i];
             }
         };
         if (e0 + (uint32_t)TILE <= n) sort_tile(std::true_type{}); else sort_tile(std::false_type{});
@@ -793,7 +841,7 @@ template <typename T> constexpr int sort_items() { return sort_items_for(sizeof(
 
 // More tiles than this: count first, no look-back (RK_SORT_LOOKBACK_TILES).
 static uint32_t sort_lookback_tiles() {
-    static const uint32_t v = [] { const char* e = std::getenv("RK_SORT_LOOKBACK_TILES"); const long x = e ? std::atol(e) : 0; return x > 0 ? (uint32_t)x : 1024u; }();
+    static const uint32_t v = [] { const char* e = std::getenv("RK_SORT_LOOKBACK_TILES"); const long x = e ? std::atol(e) : 0; return x > 0 ? (uint32_t)x : 256u; }();
     return v;
 }
 
@@ -872,9 +920,14 @@ static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, voi
         sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0, 2);
     }
     RK_LAUNCH_CHECK();
-    static const int wgs_per_cu = [] { const char* e = std::getenv("RK_SORT_WGS_PER_CU"); const int x = e ? std::atoi(e) : 0; return x > 0 ? x : 6; }();
+    // tunables, read once: workgroups of the pass kernel per CU (RK_SORT_WGS_PER_CU), XCD-contiguous tiles (RK_SORT_XCD=0: off).
+    // Large sorts launch one workgroup per tile unless told otherwise: the hardware's dispatcher balances the load
+    // better than a fixed share of tiles per resident workgroup (2^26 Float32: 866 against 986 us with 4 a CU).
+    static const int wgs_per_cu = [] { const char* e = std::getenv("RK_SORT_WGS_PER_CU"); const int x = e ? std::atoi(e) : 0; return x > 0 ? x : 0; }();
     static const int xcd_map = [] { const char* e = std::getenv("RK_SORT_XCD"); return e ? std::atoi(e) : 1; }();
-    unsigned pgrid = l.ntiles < (unsigned)(cus * wgs_per_cu) ? l.ntiles : (unsigned)(cus * wgs_per_cu);
+    unsigned pgrid;
+    if (l.counted && wgs_per_cu == 0) pgrid = (l.ntiles + 7u) & ~7u;
+    else { const unsigned cap = (unsigned)(cus * (wgs_per_cu > 0 ? wgs_per_cu : 6)); pgrid = l.ntiles < cap ? l.ntiles : cap; }
     // large sorts: each XCD takes a contiguous eighth of the tiles, so the runs that neighbouring tiles write next to
     // each other meet in one L2 (workgroups go to the XCDs round-robin by their index)
     const uint32_t xcd_chunk = (xcd_map != 0 && l.counted && pgrid % 8u == 0u) ? (l.ntiles + 7u) / 8u : 0u;

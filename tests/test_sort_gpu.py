@@ -79,7 +79,7 @@ def test_full_size_sort(rk, orc):
     assert np.array_equal(p, orc.sortperm(k, True))
 
 
-# More than 1024 tiles of 4096 keys: the sort counts the digits of every tile before each pass (no look-back).
+# More than 256 tiles of 4096 keys: the sort counts the digits of every tile before each pass (no look-back).
 LARGE = 1024 * 4096 + 4096 * 3 + 37
 
 
