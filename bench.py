@@ -40,7 +40,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 N_HEAD = 1 << 26
-TRAFFIC_BC_2_26 = 1_073_341_440   # measured HBM bytes per launch of the dominant kernel (algorithmic: 2^30)
+TRAFFIC_BC_2_26 = 1_073_318_912   # measured HBM bytes per launch of the dominant kernel (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel; algorithmic: 2^30)
 
 
 def parse():
@@ -271,7 +271,7 @@ def main():
             roofline = {"bound": "hbm", "kernel": "bc_kernel<EvalAxpbyExp,float,4,linear> (z .= a.*x .+ y.*exp.(w), 2^26 elts)",
                         "achieved": round(bytes_bc / (bc_avg * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": round(bytes_bc / (bc_avg * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/headline_step_pmc_fetch_write.txt):
+                        # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE (profiles/bench_rows_pmc_fetch_write.txt):
                         # (393238.3 KiB x 1.9999 + 262144.0 KiB x 0.9986), factors from the plain copy kernel of the same runs
                         "traffic": TRAFFIC_BC_2_26,
                         "bytes_per_launch": bytes_bc, "avg_launch_us": round(bc_avg * 1e3, 2)}
