@@ -170,9 +170,28 @@ template <typename T, int BUDGET>
 __global__ __launch_bounds__(PERM_SLAB_THREADS) void permute_slab_kernel(const T* __restrict__ src, T* __restrict__ dst, PermSlabGeom g) {
     __shared__ T lds[perm_slab_lds_elems(BUDGET)];
     const PermSlabBox box = perm_slab_box(g, (int64_t)blockIdx.x);
-    perm_slab_load(g, box, (int32_t)threadIdx.x, src, lds);
+    constexpr int V = PermSlabVec<T>::V;
+    struct alignas(16) Vec { T e[V]; };
+    if (perm_slab_load_vec_ok<T>(g, box, src)) {
+        perm_slab_load_vec<T>(g, box, (int32_t)threadIdx.x, [&](int64_t off, T (&out)[V]) {
+            const Vec v = *(const Vec*)(src + off);
+#pragma unroll
+            for (int j = 0; j < V; ++j) out[j] = v.e[j];
+        }, lds);
+    } else {
+        perm_slab_load(g, box, (int32_t)threadIdx.x, src, lds);
+    }
     __syncthreads();
-    perm_slab_store(g, box, (int32_t)threadIdx.x, lds, dst);
+    if (perm_slab_store_vec_ok<T>(g, box, dst)) {
+        perm_slab_store_vec<T>(g, box, (int32_t)threadIdx.x, lds, [&](int64_t off, const T (&in)[V]) {
+            Vec v;
+#pragma unroll
+            for (int j = 0; j < V; ++j) v.e[j] = in[j];
+            *(Vec*)(dst + off) = v;
+        });
+    } else {
+        perm_slab_store(g, box, (int32_t)threadIdx.x, lds, dst);
+    }
 }
 
 template <int E>
