@@ -473,6 +473,17 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_indexed_kernel(const BcArgs a) {
         const BcOperand& o = a.op[k];
         if (o.ptr == nullptr || (o.flat_dense != 0 && valid == VEC)) {
             load_operand<CT, VEC, false, HOMOG>(o, e0, false, in[k]);
+        } else if (o.stride0 == 0 && s0 >= (uint32_t)(VEC - 1) && valid == VEC) {
+            // extruded along dim 0 (a row vector against a matrix with short columns): the thread's VEC consecutive
+            // elements cross at most one column boundary, so the first and the last offset serve all of them -- two
+            // single loads instead of VEC (3 x N .+ 1 x N Float32: 61.8 -> 58.7 us)
+            CT first[1], last[1];
+            const int64_t off_a = (int64_t)c[0][1] * o.stride[0] + (int64_t)c[0][2] * o.stride[1] + (int64_t)c[0][3] * o.stride[2];
+            const int64_t off_b = (int64_t)c[VEC - 1][1] * o.stride[0] + (int64_t)c[VEC - 1][2] * o.stride[1] + (int64_t)c[VEC - 1][3] * o.stride[2];
+            load_typed<CT, 1, true, HOMOG>(o, off_a, true, false, first);
+            load_typed<CT, 1, true, HOMOG>(o, off_b, true, false, last);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) in[k][j] = (c[0][0] + (uint32_t)j < s0) ? first[0] : last[0];
         } else {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {

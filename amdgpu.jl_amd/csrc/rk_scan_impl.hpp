@@ -662,15 +662,23 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
     typedef typename VecOf<In, VEC>::type VI;
     typedef typename VecOf<T, VEC>::type VT;
     const int nv = ne / VEC;
-    for (int i = t; i < nv; i += 256) {
-        if constexpr (VEC == 1) {
-            lds[i] = (T)p[i];
-        } else {
-            const VI v = load_nt((const VI*)p + i);
-            VT w;
+    if constexpr (VEC == 1) {
+        for (int i = t; i < nv; i += 256) lds[i] = (T)p[i];
+    } else {
+        // at most TE / VEC / 256 = 4 vectors a thread: all loads issued before the first LDS write
+        constexpr int ROUNDS = TE / VEC / 256;
+        VI v[ROUNDS];
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) w[j] = (T)v[j];
-            ((VT*)lds)[i] = w;
+        for (int r = 0; r < ROUNDS; ++r)
+            if (t + r * 256 < nv) v[r] = load_nt((const VI*)p + t + r * 256);
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            if (t + r * 256 < nv) {
+                VT w;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) w[j] = (T)v[r][j];
+                ((VT*)lds)[t + r * 256] = w;
+            }
         }
     }
     for (int e = nv * VEC + t; e < ne; e += 256) lds[e] = (T)p[e];           // fewer than VEC elements
@@ -689,6 +697,18 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
         const bool live = l < nl && k0 < m;                // empty segments sit at the end of a group: nothing reads them
         const int sl = live ? l / inner : 0;
         T* line = lds + (live ? sl * slab + (l - sl * inner) : 0);
+        if (tpl_log2 == 0) {
+            // a lane per line: one sweep, init folded in
+            if (live) {
+                T run = init;
+                if (inclusive) {
+                    for (int k = 0; k < m; ++k) { run = op(run, line[k * inner]); line[k * inner] = run; }
+                } else {
+                    for (int k = 0; k < m; ++k) { const T x = line[k * inner]; line[k * inner] = run; run = op(run, x); }
+                }
+            }
+            continue;
+        }
         T tot = init;
         if (live) {
             tot = line[k0 * inner];
@@ -713,9 +733,13 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
         }
     }
     __syncthreads();
-    for (int i = t; i < nv; i += 256) {
-        if constexpr (VEC == 1) q[i] = lds[i];
-        else store_nt((VT*)q + i, ((const VT*)lds)[i]);
+    if constexpr (VEC == 1) {
+        for (int i = t; i < nv; i += 256) q[i] = lds[i];
+    } else {
+        constexpr int ROUNDS = TE / VEC / 256;
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r)
+            if (t + r * 256 < nv) store_nt((VT*)q + t + r * 256, ((const VT*)lds)[t + r * 256]);
     }
     for (int e = nv * VEC + t; e < ne; e += 256) q[e] = lds[e];
 }
@@ -1298,9 +1322,18 @@ inline int32_t launch_scan(const ScanArgs& a) {
                 if (spb / q > 0) spb -= spb % q;
                 else vector = false;
             }
-            const int lines = spb * (int)s.inner;
+            int lines = spb * (int)s.inner;
             int tl = 0;
             while (tl < 6 && (lines << tl) < 256 && (2 << tl) <= s.mid) ++tl;            // up to a wave per line
+            if (tl == 0 && lines > 256) {
+                // a lane per line: whole rounds of 256 lines (273 lines of 15 elements are two rounds, the second with
+                // 17 busy lanes); slabs per block stay a multiple of what keeps the blocks 16-byte aligned
+                int q = 1;
+                if (vector) { q = VEC; for (int64_t e = slab; q > 1 && e % 2 == 0; e /= 2) q /= 2; }
+                for (int cand = spb; cand * 4 >= spb * 3 && cand > 0; cand -= q) {
+                    if ((cand * (int)s.inner) % 256 == 0) { spb = cand; lines = spb * (int)s.inner; break; }
+                }
+            }
             if ((lines << tl) >= 128) {                                       // else too few lanes would scan
                 const int64_t blocks = (s.outer + spb - 1) / spb;
                 if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
