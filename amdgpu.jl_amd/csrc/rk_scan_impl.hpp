@@ -1032,10 +1032,18 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
                     const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
                     if ((ballotX & needed) == 0ull) {
                         const int cnt = np >= 0 ? np : WAVE;
-                        for (int d = 0; d < cnt; ++d) {
-                            const VT x = load_agent((const VT*)(gpayA + ((first - d) * nchains + chain) * COLS + lane * VEC));
+                        for (int d0 = 0; d0 < cnt; d0 += 4) {               // four aggregates a round trip
+                            VT x[4];
 #pragma unroll
-                            for (int j = 0; j < VEC; ++j) acc[j] = op(x[j], acc[j]);
+                            for (int u = 0; u < 4; ++u)
+                                if (d0 + u < cnt) x[u] = load_agent((const VT*)(gpayA + ((first - d0 - u) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                if (d0 + u < cnt) {
+#pragma unroll
+                                    for (int j = 0; j < VEC; ++j) acc[j] = op(x[u][j], acc[j]);
+                                }
+                            }
                         }
                         if (np >= 0) {
                             if (np >= rem) {                                // ran off the first group: nothing but init in front
@@ -1062,46 +1070,62 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
                 if (lane == 0) __hip_atomic_store(&gflag[(grp - 1) * nchains + chain], (uint64_t)tagP << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         } else {
-            // totals of the predecessors inside the group
+            // totals of the predecessors inside the group, and the group's base from its leader.  A tile that is not
+            // the last of its group needs both before it can go on, so it polls the flags of both together and then has
+            // all payloads in flight at once: two round trips instead of four.  The last tile of a group first owes
+            // its successors the group aggregate, which needs the predecessors only.
             T local[VEC];
 #pragma unroll
             for (int j = 0; j < VEC; ++j) local[j] = ident;
+            const bool owes_group = r == ROWS_GROUP - 1 && has_reader;
+            const bool with_base = grp > 0 && !owes_group;          // lane 63 polls the leader's flag in the same rounds
             for (;;) {
-                uint32_t st = DESC_A;
+                uint32_t ok = 1;
                 if (lane < r) {
                     const uint32_t tag = (uint32_t)(__hip_atomic_load(&desc[(slice - 1 - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
-                    st = tag == tagA ? DESC_A : 0u;
+                    ok = tag == tagA ? 1u : 0u;
+                } else if (with_base && lane == WAVE - 1) {
+                    ok = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
                 }
-                if (__ballot(st == 0u) == 0ull) break;
+                if (__ballot(ok == 0u) == 0ull) break;
                 if (wait_give_up(wc, rounds)) break;
             }
-            for (int d = 0; d < r; ++d) {
-                const VT x = load_agent((const VT*)(payload + ((slice - 1 - d) * nchains + chain) * COLS + lane * VEC));
+            VT gbase;
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) local[j] = op(x[j], local[j]);
+            for (int j = 0; j < VEC; ++j) gbase[j] = init;
+            {
+                VT x[ROWS_GROUP - 1];
+#pragma unroll
+                for (int d = 0; d < ROWS_GROUP - 1; ++d)
+                    if (d < r) x[d] = load_agent((const VT*)(payload + ((slice - 1 - d) * nchains + chain) * COLS + lane * VEC));
+                if (with_base) gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                for (int d = 0; d < ROWS_GROUP - 1; ++d) {
+                    if (d < r) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) local[j] = op(x[d][j], local[j]);
+                    }
+                }
             }
-            if (r == ROWS_GROUP - 1 && has_reader) {     // aggregate of the whole group, as soon as it is known
+            if (owes_group) {                            // aggregate of the whole group, as soon as it is known
                 VT t;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) t[j] = op(local[j], tot[j]);
                 store_agent((VT*)(gpayA + (grp * nchains + chain) * COLS + lane * VEC), t);
                 publish_barrier();
                 if (lane == 0) __hip_atomic_store(&gflag[grp * nchains + chain], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            if (grp > 0) {                               // the group's base, from its leader
-                for (;;) {
-                    uint32_t st = 0;
-                    if (lane == 0) st = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
-                    if (__builtin_amdgcn_readfirstlane((int)st) != 0) break;
-                    if (wait_give_up(wc, rounds)) break;
+                if (grp > 0) {                           // then the group's base, from its leader
+                    for (;;) {
+                        uint32_t st = 0;
+                        if (lane == 0) st = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
+                        if (__builtin_amdgcn_readfirstlane((int)st) != 0) break;
+                        if (wait_give_up(wc, rounds)) break;
+                    }
+                    gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
                 }
-                const VT x = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) base[j] = op(x[j], local[j]);
-            } else {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) base[j] = op(init, local[j]);
             }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) base[j] = op(gbase[j], local[j]);      // a published prefix contains init
         }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) lds_base[lane * VEC + j] = base[j];
