@@ -34,7 +34,7 @@ RK_ERR_WAIT = 10006
 RK_STATIC_SCRATCH_BYTES = 16 << 20
 
 # rk_dtype
-RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16 = range(9)
+RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16, RK_I8, RK_U16 = range(11)
 # rk_map
 RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
 RK_MAP_MAX_TOKENS, RK_MAP_MAX_CONSTS = 16, 4
@@ -48,7 +48,8 @@ RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE, RK_KIND_FINDALL = ran
  RK_BC_INV, RK_BC_IDENTITY) = range(64, 75)
 (RK_BC_LT, RK_BC_LE, RK_BC_GT, RK_BC_GE, RK_BC_EQ, RK_BC_NE, RK_BC_AND, RK_BC_OR) = range(96, 104)
 RK_BC_IFELSE = 112
-(RK_BC_NOT, RK_BC_ISODD, RK_BC_ISEVEN, RK_BC_ISNAN, RK_BC_WRAP_I32, RK_BC_WRAP_U32, RK_BC_ROUND_F16) = range(128, 135)
+(RK_BC_NOT, RK_BC_ISODD, RK_BC_ISEVEN, RK_BC_ISNAN, RK_BC_WRAP_I32, RK_BC_WRAP_U32, RK_BC_ROUND_F16,
+ RK_BC_WRAP_I8, RK_BC_WRAP_U8, RK_BC_WRAP_I16, RK_BC_WRAP_U16) = range(128, 139)
 
 
 class RkOperand(C.Structure):

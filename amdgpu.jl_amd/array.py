@@ -18,6 +18,7 @@ _DTYPE_CODE = {
     np.dtype(np.bool_): L.RK_U8, np.dtype(np.uint8): L.RK_U8,
     np.dtype(np.uint32): L.RK_U32, np.dtype(np.uint64): L.RK_U64,
     np.dtype(np.float16): L.RK_F16, np.dtype(np.int16): L.RK_I16,
+    np.dtype(np.int8): L.RK_I8, np.dtype(np.uint16): L.RK_U16,
 }
 
 

@@ -232,11 +232,15 @@ def _emit(bc: Broadcasted, operands: list, tokens: list, types: dict, int_progra
         tokens.append(L.RK_BC_ROUND_F16)
 
 
+_WRAP_TOKEN = {np.dtype(np.int32): L.RK_BC_WRAP_I32, np.dtype(np.uint32): L.RK_BC_WRAP_U32,
+               np.dtype(np.int8): L.RK_BC_WRAP_I8, np.dtype(np.uint8): L.RK_BC_WRAP_U8,
+               np.dtype(np.int16): L.RK_BC_WRAP_I16, np.dtype(np.uint16): L.RK_BC_WRAP_U16}
+
+
 def _wrap(t: np.dtype, tokens: list):
-    if t == np.int32:
-        tokens.append(L.RK_BC_WRAP_I32)
-    elif t == np.uint32:
-        tokens.append(L.RK_BC_WRAP_U32)
+    tok = _WRAP_TOKEN.get(np.dtype(t))
+    if tok is not None:
+        tokens.append(tok)
 
 
 def _compile_tree(tree: Broadcasted, operands: list):

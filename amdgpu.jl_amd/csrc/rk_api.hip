@@ -110,7 +110,7 @@ long long wait_budget() {
     return v;
 }
 
-static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_I16; }   // unsupported combinations fail in the dispatch
+static bool valid_dtype(int dt) { return dt >= RK_F32 && dt <= RK_U16; }   // unsupported combinations fail in the dispatch
 
 static bool valid_shape(int ndim, const int64_t* shape, int64_t* total) {
     if (ndim < 0 || ndim > RK_MAX_DIMS) return false;
@@ -259,6 +259,9 @@ static int32_t mapreduce_dispatch(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
             case RK_I32: return mapreduce_i32(a);
             case RK_I64: return mapreduce_i64(a);
             case RK_U8:  return mapreduce_u8(a);
+            case RK_I8:  return mapreduce_i8(a);
+            case RK_I16: return mapreduce_i16(a);
+            case RK_U16: return mapreduce_u16(a);
             case RK_U32: return mapreduce_u32(a);
             case RK_U64: return mapreduce_u64(a);
             default: return RK_ERR_UNSUPPORTED;
@@ -267,6 +270,9 @@ static int32_t mapreduce_dispatch(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
     if (in == RK_I32 && out == RK_I64) return mapreduce_i32_i64(a);
     if (in == RK_U8 && (out == RK_I64 || out == RK_U64)) return mapreduce_u8_i64(a);   // sums of bytes: the same bits either way
     if (in == RK_U32 && out == RK_U64) return mapreduce_u32_u64(a);
+    if (in == RK_I8 && out == RK_I64) return mapreduce_i8_i64(a);
+    if (in == RK_I16 && out == RK_I64) return mapreduce_i16_i64(a);
+    if (in == RK_U16 && out == RK_U64) return mapreduce_u16_u64(a);
     return RK_ERR_UNSUPPORTED;
 }
 
@@ -419,6 +425,9 @@ int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, co
         case RK_I32: return findminmax_i32(a);
         case RK_I64: return findminmax_i64(a);
         case RK_U8:  return findminmax_u8(a);
+        case RK_I8:  return findminmax_i8(a);
+        case RK_I16: return findminmax_i16(a);
+        case RK_U16: return findminmax_u16(a);
         case RK_U32: return findminmax_u32(a);
         case RK_U64: return findminmax_u64(a);
         default: return RK_ERR_UNSUPPORTED;

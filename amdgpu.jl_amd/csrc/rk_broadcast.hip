@@ -105,6 +105,9 @@ __device__ __forceinline__ void load_typed(const BcOperand& o, int64_t off, bool
         case RK_U32: load_as<CT, uint32_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         case RK_U64: load_as<CT, uint64_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         case RK_F16: load_as<CT, half_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_I8:  load_as<CT, int8_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_I16: load_as<CT, int16_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
+        case RK_U16: load_as<CT, uint16_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
         default:     load_as<CT, uint8_t, VEC, CACHED>(o.ptr, off, contiguous, wave_uniform, v); break;
     }
 }
@@ -148,6 +151,9 @@ __device__ __forceinline__ void store_dest(void* p, int dtype, int64_t off, cons
         case RK_U32: store_as<CT, uint32_t, VEC>(p, off, v); break;
         case RK_U64: store_as<CT, uint64_t, VEC>(p, off, v); break;
         case RK_F16: store_as<CT, half_t, VEC>(p, off, v); break;
+        case RK_I8:  store_as<CT, int8_t, VEC>(p, off, v); break;
+        case RK_I16: store_as<CT, int16_t, VEC>(p, off, v); break;
+        case RK_U16: store_as<CT, uint16_t, VEC>(p, off, v); break;
         default:     store_as<CT, uint8_t, VEC>(p, off, v); break;
     }
 }
@@ -603,8 +609,7 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
                               const int64_t* dest_strides, void* stream) {
     if (prog == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (ndim < 0 || ndim > RK_MAX_DIMS || (ndim > 0 && shape == nullptr)) return RK_ERR_INVALID_ARGUMENT;
-    if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_I16) return RK_ERR_INVALID_ARGUMENT;
-    if (dest_dtype == RK_I16) return RK_ERR_UNSUPPORTED;
+    if ((int)dest_dtype < RK_F32 || (int)dest_dtype > RK_U16) return RK_ERR_INVALID_ARGUMENT;
     if (prog->compute != RK_F32 && prog->compute != RK_F64 && prog->compute != RK_I64) return RK_ERR_UNSUPPORTED;
     const bool int_compute = prog->compute == RK_I64;
     if (dest_dtype == RK_F16 && int_compute) return RK_ERR_UNSUPPORTED;
@@ -635,8 +640,8 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
     }
     for (int k = 0; k < prog->n_operands; ++k) {
         const rk_operand& o = prog->operands[k];
-        if (o.dtype < RK_F32 || o.dtype > RK_I16) return RK_ERR_INVALID_ARGUMENT;
-        if (o.dtype == RK_I16 || (o.dtype == RK_F16 && int_compute)) return RK_ERR_UNSUPPORTED;
+        if (o.dtype < RK_F32 || o.dtype > RK_U16) return RK_ERR_INVALID_ARGUMENT;
+        if (o.dtype == RK_F16 && int_compute) return RK_ERR_UNSUPPORTED;
         if (o.ptr == nullptr) {
             if (o.ndim != 0) return RK_ERR_INVALID_ARGUMENT;
             for (int d = 0; d < ndim; ++d) stride[k][d] = 0;

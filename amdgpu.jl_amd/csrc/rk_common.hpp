@@ -32,8 +32,8 @@ inline size_t dtype_size(int dt) {
     switch (dt) {
         case RK_F32: case RK_I32: case RK_U32: return 4;
         case RK_F64: case RK_I64: case RK_U64: return 8;
-        case RK_U8: return 1;
-        case RK_F16: case RK_I16: return 2;
+        case RK_U8: case RK_I8: return 1;
+        case RK_F16: case RK_I16: case RK_U16: return 2;
         default: return 0;
     }
 }
@@ -351,6 +351,9 @@ template <> struct Limits<int64_t>  { static __host__ __device__ int64_t lowest(
 template <> struct Limits<uint32_t> { static __host__ __device__ uint32_t lowest() { return 0; } static __host__ __device__ uint32_t highest() { return UINT32_MAX; } };
 template <> struct Limits<uint64_t> { static __host__ __device__ uint64_t lowest() { return 0; } static __host__ __device__ uint64_t highest() { return UINT64_MAX; } };
 template <> struct Limits<uint8_t>  { static __host__ __device__ uint8_t lowest() { return 0; } static __host__ __device__ uint8_t highest() { return 255; } };
+template <> struct Limits<int8_t>   { static __host__ __device__ int8_t lowest() { return INT8_MIN; } static __host__ __device__ int8_t highest() { return INT8_MAX; } };
+template <> struct Limits<int16_t>  { static __host__ __device__ int16_t lowest() { return INT16_MIN; } static __host__ __device__ int16_t highest() { return INT16_MAX; } };
+template <> struct Limits<uint16_t> { static __host__ __device__ uint16_t lowest() { return 0; } static __host__ __device__ uint16_t highest() { return UINT16_MAX; } };
 
 // Integer arithmetic wraps like Julia's: do it on the unsigned counterpart.
 template <typename T> __host__ __device__ __forceinline__ T wrap_add(T a, T b) {
@@ -455,6 +458,25 @@ template <> struct OrderKey<uint64_t> {
     static constexpr bool LOWEST_FREE = false;
     static __device__ __forceinline__ Key make(uint64_t v, bool want_max) { const Key k = (Key)(v ^ 0x8000000000000000ull); return want_max ? k : ~k; }
     static __device__ __forceinline__ uint64_t value(Key k, bool want_max) { return (uint64_t)(want_max ? k : ~k) ^ 0x8000000000000000ull; }
+};
+// narrow integers: a 32-bit key has room below the smallest value
+template <> struct OrderKey<int8_t> {
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
+    static __device__ __forceinline__ Key make(int8_t v, bool want_max) { return want_max ? (Key)v : ~(Key)v; }
+    static __device__ __forceinline__ int8_t value(Key k, bool want_max) { return (int8_t)(want_max ? k : ~k); }
+};
+template <> struct OrderKey<int16_t> {
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
+    static __device__ __forceinline__ Key make(int16_t v, bool want_max) { return want_max ? (Key)v : ~(Key)v; }
+    static __device__ __forceinline__ int16_t value(Key k, bool want_max) { return (int16_t)(want_max ? k : ~k); }
+};
+template <> struct OrderKey<uint16_t> {
+    typedef int32_t Key;
+    static constexpr bool LOWEST_FREE = true;
+    static __device__ __forceinline__ Key make(uint16_t v, bool want_max) { return want_max ? (Key)v : ~(Key)v; }
+    static __device__ __forceinline__ uint16_t value(Key k, bool want_max) { return (uint16_t)(want_max ? k : ~k); }
 };
 template <> struct OrderKey<uint8_t> {            // Bool / UInt8: findfirst(bools) is findmax's index
     typedef int32_t Key;

@@ -15,7 +15,7 @@ __host__ __device__ constexpr int token_arity(int tok) {
            : (tok >= RK_BC_NEG && tok <= RK_BC_IDENTITY) ? 1
            : (tok >= RK_BC_LT && tok <= RK_BC_OR)      ? 2
            : (tok == RK_BC_IFELSE)                     ? 3
-           : (tok >= RK_BC_NOT && tok <= RK_BC_ROUND_F16) ? 1
+           : (tok >= RK_BC_NOT && tok <= RK_BC_WRAP_U16) ? 1
                                                        : -1;
 }
 
@@ -24,10 +24,10 @@ __host__ __device__ constexpr int token_arity(int tok) {
 __host__ __device__ constexpr bool token_int_ok(int tok) {
     return tok == RK_BC_ADD || tok == RK_BC_SUB || tok == RK_BC_MUL || tok == RK_BC_MAX || tok == RK_BC_MIN || tok == RK_BC_FMA ||
            tok == RK_BC_NEG || tok == RK_BC_ABS || tok == RK_BC_ABS2 || tok == RK_BC_IDENTITY || (tok >= RK_BC_LT && tok <= RK_BC_OR) ||
-           tok == RK_BC_IFELSE || (tok >= RK_BC_NOT && tok <= RK_BC_WRAP_U32);
+           tok == RK_BC_IFELSE || (tok >= RK_BC_NOT && tok <= RK_BC_WRAP_U32) || (tok >= RK_BC_WRAP_I8 && tok <= RK_BC_WRAP_U16);
 }
 __host__ __device__ constexpr bool token_float_ok(int tok) {
-    return tok != RK_BC_ISODD && tok != RK_BC_ISEVEN && tok != RK_BC_WRAP_I32 && tok != RK_BC_WRAP_U32;
+    return tok != RK_BC_ISODD && tok != RK_BC_ISEVEN && tok != RK_BC_WRAP_I32 && tok != RK_BC_WRAP_U32 && !(tok >= RK_BC_WRAP_I8 && tok <= RK_BC_WRAP_U16);
 }
 
 // pow and the trigonometric / hyperbolic functions exist in the full interpreter only
@@ -173,6 +173,10 @@ __device__ __forceinline__ void interp_run(const Tokens& tokens, int n_tokens, c
                         case RK_BC_ISNAN: RK_BC_UN(x * CT(0));
                         case RK_BC_WRAP_I32: RK_BC_UN((CT)(int32_t)x);
                         case RK_BC_WRAP_U32: RK_BC_UN((CT)(uint32_t)x);
+                        case RK_BC_WRAP_I8: RK_BC_UN((CT)(int8_t)x);
+                        case RK_BC_WRAP_U8: RK_BC_UN((CT)(uint8_t)x);
+                        case RK_BC_WRAP_I16: RK_BC_UN((CT)(int16_t)x);
+                        case RK_BC_WRAP_U16: RK_BC_UN((CT)(uint16_t)x);
                         default: break;
                     }
                 }

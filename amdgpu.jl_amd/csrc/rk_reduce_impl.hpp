@@ -590,23 +590,37 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
 #pragma unroll
     for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = acc[j];
     __syncthreads();
+    // thread t folds columns t, t + 256, ... of the strip: a strip has 64 * VEC columns -- 256 for 4-byte elements, one
+    // a thread; 512 or 1024 for 2- and 1-byte elements
     const int t = threadIdx.x;
-    const int64_t col = (int64_t)strip * COLS + t;
-    Acc r = Op::template identity<Acc>();
-    if (t < COLS) {
-        r = lds[0][t];
+    constexpr int CPT = (COLS + 255) / 256;              // columns per thread
+    Acc r[CPT];
 #pragma unroll
-        for (int w = 1; w < NW; ++w) r = op(r, lds[w][t]);
+    for (int c = 0; c < CPT; ++c) {
+        const int tc = t + c * 256;
+        r[c] = Op::template identity<Acc>();
+        if (tc < COLS) {
+            r[c] = lds[0][tc];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) r[c] = op(r[c], lds[w][tc]);
+        }
     }
     if (msplits == 1) {
-        if (t < COLS && col < g.inner) sink(col + o * g.inner, r);
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int tc = t + c * 256;
+            const int64_t col = (int64_t)strip * COLS + tc;
+            if (tc < COLS && col < g.inner) sink(col + o * g.inner, r[c]);
+        }
         return;
     }
     // partials[(o * strips + strip) * msplits + ms][COLS]
-    if (t < COLS) {
-        store_agent(&partials[(tile * msplits + ms) * COLS + t], r);
-        publish_barrier();
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+        const int tc = t + c * 256;
+        if (tc < COLS) store_agent(&partials[(tile * msplits + ms) * COLS + tc], r[c]);
     }
+    publish_barrier();
     __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
     if (t == 0) {
         const uint32_t old = __hip_atomic_fetch_add(&tickets[tile * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -624,16 +638,18 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
 #pragma unroll
         for (int j = 0; j < VEC; ++j) f[j] = Op::template identity<Acc>();
         int i = wave;
-        for (; i + 3 * NW < msplits; i += 4 * NW) {
-            Acc v[4][VEC];
+        if constexpr (VEC <= 4) {
+            for (; i + 3 * NW < msplits; i += 4 * NW) {
+                Acc v[4][VEC];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < 4; ++u)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) v[u][j] = prow[(int64_t)(i + u * NW) * COLS + j];
+                    for (int j = 0; j < VEC; ++j) v[u][j] = prow[(int64_t)(i + u * NW) * COLS + j];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < 4; ++u)
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) f[j] = op(f[j], v[u][j]);
+                    for (int j = 0; j < VEC; ++j) f[j] = op(f[j], v[u][j]);
+            }
         }
         for (; i < msplits; i += NW)
 #pragma unroll
@@ -643,11 +659,16 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = f[j];
         __syncthreads();
     }
-    if (t < COLS && col < g.inner) {
-        Acc f = lds[0][t];
 #pragma unroll
-        for (int w = 1; w < NW; ++w) f = op(f, lds[w][t]);
-        sink(col + o * g.inner, f);
+    for (int c = 0; c < CPT; ++c) {
+        const int tc = t + c * 256;
+        const int64_t col = (int64_t)strip * COLS + tc;
+        if (tc < COLS && col < g.inner) {
+            Acc f = lds[0][tc];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) f = op(f, lds[w][tc]);
+            sink(col + o * g.inner, f);
+        }
     }
     if (t == 0) tickets[tile * TICKET_STRIDE] = 0;
 }
@@ -1092,6 +1113,15 @@ int32_t mapreduce_u64(const MapreduceArgs&);
 int32_t findminmax_u32(const FindArgs&);
 int32_t findminmax_u64(const FindArgs&);
 int32_t findminmax_u8(const FindArgs&);
+int32_t mapreduce_i8_i64(const MapreduceArgs&);
+int32_t mapreduce_i8(const MapreduceArgs&);
+int32_t findminmax_i8(const FindArgs&);
+int32_t mapreduce_i16_i64(const MapreduceArgs&);
+int32_t mapreduce_i16(const MapreduceArgs&);
+int32_t findminmax_i16(const FindArgs&);
+int32_t mapreduce_u16_u64(const MapreduceArgs&);
+int32_t mapreduce_u16(const MapreduceArgs&);
+int32_t findminmax_u16(const FindArgs&);
 int32_t findminmax_f32(const FindArgs&);
 int32_t findminmax_f64(const FindArgs&);
 int32_t findminmax_i32(const FindArgs&);

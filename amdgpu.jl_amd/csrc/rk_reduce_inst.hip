@@ -41,7 +41,20 @@ int32_t findminmax_u64(const FindArgs& a) { return findminmax_typed<uint64_t>(a)
 // Float16 arrays: f in Float16 (abs2 rounds like Julia's), accumulation in Float32, one rounding at the end
 int32_t mapreduce_f16(const MapreduceArgs& a) { return mapreduce_typed<half_t, float, half_t>(a); }
 int32_t findminmax_f16(const FindArgs& a) { return findminmax_typed<half_t>(a); }
+#elif RK_INST == 10
+// narrow integers: sums and products in the 64-bit type Base.add_sum / mul_prod widen them to, max / min in their own
+int32_t mapreduce_i8_i64(const MapreduceArgs& a) { return mapreduce_typed<int8_t, int64_t>(a); }
+int32_t mapreduce_i8(const MapreduceArgs& a) { return mapreduce_typed<int8_t, int8_t>(a); }
+int32_t findminmax_i8(const FindArgs& a) { return findminmax_typed<int8_t>(a); }
+#elif RK_INST == 11
+int32_t mapreduce_i16_i64(const MapreduceArgs& a) { return mapreduce_typed<int16_t, int64_t>(a); }
+int32_t mapreduce_i16(const MapreduceArgs& a) { return mapreduce_typed<int16_t, int16_t>(a); }
+int32_t findminmax_i16(const FindArgs& a) { return findminmax_typed<int16_t>(a); }
+#elif RK_INST == 12
+int32_t mapreduce_u16_u64(const MapreduceArgs& a) { return mapreduce_typed<uint16_t, uint64_t>(a); }
+int32_t mapreduce_u16(const MapreduceArgs& a) { return mapreduce_typed<uint16_t, uint16_t>(a); }
+int32_t findminmax_u16(const FindArgs& a) { return findminmax_typed<uint16_t>(a); }
 #else
-#error "RK_INST must be 0..9"
+#error "RK_INST must be 0..12"
 #endif
 }  // namespace rk

@@ -53,6 +53,8 @@ rk_dtype(::Type{Float32}) = Cint(0); rk_dtype(::Type{Float64}) = Cint(1)
 rk_dtype(::Type{Int32}) = Cint(2);   rk_dtype(::Type{Int64}) = Cint(3)
 rk_dtype(::Type{Bool}) = Cint(4);    rk_dtype(::Type{UInt8}) = Cint(4)
 rk_dtype(::Type{UInt32}) = Cint(5);  rk_dtype(::Type{UInt64}) = Cint(6)
+rk_dtype(::Type{Float16}) = Cint(7); rk_dtype(::Type{Int16}) = Cint(8)
+rk_dtype(::Type{Int8}) = Cint(9);    rk_dtype(::Type{UInt16}) = Cint(10)
 rk_dtype(::Type) = nothing
 rk_map(::typeof(identity)) = Cint(0); rk_map(::typeof(abs2)) = Cint(1); rk_map(::typeof(abs)) = Cint(2)
 rk_map(_) = nothing
@@ -261,7 +263,7 @@ function native_findminmax(wantmax::Bool, A::ROCArray{T,N}, dims) where {T,N}
 end
 function enable_findminmax!()
     for (fn, wantmax) in ((:findmax, true), (:findmin, false))
-        @eval function Base.$fn(A::ROCArray{T,N}; dims=:) where {T<:Union{Float32,Float64,Int32,Int64},N}
+        @eval function Base.$fn(A::ROCArray{T,N}; dims=:) where {T<:Union{Float16,Float32,Float64,Int8,Int16,Int32,Int64,UInt16,UInt32,UInt64},N}
             isempty(A) && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)       # the stock method's error
             res = native_findminmax($wantmax, A, dims)
             res === nothing && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
@@ -412,10 +414,10 @@ function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadc
     if !(CT <: Union{Float32,Float64})
         # integer programs of + - * max min muladd - abs abs2 compute in Int64 (the store keeps the low bits);
         # with `/` or a math function Julia's result is a Float64 and so is the compute type
-        CT = all(t -> t < RK_MAX_OPERANDS || t in INT_SAFE, toks) && CT <: Union{Bool,Int32,Int64,UInt8,UInt32} ? Int64 : Float64
+        CT = all(t -> t < RK_MAX_OPERANDS || t in INT_SAFE, toks) && CT <: Union{Bool,Int8,Int16,Int32,Int64,UInt8,UInt16,UInt32} ? Int64 : Float64
         if CT === Int64 && any(t -> t in ORDER_SENSITIVE, toks) &&
-           any(o -> (o isa AbstractArray ? eltype(o) : typeof(o)) <: Union{Int32,UInt32}, ops) && count(t -> t >= RK_MAX_OPERANDS, toks) > 1
-            throw(Unsupported())                 # would need RK_BC_WRAP_I32 after the 32-bit intermediates
+           any(o -> (o isa AbstractArray ? eltype(o) : typeof(o)) <: Union{Int8,Int16,Int32,UInt8,UInt16,UInt32}, ops) && count(t -> t >= RK_MAX_OPERANDS, toks) > 1
+            throw(Unsupported())                 # would need RK_BC_WRAP_* after the narrow intermediates
         end
     end
     zeros8 = ntuple(_ -> Int64(0), 8)
@@ -556,7 +558,6 @@ function enable_permutedims!()
 end
 
 # ---- sort! / sortperm! (src/kernels/sorting.jl:1-3): default order and rev natively, closures stay with AK -------------
-rk_dtype(::Type{Float16}) = Cint(7); rk_dtype(::Type{Int16}) = Cint(8)
 const SORTABLE = Union{Float16,Float32,Float64,Int16,Int32,Int64}
 
 function enable_sort!()

@@ -70,8 +70,13 @@ typedef enum {
     RK_U64 = 6,  /* UInt64  */
     RK_F16 = 7,  /* Float16: rk_mapreduce (accumulating in Float32), rk_findminmax, rk_broadcast operands and
                   * destinations, rk_sort / rk_sortperm; not rk_accumulate (RK_ERR_UNSUPPORTED) */
-    RK_I16 = 8   /* Int16: rk_sort / rk_sortperm only.  rk_reverse and rk_permutedims take an element SIZE, not
-                  * a dtype, and so move any 2-byte element */
+    RK_I16 = 8,  /* Int16 */
+    RK_I8  = 9,  /* Int8  */
+    RK_U16 = 10  /* UInt16.  The three narrow integers: rk_mapreduce (sum / prod into Int64 or UInt64 as Base.add_sum
+                  * widens them, max / min in their own type), rk_findminmax, rk_broadcast operands and destinations
+                  * (integer programs compute in Int64 and store the low bits); Int16 also rk_sort / rk_sortperm.  Not
+                  * rk_accumulate, not rk_mapreduce_program (RK_ERR_UNSUPPORTED).  rk_reverse and rk_permutedims take an
+                  * element SIZE, not a dtype, and so move any 1- or 2-byte element */
 } rk_dtype;
 
 /* f of mapreduce(f, op, A) */
@@ -270,9 +275,10 @@ typedef enum {
     RK_BC_WRAP_I32,            /* integer programs: sign-extend the low 32 bits, i.e. the Int32 value Julia
                                 * holds at this point (needed before order-sensitive tokens only)      */
     RK_BC_WRAP_U32,            /* the same, zero-extending (UInt32)                                    */
-    RK_BC_ROUND_F16            /* Float32 programs over Float16 arrays: round to Float16 and back, after every
+    RK_BC_ROUND_F16,           /* Float32 programs over Float16 arrays: round to Float16 and back, after every
                                 * operation whose Julia result is a Float16 (Julia computes Float16 arithmetic in
                                 * Float32 and rounds each result)                                       */
+    RK_BC_WRAP_I8, RK_BC_WRAP_U8, RK_BC_WRAP_I16, RK_BC_WRAP_U16     /* as WRAP_I32 / WRAP_U32, for the narrow integers */
 } rk_bc_token;
 
 typedef struct {

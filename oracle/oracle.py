@@ -175,7 +175,12 @@ def mapreduce(f: str, op: str, A: np.ndarray, dims=None, init=None) -> np.ndarra
     A = np.asarray(A)
     axes = _normalize_dims(dims, A.ndim)
     out_dt = reduce_eltype(op, A.dtype)
-    a = _apply_map(f, _wide(A, out_dt))
+    if A.dtype.kind in "iu":
+        # f runs on the element, in the element type: abs2(x::Int16) is an Int16 and wraps; add_sum widens afterwards
+        with np.errstate(over="ignore"):
+            a = _wide(_apply_map(f, A).astype(A.dtype), out_dt)
+    else:
+        a = _apply_map(f, _wide(A, out_dt))
     base = {"add_sum": "add", "mul_prod": "mul"}.get(op, op)
     with np.errstate(over="ignore"):
         if base == "add":

@@ -179,6 +179,48 @@ def test_integer_programs_are_exact_and_wrap(rk):
     assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(big)))), big)
 
 
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.uint16, np.uint8])
+def test_narrow_integer_arrays(rk, dtype):
+    """Int8 / Int16 / UInt16 (and UInt8) operands and destinations: integer programs compute in Int64, the store keeps
+    the low bits (Julia's wrap-around), and a narrow intermediate is wrapped before an order-sensitive operation."""
+    rng = np.random.default_rng(60)
+    L = rk.lazy
+    info = np.iinfo(dtype)
+    for shape in ((1000,), (300, 70), (257, 3, 5), (4096, 64)):
+        a = rng.integers(info.min, info.max + 1, shape).astype(dtype)
+        b = rng.integers(info.min, info.max + 1, shape).astype(dtype)
+        da, db = rk.ROCArray(a), rk.ROCArray(b)
+        with np.errstate(over="ignore"):
+            got = rk.materialize(L(da) + L(db))
+            assert got.dtype == dtype and np.array_equal(rk.Array(got), (a + b).astype(dtype))
+            got = rk.materialize(L(da) * L(db) - L(da))
+            assert got.dtype == dtype and np.array_equal(rk.Array(got), (a * b - a).astype(dtype))
+            got = rk.materialize(rk.broadcast.max_(L(da), L(db)))
+            assert got.dtype == dtype and np.array_equal(rk.Array(got), np.maximum(a, b))
+            # the sum wraps in the narrow type before the comparison / max sees it
+            got = rk.materialize(rk.broadcast.max_(L(da) + L(db), L(da)))
+            assert got.dtype == dtype and np.array_equal(rk.Array(got), np.maximum((a + b).astype(dtype), a))
+            got = rk.materialize((L(da) + L(db)) > L(da))
+            assert got.dtype == np.bool_ and np.array_equal(rk.Array(got), (a + b).astype(dtype) > a)
+        # mixed with a wider type: promotes; into a Float32 destination: converts
+        w = rng.integers(-1000, 1000, shape).astype(np.int32)
+        got = rk.materialize(L(da) + L(rk.ROCArray(w)))
+        with np.errstate(over="ignore"):
+            assert got.dtype == np.promote_types(dtype, np.int32) and np.array_equal(rk.Array(got), (a.astype(got.dtype) + w.astype(got.dtype)))
+        f32 = rk.ROCArray(dims=shape, dtype=np.float32)
+        rk.materialize_(f32, L(da) * 2)
+        assert np.array_equal(rk.Array(f32), (a.astype(np.int64) * 2).astype(np.float32))      # Int8 * Int is an Int
+        # a narrow destination of a wider program keeps the low bits
+        dn = rk.ROCArray(dims=shape, dtype=dtype)
+        rk.materialize_(dn, L(rk.ROCArray(w)) * 3)
+        assert np.array_equal(rk.Array(dn), (w.astype(np.int64) * 3).astype(dtype))
+    # a row vector against a matrix
+    m = rng.integers(info.min, info.max + 1, (130, 50)).astype(dtype)
+    r = rng.integers(info.min, info.max + 1, (1, 50)).astype(dtype)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(rk.Array(rk.materialize(L(rk.ROCArray(m)) - L(rk.ROCArray(r)))), (m - r).astype(dtype))
+
+
 def test_three_operand_trees_all_operator_pairs(rk):
     """(u op1 v) op2 w and u op1 (v op2 w) run on a fused evaluator: every operator pair, both shapes, repeated and
     scalar and extruded operands; Float32 results equal NumPy's un-fused Float32 arithmetic bit for bit."""

@@ -86,6 +86,20 @@ def test_mapreduce_full_is_scalar_and_init_folds():
     assert orc.mapreduce("identity", "max", A, dims=1, init=100).tolist() == [[100.0] * 4]
 
 
+def test_map_runs_in_the_element_type():
+    """mapreduce(abs2, add_sum, x): abs2(x::Int16) is an Int16 and wraps, the widening happens in add_sum.  Worked by
+    hand: abs2(Int16(300)) = 90000 - 65536 = 24464, abs2(Int16(-200)) = 40000 - 65536 = -25536, sum -1072 (Julia:
+    sum(abs2, Int16[300, -200]) == -1072); abs(typemin(Int8)) == typemin(Int8); UInt16: 300^2 mod 2^16 = 24464."""
+    r = orc.mapreduce("abs2", "add_sum", np.array([300, -200], dtype=np.int16))
+    assert r.dtype == np.int64 and int(r) == -1072
+    r = orc.mapreduce("abs", "max", np.array([-128, 5], dtype=np.int8))
+    assert r.dtype == np.int8 and int(r) == 5                       # abs(-128) stays -128
+    r = orc.mapreduce("abs2", "add_sum", np.array([300, 2], dtype=np.uint16))
+    assert r.dtype == np.uint64 and int(r) == 24464 + 4
+    r = orc.mapreduce("abs2", "add_sum", np.array([100000, 3], dtype=np.int32))
+    assert r.dtype == np.int64 and int(r) == (100000 * 100000 - 2 * 2**32) + 9      # 10^10 wraps to 1410065408
+
+
 def test_max_min_base_rules():
     assert np.isnan(orc.maximum(np.array([1.0, np.nan, 3.0])))               # NaN propagates (Base.max)
     assert np.isnan(orc.minimum(np.array([1.0, np.nan, 3.0])))

@@ -75,6 +75,43 @@ def test_random_reductions(rk, orc):
             assert np.array_equal(got, want.astype(got.dtype))
 
 
+NARROW = [np.int8, np.int16, np.uint16]
+
+
+def test_random_narrow_integers(rk, orc):
+    """Int8 / Int16 / UInt16: sums and products in the 64-bit type Base.add_sum / mul_prod widen them to, + / max / min
+    in their own type (wrapping), findmax / findmin, all bit-exact."""
+    rng = np.random.default_rng(1011 + SEED)
+    for case in range(240):
+        shape = _shape(rng)
+        dtype = NARROW[int(rng.integers(len(NARROW)))]
+        dims = _dims(rng, len(shape))
+        op = ["add_sum", "add", "max", "min", "mul_prod"][int(rng.integers(5))]
+        f = ["identity", "abs2", "abs"][int(rng.integers(3))]
+        _say("narrow reduce", case, shape, np.dtype(dtype).name, dims, f, op)
+        info = np.iinfo(dtype)
+        if op == "mul_prod":
+            x = rng.integers(max(info.min, -2), 3, shape).astype(dtype)
+        else:
+            x = rng.integers(info.min, info.max + 1, shape).astype(dtype)
+        got = rk.mapreduce(f, op, rk.ROCArray(x), dims=dims)
+        want = orc.mapreduce(f, op, x, dims=dims)
+        got = np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape)
+        assert got.dtype == orc.reduce_eltype(op, dtype)
+        assert np.array_equal(got, want.astype(got.dtype))
+        if case % 3 == 0:
+            y = rng.integers(max(info.min, -3), 4, shape).astype(dtype)          # few distinct values: the first-index rule decides
+            dy = rk.ROCArray(y)
+            for gpu, cpu in ((rk.findmax, orc.findmax), (rk.findmin, orc.findmin)):
+                gv, gi = gpu(dy, dims=dims)
+                ov, oi = cpu(y, dims=dims)
+                if dims is None:
+                    assert gv == ov and gi == oi
+                else:
+                    assert rk.Array(gv).dtype == y.dtype and np.array_equal(rk.Array(gv), ov)
+                    assert np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
+
+
 def test_random_findminmax(rk, orc):
     rng = np.random.default_rng(1002 + SEED)
     for case in range(150):

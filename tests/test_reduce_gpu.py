@@ -459,3 +459,32 @@ def test_findmax_findmin_return_the_nan_itself(rk, dtype, utype):
                 has_nan = np.isnan(h).any(axis=ax)
                 first_nan = np.argmax(np.isnan(h), axis=ax)
                 assert np.array_equal(gi[:, ax][has_nan.reshape(-1)], first_nan.reshape(-1)[has_nan.reshape(-1)])
+
+
+@pytest.mark.parametrize("dtype", [np.bool_, np.uint8, np.float16, np.int8, np.int16, np.uint16])
+@pytest.mark.parametrize("shape", [(1024, 40), (2048, 300), (512, 7, 3), (4096, 129)])
+def test_narrow_elements_along_rows(rk, orc, dtype, shape):
+    """sum / maximum over dims=2 of 1- and 2-byte elements with long contiguous rows: a strip of the strided kernel is
+    64 sixteen-byte vectors = 512 or 1024 columns wide, more than a workgroup has threads (an earlier version folded
+    and stored only the first 256 columns of every strip)."""
+    rng = np.random.default_rng(77)
+    if np.dtype(dtype) == np.bool_:
+        x = rng.random(shape) < 0.3
+    elif np.dtype(dtype).kind == "f":
+        x = rng.standard_normal(shape).astype(dtype)
+    else:
+        info = np.iinfo(dtype)
+        x = rng.integers(info.min, info.max + 1, shape).astype(dtype)
+    dx = rk.ROCArray(x)
+    for op in (("add_sum",) if np.dtype(dtype) == np.bool_ else ("add_sum", "max")):      # count(A; dims=2) for Bool
+        got = rk.Array(rk.mapreduce("identity", op, dx, dims=2))
+        want = orc.mapreduce("identity", op, x, dims=2)
+        assert got.dtype == orc.reduce_eltype(op, x.dtype) and got.shape == want.shape
+        if got.dtype.kind == "f":
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=2e-3, atol=2e-3)
+        else:
+            assert np.array_equal(got, want.astype(got.dtype))
+    if np.dtype(dtype) != np.bool_:
+        gv, gi = rk.findmax(dx, dims=2)
+        ov, oi = orc.findmax(x, dims=2)
+        assert np.array_equal(rk.Array(gv), ov) and np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
