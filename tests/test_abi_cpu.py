@@ -70,7 +70,8 @@ def test_mapreduce_argument_validation(L):
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 9, sh, 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT     # ndim > 8
     assert f(0, 0, L.RK_F32, L.RK_F32, one, 1, L.shape_array((-1,)), 1, one, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert f(0, 0, L.RK_F32, L.RK_I32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Float32 -> Int32
-    assert f(0, 0, L.RK_I16, L.RK_I16, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Int16 reductions
+    assert f(0, 0, L.RK_I16, L.RK_F32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED           # Int16 -> Float32
+    assert f(0, 0, L.RK_I8, L.RK_I32, one, 1, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED            # Int8 sums widen to Int64 only
     # zero-length input: success without launching (src/kernels/mapreduce.jl:91), even with null pointers
     assert f(0, 0, L.RK_F32, L.RK_F32, None, 1, L.shape_array((0,)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     # a reduction that needs partials but has no workspace
@@ -85,7 +86,7 @@ def test_findminmax_and_accumulate_validation(L):
     g = L.lib.rk_findminmax
     assert g(1, L.RK_F32, None, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert g(1, L.RK_F32, one, 2, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # no output requested
-    assert g(1, L.RK_I16, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    assert g(1, 99, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT                # no such element type
     assert g(1, L.RK_F32, None, 2, L.shape_array((0, 4)), 1, None, None, None, 0, None) == L.RK_SUCCESS
     a = L.lib.rk_accumulate
     assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
@@ -93,6 +94,8 @@ def test_findminmax_and_accumulate_validation(L):
     assert a(5, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert a(2, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 0, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # exclusive max needs init
     assert a(0, L.RK_F32, L.RK_F64, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    for narrow in (L.RK_I8, L.RK_I16, L.RK_U16, L.RK_F16):                                                       # no scans of 1- and 2-byte values
+        assert a(0, narrow, narrow, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
     assert a(0, L.RK_U8, L.RK_I64, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT    # aliasing with different sizes
     assert a(0, L.RK_F32, L.RK_F32, None, None, 1, L.shape_array((0,)), 1, 1, None, None, 0, None) == L.RK_SUCCESS
     # a look-back scan without workspace
