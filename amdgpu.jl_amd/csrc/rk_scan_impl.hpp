@@ -1436,9 +1436,13 @@ inline int32_t launch_scan(const ScanArgs& a) {
     // long lines: single pass with look-back; tile = NW waves x 8 vectors, as large as the line length allows
     constexpr int KT = 8;
     const int64_t line_bytes = s.mid * (int64_t)sizeof(T);
-    // measured (Int32, 2^22 .. 2^27 elements): 16 waves beat 8 and 4 at every size -- fewer, larger tiles mean
-    // fewer look-backs; lines that barely exceed one small tile use 8 or 4
-    int nw = line_bytes > ((int64_t)64 << 10) ? 16 : (line_bytes > ((int64_t)32 << 10) ? 8 : 4);
+    // measured (4-byte elements): on lines of a megabyte and more 16 waves beat 8 and 4 -- fewer, larger tiles mean fewer
+    // look-backs (2^26 elements: 92 against 97 us).  Shorter lines leave the last 128 KiB tile of every line partly
+    // empty, and a half-idle workgroup of 1024 threads holds half a compute unit: 3000 lines of 20000 Float32 139 us
+    // with 16 waves, 85 us with 8; 1300 lines of 50000: 119 against 97; 600 lines of 100000: 88 against 85
+    // -- so 16 waves only where their tiles are at least 90 % full (65536 x 1024 Int32, two full tiles a line: 96 against 101 us)
+    const int64_t tile16 = (int64_t)ScanTile<T, KT>::TILE / 4 * 16, cover16 = (s.mid + tile16 - 1) / tile16 * tile16;
+    int nw = cover16 * 10 <= s.mid * 11 ? 16 : (line_bytes > ((int64_t)32 << 10) ? 8 : 4);
     if (tune_scan_waves() != 0) nw = tune_scan_waves();
     const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
     const int64_t tpl = (s.mid + TILE - 1) / TILE;
