@@ -279,3 +279,49 @@ def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
     np.testing.assert_allclose(rk.Array(rk.cumsum(rk.ROCArray(xf), dims=dims)), orc.cumsum(xf, dims=dims), rtol=RTOL, atol=1e-4)
     b = rng.random(shape) < 0.5
     assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=dims)), orc.cumsum(b, dims=dims))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8, np.int16, np.uint16, np.float16])
+def test_narrow_element_types(rk, orc, dtype):
+    """accumulate / cumsum / cumprod of 1- and 2-byte elements: scanned in the next wider type and stored back (the host
+    mirror's three native kernels).  Integers wrap in their own type, bit-exact; Float16 within a few Float16 roundings
+    of the Float64 scan (AcceleratedKernels rounds after every step, the native path once)."""
+    rng = np.random.default_rng(91)
+    dt = np.dtype(dtype)
+    for shape, dims in (((1000,), 1), ((70_001,), 1), ((300, 70), 1), ((300, 70), 2), ((5, 64, 9), 2), ((200_000,), None)):
+        if dt.kind == "f":
+            x = (rng.random(shape) * 0.01).astype(dt)
+        else:
+            info = np.iinfo(dt)
+            x = rng.integers(info.min, info.max + 1, shape).astype(dt)
+        dx = rk.ROCArray(x)
+        for op in ("add", "max", "min", "mul"):
+            if op == "mul":
+                # Float16: factors 2, 1/2, 2, ... along the scanned dim keep every running product within 1 .. 2
+                x2 = (rng.integers(1, 3, shape).astype(dt) if dt.kind != "f"
+                      else np.where(np.indices(shape)[(dims or 1) - 1] % 2 == 0, 2.0, 0.5).astype(dt))
+                src, dsrc = x2, rk.ROCArray(x2)
+            else:
+                src, dsrc = x, dx
+            got = rk.Array(rk.accumulate(op, dsrc, dims=dims))
+            want = orc.accumulate(op, src, dims=dims)
+            assert got.dtype == dt and got.shape == src.shape
+            if dt.kind == "f":
+                np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=4e-3, atol=1e-4)
+            else:
+                assert np.array_equal(got, want.astype(dt))
+        # exclusive with init, and in place
+        init = dt.type(3)
+        got = rk.Array(rk.accumulate("add", dx, dims=dims, init=init, inclusive=False))
+        want = orc.accumulate("add", x, dims=dims, init=init, inclusive=False)
+        if dt.kind == "f":
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=4e-3, atol=1e-4)
+        else:
+            assert np.array_equal(got, want.astype(dt))
+        dy = rk.ROCArray(x)
+        assert rk.accumulate_("add", dy, dy, dims=dims) is dy
+        want = orc.accumulate("add", x, dims=dims)
+        if dt.kind == "f":
+            np.testing.assert_allclose(rk.Array(dy).astype(np.float64), want.astype(np.float64), rtol=4e-3, atol=1e-4)
+        else:
+            assert np.array_equal(rk.Array(dy), want.astype(dt))
