@@ -17,7 +17,7 @@ import os
 import torch  # noqa: F401  (import order matters)
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "librk.so")
+LIB_PATH = os.environ.get("RK_LIBRARY") or os.path.join(HERE, "librk.so")      # RK_LIBRARY: another build of the same ABI
 
 RK_MAX_DIMS = 8
 RK_MAX_OPERANDS = 8
