@@ -336,7 +336,7 @@ template <typename In, typename Acc, typename Xf> struct ShortLinesTile {
     static constexpr int BYTES = 16384;
     static constexpr int ELEMS = BYTES / (MAPPED_IN_LDS ? sizeof(Acc) : sizeof(In));
 };
-constexpr int SHORT_LINES_MAX = 256;          // contiguous lines beyond this do as well with a wave each
+constexpr int SHORT_LINES_MAX = 512;          // contiguous lines beyond this do as well with a wave each (300 elements: 59 us with a wave a line)
 
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR>
 __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __restrict__ A, int inner, int m, int64_t nslabs, int slabs_per_block,

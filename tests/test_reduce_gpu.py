@@ -488,3 +488,23 @@ def test_narrow_elements_along_rows(rk, orc, dtype, shape):
         gv, gi = rk.findmax(dx, dims=2)
         ov, oi = orc.findmax(x, dims=2)
         assert np.array_equal(rk.Array(gv), ov) and np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
+
+
+@pytest.mark.parametrize("m", [257, 300, 400, 511, 512])
+def test_lines_of_a_few_hundred_elements(rk, orc, m):
+    """dims=1 with lines of 257 .. 512 elements: whole lines through LDS, 16 lanes a line (a wave a line idles most of
+    its second round: 300 elements 59 us -> 47 us for 2^26 bytes)."""
+    rng = np.random.default_rng(m)
+    for dtype in (np.float32, np.int32, np.float64):
+        x = (rng.standard_normal((m, 3001)) * 100).astype(dtype)
+        dx = rk.ROCArray(x)
+        got = rk.Array(rk.mapreduce("identity", "add_sum", dx, dims=1))
+        want = orc.mapreduce("identity", "add_sum", x, dims=1)
+        if np.dtype(dtype).kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-3 if dtype == np.float32 else 1e-9)
+        else:
+            assert np.array_equal(got, want)
+        assert np.array_equal(rk.Array(rk.mapreduce("abs", "max", dx, dims=1)), orc.mapreduce("abs", "max", x, dims=1).astype(dtype))
+        gv, gi = rk.findmax(dx, dims=1)
+        ov, oi = orc.findmax(x, dims=1)
+        assert np.array_equal(rk.Array(gv), ov) and np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
