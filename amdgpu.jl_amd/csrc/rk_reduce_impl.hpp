@@ -1010,6 +1010,43 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
             }
         }
     }
+    // A long reduced dim behind a short contiguous one (sum(A; dims=2) of a 64 x 1_000_000 array): lanes along `inner` fill
+    // a quarter of the strided kernel's 256-column strip (2.8 TB/s), and the narrow kernel moves 4 bytes a lane (32 x N:
+    // 3.8 TB/s).  With one or two strips in all (256 x 250_000), the last workgroup of a strip folds hundreds of rows of
+    // partials alone.  f consecutive rows are one row of f * inner elements -- the same memory -- so the array is
+    // reduced as (f * inner) x (mid / f), with full strips and at least 16 of them where a factor allows, into a
+    // temporary, whose f groups of `inner` columns a second, tiny reduction folds.
+    if (s.single_run && s.inner > 1 && s.mid >= 4096 && is_aligned(a.A, 16)) {
+        constexpr int64_t VEC = 16 / (int64_t)sizeof(In), COLS = WAVE * VEC;
+        constexpr int64_t WANT_TILES = 16;
+        const int64_t cols0 = s.inner % VEC == 0 ? COLS : WAVE;
+        const int64_t strips0 = (s.inner + cols0 - 1) / cols0;
+        const bool poor = s.inner < WAVE || s.inner * 10 < strips0 * cols0 * 7 || (cols0 == WAVE && s.inner < 4 * COLS) ||
+                          strips0 * s.outer < 4;
+        Workspace w{};
+        if (poor && carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
+            int64_t pick = 0;
+            for (int64_t f = 2; f <= 256 && f * 256 <= s.mid; ++f) {
+                const int64_t wide = s.inner * f, strips = (wide + COLS - 1) / COLS;
+                if (s.mid % f != 0 || wide % VEC != 0 || wide * 10 < strips * COLS * 9) continue;
+                if ((size_t)(wide * s.outer) * sizeof(Acc) + 256 > a.partials_cap / 4) break;
+                pick = f;
+                if (strips * s.outer >= WANT_TILES) break;
+            }
+            if (pick > 0) {
+                const int64_t f = pick, wide = s.inner * f;
+                const size_t temp_bytes = ((size_t)(wide * s.outer) * sizeof(Acc) + 255) & ~(size_t)255;
+                Acc* temp = (Acc*)((char*)w.partials + a.partials_cap - temp_bytes);
+                const size_t cap = a.partials_cap - temp_bytes;
+                const int64_t shape1[3] = {wide, s.mid / f, s.outer}, shape2[3] = {s.inner, f, s.outer};
+                ReduceSink<Acc, Op> to_temp{temp, Op::template identity<Acc>(), 0};
+                const int32_t st = launch_reduce<In, Acc>((const In*)a.A, 3, shape1, 2u, xf, Op(), to_temp, a.ws, a.ws_bytes, a.stream, cap);
+                if (st != RK_SUCCESS) return st;
+                return launch_reduce<Acc, Acc>((const Acc*)temp, 3, shape2, 2u, MapXform<Acc, Acc, MapIdentity>(), Op(), sink,
+                                               a.ws, a.ws_bytes, a.stream, cap);
+            }
+        }
+    }
     return launch_reduce<In, Acc>((const In*)a.A, a.ndim, a.shape, a.mask, xf, Op(), sink, a.ws, a.ws_bytes, a.stream, a.partials_cap);
 }
 
