@@ -44,11 +44,14 @@ __device__ __forceinline__ void emit_index(int64_t* __restrict__ ys, int64_t pos
 // scanned positions; the wave then reads the strip back in order and writes indices with coalesced stores (a
 // lane writing its own run directly makes every store instruction touch 64 different lines: 4x slower at high
 // density).  Only bit 0 of a byte is looked at (Julia's Bool).
-template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K>
+// ORDERED: one workgroup per tile, tile = blockIdx.x, the look-back and the end of the call as in scan_ordered_kernel
+// (no tile counter, only the first tile of a group of 64 reads group descriptors, each on a line of its own).
+template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K, bool ORDERED>
 __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uint8_t* __restrict__ bools, int64_t n, int64_t* __restrict__ ys,
                                                                        int64_t* __restrict__ count_out, SelShape shp, int aligned,
-                                                                       unsigned long long* counter, uint64_t* desc, int64_t ntiles,
-                                                                       int64_t ngroups, int64_t desc_capacity, WaitCtl wc) {
+                                                                       unsigned long long* counter, uint32_t* tickets, int ticket_group,
+                                                                       uint64_t* desc, int64_t ntiles, int64_t ngroups, int64_t desc_capacity,
+                                                                       WaitCtl wc) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int SEL_TILE = SEL_NW * SEL_CHUNK * SEL_K;
     __shared__ uint16_t lds_strip[SEL_NW][SEL_CHUNK];
@@ -57,12 +60,17 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
     __shared__ unsigned long long lds_id;
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     uint64_t* tile_desc = desc;                                          // [2 words][ntiles]
-    uint64_t* group_desc = desc + (int64_t)Words<int64_t>::N * ntiles;   // [2 words][ngroups]
+    uint64_t* group_desc = desc + (int64_t)Words<int64_t>::N * ntiles;   // [2 words][ngroups]; ORDERED: a line per group
     const OpAdd op;
 
-    if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    unsigned long long cur = lds_id;
+    unsigned long long cur;
+    if constexpr (ORDERED) {
+        cur = (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & ~0xffffffffull) | (unsigned long long)blockIdx.x;
+    } else {
+        if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        cur = lds_id;
+    }
     while ((int64_t)(cur & 0xffffffffull) < ntiles) {
         const int64_t tile = (int64_t)(cur & 0xffffffffull);
         const uint32_t epoch = (uint32_t)(cur >> 32);
@@ -97,16 +105,27 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
                 }
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                // bit 0 of the four bytes of a word -> bits 24..27 (the partial products land on distinct bits)
-                x[k] &= 0x01010101u;
-                const uint32_t hits = ((x[k][0] * 0x01020408u) >> 24) | ((x[k][1] * 0x01020408u) >> 20 & 0xf0u) |
-                                      ((x[k][2] * 0x01020408u) >> 16 & 0xf00u) | ((x[k][3] * 0x01020408u) >> 12 & 0xf000u);
-                const int32_t c = __popc(hits);
+            for (int k = 0; k < 4; k += 2) {
+                // bit 0 of the 16 bytes -> a 16-bit mask in memory order: a dot product of the four bytes of a word with
+                // (1, 2, 4, 8) or (16, 32, 64, 128) gathers four of them (a 32-bit multiply does too, at a quarter of
+                // the rate).  The counts of two loads share one scan across the wave (a chunk holds at most 1024 hits).
+                uint32_t hits[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const u32x4 b = x[k + h] & 0x01010101u;
+                    const uint32_t lo = __builtin_amdgcn_udot4(b[1], 0x80402010u, __builtin_amdgcn_udot4(b[0], 0x08040201u, 0u, false), false);
+                    const uint32_t hi = __builtin_amdgcn_udot4(b[3], 0x80402010u, __builtin_amdgcn_udot4(b[2], 0x08040201u, 0u, false), false);
+                    hits[h] = lo | (hi << 8);
+                }
+                const int32_t c = (int32_t)(__popc(hits[0]) | ((uint32_t)__popc(hits[1]) << 16));
                 const int32_t inc = wave_scan_inclusive(c, op, 0);
-                pk[k0 + k] = ((uint32_t)(inc - c) << 16) | hits;
-                ktot[k0 + k] = read_lane(inc, WAVE - 1);
-                carry += ktot[k0 + k];
+                const uint32_t exc = (uint32_t)(inc - c);
+                pk[k0 + k] = (exc << 16) | hits[0];
+                pk[k0 + k + 1] = (exc & 0xffff0000u) | hits[1];
+                const uint32_t tot = (uint32_t)read_lane(inc, WAVE - 1);
+                ktot[k0 + k] = (int32_t)(tot & 0xffffu);
+                ktot[k0 + k + 1] = (int32_t)(tot >> 16);
+                carry += ktot[k0 + k] + ktot[k0 + k + 1];
             }
         }
         if (lane == 0) lds_wave[wave] = carry;
@@ -121,9 +140,14 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
         if (wave == 0) {
             int64_t tile_prefix = 0;
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, (int64_t)tile_count, (epoch << 2) | DESC_A);
-            if (tile > 0)
-                tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
-                                             (int64_t)0, op, (int64_t)0, wc);
+            if (tile > 0) {
+                if constexpr (ORDERED)
+                    tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
+                                                       (int64_t)0, op, (int64_t)0, wc);
+                else
+                    tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
+                                                 (int64_t)0, op, (int64_t)0, wc);
+            }
             if (lane == 0) {
                 lds_prefix = tile_prefix;
                 if (tile == ntiles - 1 && count_out != nullptr) *count_out = tile_prefix + tile_count;
@@ -131,33 +155,50 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
         }
         __syncthreads();
         int64_t base = lds_prefix + wave_prefix;
+        // The hits of consecutive chunks share the strip while they fit (SEL_CHUNK entries; an entry is an offset from
+        // the first chunk of the batch, < 16 * 1024): a sparse mask leaves in one round per wave instead of one per
+        // chunk, each of which costs two LDS round trips.  fill, kbase: wave-uniform.
         uint16_t* strip = lds_strip[wave];
-#pragma unroll
-        for (int k = 0; k < SEL_K; ++k) {
-            if (ktot[k] == 0) continue;                                   // wave-uniform
-            int32_t p = (int32_t)(pk[k] >> 16);
-            for (uint32_t m = pk[k] & 0xffffu; m != 0u; m &= m - 1u) strip[p++] = (uint16_t)(lane * 16 + __ffs(m) - 1);
+        int32_t fill = 0, kbase = 0;
+        auto flush = [&]() {
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const int64_t i0 = e0 + wave * (SEL_CHUNK * SEL_K) + k * SEL_CHUNK;
-            for (int i = lane; i < ktot[k]; i += WAVE) emit_index<LINEAR, SMALL>(ys, base + i, i0 + strip[i], shp);
+            const int64_t i0 = e0 + wave * (SEL_CHUNK * SEL_K) + kbase * SEL_CHUNK;
+            for (int i = lane; i < fill; i += WAVE) emit_index<LINEAR, SMALL>(ys, base + i, i0 + strip[i], shp);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();                              // the strip is reused by the next chunk
-            base += ktot[k];
+            __builtin_amdgcn_wave_barrier();                              // the strip is reused by the next batch
+            base += fill;
+            fill = 0;
+        };
+#pragma unroll
+        for (int k = 0; k < SEL_K; ++k) {
+            if (ktot[k] == 0) continue;                                   // wave-uniform
+            if (fill + ktot[k] > SEL_CHUNK) flush();
+            if (fill == 0) kbase = k;
+            int32_t p = fill + (int32_t)(pk[k] >> 16);
+            const uint32_t rel = (uint32_t)((k - kbase) * SEL_CHUNK + lane * 16 - 1);
+            for (uint32_t m = pk[k] & 0xffffu; m != 0u; m &= m - 1u) strip[p++] = (uint16_t)(rel + __ffs(m));
+            fill += ktot[k];
         }
+        if (fill > 0) flush();
+        if constexpr (ORDERED) break;
         if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         cur = lds_id;
     }
-    chain_finish(cur, ntiles, (int64_t)Words<int64_t>::N * (ntiles + ngroups), counter, desc, desc_capacity);
+    if constexpr (ORDERED)
+        ordered_finish((uint32_t)(cur >> 32), (int64_t)Words<int64_t>::N * ntiles + ngroups * GROUP_DESC_STRIDE, counter, tickets, ticket_group,
+                       desc, desc_capacity);
+    else
+        chain_finish(cur, ntiles, (int64_t)Words<int64_t>::N * (ntiles + ngroups), counter, desc, desc_capacity);
 }
 
 __global__ void store_count_kernel(int64_t* p, int64_t v) { *p = v; }
 
 // 16-byte loads per lane and tile (RK_SELECT_LOADS: 4, 8 or 16).  Measured on MI355X, 2^28 Bools, 1 % / 25 % / 100 %
-// set: 4 loads 96 / 179 / 417 us, 8 loads 76 / 161 / 465 us, 16 loads 72 / 167 / 466 us: tile acquisitions are
-// serialised device-wide (one atomic each), so larger tiles win until the output dominates.
+// set, 8 waves in launch order: 4 loads 112 / 188 / 425 us, 8 loads 78 / 167 / 462 us, 16 loads 63 / 159 / 473 us: every
+// tile costs about 10 ns whatever feeds it, so larger tiles win until the output dominates.
 int tune_select_loads() {
     static const int v = [] { const char* s = std::getenv("RK_SELECT_LOADS"); const int x = s ? std::atoi(s) : 0; return (x == 4 || x == 8 || x == 16) ? x : 16; }();
     return v;
@@ -167,10 +208,19 @@ int tune_select_blocks_per_cu() {
     return v;
 }
 
+// One workgroup of 8 waves per tile in launch order (1), or persistent workgroups of 16 waves fed by a tile counter (0).
+// 2^26 / 2^28 Bools, 1 % / 25 % / 100 % set, 16 loads: ordered 22.7 / 39.4 / 122 us and 63 / 159 / 473 us, counter-fed
+// 24.1 / 40.8 / 118 and 69 / 168 / 460 us (four workgroups a compute unit overlap their phases better than two; the
+// look-back itself was not the limit: 16 waves in launch order measured 25 / 42 / 123 us).
+int tune_select_ordered() {
+    static const int v = [] { const char* s = std::getenv("RK_SELECT_ORDERED"); return s ? std::atoi(s) : 1; }();
+    return v;
+}
+
 size_t findall_workspace_need(int64_t n) {
-    const int64_t SEL_TILE = 16 * SEL_CHUNK * 4;                           // the smallest tile any configuration uses
+    const int64_t SEL_TILE = 8 * SEL_CHUNK * 4;                            // the smallest tile any configuration uses
     const int64_t ntiles = (n + SEL_TILE - 1) / SEL_TILE, ngroups = (ntiles + WAVE - 1) / WAVE;
-    return (size_t)(ntiles + ngroups) * Words<int64_t>::N * sizeof(uint64_t);
+    return ((size_t)ntiles * Words<int64_t>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);   // the ordered layout, the larger
 }
 
 }  // namespace rk
@@ -199,7 +249,8 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     }
     if (bools == nullptr || ys == nullptr) return RK_ERR_INVALID_ARGUMENT;
     if (n > 0xffffffffll) small = false;
-    const int nw = 16, kl = tune_select_loads();
+    const bool ordered = tune_select_ordered() != 0;
+    const int nw = ordered ? 8 : 16, kl = tune_select_loads();
     const int64_t SEL_TILE = (int64_t)nw * SEL_CHUNK * kl;
     const int64_t ntiles = (n + SEL_TILE - 1) / SEL_TILE, ngroups = (ntiles + WAVE - 1) / WAVE;
     if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
@@ -207,25 +258,33 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     if (!carve_workspace(ws, ws_bytes, findall_workspace_need(n), &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
     int64_t grid = (int64_t)device_info().cus * tune_select_blocks_per_cu();
-    if (grid > ntiles) grid = ntiles;
+    if (grid > ntiles || ordered) grid = ntiles;
+    const int tg = ordered_ticket_group(ntiles);
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const int aligned = is_aligned(bools, 16) ? 1 : 0;
     const WaitCtl wc = wait_ctl(w.hdr);
     hipStream_t st = (hipStream_t)stream;
-#define RK_SELECT2(LIN, SM, NWW, KK)                                                                                             \
-    findall_select_kernel<LIN, SM, NWW, KK><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned, counter,  \
-                                                                                   w.desc, ntiles, ngroups, cap, wc)
+#define RK_SELECT3(LIN, SM, NWW, KK, ORD)                                                                                        \
+    findall_select_kernel<LIN, SM, NWW, KK, ORD><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned,      \
+                                                                                        counter, w.tickets, tg, w.desc, ntiles,    \
+                                                                                        ngroups, cap, wc)
+#define RK_SELECT2(LIN, SM, KK)                                                                                                  \
+    do {                                                                                                                         \
+        if (ordered) RK_SELECT3(LIN, SM, 8, KK, true);                                                                           \
+        else RK_SELECT3(LIN, SM, 16, KK, false);                                                                                 \
+    } while (0)
 #define RK_SELECT(LIN, SM)                                                                                                       \
     do {                                                                                                                         \
-        if (kl == 4) RK_SELECT2(LIN, SM, 16, 4);                                                                                 \
-        else if (kl == 8) RK_SELECT2(LIN, SM, 16, 8);                                                                            \
-        else RK_SELECT2(LIN, SM, 16, 16);                                                                                        \
+        if (kl == 4) RK_SELECT2(LIN, SM, 4);                                                                                     \
+        else if (kl == 8) RK_SELECT2(LIN, SM, 8);                                                                                \
+        else RK_SELECT2(LIN, SM, 16);                                                                                            \
     } while (0)
     if (ndim <= 1) RK_SELECT(true, true);
     else if (small) RK_SELECT(false, true);
     else RK_SELECT(false, false);
 #undef RK_SELECT
 #undef RK_SELECT2
+#undef RK_SELECT3
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }

@@ -90,3 +90,36 @@ def test_selection_by_mask(rk, orc, dtype):
     with pytest.raises(IndexError):
         rk.getindex_mask(rk.ROCArray(x), rk.ROCArray(np.ones(5, dtype=bool)))
     assert rk.getindex_mask(rk.ROCArray(x), rk.ROCArray(np.zeros((33, 65), dtype=bool))).dims == (0,)
+
+
+def test_the_paths_the_tunables_select():
+    """RK_SELECT_ORDERED=0 (persistent workgroups fed by a tile counter) and RK_SCAN_DYNAMIC_IDS=1 (the same for the
+    long scans) are read once per process, so they are exercised in a child process: findall and a long cumsum against
+    numpy, several calls on one workspace."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = r'''
+import sys
+sys.path.insert(0, %r)
+import numpy as np
+from __graft_entry__ import load_package
+rk = load_package()
+rng = np.random.default_rng(5)
+for n, dens in ((1 << 21) + 77, 0.3), ((1 << 22), 0.01), (300_000, 1.0), (5, 0.5):
+    m = rng.random(n) < dens
+    got = rk.Array(rk.findall(rk.ROCArray(m)))
+    assert np.array_equal(got, np.flatnonzero(m) + 1), (n, dens)
+m = rng.random((257, 3001)) < 0.4
+got = rk.Array(rk.findall(rk.ROCArray(m)))
+want = np.argwhere(m.T)[:, ::-1] + 1                  # column-major order of the hits
+assert np.array_equal(got.T, want)
+x = rng.integers(-100, 100, size=(1 << 22) + 3).astype(np.int32)
+for _ in range(3):
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(x))), np.cumsum(x, dtype=np.int32))
+print("child ok")
+''' % root
+    env = dict(os.environ, RK_SELECT_ORDERED="0", RK_SCAN_DYNAMIC_IDS="1")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and "child ok" in out.stdout, out.stdout[-2000:] + out.stderr[-2000:]
