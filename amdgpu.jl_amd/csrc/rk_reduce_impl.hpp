@@ -639,14 +639,15 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         for (int j = 0; j < VEC; ++j) f[j] = Op::template identity<Acc>();
         int i = wave;
         if constexpr (VEC <= 4) {
-            for (; i + 3 * NW < msplits; i += 4 * NW) {
-                Acc v[4][VEC];
+            constexpr int FU = 4;            // rows a wave has in flight
+            for (; i + (FU - 1) * NW < msplits; i += FU * NW) {
+                Acc v[FU][VEC];
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < FU; ++u)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) v[u][j] = prow[(int64_t)(i + u * NW) * COLS + j];
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < FU; ++u)
 #pragma unroll
                     for (int j = 0; j < VEC; ++j) f[j] = op(f[j], v[u][j]);
             }
@@ -1012,11 +1013,11 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
     }
     // A long reduced dim behind a short contiguous one (sum(A; dims=2) of a 64 x 1_000_000 array): lanes along `inner` fill
     // a quarter of the strided kernel's 256-column strip (2.8 TB/s), and the narrow kernel moves 4 bytes a lane (32 x N:
-    // 3.8 TB/s).  With one or two strips in all (256 x 250_000), the last workgroup of a strip folds hundreds of rows of
+    // 3.8 TB/s; with 3 columns it holds 5 TB/s and stays: 3 x 2^24 44.7 against 45.0 us in two launches).  With one or two strips in all (256 x 250_000), the last workgroup of a strip folds hundreds of rows of
     // partials alone.  f consecutive rows are one row of f * inner elements -- the same memory -- so the array is
     // reduced as (f * inner) x (mid / f), with full strips and at least 16 of them where a factor allows, into a
     // temporary, whose f groups of `inner` columns a second, tiny reduction folds.
-    if (s.single_run && s.inner > 1 && s.mid >= 4096 && is_aligned(a.A, 16)) {
+    if (s.single_run && s.inner >= 4 && s.mid >= 4096 && is_aligned(a.A, 16)) {
         constexpr int64_t VEC = 16 / (int64_t)sizeof(In), COLS = WAVE * VEC;
         constexpr int64_t WANT_TILES = 16;
         const int64_t cols0 = s.inner % VEC == 0 ? COLS : WAVE;
