@@ -325,3 +325,31 @@ def test_narrow_element_types(rk, orc, dtype):
             np.testing.assert_allclose(rk.Array(dy).astype(np.float64), want.astype(np.float64), rtol=4e-3, atol=1e-4)
         else:
             assert np.array_equal(rk.Array(dy), want.astype(dt))
+
+
+@pytest.mark.parametrize("m", [8, 9, 11, 129, 255, 1001, 2047, 2049, 3001, 4095, 4097, 8189, 8190, 8191])
+def test_lines_that_start_at_odd_addresses(rk, orc, m):
+    """cumsum(A; dims=1) with a line length that is no whole number of 16-byte vectors: the tile is laid over the aligned
+    vectors that cover the line (every shift 0 .. 3 occurs across the lines), the head of the first and the tail of the
+    last line take their elements one by one.  8190 / 8191 Float32 no longer fit the largest tile with their shift and
+    take the element-wise kernel.  Integers bit-exact, floats rtol 1e-4 of the Float64 scan."""
+    rng = np.random.default_rng(m)
+    for dtype, n in ((np.float32, 37), (np.int32, 5), (np.float64, 6), (np.int64, 1)):
+        if dtype in (np.float64, np.int64) and m > 4097:
+            continue
+        x = (rng.standard_normal((m, n)) * 10).astype(dtype)
+        dx = rk.ROCArray(x)
+        for op, inclusive, init in (("add", True, None), ("max", True, None), ("add", False, dtype(7)), ("min", True, dtype(-2))):
+            got = rk.Array(rk.accumulate(op, dx, dims=1, init=init, inclusive=inclusive))
+            want = orc.accumulate(op, x, dims=1, init=init, inclusive=inclusive)
+            if np.dtype(dtype).kind == "f" and op == "add":
+                np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-3 if dtype == np.float32 else 1e-9)
+            else:
+                assert np.array_equal(got, want.astype(dtype)), (dtype, op)
+    b = rng.random((m, 9)) < 0.3                                   # Bool -> Int64: one-byte input vectors
+    assert np.array_equal(rk.Array(rk.cumsum(rk.ROCArray(b), dims=1)), orc.accumulate("add", b, dims=1))
+    # a view whose first element sits at an odd address, one line and many
+    flat = (rng.standard_normal(m * 3 + 5) * 10).astype(np.float32)
+    d = rk.ROCArray(flat)
+    v = d.view_range(4, m + 3)                                     # elements 4 .. m + 3 (1-based): byte offset 12
+    np.testing.assert_allclose(rk.Array(rk.cumsum(v)), np.cumsum(flat[3:m + 3].astype(np.float64)), rtol=1e-4, atol=1e-3)
