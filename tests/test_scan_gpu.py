@@ -334,8 +334,9 @@ def test_lines_that_start_at_odd_addresses(rk, orc, m):
     last line take their elements one by one.  8190 / 8191 Float32 no longer fit the largest tile with their shift and
     take the element-wise kernel.  Integers bit-exact, floats rtol 1e-4 of the Float64 scan."""
     rng = np.random.default_rng(m)
-    for dtype, n in ((np.float32, 37), (np.int32, 5), (np.float64, 6), (np.int64, 1)):
-        if dtype in (np.float64, np.int64) and m > 4097:
+    # fewer than 64 lines: a workgroup per line; 130 lines of up to 1024 elements: a wave per line
+    for dtype, n in ((np.float32, 37), (np.int32, 5), (np.float64, 6), (np.int64, 1), (np.float32, 130), (np.int64, 67)):
+        if (dtype in (np.float64, np.int64) and m > 4097) or (n > 64 and m > 1024):
             continue
         x = (rng.standard_normal((m, n)) * 10).astype(dtype)
         dx = rk.ROCArray(x)
