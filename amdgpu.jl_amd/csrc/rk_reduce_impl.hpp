@@ -526,9 +526,19 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     const int64_t o = tile / strips;
     const int strip = (int)(tile - o * strips);
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int64_t col0 = (int64_t)strip * COLS + (int64_t)lane * VEC;
-    const bool live = col0 < g.inner;      // inner % VEC == 0 on the vector path
+    const int64_t nominal = (int64_t)strip * COLS + (int64_t)lane * VEC;
+    const bool live = nominal < g.inner;
+    // 4- and 8-byte elements: vectors at any element-aligned address (load_nt_elems), so rows need be no whole number
+    // of vectors.  The last vector of such a row starts VEC elements before the row's end instead of running into the
+    // next row; the `dup` leading columns it shares with the lane before are dropped after the loop.
+    constexpr bool ANY_ALIGN = VECTOR && sizeof(In) >= 4;
+    const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
+    const int dup = (int)(nominal - col0);
     const int64_t slab = o * g.inner * g.mid;
+    auto load_row = [](const In* q) -> V {
+        if constexpr (ANY_ALIGN) return load_nt_elems<In, VEC>(q);
+        else return load_nt((const V*)q);
+    };
 
     Acc acc[VEC];
 #pragma unroll
@@ -546,7 +556,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
             V v[UNROLL];
             if (m + (UNROLL - 1) * NW < g.mid) {
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) v[u] = load_nt((const V*)(p + (m + u * NW) * g.inner));
+                for (int u = 0; u < UNROLL; ++u) v[u] = load_row(p + (m + u * NW) * g.inner);
                 if constexpr (XfIsBatch<Xf>::value) {
                     In x[UNROLL * VEC];
                     Acc y[UNROLL * VEC];
@@ -576,7 +586,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
                 }
             } else {
                 for (int64_t r = m; r < g.mid; r += NW) {
-                    const V x = load_nt((const V*)(p + r * g.inner));
+                    const V x = load_row(p + r * g.inner);
                     const typename Xf::Pos e0 = (typename Xf::Pos)r;
                     if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(x, e0));
                     else {
@@ -588,7 +598,8 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         }
     }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = acc[j];
+    for (int j = 0; j < VEC; ++j)
+        if (j >= dup) lds[wave][lane * VEC + j - dup] = acc[j];      // columns past the row's end keep whatever LDS held: never sunk
     __syncthreads();
     // thread t folds columns t, t + 256, ... of the strip: a strip has 64 * VEC columns -- 256 for 4-byte elements, one
     // a thread; 512 or 1024 for 2- and 1-byte elements
@@ -782,7 +793,8 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
     }
     if (s.inner >= 64) {
         p.kind = ReducePlan::STRIDED;
-        p.vector = (s.inner % VEC == 0) && is_aligned(A, 16);
+        // 4- and 8-byte elements: vectors at any element-aligned address, rows of any length >= a vector
+        p.vector = sizeof(In) >= 4 ? is_aligned(A, sizeof(In)) : (s.inner % VEC == 0) && is_aligned(A, 16);
         const int cols = WAVE * (p.vector ? VEC : 1);
         const int64_t strips = (s.inner + cols - 1) / cols;
         p.strips = (int)strips;
@@ -1022,7 +1034,7 @@ inline int32_t mapreduce_one(const MapreduceArgs& a, const Xf& xf) {
     if (s.single_run && s.inner >= 4 && s.mid >= 1024 && is_aligned(a.A, 16)) {
         constexpr int64_t VEC = 16 / (int64_t)sizeof(In), COLS = WAVE * VEC;
         constexpr int64_t WANT_TILES = 16;
-        const int64_t cols0 = s.inner % VEC == 0 ? COLS : WAVE;
+        const int64_t cols0 = (sizeof(In) >= 4 || s.inner % VEC == 0) ? COLS : WAVE;      // the strided kernel's strip (plan_reduce)
         const int64_t strips0 = (s.inner + cols0 - 1) / cols0;
         const bool poor = cols0 == WAVE || (s.mid >= 4096 && (s.inner < WAVE || s.inner * 10 < strips0 * cols0 * 7 || strips0 * s.outer < 4));
         Workspace w{};

@@ -98,8 +98,74 @@ static int32_t launch_reverse(const void* x, void* y, const RevGeom& g, hipStrea
     return RK_SUCCESS;
 }
 
+// ---- rows that are no whole number of 16-byte units (reverse(A; dims=1) of a 1001 x N Float32 array) ----------------
+// One element per lane moves 4 bytes a lane, 3 TB/s.  Global memory takes 16-byte accesses at any element-aligned
+// address (only LDS wants them aligned to their size), so a lane moves a group of 16 / E consecutive elements of a row
+// with one load and one store, neither 16-byte aligned in general; a flipped first dim reverses the elements inside
+// the group.  The last group of a row, when it is short, goes element by element.  Out of place only.
+template <int E> struct GroupOf;
+template <> struct GroupOf<4> { typedef uint32_t elem; typedef uint32_t type __attribute__((ext_vector_type(4), aligned(4))); };
+template <> struct GroupOf<8> { typedef uint64_t elem; typedef uint64_t type __attribute__((ext_vector_type(2), aligned(8))); };
+
+template <int E, typename I>
+__global__ __launch_bounds__(256) void reverse_groups_kernel(const typename GroupOf<E>::elem* __restrict__ x,
+                                                             typename GroupOf<E>::elem* __restrict__ y, RevGeom g, int64_t groups_per_row,
+                                                             int64_t ngroups) {
+    typedef typename GroupOf<E>::type G;
+    constexpr int N = 16 / E;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= ngroups) return;
+    const I ext0 = (I)g.ext[0];
+    const I row = (I)i / (I)groups_per_row, q = (I)i - row * (I)groups_per_row;
+    const I c0 = q * N;
+    const int n = ext0 - c0 < (I)N ? (int)(ext0 - c0) : N;
+    // the row the row moves to: dims 1 .. nd-1 flipped like flipped_index does
+    I rem = row, orow = 0, stride = 1;
+    for (int d = 1; d < g.nd; ++d) {
+        const I e = (I)g.ext[d];
+        I c;
+        if (d == g.nd - 1) c = rem;
+        else { const I qd = rem / e; c = rem - qd * e; rem = qd; }
+        if (g.flip >> d & 1u) c = e - 1 - c;
+        orow += c * stride;
+        stride *= e;
+    }
+    const bool flip0 = g.flip & 1u;
+    const int64_t src = (int64_t)row * (int64_t)ext0 + (int64_t)c0;
+    const int64_t dst = (int64_t)orow * (int64_t)ext0 + (int64_t)(flip0 ? ext0 - c0 - (I)n : c0);
+    if (n == N) {
+        G v = __builtin_nontemporal_load((const G*)(x + src));
+        if (flip0) {
+            if constexpr (N == 4) v = G{v[3], v[2], v[1], v[0]};
+            else v = G{v[1], v[0]};
+        }
+        __builtin_nontemporal_store(v, (G*)(y + dst));
+    } else {
+        for (int j = 0; j < n; ++j) y[dst + (flip0 ? n - 1 - j : j)] = x[src + j];
+    }
+}
+
+template <int E>
+static int32_t launch_reverse_groups(const void* x, void* y, const RevGeom& g, hipStream_t stream) {
+    constexpr int N = 16 / E;
+    const int64_t groups_per_row = (g.ext[0] + N - 1) / N, rows = g.total / g.ext[0];
+    if (rows != 0 && groups_per_row > INT64_MAX / rows) return RK_ERR_TOO_LARGE;
+    const int64_t ngroups = groups_per_row * rows, blocks = (ngroups + 255) / 256;
+    if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+    typedef typename GroupOf<E>::elem elem;
+    if (g.total <= 0x7fffffffll)
+        reverse_groups_kernel<E, uint32_t><<<(unsigned)blocks, 256, 0, stream>>>((const elem*)x, (elem*)y, g, groups_per_row, ngroups);
+    else
+        reverse_groups_kernel<E, int64_t><<<(unsigned)blocks, 256, 0, stream>>>((const elem*)x, (elem*)y, g, groups_per_row, ngroups);
+    RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
 template <int E>
 static int32_t reverse_elsize(const void* x, void* y, RevGeom g, bool vector, hipStream_t stream) {
+    if constexpr (E == 4 || E == 8) {
+        if (!vector && x != y && g.ext[0] >= 16 / E) return launch_reverse_groups<E>(x, y, g, stream);
+    }
     if (vector) {
         g.ext[0] = g.ext[0] * E / 16;
         g.total = g.total * E / 16;

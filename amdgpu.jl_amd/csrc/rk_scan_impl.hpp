@@ -1034,8 +1034,14 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     __shared__ T lds[NW][COLS];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int64_t o = (int64_t)blockIdx.x / strips, strip = (int64_t)blockIdx.x - o * strips;
-    const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
-    const bool live = col0 < g.inner;
+    // 4- and 8-byte elements: vectors at any element-aligned address, so rows need be no whole number of vectors.  The
+    // last vector of such a row starts VEC elements before the row's end instead of running into the next row: its
+    // leading columns are scanned, and stored, by the lane before as well, with the same values.  Column totals are
+    // kept per lane slot (`nominal`), which is the column for every other lane.
+    constexpr bool ANY_ALIGN = VECTOR && sizeof(In) >= 4 && sizeof(T) >= 4;
+    const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
+    const bool live = nominal < g.inner;
+    const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
     const int64_t slab = o * g.inner * g.mid;
     // (Running the slices last to first, so that the scan starts with what the totals pass read last, changed nothing.)
     const int64_t slice = (int64_t)blockIdx.y;
@@ -1045,14 +1051,16 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     T carry[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
-        carry[j] = (carry_in != nullptr && live) ? carry_in[(o * gridDim.y + slice) * carry_pitch + col0 + j] : init;
+        carry[j] = (carry_in != nullptr && live) ? carry_in[(o * gridDim.y + slice) * carry_pitch + nominal + j] : init;
     for (int64_t m0 = m_begin; m0 < m_end; m0 += NW * R) {
         const int64_t row0 = m0 + (int64_t)wave * R;
         T v[R][VEC];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (live && row0 + r < m_end) {
-                const VI x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
+                VI x;
+                if constexpr (ANY_ALIGN) x = load_nt_elems<In, VEC>(in + slab + (row0 + r) * g.inner + col0);
+                else x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
                 if constexpr (VEC == 1) v[r][0] = (T)x;
                 else {
 #pragma unroll
@@ -1092,7 +1100,8 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
                     for (int j = 0; j < VEC; ++j)
                         o[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r - 1][j]));
                 }
-                store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o);
+                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + slab + (row0 + r) * g.inner + col0, o);
+                else store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o);
             }
         }
     }
@@ -1109,9 +1118,15 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
     __shared__ T lds[NW][COLS];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int64_t o = (int64_t)blockIdx.x / strips, strip = (int64_t)blockIdx.x - o * strips;
-    const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
-    const bool live = col0 < g.inner;
+    constexpr bool ANY_ALIGN = VECTOR && sizeof(In) >= 4 && sizeof(T) >= 4;     // as in scan_strided_kernel
+    const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
+    const bool live = nominal < g.inner;
+    const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
     const int64_t slab = o * g.inner * g.mid;
+    auto load_row = [](const In* q) -> VI {
+        if constexpr (ANY_ALIGN) return load_elems<In, VEC>(q);
+        else return *(const VI*)q;
+    };
     const int64_t m_begin = (int64_t)blockIdx.y * rows_per_slice;
     const int64_t m_end = m_begin + rows_per_slice < g.mid ? m_begin + rows_per_slice : g.mid;
     T acc[VEC];
@@ -1125,7 +1140,7 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
         for (; m + (UNROLL - 1) * NW < m_end; m += UNROLL * NW) {
             VI x[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) x[u] = *(const VI*)(in + slab + (m + u * NW) * g.inner + col0);
+            for (int u = 0; u < UNROLL; ++u) x[u] = load_row(in + slab + (m + u * NW) * g.inner + col0);
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 if constexpr (VEC == 1) acc[0] = op(acc[0], (T)x[u]);
@@ -1136,7 +1151,7 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
             }
         }
         for (; m < m_end; m += NW) {
-            const VI x = *(const VI*)(in + slab + m * g.inner + col0);
+            const VI x = load_row(in + slab + m * g.inner + col0);
             if constexpr (VEC == 1) acc[0] = op(acc[0], (T)x);
             else {
 #pragma unroll
@@ -1345,8 +1360,12 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
         __syncthreads();
     } else {
         const int64_t o = chain / strips, strip = chain - o * strips;
-        const int64_t col0 = strip * COLS + (int64_t)lane * VEC;
-        const bool live = col0 < g.inner;                    // inner % VEC == 0: a vector is entirely inside or outside
+        // rows that are no whole number of vectors: the last vector starts VEC elements before the row's end (see
+        // scan_strided_kernel); payloads are per lane slot, the same columns in every tile of the strip
+        constexpr bool ANY_ALIGN = sizeof(In) >= 4 && sizeof(T) >= 4;
+        const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
+        const bool live = nominal < g.inner;
+        const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
         const int64_t slab = o * g.inner * g.mid;
         const int64_t row0 = slice * (NW * R) + (int64_t)wave * R;
         VT v[R];
@@ -1357,7 +1376,9 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (live && row0 + r < g.mid) {
-                const VI x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
+                VI x;
+                if constexpr (ANY_ALIGN) x = load_nt_elems<In, VEC>(in + slab + (row0 + r) * g.inner + col0);
+                else x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) v[r][j] = (T)x[j];
             } else {
@@ -1387,7 +1408,8 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
                 VT o4;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o4[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r > 0 ? r - 1 : 0][j]));
-                store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o4);
+                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + slab + (row0 + r) * g.inner + col0, o4);
+                else store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o4);
             }
         }
     }
@@ -1431,7 +1453,9 @@ template <typename In, typename T, typename Op>
 inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, bool aligned, char* scratch,
                                 size_t scratch_bytes, hipStream_t stream, const Workspace* ws = nullptr) {
     constexpr int VEC = 16 / sizeof(T);
-    const bool vec = aligned && (g.inner % VEC == 0);
+    // 4- and 8-byte elements: vectors at any element-aligned address, rows of any length (>= 64 here)
+    const bool vec = (sizeof(In) >= 4 && sizeof(T) >= 4) ? (is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) && g.inner >= VEC)
+                                                         : (aligned && g.inner % VEC == 0);
     const int cols = WAVE * (vec ? VEC : 1);
     const int64_t strips = (g.inner + cols - 1) / cols;
     if (strips * g.outer > 0x7fffffff) return RK_ERR_TOO_LARGE;

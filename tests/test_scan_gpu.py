@@ -354,3 +354,28 @@ def test_lines_that_start_at_odd_addresses(rk, orc, m):
     d = rk.ROCArray(flat)
     v = d.view_range(4, m + 3)                                     # elements 4 .. m + 3 (1-based): byte offset 12
     np.testing.assert_allclose(rk.Array(rk.cumsum(v)), np.cumsum(flat[3:m + 3].astype(np.float64)), rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("shape", [(257, 300), (1001, 1000), (4097, 130), (65, 5000), (130, 70, 5), (67, 40, 9), (8191, 33)])
+def test_scans_across_rows_that_are_no_whole_vectors(rk, orc, shape):
+    """cumsum(A; dims=2) with a first extent that is no multiple of the 16-byte vector: every row has another alignment.
+    The kernels read and write vectors at element-aligned addresses; the last vector of a row starts four (two)
+    elements before the row's end.  All three paths: one workgroup per strip, sliced with carried totals, and the
+    single pass over tiles of rows.  In place too."""
+    rng = np.random.default_rng(sum(shape))
+    for dtype in (np.float32, np.int32, np.float64, np.int64):
+        x = (rng.standard_normal(shape) * 10).astype(dtype)
+        dx = rk.ROCArray(x)
+        for op, inclusive, init in (("add", True, None), ("max", True, None), ("add", False, dtype(3))):
+            got = rk.Array(rk.accumulate(op, dx, dims=2, init=init, inclusive=inclusive))
+            want = orc.accumulate(op, x, dims=2, init=init, inclusive=inclusive)
+            if np.dtype(dtype).kind == "f" and op == "add":
+                np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-2 if dtype == np.float32 else 1e-9)
+            else:
+                assert np.array_equal(got, want.astype(dtype)), (dtype, op)
+        rk.accumulate_("add", dx, dx, dims=2)
+        want = orc.accumulate("add", x, dims=2)
+        if np.dtype(dtype).kind == "f":
+            np.testing.assert_allclose(rk.Array(dx), want, rtol=1e-4, atol=1e-2 if dtype == np.float32 else 1e-9)
+        else:
+            assert np.array_equal(rk.Array(dx), want.astype(dtype))
