@@ -240,6 +240,19 @@ template <typename T, int K> struct TileRegs {
     typename VecOf<T, VEC>::type v[K];     // scan of the wave's part up to and including (inclusive) / excluding the element
 };
 
+// Vectors at element-aligned addresses (load_nt_elems) exist for 4- and 8-byte elements; for the rest these are
+// never called (value == false) but must compile.
+template <typename In, typename T, bool OK = (sizeof(In) >= 4 && sizeof(T) >= 4)> struct ElemVectors {
+    static constexpr bool value = true;
+    template <int N> static __device__ __forceinline__ typename VecOf<In, N>::type load(const In* p) { return load_nt_elems<In, N>(p); }
+    template <int N> static __device__ __forceinline__ void store(In* p, typename VecOf<In, N>::type v) { store_nt_elems<In, N>(p, v); }
+};
+template <typename In, typename T> struct ElemVectors<In, T, false> {
+    static constexpr bool value = false;
+    template <int N> static __device__ __forceinline__ typename VecOf<In, N>::type load(const In*) { return typename VecOf<In, N>::type{}; }
+    template <int N> static __device__ __forceinline__ void store(In*, typename VecOf<In, N>::type) {}
+};
+
 // The values of a wave's part, loaded into r, scanned in place; returns the total of the part.
 template <typename T, typename Op, int K>
 __device__ __forceinline__ T tile_scan_regs(int inclusive, Op op, TileRegs<T, K>& r) {
@@ -295,8 +308,25 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
 #pragma unroll
             for (int j = 0; j < VEC; ++j) r.v[k][j] = have ? (T)x[j] : ident;
         }
+    } else if (ElemVectors<In, T>::value && valid >= VEC) {
+        // lines that start at odd addresses, or whose length is no whole number of vectors: global memory takes 16-byte
+        // accesses at any element-aligned address, so only the one vector the line's end cuts goes element by element.
+        // Unconditional loads again (a vector past the end reads the tile's first).
+        const In* p = in + e0;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int idx = woff + k * WAVE * VEC;
+            const bool whole = idx + VEC <= valid;
+            const VI x = ElemVectors<In, T>::template load<VEC>(p + (whole ? idx : 0));
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[k][j] = whole ? (T)x[j] : ident;
+            if (!whole && idx < valid) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (idx + j < valid) r.v[k][j] = (T)p[idx + j];
+            }
+        }
     } else {
-        // lines that start at odd addresses: element loads, unconditional like the vectors above
 #pragma unroll
         for (int k = 0; k < K; ++k)
 #pragma unroll
@@ -336,6 +366,20 @@ __device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int 
             for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
             if (idx < valid) store_nt((VT*)(out + e0 + idx), o);
         }
+    } else if (ElemVectors<T, T>::value) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int idx = woff + k * WAVE * VEC;
+            VT o;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
+            if (idx + VEC <= valid) ElemVectors<T, T>::template store<VEC>(out + e0 + idx, o);
+            else if (idx < valid) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    if (idx + j < valid) out[e0 + idx + j] = o[j];
+            }
+        }
     } else {
 #pragma unroll
         for (int k = 0; k < K; ++k)
@@ -365,70 +409,6 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ 
     for (int w = 0; w < NW; ++w)
         if (w < wave) wave_prefix = op(wave_prefix, lds_wave[w]);
     tile_store<T, Op, VECTOR, K>(out, e0, (int)line_len, op(init, wave_prefix), op, r);
-}
-
-// ---- the same for lines that start at odd addresses (cumsum(A; dims=1) of a 3001 x N Float32 array) ------------
-// Element-wise accesses reach 3.7 TB/s.  Here the tile is laid over the ALIGNED vectors that cover the line: `shift`
-// elements of the line's first vector belong to the line in front (identity for the scan, not stored), likewise the
-// tail of its last vector, so every lane moves whole 16-byte vectors whatever the line's address; the host launches
-// this only when `in` and `out` have the same shift.  Vectors that straddle the line's ends are read whole where that
-// stays inside the array -- everywhere but at the head of the first and the tail of the last line, which take their
-// elements one by one -- and are written element by element.  The loads are unconditional (out-of-line vectors read
-// the line's first whole vector again): a load under a condition of its own is waited for before the next is issued.
-template <typename In, typename T, typename Op, int K>
-__global__ __launch_bounds__(256) void scan_tiles_shifted_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
-                                                                 int64_t nlines, int base_shift, T init, int inclusive, Op op) {
-    constexpr int NW = 4;
-    constexpr int VEC = 16 / sizeof(T);
-    typedef typename VecOf<In, VEC>::type VI;
-    typedef typename VecOf<T, VEC>::type VT;
-    __shared__ T lds_wave[NW];
-    const T ident = Op::template identity<T>();
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int64_t line = blockIdx.x;
-    const int64_t e0 = line * line_len;
-    const int shift = (int)((base_shift + e0) % VEC);          // elements of the first vector in front of the line
-    const int lo = shift, hi = shift + (int)line_len;          // the line inside the tile
-    const In* pa = in + e0 - shift;                            // vector-aligned (the host checked base_shift)
-    T* qa = out + e0 - shift;
-    const int first_whole = shift > 0 ? VEC : 0;               // < hi: the host launches this for lines of >= 2 * VEC
-    const int woff = wave * (WAVE * VEC * K) + lane * VEC;
-    TileRegs<T, K> r;
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int idx = woff + k * WAVE * VEC;
-        const bool touches = idx < hi && idx + VEC > lo;
-        const bool outside_array = (line == 0 && idx < lo) || (line == nlines - 1 && idx + VEC > hi);
-        const bool vec_ok = touches && !outside_array;
-        const VI x = load_nt((const VI*)(pa + (vec_ok ? idx : first_whole)));
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) r.v[k][j] = (vec_ok && idx + j >= lo && idx + j < hi) ? (T)x[j] : ident;
-        if (touches && outside_array) {                        // two vectors in the whole array
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                if (idx + j >= lo && idx + j < hi) r.v[k][j] = (T)pa[idx + j];
-        }
-    }
-    const T wtot = tile_scan_regs<T, Op, K>(inclusive, op, r);
-    if (lane == 0) lds_wave[wave] = wtot;
-    __syncthreads();
-    T base = init;
-#pragma unroll
-    for (int w = 0; w < NW; ++w)
-        if (w < wave) base = op(base, lds_wave[w]);
-#pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int idx = woff + k * WAVE * VEC;
-        VT o;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
-        if (idx >= lo && idx + VEC <= hi) store_nt((VT*)(qa + idx), o);
-        else if (idx < hi && idx + VEC > lo) {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                if (idx + j >= lo && idx + j < hi) qa[idx + j] = o[j];
-        }
-    }
 }
 
 // ---- long contiguous lines: persistent workgroups, single pass, two-level decoupled look-back --------------
@@ -617,10 +597,15 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
 }
 
 // ---- contiguous lines shorter than a tile: one wave per line -------------------------------------
+// VECTOR: lines are whole 16-byte vectors at 16-byte aligned addresses.  Otherwise, for 4- and 8-byte elements, the lanes
+// still take 16 bytes each -- global memory accepts that at any element-aligned address -- and only the vector the
+// line's end cuts goes element by element (cumsum(A; dims=1) of 257 x 240000 Float32: 143 us with one element a
+// lane, 100 us).
 template <typename In, typename T, typename Op, bool VECTOR, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
                                                                 int64_t nlines, T init, int inclusive, Op op) {
-    constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
+    constexpr bool ELEMS = !VECTOR && ElemVectors<In, T>::value;        // vectors at element-aligned addresses
+    constexpr int VEC = (VECTOR || ELEMS) ? 16 / sizeof(T) : 1;
     typedef typename VecOf<T, VEC>::type VT;
     typedef typename VecOf<In, VEC>::type VI;
     const int64_t line = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
@@ -631,18 +616,24 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
     T carry = init;
     for (int64_t c = 0; c < line_len; c += WAVE * VEC) {
         const int64_t i0 = c + (int64_t)lane * VEC;
+        const bool whole = i0 + VEC <= line_len;               // VECTOR: line_len % VEC == 0, a vector is inside or outside
         T v[VEC];
-        if constexpr (VECTOR) {     // line_len % VEC == 0: a vector is entirely inside or outside
-            if (i0 < line_len) {
-                const VI x = load_nt((const VI*)(in + base + i0));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = ident;
+        if constexpr (VEC == 1) {
+            if (whole) v[0] = (T)in[base + i0];
+        } else {
+            if (whole) {
+                VI x;
+                if constexpr (ELEMS) x = ElemVectors<In, T>::template load<VEC>(in + base + i0);
+                else x = load_nt((const VI*)(in + base + i0));
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) v[j] = (T)x[j];
-            } else {
+            } else if (ELEMS && i0 < line_len) {
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) v[j] = ident;
+                for (int j = 0; j < VEC; ++j)
+                    if (i0 + j < line_len) v[j] = (T)in[base + i0 + j];
             }
-        } else {
-            v[0] = i0 < line_len ? (T)in[base + i0] : ident;
         }
 #pragma unroll
         for (int j = 1; j < VEC; ++j) v[j] = op(v[j - 1], v[j]);
@@ -650,7 +641,9 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
         const T off = op(carry, wave_shift_right(inc, ident));
         carry = op(carry, read_lane(inc, WAVE - 1));
         if (i0 < line_len) {
-            if constexpr (VECTOR) {
+            if constexpr (VEC == 1) {
+                out[base + i0] = inclusive ? op(off, v[0]) : off;
+            } else {
                 VT o;
                 if (inclusive) {
 #pragma unroll
@@ -660,68 +653,15 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
 #pragma unroll
                     for (int j = 1; j < VEC; ++j) o[j] = op(off, v[j - 1]);
                 }
-                store_nt((VT*)(out + base + i0), o);
-            } else {
-                out[base + i0] = inclusive ? op(off, v[0]) : off;
+                if (whole) {
+                    if constexpr (ELEMS) ElemVectors<T, T>::template store<VEC>(out + base + i0, o);
+                    else store_nt((VT*)(out + base + i0), o);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (i0 + j < line_len) out[base + i0 + j] = o[j];
+                }
             }
-        }
-    }
-}
-
-// ---- the same for lines that start at odd addresses: aligned vectors laid over the line ---------------------------
-// (see scan_tiles_shifted_kernel: `shift` elements of the first vector and the tail of the last belong to the
-// neighbouring lines -- identity for the scan, not stored; only the head of the first and the tail of the last line
-// are read element by element.  cumsum(A; dims=1) of a 257 x 240000 Float32 array: 143 us with element accesses.)
-template <typename In, typename T, typename Op, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void scan_wave_lines_shifted_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
-                                                                        int64_t nlines, int base_shift, T init, int inclusive, Op op) {
-    constexpr int VEC = 16 / sizeof(T);
-    typedef typename VecOf<T, VEC>::type VT;
-    typedef typename VecOf<In, VEC>::type VI;
-    const int64_t line = (int64_t)blockIdx.x * (BLOCK / WAVE) + threadIdx.x / WAVE;
-    if (line >= nlines) return;
-    const int lane = lane_id();
-    const T ident = Op::template identity<T>();
-    const int64_t e0 = line * line_len;
-    const int shift = (int)((base_shift + e0) % VEC);
-    const int lo = shift, hi = shift + (int)line_len;
-    const In* pa = in + e0 - shift;                            // vector-aligned (the host checked base_shift)
-    T* qa = out + e0 - shift;
-    const int first_whole = shift > 0 ? VEC : 0;               // < hi: lines of >= 2 * VEC elements
-    T carry = init;
-    for (int c = 0; c < hi; c += WAVE * VEC) {
-        const int idx = c + lane * VEC;
-        const bool touches = idx < hi && idx + VEC > lo;
-        const bool outside_array = (line == 0 && idx < lo) || (line == nlines - 1 && idx + VEC > hi);
-        const bool vec_ok = touches && !outside_array;
-        const VI x = load_nt((const VI*)(pa + (vec_ok ? idx : first_whole)));
-        T v[VEC];
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) v[j] = (vec_ok && idx + j >= lo && idx + j < hi) ? (T)x[j] : ident;
-        if (touches && outside_array) {                        // two vectors in the whole array
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                if (idx + j >= lo && idx + j < hi) v[j] = (T)pa[idx + j];
-        }
-#pragma unroll
-        for (int j = 1; j < VEC; ++j) v[j] = op(v[j - 1], v[j]);
-        const T inc = wave_scan_inclusive(v[VEC - 1], op, ident);
-        const T off = op(carry, wave_shift_right(inc, ident));
-        carry = op(carry, read_lane(inc, WAVE - 1));
-        VT o;
-        if (inclusive) {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) o[j] = op(off, v[j]);
-        } else {
-            o[0] = off;
-#pragma unroll
-            for (int j = 1; j < VEC; ++j) o[j] = op(off, v[j - 1]);
-        }
-        if (idx >= lo && idx + VEC <= hi) store_nt((VT*)(qa + idx), o);
-        else if (touches) {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                if (idx + j >= lo && idx + j < hi) qa[idx + j] = o[j];
         }
     }
 }
@@ -1661,16 +1601,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
     }
     // contiguous lines
     const bool lines_aligned = aligned && (nlines == 1 || s.mid % VEC == 0);
-    // lines at odd addresses: aligned vectors laid over them, when `in` and `out` are shifted alike
-    const int in_shift = (int)(((uintptr_t)in / sizeof(In)) % VEC), out_shift = (int)(((uintptr_t)out / sizeof(T)) % VEC);
-    const bool shifted_ok = !(lines_aligned && s.mid % VEC == 0) && in_shift == out_shift && is_aligned(in, sizeof(In)) &&
-                            is_aligned(out, sizeof(T)) && s.mid >= 2 * VEC;
     if (s.mid <= 1024 && nlines >= 64) {
         const int64_t blocks = (nlines + 3) / 4;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-        if (shifted_ok)
-            scan_wave_lines_shifted_kernel<In, T, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, in_shift, init, inclusive, op);
-        else if (lines_aligned && s.mid % VEC == 0)
+        if (lines_aligned && s.mid % VEC == 0)
             scan_wave_lines_kernel<In, T, Op, true, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
         else
             scan_wave_lines_kernel<In, T, Op, false, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
@@ -1681,14 +1615,6 @@ inline int32_t launch_scan(const ScanArgs& a) {
     if (s.mid <= ScanTile<T, 8>::TILE) {
         if (nlines > 0x7fffffff) return RK_ERR_TOO_LARGE;
         const unsigned grid = (unsigned)nlines;
-        if (shifted_ok && !lines_aligned && s.mid + VEC - 1 <= ScanTile<T, 8>::TILE) {
-            const int64_t span = s.mid + VEC - 1;
-            if (span <= ScanTile<T, 2>::TILE) scan_tiles_shifted_kernel<In, T, Op, 2><<<grid, 256, 0, a.stream>>>(in, out, s.mid, nlines, in_shift, init, inclusive, op);
-            else if (span <= ScanTile<T, 4>::TILE) scan_tiles_shifted_kernel<In, T, Op, 4><<<grid, 256, 0, a.stream>>>(in, out, s.mid, nlines, in_shift, init, inclusive, op);
-            else scan_tiles_shifted_kernel<In, T, Op, 8><<<grid, 256, 0, a.stream>>>(in, out, s.mid, nlines, in_shift, init, inclusive, op);
-            RK_LAUNCH_CHECK();
-            return RK_SUCCESS;
-        }
 #define RK_SCAN_TILES(KK)                                                                                             \
         do {                                                                                                          \
             if (lines_aligned) scan_tiles_kernel<In, T, Op, true, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op); \

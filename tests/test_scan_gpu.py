@@ -329,10 +329,10 @@ def test_narrow_element_types(rk, orc, dtype):
 
 @pytest.mark.parametrize("m", [8, 9, 11, 129, 255, 1001, 2047, 2049, 3001, 4095, 4097, 8189, 8190, 8191])
 def test_lines_that_start_at_odd_addresses(rk, orc, m):
-    """cumsum(A; dims=1) with a line length that is no whole number of 16-byte vectors: the tile is laid over the aligned
-    vectors that cover the line (every shift 0 .. 3 occurs across the lines), the head of the first and the tail of the
-    last line take their elements one by one.  8190 / 8191 Float32 no longer fit the largest tile with their shift and
-    take the element-wise kernel.  Integers bit-exact, floats rtol 1e-4 of the Float64 scan."""
+    """cumsum(A; dims=1) with a line length that is no whole number of 16-byte vectors: every line starts at another
+    alignment; the kernels take 16 bytes a lane at element-aligned addresses and only the vector that the line's end cuts
+    element by element.  A workgroup per line, a wave per line, and (8190 / 8191 Float32 upwards) the chained tiles.
+    Integers bit-exact, floats rtol 1e-4 of the Float64 scan."""
     rng = np.random.default_rng(m)
     # fewer than 64 lines: a workgroup per line; 130 lines of up to 1024 elements: a wave per line
     for dtype, n in ((np.float32, 37), (np.int32, 5), (np.float64, 6), (np.int64, 1), (np.float32, 130), (np.int64, 67)):
