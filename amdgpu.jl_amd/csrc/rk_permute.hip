@@ -99,7 +99,10 @@ __global__ __launch_bounds__(256) void permute_tiles_kernel(const T* __restrict_
 // tile row, so a request still spans TE * sizeof(T) contiguous bytes but with a quarter (or less) of the
 // instructions.  Needs ext[0] % V == 0 and ext[p] % V == 0 and 16-byte aligned arrays: every vector is then
 // entirely inside or outside the array, and every row start is aligned.
-template <typename T, int TE>
+// ELEMS (4- and 8-byte elements): extents and addresses need not be whole vectors -- global memory takes 16-byte
+// accesses at any element-aligned address.  The last vector of a row starts V elements before the row's end instead of
+// running past it; where that reaches back into the tile in front, the elements of this tile go one by one.
+template <typename T, int TE, bool ELEMS>
 __global__ __launch_bounds__(256) void permute_tiles_vec_kernel(const T* __restrict__ src, T* __restrict__ dst, PermGeom g, int64_t tiles0,
                                                                 int64_t tilesp) {
     constexpr int V = 16 / sizeof(T), LR = TE / V, RP = 256 / LR;
@@ -123,27 +126,40 @@ __global__ __launch_bounds__(256) void permute_tiles_vec_kernel(const T* __restr
     const int64_t i0 = t0 * TE, p0 = tp * TE;
     const int64_t n0 = g.ext[0], np = g.ext[g.p];
     if (i0 + c * V < n0) {
-        const T* s = src + sbase + i0 + c * V;
+        // first column of this lane's vector, relative to the tile: negative when the row's last vector reaches back
+        const int lc = (ELEMS && i0 + c * V + V > n0) ? (int)(n0 - V - i0) : c * V;
+        const T* s = src + sbase + i0 + lc;
 #pragma unroll
         for (int j = r; j < TE; j += RP) {
             if (p0 + j < np) {
-                const VT v = load_nt((const VT*)(s + (p0 + j) * sstride_p));
+                VT v;
+                if constexpr (ELEMS) v = load_nt_elems<T, V>(s + (p0 + j) * sstride_p);
+                else v = load_nt((const VT*)(s + (p0 + j) * sstride_p));
 #pragma unroll
-                for (int k = 0; k < V; ++k) tile[j][c * V + k] = v[k];
+                for (int k = 0; k < V; ++k)
+                    if (!ELEMS || lc + k >= 0) tile[j][lc + k] = v[k];
             }
         }
     }
     __syncthreads();
     if (p0 + c * V < np) {
-        T* q = dst + dbase + p0 + c * V;
+        const int lp = (ELEMS && p0 + c * V + V > np) ? (int)(np - V - p0) : c * V;
+        T* q = dst + dbase + p0 + lp;
         const int64_t ds0 = g.dstride[0];
 #pragma unroll
         for (int j = r; j < TE; j += RP) {
             if (i0 + j < n0) {
                 VT v;
 #pragma unroll
-                for (int k = 0; k < V; ++k) v[k] = tile[c * V + k][j];
-                store_nt((VT*)(q + (i0 + j) * ds0), v);
+                for (int k = 0; k < V; ++k) v[k] = tile[(ELEMS && lp + k < 0) ? 0 : lp + k][j];
+                if constexpr (ELEMS) {
+                    if (lp >= 0) store_nt_elems<T, V>(q + (i0 + j) * ds0, v);
+                    else {
+#pragma unroll
+                        for (int k = 0; k < V; ++k)
+                            if (lp + k >= 0) q[(i0 + j) * ds0 + k] = v[k];
+                    }
+                } else store_nt((VT*)(q + (i0 + j) * ds0), v);
             }
         }
     }
@@ -252,9 +268,22 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
             for (int d = 1; d < g.nd; ++d)
                 if (d != g.p) batch *= g.ext[d];
             if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
-            permute_tiles_vec_kernel<T, TE><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+            permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
+        }
+        if constexpr (E >= 4) {
+            if (g.ext[0] >= V && g.ext[g.p] >= V) {      // odd extents or addresses: the same tiles, element-aligned vectors
+                constexpr int TE = 64;
+                const int64_t tiles0 = (g.ext[0] + TE - 1) / TE, tilesp = (g.ext[g.p] + TE - 1) / TE;
+                int64_t batch = 1;
+                for (int d = 1; d < g.nd; ++d)
+                    if (d != g.p) batch *= g.ext[d];
+                if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+                permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+                RK_LAUNCH_CHECK();
+                return RK_SUCCESS;
+            }
         }
     }
     constexpr int PT = E == 16 ? 32 : 64;
