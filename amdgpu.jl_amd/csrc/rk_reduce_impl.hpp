@@ -317,6 +317,48 @@ __global__ __launch_bounds__(BLOCK) void reduce_thread_kernel(const In* __restri
     sink(line, a);
 }
 
+// ---- a short reduced dim behind a long contiguous one: a lane per group of columns ------------------------------
+// (sum(A; dims=2) of a 200 x 3 x 50000 or a 50000 x 3 x 200 array: the strided kernel gave every workgroup three rows
+// of a strip -- 39200 workgroups for 2.4 KB each, 2.4 TB/s; a lane per line reads 4 bytes at a time.)  A lane owns
+// VEC = 16 / sizeof(In) adjacent columns of one outer index and walks the <= 16 rows with 16-byte loads at
+// element-aligned addresses, four in flight; the last group of a row starts VEC columns before the row's end and
+// drops the columns it shares with the group before.  4- and 8-byte elements, inner >= VEC.
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink>
+__global__ __launch_bounds__(256) void reduce_cols_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
+                                                          int64_t groups_per_row, int64_t ngroups) {
+    constexpr int VEC = 16 / sizeof(In);
+    typedef typename VecOf<In, VEC>::type V;
+    typedef typename Xf::Pos Pos;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= ngroups) return;
+    const int64_t o = i / groups_per_row, q = i - o * groups_per_row;
+    const int64_t nominal = q * VEC;
+    const int64_t col0 = nominal + VEC > g.inner ? g.inner - VEC : nominal;
+    const int dup = (int)(nominal - col0);
+    const In* p = A + o * g.inner * g.mid + col0;
+    Acc acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = Op::template identity<Acc>();
+    int64_t m = 0;
+    for (; m + 4 <= g.mid; m += 4) {
+        V v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = load_nt_elems<In, VEC>(p + (m + u) * g.inner);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[u][j], (Pos)(m + u)));
+    }
+    for (; m < g.mid; ++m) {
+        const V v = load_nt_elems<In, VEC>(p + m * g.inner);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) acc[j] = acc_step(op, acc[j], xf(v[j], (Pos)m));
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        if (j >= dup) sink(o * g.inner + col0 + j, acc[j]);
+}
+
 // ---- many short lines, contiguous or with a narrow inner extent: whole slabs through LDS -----------------------
 // (sum(A; dims=1) of a 32 x 1_000_000 array; sum(A; dims=2) of a 4 x 32 x 250_000 array.)  A slab is the inner x mid
 // block of one outer index, contiguous in memory.  A wave per line leaves most lanes idle or gives each wave too
@@ -741,7 +783,7 @@ __global__ __launch_bounds__(BLOCK) void reduce_generic_kernel(const In* __restr
 
 // ---- host side: pick a kernel and launch -------------------------------------------------------------
 struct ReducePlan {
-    enum Kind { SPLIT, WAVE_LINES, THREAD_LINES, SHORT_LINES, STRIDED, NARROW, GENERIC } kind;
+    enum Kind { SPLIT, WAVE_LINES, THREAD_LINES, SHORT_LINES, STRIDED, NARROW, GENERIC, COLS } kind;
     bool    vector;
     int     splits;      // SPLIT: workgroups per line; STRIDED, NARROW: slices of mid
     int64_t rows_per_split;   // NARROW
@@ -757,7 +799,7 @@ int tune_reduce_wave_max_bytes();          // rk_api.hip
 
 template <typename In, typename Acc>
 inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, size_t cap = WS_PARTIALS_BYTES, int grid_scale = 1,
-                              int short_lines_tile = 16384 / (int)sizeof(In)) {
+                              int short_lines_tile = 16384 / (int)sizeof(In), bool cols_ok = false) {
     ReducePlan p{};
     const int cus = device_info().cus;
     const int64_t target_blocks = (int64_t)cus * tune_reduce_blocks_per_cu() * grid_scale;
@@ -791,6 +833,7 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
             return p;
         }
     }
+    if (cols_ok && s.inner >= 64 && s.mid <= 16 && nlines >= 4096 && is_aligned(A, sizeof(In))) { p.kind = ReducePlan::COLS; return p; }
     if (s.inner >= 64) {
         p.kind = ReducePlan::STRIDED;
         // 4- and 8-byte elements: vectors at any element-aligned address, rows of any length >= a vector
@@ -817,7 +860,9 @@ inline ReducePlan plan_reduce(const void* A, const Shape3& s, bool single_run, s
         return p;
     }
     if (s.mid <= 16 && nlines >= 4096) { p.kind = ReducePlan::THREAD_LINES; return p; }
-    if (s.inner > 1 && s.mid >= 1024 && s.outer <= 65535 && s.outer <= (int64_t)WS_TICKET_COUNT) {
+    // (from 64 rows on: below 1024 rows and above the 16 KiB slabs of the LDS kernel the alternative is a wave per line
+    // that reads one element in `inner` -- sum(A; dims=2) of 33 x 1000 x 1000 Float32: 0.8 TB/s)
+    if (s.inner > 1 && s.mid >= 64 && s.outer <= 65535 && s.outer <= (int64_t)WS_TICKET_COUNT) {
         p.kind = ReducePlan::NARROW;
         const int64_t rows_per_pass = 256 / s.inner;
         // every extra workgroup costs a row of partials and a longer fold: two per compute unit measured best
@@ -869,7 +914,9 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
     // (2^26 Float32, x -> x + 1: 3.4 -> 5.2 TB/s with twice the workgroups; 9 tokens: 2.3 -> 2.6 TB/s with four times)
     int grid_scale = 1;
     if constexpr (XfIsBatch<Xf>::value) grid_scale = xf.n_tokens > 4 ? 4 : 2;
-    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap, grid_scale, ShortLinesTile<In, Acc, Xf>::ELEMS);
+    // reduce_cols_kernel: 4- and 8-byte elements, f applied per element (not a traced program)
+    constexpr bool COLS_OK = sizeof(In) >= 4 && !XfIsBatch<Xf>::value;
+    const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap, grid_scale, ShortLinesTile<In, Acc, Xf>::ELEMS, COLS_OK);
     Workspace w{};
     if (p.payload > cap) return RK_ERR_WORKSPACE;   // the planner never asks for more
     if (p.payload > 0 && !carve_workspace(ws, ws_bytes, 0, &w)) return RK_ERR_WORKSPACE;
@@ -892,6 +939,17 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
                 reduce_wave_kernel<In, Acc, Xf, Op, Sink, true, 256, UNROLL><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink);
             else
                 reduce_wave_kernel<In, Acc, Xf, Op, Sink, false, 256, UNROLL><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink);
+            break;
+        }
+        case ReducePlan::COLS: {
+            if constexpr (COLS_OK) {
+                constexpr int64_t VEC = 16 / (int64_t)sizeof(In);
+                const int64_t groups_per_row = (s.inner + VEC - 1) / VEC;
+                if (groups_per_row > INT64_MAX / (s.outer > 0 ? s.outer : 1)) return RK_ERR_TOO_LARGE;
+                const int64_t ngroups = groups_per_row * s.outer, blocks = (ngroups + 255) / 256;
+                if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+                reduce_cols_kernel<In, Acc, Xf, Op, Sink><<<(unsigned)blocks, 256, 0, stream>>>(A, g, xf, op, sink, groups_per_row, ngroups);
+            }
             break;
         }
         case ReducePlan::THREAD_LINES: {

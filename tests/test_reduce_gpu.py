@@ -537,3 +537,25 @@ def test_long_reduced_dim_behind_a_short_contiguous_one(rk, orc, shape):
                 np.testing.assert_allclose(g2, w2, rtol=1e-5, atol=1e-2)
             else:
                 assert np.array_equal(g2, w2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(200, 3, 50), (70, 16, 60), (1001, 5, 7), (65, 2, 100), (4099, 9, 2), (33, 200, 40), (7, 100, 300), (63, 70, 9)])
+def test_short_or_medium_reduced_dim_in_the_middle(rk, orc, shape):
+    """dims=2 of a 3-d array.  A reduced extent <= 16 behind >= 64 contiguous columns: a lane per group of four (two)
+    columns, 16-byte loads at element-aligned addresses, the last group of a row starting early (1001, 65, 4099 columns).
+    64 .. 1023 rows behind fewer than 64 columns, in slabs above 16 KiB: runs of whole rows, not a wave per line."""
+    rng = np.random.default_rng(sum(shape))
+    for dtype in (np.float32, np.int32, np.float64, np.int64):
+        x = (rng.standard_normal(shape) * 100).astype(dtype)
+        dx = rk.ROCArray(x)
+        got = rk.Array(rk.mapreduce("identity", "add_sum", dx, dims=2))
+        want = orc.mapreduce("identity", "add_sum", x, dims=2)
+        if np.dtype(dtype).kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == np.float32 else 1e-12, atol=1e-2 if dtype == np.float32 else 1e-9)
+        else:
+            assert got.dtype == want.dtype and np.array_equal(got, want)
+        assert np.array_equal(rk.Array(rk.mapreduce("abs", "max", dx, dims=2)), orc.mapreduce("abs", "max", x, dims=2))
+        gv, gi = rk.findmin(dx, dims=2)
+        ov, oi = orc.findmin(x, dims=2)
+        assert np.array_equal(rk.Array(gv), ov) and np.array_equal(np.moveaxis(rk.Array(gi), 0, -1), oi)
