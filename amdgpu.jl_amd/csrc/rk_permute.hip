@@ -102,16 +102,34 @@ __global__ __launch_bounds__(256) void permute_tiles_kernel(const T* __restrict_
 // ELEMS (4- and 8-byte elements): extents and addresses need not be whole vectors -- global memory takes 16-byte
 // accesses at any element-aligned address.  The last vector of a row starts V elements before the row's end instead of
 // running past it; where that reaches back into the tile in front, the elements of this tile go one by one.
+constexpr int PERM_XCDS = 8;
 template <typename T, int TE, bool ELEMS>
 __global__ __launch_bounds__(256) void permute_tiles_vec_kernel(const T* __restrict__ src, T* __restrict__ dst, PermGeom g, int64_t tiles0,
-                                                                int64_t tilesp) {
+                                                                int64_t tilesp, int by_xcd) {
     constexpr int V = 16 / sizeof(T), LR = TE / V, RP = 256 / LR;
     typedef typename VecOf<T, V>::type VT;
     __shared__ T tile[TE][TE + 1];
     const int c = threadIdx.x % LR, r = threadIdx.x / LR;
+    // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own.  A tile row of the destination is TE
+    // elements; unless the destination's rows are whole 128-byte lines, two tiles that are neighbours along p write
+    // parts of one line, and from different L2s those are two partial write-backs (5000 x 6001 Float32: 2.5 TB/s
+    // against 4.0 for 5000 x 6000).  So an XCD takes every eighth tile COLUMN t0 and all tp of it, in diagonal order
+    // (power-of-two pitches: consecutive tiles must not hit one channel), which keeps p-neighbours in one L2 and a
+    // few launches apart.  Where the destination's rows ARE whole lines the plain diagonal order is the faster one
+    // (8192 x 8192: 94 against 113 us), so the host asks for this only otherwise (by_xcd).
     int64_t b = blockIdx.x;
-    const int64_t t0 = b % tiles0; b /= tiles0;
-    const int64_t tp = (b % tilesp + t0) % tilesp; b /= tilesp;      // diagonal order
+    int64_t t0, tp;
+    if (by_xcd) {
+        const int64_t xcd = b % PERM_XCDS; b /= PERM_XCDS;
+        const int64_t n0x = (tiles0 + PERM_XCDS - 1) / PERM_XCDS;
+        const int64_t t0l = b % n0x; b /= n0x;
+        t0 = t0l * PERM_XCDS + xcd;
+        tp = (b % tilesp + t0l) % tilesp; b /= tilesp;               // diagonal order
+        if (t0 >= tiles0) return;                                    // tiles0 is no multiple of 8: whole workgroups
+    } else {
+        t0 = b % tiles0; b /= tiles0;
+        tp = (b % tilesp + t0) % tilesp; b /= tilesp;                // diagonal order
+    }
     int64_t sbase = 0, dbase = 0, sstride = 1, sstride_p = 0;
     for (int d = 0; d < g.nd; ++d) {
         if (d == g.p) sstride_p = sstride;
@@ -267,8 +285,10 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
             int64_t batch = 1;
             for (int d = 1; d < g.nd; ++d)
                 if (d != g.p) batch *= g.ext[d];
-            if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
-            permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+            const int by_xcd = (g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128);     // rows of dst are no whole lines
+            const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;   // tile columns, dealt to the XCDs
+            if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+            permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -279,8 +299,10 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
                 int64_t batch = 1;
                 for (int d = 1; d < g.nd; ++d)
                     if (d != g.p) batch *= g.ext[d];
-                if (tiles0 > 0x7fffffff / tilesp || tiles0 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
-                permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(tiles0 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp);
+                const int by_xcd = (g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128);
+                const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;
+                if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+                permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
                 RK_LAUNCH_CHECK();
                 return RK_SUCCESS;
             }

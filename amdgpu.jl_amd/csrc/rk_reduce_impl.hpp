@@ -90,6 +90,8 @@ template <typename In, typename Acc> struct ProgXform {
         return y;
     }
 };
+template <typename Xf> struct XfIsArg : std::false_type {};
+template <typename T, typename P, bool WANT_MAX> struct XfIsArg<ArgXform<T, P, WANT_MAX>> : std::true_type {};
 template <typename Xf> struct XfIsBatch : std::false_type {};
 template <typename In, typename Acc> struct XfIsBatch<ProgXform<In, Acc>> : std::true_type {};
 
@@ -914,8 +916,10 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
     // (2^26 Float32, x -> x + 1: 3.4 -> 5.2 TB/s with twice the workgroups; 9 tokens: 2.3 -> 2.6 TB/s with four times)
     int grid_scale = 1;
     if constexpr (XfIsBatch<Xf>::value) grid_scale = xf.n_tokens > 4 ? 4 : 2;
-    // reduce_cols_kernel: 4- and 8-byte elements, f applied per element (not a traced program)
-    constexpr bool COLS_OK = sizeof(In) >= 4 && !XfIsBatch<Xf>::value;
+    // reduce_cols_kernel: 4- and 8-byte elements, f applied per element (not a traced program); not findmax / findmin,
+    // whose outputs (a value and ndims indices each, more bytes than the input when the reduced extent is 3) want a lane
+    // per output: 200 x 3 x 50000 Float32 dims=2 1.0 TB/s of input from the strided kernel, 0.43 from this one
+    constexpr bool COLS_OK = sizeof(In) >= 4 && !XfIsBatch<Xf>::value && !XfIsArg<Xf>::value;
     const ReducePlan p = plan_reduce<In, Acc>(A, s, s.single_run, cap, grid_scale, ShortLinesTile<In, Acc, Xf>::ELEMS, COLS_OK);
     Workspace w{};
     if (p.payload > cap) return RK_ERR_WORKSPACE;   // the planner never asks for more
