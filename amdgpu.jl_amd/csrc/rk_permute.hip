@@ -285,7 +285,9 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
             int64_t batch = 1;
             for (int d = 1; d < g.nd; ++d)
                 if (d != g.p) batch *= g.ext[d];
-            const int by_xcd = (g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128);     // rows of dst are no whole lines
+            // rows of dst are no whole lines, and dealing tile columns to 8 XCDs leaves at most an eighth of the workgroups empty
+            const int by_xcd = ((g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128)) &&
+                               (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS * 7 <= tiles0 * 8;
             const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;   // tile columns, dealt to the XCDs
             if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
             permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
@@ -299,7 +301,8 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
                 int64_t batch = 1;
                 for (int d = 1; d < g.nd; ++d)
                     if (d != g.p) batch *= g.ext[d];
-                const int by_xcd = (g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128);
+                const int by_xcd = ((g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128)) &&
+                                   (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS * 7 <= tiles0 * 8;
                 const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;
                 if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
                 permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);

@@ -1111,6 +1111,45 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
     }
 }
 
+// ---- a short scanned dim behind a long contiguous one: a lane per group of columns ------------------------------
+// (cumsum(A; dims=2) of a 50000 x 3 x 200 array: the strided kernel gives every workgroup three rows of a strip.)
+// A lane owns VEC adjacent columns of one outer index and walks the <= 16 rows, loads four rows ahead; 16-byte accesses
+// at element-aligned addresses, the last group of a row starting VEC columns before the row's end (it stores what the
+// group before stores, the same values).  4- and 8-byte elements.
+template <typename In, typename T, typename Op>
+__global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init, int inclusive,
+                                                        Op op, int64_t groups_per_row, int64_t ngroups) {
+    constexpr int VEC = 16 / sizeof(T);
+    typedef typename VecOf<In, VEC>::type VI;
+    typedef typename VecOf<T, VEC>::type VT;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= ngroups) return;
+    const int64_t o = i / groups_per_row, q = i - o * groups_per_row;
+    const int64_t col0 = q * VEC + VEC > g.inner ? g.inner - VEC : q * VEC;
+    const int64_t base = o * g.inner * g.mid + col0;
+    T run[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) run[j] = init;
+    for (int64_t m0 = 0; m0 < g.mid; m0 += 4) {
+        VI x[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) x[u] = ElemVectors<In, T>::template load<VEC>(in + base + (m0 + u < g.mid ? m0 + u : g.mid - 1) * g.inner);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (m0 + u < g.mid) {
+                VT o4;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) {
+                    const T nxt = op(run[j], (T)x[u][j]);
+                    o4[j] = inclusive ? nxt : run[j];
+                    run[j] = nxt;
+                }
+                ElemVectors<T, T>::template store<VEC>(out + base + (m0 + u) * g.inner, o4);
+            }
+        }
+    }
+}
+
 // ---- inner >= 64, few strips: tiles of rows in launch order, single pass --------------------------------------------
 // scan_strided_kernel needs one workgroup per strip of 64 * VEC columns; a 4096 x 16384 matrix scanned along its rows
 // has 16 strips.  Cutting the rows into slices makes the slices depend on each other.  The three-pass answer (column
@@ -1394,8 +1433,12 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
                                 size_t scratch_bytes, hipStream_t stream, const Workspace* ws = nullptr) {
     constexpr int VEC = 16 / sizeof(T);
     // 4- and 8-byte elements: vectors at any element-aligned address, rows of any length (>= 64 here)
-    const bool vec = (sizeof(In) >= 4 && sizeof(T) >= 4) ? (is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) && g.inner >= VEC)
-                                                         : (aligned && g.inner % VEC == 0);
+    // (in place, a row's last vector would re-read columns that the lane before -- possibly of another workgroup -- has
+    // already overwritten with results: whole-vector rows only)
+    const bool in_place = (const void*)in == (const void*)out;
+    const bool vec = (sizeof(In) >= 4 && sizeof(T) >= 4 && !(in_place && g.inner % VEC != 0))
+                         ? (is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) && g.inner >= VEC)
+                         : (aligned && g.inner % VEC == 0);
     const int cols = WAVE * (vec ? VEC : 1);
     const int64_t strips = (g.inner + cols - 1) / cols;
     if (strips * g.outer > 0x7fffffff) return RK_ERR_TOO_LARGE;
@@ -1562,6 +1605,19 @@ inline int32_t launch_scan(const ScanArgs& a) {
                 RK_LAUNCH_CHECK();
                 return RK_SUCCESS;
             }
+        }
+    }
+    if constexpr (ElemVectors<In, T>::value) {
+        // (not in place with rows that are no whole vectors: the row's last group re-reads columns of the group before)
+        if (s.inner >= 64 && s.mid <= 16 && s.inner * s.outer >= 4096 && is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) &&
+            !((const void*)in == (const void*)out && s.inner % VEC != 0)) {
+            const int64_t groups_per_row = (s.inner + VEC - 1) / VEC;
+            if (groups_per_row > INT64_MAX / s.outer) return RK_ERR_TOO_LARGE;
+            const int64_t ngroups = groups_per_row * s.outer, blocks = (ngroups + 255) / 256;
+            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            scan_cols_kernel<In, T, Op><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, groups_per_row, ngroups);
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
         }
     }
     if (s.inner >= 64) {

@@ -356,12 +356,14 @@ def test_lines_that_start_at_odd_addresses(rk, orc, m):
     np.testing.assert_allclose(rk.Array(rk.cumsum(v)), np.cumsum(flat[3:m + 3].astype(np.float64)), rtol=1e-4, atol=1e-3)
 
 
-@pytest.mark.parametrize("shape", [(257, 300), (1001, 1000), (4097, 130), (65, 5000), (130, 70, 5), (67, 40, 9), (8191, 33)])
+@pytest.mark.parametrize("shape", [(257, 300), (1001, 1000), (4097, 130), (65, 5000), (130, 70, 5), (67, 40, 9), (8191, 33),
+                                   (200, 3, 50), (1001, 5, 7), (4099, 16, 2), (256, 2, 40)])
 def test_scans_across_rows_that_are_no_whole_vectors(rk, orc, shape):
     """cumsum(A; dims=2) with a first extent that is no multiple of the 16-byte vector: every row has another alignment.
     The kernels read and write vectors at element-aligned addresses; the last vector of a row starts four (two)
-    elements before the row's end.  All three paths: one workgroup per strip, sliced with carried totals, and the
-    single pass over tiles of rows.  In place too."""
+    elements before the row's end.  All paths: one workgroup per strip, sliced with carried totals, the single pass
+    over tiles of rows, and (a scanned extent <= 16) a lane per group of columns.  In place too: there a row's last
+    vector would re-read columns another lane has already overwritten, so odd rows take the element-wise kernels."""
     rng = np.random.default_rng(sum(shape))
     for dtype in (np.float32, np.int32, np.float64, np.int64):
         x = (rng.standard_normal(shape) * 10).astype(dtype)
