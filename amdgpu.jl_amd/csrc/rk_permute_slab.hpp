@@ -25,7 +25,7 @@ namespace rk {
 
 constexpr int PERM_SLAB_MAX_DIMS = 8;
 constexpr int PERM_SLAB_THREADS = 256;
-constexpr int PERM_SLAB_SHORT = 32;        // a leading extent below this counts as short
+constexpr int PERM_SLAB_SHORT = 64;        // a leading extent below this counts as short
 constexpr int PERM_SLAB_LONG_CHUNK = 64;   // elements of a long leading dim in a box ...
 constexpr int PERM_SLAB_LONG_MAX = 256;    // ... and when the third dim is used up and the budget is not
 
