@@ -6,7 +6,7 @@
 //   * if the leading dims of the source (up to the one that becomes the destination's first) or of the destination
 //     (up to the source's first) hold at most 8 elements -- (N, 3) <-> (3, N), (2, 3, N) <-> (N, 3, 2), batches of
 //     tiny matrices -- a lane moves one such run (rk_permute_small.hpp);
-//   * if the source's or the destination's first dim is short (< 32) and a third dim can lengthen the runs --
+//   * if the source's or the destination's first dim is short (< 64) and a third dim can lengthen the runs --
 //     (2, N, 2) with perm (3, 2, 1), (4, 32, N) -> (N, 32, 4) -- a workgroup moves a box of three dims through LDS
 //     (rk_permute_slab.hpp);
 //   * otherwise 64 x 64 tiles over (src dim 1, the src dim that becomes dst dim 1) go through LDS, so that loads
