@@ -89,3 +89,14 @@ def test_short_first_dims_with_a_third_dim(rk, orc, dtype, shape, perm):
     """The source's or the destination's first dim is short and neither side is a run of at most 8 elements: boxes of
     three dims through LDS ((2, N, 2) with perm (3, 2, 1): a tile per 4 elements otherwise)."""
     _check(rk, orc, _rand(np.random.default_rng(73), dtype, shape), perm)
+
+
+@pytest.mark.parametrize("shape,perm,dtype", [((100, 100, 300), (2, 1, 3), np.float32), ((101, 99, 257), (2, 1, 3), np.int32),
+                                              ((70, 80, 256), (2, 1, 3), np.float64), ((96, 72, 4, 70), (2, 1, 3, 4), np.float32),
+                                              ((65, 110, 260), (2, 1, 3), np.uint32), ((77, 79, 300), (2, 1, 3), np.int64),
+                                              ((5001, 601), (2, 1), np.float32), ((4097, 130), (2, 1), np.float64)])
+def test_batches_of_small_matrices_and_odd_extents(rk, orc, shape, perm, dtype):
+    """permutedims(A, (2, 1, 3)) of >= 256 matrices that 64 x 64 tiles would fill poorly: whole matrices through LDS
+    (100 x 100 x 3000 Float32: 2.5 -> 5.5 TB/s).  The last two: a plain transpose whose extents are no whole vectors
+    (the vector tiles with element-aligned accesses, tile columns dealt to the XCDs)."""
+    _check(rk, orc, _rand(np.random.default_rng(5), dtype, shape), perm)
