@@ -112,20 +112,20 @@ __global__ __launch_bounds__(256) void permute_tiles_vec_kernel(const T* __restr
     const int c = threadIdx.x % LR, r = threadIdx.x / LR;
     // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own.  A tile row of the destination is TE
     // elements; unless the destination's rows are whole 128-byte lines, two tiles that are neighbours along p write
-    // parts of one line, and from different L2s those are two partial write-backs (5000 x 6001 Float32: 2.5 TB/s
-    // against 4.0 for 5000 x 6000).  So an XCD takes every eighth tile COLUMN t0 and all tp of it, in diagonal order
-    // (power-of-two pitches: consecutive tiles must not hit one channel), which keeps p-neighbours in one L2 and a
-    // few launches apart.  Where the destination's rows ARE whole lines the plain diagonal order is the faster one
-    // (8192 x 8192: 94 against 113 us), so the host asks for this only otherwise (by_xcd).
+    // parts of one line, and from different L2s -- or from one, long apart -- those are two partial write-backs
+    // (5000 x 6001 Float32: 2.5 TB/s against 4.0 for 5000 x 6000).  by_xcd: every XCD takes a contiguous eighth of the
+    // tile rows tp and walks it along p first, so neighbours along p follow each other in one L2: 5000 x 6001 95 -> 65 us,
+    // and whole-line rows gain too (8000 x 8000 102 -> 92, 5000 x 6000 60 -> 48).  Dealing tile COLUMNS to the XCDs
+    // (p-neighbours ten launches apart) gave 79 us, bands walked along dim 0 first 90.  Pitches that are multiples of
+    // 4 KiB keep the plain diagonal order (consecutive tiles must not hit one channel; 8192 x 8192: 94 us, bands 98).
     int64_t b = blockIdx.x;
     int64_t t0, tp;
     if (by_xcd) {
         const int64_t xcd = b % PERM_XCDS; b /= PERM_XCDS;
-        const int64_t n0x = (tiles0 + PERM_XCDS - 1) / PERM_XCDS;
-        const int64_t t0l = b % n0x; b /= n0x;
-        t0 = t0l * PERM_XCDS + xcd;
-        tp = (b % tilesp + t0l) % tilesp; b /= tilesp;               // diagonal order
-        if (t0 >= tiles0) return;                                    // tiles0 is no multiple of 8: whole workgroups
+        const int64_t rows = (tilesp + PERM_XCDS - 1) / PERM_XCDS;   // tile rows per XCD
+        tp = xcd * rows + b % rows; b /= rows;                       // along p first: the neighbours follow each other
+        t0 = b % tiles0; b /= tiles0;
+        if (tp >= tilesp) return;                                    // the last band is short: whole workgroups
     } else {
         t0 = b % tiles0; b /= tiles0;
         tp = (b % tilesp + t0) % tilesp; b /= tilesp;                // diagonal order
@@ -354,12 +354,12 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
             int64_t batch = 1;
             for (int d = 1; d < g.nd; ++d)
                 if (d != g.p) batch *= g.ext[d];
-            // rows of dst are no whole lines, and dealing tile columns to 8 XCDs leaves at most an eighth of the workgroups empty
-            const int by_xcd = ((g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128)) &&
-                               (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS * 7 <= tiles0 * 8;
-            const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;   // tile columns, dealt to the XCDs
-            if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
-            permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
+            // bands of tile rows for the 8 XCDs (see the kernel) unless the pitch asks for the diagonal order or too many workgroups would be empty
+            const int64_t rows8 = (tilesp + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS;
+            const int by_xcd = (g.dstride[0] * (int64_t)E) % 4096 != 0 && rows8 * 7 <= tilesp * 8;
+            const int64_t nrows = by_xcd ? rows8 : tilesp;
+            if (tiles0 > 0x7fffffff / nrows || tiles0 * nrows > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+            permute_tiles_vec_kernel<T, TE, false><<<(unsigned)(tiles0 * nrows * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -370,11 +370,11 @@ static int32_t permute_elsize(const void* src, void* dst, PermGeom g, hipStream_
                 int64_t batch = 1;
                 for (int d = 1; d < g.nd; ++d)
                     if (d != g.p) batch *= g.ext[d];
-                const int by_xcd = ((g.dstride[0] * (int64_t)E) % 128 != 0 || !is_aligned(dst, 128)) &&
-                                   (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS * 7 <= tiles0 * 8;
-                const int64_t cols8 = by_xcd ? (tiles0 + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS : tiles0;
-                if (cols8 > 0x7fffffff / tilesp || cols8 * tilesp > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
-                permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(cols8 * tilesp * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
+                const int64_t rows8 = (tilesp + PERM_XCDS - 1) / PERM_XCDS * PERM_XCDS;
+                const int by_xcd = (g.dstride[0] * (int64_t)E) % 4096 != 0 && rows8 * 7 <= tilesp * 8;
+                const int64_t nrows = by_xcd ? rows8 : tilesp;
+                if (tiles0 > 0x7fffffff / nrows || tiles0 * nrows > 0x7fffffff / batch) return RK_ERR_TOO_LARGE;
+                permute_tiles_vec_kernel<T, TE, true><<<(unsigned)(tiles0 * nrows * batch), 256, 0, stream>>>((const T*)src, (T*)dst, g, tiles0, tilesp, by_xcd);
                 RK_LAUNCH_CHECK();
                 return RK_SUCCESS;
             }
