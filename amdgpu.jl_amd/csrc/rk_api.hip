@@ -88,6 +88,13 @@ int tune_scan_rows_ordered() {
     return v;
 }
 
+// 0: scans along the second dim of arrays whose first dim is at most half a strip of columns take the two-pass tiles
+// (scan_narrow_kernel) or the strips instead of the single pass with several rows per load (RK_SCAN_ROWS_PACKED).
+int tune_scan_rows_packed() {
+    static const int v = env_int("RK_SCAN_ROWS_PACKED", 1, 0, 1);
+    return v;
+}
+
 // Workgroups per compute unit the scan across rows aims for when it cuts the rows into slices
 // (RK_SCAN_SLICE_BLOCKS_PER_CU).
 int tune_scan_slice_blocks_per_cu() {
@@ -212,6 +219,8 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
         const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 8;           // ScanTile<T>::TILE
         const int64_t tpl = (s.mid + tile - 1) / tile, gpl = (tpl + WAVE - 1) / WAVE;
         // one tagged word per 4 bytes of the value per tile, one 128-byte line per group of 64 tiles
+        // scans across rows publish 1 KiB of column totals per tile in the partials area: one flag each
+        if (s.inner > 1) need += WS_PARTIALS_BYTES / 1024 * sizeof(uint64_t);
         if (s.inner == 1 && tpl > 1) need += ((size_t)(tpl * s.outer) * (esz / 4) + (size_t)(gpl * s.outer) * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     }
     if (kind == RK_KIND_FINDALL && valid_shape(ndim, shape, &total) && total > 0) need += findall_workspace_need(total);

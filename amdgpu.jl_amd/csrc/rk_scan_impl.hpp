@@ -10,6 +10,9 @@
 //       scan_wave_lines_kernel lines shorter than a tile: one wave per line with a running carry
 //   inner  > 1 : strided lines, lanes run along the contiguous `inner` axis
 //       scan_strided_kernel    4 waves x register tiles of rows, column totals through LDS
+//       scan_rows_ordered_kernel  few strips of columns, many rows: tiles of rows in launch order, single pass
+//       scan_rows_packed_kernel   rows of 128 bytes up to half a strip: several rows per load instruction, single pass
+//       scan_cols_kernel       a scanned extent <= 16 behind >= 64 contiguous columns: a lane per group of columns
 //       scan_narrow_kernel     1 < inner < 64 with long lines: tiles of whole rows through LDS
 //   scan_thread_kernel         one lane per line (tiny lines)
 //   scan_lds_lines_kernel      short lines of any length (contiguous, or short along a narrow inner): whole slabs through LDS
@@ -1170,6 +1173,183 @@ __global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ i
 //   payload   [ntiles + 2 * groups][64 * VEC] values in the partials area: totals; group aggregates; group prefixes
 constexpr int ROWS_GROUP = 8;      // tiles of a chain per group of the two-level look-back
 
+// The look-back of one tile (run by one wave): from the tile's column totals `tot` to `base`, the prefix of everything in
+// front of the tile on its chain, `init` included.  Lane l holds the columns l * VEC .. l * VEC + VEC - 1.
+// PACKED: only the first P * VEC columns are in use (P a power of two): the leader reads the aggregates of 64 / P groups
+// with one load instruction, P lanes each, and folds them across the lanes, older ones on the left.  (All tiles of a
+// long chain look back at the same time, so a leader walks every group in flight on the chain: 128 of them with
+// 1024 tiles of one chain in flight, 32 round trips at four aggregates each.)
+template <typename T, typename Op, int VEC, bool PACKED = false>
+__device__ __forceinline__ void rows_lookback(const T (&tot)[VEC], T (&base)[VEC], T init, Op op, uint32_t epoch, int64_t tile, int64_t slice,
+                                              int64_t chain, int64_t nchains, int64_t nslices, int64_t ntiles, T* payload, uint64_t* desc,
+                                              const WaitCtl& wc, int lane, int P = WAVE) {
+    constexpr int COLS = WAVE * VEC;
+    typedef typename VecOf<T, VEC>::type VT;
+    const T ident = Op::template identity<T>();
+    const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
+    const int64_t ngroups_chain = (nslices + ROWS_GROUP - 1) / ROWS_GROUP;
+    uint64_t* gflag = desc + ntiles;                                    // [group * nchains + chain]
+    T* gpayA = payload + ntiles * COLS;                                  // aggregates of whole groups
+    T* gpayP = gpayA + ngroups_chain * nchains * COLS;                   // inclusive prefixes through a group
+    const int r = (int)(slice % ROWS_GROUP);                             // predecessors inside the group
+    const int64_t grp = slice / ROWS_GROUP;                              // groups in front of this one in the chain
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) base[j] = init;
+    const bool has_reader = slice + 1 < nslices;     // the last slice of a chain has none
+    if (has_reader && r < ROWS_GROUP - 1) {          // the group's last tile publishes the group aggregate instead
+        VT t;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) t[j] = tot[j];
+        store_agent((VT*)(payload + tile * COLS + lane * VEC), t);
+        publish_barrier();                           // the totals are at the coherent level before the flag
+        if (lane == 0) __hip_atomic_store(&desc[tile], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    long long rounds = 0;
+    if (r == 0) {
+        if (grp > 0) {
+            // leader: aggregates of the groups in front, back to the nearest published prefix; publishes the
+            // prefix through the previous group for the other tiles of its own
+            T acc[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] = ident;
+            int64_t first = grp - 1, rem = grp;
+            for (;;) {
+                uint32_t st = DESC_P;                // lanes beyond the first group: terminators
+                if (lane < rem) {
+                    const uint32_t tag = (uint32_t)(__hip_atomic_load(&gflag[(first - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+                    st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
+                }
+                const uint64_t ballotP = __ballot(st == DESC_P);
+                const uint64_t ballotX = __ballot(st == 0u);
+                const int np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
+                const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
+                if ((ballotX & needed) == 0ull) {
+                    const int cnt = np >= 0 ? np : WAVE;
+                    if constexpr (PACKED) {
+                        constexpr int U = 4;
+                        const int k = lane / P, pl = lane - k * P;          // lane pl of the k-th aggregate of a load
+                        for (int d0 = 0; d0 < cnt; d0 += (WAVE / P) * U) {
+                            VT x[U];
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {                   // distances d0 + k * U + u: a lane's are consecutive
+                                const int d = d0 + k * U + u;
+                                x[u] = load_agent((const VT*)(gpayA + ((first - (d < cnt ? d : 0)) * nchains + chain) * COLS + pl * VEC));
+                            }
+                            T part[VEC];
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) part[j] = ident;
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {
+                                if (d0 + k * U + u < cnt) {
+#pragma unroll
+                                    for (int j = 0; j < VEC; ++j) part[j] = op(x[u][j], part[j]);
+                                }
+                            }
+                            for (int delta = P; delta < WAVE; delta <<= 1) {    // lanes further up hold older aggregates
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j) part[j] = op(__shfl_down(part[j], delta, WAVE), part[j]);
+                            }
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) acc[j] = op(part[j], acc[j]);     // complete in the lanes below P
+                        }
+                    } else
+                    for (int d0 = 0; d0 < cnt; d0 += 4) {               // four aggregates a round trip
+                        VT x[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            if (d0 + u < cnt) x[u] = load_agent((const VT*)(gpayA + ((first - d0 - u) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            if (d0 + u < cnt) {
+#pragma unroll
+                                for (int j = 0; j < VEC; ++j) acc[j] = op(x[u][j], acc[j]);
+                            }
+                        }
+                    }
+                    if (np >= 0) {
+                        if (np >= rem) {                                // ran off the first group: nothing but init in front
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) base[j] = op(init, acc[j]);
+                        } else {
+                            const VT x = load_agent((const VT*)(gpayP + ((first - np) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+                            for (int j = 0; j < VEC; ++j) base[j] = op(x[j], acc[j]);   // a published prefix contains init
+                        }
+                        break;
+                    }
+                    first -= WAVE;
+                    rem -= WAVE;
+                    continue;
+                }
+                if (wait_give_up(wc, rounds)) break; // `base` is then meaningless
+            }
+            VT t;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) t[j] = base[j];
+            store_agent((VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC), t);
+            publish_barrier();
+            if (lane == 0) __hip_atomic_store(&gflag[(grp - 1) * nchains + chain], (uint64_t)tagP << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    } else {
+        // totals of the predecessors inside the group, and the group's base from its leader.  A tile that is not
+        // the last of its group needs both before it can go on, so it polls the flags of both together and then has
+        // all payloads in flight at once: two round trips instead of four.  The last tile of a group first owes
+        // its successors the group aggregate, which needs the predecessors only.
+        T local[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) local[j] = ident;
+        const bool owes_group = r == ROWS_GROUP - 1 && has_reader;
+        const bool with_base = grp > 0 && !owes_group;          // lane 63 polls the leader's flag in the same rounds
+        for (;;) {
+            uint32_t ok = 1;
+            if (lane < r) {
+                const uint32_t tag = (uint32_t)(__hip_atomic_load(&desc[(slice - 1 - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+                ok = tag == tagA ? 1u : 0u;
+            } else if (with_base && lane == WAVE - 1) {
+                ok = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
+            }
+            if (__ballot(ok == 0u) == 0ull) break;
+            if (wait_give_up(wc, rounds)) break;
+        }
+        VT gbase;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) gbase[j] = init;
+        {
+            VT x[ROWS_GROUP - 1];
+#pragma unroll
+            for (int d = 0; d < ROWS_GROUP - 1; ++d)
+                if (d < r) x[d] = load_agent((const VT*)(payload + ((slice - 1 - d) * nchains + chain) * COLS + lane * VEC));
+            if (with_base) gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
+#pragma unroll
+            for (int d = 0; d < ROWS_GROUP - 1; ++d) {
+                if (d < r) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) local[j] = op(x[d][j], local[j]);
+                }
+            }
+        }
+        if (owes_group) {                            // aggregate of the whole group, as soon as it is known
+            VT t;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) t[j] = op(local[j], tot[j]);
+            store_agent((VT*)(gpayA + (grp * nchains + chain) * COLS + lane * VEC), t);
+            publish_barrier();
+            if (lane == 0) __hip_atomic_store(&gflag[grp * nchains + chain], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (grp > 0) {                           // then the group's base, from its leader
+                for (;;) {
+                    uint32_t st = 0;
+                    if (lane == 0) st = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
+                    if (__builtin_amdgcn_readfirstlane((int)st) != 0) break;
+                    if (wait_give_up(wc, rounds)) break;
+                }
+                gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) base[j] = op(gbase[j], local[j]);      // a published prefix contains init
+    }
+}
+
 // NW waves hold rows; one more wave holds none and does the publishing and the look-back.  The registers a kernel
 // needs are the maximum over its branches, so the row data (32 registers) and the look-back's working set no longer
 // add up: 64 registers suffice and two workgroups share a compute unit (with wave 0 doing both, 25 registers spilled).
@@ -1193,13 +1373,6 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
     uint32_t epoch = 0;
     if (wave == NW) {
         epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
-        const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
-        const int64_t ngroups_chain = (nslices + ROWS_GROUP - 1) / ROWS_GROUP;
-        uint64_t* gflag = desc + ntiles;                                    // [group * nchains + chain]
-        T* gpayA = payload + ntiles * COLS;                                  // aggregates of whole groups
-        T* gpayP = gpayA + ngroups_chain * nchains * COLS;                   // inclusive prefixes through a group
-        const int r = (int)(slice % ROWS_GROUP);                             // predecessors inside the group
-        const int64_t grp = slice / ROWS_GROUP;                              // groups in front of this one in the chain
         __syncthreads();                                 // the row waves have written their column totals
         T tot[VEC], base[VEC];
 #pragma unroll
@@ -1207,133 +1380,8 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
             tot[j] = ident;
 #pragma unroll
             for (int w = 0; w < NW; ++w) tot[j] = op(tot[j], lds[w][lane * VEC + j]);
-            base[j] = init;
         }
-        const bool has_reader = slice + 1 < nslices;     // the last slice of a chain has none
-        if (has_reader && r < ROWS_GROUP - 1) {          // the group's last tile publishes the group aggregate instead
-            VT t;
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) t[j] = tot[j];
-            store_agent((VT*)(payload + tile * COLS + lane * VEC), t);
-            publish_barrier();                           // the totals are at the coherent level before the flag
-            if (lane == 0) __hip_atomic_store(&desc[tile], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        long long rounds = 0;
-        if (r == 0) {
-            if (grp > 0) {
-                // leader: aggregates of the groups in front, back to the nearest published prefix; publishes the
-                // prefix through the previous group for the other tiles of its own
-                T acc[VEC];
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = ident;
-                int64_t first = grp - 1, rem = grp;
-                for (;;) {
-                    uint32_t st = DESC_P;                // lanes beyond the first group: terminators
-                    if (lane < rem) {
-                        const uint32_t tag = (uint32_t)(__hip_atomic_load(&gflag[(first - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
-                        st = tag == tagA ? DESC_A : (tag == tagP ? DESC_P : 0u);
-                    }
-                    const uint64_t ballotP = __ballot(st == DESC_P);
-                    const uint64_t ballotX = __ballot(st == 0u);
-                    const int np = ballotP ? (__ffsll((unsigned long long)ballotP) - 1) : -1;
-                    const uint64_t needed = np >= 0 ? ((1ull << np) - 1ull) : ~0ull;
-                    if ((ballotX & needed) == 0ull) {
-                        const int cnt = np >= 0 ? np : WAVE;
-                        for (int d0 = 0; d0 < cnt; d0 += 4) {               // four aggregates a round trip
-                            VT x[4];
-#pragma unroll
-                            for (int u = 0; u < 4; ++u)
-                                if (d0 + u < cnt) x[u] = load_agent((const VT*)(gpayA + ((first - d0 - u) * nchains + chain) * COLS + lane * VEC));
-#pragma unroll
-                            for (int u = 0; u < 4; ++u) {
-                                if (d0 + u < cnt) {
-#pragma unroll
-                                    for (int j = 0; j < VEC; ++j) acc[j] = op(x[u][j], acc[j]);
-                                }
-                            }
-                        }
-                        if (np >= 0) {
-                            if (np >= rem) {                                // ran off the first group: nothing but init in front
-#pragma unroll
-                                for (int j = 0; j < VEC; ++j) base[j] = op(init, acc[j]);
-                            } else {
-                                const VT x = load_agent((const VT*)(gpayP + ((first - np) * nchains + chain) * COLS + lane * VEC));
-#pragma unroll
-                                for (int j = 0; j < VEC; ++j) base[j] = op(x[j], acc[j]);   // a published prefix contains init
-                            }
-                            break;
-                        }
-                        first -= WAVE;
-                        rem -= WAVE;
-                        continue;
-                    }
-                    if (wait_give_up(wc, rounds)) break; // `base` is then meaningless
-                }
-                VT t;
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) t[j] = base[j];
-                store_agent((VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC), t);
-                publish_barrier();
-                if (lane == 0) __hip_atomic_store(&gflag[(grp - 1) * nchains + chain], (uint64_t)tagP << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        } else {
-            // totals of the predecessors inside the group, and the group's base from its leader.  A tile that is not
-            // the last of its group needs both before it can go on, so it polls the flags of both together and then has
-            // all payloads in flight at once: two round trips instead of four.  The last tile of a group first owes
-            // its successors the group aggregate, which needs the predecessors only.
-            T local[VEC];
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) local[j] = ident;
-            const bool owes_group = r == ROWS_GROUP - 1 && has_reader;
-            const bool with_base = grp > 0 && !owes_group;          // lane 63 polls the leader's flag in the same rounds
-            for (;;) {
-                uint32_t ok = 1;
-                if (lane < r) {
-                    const uint32_t tag = (uint32_t)(__hip_atomic_load(&desc[(slice - 1 - lane) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
-                    ok = tag == tagA ? 1u : 0u;
-                } else if (with_base && lane == WAVE - 1) {
-                    ok = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
-                }
-                if (__ballot(ok == 0u) == 0ull) break;
-                if (wait_give_up(wc, rounds)) break;
-            }
-            VT gbase;
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) gbase[j] = init;
-            {
-                VT x[ROWS_GROUP - 1];
-#pragma unroll
-                for (int d = 0; d < ROWS_GROUP - 1; ++d)
-                    if (d < r) x[d] = load_agent((const VT*)(payload + ((slice - 1 - d) * nchains + chain) * COLS + lane * VEC));
-                if (with_base) gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
-#pragma unroll
-                for (int d = 0; d < ROWS_GROUP - 1; ++d) {
-                    if (d < r) {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) local[j] = op(x[d][j], local[j]);
-                    }
-                }
-            }
-            if (owes_group) {                            // aggregate of the whole group, as soon as it is known
-                VT t;
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) t[j] = op(local[j], tot[j]);
-                store_agent((VT*)(gpayA + (grp * nchains + chain) * COLS + lane * VEC), t);
-                publish_barrier();
-                if (lane == 0) __hip_atomic_store(&gflag[grp * nchains + chain], (uint64_t)tagA << 32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (grp > 0) {                           // then the group's base, from its leader
-                    for (;;) {
-                        uint32_t st = 0;
-                        if (lane == 0) st = (uint32_t)(__hip_atomic_load(&gflag[(grp - 1) * nchains + chain], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) == tagP ? 1u : 0u;
-                        if (__builtin_amdgcn_readfirstlane((int)st) != 0) break;
-                        if (wait_give_up(wc, rounds)) break;
-                    }
-                    gbase = load_agent((const VT*)(gpayP + ((grp - 1) * nchains + chain) * COLS + lane * VEC));
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) base[j] = op(gbase[j], local[j]);      // a published prefix contains init
-        }
+        rows_lookback<T, Op, VEC>(tot, base, init, op, epoch, tile, slice, chain, nchains, nslices, ntiles, payload, desc, wc, lane);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) lds_base[lane * VEC + j] = base[j];
         __syncthreads();
@@ -1399,6 +1447,130 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
     ordered_finish(lds_epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
 }
 
+// ---- VEC <= inner <= 32 * VEC, long lines: several rows per load instruction, single pass ----------------------------
+// scan_rows_ordered_kernel leaves lanes idle when a row is shorter than its 64 vectors (a row of 64 Float32: 16 of 64
+// lanes).  Here P = ceil(inner / VEC) lanes hold a row and a wave's load instruction takes Q = 64 / P consecutive rows --
+// a wave covers R * Q consecutive rows, contiguous memory.  Lane group q (lanes q * P .. q * P + P - 1) holds the R
+// consecutive rows q * R .. q * R + R - 1 in its registers, lane p of it their p-th vector (the last vector of a row
+// that is no whole number of vectors starts VEC elements before the row's end, as in scan_strided_kernel), and scans
+// them downwards; one scan of the groups' totals across the lanes (log2 Q steps) joins the groups.  (With the Q rows of a
+// load instruction consecutive instead, every register row needs such a scan across the lanes: 64 x 65536 x 16 Float32
+// 244 us, of which 100 us for the cross-lane moves.)  The rest is scan_rows_ordered_kernel with a tile of NW * R * Q rows
+// and one chain per outer index.  `in` may be `out`: the columns that two lanes hold twice belong to lanes of the same
+// load instruction, which is complete before the wave's first store.
+template <typename In, typename T, typename Op, int NW, int R>
+__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(const In* in, T* out, ScanGeom g, T init, int inclusive, Op op,
+                                                                              int P, int64_t nchains, int64_t nslices, T* payload,
+                                                                              unsigned long long* counter, uint32_t* tickets, int ticket_group,
+                                                                              uint64_t* desc, int64_t desc_capacity, WaitCtl wc) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int COLS = WAVE * VEC;
+    typedef typename VecOf<T, VEC>::type VT;
+    typedef typename VecOf<In, VEC>::type VI;
+    __shared__ T lds[NW][COLS];
+    __shared__ T lds_base[COLS];
+    const T ident = Op::template identity<T>();
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
+    const int64_t ntiles = gridDim.x;
+    const int64_t tile = blockIdx.x;
+    const int64_t slice = tile / nchains, chain = tile - slice * nchains;
+    uint32_t epoch = 0;
+    if (wave == NW) {
+        epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+        __syncthreads();                                 // the row waves have written their column totals
+        T tot[VEC], base[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) tot[j] = ident;
+#pragma unroll 5                                         // (all 15 rows in flight at once: 60 registers for 8-byte values)
+        for (int w = 0; w < NW; ++w) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) tot[j] = op(tot[j], lds[w][lane * VEC + j]);
+        }
+        int P2 = 1;                                      // the look-back folds aggregates over power-of-two lane groups
+        while (P2 < P) P2 <<= 1;
+        rows_lookback<T, Op, VEC, true>(tot, base, init, op, epoch, tile, slice, chain, nchains, nslices, ntiles, payload, desc, wc, lane, P2);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) lds_base[lane * VEC + j] = base[j];
+        __syncthreads();
+    } else {
+        const int Q = WAVE / P;
+        const int q = lane / P, p = lane - q * P;
+        const bool lane_live = q < Q;                     // 64 - P * Q lanes hold nothing
+        const int inner = (int)g.inner;
+        const int nominal = p * VEC;                      // < inner: P = ceil(inner / VEC)
+        const int col0 = nominal + VEC > inner ? inner - VEC : nominal;
+        // wave-uniform base + a 32-bit offset per lane: eight 64-bit addresses kept from the loads to the stores would not
+        // fit the 64 registers this kernel is compiled for
+        const int64_t wave_row0 = (slice * NW + __builtin_amdgcn_readfirstlane(wave)) * (int64_t)(R * Q);
+        const int64_t wave_e0 = chain * g.inner * g.mid + wave_row0 * g.inner;
+        const int64_t left = g.mid - wave_row0;
+        const int rows = left >= R * Q ? R * Q : (left > 0 ? (int)left : 0);      // rows of this wave inside the array
+        const int lrow0 = q * R;                          // first row of the lane group, inside the wave's rows
+        const unsigned off0 = (unsigned)(lrow0 * inner + col0);
+        VT v[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (lane_live && lrow0 + r < rows) {
+                const VI x = load_nt_elems<In, VEC>(in + wave_e0 + (off0 + (unsigned)(r * inner)));
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[r][j] = (T)x[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[r][j] = ident;
+            }
+        }
+#pragma unroll
+        for (int r = 1; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[r][j] = op(v[r - 1][j], v[r][j]);
+        T incl[VEC], excl[VEC];                           // the totals of the lane groups, scanned across the groups
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) incl[j] = v[R - 1][j];
+        for (int delta = P; delta < WAVE; delta <<= 1) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const T y = __shfl_up(incl[j], delta, WAVE);
+                if (lane >= delta) incl[j] = op(y, incl[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const T up = __shfl_up(incl[j], P, WAVE), all = __shfl(incl[j], (Q - 1) * P + p, WAVE);
+            excl[j] = q == 0 ? ident : up;
+            lds[wave][lane * VEC + j] = q == 0 ? all : ident;
+        }
+        __syncthreads();
+        T pre[VEC];                                       // the rows of the tile above this wave's
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            pre[j] = ident;
+            for (int w = 0; w < wave; ++w) pre[j] = op(pre[j], lds[w][p * VEC + j]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) pre[j] = op(op(lds_base[p * VEC + j], pre[j]), excl[j]);
+        if (!inclusive) {                                 // every row takes the value of the row above it
+#pragma unroll
+            for (int r = R - 1; r > 0; --r) v[r] = v[r - 1];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[0][j] = ident;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (lane_live && lrow0 + r < rows) {
+                VT o4;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o4[j] = op(pre[j], v[r][j]);
+                store_nt_elems<T, VEC>(out + wave_e0 + (off0 + (unsigned)(r * inner)), o4);
+            }
+        }
+    }
+    __shared__ uint32_t lds_epoch;
+    if (wave == NW && lane == 0) lds_epoch = epoch;
+    __syncthreads();
+    ordered_finish(lds_epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
+}
+
 // ---- host side ---------------------------------------------------------------------------------------
 template <typename T, int K> struct ScanTile {     // geometry of the tile kernels: 256 threads x K x 16 bytes of output
     static constexpr int VEC = 16 / sizeof(T);
@@ -1411,6 +1583,7 @@ inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_
 int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
+int tune_scan_rows_packed();     // rk_api.hip: 0 = short rows never take the single-pass kernel with several rows per load
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
@@ -1444,9 +1617,10 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     if (strips * g.outer > 0x7fffffff) return RK_ERR_TOO_LARGE;
     const int64_t pitch = strips * cols;
     const int64_t cus = device_info().cus;
-    if constexpr (sizeof(T) <= 4) {
+    {
         // single pass over tiles of 120 rows (7 waves of rows: 134 us against 109 for the 4096 x 16384 matrix); the payloads
-        // of all tiles and groups must fit the partials area
+        // of all tiles and groups must fit the partials area.  8-byte values too: 2048 x 16384 Float64 103 us against 139
+        // for the three passes, 4096 x 4096 Int64 54 against 70.
         constexpr int NW = 15, R = 8;              // 15 waves of rows + 1 for the look-back
         const int64_t nchains = strips * g.outer, nslices = (g.mid + NW * R - 1) / (NW * R), ntiles = nchains * nslices;
         const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
@@ -1502,6 +1676,35 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
     else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
     RK_LAUNCH_CHECK();
+    return RK_SUCCESS;
+}
+
+// Scan along `mid` for VEC <= inner <= 32 * VEC in one pass (see scan_rows_packed_kernel).  *done stays false when the
+// shape or the workspace does not fit: the caller then takes another path.
+template <typename In, typename T, typename Op>
+inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, const Workspace& w, hipStream_t stream,
+                                bool* done) {
+    *done = false;
+    if constexpr (ElemVectors<In, T>::value) {
+        constexpr int VEC = 16 / (int)sizeof(T), COLS = WAVE * VEC;
+        constexpr int NW = 15, R = 8;
+        // (rows shorter than a 128-byte line: a load instruction then takes Q short pieces R rows apart, and the two-pass
+        // tiles through LDS are two to three times faster: 7 x 4_194_304 Float32 265 against 83 us)
+        if (g.inner * sizeof(In) < 128 || g.inner * 2 > COLS || !is_aligned(in, sizeof(In)) || !is_aligned(out, sizeof(T))) return RK_SUCCESS;
+        const int P = (int)((g.inner + VEC - 1) / VEC), Q = WAVE / P;
+        const int64_t tile_rows = (int64_t)NW * R * Q;
+        const int64_t nchains = g.outer, nslices = (g.mid + tile_rows - 1) / tile_rows;
+        if (nslices < 4 || nchains >= (int64_t)device_info().cus * 4 || nslices > 0x7fffffff / nchains) return RK_SUCCESS;
+        const int64_t ntiles = nchains * nslices;
+        const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
+        if ((size_t)((ntiles + 2 * ngroups) * COLS) * sizeof(T) > WS_PARTIALS_BYTES || (size_t)(ntiles + ngroups) * sizeof(uint64_t) > w.desc_bytes)
+            return RK_SUCCESS;
+        scan_rows_packed_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
+            in, out, g, init, inclusive, op, P, nchains, nslices, (T*)w.partials, (unsigned long long*)&w.hdr->scan_counter, w.tickets,
+            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr));
+        RK_LAUNCH_CHECK();
+        *done = true;
+    }
     return RK_SUCCESS;
 }
 
@@ -1625,6 +1828,11 @@ inline int32_t launch_scan(const ScanArgs& a) {
         char* scratch = nullptr;
         size_t scratch_bytes = 0;
         const bool have_ws = carve_workspace(a.ws, a.ws_bytes, 0, &w);
+        if (have_ws && tune_scan_rows_packed() != 0) {      // rows of at most half a strip of columns
+            bool done = false;
+            const int32_t st = scan_rows_packed<In, T, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
+            if (st != RK_SUCCESS || done) return st;
+        }
         if (have_ws) { scratch = (char*)w.partials; scratch_bytes = WS_PARTIALS_BYTES; }
         return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream, have_ws ? &w : nullptr);
     }
@@ -1635,6 +1843,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
         Workspace w{};
         if (carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
             bool done = false;
+            if (tune_scan_rows_packed() != 0) {
+                const int32_t st = scan_rows_packed<In, T, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
+                if (st != RK_SUCCESS || done) return st;
+            }
             const int32_t st = scan_narrow<In, T, Op>(in, out, g, init, inclusive, op, (char*)w.partials, WS_PARTIALS_BYTES, a.stream, &done);
             if (st != RK_SUCCESS || done) return st;
         }

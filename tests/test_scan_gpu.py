@@ -381,3 +381,30 @@ def test_scans_across_rows_that_are_no_whole_vectors(rk, orc, shape):
             np.testing.assert_allclose(rk.Array(dx), want, rtol=1e-4, atol=1e-2 if dtype == np.float32 else 1e-9)
         else:
             assert np.array_equal(rk.Array(dx), want.astype(dtype))
+
+
+@pytest.mark.parametrize("shape", [(100, 50_000), (65, 30_011), (128, 9_000), (95, 20_000, 2), (32, 100_001), (33, 40_000, 3), (16, 33_000, 5),
+                                   (64, 2_000, 3), (31, 70_000), (128, 4_001), (48, 1921), (17, 200_000)])
+def test_short_rows_several_to_a_load(rk, orc, shape):
+    """cumsum(A; dims=2) with rows of 128 bytes up to half a strip of columns (32 .. 128 Float32, 16 .. 64 Float64) and long
+    lines: a load instruction takes several rows, a group of lanes each, every group scans its consecutive rows in
+    registers and one scan across the lanes joins the groups; tiles of rows in launch order with a look-back over the
+    column totals.  Odd extents (rows at every alignment, last vector shifted back), several outer indices, partial
+    last tiles, and the neighbouring shapes that take the other kernels; in place too."""
+    rng = np.random.default_rng(sum(shape))
+    for dtype in (np.float32, np.int32, np.float64, np.int64):
+        x = (rng.standard_normal(shape) * 10).astype(dtype)
+        dx = rk.ROCArray(x)
+        for op, inclusive, init in (("add", True, None), ("min", True, None), ("add", False, dtype(3))):
+            got = rk.Array(rk.accumulate(op, dx, dims=2, init=init, inclusive=inclusive))
+            want = orc.accumulate(op, x, dims=2, init=init, inclusive=inclusive)
+            if np.dtype(dtype).kind == "f" and op == "add":
+                np.testing.assert_allclose(got, want, rtol=1e-4, atol=5e-2 if dtype == np.float32 else 1e-9)
+            else:
+                assert np.array_equal(got, want.astype(dtype)), (dtype, op)
+        rk.accumulate_("add", dx, dx, dims=2)
+        want = orc.accumulate("add", x, dims=2)
+        if np.dtype(dtype).kind == "f":
+            np.testing.assert_allclose(rk.Array(dx), want, rtol=1e-4, atol=5e-2 if dtype == np.float32 else 1e-9)
+        else:
+            assert np.array_equal(rk.Array(dx), want.astype(dtype))
