@@ -1157,7 +1157,7 @@ __global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ i
 // scan_strided_kernel needs one workgroup per strip of 64 * VEC columns; a 4096 x 16384 matrix scanned along its rows
 // has 16 strips.  Cutting the rows into slices makes the slices depend on each other.  The three-pass answer (column
 // totals per slice, scan of the totals, scan from the carried-in prefix) reads the input twice: 12 bytes per element.
-// Here a tile is NW * R = 120 rows of one strip and the dependency is resolved like in the single-pass scan of long lines,
+// Here a tile is NW * R = 150 rows of one strip and the dependency is resolved like in the single-pass scan of long lines,
 // with a VECTOR for payload and two levels: a tile publishes its 64 * VEC column totals (1 KiB) and a flag, and sums
 // the totals of its predecessors inside its group of ROWS_GROUP tiles; the last tile of a group publishes the group's
 // aggregate; the first one (the leader) sums group aggregates back to the nearest published prefix and publishes the
@@ -1393,8 +1393,13 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
         const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
         const bool live = nominal < g.inner;
         const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
-        const int64_t slab = o * g.inner * g.mid;
-        const int64_t row0 = slice * (NW * R) + (int64_t)wave * R;
+        // wave-uniform row addresses + a 32-bit offset per lane (the rows of a wave are the same for all its lanes)
+        const int64_t row0 = slice * (NW * R) + (int64_t)__builtin_amdgcn_readfirstlane(wave) * R;
+        const int64_t shift = strip * COLS >= VEC ? strip * COLS - VEC : 0;     // the first lane of a strip may reach back VEC columns
+        const int64_t wave_e0 = o * g.inner * g.mid + row0 * g.inner + shift;
+        const unsigned loff = (unsigned)(col0 - shift);
+        const int64_t left = g.mid - row0;
+        const int rows = left >= R ? R : (left > 0 ? (int)left : 0);            // rows of this wave inside the array
         VT v[R];
         // (The compiler waits for the second of these loads before it issues the other six, each being under a condition
         // of its own.  Issuing all eight back to back, with clamped addresses instead of conditions, measured slower
@@ -1402,10 +1407,10 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
         // every second (108) or every fourth (106).)
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (live && row0 + r < g.mid) {
+            if (live && r < rows) {
                 VI x;
-                if constexpr (ANY_ALIGN) x = load_nt_elems<In, VEC>(in + slab + (row0 + r) * g.inner + col0);
-                else x = load_nt((const VI*)(in + slab + (row0 + r) * g.inner + col0));
+                if constexpr (ANY_ALIGN) x = load_nt_elems<In, VEC>(in + wave_e0 + r * g.inner + loff);
+                else x = load_nt((const VI*)(in + wave_e0 + r * g.inner + loff));
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) v[r][j] = (T)x[j];
             } else {
@@ -1431,12 +1436,12 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
         for (int j = 0; j < VEC; ++j) pre[j] = op(lds_base[lane * VEC + j], pre[j]);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (live && row0 + r < g.mid) {
+            if (live && r < rows) {
                 VT o4;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o4[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r > 0 ? r - 1 : 0][j]));
-                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + slab + (row0 + r) * g.inner + col0, o4);
-                else store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o4);
+                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + wave_e0 + r * g.inner + loff, o4);
+                else store_nt((VT*)(out + wave_e0 + r * g.inner + loff), o4);
             }
         }
     }
@@ -1618,10 +1623,14 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     const int64_t pitch = strips * cols;
     const int64_t cus = device_info().cus;
     {
-        // single pass over tiles of 120 rows (7 waves of rows: 134 us against 109 for the 4096 x 16384 matrix); the payloads
-        // of all tiles and groups must fit the partials area.  8-byte values too: 2048 x 16384 Float64 103 us against 139
+        // single pass over tiles of 150 rows (7 waves of rows: 134 us against 109 for the 4096 x 16384 matrix; 15 waves of 8
+        // rows 104 us, of 10 rows -- with the row addresses wave-uniform, which freed the registers -- 100, of 12 rows 105);
+        // the payloads of all tiles and groups must fit the partials area.  8-byte values too: 2048 x 16384 Float64 103 us against 139
         // for the three passes, 4096 x 4096 Int64 54 against 70.
-        constexpr int NW = 15, R = 8;              // 15 waves of rows + 1 for the look-back
+#ifndef RK_ROWS_R
+#define RK_ROWS_R 8
+#endif
+        constexpr int NW = 15, R = RK_ROWS_R;              // 15 waves of rows + 1 for the look-back
         const int64_t nchains = strips * g.outer, nslices = (g.mid + NW * R - 1) / (NW * R), ntiles = nchains * nslices;
         const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
         if (vec && ws != nullptr && tune_scan_rows_ordered() != 0 && nchains < cus * 4 && nslices >= 4 &&
@@ -1687,7 +1696,7 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
     *done = false;
     if constexpr (ElemVectors<In, T>::value) {
         constexpr int VEC = 16 / (int)sizeof(T), COLS = WAVE * VEC;
-        constexpr int NW = 15, R = 8;
+        constexpr int NW = 15, R = 8;              // (ten rows per lane group: 63 x 500_000 Float32 71 -> 79 us)
         // (rows shorter than a 128-byte line: a load instruction then takes Q short pieces R rows apart, and the two-pass
         // tiles through LDS are two to three times faster: 7 x 4_194_304 Float32 265 against 83 us)
         if (g.inner * sizeof(In) < 128 || g.inner * 2 > COLS || !is_aligned(in, sizeof(In)) || !is_aligned(out, sizeof(T))) return RK_SUCCESS;
