@@ -471,6 +471,37 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
     }
 }
 
+// ---- completion count of the workgroups that share a result ----------------------------------------------------------
+// Called by one thread after the workgroup's partials are at the coherent level; true for the last of the `n` workgroups
+// of `slot`.  Atomics on one address complete one after the other, and hundreds of workgroups that finish together
+// queue up behind one ticket (findmax(A; dims=2) of 64 x 500_000 Float32, one strip, 512 workgroups: 72 us; the same
+// data as 64 x 7812 x 64, sixty-four tickets: 25 us).  With groups > 1 the workgroups take a ticket of their group of
+// TICKET_GROUP first and only the last of a group takes the slot's own: slot * (groups + 1) + group, then + groups.
+// The group tickets are left at zero; the caller clears the slot's own when it is done (arrival_reset).
+__device__ __forceinline__ bool last_arrival(uint32_t* tickets, int64_t slot, int idx, int n, int groups) {
+    if (groups <= 1) {
+        const uint32_t old = __hip_atomic_fetch_add(&tickets[slot * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return old == (uint32_t)n - 1u;
+    }
+    uint32_t* base = tickets + slot * (groups + 1) * TICKET_STRIDE;
+    const int grp = idx / TICKET_GROUP;
+    const int gsize = grp == groups - 1 ? n - grp * TICKET_GROUP : TICKET_GROUP;
+    const uint32_t old = __hip_atomic_fetch_add(&base[grp * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old != (uint32_t)gsize - 1u) return false;
+    __hip_atomic_store(&base[grp * TICKET_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t top = __hip_atomic_fetch_add(&base[groups * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return top == (uint32_t)groups - 1u;
+}
+__device__ __forceinline__ void arrival_reset(uint32_t* tickets, int64_t slot, int groups) {
+    if (groups <= 1) tickets[slot * TICKET_STRIDE] = 0;
+    else tickets[(slot * (groups + 1) + groups) * TICKET_STRIDE] = 0;
+}
+// groups for last_arrival: two levels when more than two groups' worth of workgroups share a slot and the tickets suffice
+inline int arrival_groups(int64_t slots, int64_t n) {
+    const int64_t groups = (n + TICKET_GROUP - 1) / TICKET_GROUP;
+    return (groups > 2 && slots * (groups + 1) <= (int64_t)WS_TICKET_COUNT) ? (int)groups : 1;
+}
+
 // ---- 1 < inner < 64 with long lines: contiguous runs of whole rows ---------------------------------------
 // (sum(A; dims=2) of a 3 x 1_000_000 array, perf/array.jl:91,96; the fold over the long dim of a 2 x 3 x N array.)
 // A wave per line reads one element in `inner`, a quarter or less of every cache line at a time.  Here thread t of
@@ -480,7 +511,7 @@ __global__ __launch_bounds__(256) void reduce_short_lines_kernel(const In* __res
 // rows of one slab; partials[(o * msplits + ms) * inner + column], one ticket per slab, the last arrival folds.
 template <typename In, typename Acc, typename Xf, typename Op, typename Sink>
 __global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
-                                                            Acc* partials, uint32_t* tickets, int64_t rows_per_split) {
+                                                            Acc* partials, uint32_t* tickets, int64_t rows_per_split, int tgroups) {
     typedef typename Xf::Pos Pos;
     __shared__ Acc lds[256];
     __shared__ int is_last;
@@ -527,10 +558,7 @@ __global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict
         publish_barrier();
     }
     __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
-    if (t == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[o * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (old == (uint32_t)msplits - 1u);
-    }
+    if (t == 0) is_last = last_arrival(tickets, o, ms, msplits, tgroups);
     __syncthreads();
     if (!is_last) return;
     // the last arrival folds the msplits rows of partials the way it folded its own rows: thread t takes column
@@ -538,8 +566,18 @@ __global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     Acc f = Op::template identity<Acc>();
     if (t < T) {
+        // (eight independent loads at a time: one after the other, each waits for the one before -- msplits / R round trips)
         const int rt = t / inner, c = t - rt * inner;
-        for (int i = rt; i < msplits; i += R) f = op(f, partials[(o * msplits + i) * inner + c]);
+        const Acc* pc = partials + o * msplits * inner + c;
+        int i = rt;
+        for (; i + 7 * R < msplits; i += 8 * R) {
+            Acc v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = pc[(int64_t)(i + u * R) * inner];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) f = op(f, v[u]);
+        }
+        for (; i < msplits; i += R) f = op(f, pc[(int64_t)i * inner]);
     }
     __syncthreads();     // lds is free again
     lds[t] = f;
@@ -549,16 +587,31 @@ __global__ __launch_bounds__(256) void reduce_narrow_kernel(const In* __restrict
         for (int k = 0; k < R; ++k) r2 = op(r2, lds[t + k * inner]);
         sink(t + o * g.inner, r2);
     }
-    if (t == 0) tickets[o * TICKET_STRIDE] = 0;
+    if (t == 0) arrival_reset(tickets, o, tgroups);
 }
 
 // ---- inner >= 64: lanes along `inner` -------------------------------------------------------------
 // grid (strips * outer, msplits): the outer index shares the x axis with the strips (the y and z axes of a grid end
 // at 65535, and a 64 x 2 x 70000 array has that many outer indices and more); workgroup = 4 waves; a wave owns
 // 64 * VEC adjacent columns of a strip and every 4th row of the row batches dealt to its workgroup.
-template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int UNROLL>
+// PACKED (one strip whose rows fill at most half of it, element-aligned vectors): P = ceil(inner / VEC) lanes hold a row
+// and a load instruction takes Q = 64 / P consecutive rows; lane group q sees the rows q, q + Q, ... of what the wave
+// is dealt, and the groups are folded across the lanes at the end.  (findmax(A; dims=2) of a 64 x 500_000 Float32
+// array: 16 of 64 lanes busy, 105 us; sums of such arrays are viewed as wider ones by the host instead.)
+template <typename T> __device__ __forceinline__ T shfl_down_words(const T& v, int delta) {
+    static_assert(sizeof(T) % 4 == 0, "whole words");
+    uint32_t w[sizeof(T) / 4];
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(T) / 4; ++i) w[i] = (uint32_t)__shfl_down((int)w[i], delta, WAVE);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+template <typename In, typename Acc, typename Xf, typename Op, typename Sink, bool VECTOR, int UNROLL, bool PACKED = false>
 __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restrict__ A, LineGeom g, Xf xf, Op op, Sink sink,
-                                                             Acc* partials, uint32_t* tickets, int strips) {
+                                                             Acc* partials, uint32_t* tickets, int strips, int tgroups, int P = WAVE) {
     constexpr int VEC = VECTOR ? 16 / sizeof(In) : 1;
     constexpr int COLS = WAVE * VEC;   // columns per strip
     constexpr int NW = 4;
@@ -570,8 +623,11 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     const int64_t o = tile / strips;
     const int strip = (int)(tile - o * strips);
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int64_t nominal = (int64_t)strip * COLS + (int64_t)lane * VEC;
-    const bool live = nominal < g.inner;
+    const int Q = PACKED ? WAVE / P : 1;                // rows per load instruction
+    const int q = PACKED ? lane / P : 0;                // this lane's row among them
+    const int pl = PACKED ? lane - q * P : lane;        // this lane's vector within the row
+    const int64_t nominal = (int64_t)strip * COLS + (int64_t)pl * VEC;
+    const bool live = nominal < g.inner && q < Q;
     // 4- and 8-byte elements: vectors at any element-aligned address (load_nt_elems), so rows need be no whole number
     // of vectors.  The last vector of such a row starts VEC elements before the row's end instead of running into the
     // next row; the `dup` leading columns it shares with the lane before are dropped after the loop.
@@ -591,16 +647,19 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
     // workgroups of a strip (and, strip by strip, the whole grid) read one compact band of rows.  Giving every
     // workgroup one long contiguous slice instead spreads the reads over rows megabytes apart, which the
     // memory system serves up to 20 % slower when the row pitch is a power of two.
+    // (PACKED: what is dealt out are groups of Q consecutive rows; `m` counts groups, the lane's row is m * Q + q)
     constexpr int64_t BATCH = (int64_t)UNROLL * NW;
-    const int64_t nbatches = (g.mid + BATCH - 1) / BATCH;
+    const int64_t ngroups = PACKED ? (g.mid + Q - 1) / Q : g.mid;
+    const int64_t nbatches = (ngroups + BATCH - 1) / BATCH;
     if (live) {
-        const In* p = A + slab + col0;
+        const In* p = A + slab + col0 + (PACKED ? (int64_t)q * g.inner : 0);
+        const int64_t pitch = PACKED ? g.inner * Q : g.inner;
         for (int64_t b = ms; b < nbatches; b += msplits) {
             const int64_t m = b * BATCH + wave;
             V v[UNROLL];
-            if (m + (UNROLL - 1) * NW < g.mid) {
+            if (PACKED ? (m + (UNROLL - 1) * NW) * Q + (Q - 1) < g.mid : m + (UNROLL - 1) * NW < g.mid) {
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) v[u] = load_row(p + (m + u * NW) * g.inner);
+                for (int u = 0; u < UNROLL; ++u) v[u] = load_row(p + (m + u * NW) * pitch);
                 if constexpr (XfIsBatch<Xf>::value) {
                     In x[UNROLL * VEC];
                     Acc y[UNROLL * VEC];
@@ -620,7 +679,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
                 } else {
 #pragma unroll
                     for (int u = 0; u < UNROLL; ++u) {
-                        const typename Xf::Pos e0 = (typename Xf::Pos)(m + u * NW);
+                        const typename Xf::Pos e0 = (typename Xf::Pos)(PACKED ? (m + u * NW) * Q + q : m + u * NW);
                         if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(v[u], e0));
                         else {
 #pragma unroll
@@ -629,9 +688,9 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
                     }
                 }
             } else {
-                for (int64_t r = m; r < g.mid; r += NW) {
-                    const V x = load_row(p + r * g.inner);
-                    const typename Xf::Pos e0 = (typename Xf::Pos)r;
+                for (int64_t r = m; (PACKED ? r * Q + q : r) < g.mid; r += NW) {
+                    const V x = load_row(p + r * pitch);
+                    const typename Xf::Pos e0 = (typename Xf::Pos)(PACKED ? r * Q + q : r);
                     if constexpr (VEC == 1) acc[0] = acc_step(op, acc[0], xf(x, e0));
                     else {
 #pragma unroll
@@ -641,9 +700,19 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
             }
         }
     }
+    if constexpr (PACKED) {
+        // the lane groups of a wave, folded into group 0 (idle lanes hold the identity; a lane past the wave's end has no partner)
+        for (int delta = P; delta < WAVE; delta <<= 1) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                const Acc y = shfl_down_words(acc[j], delta);
+                if (lane + delta < WAVE) acc[j] = op(acc[j], y);
+            }
+        }
+    }
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
-        if (j >= dup) lds[wave][lane * VEC + j - dup] = acc[j];      // columns past the row's end keep whatever LDS held: never sunk
+        if (j >= dup && q == 0) lds[wave][pl * VEC + j - dup] = acc[j];      // columns past the row's end keep whatever LDS held: never sunk
     __syncthreads();
     // thread t folds columns t, t + 256, ... of the strip: a strip has 64 * VEC columns -- 256 for 4-byte elements, one
     // a thread; 512 or 1024 for 2- and 1-byte elements
@@ -673,29 +742,25 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
 #pragma unroll
     for (int c = 0; c < CPT; ++c) {
         const int tc = t + c * 256;
-        if (tc < COLS) store_agent(&partials[(tile * msplits + ms) * COLS + tc], r[c]);
+        if (tc < COLS && (int64_t)strip * COLS + tc < g.inner) store_agent(&partials[(tile * msplits + ms) * COLS + tc], r[c]);
     }
     publish_barrier();
     __syncthreads();   // every partial of this workgroup is at the coherent level before the ticket moves
-    if (t == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&tickets[tile * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        is_last = (old == (uint32_t)msplits - 1u);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    // Last arrival of the strip: fold the msplits rows of partials.  The partials were written through to the
-    // coherent level; one acquire (cache invalidate) in this single workgroup lets it read them with plain,
-    // batched loads.  Wave w folds rows w, w+4, ... for the same columns it streamed; fixed order.
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    {
-        const Acc* prow = partials + tile * msplits * COLS + lane * VEC;
+    // Fold of `nrows` rows of partials ([row][COLS]) by this workgroup: wave w folds rows w, w + 4, ... for the columns it
+    // streamed, thread t then joins the four waves for its columns; fixed order.  The rows were written through to the
+    // coherent level; one acquire (cache invalidate) lets the workgroup read them with plain, batched loads.  Lanes whose
+    // columns lie past the row's end read nothing.
+    auto fold_rows = [&](const Acc* rows, int nrows, Acc (&out)[CPT]) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const Acc* prow = rows + lane * VEC;
         Acc f[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) f[j] = Op::template identity<Acc>();
-        int i = wave;
+        const bool fold_live = (int64_t)strip * COLS + (int64_t)lane * VEC < g.inner;
+        int i = fold_live ? wave : nrows;
         if constexpr (VEC <= 4) {
-            constexpr int FU = 4;            // rows a wave has in flight
-            for (; i + (FU - 1) * NW < msplits; i += FU * NW) {
+            constexpr int FU = sizeof(Acc) * VEC <= 32 ? 8 : 4;            // rows a wave has in flight
+            for (; i + (FU - 1) * NW < nrows; i += FU * NW) {
                 Acc v[FU][VEC];
 #pragma unroll
                 for (int u = 0; u < FU; ++u)
@@ -707,26 +772,69 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
                     for (int j = 0; j < VEC; ++j) f[j] = op(f[j], v[u][j]);
             }
         }
-        for (; i < msplits; i += NW)
+        for (; i < nrows; i += NW)
 #pragma unroll
             for (int j = 0; j < VEC; ++j) f[j] = op(f[j], prow[(int64_t)i * COLS + j]);
         __syncthreads();     // lds is free again
 #pragma unroll
         for (int j = 0; j < VEC; ++j) lds[wave][lane * VEC + j] = f[j];
         __syncthreads();
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int tc = t + c * 256;
+            out[c] = Op::template identity<Acc>();
+            if (tc < COLS) {
+                out[c] = lds[0][tc];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) out[c] = op(out[c], lds[w][tc]);
+            }
+        }
+    };
+    Acc res[CPT];
+    if (tgroups > 1) {
+        // Two levels (see last_arrival): the last arrival of a group of TICKET_GROUP workgroups folds the group's rows into
+        // one row of group partials, behind the partials of all tiles, and only then takes the strip's own ticket; the last
+        // group folds the group rows.  One workgroup folding all 512 rows of a single strip took 45 of the kernel's 70 us
+        // (findmax(A; dims=2), 64 x 500_000 Float32), whatever the loads in flight: the groups fold side by side.
+        const int grp = ms / TICKET_GROUP;
+        const int gsize = grp == tgroups - 1 ? msplits - grp * TICKET_GROUP : TICKET_GROUP;
+        uint32_t* base = tickets + tile * (tgroups + 1) * TICKET_STRIDE;
+        if (t == 0) {
+            const uint32_t old = __hip_atomic_fetch_add(&base[grp * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = (old == (uint32_t)gsize - 1u);
+        }
+        __syncthreads();
+        if (!is_last) return;
+        fold_rows(partials + (tile * msplits + (int64_t)grp * TICKET_GROUP) * COLS, gsize, res);
+        Acc* gpartials = partials + (int64_t)gridDim.x * msplits * COLS;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int tc = t + c * 256;
+            if (tc < COLS && (int64_t)strip * COLS + tc < g.inner) store_agent(&gpartials[(tile * tgroups + grp) * COLS + tc], res[c]);
+        }
+        publish_barrier();
+        __syncthreads();   // (also: everybody has read is_last before it is written again)
+        if (t == 0) {
+            __hip_atomic_store(&base[grp * TICKET_STRIDE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t top = __hip_atomic_fetch_add(&base[tgroups * TICKET_STRIDE], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            is_last = (top == (uint32_t)tgroups - 1u);
+        }
+        __syncthreads();
+        if (!is_last) return;
+        fold_rows(gpartials + tile * tgroups * COLS, tgroups, res);
+    } else {
+        if (t == 0) is_last = last_arrival(tickets, tile, ms, msplits, 1);
+        __syncthreads();
+        if (!is_last) return;
+        fold_rows(partials + tile * msplits * COLS, msplits, res);     // last arrival of the strip: all its rows
     }
 #pragma unroll
     for (int c = 0; c < CPT; ++c) {
         const int tc = t + c * 256;
         const int64_t col = (int64_t)strip * COLS + tc;
-        if (tc < COLS && col < g.inner) {
-            Acc f = lds[0][tc];
-#pragma unroll
-            for (int w = 1; w < NW; ++w) f = op(f, lds[w][tc]);
-            sink(col + o * g.inner, f);
-        }
+        if (tc < COLS && col < g.inner) sink(col + o * g.inner, res[c]);
     }
-    if (t == 0) tickets[tile * TICKET_STRIDE] = 0;
+    if (t == 0) arrival_reset(tickets, tile, tgroups);
 }
 
 // ---- arbitrary masks: one wave per output ------------------------------------------------------------
@@ -977,15 +1085,27 @@ inline int32_t launch_reduce(const In* A, int ndim, const int64_t* shape, uint32
             const int64_t tiles = (int64_t)p.strips * s.outer;
             if (tiles > 0x7fffffff) return RK_ERR_TOO_LARGE;
             dim3 grid((unsigned)tiles, p.splits);
+            int tgroups = arrival_groups(tiles, p.splits);
+            // the group rows lie behind the partials: one level where they do not fit
+            if (tgroups > 1 && (size_t)(tiles * (p.splits + tgroups)) * (WAVE * (p.vector ? 16 / sizeof(In) : 1)) * sizeof(Acc) > cap) tgroups = 1;
+            if constexpr (XfIsArg<Xf>::value && sizeof(In) >= 4) {
+                constexpr int VEC = 16 / (int)sizeof(In);
+                if (p.vector && p.strips == 1 && s.inner >= VEC && s.inner * 2 <= WAVE * VEC) {
+                    reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL, true><<<grid, 256, 0, stream>>>(
+                        A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips, tgroups, (int)((s.inner + VEC - 1) / VEC));
+                    break;
+                }
+            }
             if (p.vector)
-                reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips);
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, true, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips, tgroups);
             else
-                reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips);
+                reduce_strided_kernel<In, Acc, Xf, Op, Sink, false, UNROLL><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.strips, tgroups);
             break;
         }
         case ReducePlan::NARROW: {
             dim3 grid(p.splits, (unsigned)s.outer);
-            reduce_narrow_kernel<In, Acc, Xf, Op, Sink><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.rows_per_split);
+            reduce_narrow_kernel<In, Acc, Xf, Op, Sink><<<grid, 256, 0, stream>>>(A, g, xf, op, sink, (Acc*)w.partials, w.tickets, p.rows_per_split,
+                                                                                  arrival_groups(s.outer, p.splits));
             break;
         }
         case ReducePlan::GENERIC: {

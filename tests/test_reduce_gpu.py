@@ -169,6 +169,21 @@ def test_findminmax_dims(rk, orc, shape, dims):
     _check_findminmax(rk, orc, rng.standard_normal(shape).astype(np.float32), dims)
 
 
+@pytest.mark.parametrize("shape", [(64, 50_000), (100, 30_001), (128, 20_000), (65, 40_000, 3), (96, 5_000, 2), (127, 9_999), (64, 17), (72, 3_000, 5)])
+def test_findminmax_along_long_lines_behind_short_rows(rk, orc, shape):
+    """findmax / findmin(A; dims=2) with rows of 64 .. 128 elements (Float64, Int64: 64): several rows go into one load
+    instruction, a group of lanes each, and the groups are folded across the lanes at the end.  Few distinct values, so
+    that ties between rows of different lane groups decide by the first-index rule; the neighbouring shapes take the
+    plain kernels."""
+    rng = _rng(sum(shape))
+    for dtype in (np.float32, np.float64, np.int32, np.int64):
+        A = rng.integers(-3, 4, shape).astype(dtype)
+        _check_findminmax(rk, orc, A, 2)
+    A = rng.standard_normal(shape).astype(np.float32)
+    A[shape[0] // 2, shape[1] // 3] = np.nan
+    _check_findminmax(rk, orc, A, 2)
+
+
 def test_findmax_nan_and_zero_rules(rk, orc):
     A = np.array([[1, np.nan, -0.0, 3], [np.nan, 2, 0.0, 3], [5, np.nan, -0.0, -np.inf]], dtype=np.float32)
     for dims in (1, 2, None):
