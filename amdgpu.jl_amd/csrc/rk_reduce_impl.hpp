@@ -759,7 +759,7 @@ __global__ __launch_bounds__(256) void reduce_strided_kernel(const In* __restric
         const bool fold_live = (int64_t)strip * COLS + (int64_t)lane * VEC < g.inner;
         int i = fold_live ? wave : nrows;
         if constexpr (VEC <= 4) {
-            constexpr int FU = sizeof(Acc) * VEC <= 32 ? 8 : 4;            // rows a wave has in flight
+            constexpr int FU = 4;            // rows a wave has in flight (8: registers 64 -> 96 for findmax, and the many small workgroups of a short reduced dim lose occupancy)
             for (; i + (FU - 1) * NW < nrows; i += FU * NW) {
                 Acc v[FU][VEC];
 #pragma unroll
