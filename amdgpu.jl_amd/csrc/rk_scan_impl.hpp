@@ -1627,10 +1627,7 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
         // rows 104 us, of 10 rows -- with the row addresses wave-uniform, which freed the registers -- 100, of 12 rows 105);
         // the payloads of all tiles and groups must fit the partials area.  8-byte values too: 2048 x 16384 Float64 103 us against 139
         // for the three passes, 4096 x 4096 Int64 54 against 70.
-#ifndef RK_ROWS_R
-#define RK_ROWS_R 8
-#endif
-        constexpr int NW = 15, R = RK_ROWS_R;              // 15 waves of rows + 1 for the look-back
+        constexpr int NW = 15, R = sizeof(In) >= 4 ? 10 : 8;     // 15 waves of rows + 1 for the look-back (Bool -> Int64 with ten rows: 20 registers spilled)
         const int64_t nchains = strips * g.outer, nslices = (g.mid + NW * R - 1) / (NW * R), ntiles = nchains * nslices;
         const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
         if (vec && ws != nullptr && tune_scan_rows_ordered() != 0 && nchains < cus * 4 && nslices >= 4 &&
