@@ -33,7 +33,7 @@ def _scan(L, rk, x, out, ws, dims=1):
                                ws.data_ptr(), ws.numel(), stream_ptr())
 
 
-@pytest.mark.parametrize("shape,dims", [((1 << 24,), 1), ((2048, 8192), 2)])
+@pytest.mark.parametrize("shape,dims", [((1 << 24,), 1), ((2048, 8192), 2), ((64, 200_000), 2)])
 def test_scan_gives_up_and_recovers(rk, orc, tiny_budget, shape, dims):
     L = tiny_budget
     from amdgpu_jl_amd.array import stream_ptr
