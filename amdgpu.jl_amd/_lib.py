@@ -96,6 +96,7 @@ PROTOTYPES = {
     "rk_set_wait_budget": (C.c_int64, [C.c_int64]),
     "rk_workspace_status": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_sort_status": (C.c_int32, [C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_accumulate_static_status": (C.c_int32, [C.c_void_p]),
     "rk_mapreduce": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                  C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_mapreduce_strided": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, _I64P, _I64P, C.c_uint32,
@@ -162,6 +163,11 @@ class UnsupportedError(RKError, NotImplementedError):
     it raises the one exception type a caller catches to take another path.  `status` tells the three apart."""
 
 
+class WaitError(RKError):
+    """RK_ERR_WAIT: a kernel gave up a bounded wait, so the results of that call are meaningless.  Raised where the
+    mirror synchronises anyway (``Array(x)``, a scalar fetch); the workspace has been prepared again by then."""
+
+
 DECLINED = (RK_ERR_UNSUPPORTED, RK_ERR_TOO_LARGE, RK_ERR_WORKSPACE)
 
 
@@ -172,6 +178,8 @@ def check(status: int, where: str = "") -> None:
         raise DimensionMismatch(status, where)
     if status in DECLINED:
         raise UnsupportedError(status, where)
+    if status == RK_ERR_WAIT:
+        raise WaitError(status, where)
     raise RKError(status, where)
 
 

@@ -6,7 +6,7 @@ from __future__ import annotations
 import numpy as np
 
 from . import _lib as L
-from .array import ROCArray, stream_ptr, workspace
+from .array import ROCArray, note_waiting_call, stream_ptr, workspace
 from .mapreduce import _OP, _scalar_buffer
 
 
@@ -79,6 +79,7 @@ def _launch_accumulate(op, B, A, dims, init, inclusive):
                  1 if inclusive else 0, _scalar_buffer(init, B.dtype), ws, ws_bytes)
 
         def launch_strided():
+            note_waiting_call()
             L.check(L.lib.rk_accumulate_strided(*sargs, stream_ptr()), "rk_accumulate_strided")
         return launch_strided
     bytes_needed = L.lib.rk_workspace_bytes(L.RK_KIND_ACCUMULATE, B.code, A.ndim, L.shape_array(A.dims),
@@ -90,6 +91,7 @@ def _launch_accumulate(op, B, A, dims, init, inclusive):
     fn = L.lib.rk_accumulate
 
     def launch():
+        note_waiting_call()
         L.check(fn(*args, stream_ptr()), "rk_accumulate")
     return launch
 

@@ -100,6 +100,7 @@ class ROCArray:
         """``Array(x)``: synchronises the stream and copies to the host (Julia-shaped NumPy array)."""
         n = len(self)
         nbytes = n * self.dtype.itemsize
+        check_waits()                       # the host waits here anyway: the place to learn of a give-up
         torch.cuda.current_stream().synchronize()
         raw = self.buf[self.offset:self.offset + nbytes].cpu().numpy()
         return raw.view(self.dtype)[:n].reshape(self.dims, order="F").copy()
@@ -178,3 +179,52 @@ def workspace(min_bytes: int = 0):
         L.check(L.lib.rk_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr()), "rk_workspace_init")
         _workspaces[key] = ws
     return ws.data_ptr(), ws.numel()
+
+
+# ---- give-ups of bounded waits -------------------------------------------------------------------------
+# The single-pass scans, the one-pass findall and the small sorts wait on other workgroups with a budget; a kernel that
+# runs out of it records that in the workspace (the sort: in its temporary) and finishes with meaningless results.
+# The mirror reads those records where it synchronises anyway -- Array(x), item() -- for every workspace and sort
+# temporary that such a kernel has used on the current stream since the last look, and raises.
+_waiting: set = set()          # (device, stream) keys whose workspace has been handed to a kernel with bounded waits
+_sort_tmps: dict = {}          # (device, stream) -> temporaries of sorts whose record has not been read
+
+
+def note_waiting_call() -> None:
+    """The call being issued on the current stream polls other workgroups through the stream's workspace."""
+    _waiting.add((torch.cuda.current_device(), stream_ptr()))
+
+
+def note_sort(tmp: "torch.Tensor") -> None:
+    """Keeps a sort's temporary until its record has been read (instead of freeing it at once)."""
+    pending = _sort_tmps.setdefault((torch.cuda.current_device(), stream_ptr()), [])
+    pending.append(tmp)
+    if len(pending) > 16:                   # a long run of sorts without a fetch: read the records rather than hoard memory
+        check_waits()
+
+
+def check_waits() -> None:
+    """Reads the give-up records of the current stream (synchronises it when there are any to read); raises
+    ``WaitError`` after preparing the workspace again."""
+    if torch.cuda.is_current_stream_capturing():
+        return
+    key = (torch.cuda.current_device(), stream_ptr())
+    failed = None
+    if key in _waiting:
+        _waiting.discard(key)
+        ws = _workspaces.get(key)
+        if ws is not None:
+            st = L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr())
+            if st == L.RK_ERR_WAIT:
+                L.check(L.lib.rk_workspace_init(ws.data_ptr(), ws.numel(), stream_ptr()), "rk_workspace_init")
+                failed = "a scan or findall on this stream"
+            elif st != L.RK_SUCCESS:
+                L.check(st, "rk_workspace_status")
+    for tmp in _sort_tmps.pop(key, ()):
+        st = L.lib.rk_sort_status(tmp.data_ptr(), tmp.numel(), stream_ptr())
+        if st == L.RK_ERR_WAIT:
+            failed = "a sort on this stream"
+        elif st != L.RK_SUCCESS:
+            L.check(st, "rk_sort_status")
+    if failed is not None:
+        raise L.WaitError(L.RK_ERR_WAIT, failed)

@@ -61,6 +61,20 @@ int tune_scan_backoff() {
     return v;
 }
 
+// Start-up stagger of the single-pass scan in launch order: the last workgroup of the first resident round starts this
+// many ticks of the 100 MHz clock after the first (RK_SCAN_STAGGER_TICKS; 0 = all at once).
+int tune_scan_stagger_ticks() {
+    static const int v = env_int("RK_SCAN_STAGGER_TICKS", 500, 0, 100000);
+    return v;
+}
+
+// Tile numbers of the single-pass kernels that run one tile per workgroup (RK_ORDERED_IDS): 0 = from the launch order
+// while the whole grid is resident at once and from the device-wide counter beyond that, 1 = always the launch order,
+// 2 = always the counter.  Read at every call.
+int tune_ordered_ids() {
+    return env_int("RK_ORDERED_IDS", 0, 0, 2);
+}
+
 // Persistent 256-thread workgroups per compute unit of the look-back scan; larger workgroups scale it
 // down (RK_SCAN_BLOCKS_PER_CU).
 int tune_scan_blocks_per_cu() {
@@ -180,6 +194,8 @@ static int32_t static_scratch(hipStream_t stream, void** out) {
         if (ptr == nullptr || !is_aligned(ptr, 256)) return RK_ERR_WORKSPACE;
         const int32_t st = workspace_init(ptr, RK_STATIC_SCRATCH_BYTES, stream);
         if (st != RK_SUCCESS) return st;
+        // the array serves every stream of the device from now on: nobody may see it before the fill has finished
+        RK_HIP(hipStreamSynchronize(stream));
         g_static_ptr[dev] = ptr;
     }
     *out = g_static_ptr[dev];
@@ -216,7 +232,7 @@ size_t rk_workspace_bytes(rk_opkind kind, rk_dtype dt, int ndim, const int64_t* 
         // descriptors of the look-back scan: one tagged word per 4 bytes of the value, per tile
         const Shape3 s = collapse3(ndim, shape, dims_mask);
         const size_t esz = dtype_size(dt) < 4 ? 4 : dtype_size(dt);
-        const int64_t tile = 4 * WAVE * (16 / (int64_t)esz) * 8;           // ScanTile<T>::TILE
+        const int64_t tile = (int64_t)scan_tile_waves(s.mid, esz) * WAVE * (16 / (int64_t)esz) * 8;      // the tile launch_scan picks
         const int64_t tpl = (s.mid + tile - 1) / tile, gpl = (tpl + WAVE - 1) / WAVE;
         // one tagged word per 4 bytes of the value per tile, one 128-byte line per group of 64 tiles
         // scans across rows publish 1 KiB of column totals per tile in the partials area: one flag each
@@ -500,6 +516,22 @@ int32_t rk_accumulate_static(rk_op op, rk_dtype in, rk_dtype out, const void* in
     const int32_t st = static_scratch((hipStream_t)stream, &ws);
     if (st != RK_SUCCESS) return st;
     return rk_accumulate(op, in, out, in_ptr, out_ptr, ndim, shape, dim, inclusive, init, ws, RK_STATIC_SCRATCH_BYTES, stream);
+}
+
+int32_t rk_accumulate_static_status(void* stream) {
+    int dev = 0;
+    RK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return RK_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    void* ptr = g_static_ptr[dev];
+    if (ptr == nullptr) return RK_SUCCESS;                 // never used on this device
+    const int32_t st = rk_workspace_status(ptr, RK_STATIC_SCRATCH_BYTES, stream);
+    if (st == RK_ERR_WAIT) {                               // reported once; the array starts afresh
+        const int32_t again = workspace_init(ptr, RK_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+        if (again != RK_SUCCESS) return again;
+        RK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    }
+    return st;
 }
 
 }  // extern "C"

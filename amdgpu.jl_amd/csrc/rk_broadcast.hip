@@ -13,6 +13,7 @@
 // Arithmetic is NOT contracted into FMAs: Julia evaluates a .* x .+ y as separate mul and add.
 #include <cmath>
 #include <cstring>
+#include <cstdlib>
 
 #include "rk_common.hpp"
 #include "rk_interp.hpp"
@@ -173,8 +174,8 @@ template <typename CT, int VEC, int NOPS_> struct BcFetch {
 template <int NOPS_> struct EvalInterpN {
     static constexpr int NOPS = NOPS_;             // operand slots: load what the program declares, up to this many
     static constexpr bool USES_LDS = true;
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
         interp_run<CT, VEC, BC_BLOCK, true>(a.tokens, a.n_tokens, BcFetch<CT, VEC, NOPS_>{in}, out, lds);
     }
 };
@@ -188,8 +189,8 @@ typedef EvalInterpN<4> EvalInterp4;
 struct EvalAxpbyExp {
     static constexpr int NOPS = 4;
     static constexpr bool USES_LDS = false;
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = in[0][j] * in[1][j] + in[2][j] * exp(in[3][j]);
     }
@@ -198,8 +199,8 @@ struct EvalAxpbyExp {
 struct EvalAddMul {
     static constexpr int NOPS = 3;
     static constexpr bool USES_LDS = false;
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = in[0][j] + in[1][j] * in[2][j];
     }
@@ -208,8 +209,8 @@ struct EvalAddMul {
 struct EvalCopy {
     static constexpr int NOPS = 1;
     static constexpr bool USES_LDS = false;
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = in[0][j];
     }
@@ -218,8 +219,8 @@ struct EvalCopy {
 struct EvalBinary {
     static constexpr int NOPS = 2;
     static constexpr bool USES_LDS = false;
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
         // one scalar branch on the operator, then the component loop (the other way round every element
         // would evaluate pow)
 #define RK_BC_BIN2(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = in[0][j], y = in[1][j]; out[j] = (EXPR); } } break
@@ -291,8 +292,8 @@ struct EvalChain2 {
         }
 #undef RK_BC_BIN3
     }
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
         CT t[VEC];
         if (a.tokens[3] == 2) {                     // (u op1 v) op2 w
             apply<CT, VEC>(a.tokens[2], in[0], in[1], t);
@@ -332,8 +333,8 @@ template <int NOPS_> struct EvalLeftChainN {
         }
         return true;
     }
-    template <typename CT, int VEC>
-    static __device__ __forceinline__ void run(const BcArgs& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
         CT acc[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) acc[j] = in[0][j];
@@ -435,6 +436,60 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
     CT out[VEC];
     Eval::template run<CT, VEC>(a, in, out, lds);
     store_dest<CT, VEC, HOMOG>(a.dest, a.dest_dtype, dest_off, out);
+}
+
+
+// Flat mode, every array operand and the destination of the compute type, 16-byte aligned, dense (or a scalar): the
+// arguments are one compact block -- all pointers side by side, scalars already in the compute type -- so a wave fetches
+// them with one or two scalar loads and issues its vector loads at once.  In bc_kernel each operand's pointer, stride and
+// type sit 120 bytes apart behind branches of their own: a dozen dependent scalar-load round trips in front of the
+// first vector load, a fifth of the life of a wave that moves 64 bytes a lane.  Workgroups of BC_FLAT_BLOCK threads:
+// the same kernel measured in one process on the same buffers at 64 / 128 / 256 / 512 / 1024 threads gave
+// 6.38 / 6.41 / 6.29 / 6.24 / 6.48 TB/s at 2^26 Float32 elements, 6.38 / 6.36 / 6.18 / 6.17 / 6.34 at 2^27 and
+// 6.36 / 6.25 / 6.31 / 6.24 / 6.29 at 2^28 (the plain copy: 6.70 / 6.55 / 6.51 / - / 6.41 at 2^26); two vectors a
+// thread lose 1-3 % at every size, an XCD-banded order of the workgroups changes less than the run-to-run spread.
+struct BcFlatArgs {
+    int64_t     nvec;                       // 4-element vectors
+    void*       dest;
+    const void* ptr[RK_MAX_OPERANDS];       // nullptr: scalar
+    uint64_t    scalar[RK_MAX_OPERANDS];    // bits of the value in the compute type
+    int32_t     n_operands, n_tokens;
+    int32_t     tokens[RK_MAX_PROGRAM];
+};
+constexpr int BC_FLAT_BLOCK = 64;
+
+template <typename Eval, typename CT, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void bc_flat_kernel(const BcFlatArgs a) {
+    CT* lds = (CT*)bc_lds_raw;
+    typedef typename VecOf<CT, 4>::type V;
+    const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
+    if (i >= a.nvec) return;
+    CT in[RK_MAX_OPERANDS][4];
+#pragma unroll
+    for (int k = 0; k < Eval::NOPS; ++k) {
+        if (k >= a.n_operands) continue;
+        if (a.ptr[k] != nullptr) {
+            const V x = load_nt((const V*)a.ptr[k] + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) in[k][j] = x[j];
+        } else {
+            CT x;
+            __builtin_memcpy(&x, &a.scalar[k], sizeof(CT));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) in[k][j] = x;
+        }
+    }
+    CT out[4];
+    Eval::template run<CT, 4>(a, in, out, lds);
+    V o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = out[j];
+    store_nt((V*)a.dest + i, o);
+}
+
+static int tune_bc_flat_lean() {
+    const char* e = std::getenv("RK_BC_FLAT_LEAN");
+    return e ? std::atoi(e) : 1;
 }
 
 // Indexed mode: a dense destination whose rows are no whole number of 16-byte vectors (3 x N .+ 1 x N, 17 x N .* 17 x 1,
@@ -559,6 +614,38 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
     bool homog = a.dest_dtype == (std::is_same<CT, float>::value ? RK_F32 : (std::is_same<CT, double>::value ? RK_F64 : RK_I64));
     for (int k = 0; k < a.n_operands; ++k)
         if (a.op[k].ptr != nullptr && a.op[k].dtype != a.dest_dtype) homog = false;
+    if (!rows && vec && homog && a.indexed == 0 && tune_bc_flat_lean() != 0) {
+        // (a fill reads nothing, its workgroups live too briefly for 64 threads each: 2^26 Float32 40 -> 57 us)
+        bool lean = false;
+        for (int k = 0; k < a.n_operands; ++k)
+            if (a.op[k].ptr != nullptr) lean = true;
+        for (int k = 0; k < a.n_operands; ++k)
+            if (a.op[k].ptr != nullptr && a.op[k].stride0 != 1) lean = false;      // a one-element array against a vector
+        if (lean) {
+            BcFlatArgs f;
+            std::memset(&f, 0, sizeof(f));
+            f.nvec = a.total / 4;
+            f.dest = a.dest;
+            f.n_operands = a.n_operands;
+            f.n_tokens = a.n_tokens;
+            for (int i = 0; i < a.n_tokens; ++i) f.tokens[i] = a.tokens[i];
+            for (int k = 0; k < a.n_operands; ++k) {
+                const BcOperand& o = a.op[k];
+                f.ptr[k] = o.ptr;
+                if (o.ptr == nullptr) {
+                    const CT x = (o.dtype == RK_F32 || o.dtype == RK_F64 || o.dtype == RK_F16) ? (CT)o.sf : (CT)o.si;
+                    std::memcpy(&f.scalar[k], &x, sizeof(CT));
+                }
+            }
+            // evaluators with a value stack in LDS index it by BC_BLOCK threads
+            constexpr int FB = Eval::USES_LDS ? BC_BLOCK : BC_FLAT_BLOCK;
+            const int64_t blocks = (f.nvec + FB - 1) / FB;
+            if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+            bc_flat_kernel<Eval, CT, FB><<<(unsigned)blocks, FB, lds, stream>>>(f);
+            RK_LAUNCH_CHECK();
+            return RK_SUCCESS;
+        }
+    }
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
     if (a.indexed != 0) {            // the planner sets it together with vec and rows
         const int64_t blocks = ((a.total + 3) / 4 + BC_BLOCK - 1) / BC_BLOCK;

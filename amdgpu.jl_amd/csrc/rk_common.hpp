@@ -54,7 +54,7 @@ const DeviceInfo& device_info();   // rk_api.hip
 //                                from the partials so arbitrary partial bits never look like a tag)
 struct WsHeader {
     uint64_t scan_counter;  // look-back scan: epoch << 32 | tile acquisitions of the running call
-    uint32_t wait_failed;   // set by a kernel that gave up a bounded wait (see WaitCtl); read by rk_workspace_status
+    uint32_t wait_failed;   // epoch of a call that gave up a bounded wait (see WaitCtl), 0 = none; read by rk_workspace_status
     uint32_t pad[61];
 };
 static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
@@ -315,23 +315,26 @@ __device__ __forceinline__ void publish_barrier() {
 // Every loop that polls memory written by another workgroup (look-back of the scans, of the select and of the
 // sort) counts its unsuccessful rounds.  When one wait has used `budget` rounds -- which only happens when the
 // state it polls is not what the protocol expects: a workspace that was never prepared, or one shared by calls
-// that run at the same time -- it sets the word `failed`, stops waiting and carries on with a meaningless value,
-// so that every workgroup still runs to its end and the kernel exits normally.  All waiters look at `failed`
-// every few rounds and give up with the first one.  The results of such a call are wrong; the host learns of it
-// through rk_workspace_status / rk_sort_status and has to prepare the workspace again.
+// that run at the same time -- it writes the call's `stamp` into the word `failed`, stops waiting and carries on
+// with a meaningless value, so that every workgroup still runs to its end and the kernel exits normally.  All
+// waiters of the SAME call look at `failed` every few rounds and give up with the first one; a stamp left by an
+// earlier call (the word stays set until the host has read it and prepared the workspace again) is not theirs and
+// does not stop them.  The results of the call that gave up are wrong; the host learns of it through
+// rk_workspace_status / rk_sort_status.
 struct WaitCtl {
     uint32_t* failed;
     long long budget;       // unsuccessful poll rounds one wait may spend (a round is a device-coherent load: ~1 us)
     int       backoff;      // s_sleep units between rounds
+    uint32_t  stamp;        // nonzero mark of the running call: the scan epoch (set by the kernel), 1 in the sort's own control block
 };
 // Called once per unsuccessful round by (at least) one full wave; true = stop waiting.
 __device__ __forceinline__ bool wait_give_up(const WaitCtl& w, long long& rounds) {
     ++rounds;
     if (rounds >= w.budget) {
-        __hip_atomic_store(w.failed, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(w.failed, w.stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return true;
     }
-    if ((rounds & 31) == 0 && __hip_atomic_load(w.failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return true;
+    if ((rounds & 31) == 0 && __hip_atomic_load(w.failed, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == w.stamp) return true;
     for (int b = 0; b < w.backoff; ++b) __builtin_amdgcn_s_sleep(8);
     return false;
 }

@@ -465,6 +465,7 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
     while ((int64_t)(cur & 0xffffffffull) < ntiles) {
         const int64_t tile = (int64_t)(cur & 0xffffffffull);
         const uint32_t epoch = (uint32_t)(cur >> 32);
+        wc.stamp = epoch;
         const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
         const int64_t e0 = line * line_len + tl * TILE;
         const int64_t left = line_len - tl * TILE;
@@ -495,6 +496,29 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
         cur = lds_id;
     }
     chain_finish(cur, ntiles, (int64_t)Words<T>::N * (ntiles + ngroups), counter, desc, desc_capacity);
+}
+
+// The tile of a workgroup of an "ordered" kernel (one tile per workgroup, every tile waits only for tiles of lower
+// number) and the epoch of the call.  dynamic_ids == 0: the workgroup's index -- every predecessor of a tile is then a
+// workgroup the hardware has started earlier, provided it starts workgroups in index order, which holds for one grid
+// alone on the device.  When two such grids are resident together the premise has a hole: the lowest unfinished tile of
+// grid A can be waiting for a slot on a compute unit whose slots are all held by waiting tiles of grid B, and the
+// other way round -- nothing in the way slots are handed to queues excludes it -- so a grid with more workgroups than
+// the device holds at once takes its tile numbers from the packed counter instead (dynamic_ids != 0; one device-wide
+// atomic per workgroup, which returns the epoch with the number): a tile's predecessors then belong to workgroups that
+// have already started, whatever else is resident.  A grid that fits the device whole cannot be part of such a cycle
+// through its own unstarted tiles for long: every other grid's waiting tiles depend only on their own grid.
+// `need_epoch` (wave-uniform): this wave uses the epoch -- the others of a launch-order grid skip the load and get 0.
+struct OrderedId { int64_t tile; uint32_t epoch; };
+__device__ __forceinline__ OrderedId ordered_tile_id(unsigned long long* counter, int dynamic_ids, bool need_epoch) {
+    __shared__ unsigned long long lds_ordered_id;
+    if (dynamic_ids == 0)
+        return OrderedId{(int64_t)blockIdx.x,
+                         need_epoch ? (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32) : 0u};
+    if (threadIdx.x == 0) lds_ordered_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const unsigned long long cur = lds_ordered_id;
+    return OrderedId{(int64_t)(cur & 0xffffffffull), (uint32_t)(cur >> 32)};
 }
 
 // End of a kernel whose workgroups read the epoch from the header instead of acquiring it: the workgroup that leaves
@@ -532,6 +556,14 @@ __device__ __forceinline__ void ordered_finish(uint32_t epoch, int64_t used, uns
     if (e == 0u) e = 1u;                  // tag 0 marks a cleared slot
     if (lane == 0) *counter = (unsigned long long)e << 32;
 }
+// Workgroups of `threads` threads that an ordered kernel (compiled for 8 waves per SIMD, a few hundred bytes of LDS) has
+// resident at once, and whether a grid of `nblocks` takes its tile numbers from the counter (see ordered_tile_id).
+int tune_ordered_ids();            // rk_api.hip: 0 = by grid size, 1 = always the launch order, 2 = always the counter
+inline int64_t ordered_resident(int threads) { return (int64_t)device_info().cus * (32 * WAVE / threads); }
+inline int ordered_dynamic_ids(int64_t nblocks, int threads) {
+    const int t = tune_ordered_ids();
+    return t == 1 ? 0 : (t == 2 ? 1 : (nblocks > ordered_resident(threads) ? 1 : 0));
+}
 // Workgroups per first-level exit ticket: at most half of the ticket lines in use, at least TICKET_GROUP a ticket.
 inline int ordered_ticket_group(int64_t nblocks) {
     int64_t tg = (nblocks + (int64_t)WS_TICKET_COUNT / 2 - 1) / ((int64_t)WS_TICKET_COUNT / 2);
@@ -560,7 +592,7 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
                                                                     int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                                     unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                     uint64_t* desc, int64_t ngroups_per_line, int64_t ngroups,
-                                                                    int64_t desc_capacity, WaitCtl wc) {
+                                                                    int64_t desc_capacity, WaitCtl wc, int stagger_ticks, int stagger_tiles, int dynamic_ids) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     __shared__ T lds_wave[NW];
@@ -569,9 +601,19 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     uint64_t* tile_desc = desc;                                        // [words][ntiles]
     uint64_t* group_desc = desc + (int64_t)Words<T>::N * ntiles;       // [ngroups] lines
-    const uint32_t epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
+    const OrderedId id = ordered_tile_id(counter, dynamic_ids, wave == 0);      // wave 0 looks back and leaves last
+    const uint32_t epoch = id.epoch;
+    wc.stamp = epoch;
+    // The workgroups of the first resident round start together, so they would load together, wait for their prefixes
+    // together and store together, and the rounds behind them inherit the rhythm: memory idles while everybody waits.
+    // Tile i of that round therefore starts i / stagger_tiles of `stagger_ticks` (100 MHz clock) late.
+    if (id.tile < stagger_tiles) {
+        const long long d = (long long)stagger_ticks * id.tile / stagger_tiles;
+        const long long t0 = wall_clock64();
+        while (wall_clock64() - t0 < d) __builtin_amdgcn_s_sleep(4);
+    }
     {
-        const int64_t tile = blockIdx.x;
+        const int64_t tile = id.tile;
         const int64_t line = tile / tiles_per_line, tl = tile - line * tiles_per_line;
         const int64_t e0 = line * line_len + tl * TILE;
         const int64_t left = line_len - tl * TILE;
@@ -1358,7 +1400,7 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
                                                                                int inclusive, Op op, int64_t strips, int64_t nchains,
                                                                                int64_t nslices, T* payload, unsigned long long* counter,
                                                                                uint32_t* tickets, int ticket_group, uint64_t* desc,
-                                                                               int64_t desc_capacity, WaitCtl wc) {
+                                                                               int64_t desc_capacity, WaitCtl wc, int dynamic_ids) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int COLS = WAVE * VEC;
     typedef typename VecOf<T, VEC>::type VT;
@@ -1368,11 +1410,12 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
     const T ident = Op::template identity<T>();
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     const int64_t ntiles = gridDim.x;
-    const int64_t tile = blockIdx.x;
+    const OrderedId id = ordered_tile_id(counter, dynamic_ids, wave == NW || wave == 0);    // the look-back's wave, and thread 0 at the exit
+    const int64_t tile = id.tile;
     const int64_t slice = tile / nchains, chain = tile - slice * nchains;
-    uint32_t epoch = 0;
+    const uint32_t epoch = id.epoch;
+    wc.stamp = epoch;
     if (wave == NW) {
-        epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
         __syncthreads();                                 // the row waves have written their column totals
         T tot[VEC], base[VEC];
 #pragma unroll
@@ -1445,11 +1488,7 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
             }
         }
     }
-    // the helper wave's thread 0 would do as well; ordered_finish wants thread 0 of the workgroup, so hand it the epoch
-    __shared__ uint32_t lds_epoch;
-    if (wave == NW && lane == 0) lds_epoch = epoch;
-    __syncthreads();
-    ordered_finish(lds_epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
+    ordered_finish(epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
 }
 
 // ---- VEC <= inner <= 32 * VEC, long lines: several rows per load instruction, single pass ----------------------------
@@ -1467,7 +1506,7 @@ template <typename In, typename T, typename Op, int NW, int R>
 __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(const In* in, T* out, ScanGeom g, T init, int inclusive, Op op,
                                                                               int P, int64_t nchains, int64_t nslices, T* payload,
                                                                               unsigned long long* counter, uint32_t* tickets, int ticket_group,
-                                                                              uint64_t* desc, int64_t desc_capacity, WaitCtl wc) {
+                                                                              uint64_t* desc, int64_t desc_capacity, WaitCtl wc, int dynamic_ids) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int COLS = WAVE * VEC;
     typedef typename VecOf<T, VEC>::type VT;
@@ -1477,11 +1516,12 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(co
     const T ident = Op::template identity<T>();
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     const int64_t ntiles = gridDim.x;
-    const int64_t tile = blockIdx.x;
+    const OrderedId id = ordered_tile_id(counter, dynamic_ids, wave == NW || wave == 0);    // the look-back's wave, and thread 0 at the exit
+    const int64_t tile = id.tile;
     const int64_t slice = tile / nchains, chain = tile - slice * nchains;
-    uint32_t epoch = 0;
+    const uint32_t epoch = id.epoch;
+    wc.stamp = epoch;
     if (wave == NW) {
-        epoch = (uint32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> 32);
         __syncthreads();                                 // the row waves have written their column totals
         T tot[VEC], base[VEC];
 #pragma unroll
@@ -1570,10 +1610,7 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(co
             }
         }
     }
-    __shared__ uint32_t lds_epoch;
-    if (wave == NW && lane == 0) lds_epoch = epoch;
-    __syncthreads();
-    ordered_finish(lds_epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
+    ordered_finish(epoch, ntiles + (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains, counter, tickets, ticket_group, desc, desc_capacity);
 }
 
 // ---- host side ---------------------------------------------------------------------------------------
@@ -1583,10 +1620,19 @@ template <typename T, int K> struct ScanTile {     // geometry of the tile kerne
 };
 
 int tune_scan_backoff();        // rk_api.hip
-long long wait_budget();        // rk_api.hip: poll rounds a bounded wait may spend (rk_set_wait_budget)
-inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_budget(), tune_scan_backoff()}; }
-int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_waves();          // rk_api.hip: 0 = choose by line length, else 4, 8 or 16 waves per workgroup
+// Waves per workgroup of the single-pass scan of lines of `mid` values of `esz` (>= 4) bytes; a tile is 8 16-byte vectors
+// a lane.  Shared with rk_workspace_bytes, which sizes the descriptors for the tiles chosen here.
+inline int scan_tile_waves(int64_t mid, size_t esz) {
+    if (tune_scan_waves() != 0) return tune_scan_waves();
+    const int64_t tile4 = (int64_t)4 * WAVE * (16 / (int64_t)esz) * 8;
+    const int64_t tile16 = tile4 * 4, cover16 = (mid + tile16 - 1) / tile16 * tile16;
+    return cover16 * 10 <= mid * 11 ? 16 : (mid * (int64_t)esz > ((int64_t)32 << 10) ? 8 : 4);
+}
+int tune_scan_stagger_ticks();  // rk_api.hip: start-up stagger of the ordered scan in 10 ns ticks across the first resident round
+long long wait_budget();        // rk_api.hip: poll rounds a bounded wait may spend (rk_set_wait_budget)
+inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_budget(), tune_scan_backoff(), 0u}; }   // stamp: the kernel's epoch
+int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
 int tune_scan_rows_packed();     // rk_api.hip: 0 = short rows never take the single-pass kernel with several rows per load
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
@@ -1634,7 +1680,8 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
             (size_t)((ntiles + 2 * ngroups) * cols) * sizeof(T) <= scratch_bytes && (size_t)(ntiles + ngroups) * sizeof(uint64_t) <= ws->desc_bytes) {
             scan_rows_ordered_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
                 in, out, g, init, inclusive, op, strips, nchains, nslices, (T*)scratch, (unsigned long long*)&ws->hdr->scan_counter,
-                ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr));
+                ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr),
+                ordered_dynamic_ids(ntiles, (NW + 1) * WAVE));
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -1707,7 +1754,7 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
             return RK_SUCCESS;
         scan_rows_packed_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
             in, out, g, init, inclusive, op, P, nchains, nslices, (T*)w.partials, (unsigned long long*)&w.hdr->scan_counter, w.tickets,
-            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr));
+            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE));
         RK_LAUNCH_CHECK();
         *done = true;
     }
@@ -1909,9 +1956,7 @@ inline int32_t launch_scan(const ScanArgs& a) {
     // empty, and a half-idle workgroup of 1024 threads holds half a compute unit: 3000 lines of 20000 Float32 139 us
     // with 16 waves, 85 us with 8; 1300 lines of 50000: 119 against 97; 600 lines of 100000: 88 against 85
     // -- so 16 waves only where their tiles are at least 90 % full (65536 x 1024 Int32, two full tiles a line: 96 against 101 us)
-    const int64_t tile16 = (int64_t)ScanTile<T, KT>::TILE / 4 * 16, cover16 = (s.mid + tile16 - 1) / tile16 * tile16;
-    int nw = cover16 * 10 <= s.mid * 11 ? 16 : (line_bytes > ((int64_t)32 << 10) ? 8 : 4);
-    if (tune_scan_waves() != 0) nw = tune_scan_waves();
+    const int nw = scan_tile_waves(s.mid, sizeof(T));
     const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
     const int64_t tpl = (s.mid + TILE - 1) / TILE;
     const int64_t ntiles = tpl * nlines;
@@ -1932,7 +1977,13 @@ inline int32_t launch_scan(const ScanArgs& a) {
             const int tg = ordered_ticket_group(ntiles);
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
             scan_ordered_kernel<In, T, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
-                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, tg, w.desc, gpl, ngroups, cap, wc)
+                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, tg, w.desc, gpl, ngroups, cap, wc, stagger_ticks, stagger_tiles, dyn)
+            // staggered start of the first resident round (two workgroups of 16 waves a compute unit), where more rounds
+            // follow: 5 us across the round measured best (2^26 Int32: 0 / 2 / 4 / 6 / 8 / 12 / 16 us -> 91.8 / 90.3 / 89.7 /
+            // 89.9 / 90.1 / 90.9 / 92.0 us; 2^27: 177.9 -> 174.0 us; half the round late by a fixed time gained nothing)
+            const int64_t resident = ordered_resident(nw * WAVE);
+            const int stagger_tiles = (nw == 16 && ntiles >= 2 * resident) ? (int)resident : 0, stagger_ticks = tune_scan_stagger_ticks();
+            const int dyn = ordered_dynamic_ids(ntiles, nw * WAVE);
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED
             RK_LAUNCH_CHECK();

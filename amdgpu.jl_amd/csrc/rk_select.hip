@@ -44,14 +44,15 @@ __device__ __forceinline__ void emit_index(int64_t* __restrict__ ys, int64_t pos
 // scanned positions; the wave then reads the strip back in order and writes indices with coalesced stores (a
 // lane writing its own run directly makes every store instruction touch 64 different lines: 4x slower at high
 // density).  Only bit 0 of a byte is looked at (Julia's Bool).
-// ORDERED: one workgroup per tile, tile = blockIdx.x, the look-back and the end of the call as in scan_ordered_kernel
+// ORDERED: one workgroup per tile (its number from the launch order or, for grids beyond what is resident at once, from the
+// counter: ordered_tile_id), the look-back and the end of the call as in scan_ordered_kernel
 // (no tile counter, only the first tile of a group of 64 reads group descriptors, each on a line of its own).
 template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K, bool ORDERED>
 __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uint8_t* __restrict__ bools, int64_t n, int64_t* __restrict__ ys,
                                                                        int64_t* __restrict__ count_out, SelShape shp, int aligned,
                                                                        unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                        uint64_t* desc, int64_t ntiles, int64_t ngroups, int64_t desc_capacity,
-                                                                       WaitCtl wc) {
+                                                                       WaitCtl wc, int dynamic_ids) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int SEL_TILE = SEL_NW * SEL_CHUNK * SEL_K;
     __shared__ uint16_t lds_strip[SEL_NW][SEL_CHUNK];
@@ -65,7 +66,8 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
 
     unsigned long long cur;
     if constexpr (ORDERED) {
-        cur = (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & ~0xffffffffull) | (unsigned long long)blockIdx.x;
+        const OrderedId id = ordered_tile_id(counter, dynamic_ids, true);
+        cur = ((unsigned long long)id.epoch << 32) | (unsigned long long)id.tile;
     } else {
         if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
@@ -74,6 +76,7 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
     while ((int64_t)(cur & 0xffffffffull) < ntiles) {
         const int64_t tile = (int64_t)(cur & 0xffffffffull);
         const uint32_t epoch = (uint32_t)(cur >> 32);
+        wc.stamp = epoch;
         const int64_t e0 = tile * SEL_TILE;
         const int64_t left = n - e0;
         const int valid = left < SEL_TILE ? (int)left : SEL_TILE;
@@ -276,11 +279,12 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const int aligned = is_aligned(bools, 16) ? 1 : 0;
     const WaitCtl wc = wait_ctl(w.hdr);
+    const int dyn = ordered ? ordered_dynamic_ids(ntiles, nw * WAVE) : 0;
     hipStream_t st = (hipStream_t)stream;
 #define RK_SELECT3(LIN, SM, NWW, KK, ORD)                                                                                        \
     findall_select_kernel<LIN, SM, NWW, KK, ORD><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned,      \
                                                                                         counter, w.tickets, tg, w.desc, ntiles,    \
-                                                                                        ngroups, cap, wc)
+                                                                                        ngroups, cap, wc, dyn)
 #define RK_SELECT2(LIN, SM, KK)                                                                                                  \
     do {                                                                                                                         \
         if (!ordered) RK_SELECT3(LIN, SM, 16, KK, false);                                                                        \

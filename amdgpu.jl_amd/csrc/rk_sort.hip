@@ -715,7 +715,7 @@ __global__ __launch_bounds__(SORT_BLOCK, (sort_pass_waves<T, PERM, COUNTED>())) 
                 constexpr int LB = 8;
                 int64_t t = (int64_t)tile - 1;
                 bool done = false;
-                const WaitCtl wc{&ctl->wait_failed, wait_rounds, 0};
+                const WaitCtl wc{&ctl->wait_failed, wait_rounds, 0, 1u};     // the control block belongs to this call alone
                 long long rounds = 0;
                 while (!done) {
                     uint64_t w[LB];

@@ -10,7 +10,7 @@ import numpy as np
 
 from . import _lib as L
 from .accumulate import accumulate
-from .array import ROCArray, stream_ptr, workspace
+from .array import ROCArray, note_waiting_call, stream_ptr, workspace
 from .mapreduce import count
 
 
@@ -37,6 +37,7 @@ def findall(*args) -> ROCArray:
     if total > 0:
         shape = L.shape_array(bools.dims)
         ws, ws_bytes = workspace(L.lib.rk_workspace_bytes(L.RK_KIND_FINDALL, L.RK_U8, nd, shape, 0))
+        note_waiting_call()
         L.check(L.lib.rk_findall(bools.ptr, nd, shape, ys.ptr, None, ws, ws_bytes, stream_ptr()), "rk_findall")
     return ys
 

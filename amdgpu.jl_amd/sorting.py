@@ -7,7 +7,7 @@ import numpy as np
 import torch
 
 from . import _lib as L
-from .array import ROCArray, device, stream_ptr
+from .array import ROCArray, device, note_sort, stream_ptr
 
 
 def _check(x: ROCArray, lt, by):
@@ -24,6 +24,16 @@ def _tmp(code: int, n: int, perm: bool) -> torch.Tensor:
     return t
 
 
+def _release(tmp: torch.Tensor, n: int) -> None:
+    """Sorts of up to 2^20 keys resolve their digit offsets by look-back, with bounded waits: their temporary is kept
+    until its give-up record has been read (``array.check_waits``, at the next ``Array(x)``).  Larger sorts count
+    before every pass and wait for nobody: their temporary goes back to the allocator at once."""
+    if n <= (1 << 20):
+        note_sort(tmp)
+    else:
+        tmp.record_stream(torch.cuda.current_stream())
+
+
 def sort_(x: ROCArray, *, rev: bool = False, lt=None, by=None) -> ROCArray:
     """``sort!(x; rev)``: in place, returns ``x``."""
     _check(x, lt, by)
@@ -31,7 +41,7 @@ def sort_(x: ROCArray, *, rev: bool = False, lt=None, by=None) -> ROCArray:
     if n > 1:
         tmp = _tmp(x.code, n, False)
         L.check(L.lib.rk_sort(x.code, x.ptr, n, 1 if rev else 0, tmp.data_ptr(), tmp.numel(), stream_ptr()), "rk_sort")
-        tmp.record_stream(torch.cuda.current_stream())
+        _release(tmp, n)
     return x
 
 
@@ -50,7 +60,7 @@ def sortperm_(ix: ROCArray, x: ROCArray, *, rev: bool = False, lt=None, by=None)
     if n > 0:
         tmp = _tmp(x.code, n, True)
         L.check(L.lib.rk_sortperm(x.code, x.ptr, ix.ptr, n, 1 if rev else 0, tmp.data_ptr(), tmp.numel(), stream_ptr()), "rk_sortperm")
-        tmp.record_stream(torch.cuda.current_stream())
+        _release(tmp, n)
     return ix
 
 

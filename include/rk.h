@@ -118,18 +118,26 @@ RK_API int32_t rk_workspace_init(void* ws, size_t ws_bytes, void* stream);
  * the same time, could make it wait for ever -- a hung GPU -- so every wait counts its
  * unsuccessful polls: after `rounds` of them (default 2^21, a second or two; environment
  * RK_WAIT_BUDGET) the kernel records the failure in the workspace, stops waiting and runs to
- * its end with meaningless results.  No counterpart in the reference, whose kernels never
- * wait on each other (it launches one kernel per pass, src/kernels/mapreduce.jl:158-170).
+ * its end with meaningless results.  The record names the call that failed: the other
+ * workgroups of that call give up with it, later calls on the same workspace are not touched
+ * by it and run normally, and it stays readable until the workspace is prepared again.  A
+ * binding reads it wherever it synchronises anyway (copy to the host, scalar fetch) and
+ * raises.  No counterpart in the reference, whose kernels never wait on each other (it
+ * launches one kernel per pass, src/kernels/mapreduce.jl:158-170).
  *   rk_set_wait_budget   sets the budget for later calls of this process (<= 0: the default)
  *                        and returns the previous one.
  *   rk_workspace_status  SYNCHRONISES `stream`, then returns RK_ERR_WAIT if any call on the
  *                        workspace gave up a wait since it was last prepared, else
  *                        RK_SUCCESS.  After RK_ERR_WAIT call rk_workspace_init again.
  *   rk_sort_status       the same for the temporary of rk_sort / rk_sortperm (no
- *                        preparation needed afterwards: every sort clears its temporary). */
+ *                        preparation needed afterwards: every sort clears its temporary).
+ *   rk_accumulate_static_status   the same for the library's own array behind
+ *                        rk_accumulate_static on the current device; after RK_ERR_WAIT the
+ *                        array has been prepared again before the call returns. */
 RK_API int64_t rk_set_wait_budget(int64_t rounds);
 RK_API int32_t rk_workspace_status(const void* ws, size_t ws_bytes, void* stream);
 RK_API int32_t rk_sort_status(const void* tmp, size_t tmp_bytes, void* stream);
+RK_API int32_t rk_accumulate_static_status(void* stream);
 
 /* ---- mapreduce ------------------------------------------------------------------
  * Replaces GPUArrays.mapreducedim!(f, op, R, A; init)      src/kernels/mapreduce.jl:86-173
@@ -244,7 +252,9 @@ RK_API int32_t rk_accumulate_strided(rk_op op, rk_dtype in, rk_dtype out,
  * RK_ERR_TOO_LARGE.  Calls no hipMalloc / hipFree.  Every call on a GPU uses that GPU's one
  * array: calls that overlap in time on one GPU (two streams, two threads) race and must be
  * ordered by the caller.  The first call on each device prepares the array with a small kernel
- * on `stream`; it must not be made while that stream is being captured (RK_ERR_WORKSPACE). */
+ * on `stream` and waits for it (so that calls on other streams find it prepared); it must not be
+ * made while that stream is being captured (RK_ERR_WORKSPACE).  A give-up of a bounded wait
+ * is read with rk_accumulate_static_status. */
 #define RK_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
 RK_API int32_t rk_accumulate_static(rk_op op, rk_dtype in, rk_dtype out,
                              const void* in_ptr, void* out_ptr,
