@@ -7,6 +7,7 @@ build in parallel.  hipcc cross-compiles: no GPU is needed to build.
 """
 from __future__ import annotations
 
+import hashlib
 import os
 import re
 import subprocess
@@ -36,9 +37,22 @@ UNITS = (
 )
 
 
+def _stamp_path(unit) -> str:
+    src, suffix, _ = unit
+    return os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".stamp")
+
+
+def _flags_key(unit) -> str:
+    """What the object depends on besides its sources: the compiler and every flag of the unit."""
+    return hashlib.sha256("\0".join([HIPCC, *FLAGS, *unit[2]]).encode()).hexdigest()
+
+
 def _compile(unit):
     src, suffix, extra = unit
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
+    stamp = _stamp_path(unit)
+    if os.path.exists(stamp):
+        os.remove(stamp)                 # no stamp = not a checked object: an interrupted or failed build leaves none
     cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # No kernel of this library may keep an array in private memory: the ones that did (operand registers indexed with a
@@ -82,14 +96,21 @@ def _compile(unit):
     err = "\n".join(lines)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}{suffix}:\n{err}")
+    if not private:
+        # the stamp records the flags the object was built with and that it passed the private-memory check; an
+        # incremental build recompiles every unit whose stamp is missing or was written for other flags
+        with open(stamp, "w") as f:
+            f.write(_flags_key(unit) + "\n")
     return obj, err, [f"{src}{suffix}: {p}" for p in private]
 
 
 def _stale(unit) -> bool:
-    """True when the unit's object is older than its source or any header of the library."""
+    """True when the unit's object is older than its source or any header of the library, was built with other
+    flags, or did not pass the private-memory check (no stamp)."""
     src, suffix, _ = unit
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + suffix + ".o")
-    if not os.path.exists(obj):
+    stamp = _stamp_path(unit)
+    if not os.path.exists(obj) or not os.path.exists(stamp) or open(stamp).read().strip() != _flags_key(unit):
         return True
     t = os.path.getmtime(obj)
     deps = [os.path.join(CSRC, src), os.path.join(HERE, "..", "include", "rk.h")]
@@ -106,8 +127,8 @@ def _stale(unit) -> bool:
 
 
 def build(jobs: int | None = None, verbose: bool = True, incremental: bool = False) -> str:
-    """Compile and link.  ``incremental`` recompiles only the units whose sources changed (a developer's
-    shortcut; the private-memory check then covers only those units)."""
+    """Compile and link.  ``incremental`` recompiles only the units whose sources or flags changed; every linked object
+    carries a stamp saying that it passed the private-memory check with the current flags."""
     os.makedirs(OBJ, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     units = [u for u in UNITS if _stale(u)] if incremental else list(UNITS)

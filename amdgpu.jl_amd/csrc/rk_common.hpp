@@ -55,7 +55,8 @@ const DeviceInfo& device_info();   // rk_api.hip
 struct WsHeader {
     uint64_t scan_counter;  // look-back scan: epoch << 32 | tile acquisitions of the running call
     uint32_t wait_failed;   // epoch of a call that gave up a bounded wait (see WaitCtl), 0 = none; read by rk_workspace_status
-    uint32_t pad[61];
+    uint32_t alone;         // tiles that stopped waiting and resolved their look-back alone since the workspace was prepared
+    uint32_t pad[60];
 };
 static_assert(sizeof(WsHeader) == 256, "header is one 256-byte line");
 

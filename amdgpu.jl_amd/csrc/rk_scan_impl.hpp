@@ -158,11 +158,104 @@ __device__ __forceinline__ uint32_t gdesc_read(const uint64_t* gd, int64_t g, ui
     return status;
 }
 
+// Forward progress.  A tile that waits depends on workgroups that must be running.  With tile numbers taken from the
+// launch order that holds for one grid alone on the device (workgroups start in index order), but two such grids
+// resident together can in principle starve each other of slots: the lowest unfinished tile of each waiting for a slot
+// that waiting tiles of the other hold.  So no wait here is open-ended: after `wait_patience` unsuccessful polls the
+// tile stops waiting and resolves its prefix ALONE (desc_lookback_alone): whatever a predecessor has not published it
+// computes itself from the input -- `agg_of(p)` returns the aggregate of tile p of the same line, computed by the
+// calling wave -- and publishes in the predecessor's name, so nobody else has to repeat it.  Such a tile needs no other
+// workgroup at all; the call's result is the same (bit for bit for integers; float sums may associate differently, as
+// they do between any two runs).  `helped` counts the tiles that took this path (WsHeader::alone), for tests and
+// curiosity.  The wait budget proper (RK_ERR_WAIT) is left to kernels that cannot help themselves.
+constexpr long long WAIT_PATIENCE = 4096;       // polls (a microsecond or two each) before a tile helps itself
+
+struct WaitAlone {
+    long long patience;      // min(WAIT_PATIENCE, the wait budget): tests set a budget of 1 to send every tile this way
+    uint32_t* counter;       // WsHeader::alone
+};
+__device__ __forceinline__ bool wait_expired(const WaitAlone& w, const WaitCtl& wc, long long& rounds) {
+    if (++rounds >= w.patience) return true;
+    for (int b = 0; b < wc.backoff; ++b) __builtin_amdgcn_s_sleep(8);
+    return false;
+}
+
+// Sum of the aggregates of tiles first .. first + count - 1 (count <= 64) without waiting: missing ones are computed
+// from the input and published.  One full wave; the result is wave-uniform.
+template <typename T, typename Op, typename Agg>
+__device__ __forceinline__ T desc_sum_or_compute(uint64_t* tile_desc, int64_t tstride, int64_t first, int count, uint32_t tagA, uint32_t tagP,
+                                                 Op op, T ident, const Agg& agg_of) {
+    const int lane = lane_id();
+    Words<T> tv = to_words(ident);
+    uint32_t st = DESC_A;
+    if (lane < count) st = desc_read<T>(tile_desc, tstride, first + lane, tagA, tagP, tv);
+    unsigned long long missing = __ballot(st == 0u);
+    T sum = wave_reduce(st == 0u ? ident : from_words<T>(tv), op);
+    while (missing != 0ull) {
+        const int l = __ffsll(missing) - 1;
+        missing &= missing - 1ull;
+        const T a = agg_of(first + l);
+        if (lane == 0) desc_publish(tile_desc, tstride, first + l, a, tagA);
+        sum = op(sum, a);
+    }
+    return sum;
+}
+
+// The exclusive prefix of `tile` with no help from anybody (see above).  One full wave.
+template <typename T, typename Op, typename Agg>
+__device__ __forceinline__ T desc_lookback_alone(uint64_t* tile_desc, int64_t tstride, uint64_t* gd, int64_t tile, int64_t tl, int64_t gl,
+                                              uint32_t epoch, T agg, T init, Op op, T ident, const Agg& agg_of, uint32_t* alone_counter) {
+    const int lane = lane_id();
+    const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
+    const int r = (int)(tl & (WAVE - 1));
+    const int64_t g = tl >> 6;
+    const int64_t t0 = tile - r;
+    if (lane == 0) __hip_atomic_fetch_add(alone_counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    auto group_status = [&](int64_t k, T& value) -> uint32_t {
+        Words<T> gv = to_words(ident);
+        uint32_t st = 0;
+        if (lane == 0) st = gdesc_read<T>(gd, k, tagA, tagP, gv);
+        value = read_lane(from_words<T>(gv), 0);
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)st);
+    };
+    const T local = r > 0 ? desc_sum_or_compute(tile_desc, tstride, t0, r, tagA, tagP, op, ident, agg_of) : ident;
+    if (r == WAVE - 1) {                          // the group's aggregate, unless the descriptor already says as much or more
+        T seen;
+        if (group_status(gl, seen) == 0u && lane == 0) gdesc_publish(gd, gl, op(local, agg), tagA);
+    }
+    T base = init;
+    if (g > 0) {
+        T acc = ident;
+        bool found = false;
+        for (int64_t k = gl - 1; k >= gl - g; --k) {          // the groups of this line in front, nearest first
+            T x;
+            const uint32_t st = group_status(k, x);
+            if (st == DESC_P) {
+                base = op(x, acc);                             // a published prefix contains init
+                found = true;
+                break;
+            }
+            if (st == 0u) {
+                x = desc_sum_or_compute(tile_desc, tstride, t0 - (gl - k) * WAVE, WAVE, tagA, tagP, op, ident, agg_of);
+                T seen;
+                if (group_status(k, seen) == 0u && lane == 0) gdesc_publish(gd, k, x, tagA);
+            }
+            acc = op(x, acc);
+        }
+        if (!found) base = op(init, acc);
+        if (lane == 0) gdesc_publish(gd, gl - 1, base, tagP);  // what the group's leader publishes, for the other tiles of the group
+    }
+    return op(base, local);
+}
+
 // Executed by one full wave; returns the wave-uniform exclusive prefix of `tile` (tl > 0) inside its line.
 //   tl  index of the tile in its line     gl  global index of the tile's group     agg  aggregate of this tile
+// `expired`: the patience ran out; the value returned is then meaningless and the caller resolves the prefix with
+// desc_lookback_alone (one call site, where it can first put registers it holds aside).
 template <typename T, typename Op>
 __device__ __forceinline__ T desc_lookback_leader(uint64_t* tile_desc, int64_t tstride, uint64_t* gd, int64_t tile, int64_t tl, int64_t gl,
-                                                  uint32_t epoch, T agg, T init, Op op, T ident, const WaitCtl& wc) {
+                                                  uint32_t epoch, T agg, T init, Op op, T ident, const WaitCtl& wc, const WaitAlone& wa,
+                                                  bool& expired) {
     const int lane = lane_id();
     const uint32_t tagA = (epoch << 2) | DESC_A, tagP = (epoch << 2) | DESC_P;
     const int r = (int)(tl & (WAVE - 1));           // predecessors inside the group
@@ -191,7 +284,7 @@ __device__ __forceinline__ T desc_lookback_leader(uint64_t* tile_desc, int64_t t
                 grem -= WAVE;
                 continue;
             }
-            if (wait_give_up(wc, rounds)) break;     // `base` is then meaningless
+            if (wait_expired(wa, wc, rounds)) { expired = true; return ident; }
         }
         if (lane == 0) gdesc_publish(gd, gl - 1, base, tagP);
         return base;
@@ -206,7 +299,7 @@ __device__ __forceinline__ T desc_lookback_leader(uint64_t* tile_desc, int64_t t
             local = wave_reduce(from_words<T>(tv), op);
             break;
         }
-        if (wait_give_up(wc, rounds)) break;
+        if (wait_expired(wa, wc, rounds)) { expired = true; return ident; }
     }
     if (r == WAVE - 1 && lane == 0) gdesc_publish(gd, gl, op(local, agg), tagA);
     T base = init;
@@ -220,7 +313,7 @@ __device__ __forceinline__ T desc_lookback_leader(uint64_t* tile_desc, int64_t t
                 base = read_lane(from_words<T>(gv), 0);
                 break;
             }
-            if (wait_give_up(wc, rounds)) break;
+            if (wait_expired(wa, wc, rounds)) { expired = true; return ident; }
         }
     }
     return op(base, local);
@@ -394,6 +487,27 @@ __device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int 
     }
 }
 
+// Aggregate of another tile of the same line, computed from the input by the calling wave (the look-back's way out
+// when that tile's workgroup is not there to publish it: desc_lookback_alone).  Lines of whole, aligned vectors; every
+// tile in front of another is full.
+template <typename In, typename T, typename Op, int TILE> struct ScanTileAggregate {
+    const In* first;        // first element of the asking tile
+    int64_t   tile;         // its number
+    __device__ __forceinline__ T operator()(int64_t p) const {
+        constexpr int VEC = 16 / sizeof(T);
+        typedef typename VecOf<In, VEC>::type VI;
+        const Op op;
+        const In* q = first - (tile - p) * (int64_t)TILE;
+        T acc = Op::template identity<T>();
+        for (int i = lane_id() * VEC; i < TILE; i += WAVE * VEC) {
+            const VI x = *(const VI*)(q + i);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc = op(acc, (T)x[j]);
+        }
+        return wave_reduce(acc, op);
+    }
+};
+
 // ---- contiguous lines that fit one tile: one workgroup per line, no communication ------------------------
 template <typename In, typename T, typename Op, bool VECTOR, int K>
 __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len, T init,
@@ -560,9 +674,11 @@ __device__ __forceinline__ void ordered_finish(uint32_t epoch, int64_t used, uns
 // resident at once, and whether a grid of `nblocks` takes its tile numbers from the counter (see ordered_tile_id).
 int tune_ordered_ids();            // rk_api.hip: 0 = by grid size, 1 = always the launch order, 2 = always the counter
 inline int64_t ordered_resident(int threads) { return (int64_t)device_info().cus * (32 * WAVE / threads); }
-inline int ordered_dynamic_ids(int64_t nblocks, int threads) {
+// `helps_itself`: the kernel's waits end in desc_lookback_alone, so its tiles need nobody and the launch order is safe
+// at any size.
+inline int ordered_dynamic_ids(int64_t nblocks, int threads, bool helps_itself) {
     const int t = tune_ordered_ids();
-    return t == 1 ? 0 : (t == 2 ? 1 : (nblocks > ordered_resident(threads) ? 1 : 0));
+    return t == 1 ? 0 : (t == 2 ? 1 : (!helps_itself && nblocks > ordered_resident(threads) ? 1 : 0));
 }
 // Workgroups per first-level exit ticket: at most half of the ticket lines in use, at least TICKET_GROUP a ticket.
 inline int ordered_ticket_group(int64_t nblocks) {
@@ -592,11 +708,12 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
                                                                     int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                                     unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                     uint64_t* desc, int64_t ngroups_per_line, int64_t ngroups,
-                                                                    int64_t desc_capacity, WaitCtl wc, int stagger_ticks, int stagger_tiles, int dynamic_ids) {
+                                                                    int64_t desc_capacity, WaitCtl wc, WaitAlone wa, int stagger_ticks, int stagger_tiles, int dynamic_ids) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     __shared__ T lds_wave[NW];
     __shared__ T lds_prefix;
+    __shared__ typename VecOf<T, VEC>::type lds_stash[K][WAVE];         // wave 0's registers while it resolves its prefix alone
     const T ident = Op::template identity<T>();
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     uint64_t* tile_desc = desc;                                        // [words][ntiles]
@@ -630,9 +747,24 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
             if (lane < NW) lds_wave[lane] = wave_shift_right(inc, ident);       // what lies in front of each wave inside the tile
             T tile_prefix = init;
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, tile_agg, (epoch << 2) | DESC_A);
-            if (tl > 0)
-                tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tl, line * ngroups_per_line + (tl >> 6), epoch,
-                                                   tile_agg, init, op, ident, wc);
+            if (tl > 0) {
+                // The wave's part of the tile waits in LDS while the wave looks back: the kernel is compiled for 64
+                // registers, the tile takes 32 of them, and the way out of an endless wait (desc_lookback_alone, which
+                // reads other tiles) needs more than the rest -- with the tile in registers the compiler made room in
+                // private memory, inside the tile's scan.  Sixteen LDS accesses a tile, by one wave of sixteen.
+                typedef typename VecOf<T, VEC>::type VT;
+                volatile VT* stash = &lds_stash[0][lane];
+#pragma unroll
+                for (int k = 0; k < K; ++k) stash[k * WAVE] = r.v[k];
+                bool expired = false;
+                const int64_t gl = line * ngroups_per_line + (tl >> 6);
+                tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tl, gl, epoch, tile_agg, init, op, ident, wc, wa, expired);
+                if (expired)
+                    tile_prefix = desc_lookback_alone(tile_desc, ntiles, group_desc, tile, tl, gl, epoch, tile_agg, init, op, ident,
+                                                      ScanTileAggregate<In, T, Op, TILE>{in + e0, tile}, wa.counter);
+#pragma unroll
+                for (int k = 0; k < K; ++k) r.v[k] = stash[k * WAVE];
+            }
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
@@ -1631,6 +1763,7 @@ inline int scan_tile_waves(int64_t mid, size_t esz) {
 }
 int tune_scan_stagger_ticks();  // rk_api.hip: start-up stagger of the ordered scan in 10 ns ticks across the first resident round
 long long wait_budget();        // rk_api.hip: poll rounds a bounded wait may spend (rk_set_wait_budget)
+inline WaitAlone wait_alone(WsHeader* hdr) { const long long b = wait_budget(); return WaitAlone{b < WAIT_PATIENCE ? b : WAIT_PATIENCE, &hdr->alone}; }
 inline WaitCtl wait_ctl(WsHeader* hdr) { return WaitCtl{&hdr->wait_failed, wait_budget(), tune_scan_backoff(), 0u}; }   // stamp: the kernel's epoch
 int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
@@ -1681,7 +1814,7 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
             scan_rows_ordered_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
                 in, out, g, init, inclusive, op, strips, nchains, nslices, (T*)scratch, (unsigned long long*)&ws->hdr->scan_counter,
                 ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr),
-                ordered_dynamic_ids(ntiles, (NW + 1) * WAVE));
+                ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -1754,7 +1887,7 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
             return RK_SUCCESS;
         scan_rows_packed_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
             in, out, g, init, inclusive, op, P, nchains, nslices, (T*)w.partials, (unsigned long long*)&w.hdr->scan_counter, w.tickets,
-            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE));
+            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
         RK_LAUNCH_CHECK();
         *done = true;
     }
@@ -1965,25 +2098,25 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const int64_t gpl = (tpl + WAVE - 1) / WAVE, ngroups = gpl * nlines;
     // 8-byte values and unaligned lines do not fit two workgroups a compute unit; with one, the persistent counter-fed
     // kernel is the faster of the two (cumsum of Int64[2^25]: 96 against 107 us)
-    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || !lines_aligned;
+    // (so do inputs narrower than the values -- Bool counted in Int32: the ordered kernel spills 27 registers for them)
+    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || sizeof(In) != sizeof(T) || !lines_aligned;
     const size_t need = dynamic_ids ? (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t)
                                     : ((size_t)ntiles * Words<T>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const WaitCtl wc = wait_ctl(w.hdr);
-    if constexpr (sizeof(T) <= 4) {
+    if constexpr (sizeof(T) <= 4 && sizeof(In) == sizeof(T)) {
         if (!dynamic_ids) {
-            const int tg = ordered_ticket_group(ntiles);
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
             scan_ordered_kernel<In, T, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
-                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, tg, w.desc, gpl, ngroups, cap, wc, stagger_ticks, stagger_tiles, dyn)
+                in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, ordered_ticket_group(ntiles), w.desc, gpl, ngroups, cap, wc, wait_alone(w.hdr), stagger_ticks, stagger_tiles, dyn)
             // staggered start of the first resident round (two workgroups of 16 waves a compute unit), where more rounds
             // follow: 5 us across the round measured best (2^26 Int32: 0 / 2 / 4 / 6 / 8 / 12 / 16 us -> 91.8 / 90.3 / 89.7 /
             // 89.9 / 90.1 / 90.9 / 92.0 us; 2^27: 177.9 -> 174.0 us; half the round late by a fixed time gained nothing)
             const int64_t resident = ordered_resident(nw * WAVE);
             const int stagger_tiles = (nw == 16 && ntiles >= 2 * resident) ? (int)resident : 0, stagger_ticks = tune_scan_stagger_ticks();
-            const int dyn = ordered_dynamic_ids(ntiles, nw * WAVE);
+            const int dyn = ordered_dynamic_ids(ntiles, nw * WAVE, true);
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED
             RK_LAUNCH_CHECK();

@@ -47,12 +47,33 @@ __device__ __forceinline__ void emit_index(int64_t* __restrict__ ys, int64_t pos
 // ORDERED: one workgroup per tile (its number from the launch order or, for grids beyond what is resident at once, from the
 // counter: ordered_tile_id), the look-back and the end of the call as in scan_ordered_kernel
 // (no tile counter, only the first tile of a group of 64 reads group descriptors, each on a line of its own).
+// Set bytes of another tile, counted by the calling wave (the look-back's way out when that tile's workgroup is not
+// there to publish its count: desc_lookback_alone).  Every tile in front of another is full.
+template <int SEL_TILE> struct SelectTileCount {
+    const uint8_t* bools;
+    int aligned;
+    __device__ __forceinline__ int64_t operator()(int64_t p) const {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const uint8_t* q = bools + p * (int64_t)SEL_TILE;
+        int32_t c = 0;
+        for (int i = lane_id() * 16; i < SEL_TILE; i += WAVE * 16) {
+            if (aligned) {
+                const u32x4 x = *(const u32x4*)(q + i) & 0x01010101u;
+                c += __popc(x[0]) + __popc(x[1]) + __popc(x[2]) + __popc(x[3]);
+            } else {
+                for (int b = 0; b < 16; ++b) c += q[i + b] & 1;
+            }
+        }
+        return (int64_t)wave_reduce(c, OpAdd());
+    }
+};
+
 template <bool LINEAR, bool SMALL, int SEL_NW, int SEL_K, bool ORDERED>
 __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uint8_t* __restrict__ bools, int64_t n, int64_t* __restrict__ ys,
                                                                        int64_t* __restrict__ count_out, SelShape shp, int aligned,
                                                                        unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                        uint64_t* desc, int64_t ntiles, int64_t ngroups, int64_t desc_capacity,
-                                                                       WaitCtl wc, int dynamic_ids) {
+                                                                       WaitCtl wc, WaitAlone wa, int dynamic_ids) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int SEL_TILE = SEL_NW * SEL_CHUNK * SEL_K;
     __shared__ uint16_t lds_strip[SEL_NW][SEL_CHUNK];
@@ -144,10 +165,14 @@ __global__ __launch_bounds__(SEL_NW * WAVE) void findall_select_kernel(const uin
             int64_t tile_prefix = 0;
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, (int64_t)tile_count, (epoch << 2) | DESC_A);
             if (tile > 0) {
-                if constexpr (ORDERED)
+                if constexpr (ORDERED) {
+                    bool expired = false;
                     tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
-                                                       (int64_t)0, op, (int64_t)0, wc);
-                else
+                                                       (int64_t)0, op, (int64_t)0, wc, wa, expired);
+                    if (expired)
+                        tile_prefix = desc_lookback_alone(tile_desc, ntiles, group_desc, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
+                                                          (int64_t)0, op, (int64_t)0, SelectTileCount<SEL_TILE>{bools, aligned}, wa.counter);
+                } else
                     tile_prefix = desc_lookback2(tile_desc, ntiles, group_desc, ngroups, tile, tile, tile >> 6, epoch, (int64_t)tile_count,
                                                  (int64_t)0, op, (int64_t)0, wc);
             }
@@ -279,12 +304,12 @@ extern "C" int32_t rk_findall(const uint8_t* bools, int ndim, const int64_t* sha
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const int aligned = is_aligned(bools, 16) ? 1 : 0;
     const WaitCtl wc = wait_ctl(w.hdr);
-    const int dyn = ordered ? ordered_dynamic_ids(ntiles, nw * WAVE) : 0;
+    const int dyn = ordered ? ordered_dynamic_ids(ntiles, nw * WAVE, true) : 0;
     hipStream_t st = (hipStream_t)stream;
 #define RK_SELECT3(LIN, SM, NWW, KK, ORD)                                                                                        \
     findall_select_kernel<LIN, SM, NWW, KK, ORD><<<(unsigned)grid, NWW * WAVE, 0, st>>>(bools, n, ys, count_out, shp, aligned,      \
                                                                                         counter, w.tickets, tg, w.desc, ntiles,    \
-                                                                                        ngroups, cap, wc, dyn)
+                                                                                        ngroups, cap, wc, wait_alone(w.hdr), dyn)
 #define RK_SELECT2(LIN, SM, KK)                                                                                                  \
     do {                                                                                                                         \
         if (!ordered) RK_SELECT3(LIN, SM, 16, KK, false);                                                                        \

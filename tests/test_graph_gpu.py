@@ -23,8 +23,8 @@ def test_graph_replays_match_oracle(rk, orc):
     rng = np.random.default_rng(41)
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
-        # arrays, workspaces and prepared calls are made before the capture: rk_workspace_init clears with
-        # hipMemsetAsync, which must stay out of a graph
+        # arrays, workspaces and prepared calls are made before the capture: a workspace allocated during a capture
+        # would not belong to the graph (rk_workspace_init itself is a fill kernel and could be captured)
         xf = rk.ROCArray(dims=(n,), dtype=np.float32)
         xi = rk.ROCArray(dims=(n,), dtype=np.int32)
         m2 = rk.ROCArray(dims=shape2, dtype=np.int32)

@@ -1,8 +1,9 @@
 """rk_accumulate_static (bookkeeping in the library's own device array, no workspace argument, no allocation)
-against rk_accumulate on the same inputs, through the C ABI.
+against rk_accumulate on the same inputs AND against the CPU oracle, through the C ABI.
 
-Bar: integer scans bit-exact; Float32 within rtol 1e-4 of each other (both are Float32 scans whose look-back
-association order depends on timing, so they need not agree to the bit).  Every case makes two calls in a row on the
+Bar: integer scans bit-exact (both ways); Float32 within rtol 1e-4 of the oracle's Float64 scan and of each other (both
+are Float32 scans whose look-back association order depends on timing, so they need not agree to the bit).  The calls
+run with torch's allocator watched: the entry point must not change the device memory the process holds.  Every case makes two calls in a row on the
 one shared array, the second on a smaller input, so that state left by the first call would show."""
 import ctypes as C
 
@@ -22,10 +23,23 @@ def _both(rk, x, op="add", dims=1, inclusive=True, init=None, out_dtype=None):
     rk.accumulate_(op, want, A, dims=dims, init=init, inclusive=inclusive)          # rk_accumulate with a caller workspace
     got = rk.ROCArray(dims=A.dims, dtype=out_dtype)
     got.buf.fill_(0xA5)
-    st = L.lib.rk_accumulate_static(_OP[op], A.code, got.code, A.ptr, got.ptr, A.ndim, L.shape_array(A.dims), dims,
-                                    1 if inclusive else 0, _scalar_buffer(init, out_dtype), stream_ptr())
+    ibuf = _scalar_buffer(init, out_dtype)
+    shape = L.shape_array(A.dims)
+    import torch
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    st = L.lib.rk_accumulate_static(_OP[op], A.code, got.code, A.ptr, got.ptr, A.ndim, shape, dims,
+                                    1 if inclusive else 0, ibuf, stream_ptr())
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
     assert st == 0, L.lib.rk_status_string(st)
+    assert free1 == free0, "rk_accumulate_static changed the free device memory: it must not allocate"
     return rk.Array(got), rk.Array(want)
+
+
+def _oracle(orc, x, op="add", dims=1, inclusive=True, init=None, out_dtype=None):
+    xx = x.astype(out_dtype) if out_dtype is not None else x
+    return orc.accumulate(op, xx, dims=dims, init=init, inclusive=inclusive)
 
 
 def _check(got, want):
@@ -48,7 +62,7 @@ CASES = [
 
 @pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64])
 @pytest.mark.parametrize("first,second,dims", CASES)
-def test_static_matches_workspace(rk, first, second, dims, dtype):
+def test_static_matches_workspace(rk, orc, first, second, dims, dtype):
     rng = np.random.default_rng(11)
     for shape in (first, second):
         shape = (shape,) if isinstance(shape, int) else shape
@@ -58,18 +72,21 @@ def test_static_matches_workspace(rk, first, second, dims, dtype):
             x = rng.integers(-1000, 1001, shape).astype(dtype)
         got, want = _both(rk, x, dims=dims)
         _check(got, want)
+        _check(got, _oracle(orc, x, dims=dims).astype(got.dtype))
 
 
-def test_static_exclusive_init_and_bool_counts(rk):
+def test_static_exclusive_init_and_bool_counts(rk, orc):
     rng = np.random.default_rng(12)
     x = rng.integers(-5, 6, 1_000_003).astype(np.int32)
     for n in (x.size, 70_001):
         got, want = _both(rk, x[:n].copy(), op="max", inclusive=False, init=-3)
         _check(got, want)
+        _check(got, _oracle(orc, x[:n], op="max", inclusive=False, init=-3))
     b = rng.random(3_000_000) < 0.3
     for n in (b.size, 100_000):
         got, want = _both(rk, b[:n].copy(), out_dtype=np.int64)
         _check(got, want)
+        assert np.array_equal(got, np.cumsum(b[:n], dtype=np.int64))
         assert got[-1] == np.count_nonzero(b[:n])
 
 
