@@ -35,38 +35,14 @@ def accumulate_(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusi
     return B
 
 
-# 1- and 2-byte element types have no scan kernels of their own (a tile of the scans is laid out in 16-byte vectors of
-# the value type).  They are scanned in the next wider type and stored back: Int8 / Int16 through Int32, UInt8 / UInt16
-# through UInt32 -- sums and products wrap modulo 2^32 and the store keeps the low bits, which is the narrow type's own
-# wrap-around -- and Float16 through Float32 with one rounding at the end (AcceleratedKernels rounds after every step;
-# the contract is a tolerance either way).  Three native kernels instead of one: convert, scan in place, convert.
-_WIDE = {np.dtype(np.int8): np.dtype(np.int32), np.dtype(np.int16): np.dtype(np.int32),
-         np.dtype(np.uint8): np.dtype(np.uint32), np.dtype(np.uint16): np.dtype(np.uint32),
-         np.dtype(np.float16): np.dtype(np.float32)}
-
-
-def _launch_widened(op, B, A, dims, init, inclusive):
-    from .broadcast import lazy, plan_materialize
-    wide = _WIDE[np.dtype(B.dtype)]
-    tmp = ROCArray(dims=A.dims, dtype=wide)
-    widen = plan_materialize(tmp, lazy(A))
-    scan = _launch_accumulate(op, tmp, tmp, dims, init, inclusive)
-    narrow = plan_materialize(B, lazy(tmp))
-
-    def launch():
-        widen()
-        scan()
-        narrow()
-    launch.keepalive = tmp
-    return launch
+# 1- and 2-byte element types (Int8, UInt8, Int16, UInt16, Float16) are scanned by the same kernels as the rest: the
+# library reads them narrow, scans in the next wider type -- sums and products wrap modulo 2^32 and the store keeps the
+# low bits, which is the narrow type's own wrap-around; Float16 in Float32 with one rounding at the store
+# (AcceleratedKernels rounds after every step; the contract is a tolerance either way) -- and stores them narrow.
 
 
 def _launch_accumulate(op, B, A, dims, init, inclusive):
     from .views import ROCView
-    if np.dtype(B.dtype) in _WIDE and np.dtype(A.dtype) != np.bool_ and not isinstance(A, ROCView) and not isinstance(B, ROCView):
-        if np.dtype(A.dtype) != np.dtype(B.dtype):
-            raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"accumulate! from {A.dtype} into {B.dtype}")
-        return _launch_widened(op, B, A, dims, init, inclusive)
     if isinstance(A, ROCView) or isinstance(B, ROCView):
         # wrapper arrays laid out alike (accumulate!(+, transpose(B), transpose(A))): the dims are renumbered in the ABI
         from .mapreduce import _dense_strides

@@ -478,6 +478,12 @@ int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, v
             case RK_I64: return scan_i64(a);
             case RK_U32: return scan_u32(a);
             case RK_U64: return scan_u64(a);
+            // 1- and 2-byte elements: scanned in 32 bits (Float16: in Float32, one rounding at the store), stored narrow
+            case RK_I8:  return scan_i8(a);
+            case RK_U8:  return scan_u8(a);
+            case RK_I16: return scan_i16(a);
+            case RK_U16: return scan_u16(a);
+            case RK_F16: return scan_f16(a);
             default: return RK_ERR_UNSUPPORTED;
         }
     }

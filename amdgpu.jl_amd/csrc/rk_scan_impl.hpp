@@ -349,6 +349,28 @@ template <typename In, typename T> struct ElemVectors<In, T, false> {
     template <int N> static __device__ __forceinline__ void store(In*, typename VecOf<In, N>::type) {}
 };
 
+// ---- stores of scan results ---------------------------------------------------------------------------------------------
+// The kernels compute in T; the array they fill holds Out: T itself, or a narrower type that is scanned in the next
+// wider one -- Int8 / Int16 in Int32, UInt8 / UInt16 in UInt32: the store keeps the low bits, which is the narrow type's
+// own wrap-around for + and * and the value itself for max / min; Float16 in Float32, rounded once at the store.
+template <typename Out, typename T, int N>
+__device__ __forceinline__ void out_store_nt(Out* p, typename VecOf<T, N>::type v) {        // p aligned to N * sizeof(Out)
+    if constexpr (std::is_same<Out, T>::value) store_nt((typename VecOf<T, N>::type*)p, v);
+    else if constexpr (N == 1) *p = (Out)v;
+    else {
+        typename VecOf<Out, N>::type o;
+#pragma unroll
+        for (int j = 0; j < N; ++j) o[j] = (Out)v[j];
+        store_nt((typename VecOf<Out, N>::type*)p, o);
+    }
+}
+// A vector at an element-aligned address: only where the stored type is the computed one, of 4 or 8 bytes.
+template <typename Out, typename T> struct OutElemVectors { static constexpr bool value = std::is_same<Out, T>::value && sizeof(T) >= 4; };
+template <typename Out, typename T, int N>
+__device__ __forceinline__ void out_store_elems(Out* p, typename VecOf<T, N>::type v) {
+    if constexpr (OutElemVectors<Out, T>::value) store_nt_elems<T, N>(p, v);
+}
+
 // The values of a wave's part, loaded into r, scanned in place; returns the total of the part.
 template <typename T, typename Op, int K>
 __device__ __forceinline__ T tile_scan_regs(int inclusive, Op op, TileRegs<T, K>& r) {
@@ -437,21 +459,21 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
 }
 
 // `base`: everything in front of this wave's part (init, earlier tiles, earlier waves).
-template <typename T, typename Op, bool VECTOR, int K, int NW = 4>
-__device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int valid, T base, Op op, const TileRegs<T, K>& r) {
+template <typename Out, typename T, typename Op, bool VECTOR, int K, int NW = 4>
+__device__ __forceinline__ void tile_store(Out* __restrict__ out, int64_t e0, int valid, T base, Op op, const TileRegs<T, K>& r) {
     constexpr int VEC = 16 / sizeof(T);
     constexpr int TILE = NW * WAVE * VEC * K;
     typedef typename VecOf<T, VEC>::type VT;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int woff = wave * (WAVE * VEC * K) + lane * VEC;
     if (VECTOR && valid == TILE) {
-        T* p = out + e0 + woff;
+        Out* p = out + e0 + woff;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             VT o;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
-            store_nt((VT*)(p + k * WAVE * VEC), o);
+            out_store_nt<Out, T, VEC>(p + k * WAVE * VEC, o);
         }
     } else if (VECTOR && valid % VEC == 0) {
 #pragma unroll
@@ -460,20 +482,20 @@ __device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int 
             VT o;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
-            if (idx < valid) store_nt((VT*)(out + e0 + idx), o);
+            if (idx < valid) out_store_nt<Out, T, VEC>(out + e0 + idx, o);
         }
-    } else if (ElemVectors<T, T>::value) {
+    } else if (OutElemVectors<Out, T>::value) {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int idx = woff + k * WAVE * VEC;
             VT o;
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
-            if (idx + VEC <= valid) ElemVectors<T, T>::template store<VEC>(out + e0 + idx, o);
+            if (idx + VEC <= valid) out_store_elems<Out, T, VEC>(out + e0 + idx, o);
             else if (idx < valid) {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j)
-                    if (idx + j < valid) out[e0 + idx + j] = o[j];
+                    if (idx + j < valid) out[e0 + idx + j] = (Out)o[j];
             }
         }
     } else {
@@ -482,7 +504,7 @@ __device__ __forceinline__ void tile_store(T* __restrict__ out, int64_t e0, int 
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
                 const int idx = woff + k * WAVE * VEC + j;
-                if (idx < valid) out[e0 + idx] = op(base, r.v[k][j]);
+                if (idx < valid) out[e0 + idx] = (Out)op(base, r.v[k][j]);
             }
     }
 }
@@ -509,8 +531,8 @@ template <typename In, typename T, typename Op, int TILE> struct ScanTileAggrega
 };
 
 // ---- contiguous lines that fit one tile: one workgroup per line, no communication ------------------------
-template <typename In, typename T, typename Op, bool VECTOR, int K>
-__global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len, T init,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K>
+__global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len, T init,
                                                          int inclusive, Op op) {
     constexpr int NW = 4;
     __shared__ T lds_wave[NW];
@@ -525,7 +547,7 @@ __global__ __launch_bounds__(256) void scan_tiles_kernel(const In* __restrict__ 
 #pragma unroll
     for (int w = 0; w < NW; ++w)
         if (w < wave) wave_prefix = op(wave_prefix, lds_wave[w]);
-    tile_store<T, Op, VECTOR, K>(out, e0, (int)line_len, op(init, wave_prefix), op, r);
+    tile_store<Out, T, Op, VECTOR, K>(out, e0, (int)line_len, op(init, wave_prefix), op, r);
 }
 
 // ---- long contiguous lines: persistent workgroups, single pass, two-level decoupled look-back --------------
@@ -557,8 +579,8 @@ __device__ __forceinline__ void chain_finish(unsigned long long cur, int64_t nti
     if (lane == 0) *counter = (unsigned long long)epoch << 32;
 }
 
-template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
-__global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K, int NW>
+__global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len,
                                                          int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                          unsigned long long* counter, uint64_t* desc, int64_t ngroups_per_line,
                                                          int64_t ngroups, int64_t desc_capacity, WaitCtl wc) {
@@ -604,7 +626,7 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
-        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, wave_prefix), op, r);
+        tile_store<Out, T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, wave_prefix), op, r);
         if (tid == 0) lds_id = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         cur = lds_id;
@@ -703,8 +725,8 @@ inline int ordered_ticket_group(int64_t nblocks) {
 // advances it and clears a rotating slice of unused descriptor slots, like chain_finish.
 // Compiled for 8 waves per SIMD (<= 64 registers); only launched for 4-byte values with aligned lines: 8-byte values
 // hold the same 32 registers of data but scan with twice the temporaries and spilled 20 registers at that limit.
-template <typename In, typename T, typename Op, bool VECTOR, int K, int NW>
-__global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K, int NW>
+__global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len,
                                                                     int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                                     unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                     uint64_t* desc, int64_t ngroups_per_line, int64_t ngroups,
@@ -768,7 +790,7 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
-        tile_store<T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
+        tile_store<Out, T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
     }
     ordered_finish(epoch, (int64_t)Words<T>::N * ntiles + ngroups * GROUP_DESC_STRIDE, counter, tickets, ticket_group, desc, desc_capacity);
 }
@@ -778,10 +800,10 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
 // still take 16 bytes each -- global memory accepts that at any element-aligned address -- and only the vector the
 // line's end cuts goes element by element (cumsum(A; dims=1) of 257 x 240000 Float32: 143 us with one element a
 // lane, 100 us).
-template <typename In, typename T, typename Op, bool VECTOR, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int64_t line_len,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len,
                                                                 int64_t nlines, T init, int inclusive, Op op) {
-    constexpr bool ELEMS = !VECTOR && ElemVectors<In, T>::value;        // vectors at element-aligned addresses
+    constexpr bool ELEMS = !VECTOR && ElemVectors<In, T>::value && OutElemVectors<Out, T>::value;        // vectors at element-aligned addresses
     constexpr int VEC = (VECTOR || ELEMS) ? 16 / sizeof(T) : 1;
     typedef typename VecOf<T, VEC>::type VT;
     typedef typename VecOf<In, VEC>::type VI;
@@ -819,7 +841,7 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
         carry = op(carry, read_lane(inc, WAVE - 1));
         if (i0 < line_len) {
             if constexpr (VEC == 1) {
-                out[base + i0] = inclusive ? op(off, v[0]) : off;
+                out[base + i0] = (Out)(inclusive ? op(off, v[0]) : off);
             } else {
                 VT o;
                 if (inclusive) {
@@ -831,12 +853,12 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
                     for (int j = 1; j < VEC; ++j) o[j] = op(off, v[j - 1]);
                 }
                 if (whole) {
-                    if constexpr (ELEMS) ElemVectors<T, T>::template store<VEC>(out + base + i0, o);
-                    else store_nt((VT*)(out + base + i0), o);
+                    if constexpr (ELEMS) out_store_elems<Out, T, VEC>(out + base + i0, o);
+                    else out_store_nt<Out, T, VEC>(out + base + i0, o);
                 } else {
 #pragma unroll
                     for (int j = 0; j < VEC; ++j)
-                        if (i0 + j < line_len) out[base + i0 + j] = o[j];
+                        if (i0 + j < line_len) out[base + i0 + j] = (Out)o[j];
                 }
             }
         }
@@ -844,8 +866,8 @@ __global__ __launch_bounds__(BLOCK) void scan_wave_lines_kernel(const In* __rest
 }
 
 // ---- one lane per line (tiny lines, or narrow `inner`) ---------------------------------------------
-template <typename In, typename T, typename Op, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
+template <typename In, typename T, typename Out, typename Op, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict__ in, Out* __restrict__ out, ScanGeom g, T init,
                                                             int inclusive, Op op) {
     const int64_t line = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
     if (line >= g.inner * g.outer) return;
@@ -854,8 +876,8 @@ __global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict
     T acc = init;
     for (int64_t m = 0; m < g.mid; ++m) {
         const T x = (T)in[base + m * g.inner];
-        if (inclusive) { acc = op(acc, x); out[base + m * g.inner] = acc; }
-        else { out[base + m * g.inner] = acc; acc = op(acc, x); }
+        if (inclusive) { acc = op(acc, x); out[base + m * g.inner] = (Out)acc; }
+        else { out[base + m * g.inner] = (Out)acc; acc = op(acc, x); }
     }
 }
 
@@ -866,8 +888,8 @@ __global__ __launch_bounds__(BLOCK) void scan_thread_kernel(const In* __restrict
 // vector totals are scanned over the lanes of the line by shuffles that never cross a line start.  One lane per
 // line with whole vectors reaches 1 TB/s on the same shape, one lane per line with scalars half of that
 // (cumsum of 16 x 1_000_000 Float32 along dim 1: 231 us -> 128 us -> 42 us).
-template <typename In, typename T, typename Op, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int L, int64_t nlines,
+template <typename In, typename T, typename Out, typename Op, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __restrict__ in, Out* __restrict__ out, int L, int64_t nlines,
                                                                  T init, int inclusive, Op op) {
     constexpr int VEC = 16 / sizeof(T), U = 4;
     typedef typename VecOf<In, VEC>::type VI;
@@ -904,7 +926,7 @@ __global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __res
         VT o;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) o[j] = inclusive ? op(base, loc[j]) : (j == 0 ? base : op(base, loc[j > 0 ? j - 1 : 0]));
-        if (live[u]) store_nt((VT*)out + vecidx[u], o);
+        if (live[u]) out_store_nt<Out, T, VEC>(out + vecidx[u] * VEC, o);
     }
 }
 
@@ -919,8 +941,8 @@ __global__ __launch_bounds__(BLOCK) void scan_short_lines_kernel(const In* __res
 // with 16-byte stores.
 constexpr int SCAN_LDS_LINES_MAX = 128;     // contiguous lines beyond, and whole vectors beyond 64: a wave per line does as well or better
 
-template <typename In, typename T, typename Op, bool VECTOR>
-__global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restrict__ in, T* __restrict__ out, int inner, int m, int64_t nslabs,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR>
+__global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restrict__ in, Out* __restrict__ out, int inner, int m, int64_t nslabs,
                                                              int slabs_per_block, int tpl_log2, T init, int inclusive, Op op) {
     constexpr int TE = 16384 / sizeof(T);
     __shared__ __attribute__((aligned(16))) T lds[TE];
@@ -931,7 +953,7 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
     const int ns = left < slabs_per_block ? (int)left : slabs_per_block;     // > 0 by the grid size
     const int ne = ns * slab;                                                 // <= TE by the choice of slabs_per_block
     const In* p = in + slab0 * slab;
-    T* q = out + slab0 * slab;
+    Out* q = out + slab0 * slab;
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
     typedef typename VecOf<In, VEC>::type VI;
     typedef typename VecOf<T, VEC>::type VT;
@@ -1008,14 +1030,14 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
     }
     __syncthreads();
     if constexpr (VEC == 1) {
-        for (int i = t; i < nv; i += 256) q[i] = lds[i];
+        for (int i = t; i < nv; i += 256) q[i] = (Out)lds[i];
     } else {
         constexpr int ROUNDS = TE / VEC / 256;
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r)
-            if (t + r * 256 < nv) store_nt((VT*)q + t + r * 256, ((const VT*)lds)[t + r * 256]);
+            if (t + r * 256 < nv) out_store_nt<Out, T, VEC>(q + (t + r * 256) * VEC, ((const VT*)lds)[t + r * 256]);
     }
-    for (int e = nv * VEC + t; e < ne; e += 256) q[e] = lds[e];
+    for (int e = nv * VEC + t; e < ne; e += 256) q[e] = (Out)lds[e];
 }
 
 // ---- 1 < inner < 64 with long lines: tiles of whole rows through LDS ----------------------------------
@@ -1031,8 +1053,8 @@ __global__ __launch_bounds__(256) void scan_lds_lines_kernel(const In* __restric
 // accumulate(+, 7 x 4_194_304 Float32; dims=2) 62 + 96 us for the two passes, now 24 + 46.)  `in` may be `out` (a tile is in LDS whole before any of it is written).
 template <typename T> struct NarrowTile { static constexpr int ELEMS = sizeof(T) >= 8 ? 4096 : 8192; };
 
-template <typename In, typename T, typename Op, bool TOTALS, bool VECTOR>
-__global__ __launch_bounds__(256) void scan_narrow_kernel(const In* in, T* out, ScanGeom g, int inclusive, Op op,
+template <typename In, typename T, typename Out, typename Op, bool TOTALS, bool VECTOR>
+__global__ __launch_bounds__(256) void scan_narrow_kernel(const In* in, Out* out, ScanGeom g, int inclusive, Op op,
                                                           int64_t rows_per_tile, T* carry, T init) {
     constexpr int ELEMS = NarrowTile<T>::ELEMS;
     constexpr int VEC = 16 / sizeof(T), ROUNDS = ELEMS / VEC / 256;
@@ -1125,9 +1147,9 @@ __global__ __launch_bounds__(256) void scan_narrow_kernel(const In* in, T* out, 
         if constexpr (VECTOR) {
 #pragma unroll
             for (int r = 0; r < ROUNDS; ++r)
-                if (tid + r * 256 < nv) store_nt((VT*)(out + base) + tid + r * 256, ((const VT*)tile)[tid + r * 256]);
+                if (tid + r * 256 < nv) out_store_nt<Out, T, VEC>(out + base + (tid + r * 256) * VEC, ((const VT*)tile)[tid + r * 256]);
         }
-        for (int e = nv * VEC + tid; e < count; e += 256) out[base + e] = tile[e];
+        for (int e = nv * VEC + tid; e < count; e += 256) out[base + e] = (Out)tile[e];
     }
 }
 
@@ -1139,8 +1161,8 @@ __global__ __launch_bounds__(256) void scan_narrow_kernel(const In* in, T* out, 
 // exclusive prefix of every (slice, column) comes from `carry_in` (scan_strided_totals_kernel + a scan of the
 // totals), which makes the slices independent: 12 instead of 8 bytes per element, but thousands of workgroups
 // instead of one per strip.
-template <typename In, typename T, typename Op, bool VECTOR, int R>
-__global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int R>
+__global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict__ in, Out* __restrict__ out, ScanGeom g, T init,
                                                            int inclusive, Op op, int64_t rows_per_slice,
                                                            const T* __restrict__ carry_in, int64_t carry_pitch, int64_t strips) {
     constexpr int VEC = VECTOR ? 16 / sizeof(T) : 1;
@@ -1155,7 +1177,7 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
     // last vector of such a row starts VEC elements before the row's end instead of running into the next row: its
     // leading columns are scanned, and stored, by the lane before as well, with the same values.  Column totals are
     // kept per lane slot (`nominal`), which is the column for every other lane.
-    constexpr bool ANY_ALIGN = VECTOR && sizeof(In) >= 4 && sizeof(T) >= 4;
+    constexpr bool ANY_ALIGN = VECTOR && sizeof(In) >= 4 && OutElemVectors<Out, T>::value;
     const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
     const bool live = nominal < g.inner;
     const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
@@ -1217,8 +1239,8 @@ __global__ __launch_bounds__(256) void scan_strided_kernel(const In* __restrict_
                     for (int j = 0; j < VEC; ++j)
                         o[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r - 1][j]));
                 }
-                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + slab + (row0 + r) * g.inner + col0, o);
-                else store_nt((VT*)(out + slab + (row0 + r) * g.inner + col0), o);
+                if constexpr (ANY_ALIGN) out_store_elems<Out, T, VEC>(out + slab + (row0 + r) * g.inner + col0, o);
+                else out_store_nt<Out, T, VEC>(out + slab + (row0 + r) * g.inner + col0, o);
             }
         }
     }
@@ -1293,8 +1315,8 @@ __global__ __launch_bounds__(256) void scan_strided_totals_kernel(const In* __re
 // A lane owns VEC adjacent columns of one outer index and walks the <= 16 rows, loads four rows ahead; 16-byte accesses
 // at element-aligned addresses, the last group of a row starting VEC columns before the row's end (it stores what the
 // group before stores, the same values).  4- and 8-byte elements.
-template <typename In, typename T, typename Op>
-__global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init, int inclusive,
+template <typename In, typename T, typename Out, typename Op>
+__global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ in, Out* __restrict__ out, ScanGeom g, T init, int inclusive,
                                                         Op op, int64_t groups_per_row, int64_t ngroups) {
     constexpr int VEC = 16 / sizeof(T);
     typedef typename VecOf<In, VEC>::type VI;
@@ -1321,7 +1343,7 @@ __global__ __launch_bounds__(256) void scan_cols_kernel(const In* __restrict__ i
                     o4[j] = inclusive ? nxt : run[j];
                     run[j] = nxt;
                 }
-                ElemVectors<T, T>::template store<VEC>(out + base + (m0 + u) * g.inner, o4);
+                out_store_elems<Out, T, VEC>(out + base + (m0 + u) * g.inner, o4);
             }
         }
     }
@@ -1527,8 +1549,8 @@ __device__ __forceinline__ void rows_lookback(const T (&tot)[VEC], T (&base)[VEC
 // NW waves hold rows; one more wave holds none and does the publishing and the look-back.  The registers a kernel
 // needs are the maximum over its branches, so the row data (32 registers) and the look-back's working set no longer
 // add up: 64 registers suffice and two workgroups share a compute unit (with wave 0 doing both, 25 registers spilled).
-template <typename In, typename T, typename Op, int NW, int R>
-__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(const In* __restrict__ in, T* __restrict__ out, ScanGeom g, T init,
+template <typename In, typename T, typename Out, typename Op, int NW, int R>
+__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(const In* __restrict__ in, Out* __restrict__ out, ScanGeom g, T init,
                                                                                int inclusive, Op op, int64_t strips, int64_t nchains,
                                                                                int64_t nslices, T* payload, unsigned long long* counter,
                                                                                uint32_t* tickets, int ticket_group, uint64_t* desc,
@@ -1564,7 +1586,7 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
         const int64_t o = chain / strips, strip = chain - o * strips;
         // rows that are no whole number of vectors: the last vector starts VEC elements before the row's end (see
         // scan_strided_kernel); payloads are per lane slot, the same columns in every tile of the strip
-        constexpr bool ANY_ALIGN = sizeof(In) >= 4 && sizeof(T) >= 4;
+        constexpr bool ANY_ALIGN = sizeof(In) >= 4 && OutElemVectors<Out, T>::value;
         const int64_t nominal = strip * COLS + (int64_t)lane * VEC;
         const bool live = nominal < g.inner;
         const int64_t col0 = (ANY_ALIGN && live && nominal + VEC > g.inner) ? g.inner - VEC : nominal;
@@ -1615,8 +1637,8 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
                 VT o4;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o4[j] = inclusive ? op(pre[j], v[r][j]) : (r == 0 ? pre[j] : op(pre[j], v[r > 0 ? r - 1 : 0][j]));
-                if constexpr (ANY_ALIGN) store_nt_elems<T, VEC>(out + wave_e0 + r * g.inner + loff, o4);
-                else store_nt((VT*)(out + wave_e0 + r * g.inner + loff), o4);
+                if constexpr (ANY_ALIGN) out_store_elems<Out, T, VEC>(out + wave_e0 + r * g.inner + loff, o4);
+                else out_store_nt<Out, T, VEC>(out + wave_e0 + r * g.inner + loff, o4);
             }
         }
     }
@@ -1634,8 +1656,8 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_ordered_kernel(c
 // 244 us, of which 100 us for the cross-lane moves.)  The rest is scan_rows_ordered_kernel with a tile of NW * R * Q rows
 // and one chain per outer index.  `in` may be `out`: the columns that two lanes hold twice belong to lanes of the same
 // load instruction, which is complete before the wave's first store.
-template <typename In, typename T, typename Op, int NW, int R>
-__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(const In* in, T* out, ScanGeom g, T init, int inclusive, Op op,
+template <typename In, typename T, typename Out, typename Op, int NW, int R>
+__global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(const In* in, Out* out, ScanGeom g, T init, int inclusive, Op op,
                                                                               int P, int64_t nchains, int64_t nslices, T* payload,
                                                                               unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                               uint64_t* desc, int64_t desc_capacity, WaitCtl wc, int dynamic_ids) {
@@ -1738,7 +1760,7 @@ __global__ __launch_bounds__((NW + 1) * WAVE, 8) void scan_rows_packed_kernel(co
                 VT o4;
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) o4[j] = op(pre[j], v[r][j]);
-                store_nt_elems<T, VEC>(out + wave_e0 + (off0 + (unsigned)(r * inner)), o4);
+                out_store_elems<Out, T, VEC>(out + wave_e0 + (off0 + (unsigned)(r * inner)), o4);
             }
         }
     }
@@ -1785,8 +1807,8 @@ struct ScanArgs {
 // the slices scan independently from their carried-in prefix: 12 bytes per element, but the whole device works.
 // Short slices are deliberate: workgroups that are resident together then cover a compact range of rows, which
 // the memory system serves faster than many rows far apart (measured with power-of-two row strides).
-template <typename In, typename T, typename Op>
-inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, bool aligned, char* scratch,
+template <typename In, typename T, typename Out, typename Op>
+inline int32_t scan_across_rows(const In* in, Out* out, const ScanGeom& g, T init, int inclusive, Op op, bool aligned, char* scratch,
                                 size_t scratch_bytes, hipStream_t stream, const Workspace* ws = nullptr) {
     constexpr int VEC = 16 / sizeof(T);
     // 4- and 8-byte elements: vectors at any element-aligned address, rows of any length (>= 64 here)
@@ -1794,7 +1816,7 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     // already overwritten with results: whole-vector rows only)
     const bool in_place = (const void*)in == (const void*)out;
     const bool vec = (sizeof(In) >= 4 && sizeof(T) >= 4 && !(in_place && g.inner % VEC != 0))
-                         ? (is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) && g.inner >= VEC)
+                         ? (is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(Out)) && g.inner >= VEC)
                          : (aligned && g.inner % VEC == 0);
     const int cols = WAVE * (vec ? VEC : 1);
     const int64_t strips = (g.inner + cols - 1) / cols;
@@ -1811,7 +1833,7 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
         const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
         if (vec && ws != nullptr && tune_scan_rows_ordered() != 0 && nchains < cus * 4 && nslices >= 4 &&
             (size_t)((ntiles + 2 * ngroups) * cols) * sizeof(T) <= scratch_bytes && (size_t)(ntiles + ngroups) * sizeof(uint64_t) <= ws->desc_bytes) {
-            scan_rows_ordered_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
+            scan_rows_ordered_kernel<In, T, Out, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
                 in, out, g, init, inclusive, op, strips, nchains, nslices, (T*)scratch, (unsigned long long*)&ws->hdr->scan_counter,
                 ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr),
                 ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
@@ -1831,8 +1853,8 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     }
     if (slices <= 1) {
         dim3 grid((unsigned)(strips * g.outer), 1);
-        if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
-        else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
+        if (vec) scan_strided_kernel<In, T, Out, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
+        else     scan_strided_kernel<In, T, Out, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, g.mid, nullptr, 0, strips);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
@@ -1849,26 +1871,26 @@ inline int32_t scan_across_rows(const In* in, T* out, const ScanGeom& g, T init,
     // totals are 16-byte aligned and pitch % VEC == 0
     const ScanGeom tg{pitch, slices, g.outer};
     if (slices > 128) {
-        const int32_t st = scan_across_rows<T, T, Op>(totals, totals, tg, init, 0, op, true, scratch + used,
+        const int32_t st = scan_across_rows<T, T, T, Op>(totals, totals, tg, init, 0, op, true, scratch + used,
                                                       used < scratch_bytes ? scratch_bytes - used : 0, stream);
         if (st != RK_SUCCESS) return st;
     } else {
         const int tcols = WAVE * VEC;
         const int64_t tstrips = (pitch + tcols - 1) / tcols;
         dim3 tgrid((unsigned)(tstrips * g.outer), 1);
-        scan_strided_kernel<T, T, Op, true, 8><<<tgrid, 256, 0, stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0, tstrips);
+        scan_strided_kernel<T, T, T, Op, true, 8><<<tgrid, 256, 0, stream>>>(totals, totals, tg, init, 0, op, slices, nullptr, 0, tstrips);
         RK_LAUNCH_CHECK();
     }
-    if (vec) scan_strided_kernel<In, T, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
-    else     scan_strided_kernel<In, T, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
+    if (vec) scan_strided_kernel<In, T, Out, Op, true, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
+    else     scan_strided_kernel<In, T, Out, Op, false, 8><<<grid, 256, 0, stream>>>(in, out, g, init, inclusive, op, rps, totals, pitch, strips);
     RK_LAUNCH_CHECK();
     return RK_SUCCESS;
 }
 
 // Scan along `mid` for VEC <= inner <= 32 * VEC in one pass (see scan_rows_packed_kernel).  *done stays false when the
 // shape or the workspace does not fit: the caller then takes another path.
-template <typename In, typename T, typename Op>
-inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, const Workspace& w, hipStream_t stream,
+template <typename In, typename T, typename Out, typename Op>
+inline int32_t scan_rows_packed(const In* in, Out* out, const ScanGeom& g, T init, int inclusive, Op op, const Workspace& w, hipStream_t stream,
                                 bool* done) {
     *done = false;
     if constexpr (ElemVectors<In, T>::value) {
@@ -1876,7 +1898,7 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
         constexpr int NW = 15, R = 8;              // (ten rows per lane group: 63 x 500_000 Float32 71 -> 79 us)
         // (rows shorter than a 128-byte line: a load instruction then takes Q short pieces R rows apart, and the two-pass
         // tiles through LDS are two to three times faster: 7 x 4_194_304 Float32 265 against 83 us)
-        if (g.inner * sizeof(In) < 128 || g.inner * 2 > COLS || !is_aligned(in, sizeof(In)) || !is_aligned(out, sizeof(T))) return RK_SUCCESS;
+        if (g.inner * sizeof(In) < 128 || g.inner * 2 > COLS || !is_aligned(in, sizeof(In)) || !is_aligned(out, sizeof(Out))) return RK_SUCCESS;
         const int P = (int)((g.inner + VEC - 1) / VEC), Q = WAVE / P;
         const int64_t tile_rows = (int64_t)NW * R * Q;
         const int64_t nchains = g.outer, nslices = (g.mid + tile_rows - 1) / tile_rows;
@@ -1885,7 +1907,7 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
         const int64_t ngroups = (nslices + ROWS_GROUP - 1) / ROWS_GROUP * nchains;
         if ((size_t)((ntiles + 2 * ngroups) * COLS) * sizeof(T) > WS_PARTIALS_BYTES || (size_t)(ntiles + ngroups) * sizeof(uint64_t) > w.desc_bytes)
             return RK_SUCCESS;
-        scan_rows_packed_kernel<In, T, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
+        scan_rows_packed_kernel<In, T, Out, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
             in, out, g, init, inclusive, op, P, nchains, nslices, (T*)w.partials, (unsigned long long*)&w.hdr->scan_counter, w.tickets,
             ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
         RK_LAUNCH_CHECK();
@@ -1896,14 +1918,14 @@ inline int32_t scan_rows_packed(const In* in, T* out, const ScanGeom& g, T init,
 
 // Scan along `mid` for 1 < inner < 64 (see scan_narrow_kernel).  Returns false when the tile totals do not fit the
 // scratch area: the caller then takes another path.
-template <typename In, typename T, typename Op>
-inline int32_t scan_narrow(const In* in, T* out, const ScanGeom& g, T init, int inclusive, Op op, char* scratch, size_t scratch_bytes,
+template <typename In, typename T, typename Out, typename Op>
+inline int32_t scan_narrow(const In* in, Out* out, const ScanGeom& g, T init, int inclusive, Op op, char* scratch, size_t scratch_bytes,
                            hipStream_t stream, bool* done) {
     *done = false;
     constexpr int VEC = 16 / (int)sizeof(T);
     int64_t rows_per_tile = NarrowTile<T>::ELEMS / g.inner;
     // tiles that start at whole vectors: rows_per_tile * inner, and the slab of one outer index, multiples of the vector
-    const bool vec = is_aligned(in, VEC * sizeof(In)) && is_aligned(out, 16) && rows_per_tile >= VEC &&
+    const bool vec = is_aligned(in, VEC * sizeof(In)) && is_aligned(out, VEC * sizeof(Out)) && rows_per_tile >= VEC &&
                      (g.outer == 1 || (g.inner * g.mid) % VEC == 0);
     if (vec) rows_per_tile -= rows_per_tile % VEC;
     const int64_t tiles = (g.mid + rows_per_tile - 1) / rows_per_tile;
@@ -1913,46 +1935,46 @@ inline int32_t scan_narrow(const In* in, T* out, const ScanGeom& g, T init, int 
     if (scratch == nullptr || used > scratch_bytes) return RK_SUCCESS;
     T* totals = (T*)scratch;
     dim3 grid((unsigned)tiles, (unsigned)g.outer);
-    if (vec) scan_narrow_kernel<In, T, Op, true, true><<<grid, 256, 0, stream>>>(in, nullptr, g, inclusive, op, rows_per_tile, totals, init);
-    else scan_narrow_kernel<In, T, Op, true, false><<<grid, 256, 0, stream>>>(in, nullptr, g, inclusive, op, rows_per_tile, totals, init);
+    if (vec) scan_narrow_kernel<In, T, Out, Op, true, true><<<grid, 256, 0, stream>>>(in, nullptr, g, inclusive, op, rows_per_tile, totals, init);
+    else scan_narrow_kernel<In, T, Out, Op, true, false><<<grid, 256, 0, stream>>>(in, nullptr, g, inclusive, op, rows_per_tile, totals, init);
     RK_LAUNCH_CHECK();
     // exclusive scan of the totals along the tiles, seeded with init: the (inner, tiles, outer) problem again
     const ScanGeom tg{g.inner, tiles, g.outer};
     if (tiles * g.inner <= NarrowTile<T>::ELEMS && tiles > 32) {
         // all tile totals of an outer index fit one tile: one workgroup each scans them in place
-        scan_narrow_kernel<T, T, Op, false, false><<<dim3(1, (unsigned)g.outer), 256, 0, stream>>>(totals, totals, tg, 0, op, tiles, nullptr, init);
+        scan_narrow_kernel<T, T, T, Op, false, false><<<dim3(1, (unsigned)g.outer), 256, 0, stream>>>(totals, totals, tg, 0, op, tiles, nullptr, init);
         RK_LAUNCH_CHECK();
     } else {
         bool sub = false;
         if (tiles > 32) {              // a lane per column walking more tiles than this is slower than three small launches
-            const int32_t st = scan_narrow<T, T, Op>(totals, totals, tg, init, 0, op, scratch + used, scratch_bytes - used, stream, &sub);
+            const int32_t st = scan_narrow<T, T, T, Op>(totals, totals, tg, init, 0, op, scratch + used, scratch_bytes - used, stream, &sub);
             if (st != RK_SUCCESS) return st;
         }
         if (!sub) {
             const int64_t blocks = (g.inner * g.outer + 255) / 256;
-            scan_thread_kernel<T, T, Op, 256><<<(unsigned)blocks, 256, 0, stream>>>(totals, totals, tg, init, 0, op);
+            scan_thread_kernel<T, T, T, Op, 256><<<(unsigned)blocks, 256, 0, stream>>>(totals, totals, tg, init, 0, op);
             RK_LAUNCH_CHECK();
         }
     }
-    if (vec) scan_narrow_kernel<In, T, Op, false, true><<<grid, 256, 0, stream>>>(in, out, g, inclusive, op, rows_per_tile, totals, init);
-    else scan_narrow_kernel<In, T, Op, false, false><<<grid, 256, 0, stream>>>(in, out, g, inclusive, op, rows_per_tile, totals, init);
+    if (vec) scan_narrow_kernel<In, T, Out, Op, false, true><<<grid, 256, 0, stream>>>(in, out, g, inclusive, op, rows_per_tile, totals, init);
+    else scan_narrow_kernel<In, T, Out, Op, false, false><<<grid, 256, 0, stream>>>(in, out, g, inclusive, op, rows_per_tile, totals, init);
     RK_LAUNCH_CHECK();
     *done = true;
     return RK_SUCCESS;
 }
 
-template <typename In, typename T, typename Op>
+template <typename In, typename T, typename Out, typename Op>
 inline int32_t launch_scan(const ScanArgs& a) {
     const Op op;
-    const T init = a.init ? *(const T*)a.init : Op::template identity<T>();
+    const T init = a.init ? (T)*(const Out*)a.init : Op::template identity<T>();      // `init` has the output's element type
     const In* in = (const In*)a.in;
-    T* out = (T*)a.out;
+    Out* out = (Out*)a.out;
     const uint32_t mask = (a.dim >= 1 && a.dim <= a.ndim) ? (1u << (a.dim - 1)) : 0u;
     const Shape3 s = collapse3(a.ndim, a.shape, mask);
     if (s.total == 0) return RK_SUCCESS;
     ScanGeom g{s.inner, s.mid, s.outer};
     constexpr int VEC = 16 / sizeof(T);
-    const bool aligned = is_aligned(in, VEC * sizeof(In)) && is_aligned(out, 16);
+    const bool aligned = is_aligned(in, VEC * sizeof(In)) && is_aligned(out, VEC * sizeof(Out));
     const int inclusive = a.inclusive ? 1 : 0;
 
     {
@@ -1988,9 +2010,9 @@ inline int32_t launch_scan(const ScanArgs& a) {
                 const int64_t blocks = (s.outer + spb - 1) / spb;
                 if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
                 if (vector)
-                    scan_lds_lines_kernel<In, T, Op, true><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
+                    scan_lds_lines_kernel<In, T, Out, Op, true><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
                 else
-                    scan_lds_lines_kernel<In, T, Op, false><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
+                    scan_lds_lines_kernel<In, T, Out, Op, false><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, (int)s.inner, (int)s.mid, s.outer, spb, tl, init, inclusive, op);
                 RK_LAUNCH_CHECK();
                 return RK_SUCCESS;
             }
@@ -1998,13 +2020,13 @@ inline int32_t launch_scan(const ScanArgs& a) {
     }
     if constexpr (ElemVectors<In, T>::value) {
         // (not in place with rows that are no whole vectors: the row's last group re-reads columns of the group before)
-        if (s.inner >= 64 && s.mid <= 16 && s.inner * s.outer >= 4096 && is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(T)) &&
+        if (s.inner >= 64 && s.mid <= 16 && s.inner * s.outer >= 4096 && is_aligned(in, sizeof(In)) && is_aligned(out, sizeof(Out)) &&
             !((const void*)in == (const void*)out && s.inner % VEC != 0)) {
             const int64_t groups_per_row = (s.inner + VEC - 1) / VEC;
             if (groups_per_row > INT64_MAX / s.outer) return RK_ERR_TOO_LARGE;
             const int64_t ngroups = groups_per_row * s.outer, blocks = (ngroups + 255) / 256;
             if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-            scan_cols_kernel<In, T, Op><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, groups_per_row, ngroups);
+            scan_cols_kernel<In, T, Out, Op><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, g, init, inclusive, op, groups_per_row, ngroups);
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -2016,11 +2038,11 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const bool have_ws = carve_workspace(a.ws, a.ws_bytes, 0, &w);
         if (have_ws && tune_scan_rows_packed() != 0) {      // rows of at most half a strip of columns
             bool done = false;
-            const int32_t st = scan_rows_packed<In, T, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
+            const int32_t st = scan_rows_packed<In, T, Out, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
             if (st != RK_SUCCESS || done) return st;
         }
         if (have_ws) { scratch = (char*)w.partials; scratch_bytes = WS_PARTIALS_BYTES; }
-        return scan_across_rows<In, T, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream, have_ws ? &w : nullptr);
+        return scan_across_rows<In, T, Out, Op>(in, out, g, init, inclusive, op, aligned, scratch, scratch_bytes, a.stream, have_ws ? &w : nullptr);
     }
     const int64_t nlines = s.inner * s.outer;
     if (s.inner > 1 && s.mid > 64) {
@@ -2030,10 +2052,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
         if (carve_workspace(a.ws, a.ws_bytes, 0, &w)) {
             bool done = false;
             if (tune_scan_rows_packed() != 0) {
-                const int32_t st = scan_rows_packed<In, T, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
+                const int32_t st = scan_rows_packed<In, T, Out, Op>(in, out, g, init, inclusive, op, w, a.stream, &done);
                 if (st != RK_SUCCESS || done) return st;
             }
-            const int32_t st = scan_narrow<In, T, Op>(in, out, g, init, inclusive, op, (char*)w.partials, WS_PARTIALS_BYTES, a.stream, &done);
+            const int32_t st = scan_narrow<In, T, Out, Op>(in, out, g, init, inclusive, op, (char*)w.partials, WS_PARTIALS_BYTES, a.stream, &done);
             if (st != RK_SUCCESS || done) return st;
         }
     }
@@ -2042,14 +2064,14 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const int64_t per_block = (int64_t)4 * 4 * (64 / L);            // waves x steps x lines per wave and step
         const int64_t blocks = (nlines + per_block - 1) / per_block;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-        scan_short_lines_kernel<In, T, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, L, nlines, init, inclusive, op);
+        scan_short_lines_kernel<In, T, Out, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, L, nlines, init, inclusive, op);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
     if (s.inner > 1 || s.mid <= 16) {
         const int64_t blocks = (nlines + 255) / 256;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-        scan_thread_kernel<In, T, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, g, init, inclusive, op);
+        scan_thread_kernel<In, T, Out, Op, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, g, init, inclusive, op);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
@@ -2059,9 +2081,9 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const int64_t blocks = (nlines + 3) / 4;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
         if (lines_aligned && s.mid % VEC == 0)
-            scan_wave_lines_kernel<In, T, Op, true, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
+            scan_wave_lines_kernel<In, T, Out, Op, true, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
         else
-            scan_wave_lines_kernel<In, T, Op, false, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
+            scan_wave_lines_kernel<In, T, Out, Op, false, 256><<<(unsigned)blocks, 256, 0, a.stream>>>(in, out, s.mid, nlines, init, inclusive, op);
         RK_LAUNCH_CHECK();
         return RK_SUCCESS;
     }
@@ -2071,8 +2093,8 @@ inline int32_t launch_scan(const ScanArgs& a) {
         const unsigned grid = (unsigned)nlines;
 #define RK_SCAN_TILES(KK)                                                                                             \
         do {                                                                                                          \
-            if (lines_aligned) scan_tiles_kernel<In, T, Op, true, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op); \
-            else scan_tiles_kernel<In, T, Op, false, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op);            \
+            if (lines_aligned) scan_tiles_kernel<In, T, Out, Op, true, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op); \
+            else scan_tiles_kernel<In, T, Out, Op, false, KK><<<grid, 256, 0, a.stream>>>(in, out, s.mid, init, inclusive, op);            \
         } while (0)
         if (s.mid <= ScanTile<T, 2>::TILE) RK_SCAN_TILES(2);
         else if (s.mid <= ScanTile<T, 4>::TILE) RK_SCAN_TILES(4);
@@ -2109,7 +2131,7 @@ inline int32_t launch_scan(const ScanArgs& a) {
     if constexpr (sizeof(T) <= 4 && sizeof(In) == sizeof(T)) {
         if (!dynamic_ids) {
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
-            scan_ordered_kernel<In, T, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
+            scan_ordered_kernel<In, T, Out, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
                 in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, ordered_ticket_group(ntiles), w.desc, gpl, ngroups, cap, wc, wait_alone(w.hdr), stagger_ticks, stagger_tiles, dyn)
             // staggered start of the first resident round (two workgroups of 16 waves a compute unit), where more rounds
             // follow: 5 us across the round measured best (2^26 Int32: 0 / 2 / 4 / 6 / 8 / 12 / 16 us -> 91.8 / 90.3 / 89.7 /
@@ -2127,7 +2149,7 @@ inline int32_t launch_scan(const ScanArgs& a) {
     if (grid > ntiles) grid = ntiles;
     if (grid < 1) grid = 1;
 #define RK_SCAN_CHAIN(VECF, NWW)                                                                                      \
-    scan_chain_kernel<In, T, Op, VECF, KT, NWW><<<(unsigned)grid, NWW * WAVE, 0, a.stream>>>(                          \
+    scan_chain_kernel<In, T, Out, Op, VECF, KT, NWW><<<(unsigned)grid, NWW * WAVE, 0, a.stream>>>(                          \
         in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.desc, gpl, ngroups, cap, wc)
     if (lines_aligned) {
         if (nw == 16) RK_SCAN_CHAIN(true, 16); else if (nw == 8) RK_SCAN_CHAIN(true, 8); else RK_SCAN_CHAIN(true, 4);
@@ -2139,13 +2161,13 @@ inline int32_t launch_scan(const ScanArgs& a) {
     return RK_SUCCESS;
 }
 
-template <typename In, typename T>
+template <typename In, typename T, typename Out = T>
 inline int32_t scan_typed(const ScanArgs& a) {
     switch (a.op) {
-        case RK_OP_ADD: return launch_scan<In, T, OpAdd>(a);
-        case RK_OP_MUL: return launch_scan<In, T, OpMul>(a);
-        case RK_OP_MAX: return launch_scan<In, T, OpMax>(a);
-        case RK_OP_MIN: return launch_scan<In, T, OpMin>(a);
+        case RK_OP_ADD: return launch_scan<In, T, Out, OpAdd>(a);
+        case RK_OP_MUL: return launch_scan<In, T, Out, OpMul>(a);
+        case RK_OP_MAX: return launch_scan<In, T, Out, OpMax>(a);
+        case RK_OP_MIN: return launch_scan<In, T, Out, OpMin>(a);
         default: return RK_ERR_INVALID_ARGUMENT;
     }
 }
@@ -2158,5 +2180,10 @@ int32_t scan_u8_i64(const ScanArgs&);
 int32_t scan_u8_i32(const ScanArgs&);
 int32_t scan_u32(const ScanArgs&);
 int32_t scan_u64(const ScanArgs&);
+int32_t scan_i8(const ScanArgs&);       // the narrow types: scanned in 32 bits, stored narrow
+int32_t scan_u8(const ScanArgs&);
+int32_t scan_i16(const ScanArgs&);
+int32_t scan_u16(const ScanArgs&);
+int32_t scan_f16(const ScanArgs&);
 
 }  // namespace rk

@@ -322,27 +322,12 @@ function native_accumulate_strided!(op, B::ROCStrided{TB,N}, A::ROCStrided{TA,N}
     return true
 end
 
-# 1- and 2-byte element types have no scan kernels of their own: scan in the next wider type and store back.  Integer sums
-# and products wrap modulo 2^32 and the narrowing store keeps the low bits (the narrow type's own wrap-around); Float16
-# is scanned in Float32 and rounded once.  Three native kernels: convert, scan in place, convert.
-scan_wide(::Type{Int8}) = Int32;   scan_wide(::Type{Int16}) = Int32
-scan_wide(::Type{UInt8}) = UInt32; scan_wide(::Type{UInt16}) = UInt32
-scan_wide(::Type{Float16}) = Float32
-scan_wide(::Type) = nothing
-
+# 1- and 2-byte element types (Int8, UInt8, Int16, UInt16, Float16) go through the same call: the library scans them in
+# the next wider type and stores them narrow (integers wrap like the narrow type itself; Float16 is rounded once, at
+# the store, where AcceleratedKernels rounds after every step).
 function enable_accumulate!()
     @eval function Base.accumulate!(op, B::ROCArray, A::ROCArray; init=zero(eltype(A)), dims=nothing, inclusive::Bool=true, kwargs...)
-        W = eltype(A) === eltype(B) ? scan_wide(eltype(B)) : nothing
-        if isempty(kwargs) && rk_op(op) !== nothing && W !== nothing
-            tmp = similar(A, W)
-            tmp .= A                                           # the native broadcast: widening copy
-            if native_accumulate!(op, tmp, tmp; init=convert(W, init), dims, inclusive)
-                B .= tmp                                       # narrowing store
-                AMDGPU.unsafe_free!(tmp)
-                return B
-            end
-            AMDGPU.unsafe_free!(tmp)
-        elseif isempty(kwargs) && rk_op(op) !== nothing && rk_dtype(eltype(A)) !== nothing && rk_dtype(eltype(B)) !== nothing
+        if isempty(kwargs) && rk_op(op) !== nothing && rk_dtype(eltype(A)) !== nothing && rk_dtype(eltype(B)) !== nothing
             native_accumulate!(op, B, A; init, dims, inclusive) && return B
         end
         return AMDGPU.AK.accumulate!(op, B, A, AMDGPU.ROCBackend(); init, dims, inclusive, kwargs...)

@@ -283,12 +283,20 @@ def test_short_lines_with_a_narrow_inner_extent(rk, orc, shape, dims):
 
 @pytest.mark.parametrize("dtype", [np.int8, np.uint8, np.int16, np.uint16, np.float16])
 def test_narrow_element_types(rk, orc, dtype):
-    """accumulate / cumsum / cumprod of 1- and 2-byte elements: scanned in the next wider type and stored back (the host
-    mirror's three native kernels).  Integers wrap in their own type, bit-exact; Float16 within a few Float16 roundings
-    of the Float64 scan (AcceleratedKernels rounds after every step, the native path once)."""
+    """accumulate / cumsum / cumprod of 1- and 2-byte elements, native in rk_accumulate: read narrow, scanned in the next
+    wider type, stored narrow -- one kernel, through every kernel family (shapes below).  Integers wrap in their own
+    type, bit-exact; Float16 within a few Float16 roundings of the Float64 scan (AcceleratedKernels rounds after every
+    step, the native path once)."""
     rng = np.random.default_rng(91)
     dt = np.dtype(dtype)
-    for shape, dims in (((1000,), 1), ((70_001,), 1), ((300, 70), 1), ((300, 70), 2), ((5, 64, 9), 2), ((200_000,), None)):
+    shapes = (((1000,), 1), ((70_001,), 1), ((300, 70), 1), ((300, 70), 2), ((5, 64, 9), 2), ((200_000,), None),
+              (((1 << 22) + 40,), 1),          # long line: single pass with look-back
+              ((4096, 700), 1),                # a tile a line
+              ((16, 40_000), 1), ((15, 40_001), 1),   # short lines: lane groups / whole slabs through LDS
+              ((1024, 2048), 2), ((257, 3000), 2),    # across rows: single pass / strips
+              ((3, 200_000), 2), ((64, 30_000), 2),   # narrow inner extent, long lines
+              ((4, 32, 5000), 2), ((300, 3, 200), 2)) # short scanned dim behind a narrow / a long inner extent
+    for shape, dims in shapes:
         if dt.kind == "f":
             x = (rng.random(shape) * 0.01).astype(dt)
         else:
