@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """HBM traffic per kernel from two rocprofv3 counter runs of bench.py (FETCH_SIZE, then WRITE_SIZE).
 
-    ONLY='sum Float32[2^26]|maximum|cumsum Int32[2^26]|z .= a.*x .+ y.*exp.(w) Float32[2^26]|calibration: copy z .= x Float32[2^26]|cfg2|cfg3|cumsum(B;dims=2)|cfg4|cfg5'
+    ONLY='sum Float32[2^26]|maximum|cumsum Int32[2^26]|z .= a.*x .+ y.*exp.(w) Float32[2^26]|calibration: copy z .= x Float32[2^26]|cfg2|cfg3|cumsum(B;dims=2)|cfg4|cfg5|Int16|sum(A; dims=|cumsum(A; dims=1) 15x|C .= A .+ r 3x|permutedims|reverse|findall'
     rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d F -o bench -- python3 bench.py --no-cpu --steps 5 --only "$ONLY"
     rocprofv3 --pmc WRITE_SIZE --kernel-trace --output-format csv -d W -o bench -- python3 bench.py --no-cpu --steps 5 --only "$ONLY"
     python bench_pmc_summary.py F/bench W/bench > profiles/<name>.txt
@@ -20,21 +20,33 @@ from collections import defaultdict
 KIB = 1024.0
 # (kernel-name fragment, grid work-items) -> (row of bench.py, algorithmic KiB read, written)
 M26, M27 = (1 << 26), (1 << 27)
+N25 = 1 << 25
+N15, N3 = (N25 // 15) * 15, (N25 // 3) * 3
 KNOWN = [
-    ("bc_kernel<EvalCopy", 16777216, "calibration: copy z .= x Float32[2^26]", 4 * M26 / KIB, 4 * M26 / KIB),
-    ("bc_kernel<EvalAxpbyExp", 16777216, "z .= a.*x .+ y.*exp.(w) Float32[2^26]", 12 * M26 / KIB, 4 * M26 / KIB),
-    ("bc_kernel<EvalAxpbyExp", 33554432, "cfg4a z .= a.*x .+ y.*exp.(w) 512^3", 12 * M27 / KIB, 4 * M27 / KIB),
-    ("bc_kernel<EvalRowCol", None, "cfg4b C .= A .+ r .* c 16384^2", 4 * (1 << 28) / KIB, 4 * (1 << 28) / KIB),
+    ("bc_flat_kernel<EvalCopy", 16777216, "calibration: copy z .= x Float32[2^26]", 4 * M26 / KIB, 4 * M26 / KIB),
+    ("bc_flat_kernel<EvalAxpbyExp", 16777216, "z .= a.*x .+ y.*exp.(w) Float32[2^26]", 12 * M26 / KIB, 4 * M26 / KIB),
+    ("bc_flat_kernel<EvalAxpbyExp", 33554432, "cfg4a z .= a.*x .+ y.*exp.(w) 512^3", 12 * M27 / KIB, 4 * M27 / KIB),
+    ("bc_kernel<EvalAddMul", None, "cfg4b C .= A .+ r .* c 16384^2", 4 * (1 << 28) / KIB, 4 * (1 << 28) / KIB),
     ("scan_ordered_kernel<int", 2097152, "cumsum Int32[2^26]", 4 * M26 / KIB, 4 * M26 / KIB),
     ("scan_ordered_kernel<int", 4194304, "cfg3a cumsum Int32[2^27]", 4 * M27 / KIB, 4 * M27 / KIB),
+    ("scan_ordered_kernel<short", None, "cumsum Int16[2^26] (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),
     ("scan_tiles_kernel<float", None, "cfg3b cumsum(B;dims=1) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
+    ("scan_tiles_kernel<_Float16", None, "cumsum(B;dims=1) 4096x16384 Float16 (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),
     ("scan_rows_ordered_kernel<float", None, "cumsum(B;dims=2) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
-    ("MapIdentity>, OpAdd", 131072, "sum Float32 (2^26: 262144 KiB; the 2^24 row shares this grid)", None, None),
+    ("MapIdentity>, OpAdd, ReduceSink<float, OpAdd, float>, true", 131072, "sum Float32 (2^26: 262144 KiB; the 2^24 row shares this grid)", None, None),
     ("MapIdentity>, OpMax", 131072, "maximum Float32[2^26]", 4 * M26 / KIB, 0.0),
     ("MapAbs2>, OpAdd", None, "cfg2a / cfg2b mapreduce(abs2,+) 8192^2", 4 * M26 / KIB, 32.0),
     ("ArgXform<float", None, "cfg2c findmax(A;dims=1) 8192^2", 4 * M26 / KIB, 160.0),
     ("volumerhs_vec_kernel", None, "cfg5 volumerhs! nelem=240000", 240000 * 11000 / KIB, 240000 * 2500 / KIB),
     ("volumerhs_kernel", None, "cfg5 volumerhs! nelem=4000", 4000 * 11000 / KIB, 4000 * 2500 / KIB),
+    # shapes with short or narrow extents, 2^25 elements (the rows bench.py keeps below the BASELINE configurations)
+    ("reduce_short_lines_kernel", None, "sum(A; dims=1) 32x1048576 / sum(A; dims=2) 4x32x262144", 4 * N25 / KIB, 4 * (N25 // 32) / KIB),
+    ("scan_lds_lines_kernel<float", None, "cumsum(A; dims=1) 15x2236962", 4 * N15 / KIB, 4 * N15 / KIB),
+    ("bc_indexed_kernel<EvalBinary", None, "C .= A .+ r 3x11184810 .+ 1x11184810", (4 * N3 + 4 * (N3 // 3)) / KIB, 4 * N3 / KIB),
+    ("permute_slab_kernel", None, "permutedims(A, (3,2,1)) 2x8388608x2", 4 * N25 / KIB, 4 * N25 / KIB),
+    ("permute_tiles_vec_kernel", None, "permutedims(A, (2,1)) 8192^2", 4 * M26 / KIB, 4 * M26 / KIB),
+    ("reverse_kernel", None, "reverse(A; dims=1) 8192^2", 4 * M26 / KIB, 4 * M26 / KIB),
+    ("findall_select_kernel", None, "findall(Bool[2^26], 25 % true): 1 B/elt read, 8 B per index written", M26 / KIB, 8 * 0.25 * M26 / KIB),
 ]
 
 
@@ -59,7 +71,7 @@ def main():
         sys.exit(__doc__)
     fetch, nf = load(sys.argv[1], "FETCH_SIZE")
     write, _ = load(sys.argv[2], "WRITE_SIZE")
-    cal = [k for k in fetch if k[0].startswith("bc_kernel<EvalCopy") and k[1] == 16777216]
+    cal = [k for k in fetch if k[0].startswith("bc_flat_kernel<EvalCopy") and k[1] == 16777216]
     if not cal:
         sys.exit("the calibration kernel (copy of 2^26 Float32) is not in the run")
     ff = 262144.0 / fetch[cal[0]]

@@ -39,6 +39,9 @@ def main():
     with open(base + "_kernel_trace.csv", newline="") as fh:
         for r in csv.DictReader(fh):
             t0, t1 = int(r["Start_Timestamp"]), int(r["End_Timestamp"])
+            if "at::native" in r["Kernel_Name"] or r["Kernel_Name"].startswith("__amd_rocclr"):
+                outside += 1                      # torch's own kernels (input generation, refills): not the library's
+                continue
             hit = None
             for a, b, name in ranges:
                 if a <= t0 <= b:
@@ -51,7 +54,7 @@ def main():
                    f'{r["Workgroup_Size_X"]}x{r["Workgroup_Size_Y"]}x{r["Workgroup_Size_Z"]}', r["VGPR_Count"], r["LDS_Block_Size"])
             rows[hit][key].append((t1 - t0) / 1e3)
     print("# kernels per bench row: calls, avg / min / max duration in us, grid (work-items), workgroup, VGPRs, LDS bytes")
-    print(f"# ({outside} dispatches outside any row: input generation by torch, clears)")
+    print(f"# ({outside} dispatches left out: outside any row, or torch's / the runtime's own kernels -- input generation, refills, clears)")
     for name, kernels in rows.items():
         print(f"\n== {name}")
         for (kname, grid, wg, vgpr, lds), d in sorted(kernels.items(), key=lambda kv: -sum(kv[1])):

@@ -155,6 +155,36 @@ def test_random_scans(rk, orc):
             assert np.array_equal(got, want.astype(got.dtype))
 
 
+def test_random_narrow_scans(rk, orc):
+    """Int8 / UInt8 / Int16 / UInt16 / Float16 scans over random shapes, dims, operators, init and inclusive: native in
+    rk_accumulate (scanned in 32 bits, stored narrow).  Integers wrap in their own type and must agree bit for bit."""
+    rng = np.random.default_rng(1007 + SEED)
+    for case in range(200):
+        shape = _shape(rng)
+        dtype = [np.int8, np.uint8, np.int16, np.uint16, np.float16][int(rng.integers(5))]
+        dt = np.dtype(dtype)
+        dim = int(rng.integers(1, len(shape) + 2))
+        op = ["add", "add", "max", "min", "mul"][int(rng.integers(5))]
+        inclusive = bool(rng.random() < 0.7)
+        init = int(rng.integers(0, 6)) if (not inclusive or rng.random() < 0.5) else None
+        if op == "mul" and init is None and not inclusive:
+            init = 1
+        _say("narrow scan", case, shape, dt.name, dim, op, inclusive, init)
+        if dt.kind == "f":
+            x = (rng.random(shape) * 0.01).astype(dt) if op != "mul" else (1 + rng.random(shape) * 1e-3).astype(dt)
+        else:
+            info = np.iinfo(dt)
+            x = rng.integers(info.min, info.max + 1, shape).astype(dt)
+        got = rk.Array(rk.accumulate(op, rk.ROCArray(x), dims=dim, init=None if init is None else dt.type(init), inclusive=inclusive))
+        want = orc.accumulate(op, x, dims=dim, init=None if init is None else dt.type(init), inclusive=inclusive)
+        assert got.dtype == dt and got.shape == want.shape
+        if dt.kind == "f":
+            n = shape[dim - 1] if dim <= len(shape) else 1
+            np.testing.assert_allclose(got.astype(np.float64), want.astype(np.float64), rtol=4e-3, atol=1e-3 * (1 + abs(init or 0)) if op != "mul" else 4e-3 * n)
+        else:
+            assert np.array_equal(got, want.astype(dt))
+
+
 def test_random_moves(rk, orc):
     rng = np.random.default_rng(1004 + SEED)
     for case in range(200):
