@@ -635,15 +635,18 @@ __global__ __launch_bounds__(NW * WAVE) void scan_chain_kernel(const In* __restr
 }
 
 // The tile of a workgroup of an "ordered" kernel (one tile per workgroup, every tile waits only for tiles of lower
-// number) and the epoch of the call.  dynamic_ids == 0: the workgroup's index -- every predecessor of a tile is then a
-// workgroup the hardware has started earlier, provided it starts workgroups in index order, which holds for one grid
-// alone on the device.  When two such grids are resident together the premise has a hole: the lowest unfinished tile of
-// grid A can be waiting for a slot on a compute unit whose slots are all held by waiting tiles of grid B, and the
-// other way round -- nothing in the way slots are handed to queues excludes it -- so a grid with more workgroups than
-// the device holds at once takes its tile numbers from the packed counter instead (dynamic_ids != 0; one device-wide
-// atomic per workgroup, which returns the epoch with the number): a tile's predecessors then belong to workgroups that
-// have already started, whatever else is resident.  A grid that fits the device whole cannot be part of such a cycle
-// through its own unstarted tiles for long: every other grid's waiting tiles depend only on their own grid.
+// number) and the epoch of the call.  dynamic_ids == 0: the workgroup's index.  Workgroups are dealt to the XCDs
+// round-robin by index and every XCD starts its share in index order, so for ONE grid alone on the device the lowest
+// unfinished tile is always resident and waits for nobody.  Across XCDs nothing orders the starts: tile 9 (XCD 1) may
+// be resident and waiting while tile 8 (XCD 0) still waits for a slot, and with a second such grid resident the slots
+// of XCD 0 may all be held by ITS waiting tiles, whose own lowest unfinished tile waits for a slot on XCD 1: a cycle
+// that no arbitration rule of the hardware is known to exclude.  Hence a kernel runs in launch order only where that
+// cannot happen -- its tiles help themselves when a wait drags on (desc_lookback_alone), or a tile waits only for
+// tiles of its own XCD -- and otherwise takes its tile numbers from the packed counter (dynamic_ids != 0; one
+// device-wide atomic per workgroup, which returns the epoch with the number; 8-10 % slower, the round trip sits in
+// front of every tile's loads, and neither asking for the next number behind the stores nor during the look-back of
+// the tile before hid it: 2^26 Int32 90 -> 100 / 104 / 112 us): a tile's predecessors then belong to workgroups that
+// have started, whatever else is resident.  Grids that fit the device whole stay in launch order.
 // `need_epoch` (wave-uniform): this wave uses the epoch -- the others of a launch-order grid skip the load and get 0.
 struct OrderedId { int64_t tile; uint32_t epoch; };
 __device__ __forceinline__ OrderedId ordered_tile_id(unsigned long long* counter, int dynamic_ids, bool need_epoch) {
@@ -696,12 +699,20 @@ __device__ __forceinline__ void ordered_finish(uint32_t epoch, int64_t used, uns
 // resident at once, and whether a grid of `nblocks` takes its tile numbers from the counter (see ordered_tile_id).
 int tune_ordered_ids();            // rk_api.hip: 0 = by grid size, 1 = always the launch order, 2 = always the counter
 inline int64_t ordered_resident(int threads) { return (int64_t)device_info().cus * (32 * WAVE / threads); }
-// `helps_itself`: the kernel's waits end in desc_lookback_alone, so its tiles need nobody and the launch order is safe
-// at any size.
-inline int ordered_dynamic_ids(int64_t nblocks, int threads, bool helps_itself) {
+// `launch_order_safe`: the launch order cannot starve the grid whatever else is resident -- the kernel's waits end in
+// desc_lookback_alone, so its tiles need nobody; or every tile waits only for tiles of its own XCD (see
+// rows_chains_stay_on_their_xcd).
+inline int ordered_dynamic_ids(int64_t nblocks, int threads, bool launch_order_safe) {
     const int t = tune_ordered_ids();
-    return t == 1 ? 0 : (t == 2 ? 1 : (!helps_itself && nblocks > ordered_resident(threads) ? 1 : 0));
+    return t == 1 ? 0 : (t == 2 ? 1 : (!launch_order_safe && nblocks > ordered_resident(threads) ? 1 : 0));
 }
+// The scans across rows number their tiles slice-major: tile = slice * nchains + chain, and a tile waits only for tiles
+// of its own chain.  Workgroups are dealt to the XCDs round-robin by index and each XCD starts its share in index order.
+// With the number of chains a multiple of 8 (of the number of XCDs, which divides 8) all tiles of a chain fall to one
+// XCD, so a resident tile waits only for tiles that the same XCD has started before it: the lowest resident tile of an
+// XCD waits for nobody, finishes, and so on up -- every resident tile finishes without any new workgroup having to
+// start, whatever other grids hold the remaining slots.  Other chain counts take their tile numbers from the counter.
+inline bool rows_chains_stay_on_their_xcd(int64_t nchains) { return nchains % 8 == 0; }
 // Workgroups per first-level exit ticket: at most half of the ticket lines in use, at least TICKET_GROUP a ticket.
 inline int ordered_ticket_group(int64_t nblocks) {
     int64_t tg = (nblocks + (int64_t)WS_TICKET_COUNT / 2 - 1) / ((int64_t)WS_TICKET_COUNT / 2);
@@ -709,14 +720,12 @@ inline int ordered_ticket_group(int64_t nblocks) {
 }
 
 // ---- long contiguous lines: one tile per workgroup in launch order, single pass ------------------------------------
-// Tile = blockIdx.x.  No tile counter: device-wide atomics on one address complete at about 14 ns each, which caps a
-// counter-fed kernel at 70 M tiles/s, and the counter's round trip sits in front of every tile's loads.  Forward
-// progress instead rests on the order in which the hardware starts workgroups: each XCD starts the workgroups dealt
-// to it in increasing blockIdx, so the lowest-numbered unfinished tile is always resident (it cannot be waiting for a
-// slot behind higher-numbered tiles of its own XCD, and tiles of other XCDs do not take its slots), and it waits for
-// nobody.  Should a device ever start workgroups out of order with all slots taken by waiting tiles, the bounded
-// waits end the call with RK_ERR_WAIT instead of hanging; RK_SCAN_DYNAMIC_IDS=1 selects scan_chain_kernel, whose
-// counter needs no such assumption.
+// Tile = blockIdx.x.  No tile counter: device-wide atomics on one address complete at about 14 ns each, and the
+// counter's round trip would sit in front of every tile's loads (2^26 Int32: 90 -> 100 us).  Forward progress does not
+// rest on the order in which workgroups start: a tile that has polled `wa.patience` times in vain stops waiting and
+// resolves its prefix alone, computing the aggregates nobody has published from the input (desc_lookback_alone), so
+// no tile needs another workgroup to be running.  Wave 0 parks its part of the tile in LDS while it looks back, which
+// leaves that path -- and the compiler -- the registers it needs.
 // 1024 threads x 8 vectors = 128 KiB of input per tile at <= 64 registers: two workgroups share a compute unit, one
 // loads or stores while the other waits for its prefix (at 112 registers and one workgroup per unit the wait was
 // dead time: 2^26 Int32 95.6 -> 92.5 us, 2^27 187.8 -> 180.5 us).  Smaller tiles stream better on their own (16 KiB
@@ -1836,7 +1845,7 @@ inline int32_t scan_across_rows(const In* in, Out* out, const ScanGeom& g, T ini
             scan_rows_ordered_kernel<In, T, Out, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
                 in, out, g, init, inclusive, op, strips, nchains, nslices, (T*)scratch, (unsigned long long*)&ws->hdr->scan_counter,
                 ws->tickets, ordered_ticket_group(ntiles), ws->desc, (int64_t)(ws->desc_bytes / sizeof(uint64_t)), wait_ctl(ws->hdr),
-                ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
+                ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, rows_chains_stay_on_their_xcd(nchains)));
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }
@@ -1909,7 +1918,7 @@ inline int32_t scan_rows_packed(const In* in, Out* out, const ScanGeom& g, T ini
             return RK_SUCCESS;
         scan_rows_packed_kernel<In, T, Out, Op, NW, R><<<(unsigned)ntiles, (NW + 1) * WAVE, 0, stream>>>(
             in, out, g, init, inclusive, op, P, nchains, nslices, (T*)w.partials, (unsigned long long*)&w.hdr->scan_counter, w.tickets,
-            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, false));
+            ordered_ticket_group(ntiles), w.desc, (int64_t)(w.desc_bytes / sizeof(uint64_t)), wait_ctl(w.hdr), ordered_dynamic_ids(ntiles, (NW + 1) * WAVE, rows_chains_stay_on_their_xcd(nchains)));
         RK_LAUNCH_CHECK();
         *done = true;
     }
