@@ -2129,15 +2129,14 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const int64_t gpl = (tpl + WAVE - 1) / WAVE, ngroups = gpl * nlines;
     // 8-byte values and unaligned lines do not fit two workgroups a compute unit; with one, the persistent counter-fed
     // kernel is the faster of the two (cumsum of Int64[2^25]: 96 against 107 us)
-    // (so do inputs narrower than the values -- Bool counted in Int32: the ordered kernel spills 27 registers for them)
-    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || sizeof(In) != sizeof(T) || !lines_aligned;
+    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || !lines_aligned;
     const size_t need = dynamic_ids ? (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t)
                                     : ((size_t)ntiles * Words<T>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const WaitCtl wc = wait_ctl(w.hdr);
-    if constexpr (sizeof(T) <= 4 && sizeof(In) == sizeof(T)) {
+    if constexpr (sizeof(T) <= 4) {
         if (!dynamic_ids) {
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
             scan_ordered_kernel<In, T, Out, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \

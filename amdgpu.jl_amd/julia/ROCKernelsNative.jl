@@ -82,6 +82,55 @@ function workspace(minbytes::Integer = 0)
     end
 end
 
+# ---- give-ups of bounded waits ---------------------------------------------------------------------------------
+# The scans across rows, the scan of 8-byte / unaligned lines and sorts of up to 2^20 keys wait on other workgroups with
+# a budget; a kernel that runs out of it records that in the workspace (the sort: in its temporary) and finishes with
+# meaningless results.  The records are read where the host waits for the device anyway -- Array(x), a scalar fetch --
+# for every workspace and sort temporary such a kernel has used on the task's stream since the last look; a give-up
+# prepares the workspace again and throws.  (The single-pass scan of long lines and findall never give up.)
+const waiting = Set{Tuple{Int,Ptr{Cvoid}}}()                                  # streams whose workspace a waiting kernel has used
+const sort_tmps = Dict{Tuple{Int,Ptr{Cvoid}},Vector{ROCArray{UInt8,1}}}()     # temporaries of small sorts, record unread
+note_waiting_call() = lock(() -> push!(waiting, (AMDGPU.device_id(AMDGPU.device()), stream_ptr())), workspaces_lock)
+function note_sort(tmp::ROCArray{UInt8,1}, n::Integer)
+    n > (1 << 20) && return AMDGPU.unsafe_free!(tmp)       # large sorts count before every pass and wait for nobody
+    key = (AMDGPU.device_id(AMDGPU.device()), stream_ptr())
+    pending = lock(() -> push!(get!(sort_tmps, key, ROCArray{UInt8,1}[]), tmp), workspaces_lock)
+    length(pending) > 16 && check_waits()                  # a long run of sorts without a fetch: read rather than hoard
+    return nothing
+end
+function check_waits()
+    key = (AMDGPU.device_id(AMDGPU.device()), stream_ptr())
+    failed = false
+    ws, tmps = lock(workspaces_lock) do
+        w = key in waiting ? get(workspaces, key, nothing) : nothing
+        delete!(waiting, key)
+        (w, pop!(sort_tmps, key, ROCArray{UInt8,1}[]))
+    end
+    if ws !== nothing
+        st = ccall((:rk_workspace_status, librk[]), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), pointer(ws), length(ws), stream_ptr())
+        if st == RK_ERR_WAIT
+            check(ccall((:rk_workspace_init, librk[]), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), pointer(ws), length(ws), stream_ptr()))
+            failed = true
+        else
+            check(st)
+        end
+    end
+    for tmp in tmps
+        st = ccall((:rk_sort_status, librk[]), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), pointer(tmp), sizeof(tmp), stream_ptr())
+        AMDGPU.unsafe_free!(tmp)
+        st == RK_ERR_WAIT ? (failed = true) : check(st)
+    end
+    failed && throw(RKError(RK_ERR_WAIT))
+    return nothing
+end
+# Array(x) and every scalar fetch copy device memory to the host, i.e. synchronise: the place to look.
+function enable_wait_checks!()
+    @eval function Base.Array(x::ROCArray{T,N}) where {T,N}
+        check_waits()
+        return copyto!(Array{T,N}(undef, size(x)), x)
+    end
+end
+
 dense(A::ROCArray) = true          # dense column-major storage: (pointer, dims) describes it completely
 dense(_) = false
 # wrappers over a ROCArray that are (pointer, size, strides) triples: operands / destinations of the *_strided entry points
@@ -285,6 +334,7 @@ function native_accumulate!(op, B::ROCArray{TB,N}, A::ROCArray{TA,N}; init, dims
     need = ccall((:rk_workspace_bytes, librk[]), Csize_t, (Cint, Cint, Cint, Ptr{Int64}, UInt32),
                  2, rk_dtype(TB), N, shape, dim <= N ? UInt32(1) << (dim - 1) : UInt32(0))
     ws = workspace(need)
+    note_waiting_call()
     initref = Ref(convert(TB, init))
     GC.@preserve A B ws shape initref begin
         st = ccall((:rk_accumulate, librk[]), Int32,
@@ -309,6 +359,7 @@ function native_accumulate_strided!(op, B::ROCStrided{TB,N}, A::ROCStrided{TA,N}
     need = ccall((:rk_workspace_bytes, librk[]), Csize_t, (Cint, Cint, Cint, Ptr{Int64}, UInt32),
                  2, rk_dtype(TB), N, shape[order], mdim <= N ? UInt32(1) << (mdim - 1) : UInt32(0))
     ws = workspace(need)
+    note_waiting_call()
     initref = Ref(convert(TB, init))
     GC.@preserve A B ws shape as bs initref begin
         st = ccall((:rk_accumulate_strided, librk[]), Int32,
@@ -573,7 +624,7 @@ function enable_sort!()
             st = ccall((:rk_sort, librk[]), Int32, (Cint, Ptr{Cvoid}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
                        rk_dtype(T), pointer(x), n, rev, pointer(tmp), sizeof(tmp), stream_ptr())
         end
-        AMDGPU.unsafe_free!(tmp)
+        note_sort(tmp, n)                                           # freed at once, or kept until its record has been read
         declined(st) && return (AMDGPU.AK.sort!(x; rev); x)          # rk_sort validates before it writes
         check(st)
         return x
@@ -588,7 +639,7 @@ function enable_sort!()
             st = ccall((:rk_sortperm, librk[]), Int32, (Cint, Ptr{Cvoid}, Ptr{Int64}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
                        rk_dtype(T), pointer(x), pointer(ix), n, rev, pointer(tmp), sizeof(tmp), stream_ptr())
         end
-        AMDGPU.unsafe_free!(tmp)
+        note_sort(tmp, n)
         declined(st) && return (AMDGPU.AK.sortperm!(ix, x; rev); ix)
         check(st)
         return ix
@@ -603,7 +654,7 @@ Install the native methods.  Call once after `using AMDGPU`.
 function enable!()
     isfile(librk[]) || error("librk.so not found at $(librk[]); build it with `python amdgpu.jl_amd/build.py`")
     ccall((:rk_version, librk[]), Int32, ()) >= 100 || error("librk.so is too old")
-    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!(); enable_reverse!(); enable_permutedims!(); enable_sort!()
+    enable_mapreduce!(); enable_findminmax!(); enable_accumulate!(); enable_broadcast!(); enable_findall!(); enable_reverse!(); enable_permutedims!(); enable_sort!(); enable_wait_checks!()
     return nothing
 end
 
