@@ -94,8 +94,9 @@ def test_findminmax_and_accumulate_validation(L):
     assert a(5, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert a(2, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 0, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # exclusive max needs init
     assert a(0, L.RK_F32, L.RK_F64, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
-    for narrow in (L.RK_I8, L.RK_I16, L.RK_U16, L.RK_F16):                                                       # no scans of 1- and 2-byte values
-        assert a(0, narrow, narrow, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+    for narrow in (L.RK_I8, L.RK_I16, L.RK_U16, L.RK_F16):                      # narrow scans are native, but only into their own type
+        assert a(0, narrow, L.RK_I32, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
+        assert a(0, narrow, narrow, one, C.c_void_p(0x3000), 2, L.shape_array((0, 4)), 1, 1, None, None, 0, None) == L.RK_SUCCESS
     assert a(0, L.RK_U8, L.RK_I64, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT    # aliasing with different sizes
     assert a(0, L.RK_F32, L.RK_F32, None, None, 1, L.shape_array((0,)), 1, 1, None, None, 0, None) == L.RK_SUCCESS
     # a look-back scan without workspace
