@@ -19,6 +19,6 @@ from .volumerhs import volumerhs_                                               
 from .indexing import findall, getindex_mask                                                         # noqa: F401
 from .reverse import reverse, reverse_                                                # noqa: F401
 from .permutedims import permutedims, permutedims_                                    # noqa: F401
-from .sorting import sort, sort_, sortperm, sortperm_                                 # noqa: F401
+from .sorting import sort, sort_, sortperm, sortperm_, isless, not_isless             # noqa: F401
 
 __version__ = "0.1.0"

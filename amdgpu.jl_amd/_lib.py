@@ -39,7 +39,7 @@ RK_F32, RK_F64, RK_I32, RK_I64, RK_U8, RK_U32, RK_U64, RK_F16, RK_I16, RK_I8, RK
 RK_MAP_IDENTITY, RK_MAP_ABS2, RK_MAP_ABS = range(3)
 RK_MAP_MAX_TOKENS, RK_MAP_MAX_CONSTS = 16, 4
 # rk_op
-RK_OP_ADD, RK_OP_MUL, RK_OP_MAX, RK_OP_MIN = range(4)
+RK_OP_ADD, RK_OP_MUL, RK_OP_MAX, RK_OP_MIN, RK_OP_AND, RK_OP_OR, RK_OP_XOR = range(7)
 # rk_opkind
 RK_KIND_MAPREDUCE, RK_KIND_FINDMINMAX, RK_KIND_ACCUMULATE, RK_KIND_FINDALL = range(4)
 # rk_bc_token

@@ -7,20 +7,26 @@ import numpy as np
 
 from . import _lib as L
 from .array import ROCArray, note_waiting_call, stream_ptr, workspace
-from .mapreduce import _OP, _scalar_buffer
+from .mapreduce import _scalar_buffer
+
+
+_SCAN_OP = {"add": L.RK_OP_ADD, "mul": L.RK_OP_MUL, "max": L.RK_OP_MAX, "min": L.RK_OP_MIN,
+            "and": L.RK_OP_AND, "or": L.RK_OP_OR, "xor": L.RK_OP_XOR}          # & | xor: integer element types and Bool
+_BITWISE = ("and", "or", "xor")
 
 
 def accumulate_eltype(op: str, dtype) -> np.dtype:
     """``promote_op(op, T, typeof(init))`` with the reference's default ``init = zero(eltype(A))``
-    (accumulate.jl:1,4): the eltype is preserved (Int32 stays Int32 and wraps); Bool counts in Int64."""
+    (accumulate.jl:1,4): the eltype is preserved (Int32 stays Int32 and wraps); Bool counts in Int64, and stays Bool
+    under the bitwise operators (``&``, ``|``, ``xor`` of Bools are Bools)."""
     dt = np.dtype(dtype)
-    return np.dtype(np.int64) if dt == np.bool_ else dt
+    return np.dtype(np.int64) if dt == np.bool_ and op not in _BITWISE else dt
 
 
 def accumulate_(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusive: bool = True) -> ROCArray:
     """``accumulate!(op, B, A; dims, init)``; ``B`` may be ``A`` itself.  Returns ``B``."""
-    if op not in ("add", "mul", "max", "min"):
-        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"scan operator {op!r}")
+    if op not in _SCAN_OP or (op in _BITWISE and np.dtype(B.dtype).kind not in "iub"):
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, f"scan operator {op!r} over {B.dtype}")
     if B.dims != A.dims:
         raise L.DimensionMismatch(L.RK_ERR_DIMENSION, f"accumulate!: {B.dims} vs {A.dims}")
     if dims is None:
@@ -51,7 +57,7 @@ def _launch_accumulate(op, B, A, dims, init, inclusive):
         aptr = A.sptr if isinstance(A, ROCView) else A.ptr
         bptr = B.sptr if isinstance(B, ROCView) else B.ptr
         ws, ws_bytes = workspace(16 << 20)
-        sargs = (_OP[op], A.code, B.code, aptr, bptr, A.ndim, L.shape_array(A.dims), L.shape_array(astr), L.shape_array(bstr), int(dims),
+        sargs = (_SCAN_OP[op], A.code, B.code, aptr, bptr, A.ndim, L.shape_array(A.dims), L.shape_array(astr), L.shape_array(bstr), int(dims),
                  1 if inclusive else 0, _scalar_buffer(init, B.dtype), ws, ws_bytes)
 
         def launch_strided():
@@ -62,7 +68,7 @@ def _launch_accumulate(op, B, A, dims, init, inclusive):
                                             (1 << (dims - 1)) if dims <= A.ndim else 0)
     ws, ws_bytes = workspace(bytes_needed)
     ibuf = _scalar_buffer(init, B.dtype)
-    args = (_OP[op], A.code, B.code, A.ptr, B.ptr, A.ndim, L.shape_array(A.dims), int(dims), 1 if inclusive else 0,
+    args = (_SCAN_OP[op], A.code, B.code, A.ptr, B.ptr, A.ndim, L.shape_array(A.dims), int(dims), 1 if inclusive else 0,
             ibuf, ws, ws_bytes)
     fn = L.lib.rk_accumulate
 
@@ -75,7 +81,7 @@ def _launch_accumulate(op, B, A, dims, init, inclusive):
 def plan_accumulate(op: str, B: ROCArray, A: ROCArray, dims=None, init=None, inclusive: bool = True):
     """Validate once, return a callable that repeats ``accumulate!(op, B, A; dims, init)`` with no
     per-call host work beyond the foreign call."""
-    if op not in ("add", "mul", "max", "min") or B.dims != A.dims or len(A) == 0:
+    if op not in _SCAN_OP or B.dims != A.dims or len(A) == 0:
         raise ValueError("plan_accumulate: unsupported operator, mismatched dims or empty input")
     if dims is None:
         dims = 1

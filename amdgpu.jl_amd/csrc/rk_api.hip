@@ -270,6 +270,7 @@ static int32_t mapreduce_dispatch(rk_map f, rk_op op, rk_dtype in, rk_dtype out,
     int64_t total = 0;
     if (!valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
     if ((int)f < RK_MAP_IDENTITY || (int)f > RK_MAP_ABS) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op >= RK_OP_AND && (int)op <= RK_OP_XOR) return RK_ERR_UNSUPPORTED;       // bitwise operators: scans only
     if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
     if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
     if (total == 0) return RK_SUCCESS;                     // mapreduce.jl:91
@@ -409,6 +410,7 @@ int32_t rk_mapreduce_program(const rk_map_program* f, rk_op op, rk_dtype in, rk_
                              void* stream) {
     int64_t total = 0;
     if (f == nullptr || !valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op >= RK_OP_AND && (int)op <= RK_OP_XOR) return RK_ERR_UNSUPPORTED;       // bitwise operators: scans only
     if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
     if (f->n_tokens < 1 || f->n_tokens > RK_MAP_MAX_TOKENS || f->n_consts < 0 || f->n_consts > RK_MAP_MAX_CONSTS) return RK_ERR_INVALID_ARGUMENT;
     const bool int_compute = in != RK_F32 && in != RK_F64;
@@ -463,7 +465,7 @@ int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, v
                       int dim, int32_t inclusive, const void* init, void* ws, size_t ws_bytes, void* stream) {
     int64_t total = 0;
     if (!valid_dtype(in) || !valid_dtype(out)) return RK_ERR_INVALID_ARGUMENT;
-    if ((int)op < RK_OP_ADD || (int)op > RK_OP_MIN) return RK_ERR_INVALID_ARGUMENT;
+    if ((int)op < RK_OP_ADD || (int)op > RK_OP_XOR) return RK_ERR_INVALID_ARGUMENT;
     if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
     if (dim < 1) return RK_ERR_INVALID_ARGUMENT;
     if (total == 0) return RK_SUCCESS;

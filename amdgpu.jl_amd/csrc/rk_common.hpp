@@ -415,6 +415,20 @@ struct OpMin {
     template <typename T> static __host__ __device__ __forceinline__ T identity() { return Limits<T>::highest(); }
 };
 
+// Bitwise operators (scans of integer element types): & | xor.
+struct OpAnd {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const { return (T)(a & b); }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return (T)~(T)0; }
+};
+struct OpOr {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const { return (T)(a | b); }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return T(0); }
+};
+struct OpXor {
+    template <typename T> __host__ __device__ __forceinline__ T operator()(T a, T b) const { return (T)(a ^ b); }
+    template <typename T> static __host__ __device__ __forceinline__ T identity() { return T(0); }
+};
+
 // ---- findmax / findmin: argmax over order-preserving integer keys ------------------------------
 // Base.isless is a total order on floats (-0.0 < 0.0, NaN above everything) and findmax keeps the
 // first maximum; findmin (Base.isgreater) keeps the first minimum but NaN still wins.  Each value

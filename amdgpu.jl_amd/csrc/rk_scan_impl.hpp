@@ -2176,8 +2176,18 @@ inline int32_t scan_typed(const ScanArgs& a) {
         case RK_OP_MUL: return launch_scan<In, T, Out, OpMul>(a);
         case RK_OP_MAX: return launch_scan<In, T, Out, OpMax>(a);
         case RK_OP_MIN: return launch_scan<In, T, Out, OpMin>(a);
-        default: return RK_ERR_INVALID_ARGUMENT;
+        default: break;
     }
+    // the bitwise operators: integer element types scanned into their own type
+    if constexpr (std::is_integral<T>::value && std::is_same<In, Out>::value) {
+        switch (a.op) {
+            case RK_OP_AND: return launch_scan<In, T, Out, OpAnd>(a);
+            case RK_OP_OR:  return launch_scan<In, T, Out, OpOr>(a);
+            case RK_OP_XOR: return launch_scan<In, T, Out, OpXor>(a);
+            default: break;
+        }
+    }
+    return a.op >= RK_OP_AND && a.op <= RK_OP_XOR ? RK_ERR_UNSUPPORTED : RK_ERR_INVALID_ARGUMENT;
 }
 
 int32_t scan_f32(const ScanArgs&);

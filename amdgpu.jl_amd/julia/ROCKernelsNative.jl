@@ -61,7 +61,8 @@ rk_map(_) = nothing
 rk_op(::typeof(+)) = Cint(0); rk_op(::typeof(Base.add_sum)) = Cint(0)
 rk_op(::typeof(*)) = Cint(1); rk_op(::typeof(Base.mul_prod)) = Cint(1)
 rk_op(::typeof(max)) = Cint(2); rk_op(::typeof(min)) = Cint(3)
-rk_op(_) = nothing
+rk_op(::typeof(&)) = Cint(4); rk_op(::typeof(|)) = Cint(5); rk_op(::typeof(xor)) = Cint(6)    # scans of integers and Bools only:
+rk_op(_) = nothing                                                                           # reductions decline them
 
 # ---- one workspace per (device, stream): the analogue of the per-task library handles (src/cache.jl) --------
 const WORKSPACE_BYTES = 16 << 20
@@ -201,25 +202,33 @@ struct MapSym{T} <: Real                # T: the Julia type the value would have
     toks::Vector{Int32}
     consts::Vector{Any}                 # shared by every node of one trace
 end
-operand!(s::MapSym, c::Union{Float32,Float64,Int32,Int64,Bool}) = begin
+operand!(s::MapSym, c::Union{Float32,Float64,Int32,Int64,UInt32,Bool}) = begin
     k = findfirst(==(c), s.consts)
     k === nothing && (push!(s.consts, c); k = length(s.consts))
     k > 4 && throw(Unsupported())
     Int32[k]
 end
+# Integer programs compute in Int64.  Where Julia's value is an Int32 / UInt32 -- the result of arithmetic on such
+# values -- a wrap token (RK_BC_WRAP_I32 = 132, RK_BC_WRAP_U32 = 133) restores it, so comparisons, max / min and the
+# widening sum see what Julia's wrapping arithmetic produces (mapreduce(x -> x + 1, +, ::ROCArray{Int32})).
+wrap_tokens(::Type{Int32}) = Int32[132]
+wrap_tokens(::Type{UInt32}) = Int32[133]
+wrap_tokens(::Type) = Int32[]
 for (f, tok) in ((:+, 32), (:-, 33), (:*, 34), (:/, 35), (:max, 36), (:min, 37), (:<, 96), (:<=, 97), (:>, 98), (:>=, 99),
                  (:(==), 100), (:!=, 101), (:&, 102), (:|, 103))
     R = tok >= 96 ? :(Bool) : tok == 35 ? :(typeof(one(A) / one(B))) : :(Base.promote_op($f, A, B))
-    @eval Base.$f(a::MapSym{A}, b::MapSym{B}) where {A,B} = MapSym{$R}(vcat(a.toks, b.toks, Int32($tok)), a.consts)
-    @eval Base.$f(a::MapSym{A}, b::B) where {A,B<:Union{Float32,Float64,Int32,Int64,Bool}} =
-        MapSym{$R}(vcat(a.toks, operand!(a, b), Int32($tok)), a.consts)
-    @eval Base.$f(a::A, b::MapSym{B}) where {A<:Union{Float32,Float64,Int32,Int64,Bool},B} =
-        MapSym{$R}(vcat(operand!(b, a), b.toks, Int32($tok)), b.consts)
+    W = tok <= 34 ? :(wrap_tokens($R)) : :(Int32[])           # + - * can leave the 32-bit range
+    @eval Base.$f(a::MapSym{A}, b::MapSym{B}) where {A,B} = MapSym{$R}(vcat(a.toks, b.toks, Int32($tok), $W), a.consts)
+    @eval Base.$f(a::MapSym{A}, b::B) where {A,B<:Union{Float32,Float64,Int32,Int64,UInt32,Bool}} =
+        MapSym{$R}(vcat(a.toks, operand!(a, b), Int32($tok), $W), a.consts)
+    @eval Base.$f(a::A, b::MapSym{B}) where {A<:Union{Float32,Float64,Int32,Int64,UInt32,Bool},B} =
+        MapSym{$R}(vcat(operand!(b, a), b.toks, Int32($tok), $W), b.consts)
 end
 for (f, tok) in ((:-, 64), (:abs, 65), (:abs2, 66), (:sqrt, 67), (:exp, 68), (:log, 69), (:inv, 73), (:!, 128), (:isodd, 129),
                  (:iseven, 130), (:isnan, 131))
     R = tok >= 128 ? :(Bool) : :(Base.promote_op($f, A))
-    @eval Base.$f(a::MapSym{A}) where {A} = MapSym{$R}(vcat(a.toks, Int32($tok)), a.consts)
+    W = tok in (64, 65, 66) ? :(wrap_tokens($R)) : :(Int32[])  # -x, abs(x), abs2(x) of typemin(Int32) wrap
+    @eval Base.$f(a::MapSym{A}) where {A} = MapSym{$R}(vcat(a.toks, Int32($tok), $W), a.consts)
 end
 Base.ifelse(c::MapSym{Bool}, a::MapSym{A}, b::MapSym{B}) where {A,B} =
     MapSym{promote_type(A, B)}(vcat(c.toks, a.toks, b.toks, Int32(112)), c.consts)
@@ -230,8 +239,7 @@ function trace_map(f, ::Type{T}) where {T}
     y isa MapSym || throw(Unsupported())
     R = typeof(y).parameters[1]
     toks = y.toks
-    # integer programs run in Int64: only Int64 / Bool values may reach an order-sensitive token or the reduction unwrapped
-    T <: Union{Int32,UInt32} && throw(Unsupported())
+    # (integer programs run in Int64; Int32 / UInt32 intermediates carry their wrap tokens, see wrap_tokens)
     T <: AbstractFloat && !all(c -> c isa T || c isa Integer, consts) && throw(Unsupported())      # 0.5 over Float32: a Float64 map
     length(toks) <= 16 || throw(Unsupported())
     cf = ntuple(k -> k <= length(consts) ? Float64(consts[k]) : 0.0, 4)
@@ -611,14 +619,29 @@ function enable_permutedims!()
     end
 end
 
-# ---- sort! / sortperm! (src/kernels/sorting.jl:1-3): default order and rev natively, closures stay with AK -------------
+# ---- sort! / sortperm! (src/kernels/sorting.jl:1-3) ----------------------------------------------------------------------
+# Native: the default order, `rev`, `lt = !isless` (the descending order: test/hip_rocarray/sorting.jl:20-22) and any `by`
+# whose keys `by.(x)` have a sortable eltype (:24-26): map (the fused broadcast), sortperm of the keys, gather.  Any other
+# `lt` stays with AcceleratedKernels.
 const SORTABLE = Union{Float16,Float32,Float64,Int16,Int32,Int64}
+# false / true: `lt` is isless / !isless (reverses the order); nothing: a comparator the library has no form for
+native_order(lt) = lt === isless ? false : (lt isa ComposedFunction{typeof(!),typeof(isless)} ? true : nothing)
 
 function enable_sort!()
     @eval function Base.sort!(x::ROCVector{T}; rev::Bool=false, lt=isless, by=identity, kwargs...) where {T<:SORTABLE}
-        (lt === isless && by === identity && isempty(kwargs)) || return (AMDGPU.AK.sort!(x; rev, lt, by, kwargs...); x)
+        flip = native_order(lt)
+        (flip !== nothing && isempty(kwargs)) || return (AMDGPU.AK.sort!(x; rev, lt, by, kwargs...); x)
+        rev = xor(rev, flip)
         n = length(x)
         n > 1 || return x
+        if by !== identity
+            keys = by.(x)
+            eltype(keys) <: SORTABLE || return (AMDGPU.AK.sort!(x; rev, by, kwargs...); x)
+            p = sortperm(keys; rev)
+            copyto!(x, x[p])
+            AMDGPU.unsafe_free!(keys); AMDGPU.unsafe_free!(p)
+            return x
+        end
         tmp = ROCVector{UInt8}(undef, ccall((:rk_sort_tmp_bytes, librk[]), Csize_t, (Cint, Int64, Int32), rk_dtype(T), n, 0))
         GC.@preserve x tmp begin
             st = ccall((:rk_sort, librk[]), Int32, (Cint, Ptr{Cvoid}, Int64, Int32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
@@ -630,7 +653,14 @@ function enable_sort!()
         return x
     end
     @eval function Base.sortperm!(ix::ROCVector{Int}, x::ROCVector{T}; rev::Bool=false, lt=isless, by=identity, kwargs...) where {T<:SORTABLE}
-        (lt === isless && by === identity && isempty(kwargs)) || return (AMDGPU.AK.sortperm!(ix, x; rev, lt, by, kwargs...); ix)
+        flip = native_order(lt)
+        (flip !== nothing && isempty(kwargs)) || return (AMDGPU.AK.sortperm!(ix, x; rev, lt, by, kwargs...); ix)
+        rev = xor(rev, flip)
+        if by !== identity
+            keys = by.(x)
+            eltype(keys) <: SORTABLE || return (AMDGPU.AK.sortperm!(ix, x; rev, by, kwargs...); ix)
+            return sortperm!(ix, keys; rev)
+        end
         n = length(x)
         length(ix) == n || throw(DimensionMismatch("sortperm!: index vector of length $(length(ix)) for $n keys"))
         n > 0 || return ix

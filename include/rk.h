@@ -84,7 +84,9 @@ typedef enum { RK_MAP_IDENTITY = 0, RK_MAP_ABS2 = 1, RK_MAP_ABS = 2 } rk_map;
 
 /* op of mapreduce / accumulate.  Base.add_sum / mul_prod are ADD / MUL with a wider
  * output dtype chosen by the caller (Int32 -> Int64). */
-typedef enum { RK_OP_ADD = 0, RK_OP_MUL = 1, RK_OP_MAX = 2, RK_OP_MIN = 3 } rk_op;
+/* RK_OP_AND / OR / XOR: the bitwise operators, in scans (rk_accumulate*) of integer element types and Bool only --
+ * accumulate(&, A), accumulate(|, A), accumulate(xor, A); reductions return RK_ERR_UNSUPPORTED for them. */
+typedef enum { RK_OP_ADD = 0, RK_OP_MUL = 1, RK_OP_MAX = 2, RK_OP_MIN = 3, RK_OP_AND = 4, RK_OP_OR = 5, RK_OP_XOR = 6 } rk_op;
 
 /* which entry point a workspace is sized for */
 typedef enum {

@@ -97,7 +97,7 @@ def accumulate_eltype(op: str, dtype) -> np.dtype:
     (Int32 stays Int32 and wraps), only Bool promotes to Int64.
     """
     dt = np.dtype(dtype)
-    if dt == np.bool_:
+    if dt == np.bool_ and op not in ("and", "or", "xor"):     # &, |, xor of Bools are Bools
         return np.dtype(np.int64)
     return dt
 
@@ -138,7 +138,7 @@ def _wide(a: np.ndarray, out_dtype: np.dtype) -> np.ndarray:
     """Promote to the precision the oracle computes in."""
     if out_dtype.kind == "f":
         return a.astype(np.float64)
-    if out_dtype.kind in "iu":
+    if out_dtype.kind in "iub":                  # (b: Bool under the bitwise scan operators)
         return a.astype(out_dtype)
     raise ValueError(out_dtype)
 
@@ -325,6 +325,16 @@ def findmin(A, dims=None):
 # accumulate / cumsum / cumprod   (src/kernels/accumulate.jl:1-8)
 # ---------------------------------------------------------------------------
 
+_BIT_UFUNC = {"and": np.bitwise_and, "or": np.bitwise_or, "xor": np.bitwise_xor}
+
+
+def _bit_neutral(op: str, dt: np.dtype):
+    """Neutral element of a bitwise operator: all ones for ``&`` (true for Bool), zero for ``|`` and ``xor``."""
+    if op == "and":
+        return np.bool_(True) if dt == np.bool_ else dt.type(-1 if dt.kind == "i" else np.iinfo(dt).max)
+    return dt.type(0)
+
+
 def accumulate(op: str, A: np.ndarray, dims=None, init=None, inclusive: bool = True) -> np.ndarray:
     """``accumulate(op, A; dims, init)`` as the ROCArray methods define it.
 
@@ -358,12 +368,14 @@ def accumulate(op: str, A: np.ndarray, dims=None, init=None, inclusive: bool = T
                     out = out + seed
                 elif op == "mul":
                     out = out * seed
+                elif op in _BIT_UFUNC:
+                    out = _BIT_UFUNC[op](out, seed)
                 else:
                     out = (np.maximum if op == "max" else np.minimum)(out, seed)
         if not inclusive:
             if init is None and op in ("max", "min"):
                 raise ValueError("exclusive max/min scans need init")
-            neutral = a.dtype.type(0 if op == "add" else 1)
+            neutral = _bit_neutral(op, a.dtype) if op in _BIT_UFUNC else a.dtype.type(0 if op == "add" else 1)
             out = np.full_like(a, neutral if init is None else a.dtype.type(init))
         return out
     with np.errstate(over="ignore"):
@@ -377,6 +389,9 @@ def accumulate(op: str, A: np.ndarray, dims=None, init=None, inclusive: bool = T
             fn = np.maximum if op == "max" else np.minimum
             inc = fn.accumulate(a, axis=axis)
             neutral = None
+        elif op in _BIT_UFUNC:                      # accumulate(&, A), accumulate(|, A), accumulate(xor, A)
+            inc = _BIT_UFUNC[op].accumulate(a, axis=axis)
+            neutral = _bit_neutral(op, a.dtype)
         else:
             raise ValueError(f"unknown op {op!r}")
         seed = neutral if init is None else a.dtype.type(init)
@@ -385,6 +400,8 @@ def accumulate(op: str, A: np.ndarray, dims=None, init=None, inclusive: bool = T
                 inc = inc + seed
             elif op == "mul":
                 inc = inc * seed
+            elif op in _BIT_UFUNC:
+                inc = _BIT_UFUNC[op](inc, seed)
             else:
                 inc = (np.maximum if op == "max" else np.minimum)(inc, seed)
         if inclusive:

@@ -91,7 +91,10 @@ def test_findminmax_and_accumulate_validation(L):
     a = L.lib.rk_accumulate
     assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert a(0, L.RK_F32, L.RK_F32, one, one, 2, sh, 0, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # dim is 1-based
-    assert a(5, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert a(7, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # no such operator
+    assert a(L.RK_OP_XOR, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED        # bitwise: integers only
+    m = L.lib.rk_mapreduce
+    assert m(0, L.RK_OP_AND, L.RK_I32, L.RK_I32, one, 2, sh, 1, one, None, None, 0, None) == L.RK_ERR_UNSUPPORTED        # and in scans only
     assert a(2, L.RK_F32, L.RK_F32, one, one, 2, sh, 1, 0, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # exclusive max needs init
     assert a(0, L.RK_F32, L.RK_F64, one, C.c_void_p(0x3000), 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_UNSUPPORTED
     for narrow in (L.RK_I8, L.RK_I16, L.RK_U16, L.RK_F16):                      # narrow scans are native, but only into their own type

@@ -474,3 +474,37 @@ def test_sort_matches_isless_insertion_sort(orc):
     assert np.array_equal(orc.sort(x), np.sort(x)) and np.array_equal(orc.sort(x, rev=True), np.sort(x)[::-1])
     assert orc.sort(np.array([3, 1, 2])).tolist() == [1, 2, 3]
     assert orc.sortperm(np.array([3, 1, 2])).tolist() == [2, 3, 1]                 # Base docs: sortperm([3, 1, 2])
+
+
+def test_bitwise_scans_against_a_sequential_loop():
+    """accumulate(&, A), accumulate(|, A), accumulate(xor, A): pinned by the definition itself, a sequential loop over
+    every line, for signed, unsigned and Bool element types, with and without init, inclusive and exclusive, and
+    along a dim beyond ndims (a copy with init folded in)."""
+    rng = np.random.default_rng(77)
+    py = {"and": lambda a, b: a & b, "or": lambda a, b: a | b, "xor": lambda a, b: a ^ b}
+    for dtype in (np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64, np.bool_):
+        dt = np.dtype(dtype)
+        shape = (5, 7, 3)
+        x = (rng.random(shape) < 0.6) if dt == np.bool_ else rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, shape, dtype=dt, endpoint=True)
+        for op in ("and", "or", "xor"):
+            assert orc.accumulate_eltype(op, dt) == dt                       # Bool stays Bool under these
+            for dims in (1, 2, 3, 4):
+                for init, inclusive in ((None, True), (x.reshape(-1)[3], True), (x.reshape(-1)[5], False), (None, False)):
+                    got = orc.accumulate(op, x, dims=dims, init=init, inclusive=inclusive)
+                    assert got.dtype == dt and got.shape == shape
+                    neutral = (True if dt == np.bool_ else dt.type(-1 if dt.kind == "i" else np.iinfo(dt).max)) if op == "and" else dt.type(0)
+                    seed = neutral if init is None else init
+                    want = np.empty_like(x)
+                    moved = np.moveaxis(x, dims - 1, 0) if dims <= 3 else x[None]
+                    wmoved = np.moveaxis(want, dims - 1, 0) if dims <= 3 else want[None]
+                    for idx in np.ndindex(moved.shape[1:]):
+                        run = seed
+                        for k in range(moved.shape[0]):
+                            v = moved[(k,) + idx]
+                            if inclusive:
+                                run = py[op](run, v)
+                                wmoved[(k,) + idx] = run
+                            else:
+                                wmoved[(k,) + idx] = run
+                                run = py[op](run, v)
+                    assert np.array_equal(got, want), (dt, op, dims, init, inclusive)

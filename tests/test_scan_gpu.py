@@ -416,3 +416,34 @@ def test_short_rows_several_to_a_load(rk, orc, shape):
             np.testing.assert_allclose(rk.Array(dx), want, rtol=1e-4, atol=5e-2 if dtype == np.float32 else 1e-9)
         else:
             assert np.array_equal(rk.Array(dx), want.astype(dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64, np.bool_])
+def test_bitwise_scan_operators(rk, orc, dtype):
+    """accumulate(&, A), accumulate(|, A), accumulate(xor, A) on integer element types and Bool (what AcceleratedKernels
+    accepts through src/kernels/accumulate.jl:1-8 besides + * max min), bit-exact, through every kernel family."""
+    rng = np.random.default_rng(93)
+    dt = np.dtype(dtype)
+    shapes = (((1000,), 1), (((1 << 21) + 40,), 1), ((4096, 300), 1), ((15, 20_001), 1), ((512, 1200), 2), ((3, 100_000), 2),
+              ((4, 32, 2000), 2), ((300, 3, 100), 2), ((70_001,), None))
+    for shape, dims in shapes:
+        if dt == np.bool_:
+            x = rng.random(shape) < 0.9
+        else:
+            # mostly-ones bit patterns, so that & keeps bits alive for a while and | fills up slowly from sparse ones
+            x = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, shape, dtype=dt, endpoint=True)
+        dx = rk.ROCArray(x)
+        for op in ("and", "or", "xor"):
+            src = x
+            if op == "and" and dt != np.bool_:
+                src = x | rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, shape, dtype=dt, endpoint=True)
+            elif op == "or" and dt != np.bool_:
+                src = x & rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, shape, dtype=dt, endpoint=True) & rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, shape, dtype=dt, endpoint=True)
+            d = rk.ROCArray(src) if src is not x else dx
+            got = rk.Array(rk.accumulate(op, d, dims=dims))
+            assert got.dtype == dt and np.array_equal(got, orc.accumulate(op, src, dims=dims)), (shape, dims, op)
+            init = src.reshape(-1)[7]
+            got = rk.Array(rk.accumulate(op, d, dims=dims, init=init, inclusive=False))
+            assert np.array_equal(got, orc.accumulate(op, src, dims=dims, init=init, inclusive=False)), (shape, dims, op, "exclusive")
+    with pytest.raises(NotImplementedError):
+        rk.accumulate("xor", rk.ROCArray(np.ones(8, dtype=np.float32)))

@@ -1,7 +1,8 @@
 """GPU parity of sort / sort! / sortperm / sortperm! (src/kernels/sorting.jl:1-3) against the oracle, through the
 C ABI: the sizes and element types of test/hip_rocarray/sorting.jl:5-28 for the default order and rev=true
 (values and permutations bit-exact, NaNs compared as equal), plus sizes that span many tiles, special floats,
-duplicates (stability) and small-range integers (skipped passes).  `lt` / `by` closures have no native form."""
+duplicates (stability) and small-range integers (skipped passes).  The two other forms of that test, `lt=!isless` and
+`by=k -> 2k` (:20-26), are native as well: descending order, and map -> sortperm of the keys -> gather."""
 import numpy as np
 import pytest
 
@@ -36,6 +37,32 @@ def _check(rk, orc, x):
 @pytest.mark.parametrize("sz", [1, 2, 3, 4, 33, 333, 3333, 4096])
 def test_reference_sizes_and_types(rk, orc, dtype, sz):
     _check(rk, orc, _rand(np.random.default_rng(sz), dtype, sz))
+
+
+@pytest.mark.parametrize("dtype", TYPES)
+@pytest.mark.parametrize("sz", [1, 2, 3, 4, 33, 333, 3333, 4096, 100_003])
+def test_reference_lt_and_by(rk, orc, dtype, sz):
+    """test/hip_rocarray/sorting.jl:20-26: `sort(xd; lt=!isless)`, `xd[sortperm(xd; lt=!isless)]`, `sort(xd; by=k -> 2k)`,
+    `xd[sortperm(xd; by=k -> 2k)]` against the host's sorts (the reference compares values)."""
+    x = _rand(np.random.default_rng(1000 + sz), dtype, sz)
+    if np.dtype(dtype).kind == "i":
+        x = (x // 4).astype(dtype)                              # 2k stays inside the type, as Julia's Int64 product does
+    xd = rk.ROCArray(x)
+    desc = np.sort(x)[::-1]
+    assert np.array_equal(rk.Array(rk.sort(xd, lt=rk.not_isless)), desc)
+    p = rk.Array(rk.sortperm(xd, lt=rk.not_isless))
+    assert sorted(p.tolist()) == list(range(1, sz + 1)) and np.array_equal(x[p - 1], desc)
+    by = lambda k: 2 * k                                        # noqa: E731
+    asc = np.sort(x)
+    assert np.array_equal(rk.Array(rk.sort(xd, by=by)), asc)
+    p = rk.Array(rk.sortperm(xd, by=by))
+    assert sorted(p.tolist()) == list(range(1, sz + 1)) and np.array_equal(x[p - 1], asc)
+    assert np.array_equal(rk.Array(rk.sort(xd, by=lambda k: -k)), desc)       # a `by` that reverses
+    assert np.array_equal(rk.Array(xd), x)
+    y = rk.ROCArray(x)
+    assert rk.sort_(y, by=by, rev=True) is y and np.array_equal(rk.Array(y), desc)
+    with pytest.raises(NotImplementedError):
+        rk.sort(xd, lt=lambda a, b: a < b)                      # any other comparator: the stock path
 
 
 @pytest.mark.parametrize("dtype", TYPES)
