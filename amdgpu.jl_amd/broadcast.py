@@ -46,6 +46,11 @@ class Broadcasted:
         self.f = f
         self.args = tuple(args)
 
+    def __bool__(self):
+        # `if x > 0:` inside a traced closure would otherwise take the same branch for every element, silently
+        raise L.UnsupportedError(L.RK_ERR_UNSUPPORTED, "truth value of a lazy broadcast: control flow on element values "
+                                 "cannot be traced (ifelse can)")
+
     # arithmetic builds the tree (Julia's dot operators)
     def __add__(self, o): return Broadcasted("+", (self, _leaf(o)))
     def __radd__(self, o): return Broadcasted("+", (_leaf(o), self))

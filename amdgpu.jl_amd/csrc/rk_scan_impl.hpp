@@ -2145,7 +2145,10 @@ inline int32_t launch_scan(const ScanArgs& a) {
             // follow: 5 us across the round measured best (2^26 Int32: 0 / 2 / 4 / 6 / 8 / 12 / 16 us -> 91.8 / 90.3 / 89.7 /
             // 89.9 / 90.1 / 90.9 / 92.0 us; 2^27: 177.9 -> 174.0 us; half the round late by a fixed time gained nothing)
             const int64_t resident = ordered_resident(nw * WAVE);
-            const int stagger_tiles = (nw == 16 && ntiles >= 2 * resident) ? (int)resident : 0, stagger_ticks = tune_scan_stagger_ticks();
+            // (narrow elements: half the bytes a tile, half the stagger -- Int16[2^26]: 0 / 1 / 2 / 3 / 4 / 5 / 7 us -> 53.0 / 51.9 / 51.6 /
+            // 51.6 / 51.7 / 52.7 / 53.2 us)
+            const int stagger_tiles = (nw == 16 && ntiles >= 2 * resident) ? (int)resident : 0;
+            const int stagger_ticks = tune_scan_stagger_ticks() * (int)(sizeof(In) + sizeof(Out)) / (int)(2 * sizeof(T));
             const int dyn = ordered_dynamic_ids(ntiles, nw * WAVE, true);
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED

@@ -217,3 +217,7 @@ def test_unsupported_closures(rk):
         rk.mapreduce(lambda v: rk.isodd(v), "add", x)                            # isodd of a Float32
     with pytest.raises(TypeError):
         rk.count(lambda v: v + 1, x)                                             # not a predicate
+    with pytest.raises(rk.UnsupportedError):
+        rk.sum(lambda v: v if v > 0 else -v, x)                                  # a branch on the value: ifelse can be traced, `if` cannot
+    with pytest.raises(rk.UnsupportedError):
+        rk.materialize(rk.lazy(x) if rk.lazy(x) > 0 else -rk.lazy(x))
