@@ -54,6 +54,7 @@ struct BcArgs {
     int32_t   dest_dtype;
     int64_t   dest_stride0;            // element strides of the destination over the merged dims (dense: 1, shape[0], ...)
     int64_t   dest_stride[RK_MAX_DIMS];
+    int32_t   post;                    // fused evaluators: 0, or the token applied to the result of every operation (RK_BC_ROUND_F16)
 };
 
 // ---- typed loads / stores --------------------------------------------------------------------------
@@ -185,12 +186,41 @@ template <int NOPS_> struct EvalInterpN {
 typedef EvalInterpN<RK_MAX_OPERANDS> EvalInterp;
 typedef EvalInterpN<4> EvalInterp4;
 
+// Programs over Float16 arrays are Float32 programs with RK_BC_ROUND_F16 behind every operation (Julia's Float16
+// arithmetic: compute in Float32, round).  The planner takes those tokens out when they follow EVERY operation
+// (strip_post) and the fused evaluators round each intermediate instead, so x .+ y, a .* x .+ y and the chains of
+// Float16 arrays run here and not in the interpreter, which is bound by its instructions at two bytes an element
+// (x .+ y of Float16[2^26]: 172 us).  One scalar branch per operation.
+template <typename CT, int VEC>
+__device__ __forceinline__ void bc_post(int post, CT (&v)[VEC]) {
+    if constexpr (std::is_same<CT, float>::value) {
+        if (post == RK_BC_ROUND_F16) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[j] = (CT)(half_t)v[j];
+        }
+    }
+}
+
 // z = a * x + y * exp(w)            tokens: 0 1 MUL 2 3 EXP MUL ADD
 struct EvalAxpbyExp {
     static constexpr int NOPS = 4;
     static constexpr bool USES_LDS = false;
     template <typename CT, int VEC, typename A>
-    static __device__ __forceinline__ void run(const A&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        if (a.post != 0) {
+            CT p[VEC], q[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { p[j] = in[0][j] * in[1][j]; q[j] = exp(in[3][j]); }
+            bc_post<CT, VEC>(a.post, p);
+            bc_post<CT, VEC>(a.post, q);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) q[j] = in[2][j] * q[j];
+            bc_post<CT, VEC>(a.post, q);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = p[j] + q[j];
+            bc_post<CT, VEC>(a.post, out);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = in[0][j] * in[1][j] + in[2][j] * exp(in[3][j]);
     }
@@ -200,7 +230,17 @@ struct EvalAddMul {
     static constexpr int NOPS = 3;
     static constexpr bool USES_LDS = false;
     template <typename CT, int VEC, typename A>
-    static __device__ __forceinline__ void run(const A&, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        if (a.post != 0) {
+            CT p[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) p[j] = in[1][j] * in[2][j];
+            bc_post<CT, VEC>(a.post, p);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) out[j] = in[0][j] + p[j];
+            bc_post<CT, VEC>(a.post, out);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < VEC; ++j) out[j] = in[0][j] + in[1][j] * in[2][j];
     }
@@ -230,6 +270,14 @@ struct EvalBinary {
             case RK_BC_MUL: RK_BC_BIN2(x * y);
             case RK_BC_MAX: RK_BC_BIN2(OpMax()(x, y));
             case RK_BC_MIN: RK_BC_BIN2(OpMin()(x, y));
+            case RK_BC_LT: RK_BC_BIN2(x < y ? CT(1) : CT(0));
+            case RK_BC_LE: RK_BC_BIN2(x <= y ? CT(1) : CT(0));
+            case RK_BC_GT: RK_BC_BIN2(x > y ? CT(1) : CT(0));
+            case RK_BC_GE: RK_BC_BIN2(x >= y ? CT(1) : CT(0));
+            case RK_BC_EQ: RK_BC_BIN2(x == y ? CT(1) : CT(0));
+            case RK_BC_NE: RK_BC_BIN2(x != y ? CT(1) : CT(0));
+            case RK_BC_AND: RK_BC_BIN2(((x != CT(0)) && (y != CT(0))) ? CT(1) : CT(0));
+            case RK_BC_OR: RK_BC_BIN2(((x != CT(0)) || (y != CT(0))) ? CT(1) : CT(0));
             default:
                 if constexpr (std::is_floating_point<CT>::value) {
                     if (a.tokens[2] == RK_BC_DIV) {
@@ -243,6 +291,7 @@ struct EvalBinary {
                 break;
         }
 #undef RK_BC_BIN2
+        bc_post<CT, VEC>(a.post, out);
     }
 };
 
@@ -297,11 +346,14 @@ struct EvalChain2 {
         CT t[VEC];
         if (a.tokens[3] == 2) {                     // (u op1 v) op2 w
             apply<CT, VEC>(a.tokens[2], in[0], in[1], t);
+            bc_post<CT, VEC>(a.post, t);
             apply<CT, VEC>(a.tokens[4], t, in[2], out);
         } else {                                    // u op1 (v op2 w)
             apply<CT, VEC>(a.tokens[3], in[1], in[2], t);
+            bc_post<CT, VEC>(a.post, t);
             apply<CT, VEC>(a.tokens[4], in[0], t, out);
         }
+        bc_post<CT, VEC>(a.post, out);
     }
 };
 
@@ -343,6 +395,7 @@ template <int NOPS_> struct EvalLeftChainN {
             if (k < a.n_operands) {
                 CT r[VEC];
                 EvalChain2::apply<CT, VEC>(a.tokens[2 * k], acc, in[k], r);
+                bc_post<CT, VEC>(a.post, r);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) acc[j] = r[j];
             }
@@ -455,6 +508,7 @@ struct BcFlatArgs {
     uint64_t    scalar[RK_MAX_OPERANDS];    // bits of the value in the compute type
     int32_t     n_operands, n_tokens;
     int32_t     tokens[RK_MAX_PROGRAM];
+    int32_t     post;                  // always 0: the lean kernel runs homogeneous programs, which round nowhere
 };
 constexpr int BC_FLAT_BLOCK = 64;
 
@@ -646,6 +700,27 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
             return RK_SUCCESS;
         }
     }
+    // Arrays of 1- and 2-byte elements only (Float16, Int16, Bool ...): four elements a lane are 8 or 4 bytes a request,
+    // too little to keep memory busy (copy of Int16[2^26] 4.9 TB/s, of Int8 3.7); eight a lane here.  The fused
+    // evaluators only -- the interpreter's value stack is laid out for four.
+    if constexpr (!Eval::USES_LDS) {
+        if (!rows && vec && !homog && a.indexed == 0 && a.total % 8 == 0 && dtype_size((rk_dtype)a.dest_dtype) <= 2 &&
+            is_aligned(a.dest, 8 * dtype_size((rk_dtype)a.dest_dtype))) {
+            bool narrow = true;
+            for (int k = 0; k < a.n_operands; ++k) {
+                const BcOperand& o = a.op[k];
+                if (o.ptr == nullptr) continue;
+                if (dtype_size((rk_dtype)o.dtype) > 2 || (o.stride0 == 1 && !is_aligned(o.ptr, 8 * dtype_size((rk_dtype)o.dtype)))) narrow = false;
+            }
+            if (narrow) {
+                const int64_t blocks = (a.total / 8 + BC_BLOCK - 1) / BC_BLOCK;
+                if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+                bc_kernel<Eval, CT, 8, false, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+                RK_LAUNCH_CHECK();
+                return RK_SUCCESS;
+            }
+        }
+    }
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
     if (a.indexed != 0) {            // the planner sets it together with vec and rows
         const int64_t blocks = ((a.total + 3) / 4 + BC_BLOCK - 1) / BC_BLOCK;
@@ -671,14 +746,41 @@ static bool tokens_are(const BcArgs& a, std::initializer_list<int> want) {
     return true;
 }
 
+// True: `c` is `a` without its RK_BC_ROUND_F16 tokens, which stood behind every operation and nowhere else, and
+// c.post says so: the same program for an evaluator that rounds every intermediate (bc_post).
+static bool strip_post(const BcArgs& a, BcArgs& c) {
+    int n = 0, ops = 0, posts = 0;
+    int32_t t[RK_MAX_PROGRAM];
+    for (int i = 0; i < a.n_tokens; ++i) {
+        const int tok = a.tokens[i];
+        if (tok == RK_BC_ROUND_F16) {
+            if (i == 0 || a.tokens[i - 1] < RK_BC_ADD || a.tokens[i - 1] == RK_BC_ROUND_F16) return false;   // behind an operand, or twice
+            ++posts;
+            continue;
+        }
+        if (tok >= RK_BC_ADD) ++ops;                 // operand and constant slots lie below the first operator token
+        t[n++] = tok;
+    }
+    if (posts == 0 || posts != ops) return false;
+    c = a;
+    c.n_tokens = n;
+    for (int i = 0; i < n; ++i) c.tokens[i] = t[i];
+    c.post = RK_BC_ROUND_F16;
+    return true;
+}
+
+// The programs with an evaluator of their own; `taken` = false: none of them.
 template <typename CT>
-static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
+static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool& taken) {
+    taken = true;
     if constexpr (std::is_floating_point<CT>::value) {
         if (tokens_are(a, {0, 1, RK_BC_MUL, 2, 3, RK_BC_EXP, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAxpbyExp, CT>(a, vec, rows, stream);
     }
     if (tokens_are(a, {0, 1, 2, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAddMul, CT>(a, vec, rows, stream);
     if (tokens_are(a, {0})) return bc_launch<EvalCopy, CT>(a, vec, rows, stream);
-    if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 && a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW)
+    if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 &&
+        ((a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW && !(!std::is_floating_point<CT>::value && (a.tokens[2] == RK_BC_DIV || a.tokens[2] == RK_BC_POW))) ||
+         (a.tokens[2] >= RK_BC_LT && a.tokens[2] <= RK_BC_OR)))
         return bc_launch<EvalBinary, CT>(a, vec, rows, stream);
     {
         BcArgs c;
@@ -689,6 +791,23 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
             return bc_launch<EvalLeftChainN<8>, CT>(c, vec, rows, stream);
         }
     }
+    taken = false;
+    return RK_SUCCESS;
+}
+
+template <typename CT>
+static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
+    bool taken = false;
+    if constexpr (std::is_same<CT, float>::value) {
+        // a Float16 program whose every operation rounds: the fused evaluators take it without the rounding tokens
+        BcArgs stripped;
+        if (a.post == 0 && strip_post(a, stripped)) {
+            const int32_t st = bc_dispatch_fused<CT>(stripped, vec, rows, stream, taken);
+            if (taken) return st;
+        }
+    }
+    const int32_t st = bc_dispatch_fused<CT>(a, vec, rows, stream, taken);
+    if (taken) return st;
     if (a.n_operands <= EvalInterp4::NOPS) return bc_launch<EvalInterp4, CT>(a, vec, rows, stream);
     return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
 }

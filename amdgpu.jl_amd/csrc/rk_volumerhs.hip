@@ -294,7 +294,7 @@ extern "C" int32_t rk_volumerhs_f32(float* rhs, const float* Q, const float* vge
     if (rhs == nullptr || Q == nullptr || vgeo == nullptr || D == nullptr) return RK_ERR_INVALID_ARGUMENT;
     // whole blocks of four elements with 16-byte accesses when the arrays are aligned for them; the up to three elements
     // that remain (or everything, for unaligned arrays) with the lane-per-node kernel and its 4-byte accesses
-    // Few elements (BASELINE's 4000: every workgroup of either kernel is resident at once) are bound by the latency
+    // Few elements (the 4000 of the small benchmark case: every workgroup of either kernel is resident at once) are bound by the latency
     // of one workgroup, and the lane-per-node kernel with its single barrier is the shorter one: 10.7 against 14.5 us.
     int64_t done = 0;
     if (is_aligned(rhs, 16) && is_aligned(Q, 16) && is_aligned(vgeo, 16) && nelem >= vec_min_elements()) {

@@ -12,7 +12,7 @@ Infinity Cache.  `roofline` is the dominant kernel of the step (the broadcast: 1
 element): algorithmic bytes / average launch duration over K back-to-back launches, HIP events on the
 launch stream.
 
-`configs` lists every BASELINE configuration at its own size, calibration rows (read-only, write-only and
+`configs` lists every benchmark configuration at its own size, calibration rows (read-only, write-only and
 copy kernels through the same entry points: the practical ceilings of the device) and a few extra shapes.
 Per row, the PRIMARY figure (`min_us`, `GBps`, `frac_hbm`, `elements_per_s`) is the minimum over individually
 synchronised launches -- the protocol of the reference's own benchmarks (perf/runbenchmarks.jl:18-23,81-86);
@@ -353,7 +353,7 @@ def main():
             del s_in, c_in, c_out, xs, ys, ws_, zs, ps, pc, pb
             torch.cuda.empty_cache()
 
-    # ---- every BASELINE configuration at its own size ------------------------------------------------------
+    # ---- every benchmark configuration at its own size ------------------------------------------------------
     if not args.no_configs:
         reps = max(10, min(K, 30))
         hx, hi = host.get("x"), host.get("i")
@@ -445,7 +445,13 @@ def main():
             hfo = [rk.ROCArray(dims=(rows, cols), dtype=np.float16) for _ in range(3)]
             pf16 = [plan_accumulate("add", o, x, dims=1) for o, x in zip(hfo, hf)]
             run_row("cumsum(B;dims=1) 4096x16384 Float16 (native narrow scan, 4 B/elt)", rows * cols, 4 * rows * cols, lambda i: pf16[i % 3](), reps)
-            del hf, hfo, pf16
+            # Float16 broadcast: the fused evaluators round every intermediate (Julia's Float16 arithmetic), eight elements a lane
+            hx16 = [dev_array(rand_f32(m).to(torch.float16), (m,), np.float16) for _ in range(3)]
+            hy16 = [dev_array(rand_f32(m).to(torch.float16), (m,), np.float16) for _ in range(3)]
+            hz16 = [rk.ROCArray(dims=(m,), dtype=np.float16) for _ in range(3)]
+            pb16 = [plan_materialize(z, np.float16(0.5) * rk.lazy(x) + rk.lazy(y)) for z, x, y in zip(hz16, hx16, hy16)]
+            run_row("z .= a.*x .+ y Float16[2^26] (6 B/elt)", m, 6 * m, lambda i: pb16[i % 3](), reps)
+            del hf, hfo, pf16, hx16, hy16, hz16, pb16
         # findall: the scan's direct consumer (src/kernels/indexing.jl:8-36); one pass: 1 B/elt read + 8 B per index written
         if wanted("findall"):
             m = 1 << 26

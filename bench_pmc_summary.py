@@ -39,7 +39,7 @@ KNOWN = [
     ("ArgXform<float", None, "cfg2c findmax(A;dims=1) 8192^2", 4 * M26 / KIB, 160.0),
     ("volumerhs_vec_kernel", None, "cfg5 volumerhs! nelem=240000", 240000 * 11000 / KIB, 240000 * 2500 / KIB),
     ("volumerhs_kernel", None, "cfg5 volumerhs! nelem=4000", 4000 * 11000 / KIB, 4000 * 2500 / KIB),
-    # shapes with short or narrow extents, 2^25 elements (the rows bench.py keeps below the BASELINE configurations)
+    # shapes with short or narrow extents, 2^25 elements (the rows bench.py keeps below the benchmark configurations)
     ("reduce_short_lines_kernel", None, "sum(A; dims=1) 32x1048576 / sum(A; dims=2) 4x32x262144", 4 * N25 / KIB, 4 * (N25 // 32) / KIB),
     ("scan_lds_lines_kernel<float", None, "cumsum(A; dims=1) 15x2236962", 4 * N15 / KIB, 4 * N15 / KIB),
     ("bc_indexed_kernel<EvalBinary", None, "C .= A .+ r 3x11184810 .+ 1x11184810", (4 * N3 + 4 * (N3 // 3)) / KIB, 4 * N3 / KIB),

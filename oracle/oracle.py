@@ -534,7 +534,7 @@ def _jl_extrude(a, nd):
 
 
 def broadcast_axpby_exp(a, x, y, w):
-    """``z .= a .* x .+ y .* exp.(w)`` in Float64 (BASELINE config 4a)."""
+    """``z .= a .* x .+ y .* exp.(w)`` in Float64 (benchmark configuration 4a)."""
     x, y, w = (np.asarray(v, dtype=np.float64) for v in (x, y, w))
     nd = max(x.ndim, y.ndim, w.ndim)
     return float(a) * _jl_extrude(x, nd) + _jl_extrude(y, nd) * np.exp(_jl_extrude(w, nd))
@@ -703,7 +703,7 @@ def volumerhs_loops(rhs, Q, vgeo, gravity, D):
 # ---------------------------------------------------------------------------
 
 def config_inputs(name: str, scale: float = 1.0):
-    """Seeded inputs for the BASELINE configurations (NumPy ``default_rng(seed)``).
+    """Seeded inputs for the benchmark configurations (NumPy ``default_rng(seed)``).
 
     ``scale`` < 1 shrinks the problem (tests at sizes the oracle finishes in seconds).
     The same host buffer feeds both the device path and the oracle, so no cross-language

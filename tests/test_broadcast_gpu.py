@@ -324,6 +324,51 @@ def test_float16_arrays(rk):
     assert isinstance(s, np.float16) and abs(float(s) - float((x * x).astype(np.float64).sum())) <= 2.0**-9 * float((x * x).astype(np.float64).sum())
 
 
+@pytest.mark.parametrize("shape", [(1 << 16,), (4100,), (4096 + 8,), (256, 96), (130, 67)])
+def test_narrow_arrays_in_the_fused_evaluators(rk, shape):
+    """Float16 programs whose every operation rounds run in the fused evaluators (the rounding tokens become a rounding of
+    every intermediate), eight elements a lane where sizes and alignment allow; comparisons and logic of two arrays too.
+    Bit-identical to NumPy's Float16 arithmetic, whichever kernel a shape selects."""
+    rng = _rng(29)
+    h = np.float16
+    x = rng.standard_normal(shape).astype(h)
+    y = (rng.random(shape) + 0.5).astype(h)
+    w = (rng.standard_normal(shape) * 0.5).astype(h)
+    g = (rng.random(shape) + 1.0).astype(h)
+    X, Y, W, G = (rk.ROCArray(a) for a in (x, y, w, g))
+    lz = rk.lazy
+    cases = [
+        (lz(X) + lz(Y), x + y), (lz(X) - lz(Y), x - y), (lz(X) * lz(Y), x * y), (lz(X) / lz(Y), x / y),
+        (rk.broadcast.max_(lz(X), lz(Y)), np.maximum(x, y)),
+        (h(1.5) * lz(X) + lz(Y), h(1.5) * x + y),                          # (u op v) op w
+        (lz(X) + lz(Y) * lz(W), x + y * w),                                # u op (v op w)
+        ((lz(X) - lz(W)) / lz(Y) * lz(G) + lz(W), (x - w) / y * g + w),      # a left chain of five operands
+    ]
+    for bc, want in cases:
+        got = rk.materialize(bc)
+        assert got.dtype == h
+        np.testing.assert_array_equal(rk.Array(got), want.astype(h))
+    got = rk.Array(rk.materialize(h(0.5) * lz(X) + lz(Y) * rk.broadcast.exp(lz(W))))
+    e = np.exp(w.astype(np.float32)).astype(h)                             # exp itself within an ulp of Float16; the rest exact
+    lo = h(0.5) * x + y * np.nextafter(e, h(-np.inf)); hi = h(0.5) * x + y * np.nextafter(e, h(np.inf))
+    assert np.all((got >= np.minimum(lo, hi)) & (got <= np.maximum(lo, hi)))
+    # Bool results of comparisons, logic of Bool arrays, Int16 arithmetic and order
+    a = rng.integers(-300, 300, shape).astype(np.int16)
+    b = rng.integers(-300, 300, shape).astype(np.int16)
+    p = rng.random(shape) < 0.5
+    q = rng.random(shape) < 0.5
+    A, B, P, Q = (rk.ROCArray(v) for v in (a, b, p, q))
+    for bc, want in [(lz(X) > lz(Y), x > y), (lz(X) <= lz(W), x <= w), (lz(A) < lz(B), a < b), (lz(A) == lz(B), a == b), (lz(A) != lz(B), a != b),
+                     (lz(P) & lz(Q), p & q), (lz(P) | lz(Q), p | q), (lz(A) >= lz(B), a >= b)]:
+        got = rk.materialize(bc)
+        assert got.dtype == np.bool_
+        np.testing.assert_array_equal(rk.Array(got), want)
+    for bc, want in [(lz(A) + lz(B), a + b), (lz(A) * lz(B), a * b), (rk.broadcast.min_(lz(A), lz(B)), np.minimum(a, b)), (lz(A) - lz(B) * lz(A), a - b * a)]:
+        got = rk.materialize(bc)
+        assert got.dtype == np.int16
+        np.testing.assert_array_equal(rk.Array(got), want.astype(np.int16))
+
+
 @pytest.mark.parametrize("shape,others", [((3, 40_000), [(3, 1), (1, 40_000)]), ((17, 4000), [(17, 1), (1, 4000)]), ((5, 7, 800), [(5, 1, 800), (1, 7, 1)]),
                                           ((2, 2, 2, 30_000), [(2, 1, 2, 1), (1, 2, 1, 30_000)]), ((6, 10_002), [(1, 10_002), (6, 10_002)]),
                                           ((63, 4, 100), [(63, 1, 100), (1, 4, 1)]), ((3, 40_001), [(1, 40_001), (3, 1)]), ((17, 4001), [(17, 1), (1, 4001)]),
