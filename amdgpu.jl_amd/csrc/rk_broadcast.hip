@@ -55,6 +55,7 @@ struct BcArgs {
     int64_t   dest_stride0;            // element strides of the destination over the merged dims (dense: 1, shape[0], ...)
     int64_t   dest_stride[RK_MAX_DIMS];
     int32_t   post;                    // fused evaluators: 0, or the token applied to the result of every operation (RK_BC_ROUND_F16)
+    int32_t   vecn;                    // elements a lane on the vector path: 4, or 2 when an array has 8-byte elements (16 bytes a lane)
 };
 
 // ---- typed loads / stores --------------------------------------------------------------------------
@@ -502,7 +503,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
 // 6.36 / 6.25 / 6.31 / 6.24 / 6.29 at 2^28 (the plain copy: 6.70 / 6.55 / 6.51 / - / 6.41 at 2^26); two vectors a
 // thread lose 1-3 % at every size, an XCD-banded order of the workgroups changes less than the run-to-run spread.
 struct BcFlatArgs {
-    int64_t     nvec;                       // 4-element vectors
+    int64_t     nvec;                       // 16-byte vectors
     void*       dest;
     const void* ptr[RK_MAX_OPERANDS];       // nullptr: scalar
     uint64_t    scalar[RK_MAX_OPERANDS];    // bits of the value in the compute type
@@ -512,35 +513,42 @@ struct BcFlatArgs {
 };
 constexpr int BC_FLAT_BLOCK = 64;
 
+// A lane moves 16 bytes: four 4-byte or two 8-byte elements.  (Four 8-byte elements a lane are two load instructions
+// that each touch half of every 32 bytes of the wave's 2 KiB: copy of Float64[2^26] 278 us, 3.9 TB/s.)
 template <typename Eval, typename CT, int BLOCK>
 __global__ __launch_bounds__(BLOCK) void bc_flat_kernel(const BcFlatArgs a) {
     CT* lds = (CT*)bc_lds_raw;
-    typedef typename VecOf<CT, 4>::type V;
+    constexpr int FV = 16 / sizeof(CT);
+    typedef typename VecOf<CT, FV>::type V;
     const int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x;
     if (i >= a.nvec) return;
-    CT in[RK_MAX_OPERANDS][4];
+    CT in[RK_MAX_OPERANDS][FV];
 #pragma unroll
     for (int k = 0; k < Eval::NOPS; ++k) {
         if (k >= a.n_operands) continue;
         if (a.ptr[k] != nullptr) {
             const V x = load_nt((const V*)a.ptr[k] + i);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) in[k][j] = x[j];
+            for (int j = 0; j < FV; ++j) in[k][j] = x[j];
         } else {
             CT x;
             __builtin_memcpy(&x, &a.scalar[k], sizeof(CT));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) in[k][j] = x;
+            for (int j = 0; j < FV; ++j) in[k][j] = x;
         }
     }
-    CT out[4];
-    Eval::template run<CT, 4>(a, in, out, lds);
+    CT out[FV];
+    Eval::template run<CT, FV>(a, in, out, lds);
     V o;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) o[j] = out[j];
+    for (int j = 0; j < FV; ++j) o[j] = out[j];
     store_nt((V*)a.dest + i, o);
 }
 
+static int tune_bc_narrow16() {
+    const char* e = std::getenv("RK_BC_NARROW16");
+    return e ? std::atoi(e) : 1;
+}
 static int tune_bc_flat_lean() {
     const char* e = std::getenv("RK_BC_FLAT_LEAN");
     return e ? std::atoi(e) : 1;
@@ -646,7 +654,7 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_indexed_kernel(const BcArgs a) {
 
 template <typename Eval, typename CT>
 static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
-    const int VECN = vec ? 4 : 1;
+    const int VECN = vec ? a.vecn : 1;
     dim3 grid(1, 1, 1);
     if (!rows) {
         const int64_t blocks = (a.total / VECN + BC_BLOCK - 1) / BC_BLOCK;
@@ -678,7 +686,7 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
         if (lean) {
             BcFlatArgs f;
             std::memset(&f, 0, sizeof(f));
-            f.nvec = a.total / 4;
+            f.nvec = a.total / (16 / (int64_t)sizeof(CT));
             f.dest = a.dest;
             f.n_operands = a.n_operands;
             f.n_tokens = a.n_tokens;
@@ -704,17 +712,33 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
     // too little to keep memory busy (copy of Int16[2^26] 4.9 TB/s, of Int8 3.7); eight a lane here.  The fused
     // evaluators only -- the interpreter's value stack is laid out for four.
     if constexpr (!Eval::USES_LDS) {
-        if (!rows && vec && !homog && a.indexed == 0 && a.total % 8 == 0 && dtype_size((rk_dtype)a.dest_dtype) <= 2 &&
-            is_aligned(a.dest, 8 * dtype_size((rk_dtype)a.dest_dtype))) {
+        if (!rows && vec && !homog && a.indexed == 0 && a.total % 8 == 0 && dtype_size((rk_dtype)a.dest_dtype) <= 2) {
+            size_t widest = dtype_size((rk_dtype)a.dest_dtype);
             bool narrow = true;
             for (int k = 0; k < a.n_operands; ++k) {
                 const BcOperand& o = a.op[k];
                 if (o.ptr == nullptr) continue;
-                if (dtype_size((rk_dtype)o.dtype) > 2 || (o.stride0 == 1 && !is_aligned(o.ptr, 8 * dtype_size((rk_dtype)o.dtype)))) narrow = false;
+                if (dtype_size((rk_dtype)o.dtype) > 2) narrow = false;
+                if (dtype_size((rk_dtype)o.dtype) > widest) widest = dtype_size((rk_dtype)o.dtype);
+            }
+            // sixteen where every array has 1-byte elements and the program is small (the operands of a lane are 16 values
+            // of the compute type each)
+            const int W = (widest == 1 && Eval::NOPS <= 2 && a.total % 16 == 0 && tune_bc_narrow16() != 0) ? 16 : 8;
+            if (!is_aligned(a.dest, W * dtype_size((rk_dtype)a.dest_dtype))) narrow = false;
+            for (int k = 0; k < a.n_operands; ++k) {
+                const BcOperand& o = a.op[k];
+                if (o.ptr != nullptr && o.stride0 == 1 && !is_aligned(o.ptr, W * dtype_size((rk_dtype)o.dtype))) narrow = false;
             }
             if (narrow) {
-                const int64_t blocks = (a.total / 8 + BC_BLOCK - 1) / BC_BLOCK;
+                const int64_t blocks = (a.total / W + BC_BLOCK - 1) / BC_BLOCK;
                 if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
+                if constexpr (Eval::NOPS <= 2) {
+                    if (W == 16) {
+                        bc_kernel<Eval, CT, 16, false, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+                        RK_LAUNCH_CHECK();
+                        return RK_SUCCESS;
+                    }
+                }
                 bc_kernel<Eval, CT, 8, false, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
                 RK_LAUNCH_CHECK();
                 return RK_SUCCESS;
@@ -723,10 +747,16 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
     }
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
     if (a.indexed != 0) {            // the planner sets it together with vec and rows
-        const int64_t blocks = ((a.total + 3) / 4 + BC_BLOCK - 1) / BC_BLOCK;
+        const int64_t blocks = ((a.total + VECN - 1) / VECN + BC_BLOCK - 1) / BC_BLOCK;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
-        if (homog) bc_indexed_kernel<Eval, CT, 4, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        if (VECN == 2) {
+            if (homog) bc_indexed_kernel<Eval, CT, 2, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+            else bc_indexed_kernel<Eval, CT, 2, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+        } else if (homog) bc_indexed_kernel<Eval, CT, 4, true><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
         else bc_indexed_kernel<Eval, CT, 4, false><<<(unsigned)blocks, BC_BLOCK, lds, stream>>>(a);
+    } else if (vec && VECN == 2) {
+        if (rows) { if (homog) RK_BC_LAUNCH(2, true, true); else RK_BC_LAUNCH(2, true, false); }
+        else      { if (homog) RK_BC_LAUNCH(2, false, true); else RK_BC_LAUNCH(2, false, false); }
     } else if (vec) {
         if (rows) { if (homog) RK_BC_LAUNCH(4, true, true); else RK_BC_LAUNCH(4, true, false); }
         else      { if (homog) RK_BC_LAUNCH(4, false, true); else RK_BC_LAUNCH(4, false, false); }
@@ -968,9 +998,16 @@ static int32_t broadcast_impl(const rk_program* prog, void* dest, rk_dtype dest_
             for (int d = m; d < BC_INDEXED_DIMS; ++d) a.shape[d] = 1;
         }
     }
+    // 16 bytes a lane: two elements where an array has 8-byte elements (four would be two load instructions that each touch
+    // half of every 32 bytes the wave covers: C .= A .+ r .* c on 8192^2 Float64 5.1 TB/s against 6.1 for Float32)
+    a.vecn = 4;
+    if (dtype_size(dest_dtype) == 8) a.vecn = 2;
+    for (int k = 0; k < prog->n_operands; ++k)
+        if (prog->operands[k].ptr != nullptr && dtype_size(prog->operands[k].dtype) == 8) a.vecn = 2;
     if (!linear) {
         // lanes along dim 0: TX = smallest power of two covering shape[0] / VEC, at most the workgroup
-        const int64_t n0v = (mshape[0] + (vec ? 4 : 1) - 1) / (vec ? 4 : 1);
+        const int vw = vec ? a.vecn : 1;
+        const int64_t n0v = (mshape[0] + vw - 1) / vw;
         int l2 = 0;
         while ((1 << l2) < BC_BLOCK && (1ll << l2) < n0v) ++l2;
         a.tx_log2 = l2;

@@ -451,7 +451,13 @@ def main():
             hz16 = [rk.ROCArray(dims=(m,), dtype=np.float16) for _ in range(3)]
             pb16 = [plan_materialize(z, np.float16(0.5) * rk.lazy(x) + rk.lazy(y)) for z, x, y in zip(hz16, hx16, hy16)]
             run_row("z .= a.*x .+ y Float16[2^26] (6 B/elt)", m, 6 * m, lambda i: pb16[i % 3](), reps)
-            del hf, hfo, pf16, hx16, hy16, hz16, pb16
+            # 8-byte elements: two a lane (16 bytes), not four
+            hx64 = [dev_array(rand_f32(m).to(torch.float64), (m,), np.float64) for _ in range(2)]
+            hy64 = [dev_array(rand_f32(m).to(torch.float64), (m,), np.float64) for _ in range(2)]
+            hz64 = [rk.ROCArray(dims=(m,), dtype=np.float64) for _ in range(2)]
+            pb64 = [plan_materialize(z, np.float64(0.5) * rk.lazy(x) + rk.lazy(y)) for z, x, y in zip(hz64, hx64, hy64)]
+            run_row("z .= a.*x .+ y Float64[2^26] (24 B/elt)", m, 24 * m, lambda i: pb64[i % 2](), reps)
+            del hf, hfo, pf16, hx16, hy16, hz16, pb16, hx64, hy64, hz64, pb64
         # findall: the scan's direct consumer (src/kernels/indexing.jl:8-36); one pass: 1 B/elt read + 8 B per index written
         if wanted("findall"):
             m = 1 << 26
