@@ -433,7 +433,7 @@ def main():
                     cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_dims2_f32(P(hx), I64(rows), I64(cols), P(hz), t), 8 * rows * cols, "full size"))
             del Bi, Bo, pa, pb
         # scans of 2-byte elements, native (read narrow, scanned in 32 bits, stored narrow): 4 bytes of traffic per element
-        if wanted("Int16") or wanted("Float16"):
+        if wanted("Int16") or wanted("Float16") or wanted("Float64"):
             m = 1 << 26
             hi16 = [dev_array(randint_i32(m).to(torch.int16), (m,), np.int16) for _ in range(3)]
             ho16 = [rk.ROCArray(dims=(m,), dtype=np.int16) for _ in range(3)]

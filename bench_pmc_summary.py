@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """HBM traffic per kernel from two rocprofv3 counter runs of bench.py (FETCH_SIZE, then WRITE_SIZE).
 
-    ONLY='sum Float32[2^26]|maximum|cumsum Int32[2^26]|z .= a.*x .+ y.*exp.(w) Float32[2^26]|calibration: copy z .= x Float32[2^26]|cfg2|cfg3|cumsum(B;dims=2)|cfg4|cfg5|Int16|sum(A; dims=|cumsum(A; dims=1) 15x|C .= A .+ r 3x|permutedims|reverse|findall'
+    ONLY='sum Float32[2^26]|maximum|cumsum Int32[2^26]|z .= a.*x .+ y.*exp.(w) Float32[2^26]|calibration: copy z .= x Float32[2^26]|cfg2|cfg3|cumsum(B;dims=2)|cfg4|cfg5|Int16|Float16|Float64|sum(A; dims=|cumsum(A; dims=1) 15x|C .= A .+ r 3x|permutedims|reverse|findall'
     rocprofv3 --pmc FETCH_SIZE --kernel-trace --output-format csv -d F -o bench -- python3 bench.py --no-cpu --steps 5 --only "$ONLY"
     rocprofv3 --pmc WRITE_SIZE --kernel-trace --output-format csv -d W -o bench -- python3 bench.py --no-cpu --steps 5 --only "$ONLY"
     python bench_pmc_summary.py F/bench W/bench > profiles/<name>.txt
@@ -30,6 +30,8 @@ KNOWN = [
     ("scan_ordered_kernel<int", 2097152, "cumsum Int32[2^26]", 4 * M26 / KIB, 4 * M26 / KIB),
     ("scan_ordered_kernel<int", 4194304, "cfg3a cumsum Int32[2^27]", 4 * M27 / KIB, 4 * M27 / KIB),
     ("scan_ordered_kernel<short", None, "cumsum Int16[2^26] (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),
+    ("bc_kernel<EvalChain2, float, 8", None, "z .= a.*x .+ y Float16[2^26] (6 B/elt)", 4 * M26 / KIB, 2 * M26 / KIB),
+    ("bc_flat_kernel<EvalChain2, double", None, "z .= a.*x .+ y Float64[2^26] (24 B/elt)", 16 * M26 / KIB, 8 * M26 / KIB),
     ("scan_tiles_kernel<float", None, "cfg3b cumsum(B;dims=1) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
     ("scan_tiles_kernel<_Float16", None, "cumsum(B;dims=1) 4096x16384 Float16 (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),
     ("scan_rows_ordered_kernel<float", None, "cumsum(B;dims=2) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
