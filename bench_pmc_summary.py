@@ -33,6 +33,7 @@ KNOWN = [
     ("bc_kernel<EvalChain2, float, 8", None, "z .= a.*x .+ y Float16[2^26] (6 B/elt)", 4 * M26 / KIB, 2 * M26 / KIB),
     ("bc_flat_kernel<EvalChain2, double", None, "z .= a.*x .+ y Float64[2^26] (24 B/elt)", 16 * M26 / KIB, 8 * M26 / KIB),
     ("scan_tiles_kernel<float", None, "cfg3b cumsum(B;dims=1) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
+    ("scan_tiles_kernelIDF16_", None, "cumsum(B;dims=1) 4096x16384 Float16 (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),   # (left mangled by the profiler)
     ("scan_tiles_kernel<_Float16", None, "cumsum(B;dims=1) 4096x16384 Float16 (native narrow scan, 4 B/elt)", 2 * M26 / KIB, 2 * M26 / KIB),
     ("scan_rows_ordered_kernel<float", None, "cumsum(B;dims=2) 4096x16384", 4 * M26 / KIB, 4 * M26 / KIB),
     ("MapIdentity>, OpAdd, ReduceSink<float, OpAdd, float>, true", 131072, "sum Float32 (2^26: 262144 KiB; the 2^24 row shares this grid)", None, None),
