@@ -60,7 +60,11 @@ class Broadcasted:
     def __rmul__(self, o): return Broadcasted("*", (_leaf(o), self))
     def __truediv__(self, o): return Broadcasted("/", (self, _leaf(o)))
     def __rtruediv__(self, o): return Broadcasted("/", (_leaf(o), self))
-    def __pow__(self, o): return Broadcasted("^", (self, _leaf(o)))
+    def __pow__(self, o):
+        # a literal 2 is Base.literal_pow(^, x, Val(2)) = x * x in Julia, not a call of pow
+        if type(o) is int and o == 2:
+            return Broadcasted("abs2", (self,))
+        return Broadcasted("^", (self, _leaf(o)))
     def __neg__(self): return Broadcasted("neg", (self,))
     # comparisons and logic (.<  .==  .&  .!): Bool-valued nodes
     def __lt__(self, o): return Broadcasted("<", (self, _leaf(o)))

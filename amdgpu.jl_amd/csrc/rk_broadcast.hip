@@ -173,12 +173,12 @@ template <typename CT, int VEC, int NOPS_> struct BcFetch {
         for (int j = 0; j < VEC; ++j) v[j] = in[K][j];
     }
 };
-template <int NOPS_> struct EvalInterpN {
+template <int NOPS_, bool FULL_ = true> struct EvalInterpN {
     static constexpr int NOPS = NOPS_;             // operand slots: load what the program declares, up to this many
     static constexpr bool USES_LDS = true;
     template <typename CT, int VEC, typename A>
     static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT* lds) {
-        interp_run<CT, VEC, BC_BLOCK, true>(a.tokens, a.n_tokens, BcFetch<CT, VEC, NOPS_>{in}, out, lds);
+        interp_run<CT, VEC, BC_BLOCK, FULL_>(a.tokens, a.n_tokens, BcFetch<CT, VEC, NOPS_>{in}, out, lds);
     }
 };
 // Programs over at most 4 operands (most) run a copy with half the operand registers: in rows mode it can then keep
@@ -186,6 +186,9 @@ template <int NOPS_> struct EvalInterpN {
 // bound by load latency ((A .- r) .* c .+ A on 16384^2: 1.6 TB/s).
 typedef EvalInterpN<RK_MAX_OPERANDS> EvalInterp;
 typedef EvalInterpN<4> EvalInterp4;
+// Without pow, sin, cos and tanh -- the routines that set the interpreter's register count (89 with them: five waves a
+// SIMD) -- for the programs that use none of them.
+typedef EvalInterpN<4, false> EvalInterp4Light;
 
 // Programs over Float16 arrays are Float32 programs with RK_BC_ROUND_F16 behind every operation (Julia's Float16
 // arithmetic: compute in Float32, round).  The planner takes those tokens out when they follow EVERY operation
@@ -406,6 +409,235 @@ template <int NOPS_> struct EvalLeftChainN {
     }
 };
 
+// dest = g2(g1(f0b(f0a(u)) op f1b(f1a(v))))  or  g2(g1(f0b(f0a(u))))
+// One or two operands with up to two unary functions each, a binary operator, up to two unary functions of the result:
+// exp.(x), -x, sqrt.(abs.(x)), x .* x, abs2.(x) .+ abs2.(y), 1 ./ (1 .+ exp.(.-x)), abs2.(x .- y).  The host parses the
+// postfix program into this shape (tree2_canonical) and passes seven codes in place of the tokens -- 0 = nothing -- so
+// the kernel runs a fixed sequence of scalar branches and keeps no value stack: the interpreter moves its four register
+// slots on every push and pop, some 200 instructions a vector for -x, which is what bounds it once an element has
+// two bytes (-x of Float16[2^26]: 76 us, as long as for Float32).  v == u: one load (the host leaves one operand and
+// sets the eighth code).  FULL = false leaves out pow, sin, cos, tanh, whose routines set the register count.
+// A "unary function" may also be a binary operator with a scalar: c op t or t op c (1 ./ t, 1 .+ t, a .* x): up to two
+// such scalars travel as operands 2 and 3, and the code of the slot says which and on which side
+// (token | (operand + 1) << 8 | scalar_on_the_left << 16).  So a .* x .+ b .* y and 1 ./ (1 .+ exp.(.-x)) are trees of
+// this form as well.
+enum { T2_F0A = 0, T2_F0B, T2_F1A, T2_F1B, T2_OP, T2_G1, T2_G2, T2_SAME, T2_CODES };
+template <bool FULL, int NOPS_> struct EvalTree2T {        // NOPS_ = 2: no scalar slots
+    static constexpr int NOPS = NOPS_;
+    static constexpr bool USES_LDS = false;
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void unary(int tok, int post, CT (&v)[VEC]) {
+        if (tok == 0) return;
+#define RK_T2_UN(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT x = v[j]; v[j] = (EXPR); } } break
+        switch (tok) {
+            case RK_BC_NEG: RK_T2_UN(-x);
+            case RK_BC_ABS: RK_T2_UN(x < CT(0) ? -x : (x == CT(0) ? CT(0) : x));
+            case RK_BC_ABS2: RK_T2_UN(x * x);
+            case RK_BC_NOT: RK_T2_UN(x == CT(0) ? CT(1) : CT(0));
+            default:
+                if constexpr (std::is_floating_point<CT>::value) {
+                    switch (tok) {
+                        case RK_BC_SQRT: RK_T2_UN(sqrt(x));
+                        case RK_BC_EXP: RK_T2_UN(exp(x));
+                        case RK_BC_LOG: RK_T2_UN(log(x));
+                        case RK_BC_INV: RK_T2_UN(CT(1) / x);
+                        case RK_BC_ISNAN: RK_T2_UN(x != x ? CT(1) : CT(0));
+                        case RK_BC_ROUND_F16: RK_T2_UN((CT)(half_t)x);      // a program that rounds in some places only
+                        default:
+                            if constexpr (FULL) {
+                                switch (tok) {
+                                    case RK_BC_SIN: RK_T2_UN(sin(x));
+                                    case RK_BC_COS: RK_T2_UN(cos(x));
+                                    case RK_BC_TANH: RK_T2_UN(tanh(x));
+                                    default: break;
+                                }
+                            }
+                            break;
+                    }
+                } else {
+                    switch (tok) {
+                        case RK_BC_ISODD: RK_T2_UN(x & CT(1));
+                        case RK_BC_ISEVEN: RK_T2_UN((x & CT(1)) ^ CT(1));
+                        case RK_BC_ISNAN: RK_T2_UN(x * CT(0));
+                        case RK_BC_WRAP_I32: RK_T2_UN((CT)(int32_t)x);
+                        case RK_BC_WRAP_U32: RK_T2_UN((CT)(uint32_t)x);
+                        case RK_BC_WRAP_I8: RK_T2_UN((CT)(int8_t)x);
+                        case RK_BC_WRAP_U8: RK_T2_UN((CT)(uint8_t)x);
+                        case RK_BC_WRAP_I16: RK_T2_UN((CT)(int16_t)x);
+                        case RK_BC_WRAP_U16: RK_T2_UN((CT)(uint16_t)x);
+                        default: break;
+                    }
+                }
+                break;
+        }
+#undef RK_T2_UN
+        bc_post<CT, VEC>(post, v);
+    }
+    template <typename CT, int VEC>
+    static __device__ __forceinline__ void binary(int tok, CT (&x)[VEC], const CT (&y)[VEC]) {
+#define RK_T2_BIN(EXPR) { _Pragma("unroll") for (int j = 0; j < VEC; ++j) { const CT p = x[j], q = y[j]; x[j] = (EXPR); } } break
+        switch (tok) {
+            case RK_BC_ADD: RK_T2_BIN(p + q);
+            case RK_BC_SUB: RK_T2_BIN(p - q);
+            case RK_BC_MUL: RK_T2_BIN(p * q);
+            case RK_BC_MAX: RK_T2_BIN(OpMax()(p, q));
+            case RK_BC_MIN: RK_T2_BIN(OpMin()(p, q));
+            case RK_BC_LT: RK_T2_BIN(p < q ? CT(1) : CT(0));
+            case RK_BC_LE: RK_T2_BIN(p <= q ? CT(1) : CT(0));
+            case RK_BC_GT: RK_T2_BIN(p > q ? CT(1) : CT(0));
+            case RK_BC_GE: RK_T2_BIN(p >= q ? CT(1) : CT(0));
+            case RK_BC_EQ: RK_T2_BIN(p == q ? CT(1) : CT(0));
+            case RK_BC_NE: RK_T2_BIN(p != q ? CT(1) : CT(0));
+            case RK_BC_AND: RK_T2_BIN(((p != CT(0)) && (q != CT(0))) ? CT(1) : CT(0));
+            case RK_BC_OR: RK_T2_BIN(((p != CT(0)) || (q != CT(0))) ? CT(1) : CT(0));
+            default:
+                if constexpr (std::is_floating_point<CT>::value) {
+                    if (tok == RK_BC_DIV) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) x[j] = x[j] / y[j];
+                    } else if constexpr (FULL) {       // RK_BC_POW
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) x[j] = pow(x[j], y[j]);
+                    }
+                }
+                break;
+        }
+#undef RK_T2_BIN
+    }
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        // one slot: a unary function, or a binary operator with the scalar in operand 2 or 3
+        auto slot = [&](int code, CT (&v)[VEC]) {
+            const int k = (code >> 8) & 0xff;
+            if (NOPS_ < 4 || k == 0) { unary<CT, VEC>(code, a.post, v); return; }
+            if constexpr (NOPS_ >= 4) {
+                CT c[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) c[j] = k == 3 ? in[2][j] : in[3][j];
+                if ((code >> 16) != 0) {            // c op v
+                    binary<CT, VEC>(code & 0xff, c, v);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) v[j] = c[j];
+                } else {
+                    binary<CT, VEC>(code & 0xff, v, c);
+                }
+                bc_post<CT, VEC>(a.post, v);
+            }
+        };
+        CT x[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[j] = in[0][j];
+        slot(a.tokens[T2_F0A], x);
+        slot(a.tokens[T2_F0B], x);
+        if (a.tokens[T2_OP] != 0) {
+            CT y[VEC];
+            if (a.tokens[T2_SAME] != 0) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) y[j] = in[0][j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) y[j] = in[1][j];
+            }
+            slot(a.tokens[T2_F1A], y);
+            slot(a.tokens[T2_F1B], y);
+            binary<CT, VEC>(a.tokens[T2_OP], x, y);
+            bc_post<CT, VEC>(a.post, x);
+        }
+        slot(a.tokens[T2_G1], x);
+        slot(a.tokens[T2_G2], x);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = x[j];
+    }
+    // true: `c` is `a` in this evaluator's form; `full`: the program needs pow, sin, cos or tanh
+    static bool canonical(const BcArgs& a, BcArgs& c, bool& full) {
+        struct Node { int kind, tok, l, r; };        // kind 0: operand `tok`; 1: unary of l; 2: binary of l, r
+        Node nodes[RK_MAX_PROGRAM];
+        int stack[RK_MAX_PROGRAM], sp = 0, nn = 0;
+        full = false;
+        for (int i = 0; i < a.n_tokens; ++i) {
+            const int tok = a.tokens[i];
+            if (tok >= 0 && tok < RK_MAX_OPERANDS) { nodes[nn] = Node{0, tok, -1, -1}; stack[sp++] = nn++; continue; }
+            const int ar = token_arity(tok);
+            if (tok == RK_BC_IDENTITY) continue;
+            if (!token_basic(tok)) full = true;
+            if (ar == 1 && sp >= 1) { nodes[nn] = Node{1, tok, stack[sp - 1], -1}; stack[sp - 1] = nn++; }
+            else if (ar == 2 && sp >= 2) { nodes[nn] = Node{2, tok, stack[sp - 2], stack[sp - 1]}; sp -= 1; stack[sp - 1] = nn++; }
+            else return false;                      // muladd, ifelse: the interpreter's
+        }
+        if (sp != 1) return false;
+        // unary functions -- and binary operators with a scalar -- from `n` down to the first node that is neither:
+        // innermost first in f[] (as slot codes); returns that node
+        int scalars[2], nscalars = 0;               // operands of `a` that travel as operands 2 and 3
+        auto is_scalar = [&](int n) { return nodes[n].kind == 0 && a.op[nodes[n].tok].ptr == nullptr; };
+        auto peel = [&](int n, int (&f)[4], int& nf, int limit) -> int {
+            int outer_first[4];
+            nf = 0;
+            for (;;) {
+                int code, next;
+                if (nodes[n].kind == 1) { code = nodes[n].tok; next = nodes[n].l; }
+                else if (nodes[n].kind == 2 && (is_scalar(nodes[n].l) != is_scalar(nodes[n].r) ||
+                                                (is_scalar(nodes[n].l) && is_scalar(nodes[n].r)))) {
+                    const bool left = is_scalar(nodes[n].l) && !is_scalar(nodes[n].r);     // the scalar is the left argument
+                    const int sc = nodes[left ? nodes[n].l : nodes[n].r].tok;
+                    int k = -1;
+                    for (int i = 0; i < nscalars; ++i) if (scalars[i] == sc) k = i;
+                    if (k < 0) { if (nscalars == 2) return -1; scalars[nscalars] = sc; k = nscalars++; }
+                    code = nodes[n].tok | ((k + 3) << 8) | ((left ? 1 : 0) << 16);
+                    next = left ? nodes[n].r : nodes[n].l;
+                } else break;
+                if (nf == limit) return -1;
+                outer_first[nf++] = code;
+                n = next;
+            }
+            for (int i = 0; i < nf; ++i) f[i] = outer_first[nf - 1 - i];
+            return n;
+        };
+        int32_t code[T2_CODES] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int g[4], ng = 0;
+        const int top = peel(stack[0], g, ng, 4);
+        if (top < 0) return false;
+        int ia = -1, ib = -1;
+        if (nodes[top].kind == 0) {                 // unary functions of one operand only: f0a f0b g1 g2 in order of application
+            if (ng == 0) return false;              // a plain copy has its own evaluator
+            ia = nodes[top].tok;
+            const int slot[4] = {T2_F0A, T2_F0B, T2_G1, T2_G2};
+            for (int i = 0; i < ng; ++i) code[slot[i]] = g[i];
+        } else {
+            if (ng > 2) return false;
+            int f0[4], f1[4], n0 = 0, n1 = 0;
+            const int la = peel(nodes[top].l, f0, n0, 2), lb = peel(nodes[top].r, f1, n1, 2);
+            if (la < 0 || lb < 0 || nodes[la].kind != 0 || nodes[lb].kind != 0) return false;
+            ia = nodes[la].tok; ib = nodes[lb].tok;
+            code[T2_OP] = nodes[top].tok;
+            if (n0 > 0) code[T2_F0A] = f0[0];
+            if (n0 > 1) code[T2_F0B] = f0[1];
+            if (n1 > 0) code[T2_F1A] = f1[0];
+            if (n1 > 1) code[T2_F1B] = f1[1];
+            if (ng > 0) code[T2_G1] = g[0];
+            if (ng > 1) code[T2_G2] = g[1];
+        }
+        c = a;
+        c.op[0] = a.op[ia];
+        c.n_operands = 1;
+        if (ib >= 0) {
+            if (ib == ia) code[T2_SAME] = 1;
+            else { c.op[1] = a.op[ib]; c.n_operands = 2; }
+        }
+        if (nscalars > 0) {
+            if (c.n_operands == 1) c.op[1] = a.op[scalars[0]];  // slot 1 unused: a scalar costs no load
+            for (int i = 0; i < nscalars; ++i) c.op[2 + i] = a.op[scalars[i]];
+            c.n_operands = 2 + nscalars;
+        }
+        c.n_tokens = T2_CODES;
+        for (int i = 0; i < T2_CODES; ++i) c.tokens[i] = code[i];
+        return true;
+    }
+};
+typedef EvalTree2T<false, 2> EvalTree2Light;
+typedef EvalTree2T<true, 2> EvalTree2Full;
+typedef EvalTree2T<false, 4> EvalTree2LightS;     // with scalar slots
+typedef EvalTree2T<true, 4> EvalTree2FullS;
+
 // ---- kernels --------------------------------------------------------------------------------------------
 extern __shared__ __align__(16) unsigned char bc_lds_raw[];
 
@@ -435,7 +667,8 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_kernel(const BcArgs a) {
         const int64_t row0 = rb * (rows_apart * BC_RPT) + ty;
         if (i0 >= a.shape[0] || row0 >= a.nrows) return;
         const bool wave_rows = a.tx_log2 >= 6;     // 64 or more lanes along dim 0: the lanes of a wave share their rows
-        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? 2 : 1) : (Eval::NOPS > 4 ? 2 : BC_RPT);   // rows in flight per thread, bounded by registers
+        // rows in flight per thread, bounded by registers (four operand slots of four 8-byte values each: two rows)
+        constexpr int NB = Eval::USES_LDS ? (Eval::NOPS <= 4 ? 2 : 1) : ((Eval::NOPS > 4 || (Eval::NOPS > 3 && sizeof(CT) * VEC > 16)) ? 2 : BC_RPT);
         for (int r0 = 0; r0 < BC_RPT; r0 += NB) {
             CT in[NB][RK_MAX_OPERANDS][VEC];
             int64_t doff[NB];
@@ -776,22 +1009,28 @@ static bool tokens_are(const BcArgs& a, std::initializer_list<int> want) {
     return true;
 }
 
-// True: `c` is `a` without its RK_BC_ROUND_F16 tokens, which stood behind every operation and nowhere else, and
-// c.post says so: the same program for an evaluator that rounds every intermediate (bc_post).
+// True: `c` is `a` without its RK_BC_ROUND_F16 tokens, and c.post says that every operation rounds: the same program for
+// an evaluator that rounds every intermediate (bc_post).  That holds when a rounding token follows every operation whose
+// result can need one -- negation, abs, max, min, comparisons, logic and ifelse return Float16 values as they are, the
+// planner puts no token behind them, and rounding their result again changes nothing -- and stands nowhere else.
 static bool strip_post(const BcArgs& a, BcArgs& c) {
-    int n = 0, ops = 0, posts = 0;
+    auto rounds = [](int tok) {
+        return (tok >= RK_BC_ADD && tok <= RK_BC_DIV) || tok == RK_BC_POW || tok == RK_BC_FMA || tok == RK_BC_ABS2 ||
+               (tok >= RK_BC_SQRT && tok <= RK_BC_INV);
+    };
+    int n = 0, posts = 0;
     int32_t t[RK_MAX_PROGRAM];
     for (int i = 0; i < a.n_tokens; ++i) {
         const int tok = a.tokens[i];
         if (tok == RK_BC_ROUND_F16) {
-            if (i == 0 || a.tokens[i - 1] < RK_BC_ADD || a.tokens[i - 1] == RK_BC_ROUND_F16) return false;   // behind an operand, or twice
+            if (i == 0 || !rounds(a.tokens[i - 1])) return false;        // behind an operand, an exact operation, or twice
             ++posts;
             continue;
         }
-        if (tok >= RK_BC_ADD) ++ops;                 // operand and constant slots lie below the first operator token
+        if (rounds(tok) && (i + 1 >= a.n_tokens || a.tokens[i + 1] != RK_BC_ROUND_F16)) return false;   // a Float32 intermediate
         t[n++] = tok;
     }
-    if (posts == 0 || posts != ops) return false;
+    if (posts == 0) return false;
     c = a;
     c.n_tokens = n;
     for (int i = 0; i < n; ++i) c.tokens[i] = t[i];
@@ -820,6 +1059,15 @@ static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream
             if (c.n_operands <= 6) return bc_launch<EvalLeftChainN<6>, CT>(c, vec, rows, stream);
             return bc_launch<EvalLeftChainN<8>, CT>(c, vec, rows, stream);
         }
+        bool full = false;
+        if (EvalTree2Light::canonical(a, c, full)) {
+            const bool scalars = c.n_operands > 2;
+            if (!full) return scalars ? bc_launch<EvalTree2LightS, CT>(c, vec, rows, stream) : bc_launch<EvalTree2Light, CT>(c, vec, rows, stream);
+            // (Float64 pow / sin / cos / tanh stay with the interpreter: in rows mode the compiler kept this evaluator's
+            // operands in private memory next to those routines)
+            if constexpr (!std::is_same<CT, double>::value)
+                return scalars ? bc_launch<EvalTree2FullS, CT>(c, vec, rows, stream) : bc_launch<EvalTree2Full, CT>(c, vec, rows, stream);
+        }
     }
     taken = false;
     return RK_SUCCESS;
@@ -838,7 +1086,13 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
     }
     const int32_t st = bc_dispatch_fused<CT>(a, vec, rows, stream, taken);
     if (taken) return st;
-    if (a.n_operands <= EvalInterp4::NOPS) return bc_launch<EvalInterp4, CT>(a, vec, rows, stream);
+    if (a.n_operands <= EvalInterp4::NOPS) {
+        bool heavy = false;
+        for (int i = 0; i < a.n_tokens; ++i)
+            if (a.tokens[i] == RK_BC_POW || a.tokens[i] == RK_BC_SIN || a.tokens[i] == RK_BC_COS || a.tokens[i] == RK_BC_TANH) heavy = true;
+        if (!heavy) return bc_launch<EvalInterp4Light, CT>(a, vec, rows, stream);
+        return bc_launch<EvalInterp4, CT>(a, vec, rows, stream);
+    }
     return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
 }
 

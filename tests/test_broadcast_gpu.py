@@ -324,6 +324,59 @@ def test_float16_arrays(rk):
     assert isinstance(s, np.float16) and abs(float(s) - float((x * x).astype(np.float64).sum())) <= 2.0**-9 * float((x * x).astype(np.float64).sum())
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.float16, np.int32, np.int16, np.int64])
+@pytest.mark.parametrize("shape", [(1 << 16,), (4100,), (300, 64), (130, 67), (64, 1, 50)])
+def test_one_and_two_operand_trees(rk, dtype, shape):
+    """Programs of the form g2(g1(f0b(f0a(u)) op f1b(f1a(v)))) have an evaluator without a value stack; every form it takes is
+    checked against NumPy evaluated operation by operation in the element type (Float16: rounded after every
+    operation; integers: wrap-around), on flat, rows and indexed shapes."""
+    rng = _rng(31)
+    B = rk.broadcast
+    lz = rk.lazy
+    d = np.dtype(dtype)
+    if d.kind == "f":
+        x = (rng.standard_normal(shape) * 2).astype(dtype)
+        y = (rng.random(shape) + 0.5).astype(dtype)
+    else:
+        x = rng.integers(-90, 90, shape).astype(dtype)
+        y = rng.integers(1, 90, shape).astype(dtype)
+    col = y[..., :1].copy()                      # extruded along the last dim
+    X, Y, Cc = rk.ROCArray(x), rk.ROCArray(y), rk.ROCArray(col)
+    T = dtype
+    exact = [
+        (-lz(X), -x), (B.abs_(lz(X)), np.abs(x)), (B.abs2(lz(X)), x * x), (lz(X) * lz(X), x * x), (lz(X) + lz(X), x + x),
+        (-B.abs_(lz(X)), -np.abs(x)), (B.abs2(lz(X)) + B.abs2(lz(Y)), (x * x + y * y).astype(T)),
+        (B.abs2(lz(X) - lz(Y)), ((x - y) * (x - y)).astype(T)), (-(lz(X) * lz(Cc)), -(x * col)),
+        (B.abs_(lz(X)) - B.abs_(lz(Cc)), np.abs(x) - np.abs(col)), (B.max_(-lz(X), lz(Y)), np.maximum(-x, y)),
+        (B.abs_(-B.abs2(lz(X))), np.abs(-(x * x))),
+        # binary operators with a scalar count as unary functions of the tree: a .* x .+ b .* y, c .- abs.(x), 2 .* (x .+ y) .- 1
+        (T(3) * lz(X) + T(2) * lz(Y), (T(3) * x + T(2) * y).astype(T)), (T(5) - B.abs_(lz(X)), (T(5) - np.abs(x)).astype(T)),
+        (T(2) * (lz(X) + lz(Y)) - T(1), (T(2) * (x + y) - T(1)).astype(T)), (B.max_(lz(X) * T(2), T(1)) + lz(Cc), (np.maximum(x * T(2), T(1)) + col).astype(T)),
+        (lz(X) ** 2, x * x), ((lz(X) - lz(Y)) ** 2, ((x - y) * (x - y)).astype(T)),
+    ]
+    if d.kind == "f":
+        one = T(1)
+        exact += [
+            (B.sqrt(B.abs_(lz(X))), np.sqrt(np.abs(x))), (B.inv(lz(Y)), (one / y).astype(T)), (one / lz(Y), (one / y).astype(T)),
+            (B.sqrt(lz(Y)) * B.sqrt(lz(Y)), (np.sqrt(y) * np.sqrt(y)).astype(T)), (B.sqrt(B.abs2(lz(X)) + B.abs2(lz(Y))), np.sqrt((x * x + y * y).astype(T))),
+            (B.isnan(lz(X) / lz(X)), np.isnan(x / x)),
+        ]
+    for bc, want in exact:
+        got = rk.materialize(bc)
+        np.testing.assert_array_equal(rk.Array(got), np.asarray(want).astype(got.dtype))
+    if d.kind == "f":
+        # transcendental functions: the device routines are within an ulp or two of the correctly rounded value
+        tol = {2: 2.0**-9, 4: 4e-7, 8: 1e-15}[d.itemsize]
+        x64, y64 = x.astype(np.float64), y.astype(np.float64)
+        close = [
+            (B.exp(lz(X)), np.exp(x64)), (B.tanh(lz(X)), np.tanh(x64)), (B.log(lz(Y)), np.log(y64)), (B.sin(lz(X)) * B.cos(lz(Y)), np.sin(x64) * np.cos(y64)),
+            (T(1) / (T(1) + B.exp(-lz(X))), 1 / (1 + np.exp(-x64))), (B.exp(-B.abs2(lz(X))), np.exp(-x64 * x64)), (B.log(B.exp(lz(X)) + T(1)), np.log(np.exp(x64) + 1)),
+        ]
+        for bc, want in close:
+            got = rk.Array(rk.materialize(bc)).astype(np.float64)
+            np.testing.assert_allclose(got, want, rtol=4 * tol, atol=4 * tol)
+
+
 @pytest.mark.parametrize("shape", [(1 << 16,), (4100,), (4096 + 8,), (256, 96), (130, 67)])
 def test_narrow_arrays_in_the_fused_evaluators(rk, shape):
     """Float16 programs whose every operation rounds run in the fused evaluators (the rounding tokens become a rounding of
