@@ -1012,7 +1012,7 @@ static bool tokens_are(const BcArgs& a, std::initializer_list<int> want) {
 // True: `c` is `a` without its RK_BC_ROUND_F16 tokens, and c.post says that every operation rounds: the same program for
 // an evaluator that rounds every intermediate (bc_post).  That holds when a rounding token follows every operation whose
 // result can need one -- negation, abs, max, min, comparisons, logic and ifelse return Float16 values as they are, the
-// planner puts no token behind them, and rounding their result again changes nothing -- and stands nowhere else.
+// planner need not put a token behind them, and rounding their result again changes nothing -- and behind operations only.
 static bool strip_post(const BcArgs& a, BcArgs& c) {
     auto rounds = [](int tok) {
         return (tok >= RK_BC_ADD && tok <= RK_BC_DIV) || tok == RK_BC_POW || tok == RK_BC_FMA || tok == RK_BC_ABS2 ||
@@ -1023,7 +1023,7 @@ static bool strip_post(const BcArgs& a, BcArgs& c) {
     for (int i = 0; i < a.n_tokens; ++i) {
         const int tok = a.tokens[i];
         if (tok == RK_BC_ROUND_F16) {
-            if (i == 0 || !rounds(a.tokens[i - 1])) return false;        // behind an operand, an exact operation, or twice
+            if (i == 0 || a.tokens[i - 1] < RK_BC_ADD || a.tokens[i - 1] == RK_BC_ROUND_F16) return false;   // behind an operand, or twice
             ++posts;
             continue;
         }
