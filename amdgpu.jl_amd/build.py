@@ -31,7 +31,7 @@ FLAGS = [
 
 # (source, object suffix, extra flags)
 UNITS = (
-    [("rk_api.hip", "", []), ("rk_broadcast.hip", "", []), *[("rk_broadcast.hip", f"_{n}", [f"-DRK_BC_INST={n}"]) for n in range(3)], ("rk_volumerhs.hip", "", []), ("rk_select.hip", "", []), ("rk_reverse.hip", "", []), ("rk_permute.hip", "", []), ("rk_sort.hip", "", [])]
+    [("rk_api.hip", "", []), ("rk_broadcast.hip", "", []), *[("rk_broadcast.hip", f"_{n}", [f"-DRK_BC_INST={n}"]) for n in range(6)], ("rk_volumerhs.hip", "", []), ("rk_select.hip", "", []), ("rk_reverse.hip", "", []), ("rk_permute.hip", "", []), ("rk_sort.hip", "", [])]
     + [("rk_reduce_inst.hip", f"_{n}", [f"-DRK_INST={n}"]) for n in range(13)]
     + [("rk_scan_inst.hip", f"_{n}", [f"-DRK_INST={n}"]) for n in range(13)]
 )

@@ -1038,7 +1038,19 @@ static bool strip_post(const BcArgs& a, BcArgs& c) {
     return true;
 }
 
-// The programs with an evaluator of their own; `taken` = false: none of them.
+// This file is compiled seven times: once without RK_BC_INST for the C entry points, and twice per compute type so that
+// the kernel sets build in parallel -- RK_BC_INST = 0, 1, 2 (Float32, Float64, Int64): the evaluators for copies, binary
+// operators and chains; RK_BC_INST = 3, 4, 5: the trees of one and two operands and the interpreters.
+int32_t bc_dispatch_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+int32_t bc_dispatch_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+int32_t bc_dispatch_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
+// second half: `only_fused` = take the program only if a fused evaluator (a tree) fits, else set taken = false
+int32_t bc_rest_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken);
+int32_t bc_rest_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken);
+int32_t bc_rest_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken);
+
+#if defined(RK_BC_INST) && RK_BC_INST < 3
+// The programs with an evaluator of their own among copies, binary operators and chains; `taken` = false: none of them.
 template <typename CT>
 static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool& taken) {
     taken = true;
@@ -1059,6 +1071,43 @@ static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream
             if (c.n_operands <= 6) return bc_launch<EvalLeftChainN<6>, CT>(c, vec, rows, stream);
             return bc_launch<EvalLeftChainN<8>, CT>(c, vec, rows, stream);
         }
+    }
+    taken = false;
+    return RK_SUCCESS;
+}
+
+template <typename CT>
+static int32_t bc_rest(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken) {
+    if constexpr (std::is_same<CT, float>::value) return bc_rest_f32(a, vec, rows, stream, only_fused, taken);
+    else if constexpr (std::is_same<CT, double>::value) return bc_rest_f64(a, vec, rows, stream, only_fused, taken);
+    else return bc_rest_i64(a, vec, rows, stream, only_fused, taken);
+}
+
+template <typename CT>
+static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
+    bool taken = false;
+    if constexpr (std::is_same<CT, float>::value) {
+        // a Float16 program whose every operation rounds: the fused evaluators take it without the rounding tokens
+        BcArgs stripped;
+        if (a.post == 0 && strip_post(a, stripped)) {
+            int32_t st = bc_dispatch_fused<CT>(stripped, vec, rows, stream, taken);
+            if (taken) return st;
+            st = bc_rest<CT>(stripped, vec, rows, stream, true, taken);
+            if (taken) return st;
+        }
+    }
+    const int32_t st = bc_dispatch_fused<CT>(a, vec, rows, stream, taken);
+    if (taken) return st;
+    return bc_rest<CT>(a, vec, rows, stream, false, taken);
+}
+#endif
+
+#if defined(RK_BC_INST) && RK_BC_INST >= 3
+template <typename CT>
+static int32_t bc_rest_impl(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken) {
+    taken = true;
+    {
+        BcArgs c;
         bool full = false;
         if (EvalTree2Light::canonical(a, c, full)) {
             const bool scalars = c.n_operands > 2;
@@ -1069,23 +1118,7 @@ static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream
                 return scalars ? bc_launch<EvalTree2FullS, CT>(c, vec, rows, stream) : bc_launch<EvalTree2Full, CT>(c, vec, rows, stream);
         }
     }
-    taken = false;
-    return RK_SUCCESS;
-}
-
-template <typename CT>
-static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
-    bool taken = false;
-    if constexpr (std::is_same<CT, float>::value) {
-        // a Float16 program whose every operation rounds: the fused evaluators take it without the rounding tokens
-        BcArgs stripped;
-        if (a.post == 0 && strip_post(a, stripped)) {
-            const int32_t st = bc_dispatch_fused<CT>(stripped, vec, rows, stream, taken);
-            if (taken) return st;
-        }
-    }
-    const int32_t st = bc_dispatch_fused<CT>(a, vec, rows, stream, taken);
-    if (taken) return st;
+    if (only_fused) { taken = false; return RK_SUCCESS; }
     if (a.n_operands <= EvalInterp4::NOPS) {
         bool heavy = false;
         for (int i = 0; i < a.n_tokens; ++i)
@@ -1095,18 +1128,20 @@ static int32_t bc_dispatch(const BcArgs& a, bool vec, bool rows, hipStream_t str
     }
     return bc_launch<EvalInterp, CT>(a, vec, rows, stream);
 }
+#endif
 
-// This file is compiled once per compute type (-DRK_BC_INST=0, 1, 2: Float32, Float64, Int64 kernels) and once
-// without the macro for the C entry points, so that the kernel sets build in parallel.
-int32_t bc_dispatch_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
-int32_t bc_dispatch_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
-int32_t bc_dispatch_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream);
 #if defined(RK_BC_INST) && RK_BC_INST == 0
 int32_t bc_dispatch_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<float>(a, vec, rows, stream); }
 #elif defined(RK_BC_INST) && RK_BC_INST == 1
 int32_t bc_dispatch_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<double>(a, vec, rows, stream); }
 #elif defined(RK_BC_INST) && RK_BC_INST == 2
 int32_t bc_dispatch_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream) { return bc_dispatch<int64_t>(a, vec, rows, stream); }
+#elif defined(RK_BC_INST) && RK_BC_INST == 3
+int32_t bc_rest_f32(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken) { return bc_rest_impl<float>(a, vec, rows, stream, only_fused, taken); }
+#elif defined(RK_BC_INST) && RK_BC_INST == 4
+int32_t bc_rest_f64(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken) { return bc_rest_impl<double>(a, vec, rows, stream, only_fused, taken); }
+#elif defined(RK_BC_INST) && RK_BC_INST == 5
+int32_t bc_rest_i64(const BcArgs& a, bool vec, bool rows, hipStream_t stream, bool only_fused, bool& taken) { return bc_rest_impl<int64_t>(a, vec, rows, stream, only_fused, taken); }
 #endif
 
 }  // namespace rk
