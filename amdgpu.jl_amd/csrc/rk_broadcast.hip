@@ -513,7 +513,7 @@ template <bool FULL, int NOPS_> struct EvalTree2T {        // NOPS_ = 2: no scal
             if constexpr (NOPS_ >= 4) {
                 CT c[VEC];
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) c[j] = k == 3 ? in[2][j] : in[3][j];
+                for (int j = 0; j < VEC; ++j) c[j] = k == 3 ? in[2][0] : in[3][0];      // a scalar: every component holds it
                 if ((code >> 16) != 0) {            // c op v
                     binary<CT, VEC>(code & 0xff, c, v);
 #pragma unroll
@@ -633,6 +633,148 @@ template <bool FULL, int NOPS_> struct EvalTree2T {        // NOPS_ = 2: no scal
         return true;
     }
 };
+// dest = g2(g1( m2(m1(f(u) op1 f(v))) op2 f(w) ))  or  g2(g1( f(w) op2 m2(m1(f(u) op1 f(v))) ))
+// The same with a third operand: every f, m, g up to two unary functions or scalar operators (three distinct scalars,
+// operands 3..5).  x .* y .+ sin.(w), a .* x .+ b .* y .+ c .* z, (x .- m) ./ sqrt.(v .+ eps), abs2.(x) .+ abs2.(y) .+ abs2.(z).
+// Operands that are the same array are loaded once (T3_SAME_V: v is u; T3_SAME_W: 1 = w is u, 2 = w is v).
+enum { T3_FU = 0, T3_FV = 2, T3_FW = 4, T3_M = 6, T3_G = 8, T3_OP1 = 10, T3_OP2, T3_W_LEFT, T3_SAME_V, T3_SAME_W, T3_CODES };
+template <bool FULL> struct EvalTree3T {
+    static constexpr int NOPS = 6;
+    static constexpr bool USES_LDS = false;
+    // flat mode only: in rows mode the compiler kept the six operand slots of several rows in private memory, and every
+    // further kernel of this size costs build time
+    static constexpr bool FLAT_ONLY = true;
+    typedef EvalTree2T<FULL, 4> Base;
+    template <typename CT, int VEC, typename A>
+    static __device__ __forceinline__ void run(const A& a, const CT (&in)[RK_MAX_OPERANDS][VEC], CT (&out)[VEC], CT*) {
+        auto slot = [&](int code, CT (&v)[VEC]) {
+            const int k = (code >> 8) & 0xff;
+            if (k == 0) { Base::template unary<CT, VEC>(code, a.post, v); return; }
+            CT c[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) c[j] = k == 4 ? in[3][0] : (k == 5 ? in[4][0] : in[5][0]);
+            if ((code >> 16) != 0) {            // c op v
+                Base::template binary<CT, VEC>(code & 0xff, c, v);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[j] = c[j];
+            } else {
+                Base::template binary<CT, VEC>(code & 0xff, v, c);
+            }
+            bc_post<CT, VEC>(a.post, v);
+        };
+        CT x[VEC], y[VEC], z[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            x[j] = in[0][j];
+            y[j] = a.tokens[T3_SAME_V] != 0 ? in[0][j] : in[1][j];
+            z[j] = a.tokens[T3_SAME_W] == 1 ? in[0][j] : (a.tokens[T3_SAME_W] == 2 ? in[1][j] : in[2][j]);
+        }
+        slot(a.tokens[T3_FU], x); slot(a.tokens[T3_FU + 1], x);
+        slot(a.tokens[T3_FV], y); slot(a.tokens[T3_FV + 1], y);
+        Base::template binary<CT, VEC>(a.tokens[T3_OP1], x, y);
+        bc_post<CT, VEC>(a.post, x);
+        slot(a.tokens[T3_M], x); slot(a.tokens[T3_M + 1], x);
+        slot(a.tokens[T3_FW], z); slot(a.tokens[T3_FW + 1], z);
+        if (a.tokens[T3_W_LEFT] != 0) {
+            Base::template binary<CT, VEC>(a.tokens[T3_OP2], z, x);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) x[j] = z[j];
+        } else {
+            Base::template binary<CT, VEC>(a.tokens[T3_OP2], x, z);
+        }
+        bc_post<CT, VEC>(a.post, x);
+        slot(a.tokens[T3_G], x); slot(a.tokens[T3_G + 1], x);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) out[j] = x[j];
+    }
+    static bool canonical(const BcArgs& a, BcArgs& c, bool& full) {
+        struct Node { int kind, tok, l, r; };        // kind 0: operand `tok`; 1: unary of l; 2: binary of l, r
+        Node nodes[RK_MAX_PROGRAM];
+        int stack[RK_MAX_PROGRAM], sp = 0, nn = 0;
+        full = false;
+        for (int i = 0; i < a.n_tokens; ++i) {
+            const int tok = a.tokens[i];
+            if (tok >= 0 && tok < RK_MAX_OPERANDS) { nodes[nn] = Node{0, tok, -1, -1}; stack[sp++] = nn++; continue; }
+            const int ar = token_arity(tok);
+            if (tok == RK_BC_IDENTITY) continue;
+            if (!token_basic(tok)) full = true;
+            if (ar == 1 && sp >= 1) { nodes[nn] = Node{1, tok, stack[sp - 1], -1}; stack[sp - 1] = nn++; }
+            else if (ar == 2 && sp >= 2) { nodes[nn] = Node{2, tok, stack[sp - 2], stack[sp - 1]}; sp -= 1; stack[sp - 1] = nn++; }
+            else return false;
+        }
+        if (sp != 1) return false;
+        int scalars[3], nscalars = 0;               // operands of `a` that travel as operands 3, 4, 5
+        auto is_scalar = [&](int n) { return nodes[n].kind == 0 && a.op[nodes[n].tok].ptr == nullptr; };
+        // up to two unary functions / scalar operators from `n` downwards, innermost first in f[]; returns the node below
+        auto peel = [&](int n, int (&f)[2], int& nf) -> int {
+            int outer_first[2];
+            nf = 0;
+            for (;;) {
+                int code, next;
+                if (nodes[n].kind == 1) { code = nodes[n].tok; next = nodes[n].l; }
+                else if (nodes[n].kind == 2 && (is_scalar(nodes[n].l) || is_scalar(nodes[n].r))) {
+                    const bool left = is_scalar(nodes[n].l) && !is_scalar(nodes[n].r);
+                    const int sc = nodes[left ? nodes[n].l : nodes[n].r].tok;
+                    int k = -1;
+                    for (int i = 0; i < nscalars; ++i) if (scalars[i] == sc) k = i;
+                    if (k < 0) { if (nscalars == 3) return -1; scalars[nscalars] = sc; k = nscalars++; }
+                    code = nodes[n].tok | ((k + 4) << 8) | ((left ? 1 : 0) << 16);
+                    next = left ? nodes[n].r : nodes[n].l;
+                } else break;
+                if (nf == 2) return -1;
+                outer_first[nf++] = code;
+                n = next;
+            }
+            for (int i = 0; i < nf; ++i) f[i] = outer_first[nf - 1 - i];
+            return n;
+        };
+        int32_t code[T3_CODES];
+        for (int i = 0; i < T3_CODES; ++i) code[i] = 0;
+        auto put = [&](int at, const int (&f)[2], int nf) { for (int i = 0; i < nf; ++i) code[at + i] = f[i]; };
+        int g[2], ng = 0;
+        const int top = peel(stack[0], g, ng);
+        if (top < 0 || nodes[top].kind != 2) return false;
+        put(T3_G, g, ng);
+        // one child is f(w), the other m(f(u) op1 f(v)); the left one is tried as the inner tree first
+        for (int w_left = 0; w_left < 2; ++w_left) {
+            const int saved = nscalars;
+            const int inner_n = w_left ? nodes[top].r : nodes[top].l, leaf_n = w_left ? nodes[top].l : nodes[top].r;
+            int m[2], fw[2], fu[2], fv[2], nm = 0, nw = 0, nu = 0, nv = 0;
+            const int inner = peel(inner_n, m, nm);
+            const int wl = peel(leaf_n, fw, nw);
+            if (inner >= 0 && wl >= 0 && nodes[inner].kind == 2 && nodes[wl].kind == 0) {
+                const int ul = peel(nodes[inner].l, fu, nu), vl = peel(nodes[inner].r, fv, nv);
+                if (ul >= 0 && vl >= 0 && nodes[ul].kind == 0 && nodes[vl].kind == 0) {
+                    const int iu = nodes[ul].tok, iv = nodes[vl].tok, iw = nodes[wl].tok;
+                    for (int i = T3_FU; i < T3_G; ++i) code[i] = 0;
+                    put(T3_FU, fu, nu); put(T3_FV, fv, nv); put(T3_FW, fw, nw); put(T3_M, m, nm);
+                    code[T3_OP1] = nodes[inner].tok;
+                    code[T3_OP2] = nodes[top].tok;
+                    code[T3_W_LEFT] = w_left;
+                    code[T3_SAME_V] = iv == iu ? 1 : 0;
+                    code[T3_SAME_W] = iw == iu ? 1 : (iw == iv ? 2 : 0);
+                    c = a;
+                    const BcOperand filler = nscalars > 0 ? a.op[scalars[0]] : a.op[iu];   // unused array slots: a scalar costs no load
+                    BcOperand none = filler;
+                    if (nscalars == 0) { none.ptr = nullptr; none.sf = 0.0; none.si = 0; }
+                    c.op[0] = a.op[iu];
+                    c.op[1] = code[T3_SAME_V] ? none : a.op[iv];
+                    c.op[2] = code[T3_SAME_W] ? none : a.op[iw];
+                    for (int i = 0; i < 3; ++i) c.op[3 + i] = i < nscalars ? a.op[scalars[i]] : none;
+                    c.n_operands = 3 + nscalars;
+                    c.n_tokens = T3_CODES;
+                    for (int i = 0; i < T3_CODES; ++i) c.tokens[i] = code[i];
+                    return true;
+                }
+            }
+            nscalars = saved;
+        }
+        return false;
+    }
+};
+typedef EvalTree3T<false> EvalTree3Light;
+typedef EvalTree3T<true> EvalTree3Full;
+
 typedef EvalTree2T<false, 2> EvalTree2Light;
 typedef EvalTree2T<true, 2> EvalTree2Full;
 typedef EvalTree2T<false, 4> EvalTree2LightS;     // with scalar slots
@@ -885,6 +1027,10 @@ __global__ __launch_bounds__(BC_BLOCK) void bc_indexed_kernel(const BcArgs a) {
     }
 }
 
+// Eval::FLAT_ONLY = true: no rows-mode and no indexed kernels are built for the evaluator
+template <typename E, typename = void> struct EvalFlatOnly : std::false_type {};
+template <typename E> struct EvalFlatOnly<E, std::void_t<decltype(E::FLAT_ONLY)>> : std::integral_constant<bool, E::FLAT_ONLY> {};
+
 template <typename Eval, typename CT>
 static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t stream) {
     const int VECN = vec ? a.vecn : 1;
@@ -979,6 +1125,15 @@ static int32_t bc_launch(const BcArgs& a, bool vec, bool rows, hipStream_t strea
         }
     }
 #define RK_BC_LAUNCH(V, R, H) bc_kernel<Eval, CT, V, R, H><<<grid, BC_BLOCK, lds, stream>>>(a)
+    if constexpr (EvalFlatOnly<Eval>::value) {
+        // an evaluator that exists for the flat mode only (the dispatcher sends it nothing else)
+        if (rows || a.indexed != 0) return RK_ERR_UNSUPPORTED;
+        if (vec && VECN == 2) { if (homog) RK_BC_LAUNCH(2, false, true); else RK_BC_LAUNCH(2, false, false); }
+        else if (vec)         { if (homog) RK_BC_LAUNCH(4, false, true); else RK_BC_LAUNCH(4, false, false); }
+        else                  { if (homog) RK_BC_LAUNCH(1, false, true); else RK_BC_LAUNCH(1, false, false); }
+        RK_LAUNCH_CHECK();
+        return RK_SUCCESS;
+    } else
     if (a.indexed != 0) {            // the planner sets it together with vec and rows
         const int64_t blocks = ((a.total + VECN - 1) / VECN + BC_BLOCK - 1) / BC_BLOCK;
         if (blocks > 0x7fffffff) return RK_ERR_TOO_LARGE;
@@ -1116,6 +1271,14 @@ static int32_t bc_rest_impl(const BcArgs& a, bool vec, bool rows, hipStream_t st
             // operands in private memory next to those routines)
             if constexpr (!std::is_same<CT, double>::value)
                 return scalars ? bc_launch<EvalTree2FullS, CT>(c, vec, rows, stream) : bc_launch<EvalTree2Full, CT>(c, vec, rows, stream);
+        }
+    }
+    {
+        BcArgs c;
+        bool full = false;
+        if (!rows && a.indexed == 0 && EvalTree3Light::canonical(a, c, full)) {
+            if (!full) return bc_launch<EvalTree3Light, CT>(c, vec, rows, stream);
+            if constexpr (!std::is_same<CT, double>::value) return bc_launch<EvalTree3Full, CT>(c, vec, rows, stream);
         }
     }
     if (only_fused) { taken = false; return RK_SUCCESS; }

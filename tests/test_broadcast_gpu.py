@@ -361,6 +361,19 @@ def test_one_and_two_operand_trees(rk, dtype, shape):
             (B.sqrt(lz(Y)) * B.sqrt(lz(Y)), (np.sqrt(y) * np.sqrt(y)).astype(T)), (B.sqrt(B.abs2(lz(X)) + B.abs2(lz(Y))), np.sqrt((x * x + y * y).astype(T))),
             (B.isnan(lz(X) / lz(X)), np.isnan(x / x)),
         ]
+    # three operands: m(f(u) op f(v)) op f(w) on either side, the same array in several places, three scalars
+    z = x[..., ::-1].copy() if x.ndim > 1 else x[::-1].copy()
+    Z = rk.ROCArray(z)
+    exact += [
+        (lz(X) * lz(Y) + B.abs_(lz(Z)), (x * y + np.abs(z)).astype(T)), (B.abs_(lz(Z)) - lz(X) * lz(Y), (np.abs(z) - x * y).astype(T)),
+        (T(2) * lz(X) + T(3) * lz(Y) + T(5) * lz(Z), (T(2) * x + T(3) * y + T(5) * z).astype(T)),
+        (B.abs2(lz(X)) + B.abs2(lz(Y)) + B.abs2(lz(Z)), (x * x + y * y + z * z).astype(T)),
+        (-(lz(X) - lz(Y)) * (lz(X) + T(1)), (-(x - y) * (x + T(1))).astype(T)), ((lz(X) + lz(Z)) * lz(Z) - lz(X), ((x + z) * z - x).astype(T)),
+        (B.max_(lz(X), lz(Y)) - B.min_(lz(Z), lz(X)), np.maximum(x, y) - np.minimum(z, x)),
+        (lz(X) * lz(Cc) + lz(Z), (x * col + z).astype(T)),                       # an extruded operand: rows mode, the interpreter's
+    ]
+    if d.kind == "f":
+        exact += [((lz(X) - lz(Z)) / B.sqrt(lz(Y) + T(0.5)), ((x - z) / np.sqrt(y + T(0.5))).astype(T))]
     for bc, want in exact:
         got = rk.materialize(bc)
         np.testing.assert_array_equal(rk.Array(got), np.asarray(want).astype(got.dtype))
@@ -371,6 +384,7 @@ def test_one_and_two_operand_trees(rk, dtype, shape):
         close = [
             (B.exp(lz(X)), np.exp(x64)), (B.tanh(lz(X)), np.tanh(x64)), (B.log(lz(Y)), np.log(y64)), (B.sin(lz(X)) * B.cos(lz(Y)), np.sin(x64) * np.cos(y64)),
             (T(1) / (T(1) + B.exp(-lz(X))), 1 / (1 + np.exp(-x64))), (B.exp(-B.abs2(lz(X))), np.exp(-x64 * x64)), (B.log(B.exp(lz(X)) + T(1)), np.log(np.exp(x64) + 1)),
+            (lz(X) * lz(Y) + B.sin(lz(Z)), x64 * y64 + np.sin(z.astype(np.float64))), (B.exp(lz(X) - lz(Y)) * lz(Z), np.exp(x64 - y64) * z.astype(np.float64)),
         ]
         for bc, want in close:
             got = rk.Array(rk.materialize(bc)).astype(np.float64)
