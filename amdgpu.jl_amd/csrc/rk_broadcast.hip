@@ -1213,6 +1213,20 @@ static int32_t bc_dispatch_fused(const BcArgs& a, bool vec, bool rows, hipStream
         if (tokens_are(a, {0, 1, RK_BC_MUL, 2, 3, RK_BC_EXP, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAxpbyExp, CT>(a, vec, rows, stream);
     }
     if (tokens_are(a, {0, 1, 2, RK_BC_MUL, RK_BC_ADD})) return bc_launch<EvalAddMul, CT>(a, vec, rows, stream);
+    if (a.n_tokens == 4 && a.tokens[3] == RK_BC_FMA && a.post == 0 && a.tokens[0] >= 0 && a.tokens[0] < a.n_operands &&
+        a.tokens[1] >= 0 && a.tokens[1] < a.n_operands && a.tokens[2] >= 0 && a.tokens[2] < a.n_operands) {
+        // muladd.(p, q, r) = p * q + r, unfused here as in the interpreter: the same evaluator with the operands in its order
+        // (not for Float16 programs: muladd rounds once, the evaluator's rounding would round the product too)
+        BcArgs c = a;
+        c.op[0] = a.op[a.tokens[2]];
+        c.op[1] = a.op[a.tokens[0]];
+        c.op[2] = a.op[a.tokens[1]];
+        c.n_operands = 3;
+        c.n_tokens = 5;
+        const int32_t t[5] = {0, 1, 2, RK_BC_MUL, RK_BC_ADD};
+        for (int i = 0; i < 5; ++i) c.tokens[i] = t[i];
+        return bc_launch<EvalAddMul, CT>(c, vec, rows, stream);
+    }
     if (tokens_are(a, {0})) return bc_launch<EvalCopy, CT>(a, vec, rows, stream);
     if (a.n_tokens == 3 && a.tokens[0] == 0 && a.tokens[1] == 1 &&
         ((a.tokens[2] >= RK_BC_ADD && a.tokens[2] <= RK_BC_POW && !(!std::is_floating_point<CT>::value && (a.tokens[2] == RK_BC_DIV || a.tokens[2] == RK_BC_POW))) ||

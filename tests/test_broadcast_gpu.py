@@ -372,6 +372,10 @@ def test_one_and_two_operand_trees(rk, dtype, shape):
         (B.max_(lz(X), lz(Y)) - B.min_(lz(Z), lz(X)), np.maximum(x, y) - np.minimum(z, x)),
         (lz(X) * lz(Cc) + lz(Z), (x * col + z).astype(T)),                       # an extruded operand: rows mode, the interpreter's
     ]
+    # muladd(p, q, r) = p * q + r, one rounding at the end for Float16 (computed in Float32)
+    wide = np.float32 if dtype == np.float16 else dtype
+    exact += [(B.muladd(lz(X), lz(Y), lz(Z)), (x.astype(wide) * y.astype(wide) + z.astype(wide)).astype(T)),
+              (B.muladd(lz(X), lz(X), lz(Cc)), (x.astype(wide) * x.astype(wide) + col.astype(wide)).astype(T))]
     if d.kind == "f":
         exact += [((lz(X) - lz(Z)) / B.sqrt(lz(Y) + T(0.5)), ((x - z) / np.sqrt(y + T(0.5))).astype(T))]
     for bc, want in exact:
