@@ -68,6 +68,9 @@ def parse():
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--no-configs", action="store_true", help="skip the per-configuration table")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    p.add_argument("--placement", action="store_true",
+                   help="instead of the bench line: time z .= a.*x .+ y.*exp.(w) at 2^26 elements with x, y, w, z at several "
+                        "relative placements inside one buffer and on fresh allocations, all in this one process; prints a table")
     p.add_argument("--only", default=None,
                    help="run only the rows whose name contains this text ('|' separates alternatives); skips the headline step")
     return p.parse_args()
@@ -148,6 +151,36 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         return best, e0.elapsed_time(e1) / reps
+
+    if args.placement:
+        # The headline broadcast on the same data at different relative placements of its four arrays: one buffer, the
+        # arrays `skew` bytes further apart than their size; then separately allocated arrays, three times over.
+        from amdgpu_jl_amd.broadcast import plan_materialize
+        n = N_HEAD
+        nb = 4 * n
+        a = np.float32(0.5)
+        src = [rand_f32(n), rand_f32(n), rand_f32(n, -1.0, 1.0)]
+        print(f"z .= a.*x .+ y.*exp.(w), Float32, 2^26 elements, one process; us per launch: minimum of synchronised launches / "
+              f"average of {K} back-to-back launches; GB/s of the 16 B/elt at the average")
+        skews = [0, 256, 1024, 4096, 65536, (1 << 20) + 4096, (2 << 20) + 256, (64 << 20) + 8192]
+        pool = torch.empty(4 * nb + 3 * max(skews) + 4096, dtype=torch.uint8, device=dev)
+        base = (-pool.data_ptr()) % 4096          # first array on a page boundary
+        for skew in skews:
+            arrs = [rk.ROCArray(buf=pool, dims=(n,), dtype=np.float32, offset=base + i * (nb + skew)) for i in range(4)]
+            for t, arr in zip(src, arrs[:3]):
+                pool[arr.offset:arr.offset + nb].copy_(t.view(torch.uint8).reshape(-1))
+            plan = plan_materialize(arrs[3], a * L(arrs[0]) + L(arrs[1]) * rk.broadcast.exp(L(arrs[2])))
+            best, avg = time_launches(lambda i: plan(), K)
+            print(f"  one buffer, arrays {skew:>9d} bytes apart beyond their size:   {best * 1e3:7.1f} / {avg * 1e3:7.1f} us   {16 * n / avg / 1e6:6.0f} GB/s")
+        for trial in range(3):
+            ts = [t.clone() for t in src] + [torch.empty(n, dtype=torch.float32, device=dev)]
+            arrs = [dev_array(t, (n,), np.float32) for t in ts]
+            plan = plan_materialize(arrs[3], a * L(arrs[0]) + L(arrs[1]) * rk.broadcast.exp(L(arrs[2])))
+            best, avg = time_launches(lambda i: plan(), K)
+            offs = [(t.data_ptr() - ts[0].data_ptr()) for t in ts]
+            print(f"  fresh allocations {trial + 1} (offsets from x: {offs[1]}, {offs[2]}, {offs[3]}):   {best * 1e3:7.1f} / {avg * 1e3:7.1f} us   {16 * n / avg / 1e6:6.0f} GB/s")
+            del ts, arrs, plan
+        return
 
     # ---- CPU side: the C restatement of Julia Base, timed on the host cores ------------------------------------
     cpu_lib = None
