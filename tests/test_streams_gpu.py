@@ -36,3 +36,35 @@ def test_three_streams_interleaved(rk, orc):
             assert np.array_equal(rk.Array(so), np.sort(j["f"]))
             assert np.array_equal(rk.Array(fa), np.nonzero(j["m"])[0] + 1)
             assert np.array_equal(rk.Array(mx), j["b"].max(axis=0, keepdims=True))
+
+
+def test_two_streams_beyond_residency(rk, orc):
+    """Two streams, each with grids far larger than what is resident at once (8192 tiles of the 1-D scan, 3072 of the
+    scan across rows, 512 of the select), enqueued without waiting in between, with the default wait budget: tiles of
+    two ordered grids share the compute units while each waits on predecessors of its own grid.  The 1-D scan and the
+    select cannot stall (a tile that waits too long resolves its prefix alone); the chains of the scan across rows stay
+    on one XCD each, where workgroups start in index order.  Integers, so every result is exact."""
+    rng = np.random.default_rng(52)
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    n = 1 << 26
+    jobs = []
+    for s in streams:
+        with torch.cuda.stream(s):
+            x = rng.integers(-1000, 1001, n, dtype=np.int32)
+            b = rng.integers(-1000, 1001, (4096, 16384), dtype=np.int32)
+            m = rng.random(n) < 0.25
+            jobs.append(dict(x=x, b=b, m=m, dx=rk.ROCArray(x), db=rk.ROCArray(b), dm=rk.ROCArray(m), out=[]))
+    torch.cuda.synchronize()
+    for it in range(2):
+        for s, j in zip(streams, jobs):
+            with torch.cuda.stream(s):
+                j["out"].append((rk.cumsum(j["dx"]), rk.cumsum(j["db"], dims=2), rk.findall(j["dm"])))
+    torch.cuda.synchronize()
+    for j in jobs:
+        want_x = orc.cumsum(j["x"])
+        want_b = np.cumsum(j["b"], axis=1, dtype=np.int32)
+        want_m = np.nonzero(j["m"])[0] + 1
+        for cs, c2, fa in j["out"]:
+            assert np.array_equal(rk.Array(cs), want_x)
+            assert np.array_equal(rk.Array(c2), want_b)
+            assert np.array_equal(rk.Array(fa), want_m)
