@@ -95,6 +95,13 @@ int tune_scan_dynamic_ids() {
     return v;
 }
 
+// 0: long lines of 1- and 2-byte integers are scanned in widened tiles of 32 Ki elements instead of packed ones of 128 KiB
+// (RK_SCAN_PACKED).
+int tune_scan_packed() {
+    static const int v = env_int("RK_SCAN_PACKED", 1, 0, 1);
+    return v;
+}
+
 // 0: scans across the rows of a wide matrix (few strips of columns) take the three-pass path (totals, scan of the totals,
 // scan) instead of the single-pass kernel with look-back (RK_SCAN_ROWS_ORDERED).
 int tune_scan_rows_ordered() {

@@ -509,6 +509,134 @@ __device__ __forceinline__ void tile_store(Out* __restrict__ out, int64_t e0, in
     }
 }
 
+// ---- tiles of 1- and 2-byte integers, kept packed ------------------------------------------------------------------------
+// A tile of the single-pass scan lives as long whatever it holds (its loads, a look-back, its stores), so what counts is
+// the bytes it moves.  Widened to 32-bit registers, 32 registers a lane hold 32 elements: 64 KiB of Int16, 32 KiB of Int8
+// a tile.  Here the registers keep the 16-byte vectors as they were loaded -- 8 or 16 elements each -- and a vector is
+// unpacked only while it is scanned and again when the tile's prefix is added: 128 KiB of input a tile like the 4-byte
+// types.  The values between the two steps are the scan without the tile's prefix, truncated to the element type: for
+// + and * that is the type's own wrap-around (the low bits of a sum or product depend on the low bits of the operands
+// only), for max / min / & / | / xor the values never leave the type's range.  Lines of whole, 16-byte aligned vectors.
+typedef uint32_t PackedVec __attribute__((ext_vector_type(4)));
+template <typename In, typename T> struct Packed {
+    static_assert(std::is_integral<In>::value && sizeof(In) <= 2 && sizeof(T) == 4, "1- and 2-byte integers in 32-bit registers");
+    static constexpr int PV = 16 / (int)sizeof(In);           // elements per vector
+    static constexpr int PW = 4 / (int)sizeof(In);            // elements per 32-bit word
+    static constexpr int BITS = 8 * (int)sizeof(In);
+    static __device__ __forceinline__ void unpack_word(uint32_t w, T (&e)[PW]) {
+#pragma unroll
+        for (int h = 0; h < PW; ++h) e[h] = (T)(In)(w >> (h * BITS));          // sign- or zero-extends
+    }
+    static __device__ __forceinline__ uint32_t pack_word(const T (&e)[PW]) {
+        typedef typename std::make_unsigned<In>::type UIn;
+        uint32_t x = 0;
+#pragma unroll
+        for (int h = 0; h < PW; ++h) x |= (uint32_t)(UIn)e[h] << (h * BITS);
+        return x;
+    }
+    template <typename Op> static __device__ __forceinline__ T total(const PackedVec& v, Op op) {
+        T e[PW];
+        unpack_word(v[0], e);
+        T t = e[0];
+#pragma unroll
+        for (int h = 1; h < PW; ++h) t = op(t, e[h]);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            unpack_word(v[w], e);
+#pragma unroll
+            for (int h = 0; h < PW; ++h) t = op(t, e[h]);
+        }
+        return t;
+    }
+    static __device__ __forceinline__ PackedVec splat(T x) {
+        T e[PW];
+#pragma unroll
+        for (int h = 0; h < PW; ++h) e[h] = x;
+        const uint32_t w = pack_word(e);
+        return PackedVec{w, w, w, w};
+    }
+};
+template <int K> struct PackedRegs { PackedVec v[K]; };
+
+template <typename In, typename T, typename Op, int K, int NW>
+__device__ __forceinline__ T packed_tile_load_scan(const In* __restrict__ in, int64_t e0, int valid, int inclusive, Op op, PackedRegs<K>& r) {
+    typedef Packed<In, T> P;
+    constexpr int PV = P::PV;
+    constexpr int TILE = NW * WAVE * PV * K;
+    // the identity of the ELEMENT type: it is packed with the values (exclusive scans store it, short tiles are padded
+    // with it), and the 32-bit one of max / min does not survive the truncation
+    const T ident = (T)Op::template identity<In>();
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int woff = wave * (WAVE * PV * K) + lane * PV;
+    const In* p = in + e0 + woff;
+    if (valid == TILE) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) r.v[k] = load_nt((const PackedVec*)(p + k * WAVE * PV));
+    } else {
+        // a tile that its line does not fill (valid is a whole number of vectors): every lane still issues its K loads
+        // unconditionally -- a vector past the end reads the tile's first one and becomes a vector of identities
+        const PackedVec idv = P::splat(ident);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const bool have = woff + k * WAVE * PV < valid;
+            const PackedVec x = load_nt((const PackedVec*)(have ? p + k * WAVE * PV : in + e0));
+            r.v[k] = have ? x : idv;
+        }
+    }
+    // Per vector: the lane's total first (elements unpacked on the fly), the scan of the totals across the wave, then
+    // word by word a running scan from the lane's exclusive prefix -- four or two elements unpacked at a time.
+    T carry = ident;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const T total = P::total(r.v[k], op);
+        const T inc = wave_scan_inclusive(total, op, ident);
+        T run = op(carry, wave_shift_right(inc, ident));
+        carry = op(carry, read_lane(inc, WAVE - 1));
+        PackedVec o;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            T e[P::PW], x[P::PW];
+            P::unpack_word(r.v[k][w], e);
+#pragma unroll
+            for (int h = 0; h < P::PW; ++h) {
+                const T before = run;
+                run = op(run, e[h]);
+                x[h] = inclusive ? run : before;
+            }
+            o[w] = P::pack_word(x);
+        }
+        r.v[k] = o;
+        // packed here and now: left to itself the compiler keeps the unpacked values of several vectors alive and
+        // packs them late, which spilled 16 registers
+        asm volatile("" : "+v"(r.v[k]));
+    }
+    return carry;
+}
+
+template <typename In, typename T, typename Op, int K, int NW>
+__device__ __forceinline__ void packed_tile_store(In* __restrict__ out, int64_t e0, int valid, T base, Op op, const PackedRegs<K>& r) {
+    typedef Packed<In, T> P;
+    constexpr int PV = P::PV;
+    constexpr int TILE = NW * WAVE * PV * K;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int woff = wave * (WAVE * PV * K) + lane * PV;
+    In* p = out + e0 + woff;
+    const bool full = valid == TILE;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        PackedVec o;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            T e[P::PW];
+            P::unpack_word(r.v[k][w], e);
+#pragma unroll
+            for (int h = 0; h < P::PW; ++h) e[h] = op(base, e[h]);
+            o[w] = P::pack_word(e);
+        }
+        if (full || woff + k * WAVE * PV < valid) store_nt((PackedVec*)(p + k * WAVE * PV), o);
+    }
+}
+
 // Aggregate of another tile of the same line, computed from the input by the calling wave (the look-back's way out
 // when that tile's workgroup is not there to publish it: desc_lookback_alone).  Lines of whole, aligned vectors; every
 // tile in front of another is full.
@@ -734,17 +862,20 @@ inline int ordered_ticket_group(int64_t nblocks) {
 // advances it and clears a rotating slice of unused descriptor slots, like chain_finish.
 // Compiled for 8 waves per SIMD (<= 64 registers); only launched for 4-byte values with aligned lines: 8-byte values
 // hold the same 32 registers of data but scan with twice the temporaries and spilled 20 registers at that limit.
-template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K, int NW>
+// PACKED: 1- and 2-byte integers stay packed in the registers (see Packed): the tile is 128 KiB of them, not 32 or 64.
+template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K, int NW, bool PACKED = false>
 __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len,
                                                                     int64_t tiles_per_line, int64_t ntiles, T init, int inclusive, Op op,
                                                                     unsigned long long* counter, uint32_t* tickets, int ticket_group,
                                                                     uint64_t* desc, int64_t ngroups_per_line, int64_t ngroups,
                                                                     int64_t desc_capacity, WaitCtl wc, WaitAlone wa, int stagger_ticks, int stagger_tiles, int dynamic_ids) {
-    constexpr int VEC = 16 / sizeof(T);
+    constexpr int VEC = PACKED ? 16 / (int)sizeof(In) : 16 / (int)sizeof(T);    // elements per 16-byte register group
     constexpr int TILE = NW * WAVE * VEC * K;
+    typedef typename std::conditional<PACKED, PackedRegs<K>, TileRegs<T, K>>::type Regs;
+    typedef typename std::conditional<PACKED, PackedVec, typename VecOf<T, 16 / sizeof(T)>::type>::type VT;
     __shared__ T lds_wave[NW];
     __shared__ T lds_prefix;
-    __shared__ typename VecOf<T, VEC>::type lds_stash[K][WAVE];         // wave 0's registers while it resolves its prefix alone
+    __shared__ VT lds_stash[K][WAVE];         // wave 0's registers while it resolves its prefix alone
     const T ident = Op::template identity<T>();
     const int tid = threadIdx.x, wave = tid / WAVE, lane = lane_id();
     uint64_t* tile_desc = desc;                                        // [words][ntiles]
@@ -766,8 +897,10 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
         const int64_t e0 = line * line_len + tl * TILE;
         const int64_t left = line_len - tl * TILE;
         const int valid = left < TILE ? (int)left : TILE;
-        TileRegs<T, K> r;
-        const T wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, inclusive, op, r);
+        Regs r;
+        T wtot;
+        if constexpr (PACKED) wtot = packed_tile_load_scan<In, T, Op, K, NW>(in, e0, valid, inclusive, op, r);
+        else wtot = tile_load_scan<In, T, Op, VECTOR, K, NW>(in, e0, valid, inclusive, op, r);
         if (lane == 0) lds_wave[wave] = wtot;
         __syncthreads();
         if (wave == 0) {
@@ -783,7 +916,6 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
                 // registers, the tile takes 32 of them, and the way out of an endless wait (desc_lookback_alone, which
                 // reads other tiles) needs more than the rest -- with the tile in registers the compiler made room in
                 // private memory, inside the tile's scan.  Sixteen LDS accesses a tile, by one wave of sixteen.
-                typedef typename VecOf<T, VEC>::type VT;
                 volatile VT* stash = &lds_stash[0][lane];
 #pragma unroll
                 for (int k = 0; k < K; ++k) stash[k * WAVE] = r.v[k];
@@ -799,7 +931,8 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
             if (lane == 0) lds_prefix = tile_prefix;
         }
         __syncthreads();
-        tile_store<Out, T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
+        if constexpr (PACKED) packed_tile_store<In, T, Op, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
+        else tile_store<Out, T, Op, VECTOR, K, NW>(out, e0, valid, op(lds_prefix, lds_wave[wave]), op, r);
     }
     ordered_finish(epoch, (int64_t)Words<T>::N * ntiles + ngroups * GROUP_DESC_STRIDE, counter, tickets, ticket_group, desc, desc_capacity);
 }
@@ -1800,6 +1933,7 @@ int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
 int tune_scan_rows_packed();     // rk_api.hip: 0 = short rows never take the single-pass kernel with several rows per load
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
+int tune_scan_packed();          // rk_api.hip: 0 = 1- and 2-byte integers never take the packed tiles of the single-pass scan
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
 struct ScanArgs {
@@ -2120,8 +2254,13 @@ inline int32_t launch_scan(const ScanArgs& a) {
     // empty, and a half-idle workgroup of 1024 threads holds half a compute unit: 3000 lines of 20000 Float32 139 us
     // with 16 waves, 85 us with 8; 1300 lines of 50000: 119 against 97; 600 lines of 100000: 88 against 85
     // -- so 16 waves only where their tiles are at least 90 % full (65536 x 1024 Int32, two full tiles a line: 96 against 101 us)
-    const int nw = scan_tile_waves(s.mid, sizeof(T));
-    const int64_t TILE = (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
+    // 1- and 2-byte integers on lines of whole, 16-byte aligned vectors that fill tiles of 128 KiB: the packed tiles
+    constexpr bool CAN_PACK = std::is_integral<In>::value && std::is_same<In, Out>::value && sizeof(In) <= 2 && sizeof(T) == 4;
+    constexpr int PVEC = 16 / (int)sizeof(In);
+    const bool packed = CAN_PACK && tune_scan_packed() != 0 && tune_scan_dynamic_ids() == 0 && is_aligned(in, 16) && is_aligned(out, 16) &&
+                        s.mid % PVEC == 0 && scan_tile_waves(s.mid, sizeof(In)) == 16;
+    const int nw = packed ? 16 : scan_tile_waves(s.mid, sizeof(T));
+    const int64_t TILE = packed ? (int64_t)16 * WAVE * PVEC * KT : (int64_t)ScanTile<T, KT>::TILE / 4 * nw;
     const int64_t tpl = (s.mid + TILE - 1) / TILE;
     const int64_t ntiles = tpl * nlines;
     if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
@@ -2148,8 +2287,16 @@ inline int32_t launch_scan(const ScanArgs& a) {
             // (narrow elements: half the bytes a tile, half the stagger -- Int16[2^26]: 0 / 1 / 2 / 3 / 4 / 5 / 7 us -> 53.0 / 51.9 / 51.6 /
             // 51.6 / 51.7 / 52.7 / 53.2 us)
             const int stagger_tiles = (nw == 16 && ntiles >= 2 * resident) ? (int)resident : 0;
-            const int stagger_ticks = tune_scan_stagger_ticks() * (int)(sizeof(In) + sizeof(Out)) / (int)(2 * sizeof(T));
+            const int stagger_ticks = packed ? tune_scan_stagger_ticks() : tune_scan_stagger_ticks() * (int)(sizeof(In) + sizeof(Out)) / (int)(2 * sizeof(T));
             const int dyn = ordered_dynamic_ids(ntiles, nw * WAVE, true);
+            if constexpr (CAN_PACK) {
+                if (packed) {
+                    scan_ordered_kernel<In, T, Out, Op, true, KT, 16, true><<<(unsigned)ntiles, 16 * WAVE, 0, a.stream>>>(
+                        in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, ordered_ticket_group(ntiles), w.desc, gpl, ngroups, cap, wc, wait_alone(w.hdr), stagger_ticks, stagger_tiles, dyn);
+                    RK_LAUNCH_CHECK();
+                    return RK_SUCCESS;
+                }
+            }
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED
             RK_LAUNCH_CHECK();

@@ -335,6 +335,44 @@ def test_narrow_element_types(rk, orc, dtype):
             assert np.array_equal(rk.Array(dy), want.astype(dt))
 
 
+@pytest.mark.parametrize("dtype", [np.int8, np.uint8, np.int16, np.uint16])
+def test_long_lines_of_narrow_integers(rk, orc, dtype):
+    """Lines of 1- and 2-byte integers long enough for the packed tiles of the single-pass scan (128 KiB of elements a
+    tile, kept packed in the registers): every operator, inclusive and exclusive with an init, a last tile that is
+    nearly empty or nearly full, several lines, in place.  The same arrays through the widened tiles (a length that is
+    no whole number of 16-byte vectors) as a cross-check of the shapes.  Bit-exact against the oracle."""
+    rng = np.random.default_rng(94)
+    dt = np.dtype(dtype)
+    info = np.iinfo(dt)
+    tile = 16 * 64 * 8 * (16 // dt.itemsize)
+    shapes = (((12 * tile + 48,), 1), ((13 * tile - 16,), 1), ((11 * tile, 3), 1), ((12 * tile + 3,), 1))
+    for shape, dims in shapes:
+        x = rng.integers(info.min, info.max + 1, shape).astype(dt)
+        dx = rk.ROCArray(x)
+        for op in ("add", "mul", "max", "min", "and", "or", "xor"):
+            src, d = x, dx
+            if op == "mul":
+                src = rng.integers(1, 4, shape).astype(dt)
+                d = rk.ROCArray(src)
+            elif op in ("max", "min"):
+                # a slowly drifting sequence, so that the running extremum keeps changing along the line
+                src = (np.arange(x.size).reshape(shape, order="F") // 7000 * (1 if op == "max" else -1) + rng.integers(-3, 4, shape)).astype(dt)
+                d = rk.ROCArray(src)
+            got = rk.Array(rk.accumulate(op, d, dims=dims))
+            assert got.dtype == dt and np.array_equal(got, orc.accumulate(op, src, dims=dims).astype(dt)), (shape, op)
+            init = dt.type(src.reshape(-1)[5])
+            got = rk.Array(rk.accumulate(op, d, dims=dims, init=init, inclusive=False))
+            assert np.array_equal(got, orc.accumulate(op, src, dims=dims, init=init, inclusive=False).astype(dt)), (shape, op, "exclusive")
+        if info.min < 0:
+            # an init below every element: the exclusive scan's first value is the init itself
+            init = dt.type(info.min)
+            got = rk.Array(rk.accumulate("max", dx, dims=dims, init=init, inclusive=False))
+            assert np.array_equal(got, orc.accumulate("max", x, dims=dims, init=init, inclusive=False).astype(dt))
+        dy = rk.ROCArray(x)
+        assert rk.accumulate_("add", dy, dy, dims=dims) is dy
+        assert np.array_equal(rk.Array(dy), orc.accumulate("add", x, dims=dims).astype(dt))
+
+
 @pytest.mark.parametrize("m", [8, 9, 11, 129, 255, 1001, 2047, 2049, 3001, 4095, 4097, 8189, 8190, 8191])
 def test_lines_that_start_at_odd_addresses(rk, orc, m):
     """cumsum(A; dims=1) with a line length that is no whole number of 16-byte vectors: every line starts at another

@@ -142,6 +142,27 @@ def test_ordered_scan_helps_itself(rk, orc, tiny_budget, n):
     assert L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr()) == 0
 
 
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+def test_packed_ordered_scan_helps_itself(rk, orc, tiny_budget, dtype):
+    """The same for the packed tiles of 1- and 2-byte integers (a tile is 128 KiB of elements; the aggregates a tile
+    computes for its predecessors are read from the input in the widened way)."""
+    L = tiny_budget
+    from amdgpu_jl_amd.array import stream_ptr
+    rng = np.random.default_rng(17)
+    n = (1 << 24) + 4096
+    h = rng.integers(-100, 101, n).astype(dtype)
+    x = rk.ROCArray(h)
+    out = rk.ROCArray(dims=x.dims, dtype=dtype)
+    ws = _fresh_workspace(L, 16 << 20)
+    for op, code in (("add", L.RK_OP_ADD), ("max", L.RK_OP_MAX)):
+        out.buf.zero_()
+        assert L.lib.rk_accumulate(code, x.code, out.code, x.ptr, out.ptr, 1, L.shape_array(x.dims), 1, 1, None,
+                                   ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+        assert L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+        assert np.array_equal(rk.Array(out), orc.accumulate(op, h, dims=1).astype(dtype))
+    assert _alone_count(ws) > 0
+
+
 def test_ordered_scan_of_many_lines_helps_itself(rk, orc, tiny_budget):
     L = tiny_budget
     from amdgpu_jl_amd.array import stream_ptr
