@@ -90,6 +90,20 @@ template <typename In, typename Acc> struct ProgXform {
         return y;
     }
 };
+// f = one arithmetic operator between the element and a constant -- x + c, c + x, x - c, c - x, x * c, c * x; the
+// reference's own benchmark closure is x -> x + 1 (perf/array.jl:107-122) -- needs no interpreter: it is x * m + a
+// with (m, a) = (1, c), (1, -c), (-1, c), (c, -0.0).  Each of these is the operator's own value bit for bit, fused or
+// not: a product with +-1 is exact, x - c is x + (-c) in IEEE arithmetic, and adding -0.0 changes nothing, not even
+// the sign of a zero.  Integers wrap in 64 bits like the interpreter's.
+template <typename In, typename Acc> struct AffineXform {
+    typedef int64_t Pos;
+    typedef typename ProgXform<In, Acc>::CT CT;
+    CT m, a;
+    __device__ __forceinline__ Acc operator()(In x, int64_t) const {
+        if constexpr (std::is_integral<CT>::value) return (Acc)wrap_add(wrap_mul((CT)x, m), a);
+        else return (Acc)((CT)x * m + a);
+    }
+};
 template <typename Xf> struct XfIsArg : std::false_type {};
 template <typename T, typename P, bool WANT_MAX> struct XfIsArg<ArgXform<T, P, WANT_MAX>> : std::true_type {};
 template <typename Xf> struct XfIsBatch : std::false_type {};
@@ -1272,9 +1286,33 @@ inline ProgXform<In, Acc> make_prog_xform(const rk_map_program& p) {
         xf.c[k] = k < p.n_consts ? (std::is_floating_point<CT>::value ? (CT)p.const_f[k] : (CT)p.const_i[k]) : CT(0);
     return xf;
 }
+// The three-token programs `x c op` / `c x op` with op one of + - * as x * m + a (AffineXform).
+template <typename In, typename Acc>
+inline bool affine_of(const rk_map_program& p, AffineXform<In, Acc>* out) {
+    typedef typename AffineXform<In, Acc>::CT CT;
+    if (p.n_tokens != 3 || p.n_consts < 1) return false;
+    const int t0 = p.tokens[0], t1 = p.tokens[1], op = p.tokens[2];
+    const bool x_first = t0 == 0 && t1 == 1, c_first = t0 == 1 && t1 == 0;
+    if (!x_first && !c_first) return false;
+    const CT c = std::is_floating_point<CT>::value ? (CT)p.const_f[0] : (CT)p.const_i[0];
+    const CT zero = std::is_floating_point<CT>::value ? (CT)-0.0 : CT(0);
+    switch (op) {
+        case RK_BC_ADD: *out = {CT(1), c}; return true;
+        case RK_BC_SUB:
+            if (x_first) *out = {CT(1), std::is_integral<CT>::value ? wrap_mul(c, (CT)-1) : (CT)-c};
+            else *out = {(CT)-1, c};
+            return true;
+        case RK_BC_MUL: *out = {c, zero}; return true;
+        default: return false;
+    }
+}
 template <typename In, typename Acc, bool ADD_ONLY = false>
 inline int32_t mapreduce_prog(const MapreduceArgs& a) {
     typedef ProgXform<In, Acc> Xf;
+    if (a.op == RK_OP_ADD) {
+        AffineXform<In, Acc> ax{};
+        if (affine_of<In, Acc>(*a.prog, &ax)) return mapreduce_one<In, Acc, AffineXform<In, Acc>, OpAdd>(a, ax);
+    }
     const Xf xf = make_prog_xform<In, Acc>(*a.prog);
     if constexpr (ADD_ONLY) return a.op == RK_OP_ADD ? mapreduce_one<In, Acc, Xf, OpAdd>(a, xf) : (int32_t)RK_ERR_UNSUPPORTED;
     else switch (a.op) {

@@ -58,6 +58,37 @@ def test_mapreduce_plus_one_ints(rk, orc, shape, dtype):
             assert got.dtype == dtype and np.array_equal(rk.Array(got), want)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int64, np.int32])
+def test_one_operator_closures(rk, orc, dtype):
+    """x + c, c + x, x - c, c - x, x * c, c * x under `+`: the library evaluates these without its interpreter (as
+    x * m + a), which must not change a value -- integers bit-exact, floats within the tolerance of the sums, and the
+    mapped values themselves (a reduction over a dim of extent 1; the sum starts from +0, so a -0 does not survive it,
+    here as in the reference's neutral-element reductions) exactly."""
+    rng = _rng(31)
+    c = dtype(3) if np.dtype(dtype).kind == "i" else dtype(1.7)
+    forms = [(lambda v: v + c, lambda x: x + c), (lambda v: c + v, lambda x: c + x), (lambda v: v - c, lambda x: x - c),
+             (lambda v: c - v, lambda x: c - x), (lambda v: v * c, lambda x: x * c), (lambda v: c * v, lambda x: c * x)]
+    for shape in ((100_003,), (300, 1001), (7, 33, 900)):
+        x = (rng.integers(-50, 51, shape).astype(dtype) if np.dtype(dtype).kind == "i"
+             else (rng.standard_normal(shape) * 3).astype(dtype))
+        x.reshape(-1)[:4] = [0, -0.0, 1, -1] if np.dtype(dtype).kind == "f" else [0, 0, 1, -1]
+        a = rk.ROCArray(x)
+        for f, g in forms:
+            mapped = g(x)
+            for dims in _dims_for(shape):
+                got = rk.mapreduce(f, "add", a, dims=dims)
+                want = orc.mapreduce("identity", "add", mapped, dims=dims)
+                got = np.asarray(got if dims is None else rk.Array(got)).reshape(want.shape)
+                if np.dtype(dtype).kind == "i":
+                    assert got.dtype == want.dtype and np.array_equal(got, want)
+                else:
+                    np.testing.assert_allclose(got, want, rtol=RTOL, atol=1e-3 if dtype == np.float32 else 1e-9)
+            # every output is one mapped element: the value of f itself
+            one = rk.ROCArray(x.reshape(shape + (1,)))
+            got = rk.Array(rk.mapreduce(f, "add", one, dims=len(shape) + 1)).reshape(shape)
+            assert got.dtype == mapped.dtype and np.array_equal(got, mapped)
+
+
 def test_int32_maps_wrap_like_julia(rk, orc):
     x = _rng(3).integers(-2**31, 2**31, (300, 1001)).astype(np.int32)
     with np.errstate(over="ignore"):
