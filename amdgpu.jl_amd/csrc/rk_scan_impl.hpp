@@ -392,6 +392,9 @@ __device__ __forceinline__ T tile_scan_regs(int inclusive, Op op, TileRegs<T, K>
             for (int j = VEC - 1; j > 0; --j) r.v[k][j] = op(excl, r.v[k][j - 1]);
             r.v[k][0] = excl;
         }
+        // 8-byte values: one vector at a time.  Interleaved, the wave scans of several vectors (two registers a value,
+        // no DPP form of the 64-bit operators) need more temporaries than the 64-register kernels have left
+        if constexpr (sizeof(T) == 8) asm volatile("" : "+v"(r.v[k]));
     }
     return carry;
 }
@@ -860,8 +863,9 @@ inline int ordered_ticket_group(int64_t nblocks) {
 // tiles without any look-back: 86 us) but lose more to the look-back than they gain.
 // The epoch of the call is read from the workspace header; the workgroup that leaves last (two-level exit tickets)
 // advances it and clears a rotating slice of unused descriptor slots, like chain_finish.
-// Compiled for 8 waves per SIMD (<= 64 registers); only launched for 4-byte values with aligned lines: 8-byte values
-// hold the same 32 registers of data but scan with twice the temporaries and spilled 20 registers at that limit.
+// Compiled for 8 waves per SIMD (<= 64 registers), for aligned lines.  8-byte values hold the same 32 registers of
+// data but scan with twice the temporaries: their vectors are scanned strictly one after the other (tile_scan_regs),
+// which keeps them inside the 64 registers (interleaved they spilled 20).
 // PACKED: 1- and 2-byte integers stay packed in the registers (see Packed): the tile is 128 KiB of them, not 32 or 64.
 template <typename In, typename T, typename Out, typename Op, bool VECTOR, int K, int NW, bool PACKED = false>
 __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __restrict__ in, Out* __restrict__ out, int64_t line_len,
@@ -1933,6 +1937,7 @@ int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
 int tune_scan_rows_packed();     // rk_api.hip: 0 = short rows never take the single-pass kernel with several rows per load
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
+int tune_scan_ordered8();        // rk_api.hip: 0 = 8-byte values take the counter-fed scan_chain_kernel
 int tune_scan_packed();          // rk_api.hip: 0 = 1- and 2-byte integers never take the packed tiles of the single-pass scan
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
 
@@ -2266,16 +2271,19 @@ inline int32_t launch_scan(const ScanArgs& a) {
     if (ntiles > 0x3fffffff) return RK_ERR_TOO_LARGE;
     Workspace w{};
     const int64_t gpl = (tpl + WAVE - 1) / WAVE, ngroups = gpl * nlines;
-    // 8-byte values and unaligned lines do not fit two workgroups a compute unit; with one, the persistent counter-fed
-    // kernel is the faster of the two (cumsum of Int64[2^25]: 96 against 107 us)
-    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || sizeof(T) > 4 || !lines_aligned;
+    // Unaligned lines do not fit two workgroups a compute unit; with one, the persistent counter-fed kernel is the
+    // faster of the two.  8-byte values take the launch-order kernel since their tile scan fits its 64 registers
+    // (RK_SCAN_ORDERED8=0: the counter-fed one; cumsum of Int64[2^25] 99.5 -> 88 us, Float64[2^26] 192 -> 173,
+    // Bool -> Int64 at 2^26 122 -> 101)
+    constexpr bool ORDERED8 = sizeof(T) == 8;
+    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || (sizeof(T) > 4 && !(ORDERED8 && tune_scan_ordered8() != 0)) || !lines_aligned;
     const size_t need = dynamic_ids ? (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t)
                                     : ((size_t)ntiles * Words<T>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
     const int64_t cap = (int64_t)(w.desc_bytes / sizeof(uint64_t));
     unsigned long long* counter = (unsigned long long*)&w.hdr->scan_counter;
     const WaitCtl wc = wait_ctl(w.hdr);
-    if constexpr (sizeof(T) <= 4) {
+    if constexpr (sizeof(T) <= 4 || ORDERED8) {
         if (!dynamic_ids) {
 #define RK_SCAN_ORDERED(NWW)                                                                                          \
             scan_ordered_kernel<In, T, Out, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \

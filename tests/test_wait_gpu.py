@@ -163,6 +163,26 @@ def test_packed_ordered_scan_helps_itself(rk, orc, tiny_budget, dtype):
     assert _alone_count(ws) > 0
 
 
+@pytest.mark.parametrize("dtype", [np.int64, np.float64, np.bool_])
+def test_ordered_scan_of_8_byte_values_helps_itself(rk, orc, tiny_budget, dtype):
+    """8-byte values (and Bool -> Int64) run the same single-pass kernel: with a patience of one poll the tiles resolve
+    their prefixes alone, the result is exact and the status clean."""
+    L = tiny_budget
+    from amdgpu_jl_amd.array import stream_ptr
+    rng = np.random.default_rng(18)
+    n = (1 << 23) + 2048
+    h = (rng.random(n) < 0.5) if dtype == np.bool_ else rng.integers(-1000, 1001, n).astype(dtype)
+    out_dtype = np.int64 if dtype == np.bool_ else dtype
+    x = rk.ROCArray(h)
+    out = rk.ROCArray(dims=x.dims, dtype=out_dtype)
+    ws = _fresh_workspace(L, 16 << 20)
+    assert L.lib.rk_accumulate(L.RK_OP_ADD, x.code, out.code, x.ptr, out.ptr, 1, L.shape_array(x.dims), 1, 1, None,
+                               ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+    assert L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+    assert np.array_equal(rk.Array(out), np.cumsum(h, dtype=out_dtype))        # integer-valued: exact in Float64 too
+    assert _alone_count(ws) > 0
+
+
 def test_ordered_scan_of_many_lines_helps_itself(rk, orc, tiny_budget):
     L = tiny_budget
     from amdgpu_jl_amd.array import stream_ptr
