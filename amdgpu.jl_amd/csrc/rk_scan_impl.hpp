@@ -415,6 +415,15 @@ __device__ __forceinline__ T tile_load_scan(const In* __restrict__ in, int64_t e
 #pragma unroll
             for (int j = 0; j < VEC; ++j) r.v[k][j] = (T)x[j];
         }
+    } else if (!VECTOR && ElemVectors<In, T>::value && valid == TILE) {
+        // a full tile of a line that starts at an odd address: the same loads at element-aligned addresses
+        const In* p = in + e0 + woff;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const VI x = ElemVectors<In, T>::template load<VEC>(p + k * WAVE * VEC);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) r.v[k][j] = (T)x[j];
+        }
     } else if (VECTOR && valid % VEC == 0) {
         // a tile that its line does not fill (every line of cumsum(A; dims=1) on a 3000 x N array): whole vectors all
         // the same, and every lane issues its K loads unconditionally -- a vector past the end reads the tile's first
@@ -477,6 +486,15 @@ __device__ __forceinline__ void tile_store(Out* __restrict__ out, int64_t e0, in
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
             out_store_nt<Out, T, VEC>(p + k * WAVE * VEC, o);
+        }
+    } else if (!VECTOR && OutElemVectors<Out, T>::value && valid == TILE) {
+        Out* p = out + e0 + woff;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            VT o;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o[j] = op(base, r.v[k][j]);
+            out_store_elems<Out, T, VEC>(p + k * WAVE * VEC, o);
         }
     } else if (VECTOR && valid % VEC == 0) {
 #pragma unroll
@@ -643,7 +661,7 @@ __device__ __forceinline__ void packed_tile_store(In* __restrict__ out, int64_t 
 // Aggregate of another tile of the same line, computed from the input by the calling wave (the look-back's way out
 // when that tile's workgroup is not there to publish it: desc_lookback_alone).  Lines of whole, aligned vectors; every
 // tile in front of another is full.
-template <typename In, typename T, typename Op, int TILE> struct ScanTileAggregate {
+template <typename In, typename T, typename Op, int TILE, bool VECTOR = true> struct ScanTileAggregate {
     const In* first;        // first element of the asking tile
     int64_t   tile;         // its number
     __device__ __forceinline__ T operator()(int64_t p) const {
@@ -653,7 +671,9 @@ template <typename In, typename T, typename Op, int TILE> struct ScanTileAggrega
         const In* q = first - (tile - p) * (int64_t)TILE;
         T acc = Op::template identity<T>();
         for (int i = lane_id() * VEC; i < TILE; i += WAVE * VEC) {
-            const VI x = *(const VI*)(q + i);
+            VI x;
+            if constexpr (VECTOR) x = *(const VI*)(q + i);
+            else x = ElemVectors<In, T>::template load<VEC>(q + i);        // lines at element-aligned addresses
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc = op(acc, (T)x[j]);
         }
@@ -928,7 +948,7 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
                 tile_prefix = desc_lookback_leader(tile_desc, ntiles, group_desc, tile, tl, gl, epoch, tile_agg, init, op, ident, wc, wa, expired);
                 if (expired)
                     tile_prefix = desc_lookback_alone(tile_desc, ntiles, group_desc, tile, tl, gl, epoch, tile_agg, init, op, ident,
-                                                      ScanTileAggregate<In, T, Op, TILE>{in + e0, tile}, wa.counter);
+                                                      ScanTileAggregate<In, T, Op, TILE, VECTOR>{in + e0, tile}, wa.counter);
 #pragma unroll
                 for (int k = 0; k < K; ++k) r.v[k] = stash[k * WAVE];
             }
@@ -1937,6 +1957,7 @@ int tune_scan_blocks_per_cu();  // rk_api.hip
 int tune_scan_rows_ordered();    // rk_api.hip: 0 = scans across rows always take the three-pass path
 int tune_scan_rows_packed();     // rk_api.hip: 0 = short rows never take the single-pass kernel with several rows per load
 int tune_scan_dynamic_ids();     // rk_api.hip: 1 = tile ids from a counter (scan_chain_kernel) instead of launch order
+int tune_scan_ordered_unaligned();   // rk_api.hip: 0 = lines at odd addresses take the counter-fed scan_chain_kernel
 int tune_scan_ordered8();        // rk_api.hip: 0 = 8-byte values take the counter-fed scan_chain_kernel
 int tune_scan_packed();          // rk_api.hip: 0 = 1- and 2-byte integers never take the packed tiles of the single-pass scan
 int tune_scan_slice_blocks_per_cu();  // rk_api.hip: workgroups per compute unit the sliced scan across rows aims for
@@ -2276,7 +2297,12 @@ inline int32_t launch_scan(const ScanArgs& a) {
     // (RK_SCAN_ORDERED8=0: the counter-fed one; cumsum of Int64[2^25] 99.5 -> 88 us, Float64[2^26] 192 -> 173,
     // Bool -> Int64 at 2^26 122 -> 101)
     constexpr bool ORDERED8 = sizeof(T) == 8;
-    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || (sizeof(T) > 4 && !(ORDERED8 && tune_scan_ordered8() != 0)) || !lines_aligned;
+    // lines at odd addresses (or of a length that is no whole number of vectors): the same kernel with 16-byte accesses
+    // at element-aligned addresses, where the element types allow them
+    constexpr bool ORDERED_ELEMS = ElemVectors<In, T>::value && OutElemVectors<Out, T>::value;
+    const bool ordered_unaligned = ORDERED_ELEMS && tune_scan_ordered_unaligned() != 0;
+    const bool dynamic_ids = tune_scan_dynamic_ids() != 0 || (sizeof(T) > 4 && !(ORDERED8 && tune_scan_ordered8() != 0)) ||
+                             (!lines_aligned && !ordered_unaligned);
     const size_t need = dynamic_ids ? (size_t)(ntiles + ngroups) * Words<T>::N * sizeof(uint64_t)
                                     : ((size_t)ntiles * Words<T>::N + (size_t)ngroups * GROUP_DESC_STRIDE) * sizeof(uint64_t);
     if (!carve_workspace(a.ws, a.ws_bytes, need, &w)) return RK_ERR_WORKSPACE;
@@ -2285,9 +2311,14 @@ inline int32_t launch_scan(const ScanArgs& a) {
     const WaitCtl wc = wait_ctl(w.hdr);
     if constexpr (sizeof(T) <= 4 || ORDERED8) {
         if (!dynamic_ids) {
-#define RK_SCAN_ORDERED(NWW)                                                                                          \
-            scan_ordered_kernel<In, T, Out, Op, true, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
+#define RK_SCAN_ORDERED_V(VECF, NWW)                                                                                  \
+            scan_ordered_kernel<In, T, Out, Op, VECF, KT, NWW><<<(unsigned)ntiles, NWW * WAVE, 0, a.stream>>>(               \
                 in, out, s.mid, tpl, ntiles, init, inclusive, op, counter, w.tickets, ordered_ticket_group(ntiles), w.desc, gpl, ngroups, cap, wc, wait_alone(w.hdr), stagger_ticks, stagger_tiles, dyn)
+#define RK_SCAN_ORDERED(NWW)                                                                                          \
+            do {                                                                                                      \
+                if constexpr (ORDERED_ELEMS) { if (lines_aligned) RK_SCAN_ORDERED_V(true, NWW); else RK_SCAN_ORDERED_V(false, NWW); } \
+                else RK_SCAN_ORDERED_V(true, NWW);                                                                    \
+            } while (0)
             // staggered start of the first resident round (two workgroups of 16 waves a compute unit), where more rounds
             // follow: 5 us across the round measured best (2^26 Int32: 0 / 2 / 4 / 6 / 8 / 12 / 16 us -> 91.8 / 90.3 / 89.7 /
             // 89.9 / 90.1 / 90.9 / 92.0 us; 2^27: 177.9 -> 174.0 us; half the round late by a fixed time gained nothing)
@@ -2307,6 +2338,7 @@ inline int32_t launch_scan(const ScanArgs& a) {
             }
             if (nw == 16) RK_SCAN_ORDERED(16); else if (nw == 8) RK_SCAN_ORDERED(8); else RK_SCAN_ORDERED(4);
 #undef RK_SCAN_ORDERED
+#undef RK_SCAN_ORDERED_V
             RK_LAUNCH_CHECK();
             return RK_SUCCESS;
         }

@@ -402,6 +402,40 @@ def test_lines_that_start_at_odd_addresses(rk, orc, m):
     np.testing.assert_allclose(rk.Array(rk.cumsum(v)), np.cumsum(flat[3:m + 3].astype(np.float64)), rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.float64, np.int64])
+def test_long_lines_at_odd_addresses(rk, orc, dtype):
+    """Lines longer than a tile that start at element-aligned but not 16-byte-aligned addresses -- a view x[2:end], the
+    columns of a 20001 x N matrix -- take the single-pass kernel with its 16-byte accesses at element-aligned addresses:
+    one long line (many tiles, the last one partly filled), several lines of a few tiles each, in place, exclusive with
+    an init.  Integers bit-exact, floats rtol 1e-4 of the Float64 scan."""
+    rng = np.random.default_rng(77)
+    dt = np.dtype(dtype)
+
+    def check(got, x, dims, **kw):
+        want = orc.accumulate("add", x, dims=dims, **kw)
+        if dt.kind == "f":
+            np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-2 if dt == np.float32 else 1e-8)
+        else:
+            assert np.array_equal(got, want.astype(dt))
+
+    n = (1 << 22) + 37
+    flat = rng.integers(-100, 101, n + 8).astype(dt)
+    d = rk.ROCArray(flat)
+    for first in (2, 4):                                           # byte offsets 1 and 3 elements
+        v = d.view_range(first, first + n - 1)
+        x = flat[first - 1:first - 1 + n]
+        check(rk.Array(rk.cumsum(v)), x, 1)
+        check(rk.Array(rk.accumulate("add", v, init=dt.type(5), inclusive=False)), x, 1, init=dt.type(5), inclusive=False)
+        if dt.kind != "f":
+            assert np.array_equal(rk.Array(rk.accumulate("max", v)), orc.accumulate("max", x, dims=1))
+    for shape in ((20_001, 150), (70_003, 31), (300_001, 6)):
+        x = rng.integers(-100, 101, shape).astype(dt)
+        check(rk.Array(rk.cumsum(rk.ROCArray(x), dims=1)), x, 1)
+        dy = rk.ROCArray(x)
+        assert rk.accumulate_("add", dy, dy, dims=1) is dy
+        check(rk.Array(dy), x, 1)
+
+
 @pytest.mark.parametrize("shape", [(257, 300), (1001, 1000), (4097, 130), (65, 5000), (130, 70, 5), (67, 40, 9), (8191, 33),
                                    (200, 3, 50), (1001, 5, 7), (4099, 16, 2), (256, 2, 40)])
 def test_scans_across_rows_that_are_no_whole_vectors(rk, orc, shape):

@@ -183,6 +183,22 @@ def test_ordered_scan_of_8_byte_values_helps_itself(rk, orc, tiny_budget, dtype)
     assert _alone_count(ws) > 0
 
 
+def test_ordered_scan_at_odd_addresses_helps_itself(rk, orc, tiny_budget):
+    """Lines that start at odd addresses: the tiles that help themselves read their predecessors' elements with vectors
+    at element-aligned addresses."""
+    L = tiny_budget
+    from amdgpu_jl_amd.array import stream_ptr
+    rng = np.random.default_rng(19)
+    h = rng.integers(-1000, 1001, ((1 << 21) + 1, 9), dtype=np.int32)     # nine lines of 65 tiles, every line at another alignment
+    x = rk.ROCArray(h)
+    out = rk.ROCArray(dims=x.dims, dtype=np.int32)
+    ws = _fresh_workspace(L, 16 << 20)
+    assert _scan(L, rk, x, out, ws, dims=1) == 0
+    assert L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+    assert np.array_equal(rk.Array(out), orc.accumulate("add", h, dims=1))
+    assert _alone_count(ws) > 0
+
+
 def test_ordered_scan_of_many_lines_helps_itself(rk, orc, tiny_budget):
     L = tiny_budget
     from amdgpu_jl_amd.array import stream_ptr
