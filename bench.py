@@ -465,7 +465,7 @@ def main():
             run_row("cumsum(B;dims=2) 4096x16384 Float32", rows * cols, 8 * rows * cols, lambda i: pb[i % 2](), reps,
                     cpu=lambda: cpu_row(lambda t: cpu_lib.orc_cumsum_dims2_f32(P(hx), I64(rows), I64(cols), P(hz), t), 8 * rows * cols, "full size"))
             del Bi, Bo, pa, pb
-        # scans of 2-byte elements, native (read narrow, scanned in 32 bits, stored narrow): 4 bytes of traffic per element
+        # scans of 2-byte elements, native (read narrow, scanned in 32 bits, stored narrow; integers stay packed in the registers): 4 bytes of traffic per element
         if wanted("Int16") or wanted("Float16") or wanted("Float64"):
             m = 1 << 26
             hi16 = [dev_array(randint_i32(m).to(torch.int16), (m,), np.int16) for _ in range(3)]
