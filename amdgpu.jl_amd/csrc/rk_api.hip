@@ -97,6 +97,12 @@ int tune_scan_dynamic_ids() {
 
 // 0: long lines of 1- and 2-byte integers are scanned in widened tiles of 32 Ki elements instead of packed ones of 128 KiB
 // (RK_SCAN_PACKED).
+// 0: the tile-a-line scan runs four waves a workgroup whatever the line length (RK_SCAN_TILES_WAVES).
+int tune_scan_tiles_waves() {
+    static const int v = env_int("RK_SCAN_TILES_WAVES", 1, 0, 1);
+    return v;
+}
+
 // 0: long lines at odd addresses are scanned by the persistent counter-fed kernel instead of the one in launch order
 // (RK_SCAN_ORDERED_UNALIGNED).
 int tune_scan_ordered_unaligned() {
