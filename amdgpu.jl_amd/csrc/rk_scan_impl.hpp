@@ -194,8 +194,19 @@ __device__ __forceinline__ T desc_sum_or_compute(uint64_t* tile_desc, int64_t ts
     while (missing != 0ull) {
         const int l = __ffsll(missing) - 1;
         missing &= missing - 1ull;
-        const T a = agg_of(first + l);
-        if (lane == 0) desc_publish(tile_desc, tstride, first + l, a, tagA);
+        T a = agg_of(first + l);
+        // In place (out == in) the tile's own workgroup may have started meanwhile and be storing its results over the
+        // elements just read.  It publishes its aggregate before it stores anything (publish, look-back, stores; the
+        // first tile of a line waits for its publication), so the descriptor is read once more, AFTER the elements: still
+        // empty means no store had begun when the reads finished and `a` is sound; published means the owner's value is
+        // there to take, whatever was read.
+        asm volatile("" : "+v"(a) : : "memory");          // the descriptor's load is issued behind the reads that made `a`
+        Words<T> again = to_words(ident);
+        uint32_t st2 = 0;
+        if (lane == 0) st2 = desc_read<T>(tile_desc, tstride, first + l, tagA, tagP, again);
+        st2 = (uint32_t)__builtin_amdgcn_readfirstlane((int)st2);
+        if (st2 != 0u) a = read_lane(from_words<T>(again), 0);
+        else if (lane == 0) desc_publish(tile_desc, tstride, first + l, a, tagA);
         sum = op(sum, a);
     }
     return sum;
@@ -934,6 +945,9 @@ __global__ __launch_bounds__(NW * WAVE, 8) void scan_ordered_kernel(const In* __
             if (lane < NW) lds_wave[lane] = wave_shift_right(inc, ident);       // what lies in front of each wave inside the tile
             T tile_prefix = init;
             if (lane == 0) desc_publish(tile_desc, ntiles, tile, tile_agg, (epoch << 2) | DESC_A);
+            // a line's first tile has no look-back between this and its stores: the aggregate is out before them (a tile
+            // that helps itself in an in-place scan counts on that order, see desc_sum_or_compute)
+            if (tl == 0) publish_barrier();
             if (tl > 0) {
                 // The wave's part of the tile waits in LDS while the wave looks back: the kernel is compiled for 64
                 // registers, the tile takes 32 of them, and the way out of an endless wait (desc_lookback_alone, which

@@ -199,6 +199,29 @@ def test_ordered_scan_at_odd_addresses_helps_itself(rk, orc, tiny_budget):
     assert _alone_count(ws) > 0
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int64, np.int16])
+def test_ordered_scan_in_place_helps_itself(rk, orc, tiny_budget, dtype):
+    """In place (out is in) a tile that helps itself reads elements that their own tile may be about to overwrite with its
+    results: it takes what it computed only if that tile has still not published anything when the reads are done, and
+    the tile's own aggregate otherwise.  Several rounds, a patience of one poll, exact results every time."""
+    L = tiny_budget
+    from amdgpu_jl_amd.array import stream_ptr
+    rng = np.random.default_rng(20)
+    n = (1 << 24) + 4096
+    h = rng.integers(-100, 101, n).astype(dtype)
+    want = orc.accumulate("add", h, dims=1).astype(dtype)
+    ws = _fresh_workspace(L, 16 << 20)
+    alone = 0
+    for _ in range(6):
+        y = rk.ROCArray(h)
+        assert L.lib.rk_accumulate(L.RK_OP_ADD, y.code, y.code, y.ptr, y.ptr, 1, L.shape_array(y.dims), 1, 1, None,
+                                   ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+        assert L.lib.rk_workspace_status(ws.data_ptr(), ws.numel(), stream_ptr()) == 0
+        assert np.array_equal(rk.Array(y), want)
+        alone = _alone_count(ws)
+    assert alone > 0
+
+
 def test_ordered_scan_of_many_lines_helps_itself(rk, orc, tiny_budget):
     L = tiny_budget
     from amdgpu_jl_amd.array import stream_ptr
