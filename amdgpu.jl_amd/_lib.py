@@ -107,6 +107,8 @@ PROTOTYPES = {
                                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_findminmax": (C.c_int32, [C.c_int32, C.c_int, C.c_void_p, C.c_int, _I64P, C.c_uint32,
                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "rk_findminmax_strided": (C.c_int32, [C.c_int32, C.c_int, C.c_void_p, C.c_int, _I64P, _I64P, C.c_uint32,
+                                          C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_accumulate": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,
                                   C.c_int32, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "rk_accumulate_static": (C.c_int32, [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, _I64P, C.c_int,

@@ -231,6 +231,23 @@ static int32_t static_scratch(hipStream_t stream, void** out) {
 
 using namespace rk;
 
+static int32_t findminmax_dispatch(rk_dtype in, const FindArgs& a) {
+    switch (in) {
+        case RK_F32: return findminmax_f32(a);
+        case RK_F16: return findminmax_f16(a);
+        case RK_F64: return findminmax_f64(a);
+        case RK_I32: return findminmax_i32(a);
+        case RK_I64: return findminmax_i64(a);
+        case RK_U8:  return findminmax_u8(a);
+        case RK_I8:  return findminmax_i8(a);
+        case RK_I16: return findminmax_i16(a);
+        case RK_U16: return findminmax_u16(a);
+        case RK_U32: return findminmax_u32(a);
+        case RK_U64: return findminmax_u64(a);
+        default: return RK_ERR_UNSUPPORTED;
+    }
+}
+
 extern "C" {
 
 int32_t rk_version(void) { return RK_VERSION; }
@@ -471,21 +488,43 @@ int32_t rk_findminmax(int32_t want_max, rk_dtype in, const void* A, int ndim, co
     if (A == nullptr || (vals == nullptr && cart_idx == nullptr)) return RK_ERR_INVALID_ARGUMENT;
     reduce_mask &= (1u << ndim) - 1u;
     FindArgs a{want_max ? 1 : 0, A, ndim, shape, reduce_mask, vals, cart_idx, ws, ws_bytes, (hipStream_t)stream};
-    switch (in) {
-        case RK_F32: return findminmax_f32(a);
-        case RK_F16: return findminmax_f16(a);
-        case RK_F64: return findminmax_f64(a);
-        case RK_I32: return findminmax_i32(a);
-        case RK_I64: return findminmax_i64(a);
-        case RK_U8:  return findminmax_u8(a);
-        case RK_I8:  return findminmax_i8(a);
-        case RK_I16: return findminmax_i16(a);
-        case RK_U16: return findminmax_u16(a);
-        case RK_U32: return findminmax_u32(a);
-        case RK_U64: return findminmax_u64(a);
-        default: return RK_ERR_UNSUPPORTED;
-    }
+    return findminmax_dispatch(in, a);
 }
+
+int32_t rk_findminmax_strided(int32_t want_max, rk_dtype in, const void* A, int ndim, const int64_t* shape, const int64_t* a_strides,
+                              uint32_t reduce_mask, void* vals, int64_t* cart_idx, void* ws, size_t ws_bytes, void* stream) {
+    int64_t total = 0;
+    if (!valid_dtype(in)) return RK_ERR_INVALID_ARGUMENT;
+    if (!valid_shape(ndim, shape, &total)) return RK_ERR_INVALID_ARGUMENT;
+    if (total == 0) return RK_SUCCESS;
+    if (A == nullptr || (vals == nullptr && cart_idx == nullptr)) return RK_ERR_INVALID_ARGUMENT;
+    reduce_mask &= (1u << ndim) - 1u;
+    DenseOrder o{};
+    if (!dense_order(ndim, shape, a_strides, &o)) return RK_ERR_UNSUPPORTED;
+    // the kernels number the dims by their place in memory and lay the outputs out by the kept dims in that order; the
+    // caller's outputs are dense in the LOGICAL order of the kept dims: served when the two orders agree (a transposed
+    // matrix reduced along either dim, any wrapper reduced to one kept dim or to a scalar), declined otherwise
+    // The same holds among the reduced dims: "the first of several equal winners" is the first in the wrapper's
+    // column-major order, which is the order of the memory positions only when the reduced dims keep their order.
+    uint32_t mask_mem = 0;
+    int last_kept = -1, last_reduced = -1;
+    for (int k = 0; k < ndim; ++k) {
+        const int d = o.order[k];
+        if (shape[d] == 1) { if ((reduce_mask >> d) & 1u) mask_mem |= 1u << k; continue; }
+        if ((reduce_mask >> d) & 1u) {
+            mask_mem |= 1u << k;
+            if (d < last_reduced) return RK_ERR_UNSUPPORTED;
+            last_reduced = d;
+        } else {
+            if (d < last_kept) return RK_ERR_UNSUPPORTED;
+            last_kept = d;
+        }
+    }
+    FindArgs a{want_max ? 1 : 0, A, ndim, o.shape, mask_mem, vals, cart_idx, ws, ws_bytes, (hipStream_t)stream};
+    a.slot = o.order;        // memory dim k is the wrapper's dim order[k]: the index goes out in the wrapper's coordinates
+    return findminmax_dispatch(in, a);
+}
+
 
 int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out, const void* in_ptr, void* out_ptr, int ndim, const int64_t* shape,
                       int dim, int32_t inclusive, const void* init, void* ws, size_t ws_bytes, void* stream) {

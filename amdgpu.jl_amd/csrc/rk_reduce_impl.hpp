@@ -137,6 +137,7 @@ template <typename T, typename P> struct ArgSink {
     int64_t  shape[RK_MAX_DIMS];
     bool     want_max;
     bool     absolute;   // positions are already linear offsets into A (the generic kernel)
+    int8_t   slot[RK_MAX_DIMS];   // component of the CartesianIndex that dim d of `shape` fills (d itself; a wrapper's logical dim)
     LineGeom g;
     __device__ __forceinline__ void operator()(int64_t q, ArgAcc<T, P> t) const {
         const int64_t lin = absolute ? (int64_t)t.i : line_base(g, q) + (int64_t)t.i * g.inner;
@@ -146,7 +147,7 @@ template <typename T, typename P> struct ArgSink {
             for (int d = 0; d < ndim; ++d) {
                 const int64_t c = rem % shape[d];
                 rem /= shape[d];
-                cart[q * ndim + d] = c + 1;
+                cart[q * ndim + slot[d]] = c + 1;
             }
         }
     }
@@ -1166,6 +1167,7 @@ struct FindArgs {
     const void* A; int ndim; const int64_t* shape; uint32_t mask;
     void* vals; int64_t* cart;
     void* ws; size_t ws_bytes; hipStream_t stream;
+    const int* slot = nullptr;   // CartesianIndex component per dim of `shape` (nullptr: the dim itself)
 };
 
 // Reduced dims that are not neighbours (dims=(1,3); the (1,2,4) of a batch norm): the generic kernel walks every
@@ -1342,6 +1344,7 @@ inline int32_t findminmax_pos(const FindArgs& a, const Shape3& s) {
     sink.cart = a.cart;
     sink.ndim = a.ndim;
     for (int d = 0; d < a.ndim; ++d) sink.shape[d] = a.shape[d];
+    for (int d = 0; d < RK_MAX_DIMS; ++d) sink.slot[d] = (int8_t)(a.slot != nullptr && d < a.ndim ? a.slot[d] : d);
     sink.want_max = a.want_max != 0;
     sink.absolute = !s.single_run;
     sink.g = LineGeom{s.inner, s.mid, s.inner * s.outer};

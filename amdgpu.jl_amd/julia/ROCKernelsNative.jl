@@ -10,7 +10,7 @@
 #   GPUArrays.mapreducedim!(f, op, R::AnyROCArray, A; init)  src/kernels/mapreduce.jl:86-173
 #   Base.accumulate!/accumulate/cumsum/cumprod               src/kernels/accumulate.jl:1-8
 #   Base.copyto!(dest, ::Broadcasted{<:ROCArrayStyle})       src/broadcast.jl:3-35 (+ GPUArrays _copyto!)
-#   findmax/findmin(A; dims)                                 GPUArrays findminmax -> mapreducedim!
+#   findmax/findmin(A; dims), A a ROCArray or a transpose / PermutedDimsArray of one   GPUArrays findminmax -> mapreducedim!
 #   volumerhs!(rhs, Q, vgeo, gravity, D, nelem)              perf/volumerhs.jl:200-201
 #
 # This file is shipped as text: no Julia runtime exists where this repository is built and tested, so it is
@@ -318,7 +318,43 @@ function native_findminmax(wantmax::Bool, A::ROCArray{T,N}, dims) where {T,N}
     check(st)
     return vals, idx
 end
+# A a transpose / PermutedDimsArray: the library reduces the parent in memory order and writes the index in the wrapper's
+# coordinates; it declines (-> stock method) the dim orders for which the first of equal winners or the output layout
+# would differ from the wrapper's column-major order, and views with gaps
+function native_findminmax_strided(wantmax::Bool, A::ROCWrapper{T,N}, dims) where {T,N}
+    mask = UInt32(0)
+    for d in (dims === Colon() ? (1:N) : dims)
+        d <= N && (mask |= UInt32(1) << (d - 1))
+    end
+    rdims = ntuple(d -> (mask >> (d - 1)) & 1 == 1 ? 1 : size(A, d), N)
+    vals = similar(parent(A), T, rdims)
+    idx = similar(parent(A), CartesianIndex{N}, rdims)
+    ws = workspace()
+    shape = Int64[size(A)...]
+    as = strides64(A, N)
+    GC.@preserve A vals idx ws shape as begin
+        st = ccall((:rk_findminmax_strided, librk[]), Int32,
+                   (Int32, Cint, Ptr{Cvoid}, Cint, Ptr{Int64}, Ptr{Int64}, UInt32, Ptr{Cvoid}, Ptr{Int64}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+                   wantmax, rk_dtype(T), pointer(A), N, shape, as, mask, pointer(vals),
+                   convert(Ptr{Int64}, pointer(idx)), pointer(ws), length(ws), stream_ptr())
+    end
+    declined(st) && return nothing
+    check(st)
+    return vals, idx
+end
 function enable_findminmax!()
+    for (fn, wantmax) in ((:findmax, true), (:findmin, false))
+        @eval function Base.$fn(A::ROCWrapper{T,N}; dims=:) where {T<:Union{Float16,Float32,Float64,Int8,Int16,Int32,Int64,UInt16,UInt32,UInt64},N}
+            (isempty(A) || !is_strided_wrapper(A)) && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
+            res = native_findminmax_strided($wantmax, A, dims)
+            res === nothing && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
+            vals, idx = res
+            dims === Colon() || return vals, idx
+            v = AMDGPU.@allowscalar vals[1]
+            i = AMDGPU.@allowscalar idx[1]
+            return v, (N == 1 ? i[1] : i)
+        end
+    end
     for (fn, wantmax) in ((:findmax, true), (:findmin, false))
         @eval function Base.$fn(A::ROCArray{T,N}; dims=:) where {T<:Union{Float16,Float32,Float64,Int8,Int16,Int32,Int64,UInt16,UInt32,UInt64},N}
             isempty(A) && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)       # the stock method's error

@@ -332,7 +332,7 @@ def findfirst(*args):
     return i if v else None
 
 
-def _findminmax(A: ROCArray, want_max: bool, dims):
+def _findminmax(A, want_max: bool, dims):
     if len(A) == 0:
         raise ValueError("reducing over an empty collection is not allowed")
     mask = _dims_mask(dims, A.ndim)
@@ -341,16 +341,24 @@ def _findminmax(A: ROCArray, want_max: bool, dims):
     # Array{CartesianIndex{N}}: N Int64 per element; kept as an Int64 array with a leading dim N
     idx = ROCArray(dims=(A.ndim,) + rshape, dtype=np.int64)
     ws, ws_bytes = workspace()
-    st = L.lib.rk_findminmax(1 if want_max else 0, A.code, A.ptr, A.ndim, L.shape_array(A.dims), mask,
-                             vals.ptr, idx.ptr, ws, ws_bytes, stream_ptr())
-    L.check(st, "rk_findminmax")
+    from .views import ROCView
+    if isinstance(A, ROCView):
+        # wrapper arrays (transpose, PermutedDimsArray): the index comes back in the wrapper's coordinates; orders of
+        # dims for which the first of equal winners or the output layout would differ raise UnsupportedError
+        st = L.lib.rk_findminmax_strided(1 if want_max else 0, A.code, A.sptr, A.ndim, L.shape_array(A.dims),
+                                         L.shape_array(tuple(A.strides)), mask, vals.ptr, idx.ptr, ws, ws_bytes, stream_ptr())
+        L.check(st, "rk_findminmax_strided")
+    else:
+        st = L.lib.rk_findminmax(1 if want_max else 0, A.code, A.ptr, A.ndim, L.shape_array(A.dims), mask,
+                                 vals.ptr, idx.ptr, ws, ws_bytes, stream_ptr())
+        L.check(st, "rk_findminmax")
     if dims is None:
         c = tuple(int(v) for v in idx.to_host().reshape(-1))
         return vals.item(), (c[0] if A.ndim == 1 else c)
     return vals, idx
 
 
-def findmax(A: ROCArray, dims=None):
+def findmax(A, dims=None):
     """``findmax(A; dims)``: (values, indices).  With ``dims``: ``values`` is a ROCArray with reduced
     dims of extent 1 and ``indices`` an Int64 ROCArray of dims ``(ndims(A), size(values)...)`` whose
     column ``[:, I]`` is the CartesianIndex of the winner.  Without: host scalar and index tuple
@@ -358,7 +366,7 @@ def findmax(A: ROCArray, dims=None):
     return _findminmax(A, True, dims)
 
 
-def findmin(A: ROCArray, dims=None):
+def findmin(A, dims=None):
     return _findminmax(A, False, dims)
 
 

@@ -69,13 +69,14 @@ typedef enum {
     RK_U32 = 5,  /* UInt32  */
     RK_U64 = 6,  /* UInt64  */
     RK_F16 = 7,  /* Float16: rk_mapreduce (accumulating in Float32), rk_findminmax, rk_broadcast operands and
-                  * destinations, rk_sort / rk_sortperm; not rk_accumulate (RK_ERR_UNSUPPORTED) */
+                  * destinations, rk_sort / rk_sortperm, rk_accumulate (scanned in Float32, rounded once at the store) */
     RK_I16 = 8,  /* Int16 */
     RK_I8  = 9,  /* Int8  */
     RK_U16 = 10  /* UInt16.  The three narrow integers: rk_mapreduce (sum / prod into Int64 or UInt64 as Base.add_sum
                   * widens them, max / min in their own type), rk_findminmax, rk_broadcast operands and destinations
-                  * (integer programs compute in Int64 and store the low bits); Int16 also rk_sort / rk_sortperm.  Not
-                  * rk_accumulate, not rk_mapreduce_program (RK_ERR_UNSUPPORTED).  rk_reverse and rk_permutedims take an
+                  * (integer programs compute in Int64 and store the low bits), rk_accumulate into their own type
+                  * (scanned in 32 bits, the store keeps the low bits = the type's own wrap-around); Int16 also rk_sort /
+                  * rk_sortperm.  Not rk_mapreduce_program (RK_ERR_UNSUPPORTED).  rk_reverse and rk_permutedims take an
                   * element SIZE, not a dtype, and so move any 1- or 2-byte element */
 } rk_dtype;
 
@@ -217,6 +218,18 @@ RK_API int32_t rk_findminmax(int32_t want_max, rk_dtype in,
                       void* vals, int64_t* cart_idx,
                       void* ws, size_t ws_bytes, void* stream);
 
+/* The same for wrapper arrays -- findmax(transpose(A); dims), findmin(PermutedDimsArray(A, p); dims) -- which the
+ * reference sends through the same generic findminmax of GPUArrays (src/kernels/mapreduce.jl:86-173 underneath).
+ * `shape` and `a_strides` (in elements) describe the wrapper; it must be a permutation of a dense array's dims.  The
+ * index goes out in the wrapper's coordinates, the outputs are dense in the wrapper's shape.  Served when the kept dims
+ * and the reduced dims each keep their relative order in memory (a transposed matrix along either dim, any wrapper with
+ * one reduced dim whose kept dims are in order): then "first of equal winners" and the output layout agree with the
+ * wrapper's column-major order.  Anything else is RK_ERR_UNSUPPORTED (copy the wrapper first). */
+RK_API int32_t rk_findminmax_strided(int32_t want_max, rk_dtype in,
+                      const void* A, int ndim, const int64_t* shape, const int64_t* a_strides, uint32_t reduce_mask,
+                      void* vals, int64_t* cart_idx,
+                      void* ws, size_t ws_bytes, void* stream);
+
 /* ---- accumulate / cumsum / cumprod -------------------------------------------------
  * Replaces Base.accumulate!/accumulate/cumsum/cumprod(::AnyROCArray)
  *                                                        src/kernels/accumulate.jl:1-8
@@ -226,8 +239,8 @@ RK_API int32_t rk_findminmax(int32_t want_max, rk_dtype in,
  * `out` may alias `in` when the dtypes agree.  inclusive != 0: out[k] = init op a[1] op ..
  * op a[k]; inclusive == 0: out[k] = init op a[1] op .. op a[k-1].  `init` = host pointer to
  * one `out` element or NULL for the neutral element.  Integer arithmetic wraps.
- * Supported (in -> out): same type; U8 -> I64, U8 -> I32 (Bool counts). ADD and MUL;
- * MAX/MIN for same-type scans. */
+ * Supported (in -> out): same type (every rk_dtype); U8 -> I64, U8 -> I32 (Bool counts). ADD and MUL;
+ * MAX / MIN, and AND / OR / XOR on integer types, for same-type scans. */
 RK_API int32_t rk_accumulate(rk_op op, rk_dtype in, rk_dtype out,
                       const void* in_ptr, void* out_ptr,
                       int ndim, const int64_t* shape, int dim, int32_t inclusive,

@@ -88,6 +88,13 @@ def test_findminmax_and_accumulate_validation(L):
     assert g(1, L.RK_F32, one, 2, sh, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT      # no output requested
     assert g(1, 99, one, 2, sh, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT                # no such element type
     assert g(1, L.RK_F32, None, 2, L.shape_array((0, 4)), 1, None, None, None, 0, None) == L.RK_SUCCESS
+    gs = L.lib.rk_findminmax_strided
+    tr = L.shape_array((4, 1))                                   # a 4 x 4 transpose: strides (4, 1)
+    assert gs(1, L.RK_F32, None, 2, sh, tr, 1, one, one, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert gs(1, L.RK_F32, one, 2, sh, tr, 1, None, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
+    assert gs(1, L.RK_F32, one, 2, sh, L.shape_array((2, 8)), 1, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED     # a view with gaps
+    assert gs(1, L.RK_F32, one, 2, sh, tr, 3, one, one, None, 0, None) == L.RK_ERR_UNSUPPORTED    # dims=: of a transpose: the first of equal winners differs
+    assert gs(1, L.RK_F32, None, 2, L.shape_array((0, 4)), tr, 1, None, None, None, 0, None) == L.RK_SUCCESS
     a = L.lib.rk_accumulate
     assert a(0, L.RK_F32, L.RK_F32, None, one, 2, sh, 1, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT
     assert a(0, L.RK_F32, L.RK_F32, one, one, 2, sh, 0, 1, None, None, 0, None) == L.RK_ERR_INVALID_ARGUMENT   # dim is 1-based
