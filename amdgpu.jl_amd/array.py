@@ -106,8 +106,19 @@ class ROCArray:
         return raw.view(self.dtype)[:n].reshape(self.dims, order="F").copy()
 
     def item(self):
-        a = self.to_host()
-        return a.reshape(-1)[0]
+        """The first element as a host scalar (the scalar fetch behind ``sum(x)``, ``findmax(x)``, the count of
+        ``findall``): one small copy into a pinned staging buffer kept per stream, then one stream synchronisation."""
+        if len(self) == 0:
+            raise IndexError("item() of an empty array")
+        check_waits()                       # the host waits here anyway: the place to learn of a give-up
+        n = self.dtype.itemsize
+        key = (torch.cuda.current_device(), stream_ptr())
+        pin = _staging.get(key)
+        if pin is None:
+            pin = _staging[key] = torch.empty(16, dtype=torch.uint8, pin_memory=True)
+        pin[:n].copy_(self.buf[self.offset:self.offset + n], non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return pin.numpy()[:n].view(self.dtype)[0].copy()
 
     # -- wrappers that keep the storage ----------------------------------------------------------
     def reshape(self, *dims):
@@ -186,6 +197,7 @@ def workspace(min_bytes: int = 0):
 # runs out of it records that in the workspace (the sort: in its temporary) and finishes with meaningless results.
 # The mirror reads those records where it synchronises anyway -- Array(x), item() -- for every workspace and sort
 # temporary that such a kernel has used on the current stream since the last look, and raises.
+_staging: dict = {}            # (device, stream) -> pinned bytes for scalar fetches (item())
 _waiting: set = set()          # (device, stream) keys whose workspace has been handed to a kernel with bounded waits
 _sort_tmps: dict = {}          # (device, stream) -> temporaries of sorts whose record has not been read
 
