@@ -10,7 +10,7 @@
 //
 // Up to 256 tiles (RK_SORT_LOOKBACK_TILES; 2^20 keys) the counts of the earlier tiles come from a chained look-back (tiles in
 // ticket order publish their 256 counts, one lane per digit walks back), and a pass reads and writes every key once:
-//   sort_min_kernel      one read of the keys: the smallest mapped key, which every key is taken relative to
+//   sort_min_kernel      integers: one read of the keys for the smallest mapped key, which every key is taken relative to
 //   sort_hist_kernel     one read of the keys: the 256-bin histogram of every digit at once
 //   sort_plan_kernel     exclusive scan of every histogram = first output slot of each digit value; passes whose
 //                        digit is the same for all keys are skipped (small-range integers need 1-2 passes);
@@ -199,8 +199,13 @@ __device__ __forceinline__ void count_digit(uint32_t* row, uint32_t d, bool vali
 }
 
 // ---- init: clear control block and descriptors ------------------------------------------------------------
-__global__ __launch_bounds__(256) void sort_init_kernel(uint64_t* words, int64_t nwords) {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * 256) words[i] = 0;
+// min_is_zero: the keys are not taken relative to their smallest (floats: the read that finds it saves no pass), so the
+// control block starts with ~0 in inv_min, i.e. a smallest mapped key of 0.
+__global__ __launch_bounds__(256) void sort_init_kernel(uint64_t* words, int64_t nwords, int min_is_zero) {
+    constexpr int64_t INV_MIN_WORD = (int64_t)(offsetof(SortCtl, inv_min) / sizeof(uint64_t));
+    static_assert(offsetof(SortCtl, inv_min) % sizeof(uint64_t) == 0, "inv_min is one of the cleared words");
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nwords; i += (int64_t)gridDim.x * 256)
+        words[i] = (min_is_zero && i == INV_MIN_WORD) ? ~0ull : 0ull;
 }
 
 // The two whole-array reads below take 16-byte vectors from the aligned body [head, head + nvec * VEC) of the keys
@@ -894,7 +899,11 @@ static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, voi
     const int64_t init_words = (int64_t)(l.clear_end / sizeof(uint64_t));
     int64_t g = (init_words + 255) / 256;
     if (g > cus * 16) g = cus * 16;
-    sort_init_kernel<<<(unsigned)g, 256, 0, stream>>>((uint64_t*)base, init_words);
+    // floats: no read for the smallest key.  Relative keys let small-range integers skip passes (1000 .. 1255: one pass
+    // instead of two); the exponent bytes of floats are constant or not whatever is subtracted, and the histograms of the
+    // small sorts find constant digits by themselves.
+    constexpr bool FLOAT_KEYS = !std::is_integral<T>::value;
+    sort_init_kernel<<<(unsigned)g, 256, 0, stream>>>((uint64_t*)base, init_words, FLOAT_KEYS ? 1 : 0);
     RK_LAUNCH_CHECK();
     g = (n + 256 * 16 - 1) / (256 * 16);
     if (g > cus * 8) g = cus * 8;
@@ -906,8 +915,10 @@ static int32_t sort_typed(void* keys, int64_t* perm_out, int64_t n, int rev, voi
     const unsigned gmin = (unsigned)(g < cus * 2 ? g : cus * 2), ghist = (unsigned)(g < cus * 4 ? g : cus * 4);
     // sortperm: the first pass reads the caller's keys and should write buffer A, i.e. "reads B"
     if (!l.counted) {
-        sort_min_kernel<T><<<gmin, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
-        RK_LAUNCH_CHECK();
+        if (!FLOAT_KEYS) {
+            sort_min_kernel<T><<<gmin, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
+            RK_LAUNCH_CHECK();
+        }
         sort_hist_kernel<T, PASSES><<<ghist, 256, 0, stream>>>((const T*)keys, n, head, nvec, rev, ctl);
         RK_LAUNCH_CHECK();
         sort_plan_kernel<<<1, 256, 0, stream>>>(ctl, PASSES, (uint32_t)n, perm ? 1 : 0, 0);
