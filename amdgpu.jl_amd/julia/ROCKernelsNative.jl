@@ -321,7 +321,8 @@ end
 # A a transpose / PermutedDimsArray: the library reduces the parent in memory order and writes the index in the wrapper's
 # coordinates; it declines (-> stock method) the dim orders for which the first of equal winners or the output layout
 # would differ from the wrapper's column-major order, and views with gaps
-function native_findminmax_strided(wantmax::Bool, A::ROCWrapper{T,N}, dims) where {T,N}
+function native_findminmax_strided(wantmax::Bool, A::ROCWrapper{T}, dims) where {T}
+    N = ndims(A)                 # (not a static parameter: a Transpose does not bind the alias's N)
     mask = UInt32(0)
     for d in (dims === Colon() ? (1:N) : dims)
         d <= N && (mask |= UInt32(1) << (d - 1))
@@ -344,7 +345,8 @@ function native_findminmax_strided(wantmax::Bool, A::ROCWrapper{T,N}, dims) wher
 end
 function enable_findminmax!()
     for (fn, wantmax) in ((:findmax, true), (:findmin, false))
-        @eval function Base.$fn(A::ROCWrapper{T,N}; dims=:) where {T<:Union{Float16,Float32,Float64,Int8,Int16,Int32,Int64,UInt16,UInt32,UInt64},N}
+        @eval function Base.$fn(A::ROCWrapper{T}; dims=:) where {T<:Union{Float16,Float32,Float64,Int8,Int16,Int32,Int64,UInt16,UInt32,UInt64}}
+            N = ndims(A)
             (isempty(A) || !is_strided_wrapper(A)) && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
             res = native_findminmax_strided($wantmax, A, dims)
             res === nothing && return invoke(Base.$fn, Tuple{GPUArrays.AnyGPUArray}, A; dims)
