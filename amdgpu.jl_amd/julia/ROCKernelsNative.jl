@@ -167,7 +167,8 @@ end
 
 # R or A a transpose / PermutedDimsArray / contiguous view, e.g. mapreducedim!(identity, +, transpose(R), A): the
 # library renumbers the dims of permuted-dense arrays and declines (-> stock method) views with gaps
-function native_mapreducedim_strided!(f, op, R::ROCStrided{TR}, A::ROCStrided{TA,N}, init) where {TR,TA,N}
+function native_mapreducedim_strided!(f, op, R::ROCStrided{TR}, A::ROCStrided{TA}, init) where {TR,TA}
+    N = ndims(A)                 # (not a static parameter: a Transpose does not bind the alias's N)
     Base.check_reducedims(R, A)
     isempty(A) && return true
     mask = UInt32(0)
@@ -393,7 +394,9 @@ function native_accumulate!(op, B::ROCArray{TB,N}, A::ROCArray{TA,N}; init, dims
     return true
 end
 
-function native_accumulate_strided!(op, B::ROCStrided{TB,N}, A::ROCStrided{TA,N}; init, dims, inclusive::Bool) where {TB,TA,N}
+function native_accumulate_strided!(op, B::ROCStrided{TB}, A::ROCStrided{TA}; init, dims, inclusive::Bool) where {TB,TA}
+    N = ndims(A)                 # (a Transpose does not bind the alias's N)
+    ndims(B) == N || throw(DimensionMismatch("accumulate!: $(size(B)) vs $(size(A))"))
     size(B) == size(A) || throw(DimensionMismatch("accumulate!: $(size(B)) vs $(size(A))"))
     isempty(A) && return true
     dim = dims === nothing ? (N == 1 ? 1 : throw(ArgumentError("accumulate on N-d arrays needs dims"))) : Int(dims)
@@ -505,7 +508,8 @@ function flatten_node!(ops::Vector{Any}, toks::Vector{Int32}, x)
     end
 end
 
-function native_copyto!(dest::Union{ROCArray{TD,N},ROCWrapper{TD,N}}, bc::Broadcasted) where {TD,N}
+function native_copyto!(dest::Union{ROCArray{TD},ROCWrapper{TD}}, bc::Broadcasted) where {TD}
+    N = ndims(dest)              # (a Transpose does not bind the alias's N)
     ops, toks = Any[], Int32[]
     flatten!(ops, toks, bc)
     length(toks) <= RK_MAX_PROGRAM || throw(Unsupported())
